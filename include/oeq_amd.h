@@ -1,0 +1,162 @@
+/*
+ * C ABI of liboeq_amd.so: runtime compilation (hiprtc) and launch of the
+ * per-problem HIP kernels behind TensorProduct / TensorProductConv.
+ *
+ * Plain pointers and sizes only; no torch, pybind11 or C++ types cross this
+ * boundary. Every function returns 0 on success or a negative oeq_status and
+ * leaves a message retrievable with oeq_last_error() (thread-local). Nothing
+ * in this library calls exit() or throws across the boundary.
+ *
+ * All device pointers must belong to the device that is current on the calling
+ * thread; `stream` is a hipStream_t (NULL = the default stream). Calls only
+ * enqueue work; the caller keeps the buffers alive until the stream has
+ * consumed them.
+ *
+ * Each entry point names the reference interface it stands in for
+ * (paths relative to openequivariance/openequivariance/ in the reference tree).
+ */
+#ifndef OEQ_AMD_H
+#define OEQ_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    OEQ_OK = 0,
+    OEQ_ERR_INVALID = -1,   /* bad argument (null pointer, size, role not present) */
+    OEQ_ERR_COMPILE = -2,   /* hiprtc rejected the source; log in oeq_last_error() */
+    OEQ_ERR_HIP = -3,       /* a HIP runtime call failed */
+    OEQ_ERR_NOMEM = -4
+} oeq_status;
+
+/* ---- device properties ------------------------------------------------- */
+/* Replaces DeviceProp (extension/backend/backend_hip.hpp:103-121). */
+typedef struct {
+    char name[256];
+    char arch[64];              /* e.g. "gfx950" (feature suffixes stripped) */
+    int32_t wave_size;
+    int32_t compute_units;
+    int32_t lds_per_block;      /* bytes */
+    int32_t max_threads_per_block;
+    int32_t clock_khz;
+    int32_t l2_bytes;
+    int64_t total_mem;          /* bytes */
+} oeq_device_props;
+
+int oeq_get_device_props(int device, oeq_device_props* out);
+
+/* ---- runtime compilation ---------------------------------------------- */
+/* Replaces HIPJITKernel::compile (extension/backend/backend_hip.hpp:217-288).
+ * `arch` is explicit ("gfx950"), so this works on a host with no GPU.
+ * On success *code / *code_size receive a malloc'd code object; release it
+ * with oeq_free(). On OEQ_ERR_COMPILE the compiler log is the error string. */
+int oeq_jit_compile(const char* source, const char* arch,
+                    const char* const* options, int n_options,
+                    void** code, size_t* code_size);
+void oeq_free(void* p);
+
+/* ---- a loaded set of kernels for one problem --------------------------- */
+/* Replaces JITTPImpl / JITConvImpl (extension/tensorproducts.hpp:10-113,
+ * extension/convolution.hpp:15-179) together with KernelProp
+ * (extension/torch_core.hpp:144-178). */
+typedef struct oeq_kernels oeq_kernels;
+
+typedef enum {
+    OEQ_ROLE_TP_FORWARD = 0,
+    OEQ_ROLE_TP_BACKWARD = 1,
+    OEQ_ROLE_CONV_FORWARD = 2,      /* main forward kernel (either mode) */
+    OEQ_ROLE_CONV_BACKWARD = 3,     /* main backward kernel (either mode) */
+    OEQ_ROLE_CONV_FIXUP_BACKWARD = 4,/* deterministic mode: sender-ordered segmented reduction */
+    OEQ_ROLE_SEGMENT_PTR = 5,       /* builds CSR pointers from a sorted index list */
+    OEQ_ROLE_FILL_ZERO = 6,         /* clears a buffer (used instead of memset: capture-safe) */
+    OEQ_ROLE_TP_BACKWARD_WREDUCE = 7,/* shared weights: second pass of the weight-gradient reduction */
+    OEQ_ROLE_COUNT = 8
+} oeq_role;
+
+typedef struct {
+    int32_t role;               /* oeq_role */
+    const char* kernel_name;    /* __global__ symbol (extern "C") in the code object */
+    uint32_t block_threads;
+    uint32_t units_per_block;   /* rows / nodes / edges one block handles per sweep */
+    uint32_t max_blocks;        /* 0 = one block per ceil(units/units_per_block) */
+} oeq_kernel_desc;
+
+typedef struct {
+    int64_t L1_dim, L2_dim, L3_dim, weight_numel;
+    int32_t elem_size;          /* 4 = float, 8 = double (irreps and weights alike) */
+    int32_t shared_weights;     /* weights are [weight_numel] instead of [rows, weight_numel] */
+    int32_t deterministic;      /* conv: receiver-sorted CSR mode */
+    int32_t wpartial_per_block; /* shared weights: partial weight-gradient rows each block of the
+                                   backward kernel writes (0 = none); the workspace holds
+                                   max_blocks * wpartial_per_block rows of weight_numel elements */
+} oeq_problem_dims;
+
+int oeq_kernels_create(const void* code, size_t code_size,
+                       const oeq_problem_dims* dims,
+                       const oeq_kernel_desc* descs, int n_descs,
+                       oeq_kernels** out);
+void oeq_kernels_destroy(oeq_kernels* k);
+
+/* ---- batched tensor product ------------------------------------------- */
+/* Replaces JITTPImpl::exec_tensor_product (extension/tensorproducts.hpp:75-85)
+ * as called by jit_tp_forward (extension/torch_core.hpp:274-310).
+ * L1_in [num_batch, L1_dim], L2_in [num_batch, L2_dim],
+ * W [num_batch, weight_numel] or [weight_numel], L3_out [num_batch, L3_dim]
+ * (every element is overwritten). */
+int oeq_tp_forward(oeq_kernels* k, int64_t num_batch,
+                   const void* L1_in, const void* L2_in, const void* W,
+                   void* L3_out, void* stream);
+
+/* Replaces JITTPImpl::backward (extension/tensorproducts.hpp:87-95) as called
+ * by jit_tp_backward (extension/torch_core.hpp:312-355). All three gradients
+ * are fully overwritten. With shared weights `workspace` must hold
+ * oeq_tp_backward_workspace_bytes() bytes (partial weight gradients, reduced
+ * in a fixed order: no atomics); otherwise it may be NULL. */
+int oeq_tp_backward(oeq_kernels* k, int64_t num_batch,
+                    const void* L1_in, void* L1_grad,
+                    const void* L2_in, void* L2_grad,
+                    const void* W, void* W_grad,
+                    const void* L3_grad,
+                    void* workspace, size_t workspace_bytes, void* stream);
+size_t oeq_tp_backward_workspace_bytes(const oeq_kernels* k, int64_t num_batch);
+
+/* ---- fused graph convolution ------------------------------------------ */
+/* Replaces JITConvImpl::exec_conv (extension/convolution.hpp:78-107) as called
+ * by jit_conv_forward (extension/torch_core.hpp:422-476).
+ * L1_in [node_count, L1_dim], L2_in [nnz, L2_dim], W [nnz, weight_numel] or
+ * [weight_numel], rows/cols int64 [nnz] (rows = receiver, cols = sender),
+ * L3_out [node_count, L3_dim] (cleared and fully written by this call).
+ * Deterministic mode requires rows sorted ascending and a workspace of
+ * oeq_conv_forward_workspace_bytes() bytes. */
+int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz,
+                     const void* L1_in, const void* L2_in, const void* W,
+                     void* L3_out, const int64_t* rows, const int64_t* cols,
+                     void* workspace, size_t workspace_bytes, void* stream);
+size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
+
+/* Replaces JITConvImpl::backward (extension/convolution.hpp:109-136) as called
+ * by jit_conv_backward (extension/torch_core.hpp:478-542). Deterministic mode
+ * additionally needs transpose_perm [nnz]: the permutation listing the
+ * (row-sorted) edges in sender-major order; it is ignored in atomic mode. */
+int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz,
+                      const void* L1_in, void* L1_grad,
+                      const void* L2_in, void* L2_grad,
+                      const void* W, void* W_grad,
+                      const void* L3_grad,
+                      const int64_t* rows, const int64_t* cols,
+                      const int64_t* transpose_perm,
+                      void* workspace, size_t workspace_bytes, void* stream);
+size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
+
+/* ---- diagnostics -------------------------------------------------------- */
+const char* oeq_last_error(void);
+int oeq_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OEQ_AMD_H */

@@ -1,0 +1,305 @@
+"""PyTorch custom ops over the C ABI.
+
+Stand in for the reference's native op library
+(openequivariance/openequivariance/extension/torch_core.hpp:274-644:
+``jit_tp_forward``, ``jit_tp_backward``, ``jit_conv_forward``,
+``jit_conv_backward`` and their double-backward companions) and its Python
+registrations of fake kernels, autograd and autocast
+(openequivariance/openequivariance/_torch/TensorProduct.py:182-374,
+_torch/TensorProductConv.py:280-568).
+
+The ops take an integer ``kid`` naming a compiled kernel set in a process-wide
+registry instead of a JSON byte tensor. Argument checks raise ``RuntimeError``
+with the reference's wording (torch_core.hpp:109-134).
+
+Second and higher derivatives need no extra kernels: with
+S(x, y, w, g) = <g, TP(x, y, w)> multilinear, the backward op returns
+(dS/dx, dS/dy, dS/dw) and its own vector-Jacobian product is a sum of three
+forward and three backward calls with one argument replaced by a cotangent.
+"""
+
+from __future__ import annotations
+
+import threading
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from .. import runtime as rt
+
+_registry: Dict[int, "KernelEntry"] = {}
+_registry_lock = threading.Lock()
+_next_id = [1]
+
+
+class KernelEntry:
+    """Lazily compiled kernel set + the shape facts the ops validate against."""
+
+    def __init__(self, build_fn, L1, L2, L3, WN, shared, torch_dtype, deterministic=False):
+        self.build_fn = build_fn  # () -> (source, dims, descs)
+        self.L1, self.L2, self.L3, self.WN = L1, L2, L3, WN
+        self.shared = shared
+        self.dtype = torch_dtype
+        self.deterministic = deterministic
+        self._ks: Optional[rt.KernelSet] = None
+        self._lock = threading.Lock()
+
+    def kernels(self) -> rt.KernelSet:
+        if self._ks is None:
+            with self._lock:
+                if self._ks is None:
+                    src, dims, descs = self.build_fn()
+                    self._ks = rt.get_kernel_set(src, dims, descs)
+        return self._ks
+
+
+def register_entry(entry: KernelEntry) -> int:
+    with _registry_lock:
+        kid = _next_id[0]
+        _next_id[0] += 1
+        _registry[kid] = entry
+        return kid
+
+
+def get_entry(kid: int) -> KernelEntry:
+    try:
+        return _registry[kid]
+    except KeyError:
+        raise RuntimeError(f"unknown kernel id {kid}")
+
+
+_DTYPE_CODE = {torch.float32: 1, torch.float64: 2, torch.int32: 3, torch.int64: 4, torch.uint8: 5}
+
+
+def check_tensor(t: torch.Tensor, shape: List[int], dtype: torch.dtype, name: str):
+    """torch_core.hpp:109-134."""
+    if t.dim() != len(shape) or any(int(a) != int(b) for a, b in zip(t.shape, shape)):
+        raise RuntimeError(
+            f"Shape mismatch for tensor '{name}'. Expected: {list(shape)}. Got: {list(t.shape)}"
+        )
+    if not t.is_cuda:
+        raise RuntimeError(f"Tensor '{name}' is not on the GPU.")
+    if t.dtype != dtype:
+        raise RuntimeError(
+            f"Dtype mismatch for tensor '{name}'. Expected: {_DTYPE_CODE.get(dtype, dtype)}. "
+            f"Got: {_DTYPE_CODE.get(t.dtype, t.dtype)}"
+        )
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _wshape(e: KernelEntry, n: int) -> List[int]:
+    return [e.WN] if e.shared else [n, e.WN]
+
+
+# ---------------------------------------------------------------------------
+# batch tensor product
+# ---------------------------------------------------------------------------
+
+
+@torch.library.custom_op("oeq_amd::tp_forward", mutates_args=(), device_types="cuda")
+def tp_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, kid: int) -> torch.Tensor:
+    e = get_entry(kid)
+    n = L1_in.shape[0] if L1_in.dim() > 0 else -1
+    check_tensor(L1_in, [n, e.L1], e.dtype, "L1_in")
+    check_tensor(L2_in, [n, e.L2], e.dtype, "L2_in")
+    check_tensor(W, _wshape(e, n), e.dtype, "W")
+    x, y, w = L1_in.contiguous(), L2_in.contiguous(), W.contiguous()
+    out = x.new_empty((n, e.L3))
+    with torch.cuda.device(x.device):
+        e.kernels().tp_forward(n, x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), _stream())
+    return out
+
+
+@tp_forward.register_fake
+def _(L1_in, L2_in, W, kid):
+    e = get_entry(kid)
+    return L1_in.new_empty((L1_in.shape[0], e.L3))
+
+
+@torch.library.custom_op("oeq_amd::tp_backward", mutates_args=(), device_types="cuda")
+def tp_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_grad: torch.Tensor,
+                kid: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    e = get_entry(kid)
+    n = L1_in.shape[0] if L1_in.dim() > 0 else -1
+    check_tensor(L1_in, [n, e.L1], e.dtype, "L1_in")
+    check_tensor(L2_in, [n, e.L2], e.dtype, "L2_in")
+    check_tensor(W, _wshape(e, n), e.dtype, "W")
+    check_tensor(L3_grad, [n, e.L3], e.dtype, "L3_grad")
+    x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
+    dx, dy, dw = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w)
+    with torch.cuda.device(x.device):
+        ks = e.kernels()
+        nb = ks.tp_backward_workspace_bytes(n)
+        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
+        ks.tp_backward(n, x.data_ptr(), dx.data_ptr(), y.data_ptr(), dy.data_ptr(), w.data_ptr(), dw.data_ptr(),
+                       g.data_ptr(), ws.data_ptr() if nb else 0, nb, _stream())
+    return dx, dy, dw
+
+
+@tp_backward.register_fake
+def _(L1_in, L2_in, W, L3_grad, kid):
+    return torch.empty_like(L1_in), torch.empty_like(L2_in), torch.empty_like(W)
+
+
+def _tp_fwd_setup(ctx, inputs, output):
+    ctx.kid = inputs[3]
+    ctx.save_for_backward(inputs[0], inputs[1], inputs[2])
+
+
+def _tp_fwd_backward(ctx, grad):
+    x, y, w = ctx.saved_tensors
+    dx, dy, dw = tp_backward(x, y, w, grad, ctx.kid)
+    return dx, dy, dw, None
+
+
+tp_forward.register_autograd(_tp_fwd_backward, setup_context=_tp_fwd_setup)
+
+
+def _tp_bwd_setup(ctx, inputs, output):
+    ctx.kid = inputs[4]
+    ctx.save_for_backward(inputs[0], inputs[1], inputs[2], inputs[3])
+
+
+def _zeros_if_none(t, like):
+    return torch.zeros_like(like) if t is None else t
+
+
+def _tp_bwd_backward(ctx, ddx, ddy, ddw):
+    x, y, w, g = ctx.saved_tensors
+    kid = ctx.kid
+    ddx, ddy, ddw = _zeros_if_none(ddx, x), _zeros_if_none(ddy, y), _zeros_if_none(ddw, w)
+    dx1, _, dw1 = tp_backward(x, ddy, w, g, kid)
+    dx2, dy2, _ = tp_backward(x, y, ddw, g, kid)
+    _, dy3, dw3 = tp_backward(ddx, y, w, g, kid)
+    gg = tp_forward(ddx, y, w, kid) + tp_forward(x, ddy, w, kid) + tp_forward(x, y, ddw, kid)
+    return dx1 + dx2, dy2 + dy3, dw1 + dw3, gg, None
+
+
+tp_backward.register_autograd(_tp_bwd_backward, setup_context=_tp_bwd_setup)
+
+
+# ---------------------------------------------------------------------------
+# fused convolution
+# ---------------------------------------------------------------------------
+
+
+def _conv_checks(e: KernelEntry, L1_in, L2_in, W, rows, cols, perm, L3_grad=None):
+    nodes = L1_in.shape[0] if L1_in.dim() > 0 else -1
+    nnz = rows.shape[0] if rows.dim() > 0 else -1
+    check_tensor(L1_in, [nodes, e.L1], e.dtype, "L1_in")
+    check_tensor(L2_in, [nnz, e.L2], e.dtype, "L2_in")
+    check_tensor(W, _wshape(e, nnz), e.dtype, "W")
+    if L3_grad is not None:
+        check_tensor(L3_grad, [nodes, e.L3], e.dtype, "L3_grad")
+    check_tensor(rows, [nnz], torch.int64, "rows")
+    check_tensor(cols, [nnz], torch.int64, "cols")
+    if e.deterministic:
+        check_tensor(perm, [nnz], torch.int64, "transpose perm")
+    elif torch.are_deterministic_algorithms_enabled():
+        # counterpart of at::globalContext().alertNotDeterministic (torch_core.hpp:448)
+        msg = ("OpenEquivariance_conv_atomic does not have a deterministic implementation, but you set "
+               "'torch.use_deterministic_algorithms(True)'. Use TensorProductConv(..., deterministic=True).")
+        if torch.is_deterministic_algorithms_warn_only_enabled():
+            import warnings
+            warnings.warn(msg)
+        else:
+            raise RuntimeError(msg)
+    return nodes, nnz
+
+
+@torch.library.custom_op("oeq_amd::conv_forward", mutates_args=(), device_types="cuda")
+def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows: torch.Tensor,
+                 cols: torch.Tensor, transpose_perm: torch.Tensor, kid: int) -> torch.Tensor:
+    e = get_entry(kid)
+    nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm)
+    x, y, w = L1_in.contiguous(), L2_in.contiguous(), W.contiguous()
+    r, c = rows.contiguous(), cols.contiguous()
+    out = x.new_empty((nodes, e.L3))
+    with torch.cuda.device(x.device):
+        ks = e.kernels()
+        nb = ks.conv_forward_workspace_bytes(nodes, nnz)
+        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
+        ks.conv_forward(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), r.data_ptr(),
+                        c.data_ptr(), ws.data_ptr() if nb else 0, nb, _stream())
+    return out
+
+
+@conv_forward.register_fake
+def _(L1_in, L2_in, W, rows, cols, transpose_perm, kid):
+    e = get_entry(kid)
+    return L1_in.new_empty((L1_in.shape[0], e.L3))
+
+
+@torch.library.custom_op("oeq_amd::conv_backward", mutates_args=(), device_types="cuda")
+def conv_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_grad: torch.Tensor,
+                  rows: torch.Tensor, cols: torch.Tensor, transpose_perm: torch.Tensor,
+                  kid: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    e = get_entry(kid)
+    nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm, L3_grad)
+    x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
+    r, c, p = rows.contiguous(), cols.contiguous(), transpose_perm.contiguous()
+    dx, dy, dw = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w)
+    with torch.cuda.device(x.device):
+        ks = e.kernels()
+        nb = ks.conv_backward_workspace_bytes(nodes, nnz)
+        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
+        ks.conv_backward(nodes, nnz, x.data_ptr(), dx.data_ptr(), y.data_ptr(), dy.data_ptr(), w.data_ptr(),
+                         dw.data_ptr(), g.data_ptr(), r.data_ptr(), c.data_ptr(),
+                         p.data_ptr() if e.deterministic else 0, ws.data_ptr() if nb else 0, nb, _stream())
+    return dx, dy, dw
+
+
+@conv_backward.register_fake
+def _(L1_in, L2_in, W, L3_grad, rows, cols, transpose_perm, kid):
+    return torch.empty_like(L1_in), torch.empty_like(L2_in), torch.empty_like(W)
+
+
+def _conv_fwd_setup(ctx, inputs, output):
+    ctx.kid = inputs[6]
+    ctx.save_for_backward(*inputs[:6])
+
+
+def _conv_fwd_backward(ctx, grad):
+    x, y, w, rows, cols, perm = ctx.saved_tensors
+    dx, dy, dw = conv_backward(x, y, w, grad, rows, cols, perm, ctx.kid)
+    return dx, dy, dw, None, None, None, None
+
+
+conv_forward.register_autograd(_conv_fwd_backward, setup_context=_conv_fwd_setup)
+
+
+def _conv_bwd_setup(ctx, inputs, output):
+    ctx.kid = inputs[7]
+    ctx.save_for_backward(*inputs[:7])
+
+
+def _conv_bwd_backward(ctx, ddx, ddy, ddw):
+    x, y, w, g, rows, cols, perm = ctx.saved_tensors
+    kid = ctx.kid
+    ddx, ddy, ddw = _zeros_if_none(ddx, x), _zeros_if_none(ddy, y), _zeros_if_none(ddw, w)
+    dx1, _, dw1 = conv_backward(x, ddy, w, g, rows, cols, perm, kid)
+    dx2, dy2, _ = conv_backward(x, y, ddw, g, rows, cols, perm, kid)
+    _, dy3, dw3 = conv_backward(ddx, y, w, g, rows, cols, perm, kid)
+    gg = (conv_forward(ddx, y, w, rows, cols, perm, kid) + conv_forward(x, ddy, w, rows, cols, perm, kid)
+          + conv_forward(x, y, ddw, rows, cols, perm, kid))
+    return dx1 + dx2, dy2 + dy3, dw1 + dw3, gg, None, None, None, None
+
+
+conv_backward.register_autograd(_conv_bwd_backward, setup_context=_conv_bwd_setup)
+
+
+# Mixed precision: the kernels are compiled for one dtype; under autocast the
+# ops run in that dtype (cf. the reference's register_autocast to float32,
+# _torch/TensorProduct.py:362-374).
+def _register_autocast():
+    for op in (tp_forward, tp_backward, conv_forward, conv_backward):
+        try:
+            op.register_autocast("cuda", torch.float32)
+        except Exception:  # older/newer torch without this hook: ops still validate dtypes
+            pass
+
+
+_register_autocast()

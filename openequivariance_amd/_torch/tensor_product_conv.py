@@ -1,0 +1,136 @@
+"""``TensorProductConv``: fused CG tensor product + scatter-sum over a graph.
+
+Drop-in for the reference class
+(openequivariance/openequivariance/_torch/TensorProductConv.py:32-278):
+``forward(X, Y, W, rows, cols, sender_perm=None)`` with ``rows`` = receivers and
+``cols`` = senders; ``deterministic=True`` needs row-sorted edges and the
+permutation that lists them in sender-major order.
+
+Unlike the reference, the deterministic backward does not assume a symmetric
+sparsity pattern, and the module holds no workspace of its own (scratch memory
+is allocated per call from torch's stream-ordered allocator), so two streams
+may use one module concurrently.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..codegen.lower import lower
+from ..core.spec import TPProblem
+from . import ops
+from .utils import compute_units, oeq_to_torch_dtype, torch_to_oeq_dtype
+
+
+def build_conv_module(problem: TPProblem, deterministic: bool):
+    low = lower(problem)
+    if low.mode == "uvu":
+        from ..codegen import uvu
+        return uvu.conv_module(low, deterministic, compute_units())
+    raise NotImplementedError("TensorProductConv supports 'uvu' problems only in this package")
+
+
+class TensorProductConv(torch.nn.Module):
+    r"""Computes :math:`z_i = \sum_{(i,j,e)} W_e (x_j \otimes_{CG} y_e)` over the
+    edges of a directed graph.
+
+    :param problem: specification of the tensor product.
+    :param deterministic: ``False``: any edge order, floating-point atomics.
+           ``True``: receiver-sorted CSR walk with fixed summation order
+           (bit-identical from run to run). *Default*: ``False``.
+    :param kahan: compensated summation; not implemented here (raises).
+    :param use_opaque: deprecated, ignored.
+    """
+
+    def __init__(self, problem: TPProblem, *, deterministic: bool = False, kahan: bool = False,
+                 torch_op: bool = True, use_opaque: bool = False):
+        torch.nn.Module.__init__(self)
+        self.input_args = {"problem": problem, "deterministic": deterministic, "kahan": kahan,
+                           "torch_op": torch_op, "use_opaque": use_opaque}
+        self._init_class()
+
+    def _init_class(self):
+        problem: TPProblem = self.input_args["problem"].clone()
+        deterministic = bool(self.input_args["deterministic"])
+        if self.input_args["kahan"]:
+            assert deterministic, "kahan=True requires deterministic=True"
+            raise NotImplementedError("Kahan-compensated accumulation is not implemented in this package")
+        if deterministic:
+            assert not problem.shared_weights, "Deterministic convolution does not support shared weights"
+        self.config = problem
+        self.deterministic = deterministic
+        low = lower(problem)
+        self._low = low
+        self.L1, self.L2, self.L3 = problem.irreps_in1, problem.irreps_in2, problem.irreps_out
+        self.L3_dim = low.L3
+        self.weight_numel = problem.weight_numel
+        entry = ops.KernelEntry(
+            lambda p=problem, d=deterministic: build_conv_module(p, d), low.L1, low.L2, low.L3, low.WN,
+            low.shared_weights, oeq_to_torch_dtype(problem.irrep_dtype), deterministic=deterministic,
+        )
+        self.kid = ops.register_entry(entry)
+        self._dummy_perm = None
+
+    def to(self, *args, **kwargs):
+        _device, dtype, _nb, _fmt = torch._C._nn._parse_to(*args, **kwargs)
+        if dtype is not None and dtype.is_floating_point:
+            updated = self.input_args["problem"].clone()
+            updated.irrep_dtype = torch_to_oeq_dtype(dtype)
+            updated.weight_dtype = torch_to_oeq_dtype(dtype)
+            self.input_args["problem"] = updated
+            self._init_class()
+        torch.nn.Module.to(self, *args, **kwargs)
+        return self
+
+    def _apply(self, fn, recurse=True):
+        if getattr(self, "_applying", False):
+            return super()._apply(fn, recurse)
+        current = oeq_to_torch_dtype(self.input_args["problem"].irrep_dtype)
+        probe = fn(torch.tensor(0.0, dtype=current))
+        if probe.dtype != current and probe.dtype.is_floating_point:
+            self._applying = True
+            try:
+                self.to(probe.dtype)
+            finally:
+                self._applying = False
+        return super()._apply(fn, recurse)
+
+    def __getstate__(self):
+        return self.input_args
+
+    def __setstate__(self, state):
+        torch.nn.Module.__init__(self)
+        self.input_args = state
+        self._init_class()
+
+    def reorder_weights_from_e3nn(self, weights, has_batch_dim: bool = True):
+        return weights
+
+    def reorder_weights_to_e3nn(self, weights, has_batch_dim: bool = True):
+        return weights
+
+    @staticmethod
+    def name():
+        return "LoopUnrollConv"
+
+    def forward(self, X: torch.Tensor, Y: torch.Tensor, W: torch.Tensor, rows: torch.Tensor, cols: torch.Tensor,
+                sender_perm: Optional[torch.Tensor] = None) -> torch.Tensor:
+        r"""
+        :param X: ``[|V|, irreps_in1.dim]`` node features
+        :param Y: ``[|E|, irreps_in2.dim]`` edge features
+        :param W: ``[|E|, weight_numel]`` (or ``[weight_numel]`` with shared weights)
+        :param rows: ``[|E|]`` int64 receiver of each edge (sorted when ``deterministic``)
+        :param cols: ``[|E|]`` int64 sender of each edge
+        :param sender_perm: ``[|E|]`` int64 permutation listing the edges in
+               sender-major order; required when ``deterministic``
+        :return: ``[|V|, irreps_out.dim]``
+        """
+        if sender_perm is None:
+            if self.deterministic:
+                raise RuntimeError("Shape mismatch for tensor 'transpose perm'. deterministic=True needs sender_perm")
+            if self._dummy_perm is None or self._dummy_perm.device != rows.device:
+                self._dummy_perm = torch.zeros(1, dtype=torch.int64, device=rows.device)
+            sender_perm = self._dummy_perm
+        return ops.conv_forward(X, Y, W, rows, cols, sender_perm, self.kid)

@@ -1,0 +1,164 @@
+"""Lower a TPProblem to the flat tables the HIP emitters work from.
+
+This is the planner of this package. Where the reference splits
+multiplicities into warp-sized chunks and packs instructions into shared-memory
+segments (openequivariance/openequivariance/core/ComputationSchedule.py:185-649),
+the gfx950 plan is: lanes of a wave64 are channels ``u`` of one row; rows narrower
+than a wave are packed several to a wave; rows wider than a wave are split into
+64-channel chunks owned by different waves of the same block; outputs that are
+accumulated over many edges stay in registers, grouped into "segments" that fit
+a register budget.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import List, Tuple
+
+import numpy as np
+
+from ..core.cg import sparse_cg
+from ..core.spec import TPProblem
+
+
+def filter_and_analyze_problem(problem: TPProblem) -> dict:
+    """Reject what the kernels do not cover; same rules and messages as the
+    reference (openequivariance/openequivariance/core/utils.py:81-117)."""
+    first = problem.instructions[0].connection_mode if len(problem.instructions) else None
+    for i, inst in enumerate(problem.instructions):
+        assert inst.connection_mode == first, (
+            f"All instructions must have the same connection mode, got {inst.connection_mode} and {first}"
+        )
+        assert inst.has_weight, f"All instructions must have trainable weights, got {inst.has_weight} at index {i}"
+    assert len(problem.instructions) > 0, "Tensor product has no valid instructions!"
+    assert first in ["uvu", "uvw"], f"Connection mode must be 'uvu' or 'uvw', got {first}"
+    if problem.layout == "ir_mul":
+        assert first == "uvu", "layout='ir_mul' is only supported for pure 'uvu' problems"
+    assert problem.irrep_dtype == problem.weight_dtype, (
+        f"irrep_dtype and weight_dtype must be the same, got {problem.irrep_dtype} and {problem.weight_dtype}"
+    )
+    assert not problem.internal_weights, (
+        f"Openequivariance does not support internal weights, got {problem.internal_weights}"
+    )
+    return {"is_uvw": first == "uvw"}
+
+
+@dataclass
+class Block:
+    off: int
+    mul: int
+    l: int
+
+    @property
+    def d(self) -> int:
+        return 2 * self.l + 1
+
+
+@dataclass
+class Path:
+    index: int
+    i1: int
+    i2: int
+    io: int
+    woff: int
+    coeff: float
+    nnz: List[Tuple[int, int, int, float]]  # (i, j, k, coeff * C[i,j,k]) sorted by (j, i, k)
+    l: Tuple[int, int, int] = (0, 0, 0)
+
+
+@dataclass
+class Lowered:
+    mode: str
+    ctype: str
+    elem_size: int
+    shared_weights: bool
+    in1: List[Block]
+    in2: List[Block]
+    out: List[Block]
+    paths: List[Path]
+    L1: int
+    L2: int
+    L3: int
+    WN: int
+    label: str = ""
+    # lane mapping
+    lanes_per_row: int = 64
+    rows_per_wave: int = 1
+    n_chunks: int = 1
+    max_u: int = 1
+    total_nnz: int = 0
+
+    def flops(self, direction: str) -> int:
+        """Reference FLOP convention (benchmark/metrics.py:49-94,
+        core/ConvolutionBase.py:14-54): 3 per CG non-zero forward, 9 backward,
+        times mul1*mul2, plus the weight application."""
+        per_nz = 3 if direction == "forward" else 9
+        total = 0
+        for p in self.paths:
+            a, b, o = self.in1[p.i1], self.in2[p.i2], self.out[p.io]
+            total += per_nz * len(p.nnz) * a.mul * b.mul
+            if direction == "forward":
+                if self.mode == "uvu":
+                    total += o.mul * o.d
+                else:
+                    total += a.mul * b.mul * o.d * o.mul
+        return total
+
+
+def _blocks(irreps) -> List[Block]:
+    out, off = [], 0
+    for mul, ir in irreps:
+        out.append(Block(off, mul, ir.l))
+        off += mul * ir.dim
+    return out
+
+
+def _pow2ceil(n: int) -> int:
+    return 1 << max(0, (n - 1).bit_length())
+
+
+def lower(problem: TPProblem) -> Lowered:
+    info = filter_and_analyze_problem(problem)
+    if problem.layout != "mul_ir":
+        raise NotImplementedError("layout='ir_mul' is not implemented in this package yet")
+    dtype = np.dtype(problem.irrep_dtype)
+    if dtype == np.float32:
+        ctype, es = "float", 4
+    elif dtype == np.float64:
+        ctype, es = "double", 8
+    else:
+        raise AssertionError(f"unsupported irrep dtype {dtype}")
+
+    in1, in2, out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)
+    mode = "uvw" if info["is_uvw"] else "uvu"
+    paths, woff = [], 0
+    for idx, ins in enumerate(problem.instructions):
+        a, b, o = in1[ins.i_in1], in2[ins.i_in2], out[ins.i_out]
+        if mode == "uvu":
+            assert o.mul == a.mul, "'uvu' needs mul_out == mul_in1"
+        nnz = sparse_cg(a.l, b.l, o.l, scale=ins.path_weight)
+        paths.append(Path(idx, ins.i_in1, ins.i_in2, ins.i_out, woff, ins.path_weight, nnz, (a.l, b.l, o.l)))
+        woff += math.prod(ins.path_shape)
+    assert woff == problem.weight_numel
+
+    low = Lowered(
+        mode=mode, ctype=ctype, elem_size=es, shared_weights=bool(problem.shared_weights),
+        in1=in1, in2=in2, out=out, paths=paths,
+        L1=problem.irreps_in1.dim, L2=problem.irreps_in2.dim, L3=problem.irreps_out.dim,
+        WN=problem.weight_numel, label=problem.label,
+    )
+    used_mul = [in1[p.i1].mul for p in paths]
+    low.max_u = max(used_mul)
+    low.lanes_per_row = 64 if low.max_u > 32 else _pow2ceil(low.max_u)
+    low.rows_per_wave = 64 // low.lanes_per_row
+    low.n_chunks = (low.max_u + 63) // 64
+    low.total_nnz = sum(len(p.nnz) for p in paths)
+    return low
+
+
+def float_literal(v: float, ctype: str) -> str:
+    """Exact C++17 hex-float literal of ``v`` rounded to ``ctype``."""
+    if ctype == "float":
+        return float(np.float32(v)).hex() + "f"
+    return float(v).hex()

@@ -1,0 +1,169 @@
+"""Ready-made tensor-product problems.
+
+Constructors with the same names and instruction/irrep ordering as the
+reference's problem zoo (openequivariance/openequivariance/benchmark/problems.py:14-33,
+122-196, 292-330), plus the five benchmark configurations of this package.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import numpy as np
+
+from .spec import Irrep, Irreps, TPProblem
+
+
+class FullyConnectedTPProblem(TPProblem):
+    """Every allowed (in1, in2, out) triple gets one 'uvw' path
+    (problems.py:14-33): ``i_1`` outer, ``i_2`` middle, ``i_out`` inner."""
+
+    def __init__(self, irreps_in1, irreps_in2, irreps_out, **kwargs) -> None:
+        a, b, o = Irreps(irreps_in1), Irreps(irreps_in2), Irreps(irreps_out)
+        paths = []
+        for i1, (_, ir1) in enumerate(a):
+            for i2, (_, ir2) in enumerate(b):
+                allowed = list(ir1 * ir2)
+                for io, (_, iro) in enumerate(o):
+                    if iro in allowed:
+                        paths.append((i1, i2, io, "uvw", True, 1.0))
+        super().__init__(a, b, o, paths, **kwargs)
+
+
+class ChannelwiseTPP(TPProblem):
+    """MACE/NequIP-style per-channel ('uvu') product (problems.py:122-170).
+
+    A path (i, j -> ir_out) is kept iff ``ir_out`` occurs in the target
+    ``irreps_out``; every kept path owns a separate output block of
+    multiplicity ``mul_i``. Blocks are then stably sorted by ``(l, p)`` and
+    the instruction list by output index, which also fixes the weight order.
+    """
+
+    def __init__(
+        self,
+        irreps_in1,
+        irreps_in2,
+        irreps_out,
+        label: Optional[str] = None,
+        irrep_dtype=np.float32,
+        weight_dtype=np.float32,
+    ):
+        a, b, target = Irreps(irreps_in1), Irreps(irreps_in2), Irreps(irreps_out)
+        blocks, paths = [], []
+        for i, (mul, ir_in) in enumerate(a):
+            for j, (_, ir_edge) in enumerate(b):
+                for ir_out in ir_in * ir_edge:
+                    if ir_out in target:
+                        paths.append((i, j, len(blocks), "uvu", True))
+                        blocks.append((mul, ir_out))
+        ordered, new_index, _ = Irreps(blocks).sort()
+        paths = sorted(((i, j, new_index[k], m, t) for i, j, k, m, t in paths), key=lambda t: t[2])
+        super().__init__(
+            a,
+            b,
+            ordered,
+            paths,
+            internal_weights=False,
+            shared_weights=False,
+            label=label,
+            irrep_dtype=irrep_dtype,
+            weight_dtype=weight_dtype,
+        )
+
+
+class SingleInstruction(TPProblem):
+    """One instruction ``(0, 0, 0, mode, True)`` (problems.py:173-196)."""
+
+    def __init__(self, irreps_in1, irreps_in2, irreps_in3, mode: str, label: Optional[str] = None, **kwargs):
+        kwargs.setdefault("internal_weights", False)
+        kwargs.setdefault("shared_weights", False)
+        super().__init__(
+            Irreps(irreps_in1), Irreps(irreps_in2), Irreps(irreps_in3), [(0, 0, 0, mode, True)], label=label, **kwargs
+        )
+
+
+FCTPP = FullyConnectedTPProblem
+CTPP = ChannelwiseTPP
+
+
+def mace_problems():
+    """problems.py:292-309."""
+    return [
+        CTPP("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x2e+128x3o", "mace-large"),
+        CTPP("128x0e+128x1o", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x2e", "mace-medium"),
+    ]
+
+
+def nequip_problems():
+    """problems.py:312-345."""
+    return [
+        CTPP(
+            "32x0o + 32x0e + 32x1o + 32x1e + 32x2o + 32x2e",
+            "0e + 1o + 2e",
+            "32x0o + 32x0e + 32x1o + 32x1e + 32x2o + 32x2e",
+            "nequip-lips",
+        ),
+        CTPP("64x0o + 64x0e + 64x1o + 64x1e", "0e + 1o", "64x0o + 64x0e + 64x1o + 64x1e", "nequip-revmd17-aspirin"),
+        CTPP(
+            "64x0o + 64x0e + 64x1o + 64x1e + 64x2o + 64x2e",
+            "0e + 1o + 2e",
+            "64x0o + 64x0e + 64x1o + 64x1e + 64x2o + 64x2e",
+            "nequip-revmd17-toluene",
+        ),
+        CTPP(
+            "64x0o + 64x0e + 64x1o + 64x1e + 64x2o + 64x2e + 64x3o + 64x3e",
+            "0e + 1o + 2e + 3o",
+            "64x0o + 64x0e + 64x1o + 64x1e + 64x2o + 64x2e + 64x3o + 64x3e",
+            "nequip-revmd17-benzene",
+        ),
+        CTPP("32x0o + 32x0e + 32x1o + 32x1e", "0e + 1o", "32x0o + 32x0e + 32x1o + 32x1e", "nequip-water"),
+    ]
+
+
+# ---------------------------------------------------------------------------
+# The five benchmark configurations
+# ---------------------------------------------------------------------------
+
+_DT = {"float32": np.float32, "float64": np.float64, np.float32: np.float32, np.float64: np.float64}
+
+
+def _natural_parity_target(lmax: int) -> str:
+    return "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+
+
+def config1_single_uvu(dtype=np.float32) -> TPProblem:
+    """1x2e (x) 1x3e -> 1x2e, one 'uvu' instruction, per-row weights."""
+    return TPProblem(
+        "1x2e", "1x3e", "1x2e", [(0, 0, 0, "uvu", True)],
+        shared_weights=False, internal_weights=False, label="cfg1-single-uvu",
+        irrep_dtype=_DT[dtype], weight_dtype=_DT[dtype],
+    )
+
+
+def config2_nequip_uvu(dtype=np.float32) -> TPProblem:
+    """32x{0e,1o,2e} (x) SH(lmax 3) -> all natural-parity outputs with l<=2
+    (13 'uvu' paths, one output block per path)."""
+    return CTPP("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e+1x3o", _natural_parity_target(2),
+                "cfg2-nequip-uvu", _DT[dtype], _DT[dtype])
+
+
+def config3_mace_uvu(dtype=np.float32) -> TPProblem:
+    """128x{0e,1o,2e,3o} (x) SH(lmax 3) -> all natural-parity outputs with
+    l<=3 (23 'uvu' paths; L1=2048, L3=12672, weight_numel=2944)."""
+    return CTPP("128x0e+128x1o+128x2e+128x3o", "1x0e+1x1o+1x2e+1x3o", _natural_parity_target(3),
+                "cfg3-mace-uvu", _DT[dtype], _DT[dtype])
+
+
+def config4_uvw_shared(dtype=np.float32) -> TPProblem:
+    """64x{0e,1o,2e} (x) {0e,1o,2e} -> 64x{0e,1o,2e}, fully connected 'uvw',
+    one shared weight tensor (11 paths, weight_numel=45056)."""
+    return FCTPP("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e",
+                 shared_weights=True, internal_weights=False, label="cfg4-uvw-shared",
+                 irrep_dtype=_DT[dtype], weight_dtype=_DT[dtype])
+
+
+def config5_mace_conv(dtype=np.float32) -> TPProblem:
+    """The config-3 problem, used as a fused graph convolution."""
+    p = config3_mace_uvu(dtype)
+    p.label = "cfg5-mace-conv"
+    return p

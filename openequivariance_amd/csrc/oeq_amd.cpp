@@ -1,0 +1,377 @@
+// liboeq_amd.so: host runtime behind the C ABI declared in include/oeq_amd.h.
+//
+// Host-only translation unit: compiles HIP source with hiprtc, loads the code
+// object once per device, and enqueues the generated kernels on the caller's
+// stream. The kernel argument lists used here are the contract the Python
+// code generator (openequivariance_amd/codegen) emits against.
+#include "oeq_amd.h"
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[2048];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                  \
+    do {                                                                               \
+        hipError_t e_ = (expr);                                                        \
+        if (e_ != hipSuccess)                                                          \
+            return fail(OEQ_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_));   \
+    } while (0)
+
+constexpr int kMaxDevices = 16;
+
+struct RoleInfo {
+    bool present = false;
+    std::string name;
+    unsigned block = 0;
+    unsigned units_per_block = 1;
+    unsigned max_blocks = 0;
+};
+
+struct DeviceSlot {
+    hipModule_t module = nullptr;
+    hipFunction_t fn[OEQ_ROLE_COUNT] = {};
+};
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+struct oeq_kernels {
+    std::vector<char> code;
+    oeq_problem_dims dims{};
+    RoleInfo roles[OEQ_ROLE_COUNT];
+    std::mutex mu;
+    DeviceSlot slots[kMaxDevices];
+
+    // Resolve the function for `role` on the current device (loading the code
+    // object there on first use).
+    int function(int role, hipFunction_t* out) {
+        if (role < 0 || role >= OEQ_ROLE_COUNT || !roles[role].present)
+            return fail(OEQ_ERR_INVALID, "kernel role %d is not part of this kernel set", role);
+        int dev = 0;
+        HIP_TRY(hipGetDevice(&dev));
+        if (dev < 0 || dev >= kMaxDevices) return fail(OEQ_ERR_INVALID, "device index %d out of range", dev);
+        std::lock_guard<std::mutex> lock(mu);
+        DeviceSlot& s = slots[dev];
+        if (!s.module) {
+            HIP_TRY(hipModuleLoadData(&s.module, code.data()));
+            for (int r = 0; r < OEQ_ROLE_COUNT; ++r) {
+                if (!roles[r].present) continue;
+                hipError_t e = hipModuleGetFunction(&s.fn[r], s.module, roles[r].name.c_str());
+                if (e != hipSuccess) {
+                    (void)hipModuleUnload(s.module);
+                    s.module = nullptr;
+                    return fail(OEQ_ERR_HIP, "kernel '%s' not found in code object: %s", roles[r].name.c_str(),
+                                hipGetErrorString(e));
+                }
+            }
+        }
+        *out = s.fn[role];
+        return OEQ_OK;
+    }
+
+    unsigned grid_for(int role, int64_t units) const {
+        const RoleInfo& r = roles[role];
+        int64_t blocks = (units + r.units_per_block - 1) / r.units_per_block;
+        if (blocks < 1) blocks = 1;
+        if (r.max_blocks && blocks > (int64_t)r.max_blocks) blocks = r.max_blocks;
+        if (blocks > 0x7fffffffLL) blocks = 0x7fffffffLL;
+        return (unsigned)blocks;
+    }
+
+    int launch(int role, int64_t units, void** args, void* stream) {
+        hipFunction_t fn = nullptr;
+        int rc = function(role, &fn);
+        if (rc) return rc;
+        unsigned grid = grid_for(role, units);
+        HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, roles[role].block, 1, 1, 0, (hipStream_t)stream, args, nullptr));
+        return OEQ_OK;
+    }
+
+    int fill_zero(void* p, size_t bytes, void* stream) {
+        if (bytes == 0) return OEQ_OK;
+        int64_t n = (int64_t)bytes;
+        void* args[] = {&p, &n};
+        return launch(OEQ_ROLE_FILL_ZERO, (n + 15) / 16, args, stream);
+    }
+
+    int segment_ptr(int64_t n_items, int64_t n_segments, const int64_t* keys, const int64_t* perm, int64_t* ptr,
+                    void* stream) {
+        void* args[] = {&n_items, &n_segments, &keys, &perm, &ptr};
+        return launch(OEQ_ROLE_SEGMENT_PTR, n_items + 1, args, stream);
+    }
+};
+
+extern "C" {
+
+const char* oeq_last_error(void) { return g_error.c_str(); }
+int oeq_abi_version(void) { return 1; }
+
+int oeq_get_device_props(int device, oeq_device_props* out) {
+    if (!out) return fail(OEQ_ERR_INVALID, "oeq_get_device_props: out is NULL");
+    hipDeviceProp_t p;
+    HIP_TRY(hipGetDeviceProperties(&p, device));
+    std::memset(out, 0, sizeof(*out));
+    std::snprintf(out->name, sizeof(out->name), "%s", p.name);
+    std::string arch = p.gcnArchName;
+    size_t colon = arch.find(':');
+    if (colon != std::string::npos) arch.resize(colon);
+    std::snprintf(out->arch, sizeof(out->arch), "%s", arch.c_str());
+    out->wave_size = p.warpSize;
+    out->compute_units = p.multiProcessorCount;
+    out->lds_per_block = (int32_t)p.sharedMemPerBlock;
+    out->max_threads_per_block = p.maxThreadsPerBlock;
+    out->clock_khz = p.clockRate;
+    out->l2_bytes = p.l2CacheSize;
+    out->total_mem = (int64_t)p.totalGlobalMem;
+    return OEQ_OK;
+}
+
+void oeq_free(void* p) { std::free(p); }
+
+int oeq_jit_compile(const char* source, const char* arch, const char* const* options, int n_options, void** code,
+                    size_t* code_size) {
+    if (!source || !arch || !code || !code_size) return fail(OEQ_ERR_INVALID, "oeq_jit_compile: NULL argument");
+    *code = nullptr;
+    *code_size = 0;
+    hiprtcProgram prog;
+    hiprtcResult r = hiprtcCreateProgram(&prog, source, "oeq_kernels.hip", 0, nullptr, nullptr);
+    if (r != HIPRTC_SUCCESS) return fail(OEQ_ERR_COMPILE, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+    std::vector<std::string> opts;
+    opts.push_back(std::string("--offload-arch=") + arch);
+    for (int i = 0; i < n_options; ++i) opts.emplace_back(options[i]);
+    std::vector<const char*> copts;
+    for (auto& o : opts) copts.push_back(o.c_str());
+    r = hiprtcCompileProgram(prog, (int)copts.size(), copts.data());
+    if (r != HIPRTC_SUCCESS) {
+        size_t n = 0;
+        hiprtcGetProgramLogSize(prog, &n);
+        std::string log(n, '\0');
+        if (n) hiprtcGetProgramLog(prog, &log[0]);
+        hiprtcDestroyProgram(&prog);
+        g_error = std::string("hiprtc compile failed (") + hiprtcGetErrorString(r) + "):\n" + log;
+        return OEQ_ERR_COMPILE;
+    }
+    size_t n = 0;
+    r = hiprtcGetCodeSize(prog, &n);
+    if (r != HIPRTC_SUCCESS || n == 0) {
+        hiprtcDestroyProgram(&prog);
+        return fail(OEQ_ERR_COMPILE, "hiprtcGetCodeSize: %s", hiprtcGetErrorString(r));
+    }
+    void* buf = std::malloc(n);
+    if (!buf) {
+        hiprtcDestroyProgram(&prog);
+        return fail(OEQ_ERR_NOMEM, "out of host memory for %zu-byte code object", n);
+    }
+    r = hiprtcGetCode(prog, (char*)buf);
+    hiprtcDestroyProgram(&prog);
+    if (r != HIPRTC_SUCCESS) {
+        std::free(buf);
+        return fail(OEQ_ERR_COMPILE, "hiprtcGetCode: %s", hiprtcGetErrorString(r));
+    }
+    *code = buf;
+    *code_size = n;
+    return OEQ_OK;
+}
+
+int oeq_kernels_create(const void* code, size_t code_size, const oeq_problem_dims* dims, const oeq_kernel_desc* descs,
+                       int n_descs, oeq_kernels** out) {
+    if (!code || !code_size || !dims || !descs || n_descs <= 0 || !out)
+        return fail(OEQ_ERR_INVALID, "oeq_kernels_create: NULL or empty argument");
+    if (dims->elem_size != 4 && dims->elem_size != 8)
+        return fail(OEQ_ERR_INVALID, "oeq_kernels_create: elem_size must be 4 or 8, got %d", dims->elem_size);
+    if (dims->L1_dim <= 0 || dims->L2_dim <= 0 || dims->L3_dim <= 0 || dims->weight_numel <= 0)
+        return fail(OEQ_ERR_INVALID, "oeq_kernels_create: non-positive problem dimension");
+    oeq_kernels* k = new (std::nothrow) oeq_kernels();
+    if (!k) return fail(OEQ_ERR_NOMEM, "oeq_kernels_create: out of memory");
+    k->code.assign((const char*)code, (const char*)code + code_size);
+    k->dims = *dims;
+    for (int i = 0; i < n_descs; ++i) {
+        const oeq_kernel_desc& d = descs[i];
+        if (d.role < 0 || d.role >= OEQ_ROLE_COUNT || !d.kernel_name || d.block_threads == 0 ||
+            d.block_threads > 1024 || d.units_per_block == 0) {
+            delete k;
+            return fail(OEQ_ERR_INVALID, "oeq_kernels_create: bad kernel descriptor %d", i);
+        }
+        RoleInfo& r = k->roles[d.role];
+        r.present = true;
+        r.name = d.kernel_name;
+        r.block = d.block_threads;
+        r.units_per_block = d.units_per_block;
+        r.max_blocks = d.max_blocks;
+    }
+    *out = k;
+    return OEQ_OK;
+}
+
+void oeq_kernels_destroy(oeq_kernels* k) {
+    if (!k) return;
+    for (auto& s : k->slots)
+        if (s.module) (void)hipModuleUnload(s.module);
+    delete k;
+}
+
+// ---------------------------------------------------------------------------
+// batched tensor product
+// ---------------------------------------------------------------------------
+
+int oeq_tp_forward(oeq_kernels* k, int64_t num_batch, const void* L1_in, const void* L2_in, const void* W, void* L3_out,
+                   void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_tp_forward: NULL kernel set");
+    if (num_batch < 0) return fail(OEQ_ERR_INVALID, "oeq_tp_forward: negative batch");
+    if (num_batch == 0) return OEQ_OK;
+    if (!L1_in || !L2_in || !W || !L3_out) return fail(OEQ_ERR_INVALID, "oeq_tp_forward: NULL buffer");
+    void* args[] = {&num_batch, &L1_in, &L2_in, &W, &L3_out};
+    return k->launch(OEQ_ROLE_TP_FORWARD, num_batch, args, stream);
+}
+
+size_t oeq_tp_backward_workspace_bytes(const oeq_kernels* k, int64_t num_batch) {
+    if (!k || !k->dims.shared_weights || !k->roles[OEQ_ROLE_TP_BACKWARD].present) return 0;
+    size_t rows = (size_t)k->grid_for(OEQ_ROLE_TP_BACKWARD, num_batch) * (size_t)k->dims.wpartial_per_block;
+    return align_up(rows * (size_t)k->dims.weight_numel * (size_t)k->dims.elem_size, 256);
+}
+
+int oeq_tp_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in, void* L1_grad, const void* L2_in,
+                    void* L2_grad, const void* W, void* W_grad, const void* L3_grad, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_tp_backward: NULL kernel set");
+    if (num_batch < 0) return fail(OEQ_ERR_INVALID, "oeq_tp_backward: negative batch");
+    if (!W_grad) return fail(OEQ_ERR_INVALID, "oeq_tp_backward: NULL W_grad");
+    const bool shared = k->dims.shared_weights != 0;
+    if (num_batch == 0) {
+        if (shared) return k->fill_zero(W_grad, (size_t)k->dims.weight_numel * k->dims.elem_size, stream);
+        return OEQ_OK;
+    }
+    if (!L1_in || !L1_grad || !L2_in || !L2_grad || !W || !L3_grad)
+        return fail(OEQ_ERR_INVALID, "oeq_tp_backward: NULL buffer");
+    size_t need = oeq_tp_backward_workspace_bytes(k, num_batch);
+    if (need && (!workspace || workspace_bytes < need))
+        return fail(OEQ_ERR_INVALID, "oeq_tp_backward: workspace too small (%zu < %zu bytes)", workspace_bytes, need);
+    void* wpartial = need ? workspace : nullptr;
+    void* args[] = {&num_batch, &L1_in, &L1_grad, &L2_in, &L2_grad, &W, &W_grad, &L3_grad, &wpartial};
+    int rc = k->launch(OEQ_ROLE_TP_BACKWARD, num_batch, args, stream);
+    if (rc || !shared) return rc;
+    // Second pass: sum the per-block partial weight gradients in block order.
+    int64_t n_partials = (int64_t)k->grid_for(OEQ_ROLE_TP_BACKWARD, num_batch) * k->dims.wpartial_per_block;
+    int64_t wn = k->dims.weight_numel;
+    void* rargs[] = {&n_partials, &wpartial, &W_grad, &wn};
+    return k->launch(OEQ_ROLE_TP_BACKWARD_WREDUCE, wn, rargs, stream);
+}
+
+// ---------------------------------------------------------------------------
+// fused graph convolution
+// ---------------------------------------------------------------------------
+
+size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    (void)nnz;
+    if (!k || !k->dims.deterministic) return 0;
+    return align_up((size_t)(node_count + 1) * sizeof(int64_t), 256);
+}
+
+size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    if (!k || !k->dims.deterministic) return 0;
+    size_t ptr_bytes = align_up((size_t)(node_count + 1) * sizeof(int64_t), 256);
+    size_t tmp_bytes = align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256);
+    return 2 * ptr_bytes + tmp_bytes;
+}
+
+int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
+                     const void* W, void* L3_out, const int64_t* rows, const int64_t* cols, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL kernel set");
+    if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: negative size");
+    if (node_count == 0) return OEQ_OK;
+    if (!L3_out) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL L3_out");
+    const size_t out_bytes = (size_t)node_count * k->dims.L3_dim * k->dims.elem_size;
+    if (nnz == 0) return k->fill_zero(L3_out, out_bytes, stream);
+    if (!L1_in || !L2_in || !W || !rows || !cols) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL buffer");
+    int64_t* rowptr = nullptr;
+    int rc;
+    if (k->dims.deterministic) {
+        size_t need = oeq_conv_forward_workspace_bytes(k, node_count, nnz);
+        if (!workspace || workspace_bytes < need)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_forward: workspace too small (%zu < %zu bytes)", workspace_bytes,
+                        need);
+        rowptr = (int64_t*)workspace;
+        rc = k->segment_ptr(nnz, node_count, rows, nullptr, rowptr, stream);
+        if (rc) return rc;
+    } else {
+        rc = k->fill_zero(L3_out, out_bytes, stream);
+        if (rc) return rc;
+    }
+    void* args[] = {&node_count, &nnz, &L1_in, &L2_in, &W, &L3_out, &rows, &cols, &rowptr};
+    return k->launch(OEQ_ROLE_CONV_FORWARD, k->dims.deterministic ? node_count : nnz, args, stream);
+}
+
+int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, void* L1_grad,
+                      const void* L2_in, void* L2_grad, const void* W, void* W_grad, const void* L3_grad,
+                      const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL kernel set");
+    if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: negative size");
+    const bool shared = k->dims.shared_weights != 0;
+    const size_t es = (size_t)k->dims.elem_size;
+    int rc;
+    if (shared) {
+        if (!W_grad) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL W_grad");
+        rc = k->fill_zero(W_grad, (size_t)k->dims.weight_numel * es, stream);
+        if (rc) return rc;
+    }
+    if (node_count == 0) return OEQ_OK;
+    if (!L1_grad) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL L1_grad");
+    const size_t dx_bytes = (size_t)node_count * k->dims.L1_dim * es;
+    if (nnz == 0) return k->fill_zero(L1_grad, dx_bytes, stream);
+    if (!L1_in || !L2_in || !L2_grad || !W || !W_grad || !L3_grad || !rows || !cols)
+        return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL buffer");
+
+    int64_t *rowptr = nullptr, *colptr = nullptr;
+    void* dx_tmp = nullptr;
+    if (k->dims.deterministic) {
+        if (!transpose_perm) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: deterministic mode needs transpose_perm");
+        size_t need = oeq_conv_backward_workspace_bytes(k, node_count, nnz);
+        if (!workspace || workspace_bytes < need)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: workspace too small (%zu < %zu bytes)", workspace_bytes,
+                        need);
+        size_t ptr_bytes = align_up((size_t)(node_count + 1) * sizeof(int64_t), 256);
+        rowptr = (int64_t*)workspace;
+        colptr = (int64_t*)((char*)workspace + ptr_bytes);
+        dx_tmp = (char*)workspace + 2 * ptr_bytes;
+        rc = k->segment_ptr(nnz, node_count, rows, nullptr, rowptr, stream);
+        if (rc) return rc;
+        rc = k->segment_ptr(nnz, node_count, cols, transpose_perm, colptr, stream);
+        if (rc) return rc;
+    } else {
+        rc = k->fill_zero(L1_grad, dx_bytes, stream);
+        if (rc) return rc;
+    }
+    void* args[] = {&node_count, &nnz,  &L1_in, &L1_grad, &L2_in,  &L2_grad, &W,
+                    &W_grad,     &L3_grad, &rows, &cols,    &rowptr, &dx_tmp};
+    rc = k->launch(OEQ_ROLE_CONV_BACKWARD, k->dims.deterministic ? node_count : nnz, args, stream);
+    if (rc || !k->dims.deterministic) return rc;
+    void* fargs[] = {&node_count, &nnz, &dx_tmp, &L1_grad, &transpose_perm, &colptr};
+    return k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
+}
+
+}  // extern "C"

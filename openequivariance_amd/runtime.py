@@ -1,0 +1,273 @@
+"""ctypes binding of liboeq_amd.so (the C ABI in include/oeq_amd.h) plus the
+kernel cache: source -> hiprtc code object -> loaded kernel set.
+
+Stands in for the reference's extension loader and kernel cache
+(openequivariance/openequivariance/_torch/extlib/__init__.py:36-204 and
+extension/torch_core.hpp:180-270). There is no CPU fallback: if the shared
+library is missing every entry point raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import subprocess
+import threading
+from pathlib import Path
+from typing import Dict, List, Optional, Sequence, Tuple
+
+_PKG_DIR = Path(__file__).resolve().parent
+_REPO_DIR = _PKG_DIR.parent
+_LIB_PATH = _PKG_DIR / "liboeq_amd.so"
+_SRC_PATH = _PKG_DIR / "csrc" / "oeq_amd.cpp"
+_INCLUDE_DIR = _REPO_DIR / "include"
+
+DEFAULT_ARCH = "gfx950"
+
+# Flags for every device compile. Packed-FP32 instruction selection is turned
+# off on purpose (scalar v_fma_f32 only).
+HIPRTC_OPTIONS = [
+    "-O3",
+    "--std=c++17",
+    "-ffp-contract=fast",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+ROLE_TP_FORWARD = 0
+ROLE_TP_BACKWARD = 1
+ROLE_CONV_FORWARD = 2
+ROLE_CONV_BACKWARD = 3
+ROLE_CONV_FIXUP_BACKWARD = 4
+ROLE_SEGMENT_PTR = 5
+ROLE_FILL_ZERO = 6
+ROLE_TP_BACKWARD_WREDUCE = 7
+
+
+class OeqError(RuntimeError):
+    pass
+
+
+class DeviceProps(ctypes.Structure):
+    _fields_ = [
+        ("name", ctypes.c_char * 256),
+        ("arch", ctypes.c_char * 64),
+        ("wave_size", ctypes.c_int32),
+        ("compute_units", ctypes.c_int32),
+        ("lds_per_block", ctypes.c_int32),
+        ("max_threads_per_block", ctypes.c_int32),
+        ("clock_khz", ctypes.c_int32),
+        ("l2_bytes", ctypes.c_int32),
+        ("total_mem", ctypes.c_int64),
+    ]
+
+
+class _KernelDesc(ctypes.Structure):
+    _fields_ = [
+        ("role", ctypes.c_int32),
+        ("kernel_name", ctypes.c_char_p),
+        ("block_threads", ctypes.c_uint32),
+        ("units_per_block", ctypes.c_uint32),
+        ("max_blocks", ctypes.c_uint32),
+    ]
+
+
+class _ProblemDims(ctypes.Structure):
+    _fields_ = [
+        ("L1_dim", ctypes.c_int64),
+        ("L2_dim", ctypes.c_int64),
+        ("L3_dim", ctypes.c_int64),
+        ("weight_numel", ctypes.c_int64),
+        ("elem_size", ctypes.c_int32),
+        ("shared_weights", ctypes.c_int32),
+        ("deterministic", ctypes.c_int32),
+        ("wpartial_per_block", ctypes.c_int32),
+    ]
+
+
+def build_library(verbose: bool = False) -> Path:
+    """Compile csrc/oeq_amd.cpp into liboeq_amd.so next to this file."""
+    cmd = [
+        "hipcc", "-O2", "-std=c++17", "-shared", "-fPIC", f"-I{_INCLUDE_DIR}",
+        str(_SRC_PATH), "-o", str(_LIB_PATH), "-lhiprtc",
+    ]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise OeqError(f"building liboeq_amd.so failed:\n{res.stdout}\n{res.stderr}")
+    if verbose:
+        print(" ".join(cmd))
+    return _LIB_PATH
+
+
+_lib = None
+_lib_lock = threading.Lock()
+
+_P = ctypes.c_void_p
+_I64 = ctypes.c_int64
+_SZ = ctypes.c_size_t
+
+EXPORTS = {
+    "oeq_get_device_props": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(DeviceProps)]),
+    "oeq_jit_compile": (ctypes.c_int, [ctypes.c_char_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_char_p),
+                                       ctypes.c_int, ctypes.POINTER(_P), ctypes.POINTER(_SZ)]),
+    "oeq_free": (None, [_P]),
+    "oeq_kernels_create": (ctypes.c_int, [_P, _SZ, ctypes.POINTER(_ProblemDims), ctypes.POINTER(_KernelDesc),
+                                          ctypes.c_int, ctypes.POINTER(_P)]),
+    "oeq_kernels_destroy": (None, [_P]),
+    "oeq_tp_forward": (ctypes.c_int, [_P, _I64, _P, _P, _P, _P, _P]),
+    "oeq_tp_backward": (ctypes.c_int, [_P, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "oeq_tp_backward_workspace_bytes": (_SZ, [_P, _I64]),
+    "oeq_conv_forward": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "oeq_conv_forward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_conv_backward": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "oeq_conv_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_last_error": (ctypes.c_char_p, []),
+    "oeq_abi_version": (ctypes.c_int, []),
+}
+
+
+def lib_path() -> Path:
+    return _LIB_PATH
+
+
+def load_library():
+    """Load liboeq_amd.so (building it first only if no built file exists)."""
+    global _lib
+    with _lib_lock:
+        if _lib is not None:
+            return _lib
+        if not _LIB_PATH.exists():
+            build_library()
+        lib = ctypes.CDLL(str(_LIB_PATH))
+        for name, (res, args) in EXPORTS.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+        return lib
+
+
+def _check(rc: int, what: str):
+    if rc != 0:
+        msg = load_library().oeq_last_error()
+        raise OeqError(f"{what} failed ({rc}): {msg.decode(errors='replace') if msg else ''}")
+
+
+def device_props(device: int = 0) -> DeviceProps:
+    props = DeviceProps()
+    _check(load_library().oeq_get_device_props(device, ctypes.byref(props)), "oeq_get_device_props")
+    return props
+
+
+# ---------------------------------------------------------------------------
+# compile + on-disk cache of code objects
+# ---------------------------------------------------------------------------
+
+
+def cache_dir() -> Path:
+    d = os.environ.get("OEQ_AMD_CACHE_DIR")
+    path = Path(d) if d else _PKG_DIR / "_kcache"
+    path.mkdir(parents=True, exist_ok=True)
+    return path
+
+
+def source_hash(source: str, arch: str = DEFAULT_ARCH, options: Optional[Sequence[str]] = None) -> str:
+    h = hashlib.sha256()
+    h.update(arch.encode())
+    h.update("\0".join(options if options is not None else HIPRTC_OPTIONS).encode())
+    h.update(source.encode())
+    return h.hexdigest()[:24]
+
+
+def compile_source(source: str, arch: str = DEFAULT_ARCH, options: Optional[Sequence[str]] = None,
+                   use_disk_cache: bool = True) -> bytes:
+    """HIP source -> code object bytes (hiprtc; needs no GPU)."""
+    opts = list(options if options is not None else HIPRTC_OPTIONS)
+    key = source_hash(source, arch, opts)
+    path = cache_dir() / f"{key}.hsaco"
+    if use_disk_cache and path.exists():
+        return path.read_bytes()
+    lib = load_library()
+    c_opts = (ctypes.c_char_p * len(opts))(*[o.encode() for o in opts])
+    code = _P()
+    size = _SZ()
+    rc = lib.oeq_jit_compile(source.encode(), arch.encode(), c_opts, len(opts), ctypes.byref(code), ctypes.byref(size))
+    _check(rc, "oeq_jit_compile")
+    try:
+        blob = ctypes.string_at(code.value, size.value)
+    finally:
+        lib.oeq_free(code)
+    if use_disk_cache:
+        tmp = path.with_suffix(f".tmp{os.getpid()}")
+        tmp.write_bytes(blob)
+        os.replace(tmp, path)
+    return blob
+
+
+class KernelSet:
+    """A loaded code object with its launch descriptors (oeq_kernels*)."""
+
+    def __init__(self, code: bytes, dims: dict, descs: List[Tuple[int, str, int, int, int]]):
+        lib = load_library()
+        self._lib = lib
+        self._names = [d[1].encode() for d in descs]
+        arr = (_KernelDesc * len(descs))()
+        for slot, (role, _name, block, upb, maxb), enc in zip(arr, descs, self._names):
+            slot.role, slot.kernel_name, slot.block_threads = role, enc, block
+            slot.units_per_block, slot.max_blocks = upb, maxb
+        pd = _ProblemDims(**dims)
+        handle = _P()
+        _check(lib.oeq_kernels_create(code, len(code), ctypes.byref(pd), arr, len(descs), ctypes.byref(handle)),
+               "oeq_kernels_create")
+        self.handle = handle
+        self.dims = dict(dims)
+
+    def __del__(self):
+        try:
+            if getattr(self, "handle", None):
+                self._lib.oeq_kernels_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+    # thin wrappers; pointers are ints (tensor.data_ptr()), stream is an int
+    def tp_forward(self, n, x, y, w, out, stream):
+        _check(self._lib.oeq_tp_forward(self.handle, n, x, y, w, out, stream), "oeq_tp_forward")
+
+    def tp_backward_workspace_bytes(self, n) -> int:
+        return self._lib.oeq_tp_backward_workspace_bytes(self.handle, n)
+
+    def tp_backward(self, n, x, dx, y, dy, w, dw, g, ws, ws_bytes, stream):
+        _check(self._lib.oeq_tp_backward(self.handle, n, x, dx, y, dy, w, dw, g, ws, ws_bytes, stream),
+               "oeq_tp_backward")
+
+    def conv_forward_workspace_bytes(self, nodes, nnz) -> int:
+        return self._lib.oeq_conv_forward_workspace_bytes(self.handle, nodes, nnz)
+
+    def conv_backward_workspace_bytes(self, nodes, nnz) -> int:
+        return self._lib.oeq_conv_backward_workspace_bytes(self.handle, nodes, nnz)
+
+    def conv_forward(self, nodes, nnz, x, y, w, out, rows, cols, ws, ws_bytes, stream):
+        _check(self._lib.oeq_conv_forward(self.handle, nodes, nnz, x, y, w, out, rows, cols, ws, ws_bytes, stream),
+               "oeq_conv_forward")
+
+    def conv_backward(self, nodes, nnz, x, dx, y, dy, w, dw, g, rows, cols, perm, ws, ws_bytes, stream):
+        _check(self._lib.oeq_conv_backward(self.handle, nodes, nnz, x, dx, y, dy, w, dw, g, rows, cols, perm, ws,
+                                           ws_bytes, stream), "oeq_conv_backward")
+
+
+_kernel_cache: Dict[str, KernelSet] = {}
+_kernel_cache_lock = threading.Lock()
+
+
+def get_kernel_set(source: str, dims: dict, descs: List[Tuple[int, str, int, int, int]],
+                   arch: str = DEFAULT_ARCH) -> KernelSet:
+    """Process-wide cache keyed by the source hash; compile happens under the lock
+    (as in the reference, torch_core.hpp:192-231), launches do not."""
+    key = source_hash(source, arch) + repr(sorted(dims.items())) + repr(descs)
+    with _kernel_cache_lock:
+        ks = _kernel_cache.get(key)
+        if ks is None:
+            ks = KernelSet(compile_source(source, arch), dims, descs)
+            _kernel_cache[key] = ks
+        return ks
