@@ -1,0 +1,284 @@
+"""HIP source generator for fully-connected ('uvw') tensor products.
+
+Replaces the reference's 'uvw' branch of the unrolled templates and its
+register-tiled warp matmul (openequivariance/openequivariance/templates/
+loop_unroll_tp.cuh:55-84, 217-272 and templates/wmm.cuh:1-87).
+
+Two kernel families are generated:
+
+* a general one (any multiplicities, per-row or shared weights): lanes are
+  input channels ``u`` for the CG contraction and for everything in the backward
+  pass; the forward channel mix runs with lanes = output channels ``w`` and reads
+  the per-``u`` intermediates back from LDS as broadcasts;
+* for shared weights with 64-wide channel blocks, an MFMA kernel (see
+  ``uvw_mfma.py``) that batches rows so that the channel mix is a dense GEMM.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, Tuple
+
+from .common import Src, prelude, utility_kernels
+from .lower import Lowered, Path, float_literal
+
+WAVES_PER_BLOCK = 4
+
+
+def _pow2ceil(n: int) -> int:
+    return 1 << max(0, (n - 1).bit_length())
+
+
+class UvwEmitter:
+    def __init__(self, low: Lowered):
+        assert low.mode == "uvw"
+        self.low = low
+        self.T = low.ctype
+        self.l2_pad = _pow2ceil(low.L2)
+        self.max_d3 = max(low.out[p.io].d for p in low.paths)
+
+    def lit(self, v: float) -> str:
+        return float_literal(v, self.T)
+
+    def _products(self, s: Src, p: Path) -> Dict[int, Tuple[str, bool]]:
+        b2 = self.low.in2[p.i2]
+        for j in sorted({j for _, j, _, _ in p.nnz}):
+            s(f"const T y{j} = yrow[{b2.off} + v * {b2.d} + {j}];")
+        names, out = {}, {}
+        for n, (i, j, k, c) in enumerate(p.nnz):
+            key = (self.lit(abs(c)), j)
+            if key not in names:
+                names[key] = f"q{len(names)}"
+                s(f"const T {names[key]} = T({key[0]}) * y{j};")
+            out[n] = (names[key], c < 0)
+        return out
+
+    def _row_loop_open(self, s: Src):
+        s("const int lane = oeq_lane();")
+        s("const int wave = oeq_wave();")
+        s(f"for (i64 base = (i64)blockIdx.x * {WAVES_PER_BLOCK}; base < num_batch; "
+          f"base += (i64)gridDim.x * {WAVES_PER_BLOCK}) {{")
+        s.level += 1
+        s("const i64 row = base + wave;")
+        s("const bool live = row < num_batch;")
+        s("const i64 rowc = live ? row : num_batch - 1;")
+
+    # ------------------------------------------------------------- forward
+    def emit_forward(self, s: Src):
+        low = self.low
+        block = 64 * WAVES_PER_BLOCK
+        s.open(
+            f'extern "C" __global__ __launch_bounds__({block}) void forward(i64 num_batch, '
+            "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, T* __restrict__ L3_out)"
+        )
+        s(f"__shared__ T s_t[{WAVES_PER_BLOCK}][{self.max_d3}][64];")
+        self._row_loop_open(s)
+        s(f"const T* xrow = L1_in + rowc * {low.L1};")
+        s(f"const T* yrow = L2_in + rowc * {low.L2};")
+        s(f"const T* wrow = W{'' if low.shared_weights else f' + rowc * {low.WN}'};")
+        s(f"T* zrow = L3_out + rowc * {low.L3};")
+        for io, bo in enumerate(low.out):
+            paths = [p for p in low.paths if p.io == io]
+            s(f"// ---- out[{io}]: {bo.mul} x l={bo.l}")
+            s.open(f"for (int wc = 0; wc < {bo.mul}; wc += 64)")
+            s("const int w = wc + lane;")
+            s(f"T acc[{bo.d}];")
+            for k in range(bo.d):
+                s(f"acc[{k}] = T(0);")
+            for p in paths:
+                b1, b2 = low.in1[p.i1], low.in2[p.i2]
+                s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l}) {b1.mul}x{b2.mul}->{bo.mul}")
+                s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
+                s.open(f"for (int uc = 0; uc < {b1.mul}; uc += 64)")
+                s.open("")
+                s("const int u = uc + lane;")
+                s(f"T x[{b1.d}];")
+                s.open(f"if (u < {b1.mul})")
+                for i in range(b1.d):
+                    s(f"x[{i}] = xrow[{b1.off} + u * {b1.d} + {i}];")
+                s.close(" else {")
+                s.level += 1
+                for i in range(b1.d):
+                    s(f"x[{i}] = T(0);")
+                s.close()
+                prods = self._products(s, p)
+                started = set()
+                for n, (i, j, k, c) in enumerate(p.nnz):
+                    q, neg = prods[n]
+                    if k not in started:
+                        s(f"T t{k} = {'-' if neg else ''}{q} * x[{i}];")
+                        started.add(k)
+                    else:
+                        s(f"t{k} {'-=' if neg else '+='} {q} * x[{i}];")
+                s("__syncthreads();")
+                for k in range(bo.d):
+                    s(f"s_t[wave][{k}][lane] = {'t%d' % k if k in started else 'T(0)'};")
+                s("__syncthreads();")
+                s.close()
+                s(f"const int nu = ({b1.mul} - uc < 64) ? {b1.mul} - uc : 64;")
+                s(f"const T* wp = wrow + {p.woff} + ((i64)uc * {b2.mul} + v) * {bo.mul} + w;")
+                s.open(f"if (w < {bo.mul})")
+                s.open("for (int uu = 0; uu < nu; ++uu)")
+                s(f"const T wv = wp[(i64)uu * {b2.mul * bo.mul}];")
+                for k in range(bo.d):
+                    s(f"acc[{k}] += wv * s_t[wave][{k}][uu];")
+                s.close()
+                s.close()
+                s.close()
+                s.close()
+            s.open(f"if (live && w < {bo.mul})")
+            for k in range(bo.d):
+                s(f"zrow[{bo.off} + w * {bo.d} + {k}] = acc[{k}];")
+            s.close()
+            s.close()
+        s.close()
+        s.close()
+        return block
+
+    # ------------------------------------------------------------ backward
+    def emit_backward(self, s: Src):
+        low = self.low
+        shared = low.shared_weights
+        block = 64 * WAVES_PER_BLOCK
+        s.open(
+            f'extern "C" __global__ __launch_bounds__({block}) void backward(i64 num_batch, '
+            "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
+            "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
+            "const T* __restrict__ L3_grad, T* __restrict__ wpartial)"
+        )
+        if shared:
+            s(f"T* prow = wpartial + ((i64)blockIdx.x * {WAVES_PER_BLOCK} + oeq_wave()) * {low.WN};")
+            s("bool first = true;")
+        self._row_loop_open(s)
+        s(f"const T* xrow = L1_in + rowc * {low.L1};")
+        s(f"const T* yrow = L2_in + rowc * {low.L2};")
+        s(f"const T* wrow = W{'' if shared else f' + rowc * {low.WN}'};")
+        s(f"const T* grow = L3_grad + rowc * {low.L3};")
+        s(f"T* dxrow = L1_grad + rowc * {low.L1};")
+        if not shared:
+            s(f"T* dwrow = W_grad + rowc * {low.WN};")
+        s(f"T dy[{self.l2_pad}];")
+        s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+        for i1, b1 in enumerate(low.in1):
+            paths = [p for p in low.paths if p.i1 == i1]
+            s(f"// ---- in1[{i1}]: {b1.mul} x l={b1.l}")
+            s.open(f"for (int uc = 0; uc < {b1.mul}; uc += 64)")
+            s("const int u = uc + lane;")
+            s(f"const bool uok = u < {b1.mul};")
+            s(f"T x[{b1.d}], dx[{b1.d}];")
+            for i in range(b1.d):
+                s(f"x[{i}] = uok ? xrow[{b1.off} + u * {b1.d} + {i}] : T(0); dx[{i}] = T(0);")
+            for p in paths:
+                b2, bo = low.in2[p.i2], low.out[p.io]
+                s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
+                s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
+                prods = self._products(s, p)
+                s(f"const i64 wbase = {p.woff} + ((i64)u * {b2.mul} + v) * {bo.mul};")
+                # G_k = sum_w W[u,v,w] * g[w,k]
+                for k in range(bo.d):
+                    s(f"T G{k} = T(0);")
+                s.open("if (uok)")
+                s.open(f"for (int w = 0; w < {bo.mul}; ++w)")
+                s("const T wv = wrow[wbase + w];")
+                for k in range(bo.d):
+                    s(f"G{k} += wv * grow[{bo.off} + w * {bo.d} + {k}];")
+                s.close()
+                s.close()
+                fstart = set()
+                for n, (i, j, k, c) in enumerate(p.nnz):
+                    q, neg = prods[n]
+                    s(f"dx[{i}] {'-=' if neg else '+='} {q} * G{k};")
+                    if k not in fstart:
+                        s(f"T f{k} = {'-' if neg else ''}{q} * x[{i}];")
+                        fstart.add(k)
+                    else:
+                        s(f"f{k} {'-=' if neg else '+='} {q} * x[{i}];")
+                pair = {}
+                for n, (i, j, k, c) in enumerate(p.nnz):
+                    if (i, k) not in pair:
+                        pair[(i, k)] = f"xg{len(pair)}"
+                        s(f"const T {pair[(i, k)]} = x[{i}] * G{k};")
+                    s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * {pair[(i, k)]};")
+                # dW[u,v,w] = sum_k f_k * g[w,k]
+                s.open(f"if (uok{' && live' if not shared else ''})")
+                s.open(f"for (int w = 0; w < {bo.mul}; ++w)")
+                terms = [f"f{k} * grow[{bo.off} + w * {bo.d} + {k}]" for k in sorted(fstart)]
+                s(f"T dwv = {terms[0]};")
+                for t in terms[1:]:
+                    s(f"dwv += {t};")
+                if shared:
+                    s("if (!live) dwv = T(0);")
+                    s("prow[wbase + w] = first ? dwv : prow[wbase + w] + dwv;")
+                else:
+                    s("dwrow[wbase + w] = dwv;")
+                s.close()
+                s.close()
+                s.close()
+            s.open("if (live && uok)")
+            for i in range(b1.d):
+                s(f"dxrow[{b1.off} + u * {b1.d} + {i}] = dx[{i}];")
+            s.close()
+            if not paths:
+                pass
+            s.close()
+        if shared:
+            s("first = false;")
+        # dY: butterfly over the 64 lanes
+        n = self.l2_pad
+        s(f"T rv[{n}];")
+        for j in range(n):
+            s(f"rv[{j}] = dy[{j}];")
+        s("int dyidx = 0;")
+        cur, dup, m = n, 0, 32
+        while m >= 1:
+            if cur > 1:
+                half = cur // 2
+                s.open("")
+                s(f"const bool hi = (lane & {m}) != 0;")
+                for j in range(half):
+                    s(f"{{ const T keep = hi ? rv[{j + half}] : rv[{j}]; const T send = hi ? rv[{j}] : rv[{j + half}]; "
+                      f"rv[{j}] = keep + __shfl_xor(send, {m}); }}")
+                s(f"dyidx += hi ? {half} : 0;")
+                s.close()
+                cur = half
+            else:
+                s(f"rv[0] += __shfl_xor(rv[0], {m});")
+                dup |= m
+            m //= 2
+        s.open(f"if (live && (lane & {dup}) == 0)")
+        for j in range(cur):
+            s(f"if (dyidx + {j} < {low.L2}) L2_grad[rowc * {low.L2} + dyidx + {j}] = rv[{j}];")
+        s.close()
+        s.close()
+        if shared:
+            # a wave that saw no row still owns a partial row: clear it
+            s.open("if (first)")
+            s(f"for (int t = oeq_lane(); t < {low.WN}; t += 64) prow[t] = T(0);")
+            s.close()
+        s.close()
+        return block
+
+
+def tp_module(low: Lowered, compute_units: int = 256):
+    from .. import runtime as rt
+
+    if low.shared_weights:
+        from . import uvw_mfma
+        if uvw_mfma.supported(low):
+            return uvw_mfma.tp_module(low, compute_units)
+    em = UvwEmitter(low)
+    s = Src()
+    s(prelude(low.ctype))
+    s(utility_kernels())
+    blk_f = em.emit_forward(s)
+    blk_b = em.emit_backward(s)
+    max_blocks_b = compute_units * 2
+    descs = [
+        (rt.ROLE_TP_FORWARD, "forward", blk_f, WAVES_PER_BLOCK, compute_units * 16),
+        (rt.ROLE_TP_BACKWARD, "backward", blk_b, WAVES_PER_BLOCK, max_blocks_b if low.shared_weights else compute_units * 16),
+        (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
+        (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0),
+    ]
+    dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
+                shared_weights=int(low.shared_weights), deterministic=0,
+                wpartial_per_block=WAVES_PER_BLOCK if low.shared_weights else 0)
+    return s.text(), dims, descs

@@ -1,0 +1,103 @@
+"""The C-ABI library loads, exports every symbol the header declares, compiles
+generated sources for gfx950 with no GPU present and reports errors through
+return codes. No kernel is launched here."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from openequivariance_amd import runtime as rt
+from openequivariance_amd.codegen.lower import lower
+from openequivariance_amd.core import problems as P
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "oeq_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(oeq_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = rt.load_library()
+    names = _declared_functions()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/oeq_amd.h but not exported"
+    assert set(names) == set(rt.EXPORTS), "ctypes table and header disagree"
+    assert lib.oeq_abi_version() == 1
+
+
+def test_compile_error_is_reported_not_fatal():
+    with pytest.raises(rt.OeqError, match="hiprtc compile failed"):
+        rt.compile_source("this is not HIP", use_disk_cache=False)
+    blob = rt.compile_source('extern "C" __global__ void k(float* p) { p[threadIdx.x] = 1.0f; }', use_disk_cache=False)
+    assert blob[:4] == b"\x7fELF"
+
+
+def test_kernels_create_validates_arguments():
+    lib = rt.load_library()
+    dims = dict(L1_dim=4, L2_dim=1, L3_dim=4, weight_numel=1, elem_size=3, shared_weights=0, deterministic=0,
+                wpartial_per_block=0)
+    with pytest.raises(rt.OeqError, match="elem_size"):
+        rt.KernelSet(b"\x7fELFxxxx", dims, [(rt.ROLE_TP_FORWARD, "forward", 64, 1, 0)])
+    dims["elem_size"] = 4
+    with pytest.raises(rt.OeqError, match="descriptor"):
+        rt.KernelSet(b"\x7fELFxxxx", dims, [(rt.ROLE_TP_FORWARD, "forward", 0, 1, 0)])
+    ks = rt.KernelSet(b"\x7fELFxxxx", dims, [(rt.ROLE_TP_FORWARD, "forward", 64, 1, 0)])
+    # zero-sized work returns before touching the device; bad sizes are rejected
+    assert lib.oeq_tp_forward(ks.handle, 0, None, None, None, None, None) == 0
+    assert lib.oeq_tp_forward(ks.handle, -1, None, None, None, None, None) == -1
+    assert b"negative" in lib.oeq_last_error()
+    assert lib.oeq_tp_forward(None, 1, None, None, None, None, None) == -1
+    assert ks.conv_forward_workspace_bytes(10, 10) == 0
+    dims["deterministic"] = 1
+    ks2 = rt.KernelSet(b"\x7fELFxxxx", dims, [(rt.ROLE_CONV_FORWARD, "forward", 64, 1, 0)])
+    assert ks2.conv_forward_workspace_bytes(31, 10) == 256
+    assert ks2.conv_backward_workspace_bytes(31, 10) == 2 * 256 + 256  # 10*4*4 = 160 -> 256
+
+
+ALL = [P.config1_single_uvu, P.config2_nequip_uvu, P.config3_mace_uvu, P.config4_uvw_shared,
+       lambda: P.config3_mace_uvu(np.float64)]
+
+
+@pytest.mark.parametrize("make", ALL)
+def test_generated_tp_sources_compile_for_gfx950(make):
+    from openequivariance_amd._torch.tensor_product import build_tp_module
+    src, dims, descs = build_tp_module(make())
+    blob = rt.compile_source(src)
+    assert blob[:4] == b"\x7fELF"
+    names = {d[1] for d in descs}
+    assert {"forward", "backward"} <= names
+    for n in names:
+        assert n.encode() in blob
+
+
+@pytest.mark.parametrize("det", [False, True])
+@pytest.mark.parametrize("make", [P.config1_single_uvu, P.config2_nequip_uvu, P.config5_mace_conv,
+                                  lambda: P.config5_mace_conv(np.float64)])
+def test_generated_conv_sources_compile_for_gfx950(make, det):
+    from openequivariance_amd._torch.tensor_product_conv import build_conv_module
+    src, dims, descs = build_conv_module(make(), det)
+    blob = rt.compile_source(src)
+    names = {d[1] for d in descs}
+    assert {"forward", "backward"} <= names and (("fixup_backward" in names) == det)
+    assert dims["deterministic"] == int(det)
+    # generated code must not carry packed-FP32 arithmetic or anything CUDA-flavoured
+    assert "__syncwarp" not in src and "cuda" not in src.lower()
+
+
+def test_lowering_lane_mapping():
+    low = lower(P.config3_mace_uvu())
+    assert (low.lanes_per_row, low.rows_per_wave, low.n_chunks) == (64, 1, 2)
+    low = lower(P.config2_nequip_uvu())
+    assert (low.lanes_per_row, low.rows_per_wave, low.n_chunks) == (32, 2, 1)
+    low = lower(P.config1_single_uvu())
+    assert (low.lanes_per_row, low.rows_per_wave, low.n_chunks) == (1, 64, 1)
+    assert lower(P.config3_mace_uvu()).flops("forward") == 148224
+    assert lower(P.config3_mace_uvu()).flops("backward") == 406656
+    assert lower(P.config2_nequip_uvu()).flops("forward") == 13376
