@@ -1,0 +1,196 @@
+"""GPU parity of the fused convolution against the CPU oracle (tensor product
+on gathered sender rows + scatter-add), atomic and deterministic modes."""
+
+import numpy as np
+import pytest
+import torch
+
+import openequivariance_amd as oeq
+from openequivariance_amd.core import problems as P
+from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
+from oracle import e3nn_ref as R
+from gpu_util import err, tol_of
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph(n_nodes, deg, seed, punch_holes=True):
+    coords, rows, cols, vec = periodic_radius_graph(n_nodes, deg, 5.0, seed)
+    if punch_holes:  # node 3 fully isolated, node 5 receives nothing, edges no longer symmetric
+        keep = (rows != 3) & (cols != 3) & (rows != 5)
+        rows, cols = rows[keep], cols[keep]
+    return coords, rows, cols
+
+
+def _buffers(problem, n_nodes, E, seed):
+    rng = np.random.default_rng(seed)
+    dt = np.dtype(problem.irrep_dtype)
+    X = rng.uniform(size=(n_nodes, problem.irreps_in1.dim)).astype(dt)
+    Y = rng.uniform(size=(E, problem.irreps_in2.dim)).astype(dt)
+    W = rng.uniform(size=(problem.weight_numel,) if problem.shared_weights else (E, problem.weight_numel)).astype(dt)
+    G = rng.uniform(size=(n_nodes, problem.irreps_out.dim)).astype(dt)
+    return X, Y, W, G
+
+
+def _odd(shared):
+    return oeq.TPProblem("5x1e+3x2e", "2x1e+1x0e", "5x1e+3x2e+5x0e",
+                         [(0, 0, 0, "uvu", True), (0, 1, 0, "uvu", True), (1, 0, 1, "uvu", True),
+                          (0, 0, 2, "uvu", True)], shared_weights=shared, internal_weights=False, label="odd-uvu")
+
+
+CASES = [
+    ("cfg1", P.config1_single_uvu, 40, 6),
+    ("cfg2", P.config2_nequip_uvu, 60, 8),
+    ("cfg5-f32", P.config5_mace_conv, 50, 8),
+    ("cfg5-f64", lambda: P.config5_mace_conv(np.float64), 30, 6),
+    ("mace-large", lambda: P.mace_problems()[0], 40, 6),
+    ("odd", lambda: _odd(False), 40, 6),
+    ("odd-shared", lambda: _odd(True), 40, 6),
+]
+
+
+@pytest.mark.parametrize("name,make,n_nodes,deg", CASES, ids=[c[0] for c in CASES])
+def test_conv_matches_oracle(name, make, n_nodes, deg):
+    problem = make()
+    tol = tol_of(problem)
+    coords, rows, cols = _graph(n_nodes, deg, seed=0)
+    E = len(rows)
+    X, Y, W, G = _buffers(problem, n_nodes, E, seed=12345)
+    ref = R.Problem.from_spec(problem)
+    z_ref = R.conv_forward(ref, X, Y, W, rows, cols)
+    dx_ref, dy_ref, dw_ref = R.conv_backward(ref, X, Y, W, G, rows, cols)
+    assert np.all(z_ref[3] == 0) and np.all(z_ref[5] == 0) and np.all(dx_ref[3] == 0)
+    rng = np.random.default_rng(1)
+    modes = [False] if problem.shared_weights else [False, True]
+    for det in modes:
+        if det:
+            g = CoordGraph(coords, rows, cols)
+            order, r_, c_, perm = g.order, g.rows, g.cols, g.transpose_perm
+        else:
+            order = rng.permutation(E)
+            r_, c_, perm = rows[order], cols[order], None
+        conv = oeq.TensorProductConv(problem, deterministic=det)
+        tX = torch.tensor(X, device="cuda", requires_grad=True)
+        tY = torch.tensor(Y[order], device="cuda", requires_grad=True)
+        tW = torch.tensor(W if problem.shared_weights else W[order], device="cuda", requires_grad=True)
+        tr, tc = torch.tensor(r_, device="cuda"), torch.tensor(c_, device="cuda")
+        tp = torch.tensor(perm, device="cuda") if perm is not None else None
+        z = conv(tX, tY, tW, tr, tc, tp)
+        assert err(z, z_ref) <= tol, (name, det)
+        z.backward(torch.tensor(G, device="cuda"))
+        assert err(tX.grad, dx_ref) <= tol, (name, det)
+        assert err(tY.grad, dy_ref[order]) <= tol, (name, det)
+        wtol = tol * (np.sqrt(E) if problem.shared_weights else 1.0)
+        assert err(tW.grad, dw_ref if problem.shared_weights else dw_ref[order]) <= wtol, (name, det)
+
+
+def test_reference_toy_graph():
+    """The 3-node / 4-edge graph of the reference's tutorial
+    (tests/example_test.py:46-82): atomic and deterministic calls agree with the
+    oracle; sender_perm is the argsort by sender of the receiver-sorted edges."""
+    problem = P.config1_single_uvu()
+    rows = np.array([0, 1, 1, 2])
+    cols = np.array([1, 0, 2, 1])
+    rng = np.random.default_rng(0)
+    X, Y, W = (rng.uniform(size=s).astype(np.float32) for s in ((3, 5), (4, 7), (4, 1)))
+    z_ref = R.conv_forward(R.Problem.from_spec(problem), X, Y, W, rows, cols)
+    tX, tY, tW = (torch.tensor(a, device="cuda") for a in (X, Y, W))
+    tr, tc = torch.tensor(rows, device="cuda"), torch.tensor(cols, device="cuda")
+    z = oeq.TensorProductConv(problem, deterministic=False).forward(tX, tY, tW, tr, tc)
+    assert err(z, z_ref) <= 1e-5
+    sender_perm = torch.argsort(tc, stable=True)
+    z = oeq.TensorProductConv(problem, deterministic=True).forward(tX, tY, tW, tr, tc, sender_perm)
+    assert err(z, z_ref) <= 1e-5
+
+
+def test_deterministic_mode_is_bitwise_reproducible():
+    problem = P.config5_mace_conv()
+    coords, rows, cols = _graph(300, 16, seed=2, punch_holes=False)
+    g = CoordGraph(coords, rows, cols)
+    E = g.nnz
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    X = torch.randn(300, 2048, device="cuda", generator=gen, requires_grad=True)
+    Y = torch.randn(E, 16, device="cuda", generator=gen, requires_grad=True)
+    W = torch.randn(E, 2944, device="cuda", generator=gen, requires_grad=True)
+    G = torch.randn(300, 12672, device="cuda", generator=gen)
+    tr, tc, tp = (torch.tensor(a, device="cuda") for a in (g.rows, g.cols, g.transpose_perm))
+    conv = oeq.TensorProductConv(problem, deterministic=True)
+    results = []
+    for _ in range(5):
+        for t in (X, Y, W):
+            t.grad = None
+        z = conv(X, Y, W, tr, tc, tp)
+        z.backward(G)
+        results.append((z.detach().clone(), X.grad.clone(), Y.grad.clone(), W.grad.clone()))
+        torch.randn(1 << 22, device="cuda")  # unrelated work between runs
+    for other in results[1:]:
+        for a, b in zip(results[0], other):
+            assert torch.equal(a, b)
+    # atomic mode agrees with it to tolerance
+    conv_a = oeq.TensorProductConv(problem, deterministic=False)
+    za = conv_a(X, Y, W, tr, tc)
+    scale = results[0][0].abs().max()
+    assert (za - results[0][0]).abs().max() / scale <= 1e-5
+
+
+def test_no_edges_and_no_nodes():
+    problem = P.config1_single_uvu()
+    for det in (False, True):
+        conv = oeq.TensorProductConv(problem, deterministic=det)
+        e = torch.zeros(0, dtype=torch.int64, device="cuda")
+        X = torch.rand(4, 5, device="cuda", requires_grad=True)
+        Y = torch.rand(0, 7, device="cuda", requires_grad=True)
+        W = torch.rand(0, 1, device="cuda", requires_grad=True)
+        z = conv(X, Y, W, e, e, e if det else None)
+        assert z.shape == (4, 5) and torch.count_nonzero(z) == 0
+        z.backward(torch.ones_like(z))
+        assert torch.count_nonzero(X.grad) == 0
+
+
+def test_star_graph_closed_form():
+    """All edges into node 0: Z[0] is the plain sum of the per-edge products."""
+    problem = P.config2_nequip_uvu()
+    n, E = 9, 8
+    rows = np.zeros(E, dtype=np.int64)
+    cols = np.arange(1, n, dtype=np.int64)
+    X, Y, W, _ = _buffers(problem, n, E, seed=4)
+    tp = oeq.TensorProduct(problem)
+    msgs = tp(torch.tensor(X[cols], device="cuda"), torch.tensor(Y, device="cuda"), torch.tensor(W, device="cuda"))
+    conv = oeq.TensorProductConv(problem, deterministic=True)
+    tr, tc = torch.tensor(rows, device="cuda"), torch.tensor(cols, device="cuda")
+    z = conv(torch.tensor(X, device="cuda"), torch.tensor(Y, device="cuda"), torch.tensor(W, device="cuda"), tr, tc,
+             torch.arange(E, device="cuda"))
+    assert torch.count_nonzero(z[1:]) == 0
+    assert (z[0] - msgs.double().sum(0).float()).abs().max() / z[0].abs().max() <= 1e-5
+
+
+def test_conv_input_validation():
+    problem = P.config1_single_uvu()
+    conv = oeq.TensorProductConv(problem, deterministic=True)
+    X, Y, W = torch.rand(3, 5, device="cuda"), torch.rand(4, 7, device="cuda"), torch.rand(4, 1, device="cuda")
+    rows = torch.tensor([0, 1, 1, 2], device="cuda")
+    cols = torch.tensor([1, 0, 2, 1], device="cuda")
+    perm = torch.argsort(cols, stable=True)
+    conv(X, Y, W, rows, cols, perm)
+    with pytest.raises(RuntimeError, match="Shape mismatch"):
+        conv(X, Y[:3], W, rows, cols, perm)
+    with pytest.raises(RuntimeError, match="Shape mismatch"):
+        conv(X, Y, W, rows, cols, perm[:2])
+    with pytest.raises(RuntimeError, match="Dtype mismatch"):
+        conv(X, Y, W, rows.int(), cols, perm)
+    with pytest.raises(RuntimeError, match="is not on the GPU"):
+        conv(X, Y, W, rows.cpu(), cols, perm)
+
+
+def test_conv_double_backward_runs():
+    problem = P.config1_single_uvu(np.float64)
+    conv = oeq.TensorProductConv(problem, deterministic=True)
+    rows = torch.tensor([0, 1, 1, 2], device="cuda")
+    cols = torch.tensor([1, 0, 2, 1], device="cuda")
+    perm = torch.argsort(cols, stable=True)
+    X = torch.rand(3, 5, device="cuda", dtype=torch.float64, requires_grad=True)
+    Y = torch.rand(4, 7, device="cuda", dtype=torch.float64, requires_grad=True)
+    W = torch.rand(4, 1, device="cuda", dtype=torch.float64, requires_grad=True)
+    assert torch.autograd.gradcheck(lambda a, b, c: conv(a, b, c, rows, cols, perm), (X, Y, W), eps=1e-6, atol=1e-6)
+    assert torch.autograd.gradgradcheck(lambda a, b, c: conv(a, b, c, rows, cols, perm), (X, Y, W), eps=1e-6,
+                                        atol=1e-6)

@@ -1,0 +1,207 @@
+"""GPU parity of the batched tensor product against the CPU oracle, through
+the torch ops and directly through the C ABI. Tolerances: max normalised error
+<= 1e-5 (fp32) and <= 1e-12 (fp64) against the float64 oracle."""
+
+import numpy as np
+import pytest
+import torch
+
+import openequivariance_amd as oeq
+from openequivariance_amd.core import problems as P
+from oracle import e3nn_ref as R
+from gpu_util import err, to_gpu, tol_of, tp_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _odd_uvu(shared):
+    return oeq.TPProblem("5x1e+3x2e", "2x1e+1x0e", "5x1e+3x2e+5x0e",
+                         [(0, 0, 0, "uvu", True), (0, 1, 0, "uvu", True), (1, 0, 1, "uvu", True),
+                          (0, 0, 2, "uvu", True)], shared_weights=shared, internal_weights=False, label="odd-uvu")
+
+
+def _odd_uvw(shared):
+    return oeq.TPProblem("5x1e+3x2e+70x0e", "2x1e+1x0e", "7x1e+3x2e+100x0e",
+                         [(0, 0, 0, "uvw", True), (0, 1, 0, "uvw", True), (1, 0, 1, "uvw", True),
+                          (0, 0, 2, "uvw", True), (2, 1, 2, "uvw", True, 0.3)], shared_weights=shared,
+                         internal_weights=False, label="odd-uvw")
+
+
+CASES = [
+    ("cfg1-b1000", P.config1_single_uvu, 1000),
+    ("cfg1-b37", P.config1_single_uvu, 37),
+    ("cfg1-f64", lambda: P.config1_single_uvu(np.float64), 129),
+    ("cfg2", P.config2_nequip_uvu, 301),
+    ("cfg3-f32", P.config3_mace_uvu, 203),
+    ("cfg3-f64", lambda: P.config3_mace_uvu(np.float64), 101),
+    ("cfg4-shared", P.config4_uvw_shared, 257),
+    ("cfg4-f64", lambda: P.config4_uvw_shared(np.float64), 50),
+    ("mace-large", lambda: P.mace_problems()[0], 99),
+    ("nequip-aspirin", lambda: P.nequip_problems()[1], 99),
+    ("odd-uvu", lambda: _odd_uvu(False), 77),
+    ("odd-uvu-shared", lambda: _odd_uvu(True), 77),
+    ("wide-uvu-shared", lambda: oeq.TPProblem(
+        "100x1e+70x2e", "1x1e+1x0e", "100x1e+70x2e+100x0e",
+        [(0, 0, 0, "uvu", True), (0, 1, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 0, 2, "uvu", True)],
+        shared_weights=True, internal_weights=False), 77),
+    ("uvu-l5", lambda: P.SingleInstruction("33x5e", "1x3e", "33x5e", "uvu"), 40),
+    ("uvu-mul2", lambda: P.SingleInstruction("19x2e", "3x1e", "19x2e", "uvu"), 40),
+    ("uvu-mul2-big", lambda: P.SingleInstruction("4x1e", "12x1e", "4x1e", "uvu"), 40),
+    ("uvw-unshared", lambda: P.FullyConnectedTPProblem("16x0e+16x1o", "1x0e+1x1o", "16x0e+16x1o",
+                                                      shared_weights=False, internal_weights=False), 33),
+    ("odd-uvw", lambda: _odd_uvw(False), 21),
+    ("odd-uvw-shared", lambda: _odd_uvw(True), 21),
+]
+
+
+@pytest.mark.parametrize("name,make,B", CASES, ids=[c[0] for c in CASES])
+def test_forward_backward_match_oracle(name, make, B):
+    problem = make()
+    tol = tol_of(problem)
+    x, y, w, g = tp_inputs(problem, B, seed=12345)
+    ref = R.Problem.from_spec(problem)
+    z_ref = R.tp_forward(ref, x, y, w)
+    dx_ref, dy_ref, dw_ref = R.tp_backward(ref, x, y, w, g)
+    tp = oeq.TensorProduct(problem)
+    tx, ty, tw = to_gpu(x, y, w, requires_grad=True)
+    (tg,) = to_gpu(g)
+    z = tp(tx, ty, tw)
+    assert z.shape == (B, problem.irreps_out.dim)
+    assert err(z, z_ref) <= tol
+    z.backward(tg)
+    assert err(tx.grad, dx_ref) <= tol
+    assert err(ty.grad, dy_ref) <= tol
+    # a shared weight gradient sums `B` terms: allow the accumulated rounding of that sum
+    wtol = tol * (max(1.0, np.sqrt(B)) if problem.shared_weights else 1.0)
+    assert err(tw.grad, dw_ref) <= wtol
+
+
+def test_same_precision_reference_is_not_closer_by_accident():
+    """fp32 kernel vs the oracle evaluated in fp32: same order of error."""
+    problem = P.config3_mace_uvu()
+    x, y, w, g = tp_inputs(problem, 64, seed=1)
+    ref = R.Problem.from_spec(problem)
+    z32 = R.tp_forward(ref, x, y, w, dtype=np.float32)
+    tp = oeq.TensorProduct(problem)
+    z = tp(*to_gpu(x, y, w))
+    assert err(z, z32) <= 1e-5
+
+
+def test_c_abi_direct_call():
+    """Call oeq_tp_forward / oeq_tp_backward through ctypes with raw pointers."""
+    from openequivariance_amd import runtime as rt
+    from openequivariance_amd._torch.tensor_product import build_tp_module
+    problem = P.config2_nequip_uvu()
+    src, dims, descs = build_tp_module(problem)
+    ks = rt.get_kernel_set(src, dims, descs)
+    B = 123
+    x, y, w, g = tp_inputs(problem, B, seed=7)
+    tx, ty, tw, tg = to_gpu(x, y, w, g)
+    out = torch.empty(B, problem.irreps_out.dim, device="cuda")
+    dx, dy, dw = torch.empty_like(tx), torch.empty_like(ty), torch.empty_like(tw)
+    stream = torch.cuda.current_stream().cuda_stream
+    ks.tp_forward(B, tx.data_ptr(), ty.data_ptr(), tw.data_ptr(), out.data_ptr(), stream)
+    ks.tp_backward(B, tx.data_ptr(), dx.data_ptr(), ty.data_ptr(), dy.data_ptr(), tw.data_ptr(), dw.data_ptr(),
+                   tg.data_ptr(), 0, 0, stream)
+    torch.cuda.synchronize()
+    ref = R.Problem.from_spec(problem)
+    assert err(out, R.tp_forward(ref, x, y, w)) <= 1e-5
+    dx_ref, dy_ref, dw_ref = R.tp_backward(ref, x, y, w, g)
+    assert err(dx, dx_ref) <= 1e-5 and err(dy, dy_ref) <= 1e-5 and err(dw, dw_ref) <= 1e-5
+    # NULL buffers are refused with an error code, not a fault
+    with pytest.raises(rt.OeqError, match="NULL buffer"):
+        ks.tp_forward(B, 0, ty.data_ptr(), tw.data_ptr(), out.data_ptr(), stream)
+
+
+def test_empty_batch():
+    tp = oeq.TensorProduct(P.config1_single_uvu())
+    z = tp(torch.zeros(0, 5, device="cuda"), torch.zeros(0, 7, device="cuda"), torch.zeros(0, 1, device="cuda"))
+    assert z.shape == (0, 5)
+
+
+def test_full_size_properties_cfg3():
+    """At the benchmark batch the oracle is too slow: check size-independent
+    properties instead (agreement of a row sample with the oracle, linearity in
+    each argument, independence of rows from their neighbours)."""
+    problem = P.config3_mace_uvu()
+    B = 100000
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(B, 2048, device="cuda", generator=gen)
+    y = torch.randn(B, 16, device="cuda", generator=gen)
+    w = torch.randn(B, 2944, device="cuda", generator=gen)
+    tp = oeq.TensorProduct(problem)
+    z = tp(x, y, w)
+    idx = torch.tensor([0, 1, 63, 64, 4097, B // 2, B - 2, B - 1], device="cuda")
+    ref = R.Problem.from_spec(problem)
+    z_ref = R.tp_forward(ref, x[idx].cpu().numpy(), y[idx].cpu().numpy(), w[idx].cpu().numpy())
+    assert err(z[idx], z_ref) <= 1e-5
+    assert torch.equal(tp(x[idx], y[idx], w[idx]), z[idx])  # a row does not depend on its position
+    z2 = tp(2.0 * x, y, w)
+    assert torch.equal(z2, 2.0 * z)  # scaling by 2 is exact in binary floating point
+    z3 = tp(x, y, -w)
+    assert torch.equal(z3, -z)
+    assert torch.isfinite(z).all()
+
+
+def test_double_backward_matches_autograd_of_oracle_formula():
+    """Second derivatives come from compositions of the forward/backward ops;
+    compare with torch autograd through an einsum restatement in float64."""
+    problem = P.config1_single_uvu(np.float64)
+    B = 16
+    x, y, w, g = tp_inputs(problem, B, seed=3)
+    C = torch.tensor(R.wigner_3j_ref(2, 3, 2) * np.sqrt(5.0))
+
+    def ref_fn(tx, ty, tw):
+        return torch.einsum("ijk,zi,zj,z->zk", C, tx, ty, tw[:, 0])
+
+    tp = oeq.TensorProduct(problem)
+    outs = []
+    for fn, dev in ((ref_fn, "cpu"), (tp, "cuda")):
+        tx, ty, tw = (torch.tensor(a, device=dev, requires_grad=True) for a in (x, y, w))
+        tg = torch.tensor(g, device=dev, requires_grad=True)
+        z = fn(tx, ty, tw) if dev == "cuda" else fn(tx, ty, tw)
+        dx, dy, dw = torch.autograd.grad(z, (tx, ty, tw), tg, create_graph=True)
+        loss = (dx ** 2).sum() + (dy ** 2).sum() + (dw ** 2).sum()
+        second = torch.autograd.grad(loss, (tx, ty, tw, tg))
+        outs.append([t.detach().cpu().numpy() for t in second])
+    for a, b in zip(outs[1], outs[0]):
+        assert R.normalized_error(a, b) <= 1e-12
+
+
+def test_input_validation_messages():
+    tp = oeq.TensorProduct(P.config1_single_uvu())
+    x, y, w = (torch.rand(8, n, device="cuda") for n in (5, 7, 1))
+    tp(x, y, w)
+    with pytest.raises(RuntimeError, match="Shape mismatch"):
+        tp(x.unsqueeze(1), y, w)
+    with pytest.raises(RuntimeError, match="Shape mismatch"):
+        tp(x, y[:, :6], w)
+    with pytest.raises(RuntimeError, match="Shape mismatch"):
+        tp(x, y, torch.rand(9, 1, device="cuda"))
+    with pytest.raises(RuntimeError, match="Dtype mismatch"):
+        tp(x, y.to(torch.bfloat16), w)
+    with pytest.raises(RuntimeError, match="Dtype mismatch"):
+        tp(x.double(), y, w)
+
+
+def test_module_to_dtype_respecialises():
+    tp = oeq.TensorProduct(P.config2_nequip_uvu())
+    tp = tp.to(torch.float64)
+    problem = P.config2_nequip_uvu(np.float64)
+    x, y, w, _ = tp_inputs(problem, 9, seed=5)
+    z = tp(*to_gpu(x, y, w))
+    assert z.dtype == torch.float64
+    assert err(z, R.tp_forward(R.Problem.from_spec(problem), x, y, w)) <= 1e-12
+
+
+def test_runs_on_a_side_stream():
+    tp = oeq.TensorProduct(P.config2_nequip_uvu())
+    problem = P.config2_nequip_uvu()
+    x, y, w, _ = tp_inputs(problem, 64, seed=9)
+    tx, ty, tw = to_gpu(x, y, w)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        z = tp(tx, ty, tw)
+    side.synchronize()
+    assert err(z, R.tp_forward(R.Problem.from_spec(problem), x, y, w)) <= 1e-5
