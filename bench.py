@@ -1,0 +1,227 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused equivariant graph convolution at MACE shape.
+
+One step = forward + backward of ``TensorProductConv`` (deterministic mode) on a
+synthetic periodic radius graph: N = 50000 nodes, mean degree ~32 (E ~ 1.6 M),
+X = 128x{0e,1o,2e,3o}, Y = spherical harmonics lmax 3, 23 'uvu' paths, fp32.
+All inputs are resident in HBM before the timed region starts. The atomic mode
+(shuffled edge order) is timed beside it and reported in ``modes``.
+
+Prints ONE JSON line (rank 0). ``value`` = edges per second of the whole step.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--nodes", type=int, default=50000)
+    ap.add_argument("--degree", type=float, default=32.0)
+    ap.add_argument("--atomic-steps", type=int, default=3)
+    ap.add_argument("--cpu-receivers", type=int, default=48, help="receivers in the CPU-baseline sub-graph (0 = skip)")
+    ap.add_argument("--no-atomic", action="store_true")
+    return ap.parse_args()
+
+
+def time_steps(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def cpu_baseline(problem, graph, Ysh, n_receivers, seed=0):
+    """e3nn-equivalent torch-CPU einsum + index_add (oracle/torch_ref.py), forward
+    and backward, on the sub-graph made of the first receivers and all their
+    edges; same problem, fp32, all host threads."""
+    import numpy as np
+    import torch
+    from oracle import e3nn_ref as R
+    from oracle.torch_ref import TorchConv
+
+    cores = os.cpu_count() or 1
+    threads = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(threads)
+    e_end = int(np.searchsorted(graph.rows, n_receivers, side="left"))
+    rows = torch.tensor(graph.rows[:e_end])
+    cols_np = graph.cols[:e_end]
+    # compact the senders that occur so the sample does not carry all 50000 rows of X
+    uniq, inv = np.unique(np.concatenate([cols_np, np.arange(n_receivers)]), return_inverse=True)
+    cols = torch.tensor(inv[:e_end])
+    n_local = len(uniq)
+    gen = torch.Generator().manual_seed(seed)
+    X = torch.randn(n_local, problem.irreps_in1.dim, generator=gen, requires_grad=True)
+    Y = torch.tensor(Ysh[:e_end], requires_grad=True)
+    W = torch.randn(e_end, problem.weight_numel, generator=gen, requires_grad=True)
+    conv = TorchConv(R.Problem.from_spec(problem), torch.float32)
+    # receivers keep their ids 0..n_receivers-1 only if those ids are the first n_receivers of uniq
+    recv_local = torch.tensor(np.searchsorted(uniq, graph.rows[:e_end]))
+
+    def step():
+        for t in (X, Y, W):
+            t.grad = None
+        Z = conv(X, Y, W, recv_local, cols)
+        Z.backward(torch.ones_like(Z))
+
+    step()
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or (time.perf_counter() - t0 < 10.0 and reps < 50):
+        step()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {
+        "value": e_end / dt, "unit": "edges/s", "cores": threads, "kind": "port",
+        "sample": f"fwd+bwd on the sub-graph of the first {n_receivers} receivers ({e_end} edges, {n_local} nodes), "
+                  f"torch-CPU einsum + index_add restatement of e3nn (e3nn not installed), fp32, {reps} reps",
+        "seconds_per_step": dt, "host_cpus": cores,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
+              "use --gpus 1. See DESIGN.md for how the path would shard.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import openequivariance_amd as oeq
+    from openequivariance_amd import runtime as rt
+    from openequivariance_amd._torch import ops
+    from openequivariance_amd.codegen.lower import lower
+    from openequivariance_amd.core import problems as P
+    from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
+    from openequivariance_amd.core.sh import spherical_harmonics
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU (there is no CPU fallback for the product path)"
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    problem = P.config5_mace_conv()
+    low = lower(problem)
+    L1, L2, L3, WN = low.L1, low.L2, low.L3, low.WN
+
+    coords, rows, cols, vec = periodic_radius_graph(args.nodes, args.degree, 5.0, seed=0)
+    graph = CoordGraph(coords, rows, cols, "periodic-radius")
+    N, E = graph.node_count, graph.nnz
+    Ysh = spherical_harmonics(3, vec).astype(np.float32)[graph.order]
+
+    gen = torch.Generator(device=dev).manual_seed(0)
+    X = torch.randn(N, L1, device=dev, generator=gen)
+    W = torch.randn(E, WN, device=dev, generator=gen)
+    G = torch.randn(N, L3, device=dev, generator=gen)
+    Y = torch.tensor(Ysh, device=dev)
+    tr, tc, tp = (torch.tensor(a, device=dev) for a in (graph.rows, graph.cols, graph.transpose_perm))
+
+    es = 4
+    fwd_bytes = (E * (L2 + WN) + N * (L1 + L3)) * es
+    bwd_bytes = (2 * E * (L2 + WN) + N * (L1 + L3) + N * L1) * es
+    fwd_flops, bwd_flops = low.flops("forward") + L3, low.flops("backward")  # per edge (conv adds the scatter)
+
+    # ---- deterministic mode: the timed K steps --------------------------------
+    conv = oeq.TensorProductConv(problem, deterministic=True)
+    kid = conv.kid
+
+    def step_det():
+        ops.conv_forward(X, Y, W, tr, tc, tp, kid)
+        ops.conv_backward(X, Y, W, G, tr, tc, tp, kid)
+
+    ms_det = time_steps(step_det, args.steps, args.warmup)
+
+    # per-kernel durations with HIP events on the launch stream, over K more steps
+    ks = ops.get_entry(kid).kernels()
+    ks.timing_enable(True)
+    for _ in range(args.steps):
+        step_det()
+    torch.cuda.synchronize()
+    kt = {name: ks.timing_collect(role) for name, role in
+          (("forward", rt.ROLE_CONV_FORWARD), ("backward", rt.ROLE_CONV_BACKWARD),
+           ("fixup_backward", rt.ROLE_CONV_FIXUP_BACKWARD), ("oeq_segment_ptr", rt.ROLE_SEGMENT_PTR))}
+    ks.timing_enable(False)
+    avg = {k: (v[0] / v[1] if v[1] else 0.0) for k, v in kt.items()}
+
+    # dominant kernel: conv `backward` (reads X[cols], Y, W, dZ; writes dY, dW and the per-edge dX terms)
+    bwd_kernel_bytes = (2 * E * (L2 + WN) + N * (L1 + L3)) * es
+    achieved = bwd_kernel_bytes / (avg["backward"] * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm", "kernel": "backward (TensorProductConv, deterministic)",
+        "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+        "traffic": None,
+        "algorithmic_bytes_per_launch": bwd_kernel_bytes, "avg_kernel_ms": avg["backward"],
+        "launches_timed": kt["backward"][1],
+    }
+
+    modes = {
+        "deterministic": {
+            "ms_per_step": ms_det, "edges_per_s": E / (ms_det * 1e-3),
+            "gflops": (fwd_flops + bwd_flops) * E / (ms_det * 1e-3) / 1e9,
+            "hbm_roofline_frac": (fwd_bytes + bwd_bytes) / (ms_det * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "kernel_ms": avg,
+        }
+    }
+
+    # ---- atomic mode, shuffled edge order ---------------------------------------
+    if not args.no_atomic:
+        perm = torch.randperm(E, device=dev, generator=gen)
+        Ya, Wa, ra, ca = Y[perm].contiguous(), W[perm].contiguous(), tr[perm].contiguous(), tc[perm].contiguous()
+        conv_a = oeq.TensorProductConv(problem, deterministic=False)
+        dummy = torch.zeros(1, dtype=torch.int64, device=dev)
+
+        def step_atomic():
+            ops.conv_forward(X, Ya, Wa, ra, ca, dummy, conv_a.kid)
+            ops.conv_backward(X, Ya, Wa, G, ra, ca, dummy, conv_a.kid)
+
+        ms_at = time_steps(step_atomic, args.atomic_steps, 1)
+        modes["atomic_shuffled"] = {
+            "ms_per_step": ms_at, "edges_per_s": E / (ms_at * 1e-3),
+            "gflops": (fwd_flops + bwd_flops) * E / (ms_at * 1e-3) / 1e9,
+            "hbm_roofline_frac": (fwd_bytes + bwd_bytes) / (ms_at * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "steps": args.atomic_steps,
+        }
+        del Ya, Wa
+
+    cpu = None
+    if args.cpu_receivers > 0:
+        cpu = cpu_baseline(problem, graph, Ysh, args.cpu_receivers)
+
+    out = {
+        "metric": "fused conv fwd+bwd edges/s at MACE shape (deterministic mode)",
+        "value": E / (ms_det * 1e-3), "unit": "edges/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_det,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "cfg5: TensorProductConv fwd+bwd, MACE shape 128x{0e,1o,2e,3o} x SH(lmax3), 23 uvu paths",
+                   "nodes": N, "edges": E, "L1": L1, "L2": L2, "L3": L3, "weight_numel": WN,
+                   "graph": "uniform points in a periodic cube, cutoff 5.0, directed both ways, seed 0"},
+        "gflops": modes["deterministic"]["gflops"],
+        "hbm_roofline_frac_step": modes["deterministic"]["hbm_roofline_frac"],
+        "algorithmic_bytes_per_edge": {"forward": fwd_bytes / E, "backward": bwd_bytes / E},
+        "flops_per_edge": {"forward": fwd_flops, "backward": bwd_flops},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "modes": modes,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -152,6 +152,14 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz,
                       void* workspace, size_t workspace_bytes, void* stream);
 size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
 
+/* ---- per-kernel timing --------------------------------------------------- */
+/* Replaces GPUTimer (extension/backend/backend_hip.hpp:67-101). While enabled,
+ * every kernel this set launches is bracketed by HIP events on the stream it is
+ * launched on. oeq_kernel_timing_collect() waits for the recorded launches of
+ * `role`, returns their summed duration and count, and forgets them. */
+int oeq_kernel_timing_enable(oeq_kernels* k, int enable);
+int oeq_kernel_timing_collect(oeq_kernels* k, int role, double* total_ms, int64_t* launches);
+
 /* ---- diagnostics -------------------------------------------------------- */
 const char* oeq_last_error(void);
 int oeq_abi_version(void);

@@ -54,6 +54,11 @@ struct DeviceSlot {
     hipFunction_t fn[OEQ_ROLE_COUNT] = {};
 };
 
+struct TimedLaunch {
+    int role;
+    hipEvent_t start, stop;
+};
+
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
@@ -64,6 +69,8 @@ struct oeq_kernels {
     RoleInfo roles[OEQ_ROLE_COUNT];
     std::mutex mu;
     DeviceSlot slots[kMaxDevices];
+    bool timing = false;
+    std::vector<TimedLaunch> timed;
 
     // Resolve the function for `role` on the current device (loading the code
     // object there on first use).
@@ -106,7 +113,20 @@ struct oeq_kernels {
         int rc = function(role, &fn);
         if (rc) return rc;
         unsigned grid = grid_for(role, units);
+        if (!timing) {
+            HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, roles[role].block, 1, 1, 0, (hipStream_t)stream, args,
+                                          nullptr));
+            return OEQ_OK;
+        }
+        // profiling mode: bracket this one kernel with events on its own stream
+        TimedLaunch t{role, nullptr, nullptr};
+        HIP_TRY(hipEventCreate(&t.start));
+        HIP_TRY(hipEventCreate(&t.stop));
+        HIP_TRY(hipEventRecord(t.start, (hipStream_t)stream));
         HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, roles[role].block, 1, 1, 0, (hipStream_t)stream, args, nullptr));
+        HIP_TRY(hipEventRecord(t.stop, (hipStream_t)stream));
+        std::lock_guard<std::mutex> lock(mu);
+        timed.push_back(t);
         return OEQ_OK;
     }
 
@@ -231,6 +251,37 @@ void oeq_kernels_destroy(oeq_kernels* k) {
     for (auto& s : k->slots)
         if (s.module) (void)hipModuleUnload(s.module);
     delete k;
+}
+
+int oeq_kernel_timing_enable(oeq_kernels* k, int enable) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_kernel_timing_enable: NULL kernel set");
+    std::lock_guard<std::mutex> lock(k->mu);
+    k->timing = enable != 0;
+    return OEQ_OK;
+}
+
+int oeq_kernel_timing_collect(oeq_kernels* k, int role, double* total_ms, int64_t* launches) {
+    if (!k || !total_ms || !launches) return fail(OEQ_ERR_INVALID, "oeq_kernel_timing_collect: NULL argument");
+    std::vector<TimedLaunch> mine, rest;
+    {
+        std::lock_guard<std::mutex> lock(k->mu);
+        for (auto& t : k->timed) (t.role == role ? mine : rest).push_back(t);
+        k->timed.swap(rest);
+    }
+    double sum = 0.0;
+    int rc = OEQ_OK;
+    for (auto& t : mine) {
+        float ms = 0.f;
+        hipError_t e = hipEventSynchronize(t.stop);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, t.start, t.stop);
+        if (e != hipSuccess) rc = fail(OEQ_ERR_HIP, "kernel timing failed: %s", hipGetErrorString(e));
+        sum += ms;
+        (void)hipEventDestroy(t.start);
+        (void)hipEventDestroy(t.stop);
+    }
+    *total_ms = sum;
+    *launches = (int64_t)mine.size();
+    return rc;
 }
 
 // ---------------------------------------------------------------------------

@@ -121,6 +121,9 @@ EXPORTS = {
     "oeq_conv_forward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_backward": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_conv_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_kernel_timing_enable": (ctypes.c_int, [_P, ctypes.c_int]),
+    "oeq_kernel_timing_collect": (ctypes.c_int, [_P, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                                                 ctypes.POINTER(_I64)]),
     "oeq_last_error": (ctypes.c_char_p, []),
     "oeq_abi_version": (ctypes.c_int, []),
 }
@@ -229,6 +232,16 @@ class KernelSet:
                 self.handle = None
         except Exception:
             pass
+
+    def timing_enable(self, on: bool):
+        _check(self._lib.oeq_kernel_timing_enable(self.handle, int(on)), "oeq_kernel_timing_enable")
+
+    def timing_collect(self, role: int) -> Tuple[float, int]:
+        """(summed milliseconds, launches) of the kernels of `role` recorded since the last call."""
+        ms, n = ctypes.c_double(), _I64()
+        _check(self._lib.oeq_kernel_timing_collect(self.handle, role, ctypes.byref(ms), ctypes.byref(n)),
+               "oeq_kernel_timing_collect")
+        return ms.value, n.value
 
     # thin wrappers; pointers are ints (tensor.data_ptr()), stream is an int
     def tp_forward(self, n, x, y, w, out, stream):
