@@ -83,6 +83,8 @@ typedef struct {
     uint32_t block_threads;
     uint32_t units_per_block;   /* rows / nodes / edges one block handles per sweep */
     uint32_t max_blocks;        /* 0 = one block per ceil(units/units_per_block) */
+    uint32_t grid_multiple;     /* 0/1 = none; else the grid is rounded up to a multiple of this (kernels that
+                                   remap blockIdx so that each XCD walks a contiguous range of units) */
 } oeq_kernel_desc;
 
 typedef struct {

@@ -11,15 +11,16 @@ loop_unroll_conv_det.cuh:96-293) with a different decomposition:
   by all channels (the row's Y) is wave-uniform when a row fills a wave;
 * the convolution keeps the receiver's output (forward) or output gradient
   (backward) in registers across all edges of that receiver (CSR walk), so Z and
-  dZ move once per node instead of once per edge;
+  dZ move once per node instead of once per edge, and the operands of the next
+  edge are fetched into a second register set while the current edge is computed;
 * dY is accumulated per lane over all paths and reduced once per row with a
   halving butterfly; nothing in deterministic mode uses atomics.
 """
 
 from __future__ import annotations
 
-from collections import OrderedDict
-from typing import Dict, List, Tuple
+import os
+from typing import Callable, Dict, List, Optional, Tuple
 
 from .common import Src, fixup_backward_kernel, prelude, utility_kernels
 from .lower import Lowered, Path, float_literal
@@ -29,6 +30,18 @@ UNROLL_V_LIMIT = 8
 
 def _pow2ceil(n: int) -> int:
     return 1 << max(0, (n - 1).bit_length())
+
+
+def tuning(defaults: dict) -> dict:
+    """Kernel-shape knobs; ``OEQ_AMD_TUNE="key=value,..."`` overrides them
+    (integers), which is how the defaults below were chosen on the GPU."""
+    out = dict(defaults)
+    for item in os.environ.get("OEQ_AMD_TUNE", "").split(","):
+        if "=" in item:
+            k, v = item.split("=", 1)
+            if k.strip() in out:
+                out[k.strip()] = int(v)
+    return out
 
 
 class UvuEmitter:
@@ -41,11 +54,12 @@ class UvuEmitter:
         self.R = low.rows_per_wave
         self.NCH = low.n_chunks
         self.used_in1 = sorted({p.i1 for p in low.paths})
+        self.used_out = sorted({p.io for p in low.paths})
         # output segments (register-resident accumulators of the conv forward)
         budget = max(1, acc_budget_words // self.words)
-        self.segments: List[List[int]] = []  # lists of out-block indices
+        self.segments: List[List[int]] = []
         cur, cur_sz = [], 0
-        for io in sorted({p.io for p in low.paths}):
+        for io in self.used_out:
             d = low.out[io].d
             if cur and cur_sz + d > budget:
                 self.segments.append(cur)
@@ -54,34 +68,63 @@ class UvuEmitter:
             cur_sz += d
         if cur:
             self.segments.append(cur)
-        self.untouched_out = [io for io in range(len(low.out)) if io not in {p.io for p in low.paths}]
-        self.g_resident = sum(low.out[io].d for io in {p.io for p in low.paths}) * self.words <= g_resident_words
+        self.seg_in1 = [sorted({p.i1 for p in low.paths if p.io in seg}) for seg in self.segments]
+        self.untouched_out = [io for io in range(len(low.out)) if io not in self.used_out]
+        self.g_resident = sum(low.out[io].d for io in self.used_out) * self.words <= g_resident_words
         self.l2_pad = _pow2ceil(low.L2)
+        # per-lane weight slots: one per (path, v), in path order
+        self.wslot: Dict[int, int] = {}
+        n = 0
+        for p in low.paths:
+            self.wslot[p.index] = n
+            n += low.in2[p.i2].mul
+        self.n_wslots = n
+        # operands of an edge can be fetched ahead into registers when every index is a constant
+        self.can_preload = (
+            all(low.in2[p.i2].mul <= UNROLL_V_LIMIT for p in low.paths) and low.L2 <= 32 and self.n_wslots <= 64
+        )
 
     # ------------------------------------------------------------------ utils
     def lit(self, v: float) -> str:
         return float_literal(v, self.T)
 
-    def _v_range(self, p: Path):
-        V = self.low.in2[p.i2].mul
-        return V
-
-    def _products(self, s: Src, p: Path, vexpr: str) -> Dict[int, Tuple[str, bool]]:
-        """Emit y loads and the distinct |c|*y_j products of a path. Returns
-        nnz index -> (operand name, negative)."""
+    # operand accessors -------------------------------------------------------
+    def _acc_pointer(self):
         low = self.low
-        b2 = low.in2[p.i2]
-        js = sorted({j for _, j, _, _ in p.nnz})
-        for j in js:
-            s(f"const T y{j} = yrow[{b2.off} + ({vexpr}) * {b2.d} + {j}];")
+
+        def y(p: Path, v: str, j: int) -> str:
+            b2 = low.in2[p.i2]
+            return f"yrow[{b2.off} + ({v}) * {b2.d} + {j}]"
+
+        def w(p: Path, v: str) -> str:
+            return f"((u < {low.in1[p.i1].mul}) ? wrow[{p.woff} + u * {low.in2[p.i2].mul} + ({v})] : T(0))"
+
+        return y, w
+
+    def _acc_preloaded(self, name: str = "d"):
+        low = self.low
+
+        def y(p: Path, v: str, j: int) -> str:
+            b2 = low.in2[p.i2]
+            return f"{name}.y[{b2.off + int(v) * b2.d + j}]"
+
+        def w(p: Path, v: str) -> str:
+            return f"{name}.w[{self.wslot[p.index] + int(v)}]"
+
+        return y, w
+
+    def _products(self, s: Src, p: Path, v: str, yacc) -> Dict[int, Tuple[str, bool]]:
+        """Emit the distinct |c|*y_j products of a path. Returns nnz index ->
+        (operand name, negative)."""
+        for j in sorted({j for _, j, _, _ in p.nnz}):
+            s(f"const T y{j} = {yacc(p, v, j)};")
         names: Dict[Tuple[str, int], str] = {}
         out = {}
         for n, (i, j, k, c) in enumerate(p.nnz):
             key = (self.lit(abs(c)), j)
             if key not in names:
-                nm = f"q{len(names)}"
-                names[key] = nm
-                s(f"const T {nm} = T({key[0]}) * y{j};")
+                names[key] = f"q{len(names)}"
+                s(f"const T {names[key]} = T({key[0]}) * y{j};")
             out[n] = (names[key], c < 0)
         return out
 
@@ -99,14 +142,8 @@ class UvuEmitter:
                 s(f"{dst}.b{b}[{i}] = T(0);")
             s.close()
 
-    def _struct_x(self, s: Src):
-        s("struct X_t {")
-        for b in self.used_in1:
-            s(f"    T b{b}[{self.low.in1[b].d}];")
-        s("};")
-
-    def _for_v(self, s: Src, p: Path, body):
-        V = self._v_range(p)
+    def _for_v(self, s: Src, p: Path, body: Callable[[str], None]):
+        V = self.low.in2[p.i2].mul
         if V <= UNROLL_V_LIMIT:
             for v in range(V):
                 s.open("")
@@ -118,10 +155,19 @@ class UvuEmitter:
             body("v")
             s.close()
 
-    # --------------------------------------------------------- forward cores
-    def emit_forward_cores(self, s: Src):
+    # ------------------------------------------------------- shared structs
+    def emit_structs(self, s: Src):
         low = self.low
-        self._struct_x(s)
+        s("struct X_t {")
+        for b in self.used_in1:
+            s(f"    T b{b}[{low.in1[b].d}];")
+        s("};")
+        s("struct G_t {")
+        for io in self.used_out:
+            s(f"    T o{io}[{low.out[io].d}];")
+        s("};")
+        if self.can_preload:
+            s(f"struct E_t {{ X_t x; T w[{self.n_wslots}]; T y[{low.L2}]; }};")
         for si, seg in enumerate(self.segments):
             s(f"struct A{si}_t {{")
             for io in seg:
@@ -132,36 +178,73 @@ class UvuEmitter:
                 for k in range(low.out[io].d):
                     s(f"a.o{io}[{k}] = T(0);")
             s.close()
-            # a += sum over the segment's paths of w * CG(x, y)
+
+    def _emit_load_edge(self, s: Src, name: str, in1_blocks: List[int], paths: List[Path]):
+        """load_edge: fetch X[cols[e]] (the listed blocks), the weights of the
+        listed paths and the edge's Y into an E_t."""
+        low = self.low
+        s.open(
+            f"OEQ_DEV void {name}(E_t& d, const i64 e, const T* __restrict__ L1_in, const T* __restrict__ L2_in, "
+            "const T* __restrict__ W, const i64* __restrict__ cols, const int u)"
+        )
+        s("const i64 c = cols[e];")
+        s(f"const T* xrow = L1_in + c * {low.L1};")
+        s(f"const T* yrow = L2_in + e * {low.L2};")
+        s(f"const T* wrow = W{'' if low.shared_weights else f' + e * {low.WN}'};")
+        _, wptr = self._acc_pointer()
+        for p in paths:
+            for v in range(low.in2[p.i2].mul):
+                s(f"d.w[{self.wslot[p.index] + v}] = {wptr(p, str(v))};")
+        self._load_x(s, "xrow", in1_blocks, "d.x")
+        for j in range(low.L2):
+            s(f"d.y[{j}] = yrow[{j}];")
+        s.close()
+
+    # --------------------------------------------------------- forward cores
+    def _emit_fwd_seg(self, s: Src, si: int, preloaded: bool):
+        low = self.low
+        seg = self.segments[si]
+        if preloaded:
+            yacc, wacc = self._acc_preloaded("d")
+            s.open(f"OEQ_DEV void fwd_seg{si}_pre(const E_t& d, A{si}_t& a)")
+            xname = "d.x"
+        else:
+            yacc, wacc = self._acc_pointer()
             s.open(
                 f"OEQ_DEV void fwd_seg{si}(const X_t& x, const T* __restrict__ yrow, "
                 f"const T* __restrict__ wrow, const int u, A{si}_t& a)"
             )
-            for p in low.paths:
-                if p.io not in seg:
-                    continue
-                b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
-                V = b2.mul
-                s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l}) in1[{p.i1}] x in2[{p.i2}] -> out[{p.io}], nnz={len(p.nnz)}")
+            xname = "x"
+        for p in low.paths:
+            if p.io not in seg:
+                continue
+            b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
+            s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l}) in1[{p.i1}] x in2[{p.i2}] -> out[{p.io}], nnz={len(p.nnz)}")
 
-                def body(v, p=p, b1=b1, bo=bo, V=V):
-                    prods = self._products(s, p, v)
-                    started = set()
-                    for n, (i, j, k, c) in enumerate(p.nnz):
-                        q, neg = prods[n]
-                        if k not in started:
-                            s(f"T t{k} = {'-' if neg else ''}{q} * x.b{p.i1}[{i}];")
-                            started.add(k)
-                        else:
-                            s(f"t{k} {'-=' if neg else '+='} {q} * x.b{p.i1}[{i}];")
-                    s(f"const T wv = (u < {b1.mul}) ? wrow[{p.woff} + u * {V} + ({v})] : T(0);")
-                    for k in sorted(started):
-                        s(f"a.o{p.io}[{k}] += wv * t{k};")
+            def body(v, p=p):
+                prods = self._products(s, p, v, yacc)
+                started = set()
+                for n, (i, j, k, c) in enumerate(p.nnz):
+                    q, neg = prods[n]
+                    if k not in started:
+                        s(f"T t{k} = {'-' if neg else ''}{q} * {xname}.b{p.i1}[{i}];")
+                        started.add(k)
+                    else:
+                        s(f"t{k} {'-=' if neg else '+='} {q} * {xname}.b{p.i1}[{i}];")
+                s(f"const T wv = {wacc(p, v)};")
+                for k in sorted(started):
+                    s(f"a.o{p.io}[{k}] += wv * t{k};")
 
-                self._for_v(s, p, body)
-            s.close()
-            # needed in1 blocks of this segment
-        self.seg_in1 = [sorted({p.i1 for p in low.paths if p.io in seg}) for seg in self.segments]
+            self._for_v(s, p, body)
+        s.close()
+
+    def emit_forward_cores(self, s: Src, preloaded: bool):
+        for si in range(len(self.segments)):
+            self._emit_fwd_seg(s, si, False)
+            if preloaded and self.can_preload:
+                paths = [p for p in self.low.paths if p.io in self.segments[si]]
+                self._emit_load_edge(s, f"load_edge_f{si}", self.seg_in1[si], paths)
+                self._emit_fwd_seg(s, si, True)
 
     def _store_seg(self, s: Src, si: int, rowexpr: str, guard: str, atomic: bool = False):
         low = self.low
@@ -186,7 +269,7 @@ class UvuEmitter:
               f"({rowexpr})[{bo.off} + t] = T(0);")
             s.close()
 
-    def _lane_prologue(self, s: Src, G: int):
+    def _lane_prologue(self, s: Src):
         s("const int lane = oeq_lane();")
         s("const int wave = oeq_wave();")
         s(f"const int chunk = wave % {self.NCH};")
@@ -200,15 +283,22 @@ class UvuEmitter:
         s("const int u = chunk * 64 + ul;")
         s("(void)r; (void)g; (void)lane;")
 
+    @staticmethod
+    def _attrs(block: int, waves_per_eu: int) -> str:
+        a = f"__launch_bounds__({block})"
+        if waves_per_eu:
+            a += f" __attribute__((amdgpu_waves_per_eu({waves_per_eu}, {waves_per_eu})))"
+        return a
+
     # ---------------------------------------------------------- TP forward
-    def emit_tp_forward(self, s: Src, G: int):
+    def emit_tp_forward(self, s: Src, G: int, waves_per_eu: int = 0):
         low = self.low
         block = 64 * self.NCH * G
         s.open(
-            f'extern "C" __global__ __launch_bounds__({block}) void forward(i64 num_batch, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void forward(i64 num_batch, '
             "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, T* __restrict__ L3_out)"
         )
-        self._lane_prologue(s, G)
+        self._lane_prologue(s)
         s(f"const i64 ngroups = (num_batch + {self.R - 1}) / {self.R};")
         s.open(f"for (i64 grp = (i64)blockIdx.x * {G} + g; grp < ngroups; grp += (i64)gridDim.x * {G})")
         s(f"const i64 row = grp * {self.R} + r;")
@@ -232,37 +322,101 @@ class UvuEmitter:
         return block
 
     # ---------------------------------------------------------- conv forward
-    def emit_conv_forward(self, s: Src, G: int, deterministic: bool):
+    def _edge_loop(self, s: Src, first: str, last: str, load: Callable[[str, str], None],
+                   compute: Callable[[str, str], None], pipelined: bool, before_edge: Callable[[str], None] = None):
+        """Walk edges ``first, first+R, ... < last``. Pipelined: two operand
+        sets (A, B); the next edge's loads are issued before the current edge is
+        computed. ``load(buf, e)`` / ``compute(buf, e)`` emit code."""
+        R = self.R
+        if not pipelined:
+            s.open(f"for (i64 e = {first}; e < {last}; e += {R})")
+            if before_edge:
+                before_edge("e")
+            load("A", "e")
+            compute("A", "e")
+            s.close()
+            return
+        s(f"i64 e = {first};")
+        s.open(f"if (e < {last})")
+        load("A", "e")
+        s.close()
+        s.open(f"while (e < {last})")
+        s(f"const i64 en = e + {R};")
+        s.open(f"if (en < {last})")
+        load("B", "en")
+        s.close()
+        if before_edge:
+            before_edge("e")
+        compute("A", "e")
+        s.open(f"if (en < {last})")
+        s(f"const i64 en2 = en + {R};")
+        s.open(f"if (en2 < {last})")
+        load("A", "en2")
+        s.close()
+        if before_edge:
+            before_edge("en")
+        compute("B", "en")
+        s.close()
+        s(f"e += {2 * R};")
+        s.close()
+
+    def _node_loop_open(self, s: Src, G: int, xcd: int):
+        """One wave group per receiver node. Workgroups are handed to the XCDs
+        round-robin; with ``xcd`` > 1 (grid a multiple of it) block ids are remapped
+        so that each XCD walks one contiguous range of nodes and neighbouring
+        receivers share their senders' rows through that XCD's L2."""
+        if xcd > 1:
+            s(f"const i64 vper = (i64)gridDim.x / {xcd};")
+            s(f"const i64 vblk = ((i64)blockIdx.x % {xcd}) * vper + (i64)blockIdx.x / {xcd};")
+            s.open(f"for (i64 node = vblk * {G} + g; node < node_count; node += node_count + 1)")
+        else:
+            s.open(f"for (i64 node = (i64)blockIdx.x * {G} + g; node < node_count; node += (i64)gridDim.x * {G})")
+
+    def emit_conv_forward(self, s: Src, G: int, deterministic: bool, pipelined: bool, waves_per_eu: int = 0,
+                          xcd: int = 1):
         low = self.low
         block = 64 * self.NCH * G
         R = self.R
+        pipelined = pipelined and self.can_preload
         s.open(
-            f'extern "C" __global__ __launch_bounds__({block}) void forward(i64 node_count, i64 nnz, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void forward(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
             "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr)"
         )
-        self._lane_prologue(s, G)
+        self._lane_prologue(s)
+        if self.can_preload:
+            s("E_t A, B;")
 
-        def edge_body(si):
-            s("const i64 c = cols[e];")
-            s(f"const T* xrow = L1_in + c * {low.L1};")
-            s(f"const T* yrow = L2_in + e * {low.L2};")
-            s(f"const T* wrow = W{'' if low.shared_weights else f' + e * {low.WN}'};")
-            s("X_t x;")
-            self._load_x(s, "xrow", self.seg_in1[si])
-            s(f"fwd_seg{si}(x, yrow, wrow, u, a);")
+        def make_load(si):
+            def load(buf, e):
+                if self.can_preload:
+                    s(f"load_edge_f{si}({buf}, {e}, L1_in, L2_in, W, cols, u);")
+            return load
+
+        def make_compute(si):
+            def compute(buf, e):
+                if self.can_preload:
+                    s(f"fwd_seg{si}_pre({buf}, a);")
+                else:
+                    s.open("")
+                    s(f"const T* xrow = L1_in + cols[{e}] * {low.L1};")
+                    s(f"const T* yrow = L2_in + {e} * {low.L2};")
+                    s(f"const T* wrow = W{'' if low.shared_weights else f' + {e} * {low.WN}'};")
+                    s("X_t x;")
+                    self._load_x(s, "xrow", self.seg_in1[si])
+                    s(f"fwd_seg{si}(x, yrow, wrow, u, a);")
+                    s.close()
+            return compute
 
         if deterministic:
-            s.open(f"for (i64 node = (i64)blockIdx.x * {G} + g; node < node_count; node += (i64)gridDim.x * {G})")
+            self._node_loop_open(s, G, xcd)
             s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
             s(f"T* zrow = L3_out + node * {low.L3};")
             for si in range(len(self.segments)):
                 s.open("")
                 s(f"A{si}_t a; zero_seg{si}(a);")
-                s.open(f"for (i64 e = e0 + r; e < e1; e += {R})")
-                edge_body(si)
-                s.close()
+                self._edge_loop(s, "e0 + r", "e1", make_load(si), make_compute(si), pipelined)
                 if R > 1:
                     # fold the R lane groups (fixed order) into group 0
                     for io in self.segments[si]:
@@ -285,18 +439,21 @@ class UvuEmitter:
                 s.open("")
                 s(f"A{si}_t a; zero_seg{si}(a);")
                 s("i64 cur = -1;")
-                s.open(f"for (i64 e = eb + r; e < ee; e += {R})")
-                s("const i64 row = rows[e];")
-                s.open("if (row != cur)")
-                s.open("if (cur >= 0)")
-                s(f"T* zrow = L3_out + cur * {low.L3};")
-                self._store_seg(s, si, "zrow", "true", atomic=True)
-                s.close()
-                s(f"zero_seg{si}(a);")
-                s("cur = row;")
-                s.close()
-                edge_body(si)
-                s.close()
+
+                def before_edge(e, si=si):
+                    s.open("")
+                    s(f"const i64 row = rows[{e}];")
+                    s.open("if (row != cur)")
+                    s.open("if (cur >= 0)")
+                    s(f"T* zrow = L3_out + cur * {low.L3};")
+                    self._store_seg(s, si, "zrow", "true", atomic=True)
+                    s.close()
+                    s(f"zero_seg{si}(a);")
+                    s("cur = row;")
+                    s.close()
+                    s.close()
+
+                self._edge_loop(s, "eb + r", "ee", make_load(si), make_compute(si), pipelined, before_edge)
                 s.open("if (cur >= 0)")
                 s(f"T* zrow = L3_out + cur * {low.L3};")
                 self._store_seg(s, si, "zrow", "true", atomic=True)
@@ -306,13 +463,6 @@ class UvuEmitter:
         return block
 
     # ------------------------------------------------------- backward pieces
-    def _struct_bwd(self, s: Src):
-        low = self.low
-        s("struct G_t {")
-        for io in sorted({p.io for p in low.paths}):
-            s(f"    T o{io}[{low.out[io].d}];")
-        s("};")
-
     def _load_g(self, s: Src, rowexpr: str, ios: List[int], dst: str = "gr"):
         low = self.low
         for io in ios:
@@ -327,15 +477,12 @@ class UvuEmitter:
                 s(f"{dst}.o{io}[{k}] = T(0);")
             s.close()
 
-    def _bwd_paths(self, s: Src, *, g_on_demand_row: str = None, dw_mode: str = "store",
-                   g_guard: str = None, dw_guard: str = None):
-        """Straight-line backward of all paths. Expects in scope: x (X_t), dx (X_t),
-        dy[L2_PAD], yrow, wrow, u and either gr (G_t, resident) or a row pointer to
-        load output gradients from on demand. dw_mode: 'store' (dwrow[...] = v) or
-        'acc' (dwacc[slot] += v)."""
+    def _bwd_paths(self, s: Src, *, xname: str, yacc, wacc, g_on_demand_row: Optional[str] = None,
+                   dw_mode: str = "store", g_guard: Optional[str] = None, dw_guard: Optional[str] = None):
+        """Straight-line backward of all paths. In scope: ``xname`` (X_t), dx (X_t),
+        dy[], u, and either gr (G_t, resident) or a row pointer to load output
+        gradients from. dw_mode 'store': dwrow[...] = v; 'acc': dwacc[slot] += v."""
         low = self.low
-        last_io = None
-        slot = 0
         for p in sorted(low.paths, key=lambda q: (q.io, q.index)):
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
             V = b2.mul
@@ -355,26 +502,23 @@ class UvuEmitter:
                 gname = lambda k: f"gk[{k}]"
             else:
                 gname = lambda k, io=p.io: f"gr.o{io}[{k}]"
+            base_slot = self.wslot[p.index]
 
-            base_slot = slot
-
-            def body(v, p=p, b1=b1, b2=b2, bo=bo, V=V, gname=gname, base_slot=base_slot):
-                prods = self._products(s, p, v)
-                s(f"const T wv = (u < {b1.mul}) ? wrow[{p.woff} + u * {V} + ({v})] : T(0);")
+            def body(v, p=p, b1=b1, b2=b2, V=V, gname=gname, base_slot=base_slot):
+                prods = self._products(s, p, v, yacc)
+                s(f"const T wv = {wacc(p, v)};")
                 ks = sorted({k for _, _, k, _ in p.nnz})
                 for k in ks:
                     s(f"const T gw{k} = {gname(k)} * wv;")
-                # dx_i += q * gw_k ; f_k += q * x_i
                 fstart = set()
                 for n, (i, j, k, c) in enumerate(p.nnz):
                     q, neg = prods[n]
                     s(f"dx.b{p.i1}[{i}] {'-=' if neg else '+='} {q} * gw{k};")
                     if k not in fstart:
-                        s(f"T f{k} = {'-' if neg else ''}{q} * x.b{p.i1}[{i}];")
+                        s(f"T f{k} = {'-' if neg else ''}{q} * {xname}.b{p.i1}[{i}];")
                         fstart.add(k)
                     else:
-                        s(f"f{k} {'-=' if neg else '+='} {q} * x.b{p.i1}[{i}];")
-                # dw = sum_k g_k f_k
+                        s(f"f{k} {'-=' if neg else '+='} {q} * {xname}.b{p.i1}[{i}];")
                 terms = [f"{gname(k)} * f{k}" for k in ks]
                 s(f"T dwv = {terms[0]};")
                 for t in terms[1:]:
@@ -383,36 +527,16 @@ class UvuEmitter:
                     s(f"if (u < {b1.mul}{' && ' + dw_guard if dw_guard else ''}) "
                       f"dwrow[{p.woff} + u * {V} + ({v})] = dwv;")
                 else:
-                    if V <= UNROLL_V_LIMIT:
-                        s(f"dwacc[{base_slot} + {v}] += dwv;")
-                    else:
-                        s(f"dwacc[{base_slot} + v] += dwv;")
-                # dy_j += c * x_i * gw_k   (products shared between non-zeros with equal (i,k))
+                    s(f"dwacc[{base_slot} + {v}] += dwv;")
                 pair = {}
                 for n, (i, j, k, c) in enumerate(p.nnz):
                     if (i, k) not in pair:
-                        nm = f"xg{len(pair)}"
-                        pair[(i, k)] = nm
-                        s(f"const T {nm} = x.b{p.i1}[{i}] * gw{k};")
+                        pair[(i, k)] = f"xg{len(pair)}"
+                        s(f"const T {pair[(i, k)]} = {xname}.b{p.i1}[{i}] * gw{k};")
                     s(f"dy[{b2.off} + ({v}) * {b2.d} + {j}] += T({self.lit(c)}) * {pair[(i, k)]};")
 
             self._for_v(s, p, body)
-            slot += V
             s.close()
-        return slot
-
-    def n_dw_slots(self) -> int:
-        return sum(self.low.in2[p.i2].mul for p in self.low.paths)
-
-    def _dw_slot_map(self):
-        """(path, v) -> slot in the per-lane shared-weight accumulator, in the
-        order _bwd_paths visits them."""
-        out, slot = [], 0
-        for p in sorted(self.low.paths, key=lambda q: (q.io, q.index)):
-            V = self.low.in2[p.i2].mul
-            out.append((p, slot))
-            slot += V
-        return out
 
     def _dy_reduce(self, s: Src):
         """Halving butterfly over the lanes of one row. Leaves, in every lane,
@@ -442,9 +566,10 @@ class UvuEmitter:
             m //= 2
         return cur, dup
 
-    def _dy_finish(self, s: Src, dst_row: str, live: str, G: int, sync: bool):
+    def _dy_finish(self, s: Src, dst_row: str, live: str):
         """Cross-lane (and cross-chunk) reduction of dy, then write of the row."""
         low = self.low
+        s.open("")
         cur, dup = self._dy_reduce(s)
         if self.NCH == 1:
             s.open(f"if ({live} && (ul & {dup}) == 0)")
@@ -466,6 +591,7 @@ class UvuEmitter:
             s.close()
             s.close()
             s("__syncthreads();")
+        s.close()
 
     def _store_dx(self, s: Src, rowexpr: str, guard: str, atomic: bool = False):
         low = self.low
@@ -496,23 +622,26 @@ class UvuEmitter:
             for i in range(self.low.in1[b].d):
                 s(f"{name}.b{b}[{i}] = T(0);")
 
+    def _dw_slots(self):
+        return [(p, self.wslot[p.index]) for p in self.low.paths]
+
     # ---------------------------------------------------------- TP backward
-    def emit_tp_backward(self, s: Src, G: int):
+    def emit_tp_backward(self, s: Src, G: int, waves_per_eu: int = 0):
         low = self.low
         block = 64 * self.NCH * G
         shared = low.shared_weights
         s.open(
-            f'extern "C" __global__ __launch_bounds__({block}) void backward(i64 num_batch, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void backward(i64 num_batch, '
             "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
             "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
             "const T* __restrict__ L3_grad, T* __restrict__ wpartial)"
         )
-        self._lane_prologue(s, G)
+        self._lane_prologue(s)
         if self.NCH > 1:
             s(f"__shared__ T s_dy[{G}][{self.NCH}][{self.l2_pad}];")
         if shared:
-            s(f"T dwacc[{self.n_dw_slots()}];")
-            s(f"for (int t = 0; t < {self.n_dw_slots()}; ++t) dwacc[t] = T(0);")
+            s(f"T dwacc[{self.n_wslots}];")
+            s(f"for (int t = 0; t < {self.n_wslots}; ++t) dwacc[t] = T(0);")
         s(f"const i64 ngroups = (num_batch + {self.R - 1}) / {self.R};")
         # uniform trip count per block: the dY reduction contains block barriers
         s.open(f"for (i64 base = (i64)blockIdx.x * {G}; base < ngroups; base += (i64)gridDim.x * {G})")
@@ -533,25 +662,25 @@ class UvuEmitter:
         s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
         # rows past the end of the batch are clamped duplicates: their gradients are
         # zeroed (shared weights) and none of their results is stored
-        self._bwd_paths(s, g_on_demand_row="grow", dw_mode="acc" if shared else "store",
-                        g_guard="live" if shared else None, dw_guard="live")
+        yacc, wacc = self._acc_pointer()
+        self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, g_on_demand_row="grow",
+                        dw_mode="acc" if shared else "store", g_guard="live" if shared else None, dw_guard="live")
         s(f"T* dxrow = L1_grad + rowc * {low.L1};")
         self._store_dx(s, "dxrow", "live")
         self._zero_untouched_in1(s, "dxrow", "live")
-        self._dy_finish(s, f"L2_grad + rowc * {low.L2}", "live", G, True)
+        self._dy_finish(s, f"L2_grad + rowc * {low.L2}", "live")
         s.close()
         if shared:
             # fold the R row groups of the wave, then every wave group writes one partial row
-            slots = self._dw_slot_map()
             if self.R > 1:
-                s.open(f"for (int t = 0; t < {self.n_dw_slots()}; ++t)")
+                s.open(f"for (int t = 0; t < {self.n_wslots}; ++t)")
                 m = self.LPR
                 while m < 64:
                     s(f"dwacc[t] += __shfl_xor(dwacc[t], {m});")
                     m *= 2
                 s.close()
             s(f"T* prow = wpartial + ((i64)blockIdx.x * {G} + g) * {low.WN};")
-            for p, slot in slots:
+            for p, slot in self._dw_slots():
                 b1, V = low.in1[p.i1], low.in2[p.i2].mul
                 s.open(f"if (r == 0 && u < {b1.mul})")
                 s(f"for (int v = 0; v < {V}; ++v) prow[{p.woff} + u * {V} + v] = dwacc[{slot} + v];")
@@ -560,86 +689,94 @@ class UvuEmitter:
         return block
 
     # -------------------------------------------------------- conv backward
-    def emit_conv_backward(self, s: Src, deterministic: bool, G: int):
+    def emit_conv_backward(self, s: Src, deterministic: bool, G: int, pipelined: bool, waves_per_eu: int = 0,
+                           g_resident: Optional[bool] = None, xcd: int = 1):
         low = self.low
         shared = low.shared_weights
         if self.NCH > 1:
             G = 1  # one node (or edge range) per block: the per-edge dY reduction uses block barriers
         block = 64 * self.NCH * G
-        R = self.R
+        pipelined = pipelined and self.can_preload
+        if self.can_preload:
+            self._emit_load_edge(s, "load_edge_b", self.used_in1, low.paths)
         s.open(
-            f'extern "C" __global__ __launch_bounds__({block}) void backward(i64 node_count, i64 nnz, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void backward(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
             "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
             "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp)"
         )
-        self._lane_prologue(s, G)
+        self._lane_prologue(s)
         if self.NCH > 1:
             s(f"__shared__ T s_dy[{G}][{self.NCH}][{self.l2_pad}];")
         if shared:
-            s(f"T dwacc[{self.n_dw_slots()}];")
-            s(f"for (int t = 0; t < {self.n_dw_slots()}; ++t) dwacc[t] = T(0);")
-        resident = deterministic and self.g_resident
+            s(f"T dwacc[{self.n_wslots}];")
+            s(f"for (int t = 0; t < {self.n_wslots}; ++t) dwacc[t] = T(0);")
+        if self.can_preload:
+            s("E_t A, B;")
+        resident = deterministic and (self.g_resident if g_resident is None else g_resident)
 
-        def edge_body(grow_expr):
-            s("const i64 c = cols[e];")
-            s(f"const T* xrow = L1_in + c * {low.L1};")
-            s(f"const T* yrow = L2_in + e * {low.L2};")
-            s(f"const T* wrow = W{'' if shared else f' + e * {low.WN}'};")
-            if not shared:
-                s(f"T* dwrow = W_grad + e * {low.WN};")
-            s("X_t x, dx;")
-            self._load_x(s, "xrow", self.used_in1)
-            self._zero_x(s, "dx")
-            s(f"T dy[{self.l2_pad}];")
-            s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
-            if resident:
-                self._bwd_paths(s, dw_mode="acc" if shared else "store")
-            else:
-                s(f"const T* grow = {grow_expr};")
-                self._bwd_paths(s, g_on_demand_row="grow", dw_mode="acc" if shared else "store")
-            if deterministic:
-                s(f"T* dxrow = dx_tmp + e * {low.L1};")
-                self._store_dx(s, "dxrow", "true")
-                self._zero_untouched_in1(s, "dxrow", "true")
-            else:
-                s(f"T* dxrow = L1_grad + c * {low.L1};")
-                self._store_dx(s, "dxrow", "true", atomic=True)
+        def load(buf, e):
+            if self.can_preload:
+                s(f"load_edge_b({buf}, {e}, L1_in, L2_in, W, cols, u);")
+
+        def make_compute(grow_expr_of):
+            def compute(buf, e):
+                s.open("")
+                if self.can_preload:
+                    yacc, wacc = self._acc_preloaded(buf)
+                    xname = f"{buf}.x"
+                else:
+                    yacc, wacc = self._acc_pointer()
+                    xname = "x"
+                    s(f"const T* xrow = L1_in + cols[{e}] * {low.L1};")
+                    s(f"const T* yrow = L2_in + {e} * {low.L2};")
+                    s(f"const T* wrow = W{'' if shared else f' + {e} * {low.WN}'};")
+                    s("X_t x;")
+                    self._load_x(s, "xrow", self.used_in1)
+                if not shared:
+                    s(f"T* dwrow = W_grad + {e} * {low.WN};")
+                s("X_t dx;")
+                self._zero_x(s, "dx")
+                s(f"T dy[{self.l2_pad}];")
+                s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+                if resident:
+                    self._bwd_paths(s, xname=xname, yacc=yacc, wacc=wacc, dw_mode="acc" if shared else "store")
+                else:
+                    s(f"const T* grow = {grow_expr_of(e)};")
+                    self._bwd_paths(s, xname=xname, yacc=yacc, wacc=wacc, g_on_demand_row="grow",
+                                    dw_mode="acc" if shared else "store")
+                if deterministic:
+                    s(f"T* dxrow = dx_tmp + {e} * {low.L1};")
+                    self._store_dx(s, "dxrow", "true")
+                    self._zero_untouched_in1(s, "dxrow", "true")
+                else:
+                    s(f"T* dxrow = L1_grad + cols[{e}] * {low.L1};")
+                    self._store_dx(s, "dxrow", "true", atomic=True)
+                self._dy_finish(s, f"L2_grad + {e} * {low.L2}", "true")
+                s.close()
+            return compute
 
         if deterministic:
-            s.open(f"for (i64 node = (i64)blockIdx.x * {G} + g; node < node_count; node += (i64)gridDim.x * {G})")
+            self._node_loop_open(s, G, xcd)
             s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
             if resident:
                 s("G_t gr;")
-                self._load_g(s, f"L3_grad + node * {low.L3}", sorted({p.io for p in low.paths}))
-            if self.NCH > 1:
-                # all waves of the block walk the same edges: barriers inside are uniform
-                s.open("for (i64 e = e0; e < e1; ++e)")
-                edge_body(f"L3_grad + node * {low.L3}")
-                self._dy_finish(s, f"L2_grad + e * {low.L2}", "true", G, True)
-                s.close()
-            else:
-                s.open(f"for (i64 e = e0 + r; e < e1; e += {R})")
-                edge_body(f"L3_grad + node * {low.L3}")
-                self._dy_finish(s, f"L2_grad + e * {low.L2}", "true", G, False)
-                s.close()
+                self._load_g(s, f"L3_grad + node * {low.L3}", self.used_out)
+            # with more than one chunk all waves of the block walk the same edges, so the
+            # block barriers of the dY reduction are reached uniformly
+            self._edge_loop(s, "e0 + r", "e1", load, make_compute(lambda e: f"L3_grad + node * {low.L3}"), pipelined)
             s.close()
         else:
             s(f"const i64 ngrp = (i64)gridDim.x * {G};")
             s("const i64 per = (nnz + ngrp - 1) / ngrp;")
             s(f"const i64 eb = ((i64)blockIdx.x * {G} + g) * per;")
             s("const i64 ee = (eb + per < nnz) ? eb + per : nnz;")
-            if self.NCH > 1:
-                s.open("for (i64 e = eb; e < ee; ++e)")
-            else:
-                s.open(f"for (i64 e = eb + r; e < ee; e += {R})")
-            edge_body(f"L3_grad + rows[e] * {low.L3}")
-            self._dy_finish(s, f"L2_grad + e * {low.L2}", "true", G, self.NCH > 1)
-            s.close()
+            self._edge_loop(s, "eb + r", "ee", load, make_compute(lambda e: f"L3_grad + rows[{e}] * {low.L3}"),
+                            pipelined)
         if shared:
             # shared weights: one atomic add per weight per wave (atomic mode only)
-            for p, slot in self._dw_slot_map():
+            for p, slot in self._dw_slots():
                 b1, V = low.in1[p.i1], low.in2[p.i2].mul
                 s.open(f"if (u < {b1.mul})")
                 s(f"for (int v = 0; v < {V}; ++v) oeq_atomic_add(W_grad + {p.woff} + u * {V} + v, dwacc[{slot} + v]);")
@@ -657,16 +794,16 @@ def tp_module(low: Lowered, compute_units: int = 256):
     """Source + launch descriptors for the batch tensor product (forward, backward)."""
     from .. import runtime as rt
 
-    em = UvuEmitter(low, acc_budget_words=48)
+    t = tuning(dict(tp_acc=48, tp_gf=max(1, 4 // low.n_chunks), tp_gb=max(1, 4 // low.n_chunks), tp_wf=0, tp_wb=0))
+    em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels())
-    em.emit_forward_cores(s)
-    em._struct_bwd(s)
-    G_f = max(1, 4 // em.NCH)
-    G_b = max(1, 4 // em.NCH)
-    blk_f = em.emit_tp_forward(s, G_f)
-    blk_b = em.emit_tp_backward(s, G_b)
+    em.emit_structs(s)
+    em.emit_forward_cores(s, preloaded=False)
+    G_f, G_b = t["tp_gf"], t["tp_gb"]
+    blk_f = em.emit_tp_forward(s, G_f, t["tp_wf"])
+    blk_b = em.emit_tp_backward(s, G_b, t["tp_wb"])
     max_blocks_b = compute_units * 8
     descs = [
         (rt.ROLE_TP_FORWARD, "forward", blk_f, G_f * em.R, 0),
@@ -685,16 +822,20 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256):
     from .. import runtime as rt
 
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
-    em = UvuEmitter(low)
+    t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=1, conv_pipe_b=0,
+                    conv_wf=0, conv_wb=2, conv_gres=-1, conv_xcd=8))
+    em = UvuEmitter(low, acc_budget_words=t["conv_acc"])
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels())
-    em.emit_forward_cores(s)
-    em._struct_bwd(s)
-    G_f = max(1, 4 // em.NCH)
-    G_b = 1 if em.NCH > 1 else 4
-    blk_f = em.emit_conv_forward(s, G_f, deterministic)
-    blk_b = em.emit_conv_backward(s, deterministic, G_b)
+    em.emit_structs(s)
+    em.emit_forward_cores(s, preloaded=True)
+    G_f = t["conv_gf"]
+    G_b = 1 if em.NCH > 1 else t["conv_gb"]
+    xcd = max(1, t["conv_xcd"])
+    blk_f = em.emit_conv_forward(s, G_f, deterministic, bool(t["conv_pipe_f"]), t["conv_wf"], xcd)
+    gres = None if t["conv_gres"] < 0 else bool(t["conv_gres"])
+    blk_b = em.emit_conv_backward(s, deterministic, G_b, bool(t["conv_pipe_b"]), t["conv_wb"], gres, xcd)
     descs = [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, compute_units * 16),
@@ -702,8 +843,8 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256):
     if deterministic:
         s(fixup_backward_kernel(low.L1))
         descs += [
-            (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f, 0),
-            (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b, 0),
+            (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f, 0, xcd),
+            (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b, 0, xcd),
             (rt.ROLE_CONV_FIXUP_BACKWARD, "fixup_backward", 256, 1, 0),
         ]
     else:

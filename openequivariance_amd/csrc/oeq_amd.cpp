@@ -47,6 +47,7 @@ struct RoleInfo {
     unsigned block = 0;
     unsigned units_per_block = 1;
     unsigned max_blocks = 0;
+    unsigned grid_multiple = 0;
 };
 
 struct DeviceSlot {
@@ -104,6 +105,7 @@ struct oeq_kernels {
         int64_t blocks = (units + r.units_per_block - 1) / r.units_per_block;
         if (blocks < 1) blocks = 1;
         if (r.max_blocks && blocks > (int64_t)r.max_blocks) blocks = r.max_blocks;
+        if (r.grid_multiple > 1) blocks = (blocks + r.grid_multiple - 1) / r.grid_multiple * r.grid_multiple;
         if (blocks > 0x7fffffffLL) blocks = 0x7fffffffLL;
         return (unsigned)blocks;
     }
@@ -241,6 +243,7 @@ int oeq_kernels_create(const void* code, size_t code_size, const oeq_problem_dim
         r.block = d.block_threads;
         r.units_per_block = d.units_per_block;
         r.max_blocks = d.max_blocks;
+        r.grid_multiple = d.grid_multiple;
     }
     *out = k;
     return OEQ_OK;

@@ -69,6 +69,7 @@ class _KernelDesc(ctypes.Structure):
         ("block_threads", ctypes.c_uint32),
         ("units_per_block", ctypes.c_uint32),
         ("max_blocks", ctypes.c_uint32),
+        ("grid_multiple", ctypes.c_uint32),
     ]
 
 
@@ -215,9 +216,11 @@ class KernelSet:
         self._lib = lib
         self._names = [d[1].encode() for d in descs]
         arr = (_KernelDesc * len(descs))()
-        for slot, (role, _name, block, upb, maxb), enc in zip(arr, descs, self._names):
+        for slot, desc, enc in zip(arr, descs, self._names):
+            role, _name, block, upb, maxb = desc[:5]
             slot.role, slot.kernel_name, slot.block_threads = role, enc, block
             slot.units_per_block, slot.max_blocks = upb, maxb
+            slot.grid_multiple = desc[5] if len(desc) > 5 else 0
         pd = _ProblemDims(**dims)
         handle = _P()
         _check(lib.oeq_kernels_create(code, len(code), ctypes.byref(pd), arr, len(descs), ctypes.byref(handle)),
