@@ -84,6 +84,164 @@ class UvuEmitter:
             all(low.in2[p.i2].mul <= UNROLL_V_LIMIT for p in low.paths) and low.L2 <= 32 and self.n_wslots <= 64
         )
 
+        self.stage = self._stage_layout()
+        self.stage3 = self._stage3_layout()
+
+    def _stage_layout(self):
+        """Layout of one wave's LDS staging buffer for the operands of an edge
+        (the wave's 64-channel slice of X[sender] and of W[edge]), filled by
+        direct global->LDS loads of 16 B per lane. None when the problem does not
+        have the regular shape this needs."""
+        low = self.low
+        if not (self.R == 1 and self.can_preload and self.words == 1 and len(self.segments) == 1
+                and not low.shared_weights):
+            return None
+        U = 64 * self.NCH
+        if any(low.in1[b].mul != U or low.in1[b].off % 4 for b in self.used_in1):
+            return None
+        if any(low.in2[p.i2].mul != 1 or p.woff != p.index * U for p in low.paths):
+            return None
+        if low.L1 % 4 or low.WN % 4:
+            return None
+        xl, units = {}, 0
+        for b in self.used_in1:
+            xl[b] = units * 4
+            units += 16 * low.in1[b].d
+        nqx = (units + 63) // 64
+        nuw = 16 * len(low.paths)
+        nqw = (nuw + 63) // 64
+        return dict(U=U, xl=xl, nux=units, nqx=nqx, nuw=nuw, nqw=nqw, XF=nqx * 256, floats=(nqx + nqw) * 256)
+
+    def _emit_stage_offsets(self, s: Src):
+        """Per-lane source offsets (in elements) of the staging loads; loop invariant."""
+        low, st = self.low, self.stage
+        for q in range(st["nqx"]):
+            s(f"int xoff{q};")
+            s.open("")
+            s(f"int t = {q * 64} + lane; if (t > {st['nux'] - 1}) t = {st['nux'] - 1};")
+            expr, pu = None, 0
+            terms = []
+            for b in self.used_in1:
+                blk = low.in1[b]
+                n = 16 * blk.d
+                terms.append((pu, pu + n, f"{blk.off} + chunk * {64 * blk.d} + (t - {pu}) * 4"))
+                pu += n
+            code = terms[-1][2]
+            for lo, hi, ex in reversed(terms[:-1]):
+                code = f"(t < {hi}) ? ({ex}) : ({code})"
+            s(f"xoff{q} = {code};")
+            s.close()
+        for q in range(st["nqw"]):
+            s(f"int woff{q};")
+            s.open("")
+            s(f"int t = {q * 64} + lane; if (t > {st['nuw'] - 1}) t = {st['nuw'] - 1};")
+            s(f"woff{q} = (t >> 4) * {st['U']} + chunk * 64 + (t & 15) * 4;")
+            s.close()
+
+    def _emit_stage_issue(self, s: Src, e: str):
+        low, st = self.low, self.stage
+        s.open("")
+        s(f"const T* sx = L1_in + cols[{e}] * {low.L1};")
+        s(f"const T* sw = W + ({e}) * {low.WN};")
+        for q in range(st["nqx"]):
+            s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sx + xoff{q}), (OEQ_LPTR)(&s_stage[wave][{q * 256}]), 16, 0, 0);")
+        for q in range(st["nqw"]):
+            s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sw + woff{q}), "
+              f"(OEQ_LPTR)(&s_stage[wave][{st['XF'] + q * 256}]), 16, 0, 0);")
+        for j in range(low.L2):
+            s(f"yn[{j}] = L2_in[({e}) * {low.L2} + {j}];")
+        s.close()
+
+    def _emit_stage_read(self, s: Src, buf: str):
+        low, st = self.low, self.stage
+        for b in self.used_in1:
+            blk = low.in1[b]
+            for i in range(blk.d):
+                s(f"{buf}.x.b{b}[{i}] = s_stage[wave][{st['xl'][b]} + ul * {blk.d} + {i}];")
+        for p in low.paths:
+            s(f"{buf}.w[{self.wslot[p.index]}] = s_stage[wave][{st['XF'] + p.index * 64} + ul];")
+        for j in range(low.L2):
+            s(f"{buf}.y[{j}] = yn[{j}];")
+
+    # ---- double-buffered staging: X, W and Y of an edge live only in LDS ------------
+    def _stage3_layout(self):
+        """Two LDS buffers per wave (separate arrays, so that reads of one do not
+        wait for loads into the other); the contraction reads its operands from
+        LDS where it uses them, so no register copy of an edge's operands exists."""
+        if self.stage is None or self.low.L2 % 4:
+            return None
+        st = dict(self.stage)
+        npaths = len(self.low.paths)
+        st["XF"] = st["nux"] * 4
+        st["YOFF"] = st["XF"] + 64 * npaths
+        st["nuwy"] = 16 * npaths + self.low.L2 // 4
+        st["nqw"] = (st["nuwy"] + 63) // 64
+        st["floats"] = st["XF"] + st["nuwy"] * 4
+        return st
+
+    def _emit_stage3_offsets(self, s: Src):
+        low, st = self.low, self.stage3
+        for q in range(st["nqx"]):
+            s(f"int xoff{q};")
+            s.open("")
+            s(f"int t = {q * 64} + lane; if (t > {st['nux'] - 1}) t = {st['nux'] - 1};")
+            terms, pu = [], 0
+            for b in self.used_in1:
+                blk = low.in1[b]
+                n = 16 * blk.d
+                terms.append((pu + n, f"{blk.off} + chunk * {64 * blk.d} + (t - {pu}) * 4"))
+                pu += n
+            code = terms[-1][1]
+            for hi, ex in reversed(terms[:-1]):
+                code = f"(t < {hi}) ? ({ex}) : ({code})"
+            s(f"xoff{q} = {code};")
+            s.close()
+        nuw = 16 * len(low.paths)
+        for q in range(st["nqw"]):
+            # units below nuw are weights (16 per path), the rest is the edge's Y row
+            s(f"int woff{q}; bool wsel{q};")
+            s.open("")
+            s(f"int t = {q * 64} + lane; if (t > {st['nuwy'] - 1}) t = {st['nuwy'] - 1};")
+            s(f"wsel{q} = t < {nuw};")
+            s(f"woff{q} = wsel{q} ? ((t >> 4) * {st['U']} + chunk * 64 + (t & 15) * 4) : ((t - {nuw}) * 4);")
+            s.close()
+
+    def _emit_stage3_issue(self, s: Src, buf: str, e: str):
+        low, st = self.low, self.stage3
+        s.open("")
+        s(f"const T* sx = L1_in + cols[{e}] * {low.L1};")
+        s(f"const T* sw = W + ({e}) * {low.WN};")
+        s(f"const T* sy = L2_in + ({e}) * {low.L2};")
+        for q in range(st["nqx"]):
+            n = min(64, st["nux"] - q * 64)
+            guard = f"if (lane < {n}) " if n < 64 else ""
+            s(f"{guard}__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sx + xoff{q}), "
+              f"(OEQ_LPTR)(&s_stage{buf}[wave][{q * 256}]), 16, 0, 0);")
+        for q in range(st["nqw"]):
+            n = min(64, st["nuwy"] - q * 64)
+            guard = f"if (lane < {n}) " if n < 64 else ""
+            s(f"{guard}__builtin_amdgcn_global_load_lds((const OEQ_GPTR)((wsel{q} ? sw : sy) + woff{q}), "
+              f"(OEQ_LPTR)(&s_stage{buf}[wave][{st['XF'] + q * 256}]), 16, 0, 0);")
+        s.close()
+
+    def _acc_staged3(self, sb: str):
+        low, st = self.low, self.stage3
+
+        def x(b: int, i: int) -> str:
+            return f"{sb}[{st['xl'][b]} + ul * {low.in1[b].d} + {i}]"
+
+        def y(p: Path, v: str, j: int) -> str:
+            return f"{sb}[{st['YOFF'] + low.in2[p.i2].off + j}]"
+
+        def w(p: Path, v: str) -> str:
+            return f"{sb}[{st['XF'] + p.index * 64} + ul]"
+
+        return x, y, w
+
+    @staticmethod
+    def _xv(xname, b: int, i: int) -> str:
+        return xname(b, i) if callable(xname) else f"{xname}.b{b}[{i}]"
+
     # ------------------------------------------------------------------ utils
     def lit(self, v: float) -> str:
         return float_literal(v, self.T)
@@ -201,10 +359,13 @@ class UvuEmitter:
         s.close()
 
     # --------------------------------------------------------- forward cores
-    def _emit_fwd_seg(self, s: Src, si: int, preloaded: bool):
+    def _emit_fwd_seg(self, s: Src, si: int, preloaded):
         low = self.low
         seg = self.segments[si]
-        if preloaded:
+        if preloaded == "lds":
+            xname, yacc, wacc = self._acc_staged3("sb")
+            s.open(f"OEQ_DEV void fwd_seg{si}_lds(const T* sb, const int ul, A{si}_t& a)")
+        elif preloaded:
             yacc, wacc = self._acc_preloaded("d")
             s.open(f"OEQ_DEV void fwd_seg{si}_pre(const E_t& d, A{si}_t& a)")
             xname = "d.x"
@@ -227,10 +388,10 @@ class UvuEmitter:
                 for n, (i, j, k, c) in enumerate(p.nnz):
                     q, neg = prods[n]
                     if k not in started:
-                        s(f"T t{k} = {'-' if neg else ''}{q} * {xname}.b{p.i1}[{i}];")
+                        s(f"T t{k} = {'-' if neg else ''}{q} * {self._xv(xname, p.i1, i)};")
                         started.add(k)
                     else:
-                        s(f"t{k} {'-=' if neg else '+='} {q} * {xname}.b{p.i1}[{i}];")
+                        s(f"t{k} {'-=' if neg else '+='} {q} * {self._xv(xname, p.i1, i)};")
                 s(f"const T wv = {wacc(p, v)};")
                 for k in sorted(started):
                     s(f"a.o{p.io}[{k}] += wv * t{k};")
@@ -245,6 +406,8 @@ class UvuEmitter:
                 paths = [p for p in self.low.paths if p.io in self.segments[si]]
                 self._emit_load_edge(s, f"load_edge_f{si}", self.seg_in1[si], paths)
                 self._emit_fwd_seg(s, si, True)
+            if preloaded and self.stage3 is not None:
+                self._emit_fwd_seg(s, si, "lds")
 
     def _store_seg(self, s: Src, si: int, rowexpr: str, guard: str, atomic: bool = False):
         low = self.low
@@ -323,11 +486,66 @@ class UvuEmitter:
 
     # ---------------------------------------------------------- conv forward
     def _edge_loop(self, s: Src, first: str, last: str, load: Callable[[str, str], None],
-                   compute: Callable[[str, str], None], pipelined: bool, before_edge: Callable[[str], None] = None):
+                   compute: Callable[[str, str], None], pipelined: int, before_edge: Callable[[str], None] = None):
         """Walk edges ``first, first+R, ... < last``. Pipelined: two operand
         sets (A, B); the next edge's loads are issued before the current edge is
         computed. ``load(buf, e)`` / ``compute(buf, e)`` emit code."""
         R = self.R
+        def vmcnt(n: int) -> str:
+            # s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt = simm16[3:0] | simm16[15:14] << 4)
+            return f"__builtin_amdgcn_s_waitcnt({(n & 15) | 0x0F70 | ((n >> 4) << 14)}); /* vmcnt({n}) */"
+
+        lgkm0 = "__builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): LDS reads retired before the buffer is refilled"
+        if pipelined == 3:
+            # Two LDS buffers per wave, loads one edge ahead. Stores and atomics of the loop body share
+            # the vector-memory counter, so the wait before an edge is for everything outstanding.
+            s(f"i64 e = {first};")
+            s.open(f"if (e < {last})")
+            self._emit_stage3_issue(s, "A", "e")
+            s.close()
+            s.open(f"while (e < {last})")
+            s("const i64 en = e + 1;")
+            s(vmcnt(0))
+            s.open(f"if (en < {last})")
+            self._emit_stage3_issue(s, "B", "en")
+            s.close()
+            if before_edge:
+                before_edge("e")
+            compute("A", "e")
+            s(lgkm0)
+            s.open(f"if (en < {last})")
+            s(vmcnt(0))
+            s.open(f"if (e + 2 < {last})")
+            self._emit_stage3_issue(s, "A", "e + 2")
+            s.close()
+            if before_edge:
+                before_edge("en")
+            compute("B", "en")
+            s(lgkm0)
+            s.close()
+            s("e += 2;")
+            s.close()
+            return
+        if pipelined == 2:
+            # one LDS buffer per wave, copied to registers before the next edge's loads are issued
+            s(f"T yn[{self.low.L2}];")
+            s(f"i64 e = {first};")
+            s.open(f"if (e < {last})")
+            self._emit_stage_issue(s, "e")
+            s.close()
+            s.open(f"while (e < {last})")
+            s(vmcnt(0))
+            self._emit_stage_read(s, "A")
+            s(lgkm0)
+            s.open(f"if (e + 1 < {last})")
+            self._emit_stage_issue(s, "e + 1")
+            s.close()
+            if before_edge:
+                before_edge("e")
+            compute("A", "e")
+            s("++e;")
+            s.close()
+            return
         if not pipelined:
             s.open(f"for (i64 e = {first}; e < {last}; e += {R})")
             if before_edge:
@@ -360,6 +578,17 @@ class UvuEmitter:
         s(f"e += {2 * R};")
         s.close()
 
+    def _edge_mode(self, pipelined: int) -> int:
+        """0: load, then compute; 1: next edge's operands prefetched into a second register set;
+        2: next edge's operands prefetched into the wave's LDS staging buffer."""
+        if pipelined == 3 and self.stage3 is not None:
+            return 3
+        if pipelined >= 2 and self.stage is not None:
+            return 2
+        if pipelined and self.can_preload:
+            return 1
+        return 0
+
     def _node_loop_open(self, s: Src, G: int, xcd: int):
         """One wave group per receiver node. Workgroups are handed to the XCDs
         round-robin; with ``xcd`` > 1 (grid a multiple of it) block ids are remapped
@@ -377,7 +606,7 @@ class UvuEmitter:
         low = self.low
         block = 64 * self.NCH * G
         R = self.R
-        pipelined = pipelined and self.can_preload
+        mode = self._edge_mode(pipelined)
         s.open(
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void forward(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
@@ -387,6 +616,13 @@ class UvuEmitter:
         self._lane_prologue(s)
         if self.can_preload:
             s("E_t A, B;")
+        if mode == 2:
+            s(f"__shared__ __attribute__((aligned(16))) T s_stage[{self.NCH * G}][{self.stage['floats']}];")
+            self._emit_stage_offsets(s)
+        if mode == 3:
+            for b in "AB":
+                s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
+            self._emit_stage3_offsets(s)
 
         def make_load(si):
             def load(buf, e):
@@ -396,7 +632,9 @@ class UvuEmitter:
 
         def make_compute(si):
             def compute(buf, e):
-                if self.can_preload:
+                if mode == 3:
+                    s(f"fwd_seg{si}_lds(&s_stage{buf}[wave][0], ul, a);")
+                elif self.can_preload:
                     s(f"fwd_seg{si}_pre({buf}, a);")
                 else:
                     s.open("")
@@ -416,7 +654,7 @@ class UvuEmitter:
             for si in range(len(self.segments)):
                 s.open("")
                 s(f"A{si}_t a; zero_seg{si}(a);")
-                self._edge_loop(s, "e0 + r", "e1", make_load(si), make_compute(si), pipelined)
+                self._edge_loop(s, "e0 + r", "e1", make_load(si), make_compute(si), mode)
                 if R > 1:
                     # fold the R lane groups (fixed order) into group 0
                     for io in self.segments[si]:
@@ -453,7 +691,7 @@ class UvuEmitter:
                     s.close()
                     s.close()
 
-                self._edge_loop(s, "eb + r", "ee", make_load(si), make_compute(si), pipelined, before_edge)
+                self._edge_loop(s, "eb + r", "ee", make_load(si), make_compute(si), mode, before_edge)
                 s.open("if (cur >= 0)")
                 s(f"T* zrow = L3_out + cur * {low.L3};")
                 self._store_seg(s, si, "zrow", "true", atomic=True)
@@ -508,32 +746,35 @@ class UvuEmitter:
                 prods = self._products(s, p, v, yacc)
                 s(f"const T wv = {wacc(p, v)};")
                 ks = sorted({k for _, _, k, _ in p.nnz})
+                js = sorted({j for _, j, _, _ in p.nnz})
+                # dX: dx_i += (|c| y_j) * (g_k w)
                 for k in ks:
                     s(f"const T gw{k} = {gname(k)} * wv;")
-                fstart = set()
                 for n, (i, j, k, c) in enumerate(p.nnz):
                     q, neg = prods[n]
                     s(f"dx.b{p.i1}[{i}] {'-=' if neg else '+='} {q} * gw{k};")
-                    if k not in fstart:
-                        s(f"T f{k} = {'-' if neg else ''}{q} * {xname}.b{p.i1}[{i}];")
-                        fstart.add(k)
+                # h_j = sum_ik c x_i g_k is the unweighted dY term of this lane; it also gives
+                # dW = sum_j y_j h_j, so the forward contraction need not be recomputed
+                pair, hstart = {}, set()
+                for n, (i, j, k, c) in enumerate(p.nnz):
+                    if (i, k) not in pair:
+                        pair[(i, k)] = f"xg{len(pair)}"
+                        s(f"const T {pair[(i, k)]} = {self._xv(xname, p.i1, i)} * {gname(k)};")
+                    if j not in hstart:
+                        s(f"T h{j} = T({self.lit(c)}) * {pair[(i, k)]};")
+                        hstart.add(j)
                     else:
-                        s(f"f{k} {'-=' if neg else '+='} {q} * {xname}.b{p.i1}[{i}];")
-                terms = [f"{gname(k)} * f{k}" for k in ks]
-                s(f"T dwv = {terms[0]};")
-                for t in terms[1:]:
-                    s(f"dwv += {t};")
+                        s(f"h{j} += T({self.lit(c)}) * {pair[(i, k)]};")
+                s(f"T dwv = y{js[0]} * h{js[0]};")
+                for j in js[1:]:
+                    s(f"dwv += y{j} * h{j};")
                 if dw_mode == "store":
                     s(f"if (u < {b1.mul}{' && ' + dw_guard if dw_guard else ''}) "
                       f"dwrow[{p.woff} + u * {V} + ({v})] = dwv;")
                 else:
                     s(f"dwacc[{base_slot} + {v}] += dwv;")
-                pair = {}
-                for n, (i, j, k, c) in enumerate(p.nnz):
-                    if (i, k) not in pair:
-                        pair[(i, k)] = f"xg{len(pair)}"
-                        s(f"const T {pair[(i, k)]} = {xname}.b{p.i1}[{i}] * gw{k};")
-                    s(f"dy[{b2.off} + ({v}) * {b2.d} + {j}] += T({self.lit(c)}) * {pair[(i, k)]};")
+                for j in js:
+                    s(f"dy[{b2.off} + ({v}) * {b2.d} + {j}] += wv * h{j};")
 
             self._for_v(s, p, body)
             s.close()
@@ -696,7 +937,7 @@ class UvuEmitter:
         if self.NCH > 1:
             G = 1  # one node (or edge range) per block: the per-edge dY reduction uses block barriers
         block = 64 * self.NCH * G
-        pipelined = pipelined and self.can_preload
+        mode = self._edge_mode(pipelined)
         if self.can_preload:
             self._emit_load_edge(s, "load_edge_b", self.used_in1, low.paths)
         s.open(
@@ -714,6 +955,13 @@ class UvuEmitter:
             s(f"for (int t = 0; t < {self.n_wslots}; ++t) dwacc[t] = T(0);")
         if self.can_preload:
             s("E_t A, B;")
+        if mode == 2:
+            s(f"__shared__ __attribute__((aligned(16))) T s_stage[{self.NCH * G}][{self.stage['floats']}];")
+            self._emit_stage_offsets(s)
+        if mode == 3:
+            for b in "AB":
+                s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
+            self._emit_stage3_offsets(s)
         resident = deterministic and (self.g_resident if g_resident is None else g_resident)
 
         def load(buf, e):
@@ -723,7 +971,10 @@ class UvuEmitter:
         def make_compute(grow_expr_of):
             def compute(buf, e):
                 s.open("")
-                if self.can_preload:
+                if mode == 3:
+                    s(f"const T* sb = &s_stage{buf}[wave][0];")
+                    xname, yacc, wacc = self._acc_staged3("sb")
+                elif self.can_preload:
                     yacc, wacc = self._acc_preloaded(buf)
                     xname = f"{buf}.x"
                 else:
@@ -765,7 +1016,7 @@ class UvuEmitter:
                 self._load_g(s, f"L3_grad + node * {low.L3}", self.used_out)
             # with more than one chunk all waves of the block walk the same edges, so the
             # block barriers of the dY reduction are reached uniformly
-            self._edge_loop(s, "e0 + r", "e1", load, make_compute(lambda e: f"L3_grad + node * {low.L3}"), pipelined)
+            self._edge_loop(s, "e0 + r", "e1", load, make_compute(lambda e: f"L3_grad + node * {low.L3}"), mode)
             s.close()
         else:
             s(f"const i64 ngrp = (i64)gridDim.x * {G};")
@@ -773,7 +1024,7 @@ class UvuEmitter:
             s(f"const i64 eb = ((i64)blockIdx.x * {G} + g) * per;")
             s("const i64 ee = (eb + per < nnz) ? eb + per : nnz;")
             self._edge_loop(s, "eb + r", "ee", load, make_compute(lambda e: f"L3_grad + rows[{e}] * {low.L3}"),
-                            pipelined)
+                            mode)
         if shared:
             # shared weights: one atomic add per weight per wave (atomic mode only)
             for p, slot in self._dw_slots():
@@ -822,8 +1073,8 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256):
     from .. import runtime as rt
 
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
-    t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=1, conv_pipe_b=0,
-                    conv_wf=0, conv_wb=2, conv_gres=-1, conv_xcd=8))
+    t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
+                    conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8))
     em = UvuEmitter(low, acc_budget_words=t["conv_acc"])
     s = Src()
     s(prelude(low.ctype))
@@ -833,9 +1084,9 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256):
     G_f = t["conv_gf"]
     G_b = 1 if em.NCH > 1 else t["conv_gb"]
     xcd = max(1, t["conv_xcd"])
-    blk_f = em.emit_conv_forward(s, G_f, deterministic, bool(t["conv_pipe_f"]), t["conv_wf"], xcd)
+    blk_f = em.emit_conv_forward(s, G_f, deterministic, t["conv_pipe_f"], t["conv_wf"], xcd)
     gres = None if t["conv_gres"] < 0 else bool(t["conv_gres"])
-    blk_b = em.emit_conv_backward(s, deterministic, G_b, bool(t["conv_pipe_b"]), t["conv_wb"], gres, xcd)
+    blk_b = em.emit_conv_backward(s, deterministic, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd)
     descs = [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, compute_units * 16),
