@@ -84,6 +84,7 @@ class UvuEmitter:
             all(low.in2[p.i2].mul <= UNROLL_V_LIMIT for p in low.paths) and low.L2 <= 32 and self.n_wslots <= 64
         )
 
+        self.tr_atomics = False  # set by the conv kernels that declare the s_tr tile
         self.stage = self._stage_layout()
         self.stage3 = self._stage3_layout()
 
@@ -409,8 +410,33 @@ class UvuEmitter:
             if preloaded and self.stage3 is not None:
                 self._emit_fwd_seg(s, si, "lds")
 
+    def _regular_wave(self) -> bool:
+        """Every used block is exactly 64 channels per wave-chunk and a row fills the wave."""
+        low = self.low
+        U = 64 * self.NCH
+        return (self.R == 1 and all(low.in1[b].mul == U for b in self.used_in1)
+                and all(low.out[io].mul == U for io in self.used_out))
+
+    def _atomic_block_transposed(self, s: Src, rowexpr: str, off: int, d: int, val: Callable[[int], str]):
+        """Atomic accumulation of one [64 x d] channel block. The lane-per-channel registers go
+        through a wave-private LDS tile so that every atomic instruction of the wave covers 64
+        consecutive elements (two cache lines) instead of 64 elements ``d`` apart."""
+        # lanes exchange data through the tile: the wave-scope fences keep the compiler from
+        # reordering one lane's reads against its own (different-address) writes
+        s("oeq_wave_sync();")
+        for k in range(d):
+            s(f"s_tr[wave][ul * {d} + {k}] = {val(k)};")
+        s("oeq_wave_sync();")
+        for t in range(d):
+            s(f"oeq_atomic_add({rowexpr} + {off} + chunk * {64 * d} + {t * 64} + ul, s_tr[wave][{t * 64} + ul]);")
+
     def _store_seg(self, s: Src, si: int, rowexpr: str, guard: str, atomic: bool = False):
         low = self.low
+        if atomic and self.tr_atomics:
+            for io in self.segments[si]:
+                bo = low.out[io]
+                self._atomic_block_transposed(s, rowexpr, bo.off, bo.d, lambda k, io=io: f"a.o{io}[{k}]")
+            return
         for io in self.segments[si]:
             bo = low.out[io]
             s.open(f"if ({guard} && u < {bo.mul})")
@@ -602,7 +628,7 @@ class UvuEmitter:
             s.open(f"for (i64 node = (i64)blockIdx.x * {G} + g; node < node_count; node += (i64)gridDim.x * {G})")
 
     def emit_conv_forward(self, s: Src, G: int, deterministic: bool, pipelined: bool, waves_per_eu: int = 0,
-                          xcd: int = 1):
+                          xcd: int = 1, tr_atomics: bool = True):
         low = self.low
         block = 64 * self.NCH * G
         R = self.R
@@ -623,6 +649,9 @@ class UvuEmitter:
             for b in "AB":
                 s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
             self._emit_stage3_offsets(s)
+        self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave()
+        if self.tr_atomics:
+            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.out[io].d for io in self.used_out)}];")
 
         def make_load(si):
             def load(buf, e):
@@ -836,6 +865,11 @@ class UvuEmitter:
 
     def _store_dx(self, s: Src, rowexpr: str, guard: str, atomic: bool = False):
         low = self.low
+        if atomic and self.tr_atomics:
+            for b in self.used_in1:
+                blk = low.in1[b]
+                self._atomic_block_transposed(s, rowexpr, blk.off, blk.d, lambda i, b=b: f"dx.b{b}[{i}]")
+            return
         for b in self.used_in1:
             blk = low.in1[b]
             s.open(f"if ({guard} && u < {blk.mul})")
@@ -931,7 +965,7 @@ class UvuEmitter:
 
     # -------------------------------------------------------- conv backward
     def emit_conv_backward(self, s: Src, deterministic: bool, G: int, pipelined: bool, waves_per_eu: int = 0,
-                           g_resident: Optional[bool] = None, xcd: int = 1):
+                           g_resident: Optional[bool] = None, xcd: int = 1, tr_atomics: bool = True):
         low = self.low
         shared = low.shared_weights
         if self.NCH > 1:
@@ -962,6 +996,9 @@ class UvuEmitter:
             for b in "AB":
                 s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
             self._emit_stage3_offsets(s)
+        self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave()
+        if self.tr_atomics:
+            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.in1[b].d for b in self.used_in1)}];")
         resident = deterministic and (self.g_resident if g_resident is None else g_resident)
 
         def load(buf, e):
@@ -1074,7 +1111,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256):
 
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
     t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
-                    conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8))
+                    conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1))
     em = UvuEmitter(low, acc_budget_words=t["conv_acc"])
     s = Src()
     s(prelude(low.ctype))
@@ -1084,9 +1121,9 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256):
     G_f = t["conv_gf"]
     G_b = 1 if em.NCH > 1 else t["conv_gb"]
     xcd = max(1, t["conv_xcd"])
-    blk_f = em.emit_conv_forward(s, G_f, deterministic, t["conv_pipe_f"], t["conv_wf"], xcd)
+    blk_f = em.emit_conv_forward(s, G_f, deterministic, t["conv_pipe_f"], t["conv_wf"], xcd, bool(t["conv_tra"]))
     gres = None if t["conv_gres"] < 0 else bool(t["conv_gres"])
-    blk_b = em.emit_conv_backward(s, deterministic, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd)
+    blk_b = em.emit_conv_backward(s, deterministic, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd, bool(t["conv_tra"]))
     descs = [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, compute_units * 16),
