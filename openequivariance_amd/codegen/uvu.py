@@ -1082,7 +1082,11 @@ def tp_module(low: Lowered, compute_units: int = 256):
     """Source + launch descriptors for the batch tensor product (forward, backward)."""
     from .. import runtime as rt
 
-    t = tuning(dict(tp_acc=48, tp_gf=max(1, 4 // low.n_chunks), tp_gb=max(1, 4 // low.n_chunks), tp_wf=0, tp_wb=0))
+    # occupancy hints measured on MI355X: wide (multi-chunk) fp32 rows run best at 2 waves/SIMD, narrow ones
+    # at 2 (forward) and 3 (backward); fp64 is left to the compiler
+    f32 = low.elem_size == 4
+    t = tuning(dict(tp_acc=48, tp_gf=max(1, 4 // low.n_chunks), tp_gb=max(1, 4 // low.n_chunks),
+                    tp_wf=2 if f32 else 0, tp_wb=(2 if low.n_chunks > 1 else 3) if f32 else 0))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     s = Src()
     s(prelude(low.ctype))
