@@ -33,6 +33,8 @@ def parse():
     ap.add_argument("--atomic-steps", type=int, default=3)
     ap.add_argument("--cpu-receivers", type=int, default=48, help="receivers in the CPU-baseline sub-graph (0 = skip)")
     ap.add_argument("--no-atomic", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the side measurements (spatially ordered nodes, batch tensor-product configs)")
     return ap.parse_args()
 
 
@@ -93,6 +95,67 @@ def cpu_baseline(problem, graph, Ysh, n_receivers, seed=0):
                   f"torch-CPU einsum + index_add restatement of e3nn (e3nn not installed), fp32, {reps} reps",
         "seconds_per_step": dt, "host_cpus": cores,
     }
+
+
+def tp_config_table(dev):
+    """Side measurements: the batched tensor product at configs 1-4 (forward and backward timed
+    separately, median of 10). Bytes = every operand once per row (shared weights once per call);
+    FLOPs by the reference's convention, and dense 2*u*w*(2l+1) per path for the MFMA config."""
+    import numpy as np
+    import torch
+
+    import openequivariance_amd as oeq
+    from openequivariance_amd._torch import ops
+    from openequivariance_amd.codegen.lower import lower
+    from openequivariance_amd.core import problems as P
+
+    def med(fn, warm=3, it=10):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(it):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b))
+        return float(np.median(ts))
+
+    cases = [("cfg1 single uvu f32", P.config1_single_uvu(), 100000), ("cfg2 nequip uvu f32", P.config2_nequip_uvu(), 200000),
+             ("cfg3 mace uvu f32", P.config3_mace_uvu(), 500000), ("cfg3 mace uvu f64", P.config3_mace_uvu(np.float64), 500000),
+             ("cfg4 uvw shared f32 (MFMA)", P.config4_uvw_shared(), 262144)]
+    table = []
+    for name, prob, B in cases:
+        low = lower(prob)
+        es = low.elem_size
+        dt = torch.float32 if es == 4 else torch.float64
+        x = torch.randn(B, low.L1, device=dev, dtype=dt)
+        y = torch.randn(B, low.L2, device=dev, dtype=dt)
+        w = torch.randn((low.WN,) if prob.shared_weights else (B, low.WN), device=dev, dtype=dt)
+        g = torch.randn(B, low.L3, device=dev, dtype=dt)
+        tp = oeq.TensorProduct(prob)
+        tf = med(lambda: ops.tp_forward(x, y, w, tp.kid))
+        tb = med(lambda: ops.tp_backward(x, y, w, g, tp.kid))
+        wrow = 0 if prob.shared_weights else low.WN
+        wcall = low.WN * es if prob.shared_weights else 0
+        fb = B * (low.L1 + low.L2 + low.L3 + wrow) * es + wcall
+        bb = B * (2 * low.L1 + 2 * low.L2 + low.L3 + 2 * wrow) * es + 2 * wcall
+        row = {"config": name, "rows": B, "fwd_ms": tf, "bwd_ms": tb,
+               "fwd_rows_per_s": B / tf * 1e3, "bwd_rows_per_s": B / tb * 1e3,
+               "fwd_gflops": B * low.flops("forward") / tf / 1e6, "bwd_gflops": B * low.flops("backward") / tb / 1e6,
+               "fwd_hbm_frac": fb / tf / 1e6 / HBM_PEAK_GBS, "bwd_hbm_frac": bb / tb / 1e6 / HBM_PEAK_GBS}
+        if low.mode == "uvw":
+            dense = sum(2 * low.in1[p.i1].mul * low.in2[p.i2].mul * low.out[p.io].mul * low.out[p.io].d for p in low.paths)
+            row["fwd_dense_tflops"] = B * dense / tf / 1e9
+            row["bwd_dense_tflops"] = 2 * B * dense / tb / 1e9
+            row["fwd_mfma_frac"] = row["fwd_dense_tflops"] / 157.3
+            row["bwd_mfma_frac"] = row["bwd_dense_tflops"] / 157.3
+        table.append(row)
+        del x, y, w, g
+        torch.cuda.empty_cache()
+    return table
 
 
 def main():
@@ -199,9 +262,47 @@ def main():
         }
         del Ya, Wa
 
+    extras = {}
+    if not args.no_extras:
+        # Same graph with nodes numbered along a Z-order curve (core/graph.py: spatial_order): a
+        # relabelling the caller can apply once per structure; it lets gathered sender rows hit in L2.
+        from openequivariance_amd.core.graph import relabel_nodes, spatial_order
+        order_n = spatial_order(coords)
+        rows_s, cols_s = relabel_nodes(order_n, rows, cols)
+        gs = CoordGraph(coords[order_n], rows_s, cols_s, "periodic-radius-zorder")
+        # edge e of `graph` is edge graph.order[e] of the generated list; reuse its Y/W rows by matching edge ids
+        Ys = torch.tensor(spherical_harmonics(3, vec).astype(np.float32)[gs.order], device=dev)
+        trs, tcs, tps = (torch.tensor(a, device=dev) for a in (gs.rows, gs.cols, gs.transpose_perm))
+
+        def step_sp():
+            ops.conv_forward(X, Ys, W, trs, tcs, tps, kid)
+            ops.conv_backward(X, Ys, W, G, trs, tcs, tps, kid)
+
+        ms_sp = time_steps(step_sp, args.steps, args.warmup)
+        modes["deterministic_zorder_nodes"] = {
+            "ms_per_step": ms_sp, "edges_per_s": E / (ms_sp * 1e-3),
+            "gflops": (fwd_flops + bwd_flops) * E / (ms_sp * 1e-3) / 1e9,
+            "hbm_roofline_frac": (fwd_bytes + bwd_bytes) / (ms_sp * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        }
+        del Ys, trs, tcs, tps
+
     cpu = None
     if args.cpu_receivers > 0:
         cpu = cpu_baseline(problem, graph, Ysh, args.cpu_receivers)
+
+    if not args.no_extras:
+        del X, W, G, Y
+        torch.cuda.empty_cache()
+        extras["tp_configs"] = tp_config_table(dev)
+
+    traffic_path = os.path.join(ROOT, "profiles", "conv_cfg5_traffic.json")
+    if os.path.exists(traffic_path):
+        # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+        # this same command (scaled by a copy-kernel calibration); see profiles/conv_cfg5_deterministic.md
+        with open(traffic_path) as f:
+            tr = json.load(f)
+        if tr.get("edges") == E:
+            roofline["traffic"] = tr["backward_bytes_per_launch"]
 
     out = {
         "metric": "fused conv fwd+bwd edges/s at MACE shape (deterministic mode)",
@@ -220,6 +321,7 @@ def main():
         "cpu_baseline": cpu,
         "modes": modes,
     }
+    out.update(extras)
     print(json.dumps(out))
 
 

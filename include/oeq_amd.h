@@ -77,6 +77,8 @@ typedef enum {
     OEQ_ROLE_COUNT = 8
 } oeq_role;
 
+/* Several descriptors may name the same role: those kernels are launched back to back, in
+ * descriptor order, with the same arguments and launch shape (that of the last descriptor). */
 typedef struct {
     int32_t role;               /* oeq_role */
     const char* kernel_name;    /* __global__ symbol (extern "C") in the code object */

@@ -9,18 +9,31 @@ reference does this mix with a scalar-FMA warp matmul on 32-wide chunks
 (openequivariance/openequivariance/templates/wmm.cuh:1-87,
 loop_unroll_tp.cuh:55-84, 217-272).
 
-Work decomposition: a block of 4 waves owns a tile of 16 batch rows at a time.
+Work decomposition: a block of 4 waves owns a tile of 16 batch rows at a time;
+wave ``w`` owns output channels (forward) or input channels (backward)
+``16w .. 16w+15`` of every 64-channel block. Forward and backward are each a
+short sequence of kernels launched back to back with the same arguments:
 
-* forward: the block computes T of one path for the tile into LDS (lanes = u,
-  4 rows per wave), then each wave multiplies the 16 x d3 row block with its own
-  16-wide slices of the output channels; accumulators of an output irrep live in
-  registers across all paths that feed it.
-* backward: the dZ tile is staged in LDS once. Per path, G = dZ W^T comes out of
-  MFMA in a layout (lane = 4 rows x one channel) on which the vector-ALU part
-  (dX, dY and T) runs directly; T goes to LDS and the weight gradient
-  dW += T^T dZ is accumulated by MFMA in registers over all tiles of the block
-  (wave = 16-channel slice of u). Blocks write partial weight gradients that a
-  second kernel sums in block order: no atomics, deterministic.
+* forward, one kernel per output irrep: the wave's slices of the weight
+  matrices of the paths feeding that irrep stay in registers in MFMA B-operand
+  layout (16 registers per path) for the whole kernel. Per path the block
+  computes T for the tile into LDS (lanes = u, 4 rows per wave; the X values of
+  the next path are fetched into registers while the current path's MFMAs run),
+  then each wave multiplies the 16 x d3 row block by its weight slice. The T
+  tile is double buffered: one block barrier per path.
+* backward, one kernel per input irrep (dX and the dY terms of its paths): the
+  dZ tile is staged in LDS; per path G = dZ W^T comes out of MFMA in a layout
+  (lane = 4 rows x one channel) on which the vector-ALU part runs directly, with
+  W^T slices register-resident. A tile is always handled by the same thread of
+  the same block, so later kernels add their dY terms with plain
+  read-modify-writes in a fixed order.
+* backward, one kernel per output irrep (dW of the paths feeding it): T is
+  recomputed into LDS and dW += T^T dZ is accumulated by MFMA in registers over
+  all tiles of the block. Blocks write partial weight gradients that a last
+  kernel sums in block order: no atomics, deterministic.
+
+Splitting by irrep keeps each kernel under 256 registers (two waves per SIMD),
+so one wave's LDS/global latencies hide behind the other's MFMAs.
 
 Operand layouts of v_mfma_f32_16x16x4_f32 used below (lane l of 64):
 A[m][k]: m = l % 16, k = l / 16;  B[k][n]: k = l / 16, n = l % 16;
@@ -37,6 +50,7 @@ from .lower import Lowered, Path, float_literal
 RT = 16          # rows per tile
 WAVES = 4        # waves per block
 TPAD = RT + 1    # padded row stride of the T tile in LDS (bank spread)
+MFMA = "__builtin_amdgcn_mfma_f32_16x16x4f32"
 
 
 def supported(low: Lowered) -> bool:
@@ -46,35 +60,34 @@ def supported(low: Lowered) -> bool:
         return False
     for p in low.paths:
         a, b, o = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
-        if b.mul != 1 or a.mul != 64 or o.mul % 64 != 0 or o.mul > 256:
+        if b.mul != 1 or a.mul != 64 or o.mul != 64:
             return False
-    n_dw = sum((low.in1[p.i1].mul // 64) * (low.out[p.io].mul // 16) * 4 for p in low.paths)
-    return n_dw <= 256
-
-
-def _pow2ceil(n: int) -> int:
-    return 1 << max(0, (n - 1).bit_length())
+    return 16 * len(low.paths) <= 192
 
 
 class MfmaEmitter:
     def __init__(self, low: Lowered):
         self.low = low
         self.max_d3 = max(low.out[p.io].d for p in low.paths)
-        self.gstride = low.L3 + (1 if low.L3 % 32 != 1 else 0)  # odd-ish row stride of the dZ tile in LDS
-        if self.gstride % 2 == 0:
+        self.max_d1 = max(low.in1[p.i1].d for p in low.paths)
+        self.gstride = low.L3 + 1
+        while self.gstride % 32 != 1:
             self.gstride += 1
+        # order in which the forward / dW sweeps visit the paths: grouped by output block
+        self.fwd_order: List[Path] = [p for io in range(len(low.out)) for p in low.paths if p.io == io]
+        from .uvu import tuning
+        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2))
 
     def lit(self, v):
         return float_literal(v, "float")
 
-    # ---- CG part of one path for one (row, channel): t_k, and in the backward dx, dy
+    # ---- CG part of one path for one (row, channel)
     def _emit_path_fns(self, s: Src):
         low = self.low
         for p in low.paths:
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
-            js = sorted({j for _, j, _, _ in p.nnz})
 
-            def products():
+            def products(p=p, b2=b2):
                 names, out = {}, {}
                 for n, (i, j, k, c) in enumerate(p.nnz):
                     key = (self.lit(abs(c)), j)
@@ -84,206 +97,267 @@ class MfmaEmitter:
                     out[n] = (names[key], c < 0)
                 return out
 
-            # forward: t[k] = sum c x_i y_j
-            s.open(f"OEQ_DEV void cg_fwd{p.index}(const T* __restrict__ xp, const T* __restrict__ y, T (&t)[{bo.d}])")
-            for i in range(b1.d):
-                s(f"const T x{i} = xp[{i}];")
+            # t[k] = sum c x_i y_j
+            s.open(f"OEQ_DEV void cg_fwd{p.index}(const T (&x)[{self.max_d1}], const T* y, T (&t)[{bo.d}])")
             prods = products()
             started = set()
             for n, (i, j, k, c) in enumerate(p.nnz):
                 q, neg = prods[n]
                 if k not in started:
-                    s(f"t[{k}] = {'-' if neg else ''}{q} * x{i};")
+                    s(f"t[{k}] = {'-' if neg else ''}{q} * x[{i}];")
                     started.add(k)
                 else:
-                    s(f"t[{k}] {'-=' if neg else '+='} {q} * x{i};")
+                    s(f"t[{k}] {'-=' if neg else '+='} {q} * x[{i}];")
             for k in range(bo.d):
                 if k not in started:
                     s(f"t[{k}] = T(0);")
             s.close()
-            # backward: given G[k] = sum_w W[u,w] dZ[w,k]
+            # given G[k] = sum_w W[u,w] dZ[w,k]:  dx_i += c y_j G_k,  dy_j += c x_i G_k
             s.open(
-                f"OEQ_DEV void cg_bwd{p.index}(const T* __restrict__ xp, const T* y, const T (&G)[{bo.d}], "
-                f"T (&dx)[{b1.d}], T (&dy)[{low.L2}], T (&t)[{bo.d}])"
+                f"OEQ_DEV void cg_bwd{p.index}(const T (&x)[{self.max_d1}], const T* y, const T (&G)[{bo.d}], "
+                f"T (&dx)[{b1.d}], T (&dy)[{low.L2}])"
             )
-            for i in range(b1.d):
-                s(f"const T x{i} = xp[{i}];")
             prods = products()
-            started = set()
             for n, (i, j, k, c) in enumerate(p.nnz):
                 q, neg = prods[n]
                 s(f"dx[{i}] {'-=' if neg else '+='} {q} * G[{k}];")
-                if k not in started:
-                    s(f"t[{k}] = {'-' if neg else ''}{q} * x{i};")
-                    started.add(k)
-                else:
-                    s(f"t[{k}] {'-=' if neg else '+='} {q} * x{i};")
-            for k in range(bo.d):
-                if k not in started:
-                    s(f"t[{k}] = T(0);")
             pair = {}
             for n, (i, j, k, c) in enumerate(p.nnz):
                 if (i, k) not in pair:
                     pair[(i, k)] = f"xg{len(pair)}"
-                    s(f"const T {pair[(i, k)]} = x{i} * G[{k}];")
+                    s(f"const T {pair[(i, k)]} = x[{i}] * G[{k}];")
                 s(f"dy[{b2.off + j}] += T({self.lit(c)}) * {pair[(i, k)]};")
             s.close()
 
-    # ------------------------------------------------------------- forward
-    def emit_forward(self, s: Src):
-        low = self.low
-        s.open(
-            f'extern "C" __global__ __launch_bounds__({64 * WAVES}) void forward(i64 num_batch, '
-            "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, T* __restrict__ L3_out)"
-        )
-        s(f"__shared__ T s_T[{self.max_d3}][64][{TPAD}];")
-        s("const int lane = oeq_lane();")
-        s("const int wave = oeq_wave();")
-        s("const int l16 = lane & 15, lq = lane >> 4;")
-        s(f"const i64 ntiles = (num_batch + {RT - 1}) / {RT};")
-        s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
-        s(f"const i64 row0 = tile * {RT};")
-        for io, bo in enumerate(low.out):
-            paths = [p for p in low.paths if p.io == io]
-            ntw = bo.mul // 64  # 16-wide output slices per wave
-            s(f"// ---- out[{io}]: {bo.mul} x l={bo.l}")
-            s.open("")
-            s(f"v4f acc[{bo.d}][{ntw}];")
-            for k in range(bo.d):
-                for j in range(ntw):
-                    s(f"acc[{k}][{j}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
-            for p in paths:
-                b1 = low.in1[p.i1]
-                s(f"// path {p.index}: l=({b1.l},{low.in2[p.i2].l},{bo.l})")
-                s.open(f"for (int uc = 0; uc < {b1.mul}; uc += 64)")
-                s("__syncthreads();")
-                s.open(f"for (int rr = 0; rr < {RT // WAVES}; ++rr)")
-                s(f"const int r = wave * {RT // WAVES} + rr;")
-                s("i64 row = row0 + r; if (row >= num_batch) row = num_batch - 1;")
-                s(f"T t[{bo.d}];")
-                s(f"cg_fwd{p.index}(L1_in + row * {low.L1} + {b1.off} + (uc + lane) * {b1.d}, L2_in + row * {low.L2}, t);")
-                for k in range(bo.d):
-                    s(f"s_T[{k}][lane][r] = t[{k}];")
-                s.close()
-                s("__syncthreads();")
-                s("#pragma unroll 4")
-                s.open("for (int st = 0; st < 16; ++st)")
-                for k in range(bo.d):
-                    s(f"const T a{k} = s_T[{k}][4 * st + lq][l16];")
-                for j in range(ntw):
-                    s(f"const T b{j} = W[{p.woff} + (i64)(uc + 4 * st + lq) * {bo.mul} + {16 * WAVES * j} + wave * 16 + l16];")
-                for j in range(ntw):
-                    for k in range(bo.d):
-                        s(f"acc[{k}][{j}] = __builtin_amdgcn_mfma_f32_16x16x4f32(a{k}, b{j}, acc[{k}][{j}], 0, 0, 0);")
-                s.close()
-                s.close()
-            # D layout: rows 4*lq + i, column (channel) l16 of the wave's slice
-            for j in range(ntw):
-                s.open("for (int i = 0; i < 4; ++i)")
-                s("const i64 row = row0 + 4 * lq + i;")
-                s.open("if (row < num_batch)")
-                s(f"T* zp = L3_out + row * {low.L3} + {bo.off} + ({16 * WAVES * j} + wave * 16 + l16) * {bo.d};")
-                for k in range(bo.d):
-                    s(f"zp[{k}] = acc[{k}][{j}][i];")
-                s.close()
-                s.close()
-            s.close()
-        s.close()
-        s.close()
-
-    # ------------------------------------------------------------ backward
-    def dw_layout(self) -> Dict[int, Tuple[int, int]]:
-        """path -> (first accumulator index, number of 16-wide w slices)."""
-        out, n = {}, 0
-        for p in self.low.paths:
-            nw = self.low.out[p.io].mul // 16
-            out[p.index] = (n, nw)
-            n += nw
-        self.n_dw = n
-        return out
-
-    def _stage_tile(self, s: Src, with_y: bool):
-        low = self.low
-        s("__syncthreads();")
-        s.open(f"for (int t = tid; t < {RT * low.L3}; t += {64 * WAVES})")
-        s(f"const int r = t / {low.L3}, c = t % {low.L3};")
-        s(f"s_g[r][c] = (row0 + r < num_batch) ? L3_grad[(row0 + r) * {low.L3} + c] : T(0);")
-        s.close()
-        if with_y:
-            s.open(f"for (int t = tid; t < {RT * low.L2}; t += {64 * WAVES})")
-            s(f"const int r = t / {low.L2}, c = t % {low.L2};")
-            s(f"s_y[r][c] = (row0 + r < num_batch) ? L2_in[(row0 + r) * {low.L2} + c] : T(0);")
-            s.close()
-        s("__syncthreads();")
-
-    def emit_backward(self, s: Src):
-        """Two sweeps over the block's tiles inside one kernel, so that the
-        register sets of the two halves (dX/dY state vs. the weight-gradient
-        accumulators) are never live together."""
-        low = self.low
-        dwl = self.dw_layout()
-        L2p = low.L2
-        s.open(
-            f'extern "C" __global__ __launch_bounds__({64 * WAVES}) void backward(i64 num_batch, '
-            "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
-            "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
-            "const T* __restrict__ L3_grad, T* __restrict__ wpartial)"
-        )
-        s(f"__shared__ T s_g[{RT}][{self.gstride}];")
-        s(f"__shared__ T s_T[{self.max_d3}][64][{TPAD}];")
-        s(f"__shared__ T s_y[{RT}][{L2p}];")
-        s(f"__shared__ T s_dy[{WAVES}][{RT}][{L2p}];")
+    def _prologue(self, s: Src):
         s("const int lane = oeq_lane();")
         s("const int wave = oeq_wave();")
         s("const int l16 = lane & 15, lq = lane >> 4;")
         s("const int tid = (int)threadIdx.x;")
         s(f"const i64 ntiles = (num_batch + {RT - 1}) / {RT};")
+        s("(void)tid; (void)lane;")
 
-        # ---------------- sweep 1: dX, dY --------------------------------------
-        s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
-        s(f"const i64 row0 = tile * {RT};")
-        self._stage_tile(s, with_y=True)
-        s(f"T dy[4][{L2p}];")
-        s(f"for (int i = 0; i < 4; ++i) for (int j = 0; j < {L2p}; ++j) dy[i][j] = T(0);")
+    def _stage_y(self, s: Src):
+        low = self.low
+        s.open(f"for (int t = tid; t < {RT * low.L2}; t += {64 * WAVES})")
+        s(f"const int r = t / {low.L2}, c = t % {low.L2};")
+        s(f"s_y[r][c] = (row0 + r < num_batch) ? L2_in[(row0 + r) * {low.L2} + c] : T(0);")
+        s.close()
+
+    def _stage_g(self, s: Src, col0: int = 0, ncols: int = None):
+        """dZ tile (columns col0 .. col0+ncols) -> LDS, rows past the batch zeroed. All loads of a
+        thread are issued before the first LDS store, so their latencies overlap."""
+        low = self.low
+        ncols = low.L3 if ncols is None else ncols
+        nthreads = 64 * WAVES
+        if low.L3 % 4 == 0 and col0 % 4 == 0 and ncols % 4 == 0:
+            nvec = RT * ncols // 4
+            iters = (nvec + nthreads - 1) // nthreads
+            s.open("")
+            s(f"float4 gv[{iters}];")
+            s("#pragma unroll")
+            s.open(f"for (int it = 0; it < {iters}; ++it)")
+            s(f"const int t = tid + it * {nthreads};")
+            s(f"const int r = t / {ncols // 4}, c = {col0} + (t % {ncols // 4}) * 4;")
+            s(f"gv[it] = (t < {nvec} && row0 + r < num_batch) ? "
+              f"*(const float4*)(L3_grad + (row0 + r) * {low.L3} + c) : make_float4(0.f, 0.f, 0.f, 0.f);")
+            s.close()
+            s("#pragma unroll")
+            s.open(f"for (int it = 0; it < {iters}; ++it)")
+            s(f"const int t = tid + it * {nthreads};")
+            s(f"const int r = t / {ncols // 4}, c = {col0} + (t % {ncols // 4}) * 4;")
+            s.open(f"if (t < {nvec})")
+            s("s_g[r][c] = gv[it].x; s_g[r][c + 1] = gv[it].y; s_g[r][c + 2] = gv[it].z; s_g[r][c + 3] = gv[it].w;")
+            s.close()
+            s.close()
+            s.close()
+        else:
+            s.open(f"for (int t = tid; t < {RT * ncols}; t += {nthreads})")
+            s(f"const int r = t / {ncols}, c = {col0} + t % {ncols};")
+            s(f"s_g[r][c] = (row0 + r < num_batch) ? L3_grad[(row0 + r) * {low.L3} + c] : T(0);")
+            s.close()
+
+    def _load_x_rows(self, s: Src, dst: str, p: Path):
+        """X of the wave's 4 rows for path p, lanes = channel u (T-compute layout)."""
+        low = self.low
+        b1 = low.in1[p.i1]
+        s.open(f"for (int rr = 0; rr < {RT // WAVES}; ++rr)")
+        s(f"i64 row = row0 + wave * {RT // WAVES} + rr; if (row >= num_batch) row = num_batch - 1;")
+        s(f"const T* xp = L1_in + row * {low.L1} + {b1.off} + lane * {b1.d};")
+        for i in range(b1.d):
+            s(f"{dst}[rr][{i}] = xp[{i}];")
+        s.close()
+
+    def _t_compute(self, s: Src, p: Path, xsrc: str, buf: str):
+        low = self.low
+        bo = low.out[p.io]
+        s.open(f"for (int rr = 0; rr < {RT // WAVES}; ++rr)")
+        s(f"const int r = wave * {RT // WAVES} + rr;")
+        s(f"T t[{bo.d}];")
+        s(f"cg_fwd{p.index}({xsrc}[rr], s_y[r], t);")
+        for k in range(bo.d):
+            s(f"s_T[{buf}][{k}][lane][r] = t[{k}];")
+        s.close()
+
+    # ------------------------------------------------------------- forward
+    def _load_wreg(self, s: Src, paths: List[Path], transposed: bool):
+        for p in paths:
+            s(f"T wreg{p.index}[16];")
+            s("#pragma unroll")
+            if transposed:  # B[k = w = 4 st + lq][n = l16] = W_p[u][w]
+                s(f"for (int st = 0; st < 16; ++st) wreg{p.index}[st] = W[{p.woff} + u * 64 + 4 * st + lq];")
+            else:           # B[k = u' = 4 st + lq][n = l16] = W_p[u'][w = 16 wave + l16]
+                s(f"for (int st = 0; st < 16; ++st) wreg{p.index}[st] = "
+                  f"W[{p.woff} + (4 * st + lq) * 64 + wave * 16 + l16];")
+
+    FWD_SIG = ("(i64 num_batch, const T* __restrict__ L1_in, const T* __restrict__ L2_in, "
+               "const T* __restrict__ W, T* __restrict__ L3_out)")
+    BWD_SIG = ("(i64 num_batch, const T* __restrict__ L1_in, T* __restrict__ L1_grad, "
+               "const T* __restrict__ L2_in, T* __restrict__ L2_grad, const T* __restrict__ W, "
+               "T* __restrict__ W_grad, const T* __restrict__ L3_grad, T* __restrict__ wpartial)")
+
+    def _kernel_open(self, s: Src, name: str, sig: str, waves_per_eu: int = 0):
+        attr = f"__launch_bounds__({64 * WAVES})"
+        if waves_per_eu:
+            attr += f" __attribute__((amdgpu_waves_per_eu({waves_per_eu}, {waves_per_eu})))"
+        s.open(f'extern "C" __global__ {attr} void {name}{sig}')
+
+    def emit_forward(self, s: Src) -> List[str]:
+        """One kernel per output irrep (launched back to back), so that only the weights of the
+        paths feeding that irrep (16 registers each) are resident and register allocation is per
+        irrep. Returns the kernel names in launch order."""
+        low = self.low
+        names = []
+        for io, bo in enumerate(low.out):
+            order = [p for p in low.paths if p.io == io]
+            name = "forward" if not names else f"forward_o{io}"
+            names.append(name)
+            s(f"// ======== out[{io}]: {bo.mul} x l={bo.l}")
+            self._kernel_open(s, name, self.FWD_SIG, self.tune["uvw_wf"])
+            if not order:
+                self._prologue(s)
+                s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
+                s(f"const i64 row0 = tile * {RT};")
+                s.open(f"for (int t = tid; t < {RT * bo.mul * bo.d}; t += {64 * WAVES})")
+                s(f"const int r = t / {bo.mul * bo.d}, c = t % {bo.mul * bo.d};")
+                s(f"if (row0 + r < num_batch) L3_out[(row0 + r) * {low.L3} + {bo.off} + c] = T(0);")
+                s.close()
+                s.close()
+                s.close()
+                continue
+            s(f"__shared__ T s_T[2][{bo.d}][64][{TPAD}];")
+            s(f"__shared__ T s_y[{RT}][{low.L2}];")
+            self._prologue(s)
+            s(f"T xa[{RT // WAVES}][{self.max_d1}], xb[{RT // WAVES}][{self.max_d1}];")
+            self._load_wreg(s, order, transposed=False)
+            s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
+            s(f"const i64 row0 = tile * {RT};")
+            s("__syncthreads();  // all reads of the previous tile's LDS data are done")
+            self._stage_y(s)
+            self._load_x_rows(s, "xa", order[0])
+            s("__syncthreads();")
+            s(f"v4f acc[{bo.d}];")
+            for k in range(bo.d):
+                s(f"acc[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+            cur, nxt = "xa", "xb"
+            for n, p in enumerate(order):
+                buf = n % 2
+                s(f"// path {p.index}: l=({low.in1[p.i1].l},{low.in2[p.i2].l},{bo.l})")
+                self._t_compute(s, p, cur, str(buf))
+                if n + 1 < len(order):
+                    self._load_x_rows(s, nxt, order[n + 1])
+                s("__syncthreads();")
+                s("#pragma unroll")
+                s.open("for (int st = 0; st < 16; ++st)")
+                for k in range(bo.d):
+                    s(f"acc[{k}] = {MFMA}(s_T[{buf}][{k}][4 * st + lq][l16], wreg{p.index}[st], acc[{k}], 0, 0, 0);")
+                s.close()
+                cur, nxt = nxt, cur
+            # D layout: rows 4*lq + i, column (channel) l16 of the wave's slice
+            s("#pragma unroll")
+            s.open("for (int i = 0; i < 4; ++i)")
+            s("const i64 row = row0 + 4 * lq + i;")
+            s.open("if (row < num_batch)")
+            s(f"T* zp = L3_out + row * {low.L3} + {bo.off} + (wave * 16 + l16) * {bo.d};")
+            for k in range(bo.d):
+                s(f"zp[{k}] = acc[{k}][i];")
+            s.close()
+            s.close()
+            s.close()
+            s.close()
+        return names
+
+    # ------------------------------------------------------------ backward
+    def emit_backward(self, s: Src) -> List[str]:
+        """One kernel per input irrep (dX of that irrep and the dY contributions of its paths) and
+        one per output irrep (dW of the paths feeding it), launched back to back. A tile is always
+        handled by the same block and thread, so the dY contributions of successive kernels are
+        added in a fixed order with plain read-modify-writes. Returns the kernel names."""
+        low = self.low
+        names = []
+        # ---------------- dX, dY ------------------------------------------------
+        first_dy = True
         for i1, b1 in enumerate(low.in1):
             paths = [p for p in low.paths if p.i1 == i1]
-            s(f"// ---- in1[{i1}]: {b1.mul} x l={b1.l}")
+            name = "backward" if not names else f"backward_x{i1}"
+            names.append(name)
+            s(f"// ======== in1[{i1}]: {b1.mul} x l={b1.l}")
+            self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_wx"])
             if not paths:
+                self._prologue(s)
+                s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
+                s(f"const i64 row0 = tile * {RT};")
                 s.open(f"for (int t = tid; t < {RT * b1.mul * b1.d}; t += {64 * WAVES})")
                 s(f"const int r = t / {b1.mul * b1.d}, c = t % {b1.mul * b1.d};")
                 s(f"if (row0 + r < num_batch) L1_grad[(row0 + r) * {low.L1} + {b1.off} + c] = T(0);")
                 s.close()
+                s.close()
+                s.close()
                 continue
-            s.open("")
-            s(f"T dx[4][{b1.d}];")
-            s(f"for (int i = 0; i < 4; ++i) for (int c = 0; c < {b1.d}; ++c) dx[i][c] = T(0);")
-            s("const int u = wave * 16 + l16;")
+            s(f"__shared__ T s_g[{RT}][{self.gstride}];")
+            s(f"__shared__ T s_y[{RT}][{low.L2}];")
+            s(f"__shared__ T s_dy[{WAVES}][{RT}][{low.L2}];")
+            self._prologue(s)
+            s("const int u = wave * 16 + l16;  // channel of this lane in the MFMA result layout")
+            self._load_wreg(s, paths, transposed=True)
+            s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
+            s(f"const i64 row0 = tile * {RT};")
+            s("__syncthreads();")
+            self._stage_g(s)
+            self._stage_y(s)
+            # X of the lane's 4 (row, channel) pairs: issued before the barrier and the MFMA loop
+            s(f"T x[4][{self.max_d1}], dx[4][{b1.d}], dy[4][{low.L2}];")
+            s("#pragma unroll")
+            s.open("for (int i = 0; i < 4; ++i)")
+            s("i64 row = row0 + 4 * lq + i; if (row >= num_batch) row = num_batch - 1;")
+            s(f"const T* xp = L1_in + row * {low.L1} + {b1.off} + u * {b1.d};")
+            for c in range(b1.d):
+                s(f"x[i][{c}] = xp[{c}]; dx[i][{c}] = T(0);")
+            s(f"for (int j = 0; j < {low.L2}; ++j) dy[i][j] = T(0);")
+            s.close()
+            s("__syncthreads();")
             for p in paths:
                 b2, bo = low.in2[p.i2], low.out[p.io]
                 s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
                 s.open("")
-                # G[k] = sum_w dZ[(r,k), w] * W[u, w]   (A = dZ tile, B = W^T)
+                # G[k] = sum_w dZ[(r,k), w] * W[u, w]   (A = dZ tile, B = W^T slice in registers)
                 s(f"v4f G[{bo.d}];")
                 for k in range(bo.d):
                     s(f"G[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
-                s("#pragma unroll 2")
-                s.open(f"for (int st = 0; st < {bo.mul // 4}; ++st)")
+                s("#pragma unroll")
+                s.open("for (int st = 0; st < 16; ++st)")
                 for k in range(bo.d):
-                    s(f"const T a{k} = s_g[l16][{bo.off} + (4 * st + lq) * {bo.d} + {k}];")
-                s(f"const T b = W[{p.woff} + (i64)u * {bo.mul} + 4 * st + lq];")
-                for k in range(bo.d):
-                    s(f"G[{k}] = __builtin_amdgcn_mfma_f32_16x16x4f32(a{k}, b, G[{k}], 0, 0, 0);")
+                    s(f"G[{k}] = {MFMA}(s_g[l16][{bo.off} + (4 * st + lq) * {bo.d} + {k}], wreg{p.index}[st], G[{k}], 0, 0, 0);")
                 s.close()
-                # vector-ALU part on the D layout: lane = rows 4*lq+i, channel u
                 s("#pragma unroll")
                 s.open("for (int i = 0; i < 4; ++i)")
-                s("i64 row = row0 + 4 * lq + i; if (row >= num_batch) row = num_batch - 1;")
-                s(f"T Gk[{bo.d}], t[{bo.d}];")
+                s(f"T Gk[{bo.d}];")
                 for k in range(bo.d):
                     s(f"Gk[{k}] = G[{k}][i];")
-                s(f"cg_bwd{p.index}(L1_in + row * {low.L1} + {b1.off} + u * {b1.d}, s_y[4 * lq + i], Gk, dx[i], dy[i], t);")
+                s(f"cg_bwd{p.index}(x[i], s_y[4 * lq + i], Gk, dx[i], dy[i]);")
                 s.close()
                 s.close()
+            s("#pragma unroll")
             s.open("for (int i = 0; i < 4; ++i)")
             s("const i64 row = row0 + 4 * lq + i;")
             s.open("if (row < num_batch)")
@@ -292,67 +366,81 @@ class MfmaEmitter:
                 s(f"dp[{c}] = dx[i][{c}];")
             s.close()
             s.close()
+            # dY: sum over the 16 channels of the lane group, then over the 4 waves through LDS
+            s.open("for (int i = 0; i < 4; ++i)")
+            s.open(f"for (int j = 0; j < {low.L2}; ++j)")
+            s("T v = dy[i][j];")
+            for m in (1, 2, 4, 8):
+                s(f"v += __shfl_xor(v, {m});")
+            s("if (l16 == 0) s_dy[wave][4 * lq + i][j] = v;")
             s.close()
-        # dY: sum over the 16 channels of the lane group, then over the 4 waves through LDS
-        s.open("for (int i = 0; i < 4; ++i)")
-        s.open(f"for (int j = 0; j < {L2p}; ++j)")
-        s("T v = dy[i][j];")
-        for m in (1, 2, 4, 8):
-            s(f"v += __shfl_xor(v, {m});")
-        s("if (l16 == 0) s_dy[wave][4 * lq + i][j] = v;")
-        s.close()
-        s.close()
-        s("__syncthreads();")
-        s.open(f"for (int t = tid; t < {RT * low.L2}; t += {64 * WAVES})")
-        s(f"const int r = t / {low.L2}, c = t % {low.L2};")
-        s("const T tot = ((s_dy[0][r][c] + s_dy[1][r][c]) + s_dy[2][r][c]) + s_dy[3][r][c];")
-        s(f"if (row0 + r < num_batch) L2_grad[(row0 + r) * {low.L2} + c] = tot;")
-        s.close()
-        s.close()
-
-        # ---------------- sweep 2: dW ------------------------------------------
-        s(f"v4f dw[{self.n_dw}];")
-        for n in range(self.n_dw):
-            s(f"dw[{n}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
-        s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
-        s(f"const i64 row0 = tile * {RT};")
-        self._stage_tile(s, with_y=False)
-        for p in low.paths:
-            b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
-            base, nw = dwl[p.index]
-            s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
-            s("__syncthreads();  // readers of the previous s_T are done")
-            s.open(f"for (int rr = 0; rr < {RT // WAVES}; ++rr)")
-            s(f"const int r = wave * {RT // WAVES} + rr;")
-            s("i64 row = row0 + r; if (row >= num_batch) row = num_batch - 1;")
-            s(f"T t[{bo.d}];")
-            s(f"cg_fwd{p.index}(L1_in + row * {low.L1} + {b1.off} + lane * {b1.d}, L2_in + row * {low.L2}, t);")
-            for k in range(bo.d):
-                s(f"s_T[{k}][lane][r] = t[{k}];")
             s.close()
             s("__syncthreads();")
-            # dW[u, w] += sum_(k,r) T[(k,r), u] * dZ[(k,r), w]   (A = T^T, B = dZ tile; zero dZ rows past the batch)
-            s("#pragma unroll 2")
-            s.open(f"for (int st = 0; st < {4 * bo.d}; ++st)")
-            s("const int kq = 4 * st + lq;")
-            s("const int kk = kq >> 4, rr = kq & 15;")
-            s("const T a = s_T[kk][wave * 16 + l16][rr];")
-            for n in range(nw):
-                s(f"const T b{n} = s_g[rr][{bo.off} + ({16 * n} + l16) * {bo.d} + kk];")
-            for n in range(nw):
-                s(f"dw[{base + n}] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b{n}, dw[{base + n}], 0, 0, 0);")
+            s.open(f"for (int t = tid; t < {RT * low.L2}; t += {64 * WAVES})")
+            s(f"const int r = t / {low.L2}, c = t % {low.L2};")
+            s("const T tot = ((s_dy[0][r][c] + s_dy[1][r][c]) + s_dy[2][r][c]) + s_dy[3][r][c];")
+            s(f"if (row0 + r < num_batch) L2_grad[(row0 + r) * {low.L2} + c] {'=' if first_dy else '+='} tot;")
             s.close()
-        s.close()
-        # partial weight gradient of this block (D layout: rows = channels u, columns = w)
-        s(f"T* prow = wpartial + (i64)blockIdx.x * {low.WN};")
-        for p in low.paths:
-            base, nw = dwl[p.index]
-            bo = low.out[p.io]
-            for n in range(nw):
-                s.open("for (int i = 0; i < 4; ++i)")
-                s(f"prow[{p.woff} + (i64)(wave * 16 + 4 * lq + i) * {bo.mul} + {16 * n} + l16] = dw[{base + n}][i];")
+            s.close()
+            s.close()
+            first_dy = False
+
+        # ---------------- dW ----------------------------------------------------
+        for io, bo in enumerate(low.out):
+            order = [p for p in low.paths if p.io == io]
+            if not order:
+                continue
+            name = f"backward_w{io}"
+            names.append(name)
+            s(f"// ======== dW of the paths into out[{io}]")
+            self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_ww"])
+            s(f"__shared__ T s_g[{RT}][{self.gstride}];")
+            s(f"__shared__ T s_T[2][{bo.d}][64][{TPAD}];")
+            s(f"__shared__ T s_y[{RT}][{low.L2}];")
+            self._prologue(s)
+            s("const int u = wave * 16 + l16;")
+            s(f"T* prow = wpartial + (i64)blockIdx.x * {low.WN};")
+            s(f"T xa[{RT // WAVES}][{self.max_d1}], xb[{RT // WAVES}][{self.max_d1}];")
+            # dw{p}[n]: D tile rows = channels u of the wave's slice, columns = w in 16 n .. 16 n + 15
+            for p in order:
+                s(f"v4f dw{p.index}[4];")
+                s(f"for (int n = 0; n < 4; ++n) dw{p.index}[n] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+            s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
+            s(f"const i64 row0 = tile * {RT};")
+            s("__syncthreads();")
+            # only this irrep's columns of the dZ tile are needed
+            self._stage_g(s, bo.off, bo.mul * bo.d)
+            self._stage_y(s)
+            self._load_x_rows(s, "xa", order[0])
+            s("__syncthreads();")
+            cur, nxt = "xa", "xb"
+            for n, p in enumerate(order):
+                b1, b2 = low.in1[p.i1], low.in2[p.i2]
+                buf = n % 2
+                s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
+                self._t_compute(s, p, cur, str(buf))
+                if n + 1 < len(order):
+                    self._load_x_rows(s, nxt, order[n + 1])
+                s("__syncthreads();")
+                # dW[u, w] += sum_(k,r) T[(k,r), u] * dZ[(k,r), w]   (A = T^T, B = dZ tile)
+                s("#pragma unroll")
+                s.open(f"for (int st = 0; st < {4 * bo.d}; ++st)")
+                s("const int kq = 4 * st + lq;")
+                s("const int kk = kq >> 4, rr = kq & 15;")
+                s(f"const T a = s_T[{buf}][kk][u][rr];")
+                for nn in range(4):
+                    s(f"dw{p.index}[{nn}] = {MFMA}(a, s_g[rr][{bo.off} + ({16 * nn} + l16) * {bo.d} + kk], dw{p.index}[{nn}], 0, 0, 0);")
                 s.close()
-        s.close()
+                cur, nxt = nxt, cur
+            s.close()
+            for p in order:
+                for nn in range(4):
+                    s("#pragma unroll")
+                    s.open("for (int i = 0; i < 4; ++i)")
+                    s(f"prow[{p.woff} + (wave * 16 + 4 * lq + i) * 64 + {16 * nn} + l16] = dw{p.index}[{nn}][i];")
+                    s.close()
+            s.close()
+        return names
 
 
 def tp_module(low: Lowered, compute_units: int = 256):
@@ -364,12 +452,12 @@ def tp_module(low: Lowered, compute_units: int = 256):
     s("typedef float v4f __attribute__((ext_vector_type(4)));")
     s(utility_kernels())
     em._emit_path_fns(s)
-    em.emit_forward(s)
-    em.emit_backward(s)
-    max_blocks_b = compute_units * 2
-    descs = [
-        (rt.ROLE_TP_FORWARD, "forward", 64 * WAVES, RT, compute_units * 8),
-        (rt.ROLE_TP_BACKWARD, "backward", 64 * WAVES, RT, max_blocks_b),
+    fwd_names = em.emit_forward(s)
+    bwd_names = em.emit_backward(s)
+    max_blocks = compute_units * em.tune["uvw_blocks"]
+    descs = [(rt.ROLE_TP_FORWARD, n, 64 * WAVES, RT, max_blocks) for n in fwd_names]
+    descs += [(rt.ROLE_TP_BACKWARD, n, 64 * WAVES, RT, max_blocks) for n in bwd_names]
+    descs += [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0),
     ]

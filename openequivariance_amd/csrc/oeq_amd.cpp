@@ -41,9 +41,11 @@ int fail(int code, const char* fmt, ...) {
 
 constexpr int kMaxDevices = 16;
 
+// A role is one kernel, or several launched back to back with the same arguments and the same
+// launch shape (descriptors naming the same role, in order); `names` lists them.
 struct RoleInfo {
     bool present = false;
-    std::string name;
+    std::vector<std::string> names;
     unsigned block = 0;
     unsigned units_per_block = 1;
     unsigned max_blocks = 0;
@@ -52,7 +54,7 @@ struct RoleInfo {
 
 struct DeviceSlot {
     hipModule_t module = nullptr;
-    hipFunction_t fn[OEQ_ROLE_COUNT] = {};
+    std::vector<hipFunction_t> fn[OEQ_ROLE_COUNT];
 };
 
 struct TimedLaunch {
@@ -75,7 +77,7 @@ struct oeq_kernels {
 
     // Resolve the function for `role` on the current device (loading the code
     // object there on first use).
-    int function(int role, hipFunction_t* out) {
+    int functions(int role, const std::vector<hipFunction_t>** out) {
         if (role < 0 || role >= OEQ_ROLE_COUNT || !roles[role].present)
             return fail(OEQ_ERR_INVALID, "kernel role %d is not part of this kernel set", role);
         int dev = 0;
@@ -87,16 +89,21 @@ struct oeq_kernels {
             HIP_TRY(hipModuleLoadData(&s.module, code.data()));
             for (int r = 0; r < OEQ_ROLE_COUNT; ++r) {
                 if (!roles[r].present) continue;
-                hipError_t e = hipModuleGetFunction(&s.fn[r], s.module, roles[r].name.c_str());
-                if (e != hipSuccess) {
-                    (void)hipModuleUnload(s.module);
-                    s.module = nullptr;
-                    return fail(OEQ_ERR_HIP, "kernel '%s' not found in code object: %s", roles[r].name.c_str(),
-                                hipGetErrorString(e));
+                s.fn[r].clear();
+                for (const std::string& name : roles[r].names) {
+                    hipFunction_t f = nullptr;
+                    hipError_t e = hipModuleGetFunction(&f, s.module, name.c_str());
+                    if (e != hipSuccess) {
+                        (void)hipModuleUnload(s.module);
+                        s.module = nullptr;
+                        return fail(OEQ_ERR_HIP, "kernel '%s' not found in code object: %s", name.c_str(),
+                                    hipGetErrorString(e));
+                    }
+                    s.fn[r].push_back(f);
                 }
             }
         }
-        *out = s.fn[role];
+        *out = &s.fn[role];
         return OEQ_OK;
     }
 
@@ -111,21 +118,24 @@ struct oeq_kernels {
     }
 
     int launch(int role, int64_t units, void** args, void* stream) {
-        hipFunction_t fn = nullptr;
-        int rc = function(role, &fn);
+        const std::vector<hipFunction_t>* fns = nullptr;
+        int rc = functions(role, &fns);
         if (rc) return rc;
         unsigned grid = grid_for(role, units);
         if (!timing) {
-            HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, roles[role].block, 1, 1, 0, (hipStream_t)stream, args,
-                                          nullptr));
+            for (hipFunction_t fn : *fns)
+                HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, roles[role].block, 1, 1, 0, (hipStream_t)stream, args,
+                                              nullptr));
             return OEQ_OK;
         }
-        // profiling mode: bracket this one kernel with events on its own stream
+        // profiling mode: bracket the role's kernels with events on their own stream
         TimedLaunch t{role, nullptr, nullptr};
         HIP_TRY(hipEventCreate(&t.start));
         HIP_TRY(hipEventCreate(&t.stop));
         HIP_TRY(hipEventRecord(t.start, (hipStream_t)stream));
-        HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, roles[role].block, 1, 1, 0, (hipStream_t)stream, args, nullptr));
+        for (hipFunction_t fn : *fns)
+            HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, roles[role].block, 1, 1, 0, (hipStream_t)stream, args,
+                                          nullptr));
         HIP_TRY(hipEventRecord(t.stop, (hipStream_t)stream));
         std::lock_guard<std::mutex> lock(mu);
         timed.push_back(t);
@@ -239,7 +249,7 @@ int oeq_kernels_create(const void* code, size_t code_size, const oeq_problem_dim
         }
         RoleInfo& r = k->roles[d.role];
         r.present = true;
-        r.name = d.kernel_name;
+        r.names.emplace_back(d.kernel_name);
         r.block = d.block_threads;
         r.units_per_block = d.units_per_block;
         r.max_blocks = d.max_blocks;
