@@ -35,6 +35,9 @@ def parse():
     ap.add_argument("--no-atomic", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the side measurements (spatially ordered nodes, batch tensor-product configs)")
+    ap.add_argument("--only-tp", default=None, metavar="N",
+                    help="run only the batched tensor-product side measurement for config N (1, 2, 3, 3d, 4) "
+                         "and print its row; used for per-kernel profiles")
     return ap.parse_args()
 
 
@@ -97,7 +100,7 @@ def cpu_baseline(problem, graph, Ysh, n_receivers, seed=0):
     }
 
 
-def tp_config_table(dev):
+def tp_config_table(dev, only=None):
     """Side measurements: the batched tensor product at configs 1-4 (forward and backward timed
     separately, median of 10). Bytes = every operand once per row (shared weights once per call);
     FLOPs by the reference's convention, and dense 2*u*w*(2l+1) per path for the MFMA config."""
@@ -126,6 +129,8 @@ def tp_config_table(dev):
     cases = [("cfg1 single uvu f32", P.config1_single_uvu(), 100000), ("cfg2 nequip uvu f32", P.config2_nequip_uvu(), 200000),
              ("cfg3 mace uvu f32", P.config3_mace_uvu(), 500000), ("cfg3 mace uvu f64", P.config3_mace_uvu(np.float64), 500000),
              ("cfg4 uvw shared f32 (MFMA)", P.config4_uvw_shared(), 262144)]
+    if only is not None:
+        cases = [cases[["1", "2", "3", "3d", "4"].index(only)]]
     table = []
     for name, prob, B in cases:
         low = lower(prob)
@@ -167,6 +172,11 @@ def main():
 
     import numpy as np
     import torch
+
+    if args.only_tp is not None:
+        assert torch.cuda.is_available(), "bench.py needs a GPU"
+        print(json.dumps(tp_config_table("cuda:0", args.only_tp)[0]))
+        return
 
     import openequivariance_amd as oeq
     from openequivariance_amd import runtime as rt
@@ -270,7 +280,6 @@ def main():
         order_n = spatial_order(coords)
         rows_s, cols_s = relabel_nodes(order_n, rows, cols)
         gs = CoordGraph(coords[order_n], rows_s, cols_s, "periodic-radius-zorder")
-        # edge e of `graph` is edge graph.order[e] of the generated list; reuse its Y/W rows by matching edge ids
         Ys = torch.tensor(spherical_harmonics(3, vec).astype(np.float32)[gs.order], device=dev)
         trs, tcs, tps = (torch.tensor(a, device=dev) for a in (gs.rows, gs.cols, gs.transpose_perm))
 
