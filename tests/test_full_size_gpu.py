@@ -1,0 +1,129 @@
+"""Benchmark-size runs, where the float64 oracle is too slow to evaluate everything: agreement of a
+sample with the oracle plus size-independent properties (exact scaling laws, edge-order invariance,
+atomic vs deterministic agreement, bitwise reproducibility)."""
+
+import numpy as np
+import pytest
+import torch
+
+import openequivariance_amd as oeq
+from openequivariance_amd.core import problems as P
+from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
+from openequivariance_amd.core.sh import spherical_harmonics
+from oracle import e3nn_ref as R
+from gpu_util import err
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(a, b):
+    return float((a - b).abs().max() / b.abs().max())
+
+
+def test_cfg2_full_batch():
+    problem = P.config2_nequip_uvu()
+    B = 200000
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(B, 288, device="cuda", generator=gen, requires_grad=True)
+    v = torch.randn(B, 3, device="cuda", generator=gen)
+    y = torch.tensor(spherical_harmonics(3, v.cpu().numpy()).astype(np.float32), device="cuda").requires_grad_(True)
+    w = torch.randn(B, 416, device="cuda", generator=gen, requires_grad=True)
+    g = torch.randn(B, 1376, device="cuda", generator=gen)
+    tp = oeq.TensorProduct(problem)
+    z = tp(x, y, w)
+    z.backward(g)
+    idx = torch.tensor([0, 1, 2, 31, 32, 33, 65535, 65536, B - 3, B - 2, B - 1], device="cuda")
+    ref = R.Problem.from_spec(problem)
+    xs, ys, ws, gs = (t[idx].detach().cpu().numpy() for t in (x, y, w, g))
+    assert err(z[idx], R.tp_forward(ref, xs, ys, ws)) <= 1e-5
+    dx, dy, dw = R.tp_backward(ref, xs, ys, ws, gs)
+    assert err(x.grad[idx], dx) <= 1e-5 and err(y.grad[idx], dy) <= 1e-5 and err(w.grad[idx], dw) <= 1e-5
+    assert torch.equal(tp(4.0 * x, y, 0.5 * w), 2.0 * z)  # powers of two scale exactly
+    assert torch.isfinite(z).all() and torch.isfinite(x.grad).all()
+
+
+def test_cfg4_full_batch_mfma():
+    problem = P.config4_uvw_shared()
+    B = 262144
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn(B, 576, device="cuda", generator=gen, requires_grad=True)
+    v = torch.randn(B, 3, device="cuda", generator=gen)
+    y = torch.tensor(spherical_harmonics(2, v.cpu().numpy()).astype(np.float32), device="cuda").requires_grad_(True)
+    w = (torch.randn(45056, device="cuda", generator=gen) / np.sqrt(64 * 11)).requires_grad_(True)
+    g = torch.randn(B, 576, device="cuda", generator=gen)
+    tp = oeq.TensorProduct(problem)
+    z = tp(x, y, w)
+    z.backward(g)
+    idx = torch.tensor([0, 1, 15, 16, 17, 4095, 4096, B - 17, B - 16, B - 1], device="cuda")
+    ref = R.Problem.from_spec(problem)
+    xs, ys, gs = (t[idx].detach().cpu().numpy() for t in (x, y, g))
+    wn = w.detach().cpu().numpy()
+    assert err(z[idx], R.tp_forward(ref, xs, ys, wn)) <= 1e-5
+    dx, dy, _ = R.tp_backward(ref, xs, ys, wn, gs)
+    assert err(x.grad[idx], dx) <= 1e-5 and err(y.grad[idx], dy) <= 1e-5
+    # weight gradient: linear in the output gradient; a sum over disjoint row sets adds up
+    half = B // 2
+    _, _, dw1 = torch.ops.oeq_amd.tp_backward(x[:half].detach(), y[:half].detach(), w.detach(), g[:half], tp.kid)
+    _, _, dw2 = torch.ops.oeq_amd.tp_backward(x[half:].detach(), y[half:].detach(), w.detach(), g[half:], tp.kid)
+    assert _rel(dw1 + dw2, w.grad) <= 1e-5
+    # and it matches the oracle on a slice small enough to evaluate (first 2048 rows)
+    n = 2048
+    _, _, dws = torch.ops.oeq_amd.tp_backward(x[:n].detach(), y[:n].detach(), w.detach(), g[:n], tp.kid)
+    _, _, dw_ref = R.tp_backward(ref, x[:n].detach().cpu().numpy(), y[:n].detach().cpu().numpy(), wn,
+                                 g[:n].cpu().numpy())
+    assert err(dws, dw_ref) <= 1e-5
+    # deterministic reduction: bitwise equal on a second run
+    _, _, dw_again = torch.ops.oeq_amd.tp_backward(x.detach(), y.detach(), w.detach(), g, tp.kid)
+    assert torch.equal(dw_again, w.grad)
+
+
+def test_cfg5_full_graph():
+    problem = P.config5_mace_conv()
+    N = 50000
+    coords, rows, cols, vec = periodic_radius_graph(N, 32.0, 5.0, seed=0)
+    g = CoordGraph(coords, rows, cols)
+    E = g.nnz
+    assert 1.5e6 < E < 1.7e6
+    Y = torch.tensor(spherical_harmonics(3, vec).astype(np.float32)[g.order], device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    X = torch.randn(N, 2048, device="cuda", generator=gen)
+    W = torch.randn(E, 2944, device="cuda", generator=gen)
+    G = torch.randn(N, 12672, device="cuda", generator=gen)
+    tr, tc, tp = (torch.tensor(a, device="cuda") for a in (g.rows, g.cols, g.transpose_perm))
+    det = oeq.TensorProductConv(problem, deterministic=True)
+    ops = torch.ops.oeq_amd
+    z = ops.conv_forward(X, Y, W, tr, tc, tp, det.kid)
+    dx, dy, dw = ops.conv_backward(X, Y, W, G, tr, tc, tp, det.kid)
+    # bitwise reproducible
+    z2 = ops.conv_forward(X, Y, W, tr, tc, tp, det.kid)
+    dx2, dy2, dw2 = ops.conv_backward(X, Y, W, G, tr, tc, tp, det.kid)
+    assert torch.equal(z, z2) and torch.equal(dx, dx2) and torch.equal(dy, dy2) and torch.equal(dw, dw2)
+    # oracle on the sub-graph of a few receivers (forward) and on a few edges / senders (backward)
+    ref = R.Problem.from_spec(problem)
+    recv = [0, 1, 777, N - 1]
+    for r in recv:
+        e0, e1 = np.searchsorted(g.rows, [r, r + 1])
+        sl = slice(e0, e1)
+        msg = R.tp_forward(ref, X[tc[sl]].cpu().numpy(), Y[sl].cpu().numpy(), W[sl].cpu().numpy())
+        assert err(z[r], msg.sum(0)) <= 1e-5
+        gx, gy, gw = R.tp_backward(ref, X[tc[sl]].cpu().numpy(), Y[sl].cpu().numpy(), W[sl].cpu().numpy(),
+                                   G[r:r + 1].expand(e1 - e0, -1).cpu().numpy())
+        assert err(dy[sl], gy) <= 1e-5 and err(dw[sl], gw) <= 1e-5
+    s = 4242  # one sender: sum of the dX terms of its out-edges
+    es = np.nonzero(g.cols == s)[0]
+    te = torch.tensor(es, device="cuda")
+    gx, _, _ = R.tp_backward(ref, X[tc[te]].cpu().numpy(), Y[te].cpu().numpy(), W[te].cpu().numpy(),
+                             G[tr[te]].cpu().numpy())
+    assert err(dx[s], gx.sum(0)) <= 1e-5
+    # atomic mode on shuffled edges agrees with the deterministic result
+    perm = torch.randperm(E, device="cuda", generator=gen)
+    at = oeq.TensorProductConv(problem, deterministic=False)
+    dummy = torch.zeros(1, dtype=torch.int64, device="cuda")
+    Yp, Wp, rp, cp = Y[perm].contiguous(), W[perm].contiguous(), tr[perm].contiguous(), tc[perm].contiguous()
+    za = ops.conv_forward(X, Yp, Wp, rp, cp, dummy, at.kid)
+    assert _rel(za, z) <= 1e-5
+    dxa, dya, dwa = ops.conv_backward(X, Yp, Wp, G, rp, cp, dummy, at.kid)
+    assert _rel(dxa, dx) <= 1e-5 and _rel(dya, dy[perm]) <= 1e-5 and _rel(dwa, dw[perm]) <= 1e-5
+    # exact scaling laws
+    assert torch.equal(ops.conv_forward(2.0 * X, Y, W, tr, tc, tp, det.kid), 2.0 * z)
+    assert torch.isfinite(z).all() and torch.isfinite(dx).all()
