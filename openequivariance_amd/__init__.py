@@ -21,8 +21,11 @@ if os.environ.get("OEQ_NOTORCH") != "1":
     from ._torch.tensor_product_conv import TensorProductConv
     from ._torch.utils import torch_to_oeq_dtype
 
+    from .core.problems import ChannelwiseTPP, FullyConnectedTPProblem, SingleInstruction
+
     torch.serialization.add_safe_globals(
-        [TensorProduct, TensorProductConv, TPProblem, Irrep, Irreps, _MulIr, Instruction, np.float32, np.float64]
+        [TensorProduct, TensorProductConv, TPProblem, Irrep, Irreps, _MulIr, Instruction, np.float32, np.float64,
+         ChannelwiseTPP, FullyConnectedTPProblem, SingleInstruction]
     )
 
 

@@ -1,0 +1,92 @@
+"""The ops behave as well-formed torch custom ops: opcheck (schema, fake kernels, autograd
+registration), torch.compile, autocast, save/load (cf. the reference's tests/export_test.py:89-225)."""
+
+import io
+
+import numpy as np
+import pytest
+import torch
+
+import openequivariance_amd as oeq
+from openequivariance_amd.core import problems as P
+from oracle import e3nn_ref as R
+from gpu_util import err, to_gpu, tp_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tp_and_inputs():
+    problem = P.config2_nequip_uvu()
+    tp = oeq.TensorProduct(problem)
+    x, y, w, g = tp_inputs(problem, 48, seed=11)
+    z_ref = R.tp_forward(R.Problem.from_spec(problem), x, y, w)
+    return problem, tp, (x, y, w, g), z_ref
+
+
+def test_opcheck_tp(tp_and_inputs):
+    problem, tp, (x, y, w, g), _ = tp_and_inputs
+    tx, ty, tw = to_gpu(x, y, w, requires_grad=True)
+    (tg,) = to_gpu(g)
+    torch.library.opcheck(torch.ops.oeq_amd.tp_forward.default, (tx, ty, tw, tp.kid),
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+    torch.library.opcheck(torch.ops.oeq_amd.tp_backward.default, (tx, ty, tw, tg, tp.kid),
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+
+
+def test_opcheck_conv():
+    problem = P.config1_single_uvu()
+    conv = oeq.TensorProductConv(problem, deterministic=True)
+    rows = torch.tensor([0, 1, 1, 2], device="cuda")
+    cols = torch.tensor([1, 0, 2, 1], device="cuda")
+    perm = torch.argsort(cols, stable=True)
+    X = torch.rand(3, 5, device="cuda", requires_grad=True)
+    Y = torch.rand(4, 7, device="cuda", requires_grad=True)
+    W = torch.rand(4, 1, device="cuda", requires_grad=True)
+    torch.library.opcheck(torch.ops.oeq_amd.conv_forward.default, (X, Y, W, rows, cols, perm, conv.kid),
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+
+
+def test_torch_compile(tp_and_inputs):
+    problem, tp, (x, y, w, g), z_ref = tp_and_inputs
+    tx, ty, tw = to_gpu(x, y, w, requires_grad=True)
+    compiled = torch.compile(lambda a, b, c: tp(a, b, c) * 2.0, fullgraph=True)
+    z = compiled(tx, ty, tw)
+    assert err(z, 2.0 * z_ref) <= 1e-5
+    z.sum().backward()
+    dx_ref, _, _ = R.tp_backward(R.Problem.from_spec(problem), x, y, w, 2.0 * np.ones_like(z_ref))
+    assert err(tx.grad, dx_ref) <= 1e-5
+
+
+def test_autocast_runs_in_module_dtype(tp_and_inputs):
+    problem, tp, (x, y, w, g), z_ref = tp_and_inputs
+    tx, ty, tw = to_gpu(x, y, w)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        z = tp(tx, ty, tw)
+    assert z.dtype == torch.float32 and err(z, z_ref) <= 1e-5
+
+
+def test_save_load_module(tp_and_inputs):
+    problem, tp, (x, y, w, g), z_ref = tp_and_inputs
+    buf = io.BytesIO()
+    torch.save(tp, buf)
+    buf.seek(0)
+    tp2 = torch.load(buf, weights_only=True)
+    assert err(tp2(*to_gpu(x, y, w)), z_ref) <= 1e-5
+
+
+def test_module_inside_a_model_moves_with_to():
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.tp = oeq.TensorProduct(P.config1_single_uvu())
+            self.lin = torch.nn.Linear(5, 5)
+
+        def forward(self, x, y, w):
+            return self.lin(self.tp(x, y, w))
+
+    net = Net().to("cuda").to(torch.float64)
+    x, y, w = (torch.rand(10, n, device="cuda", dtype=torch.float64) for n in (5, 7, 1))
+    out = net(x, y, w)
+    assert out.dtype == torch.float64 and out.shape == (10, 5)
+    assert net.tp.config.irrep_dtype == np.float64
