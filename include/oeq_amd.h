@@ -74,7 +74,8 @@ typedef enum {
     OEQ_ROLE_SEGMENT_PTR = 5,       /* builds CSR pointers from a sorted index list */
     OEQ_ROLE_FILL_ZERO = 6,         /* clears a buffer (used instead of memset: capture-safe) */
     OEQ_ROLE_TP_BACKWARD_WREDUCE = 7,/* shared weights: second pass of the weight-gradient reduction */
-    OEQ_ROLE_COUNT = 8
+    OEQ_ROLE_SEGMENT_SUM = 8,       /* ordered sum of rows over the segments of a sorted key list */
+    OEQ_ROLE_COUNT = 9
 } oeq_role;
 
 /* Several descriptors may name the same role: those kernels are launched back to back, in
@@ -155,6 +156,18 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz,
                       const int64_t* transpose_perm,
                       void* workspace, size_t workspace_bytes, void* stream);
 size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
+
+/* ---- ordered segment sum -------------------------------------------------- */
+/* dst[s, :] = sum, in list order, of src[item, :] over the items whose key is s, for s < n_segments.
+ * The list is 0..n_items-1, or perm[0..n_items-1] when perm != NULL, and keys must be non-decreasing
+ * along it. Rows have row_len elements of the kernel set's element type. Deterministic (no atomics).
+ * Replaces the reference's scatter_add_wrapper (core/ConvolutionBase.py:292-301) where a fixed
+ * summation order is wanted; used by the unfused 'uvw' convolution. The workspace must hold
+ * oeq_segment_sum_workspace_bytes() bytes. */
+int oeq_segment_sum(oeq_kernels* k, int64_t n_segments, int64_t n_items, int64_t row_len,
+                    const void* src, void* dst, const int64_t* keys, const int64_t* perm,
+                    void* workspace, size_t workspace_bytes, void* stream);
+size_t oeq_segment_sum_workspace_bytes(const oeq_kernels* k, int64_t n_segments);
 
 /* ---- per-kernel timing --------------------------------------------------- */
 /* Replaces GPUTimer (extension/backend/backend_hip.hpp:67-101). While enabled,

@@ -35,8 +35,9 @@ _next_id = [1]
 class KernelEntry:
     """Lazily compiled kernel set + the shape facts the ops validate against."""
 
-    def __init__(self, build_fn, L1, L2, L3, WN, shared, torch_dtype, deterministic=False):
+    def __init__(self, build_fn, L1, L2, L3, WN, shared, torch_dtype, deterministic=False, unfused=False):
         self.build_fn = build_fn  # () -> (source, dims, descs)
+        self.unfused = unfused  # convolution = gather + batch kernels + scatter (no fused kernel for this problem)
         self.L1, self.L2, self.L3, self.WN = L1, L2, L3, WN
         self.shared = shared
         self.dtype = torch_dtype
@@ -210,6 +211,41 @@ def _conv_checks(e: KernelEntry, L1_in, L2_in, W, rows, cols, perm, L3_grad=None
     return nodes, nnz
 
 
+def _segment_sum(ks, src: torch.Tensor, n_segments: int, keys: torch.Tensor, perm: Optional[torch.Tensor]):
+    """Ordered sum of the rows of ``src`` over runs of equal ``keys`` (read through ``perm`` if given)."""
+    dst = src.new_empty((n_segments, src.shape[1]))
+    nb = ks.segment_sum_workspace_bytes(n_segments)
+    ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=src.device)
+    ks.segment_sum(n_segments, src.shape[0], src.shape[1], src.data_ptr(), dst.data_ptr(), keys.data_ptr(),
+                   perm.data_ptr() if perm is not None else 0, ws.data_ptr(), nb, _stream())
+    return dst
+
+
+def _scatter_rows(e: KernelEntry, ks, src, n_segments, keys, perm):
+    """Sum edge rows into node rows: fixed order when deterministic, torch's atomic index_add_ otherwise
+    (the reference's unfused path, core/ConvolutionBase.py:292-301, is the latter)."""
+    if e.deterministic:
+        return _segment_sum(ks, src, n_segments, keys, perm)
+    return src.new_zeros((n_segments, src.shape[1])).index_add_(0, keys, src)
+
+
+def _unfused_forward(e, ks, x, y, w, r, c, nodes, nnz):
+    xe = x.index_select(0, c)
+    msg = x.new_empty((nnz, e.L3))
+    ks.tp_forward(nnz, xe.data_ptr(), y.data_ptr(), w.data_ptr(), msg.data_ptr(), _stream())
+    return _scatter_rows(e, ks, msg, nodes, r, None)
+
+
+def _unfused_backward(e, ks, x, y, w, g, r, c, p, nodes, nnz):
+    xe, ge = x.index_select(0, c), g.index_select(0, r)
+    dxe, dy, dw = torch.empty_like(xe), torch.empty_like(y), torch.empty_like(w)
+    nb = ks.tp_backward_workspace_bytes(nnz)
+    ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
+    ks.tp_backward(nnz, xe.data_ptr(), dxe.data_ptr(), y.data_ptr(), dy.data_ptr(), w.data_ptr(), dw.data_ptr(),
+                   ge.data_ptr(), ws.data_ptr() if nb else 0, nb, _stream())
+    return _scatter_rows(e, ks, dxe, nodes, c, p if e.deterministic else None), dy, dw
+
+
 @torch.library.custom_op("oeq_amd::conv_forward", mutates_args=(), device_types="cuda")
 def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows: torch.Tensor,
                  cols: torch.Tensor, transpose_perm: torch.Tensor, kid: int) -> torch.Tensor:
@@ -217,6 +253,9 @@ def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows
     nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm)
     x, y, w = L1_in.contiguous(), L2_in.contiguous(), W.contiguous()
     r, c = rows.contiguous(), cols.contiguous()
+    if e.unfused:
+        with torch.cuda.device(x.device):
+            return _unfused_forward(e, e.kernels(), x, y, w, r, c, nodes, nnz)
     out = x.new_empty((nodes, e.L3))
     with torch.cuda.device(x.device):
         ks = e.kernels()
@@ -241,6 +280,9 @@ def conv_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_
     nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm, L3_grad)
     x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
     r, c, p = rows.contiguous(), cols.contiguous(), transpose_perm.contiguous()
+    if e.unfused:
+        with torch.cuda.device(x.device):
+            return _unfused_backward(e, e.kernels(), x, y, w, g, r, c, p, nodes, nnz)
     dx, dy, dw = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w)
     with torch.cuda.device(x.device):
         ks = e.kernels()

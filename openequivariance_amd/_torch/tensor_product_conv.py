@@ -29,7 +29,16 @@ def build_conv_module(problem: TPProblem, deterministic: bool):
     if low.mode == "uvu":
         from ..codegen import uvu
         return uvu.conv_module(low, deterministic, compute_units())
-    raise NotImplementedError("TensorProductConv supports 'uvu' problems only in this package")
+    # 'uvw': no fused kernel; the batch kernels run on gathered rows and an ordered segment sum (or torch's
+    # index_add_ in atomic mode) scatters the result, like the reference's unfused convolution
+    # (core/ConvolutionBase.py:292-301, _torch/TensorProductConv.py:595-640).
+    from .. import runtime as rt
+    from ..codegen import uvw
+    cu = compute_units()
+    src, dims, descs = uvw.tp_module(low, cu)
+    descs = list(descs) + [(rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, cu * 16),
+                           (rt.ROLE_SEGMENT_SUM, "oeq_segment_sum", 256, 1, cu * 32)]
+    return src, dims, descs
 
 
 class TensorProductConv(torch.nn.Module):
@@ -69,6 +78,7 @@ class TensorProductConv(torch.nn.Module):
         entry = ops.KernelEntry(
             lambda p=problem, d=deterministic: build_conv_module(p, d), low.L1, low.L2, low.L3, low.WN,
             low.shared_weights, oeq_to_torch_dtype(problem.irrep_dtype), deterministic=deterministic,
+            unfused=low.mode != "uvu",
         )
         self.kid = ops.register_entry(entry)
         self._dummy_perm = None

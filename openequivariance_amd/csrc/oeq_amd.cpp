@@ -266,6 +266,29 @@ void oeq_kernels_destroy(oeq_kernels* k) {
     delete k;
 }
 
+size_t oeq_segment_sum_workspace_bytes(const oeq_kernels* k, int64_t n_segments) {
+    (void)k;
+    return align_up((size_t)(n_segments + 1) * sizeof(int64_t), 256);
+}
+
+int oeq_segment_sum(oeq_kernels* k, int64_t n_segments, int64_t n_items, int64_t row_len, const void* src, void* dst,
+                    const int64_t* keys, const int64_t* perm, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_segment_sum: NULL kernel set");
+    if (n_segments < 0 || n_items < 0 || row_len <= 0) return fail(OEQ_ERR_INVALID, "oeq_segment_sum: bad size");
+    if (n_segments == 0) return OEQ_OK;
+    if (!dst) return fail(OEQ_ERR_INVALID, "oeq_segment_sum: NULL dst");
+    if (n_items == 0) return k->fill_zero(dst, (size_t)n_segments * row_len * k->dims.elem_size, stream);
+    if (!src || !keys) return fail(OEQ_ERR_INVALID, "oeq_segment_sum: NULL buffer");
+    size_t need = oeq_segment_sum_workspace_bytes(k, n_segments);
+    if (!workspace || workspace_bytes < need)
+        return fail(OEQ_ERR_INVALID, "oeq_segment_sum: workspace too small (%zu < %zu bytes)", workspace_bytes, need);
+    int64_t* ptr = (int64_t*)workspace;
+    int rc = k->segment_ptr(n_items, n_segments, keys, perm, ptr, stream);
+    if (rc) return rc;
+    void* args[] = {&n_segments, &n_items, &row_len, &src, &dst, &perm, &ptr};
+    return k->launch(OEQ_ROLE_SEGMENT_SUM, n_segments, args, stream);
+}
+
 int oeq_kernel_timing_enable(oeq_kernels* k, int enable) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_kernel_timing_enable: NULL kernel set");
     std::lock_guard<std::mutex> lock(k->mu);

@@ -42,6 +42,7 @@ ROLE_CONV_FIXUP_BACKWARD = 4
 ROLE_SEGMENT_PTR = 5
 ROLE_FILL_ZERO = 6
 ROLE_TP_BACKWARD_WREDUCE = 7
+ROLE_SEGMENT_SUM = 8
 
 
 class OeqError(RuntimeError):
@@ -122,6 +123,8 @@ EXPORTS = {
     "oeq_conv_forward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_backward": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_conv_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_segment_sum": (ctypes.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _SZ, _P]),
+    "oeq_segment_sum_workspace_bytes": (_SZ, [_P, _I64]),
     "oeq_kernel_timing_enable": (ctypes.c_int, [_P, ctypes.c_int]),
     "oeq_kernel_timing_collect": (ctypes.c_int, [_P, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
                                                  ctypes.POINTER(_I64)]),
@@ -256,6 +259,13 @@ class KernelSet:
     def tp_backward(self, n, x, dx, y, dy, w, dw, g, ws, ws_bytes, stream):
         _check(self._lib.oeq_tp_backward(self.handle, n, x, dx, y, dy, w, dw, g, ws, ws_bytes, stream),
                "oeq_tp_backward")
+
+    def segment_sum_workspace_bytes(self, n_segments) -> int:
+        return self._lib.oeq_segment_sum_workspace_bytes(self.handle, n_segments)
+
+    def segment_sum(self, n_segments, n_items, row_len, src, dst, keys, perm, ws, ws_bytes, stream):
+        _check(self._lib.oeq_segment_sum(self.handle, n_segments, n_items, row_len, src, dst, keys, perm, ws,
+                                         ws_bytes, stream), "oeq_segment_sum")
 
     def conv_forward_workspace_bytes(self, nodes, nnz) -> int:
         return self._lib.oeq_conv_forward_workspace_bytes(self.handle, nodes, nnz)

@@ -38,6 +38,11 @@ def _odd(shared):
                           (0, 0, 2, "uvu", True)], shared_weights=shared, internal_weights=False, label="odd-uvu")
 
 
+def _fc(shared):
+    return P.FullyConnectedTPProblem("4x0e+3x1o", "1x0e+2x1o", "5x0e+2x1o+1x2e", shared_weights=shared,
+                                     internal_weights=False, label="fc-uvw")
+
+
 CASES = [
     ("cfg1", P.config1_single_uvu, 40, 6),
     ("cfg2", P.config2_nequip_uvu, 60, 8),
@@ -46,6 +51,10 @@ CASES = [
     ("mace-large", lambda: P.mace_problems()[0], 40, 6),
     ("odd", lambda: _odd(False), 40, 6),
     ("odd-shared", lambda: _odd(True), 40, 6),
+    # 'uvw' problems: no fused kernel, batch kernels on gathered rows + ordered segment sum / index_add_
+    ("uvw", lambda: _fc(False), 40, 6),
+    ("uvw-shared", lambda: _fc(True), 40, 6),
+    ("uvw-cfg4-mfma", P.config4_uvw_shared, 30, 5),
 ]
 
 
