@@ -19,7 +19,7 @@ if os.environ.get("OEQ_NOTORCH") != "1":
 
     from ._torch.tensor_product import TensorProduct
     from ._torch.tensor_product_conv import TensorProductConv
-    from ._torch.utils import torch_to_oeq_dtype
+    from ._torch.utils import torch_to_oeq_dtype, transpose_irreps
 
     from .core.problems import ChannelwiseTPP, FullyConnectedTPProblem, SingleInstruction
 
@@ -36,4 +36,4 @@ def torch_ext_so_path():
 
 
 __all__ = ["TPProblem", "Irrep", "Irreps", "Instruction", "TensorProduct", "TensorProductConv",
-           "torch_to_oeq_dtype", "torch_ext_so_path"]
+           "torch_to_oeq_dtype", "transpose_irreps", "torch_ext_so_path"]

@@ -37,3 +37,25 @@ def compute_units() -> int:
             n = int(rt.device_props(torch.cuda.current_device()).compute_units)
         _cu_cache[0] = n
     return _cu_cache[0]
+
+
+def transpose_irreps(array: torch.Tensor, irreps, src_layout: str, dst_layout: str) -> torch.Tensor:
+    r"""Re-lay-out the trailing (feature) dimension of an irrep-packed tensor between
+    ``"mul_ir"`` (blocks stored ``[mul, 2l+1]``) and ``"ir_mul"`` (``[2l+1, mul]``); same
+    contract as the reference function
+    (openequivariance/openequivariance/_torch/utils.py:80-147): leading dimensions
+    are kept, the result is a new tensor (a clone when both layouts agree) and the
+    operation is differentiable (one ``index_select``).
+
+    :raises TypeError: if ``array`` is not a tensor.
+    :raises ValueError: for layouts other than ``"mul_ir"`` / ``"ir_mul"``.
+    """
+    from ..core.layout import check_layouts, layout_permutation
+
+    check_layouts(src_layout, dst_layout)
+    if not isinstance(array, torch.Tensor):
+        raise TypeError(f"Expected torch.Tensor, got {type(array)}")
+    if src_layout == dst_layout:
+        return array.clone()
+    index = torch.from_numpy(layout_permutation(irreps, src_layout, dst_layout).copy()).to(array.device)
+    return array.index_select(-1, index)

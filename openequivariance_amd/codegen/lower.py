@@ -88,6 +88,8 @@ class Lowered:
     n_chunks: int = 1
     max_u: int = 1
     total_nnz: int = 0
+    # True: every irrep block of a row is stored [2l+1, mul] (component-major) instead of [mul, 2l+1]
+    ir_mul: bool = False
 
     def flops(self, direction: str) -> int:
         """Reference FLOP convention (benchmark/metrics.py:49-94,
@@ -120,8 +122,6 @@ def _pow2ceil(n: int) -> int:
 
 def lower(problem: TPProblem) -> Lowered:
     info = filter_and_analyze_problem(problem)
-    if problem.layout != "mul_ir":
-        raise NotImplementedError("layout='ir_mul' is not implemented in this package yet")
     dtype = np.dtype(problem.irrep_dtype)
     if dtype == np.float32:
         ctype, es = "float", 4
@@ -148,6 +148,7 @@ def lower(problem: TPProblem) -> Lowered:
         L1=problem.irreps_in1.dim, L2=problem.irreps_in2.dim, L3=problem.irreps_out.dim,
         WN=problem.weight_numel, label=problem.label,
     )
+    low.ir_mul = problem.layout == "ir_mul"
     used_mul = [in1[p.i1].mul for p in paths]
     low.max_u = max(used_mul)
     low.lanes_per_row = 64 if low.max_u > 32 else _pow2ceil(low.max_u)

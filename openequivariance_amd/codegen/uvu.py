@@ -48,6 +48,7 @@ class UvuEmitter:
     def __init__(self, low: Lowered, *, acc_budget_words: int = 128, g_resident_words: int = 128):
         assert low.mode == "uvu"
         self.low = low
+        self.ir_mul = low.ir_mul
         self.T = low.ctype
         self.words = 1 if low.elem_size == 4 else 2
         self.LPR = low.lanes_per_row
@@ -113,6 +114,16 @@ class UvuEmitter:
         nqw = (nuw + 63) // 64
         return dict(U=U, xl=xl, nux=units, nqx=nqx, nuw=nuw, nqw=nqw, XF=nqx * 256, floats=(nqx + nqw) * 256)
 
+    def _stage_src(self, blk, first_unit: int) -> str:
+        """Row offset of the 16-byte unit ``t`` of the wave's slice of a block (units in LDS order)."""
+        if self.ir_mul:  # component i = 16 units of 4 channels each
+            return (f"{blk.off} + ((t - {first_unit}) >> 4) * {blk.mul} + chunk * 64 + ((t - {first_unit}) & 15) * 4")
+        return f"{blk.off} + chunk * {64 * blk.d} + (t - {first_unit}) * 4"
+
+    def _stage_x(self, blk, base: int, i: int) -> str:
+        """Index of (lane's channel, component i) in a staged block starting at ``base``."""
+        return f"{base + i * 64} + ul" if self.ir_mul else f"{base} + ul * {blk.d} + {i}"
+
     def _emit_stage_offsets(self, s: Src):
         """Per-lane source offsets (in elements) of the staging loads; loop invariant."""
         low, st = self.low, self.stage
@@ -125,7 +136,7 @@ class UvuEmitter:
             for b in self.used_in1:
                 blk = low.in1[b]
                 n = 16 * blk.d
-                terms.append((pu, pu + n, f"{blk.off} + chunk * {64 * blk.d} + (t - {pu}) * 4"))
+                terms.append((pu, pu + n, self._stage_src(blk, pu)))
                 pu += n
             code = terms[-1][2]
             for lo, hi, ex in reversed(terms[:-1]):
@@ -158,7 +169,7 @@ class UvuEmitter:
         for b in self.used_in1:
             blk = low.in1[b]
             for i in range(blk.d):
-                s(f"{buf}.x.b{b}[{i}] = s_stage[wave][{st['xl'][b]} + ul * {blk.d} + {i}];")
+                s(f"{buf}.x.b{b}[{i}] = s_stage[wave][{self._stage_x(blk, st['xl'][b], i)}];")
         for p in low.paths:
             s(f"{buf}.w[{self.wslot[p.index]}] = s_stage[wave][{st['XF'] + p.index * 64} + ul];")
         for j in range(low.L2):
@@ -190,7 +201,7 @@ class UvuEmitter:
             for b in self.used_in1:
                 blk = low.in1[b]
                 n = 16 * blk.d
-                terms.append((pu + n, f"{blk.off} + chunk * {64 * blk.d} + (t - {pu}) * 4"))
+                terms.append((pu + n, self._stage_src(blk, pu)))
                 pu += n
             code = terms[-1][1]
             for hi, ex in reversed(terms[:-1]):
@@ -229,7 +240,7 @@ class UvuEmitter:
         low, st = self.low, self.stage3
 
         def x(b: int, i: int) -> str:
-            return f"{sb}[{st['xl'][b]} + ul * {low.in1[b].d} + {i}]"
+            return f"{sb}[{self._stage_x(low.in1[b], st['xl'][b], i)}]"
 
         def y(p: Path, v: str, j: int) -> str:
             return f"{sb}[{st['YOFF'] + low.in2[p.i2].off + j}]"
@@ -238,6 +249,19 @@ class UvuEmitter:
             return f"{sb}[{st['XF'] + p.index * 64} + ul]"
 
         return x, y, w
+
+    def _lane_ptr(self, blk) -> Tuple[str, int]:
+        """(offset of channel ``u``'s first component within a row, stride between components) of a block:
+        [mul, 2l+1] rows keep a channel's components together, [2l+1, mul] rows keep a component's channels
+        together (then a wave's accesses are contiguous without any per-lane vector)."""
+        if self.ir_mul:
+            return f"{blk.off} + u", blk.mul
+        return f"{blk.off} + u * {blk.d}", 1
+
+    def _y_index(self, b2, v: str, j: int) -> str:
+        if self.ir_mul:
+            return f"{b2.off + j * b2.mul} + ({v})"
+        return f"{b2.off} + ({v}) * {b2.d} + {j}"
 
     @staticmethod
     def _xv(xname, b: int, i: int) -> str:
@@ -252,8 +276,7 @@ class UvuEmitter:
         low = self.low
 
         def y(p: Path, v: str, j: int) -> str:
-            b2 = low.in2[p.i2]
-            return f"yrow[{b2.off} + ({v}) * {b2.d} + {j}]"
+            return f"yrow[{self._y_index(low.in2[p.i2], v, j)}]"
 
         def w(p: Path, v: str) -> str:
             return f"((u < {low.in1[p.i1].mul}) ? wrow[{p.woff} + u * {low.in2[p.i2].mul} + ({v})] : T(0))"
@@ -265,7 +288,7 @@ class UvuEmitter:
 
         def y(p: Path, v: str, j: int) -> str:
             b2 = low.in2[p.i2]
-            return f"{name}.y[{b2.off + int(v) * b2.d + j}]"
+            return f"{name}.y[{b2.off + (j * b2.mul + int(v) if self.ir_mul else int(v) * b2.d + j)}]"
 
         def w(p: Path, v: str) -> str:
             return f"{name}.w[{self.wslot[p.index] + int(v)}]"
@@ -292,9 +315,10 @@ class UvuEmitter:
         for b in blocks:
             blk = low.in1[b]
             s.open(f"if (u < {blk.mul})")
-            s(f"const T* xp = {rowexpr} + {blk.off} + u * {blk.d};")
+            base, st = self._lane_ptr(blk)
+            s(f"const T* xp = {rowexpr} + {base};")
             for i in range(blk.d):
-                s(f"{dst}.b{b}[{i}] = xp[{i}];")
+                s(f"{dst}.b{b}[{i}] = xp[{i * st}];")
             s.close(" else {")
             s.level += 1
             for i in range(blk.d):
@@ -440,12 +464,13 @@ class UvuEmitter:
         for io in self.segments[si]:
             bo = low.out[io]
             s.open(f"if ({guard} && u < {bo.mul})")
-            s(f"T* zp = {rowexpr} + {bo.off} + u * {bo.d};")
+            base, st = self._lane_ptr(bo)
+            s(f"T* zp = {rowexpr} + {base};")
             for k in range(bo.d):
                 if atomic:
-                    s(f"oeq_atomic_add(zp + {k}, a.o{io}[{k}]);")
+                    s(f"oeq_atomic_add(zp + {k * st}, a.o{io}[{k}]);")
                 else:
-                    s(f"zp[{k}] = a.o{io}[{k}];")
+                    s(f"zp[{k * st}] = a.o{io}[{k}];")
             s.close()
 
     def _zero_untouched_out(self, s: Src, rowexpr: str, guard: str):
@@ -649,7 +674,7 @@ class UvuEmitter:
             for b in "AB":
                 s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
             self._emit_stage3_offsets(s)
-        self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave()
+        self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave() and not self.ir_mul
         if self.tr_atomics:
             s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.out[io].d for io in self.used_out)}];")
 
@@ -735,9 +760,10 @@ class UvuEmitter:
         for io in ios:
             bo = low.out[io]
             s.open(f"if (u < {bo.mul})")
-            s(f"const T* gp = {rowexpr} + {bo.off} + u * {bo.d};")
+            base, st = self._lane_ptr(bo)
+            s(f"const T* gp = {rowexpr} + {base};")
             for k in range(bo.d):
-                s(f"{dst}.o{io}[{k}] = gp[{k}];")
+                s(f"{dst}.o{io}[{k}] = gp[{k * st}];")
             s.close(" else {")
             s.level += 1
             for k in range(bo.d):
@@ -758,9 +784,10 @@ class UvuEmitter:
             if g_on_demand_row is not None:
                 s(f"T gk[{bo.d}];")
                 s.open(f"if (u < {bo.mul}{' && ' + g_guard if g_guard else ''})")
-                s(f"const T* gp = {g_on_demand_row} + {bo.off} + u * {bo.d};")
+                base, st = self._lane_ptr(bo)
+                s(f"const T* gp = {g_on_demand_row} + {base};")
                 for k in range(bo.d):
-                    s(f"gk[{k}] = gp[{k}];")
+                    s(f"gk[{k}] = gp[{k * st}];")
                 s.close(" else {")
                 s.level += 1
                 for k in range(bo.d):
@@ -803,7 +830,7 @@ class UvuEmitter:
                 else:
                     s(f"dwacc[{base_slot} + {v}] += dwv;")
                 for j in js:
-                    s(f"dy[{b2.off} + ({v}) * {b2.d} + {j}] += wv * h{j};")
+                    s(f"dy[{self._y_index(b2, v, j)}] += wv * h{j};")
 
             self._for_v(s, p, body)
             s.close()
@@ -873,12 +900,13 @@ class UvuEmitter:
         for b in self.used_in1:
             blk = low.in1[b]
             s.open(f"if ({guard} && u < {blk.mul})")
-            s(f"T* dp = {rowexpr} + {blk.off} + u * {blk.d};")
+            base, st = self._lane_ptr(blk)
+            s(f"T* dp = {rowexpr} + {base};")
             for i in range(blk.d):
                 if atomic:
-                    s(f"oeq_atomic_add(dp + {i}, dx.b{b}[{i}]);")
+                    s(f"oeq_atomic_add(dp + {i * st}, dx.b{b}[{i}]);")
                 else:
-                    s(f"dp[{i}] = dx.b{b}[{i}];")
+                    s(f"dp[{i * st}] = dx.b{b}[{i}];")
             s.close()
 
     def _zero_untouched_in1(self, s: Src, rowexpr: str, guard: str):
@@ -996,7 +1024,7 @@ class UvuEmitter:
             for b in "AB":
                 s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
             self._emit_stage3_offsets(s)
-        self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave()
+        self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave() and not self.ir_mul
         if self.tr_atomics:
             s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.in1[b].d for b in self.used_in1)}];")
         resident = deterministic and (self.g_resident if g_resident is None else g_resident)
