@@ -272,6 +272,19 @@ def main():
         }
         del Ya, Wa
 
+        # atomic mode on the receiver-sorted list: runs of one receiver are summed in registers and
+        # flushed once, so the atomics are per node, not per edge
+        def step_atomic_sorted():
+            ops.conv_forward(X, Y, W, tr, tc, dummy, conv_a.kid)
+            ops.conv_backward(X, Y, W, G, tr, tc, dummy, conv_a.kid)
+
+        ms_as = time_steps(step_atomic_sorted, args.steps, 1)
+        modes["atomic_sorted"] = {
+            "ms_per_step": ms_as, "edges_per_s": E / (ms_as * 1e-3),
+            "gflops": (fwd_flops + bwd_flops) * E / (ms_as * 1e-3) / 1e9,
+            "hbm_roofline_frac": (fwd_bytes + bwd_bytes) / (ms_as * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        }
+
     extras = {}
     if not args.no_extras:
         # Same graph with nodes numbered along a Z-order curve (core/graph.py: spatial_order): a

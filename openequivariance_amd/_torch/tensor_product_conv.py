@@ -24,18 +24,18 @@ from . import ops
 from .utils import compute_units, oeq_to_torch_dtype, torch_to_oeq_dtype
 
 
-def build_conv_module(problem: TPProblem, deterministic: bool):
+def build_conv_module(problem: TPProblem, deterministic: bool, kahan: bool = False):
     low = lower(problem)
     if low.mode == "uvu":
         from ..codegen import uvu
-        return uvu.conv_module(low, deterministic, compute_units())
+        return uvu.conv_module(low, deterministic, compute_units(), kahan)
     # 'uvw': no fused kernel; the batch kernels run on gathered rows and an ordered segment sum (or torch's
     # index_add_ in atomic mode) scatters the result, like the reference's unfused convolution
     # (core/ConvolutionBase.py:292-301, _torch/TensorProductConv.py:595-640).
     from .. import runtime as rt
     from ..codegen import uvw
     cu = compute_units()
-    src, dims, descs = uvw.tp_module(low, cu)
+    src, dims, descs = uvw.tp_module(low, cu, kahan)
     descs = list(descs) + [(rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, cu * 16),
                            (rt.ROLE_SEGMENT_SUM, "oeq_segment_sum", 256, 1, cu * 32)]
     return src, dims, descs
@@ -49,7 +49,8 @@ class TensorProductConv(torch.nn.Module):
     :param deterministic: ``False``: any edge order, floating-point atomics.
            ``True``: receiver-sorted CSR walk with fixed summation order
            (bit-identical from run to run). *Default*: ``False``.
-    :param kahan: compensated summation; not implemented here (raises).
+    :param kahan: with ``deterministic=True``: Kahan-compensated summation over the edges of a node
+           (receiver's output in forward, sender's gradient in backward). *Default*: ``False``.
     :param use_opaque: deprecated, ignored.
     """
 
@@ -63,9 +64,9 @@ class TensorProductConv(torch.nn.Module):
     def _init_class(self):
         problem: TPProblem = self.input_args["problem"].clone()
         deterministic = bool(self.input_args["deterministic"])
-        if self.input_args["kahan"]:
+        kahan = bool(self.input_args["kahan"])
+        if kahan:
             assert deterministic, "kahan=True requires deterministic=True"
-            raise NotImplementedError("Kahan-compensated accumulation is not implemented in this package")
         if deterministic:
             assert not problem.shared_weights, "Deterministic convolution does not support shared weights"
         self.config = problem
@@ -76,7 +77,7 @@ class TensorProductConv(torch.nn.Module):
         self.L3_dim = low.L3
         self.weight_numel = problem.weight_numel
         entry = ops.KernelEntry(
-            lambda p=problem, d=deterministic: build_conv_module(p, d), low.L1, low.L2, low.L3, low.WN,
+            lambda p=problem, d=deterministic, k=kahan: build_conv_module(p, d, k), low.L1, low.L2, low.L3, low.WN,
             low.shared_weights, oeq_to_torch_dtype(problem.irrep_dtype), deterministic=deterministic,
             unfused=low.mode != "uvu",
         )

@@ -45,10 +45,12 @@ def tuning(defaults: dict) -> dict:
 
 
 class UvuEmitter:
-    def __init__(self, low: Lowered, *, acc_budget_words: int = 128, g_resident_words: int = 128):
+    def __init__(self, low: Lowered, *, acc_budget_words: int = 128, g_resident_words: int = 128,
+                 kahan: bool = False):
         assert low.mode == "uvu"
         self.low = low
         self.ir_mul = low.ir_mul
+        self.kahan = kahan  # conv forward: compensated (Kahan) summation over a receiver's edges
         self.T = low.ctype
         self.words = 1 if low.elem_size == 4 else 2
         self.LPR = low.lanes_per_row
@@ -361,6 +363,15 @@ class UvuEmitter:
                 for k in range(low.out[io].d):
                     s(f"a.o{io}[{k}] = T(0);")
             s.close()
+            if self.kahan:
+                # c holds one edge's contribution plus the rounding error carried from the previous
+                # addition; afterwards it holds the part of it that did not fit into a
+                s.open(f"OEQ_DEV void kahan_seg{si}(A{si}_t& c, A{si}_t& a)")
+                for io in seg:
+                    for k in range(low.out[io].d):
+                        e = f"o{io}[{k}]"
+                        s(f"{{ const T y = c.{e}; const T t = a.{e} + y; c.{e} = y - (t - a.{e}); a.{e} = t; }}")
+                s.close()
 
     def _emit_load_edge(self, s: Src, name: str, in1_blocks: List[int], paths: List[Path]):
         """load_edge: fetch X[cols[e]] (the listed blocks), the weights of the
@@ -684,22 +695,30 @@ class UvuEmitter:
                     s(f"load_edge_f{si}({buf}, {e}, L1_in, L2_in, W, cols, u);")
             return load
 
+        kahan = self.kahan and deterministic
+        acc = "c" if kahan else "a"
+
         def make_compute(si):
             def compute(buf, e):
-                if mode == 3:
-                    s(f"fwd_seg{si}_lds(&s_stage{buf}[wave][0], ul, a);")
-                elif self.can_preload:
-                    s(f"fwd_seg{si}_pre({buf}, a);")
-                else:
-                    s.open("")
-                    s(f"const T* xrow = L1_in + cols[{e}] * {low.L1};")
-                    s(f"const T* yrow = L2_in + {e} * {low.L2};")
-                    s(f"const T* wrow = W{'' if low.shared_weights else f' + {e} * {low.WN}'};")
-                    s("X_t x;")
-                    self._load_x(s, "xrow", self.seg_in1[si])
-                    s(f"fwd_seg{si}(x, yrow, wrow, u, a);")
-                    s.close()
+                inner(si, buf, e)
+                if kahan:
+                    s(f"kahan_seg{si}(c, a);")
             return compute
+
+        def inner(si, buf, e):
+            if mode == 3:
+                s(f"fwd_seg{si}_lds(&s_stage{buf}[wave][0], ul, {acc});")
+            elif self.can_preload:
+                s(f"fwd_seg{si}_pre({buf}, {acc});")
+            else:
+                s.open("")
+                s(f"const T* xrow = L1_in + cols[{e}] * {low.L1};")
+                s(f"const T* yrow = L2_in + {e} * {low.L2};")
+                s(f"const T* wrow = W{'' if low.shared_weights else f' + {e} * {low.WN}'};")
+                s("X_t x;")
+                self._load_x(s, "xrow", self.seg_in1[si])
+                s(f"fwd_seg{si}(x, yrow, wrow, u, {acc});")
+                s.close()
 
         if deterministic:
             self._node_loop_open(s, G, xcd)
@@ -708,6 +727,8 @@ class UvuEmitter:
             for si in range(len(self.segments)):
                 s.open("")
                 s(f"A{si}_t a; zero_seg{si}(a);")
+                if kahan:
+                    s(f"A{si}_t c; zero_seg{si}(c);")
                 self._edge_loop(s, "e0 + r", "e1", make_load(si), make_compute(si), mode)
                 if R > 1:
                     # fold the R lane groups (fixed order) into group 0
@@ -1137,17 +1158,23 @@ def tp_module(low: Lowered, compute_units: int = 256):
     return s.text(), dims, descs
 
 
-def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256):
-    """Source + launch descriptors for the fused convolution (forward, backward)."""
+def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kahan: bool = False):
+    """Source + launch descriptors for the fused convolution (forward, backward). ``kahan``
+    (deterministic mode only): compensated summation where rows are summed over edges, i.e. the
+    receiver's output in `forward` and the sender's gradient in `fixup_backward`, as in the
+    reference (templates/loop_unroll_conv_det.cuh:70-94, 135-160, 227-271)."""
     from .. import runtime as rt
 
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
     t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
                     conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1))
-    em = UvuEmitter(low, acc_budget_words=t["conv_acc"])
+    assert deterministic or not kahan, "kahan=True requires deterministic=True"
+    if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
+        t["conv_acc"] = min(t["conv_acc"], 48)
+    em = UvuEmitter(low, acc_budget_words=t["conv_acc"], kahan=kahan)
     s = Src()
     s(prelude(low.ctype))
-    s(utility_kernels())
+    s(utility_kernels(kahan))
     em.emit_structs(s)
     em.emit_forward_cores(s, preloaded=True)
     G_f = t["conv_gf"]
@@ -1161,7 +1188,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256):
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, compute_units * 16),
     ]
     if deterministic:
-        s(fixup_backward_kernel(low.L1))
+        s(fixup_backward_kernel(low.L1, kahan))
         descs += [
             (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f, 0, xcd),
             (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b, 0, xcd),

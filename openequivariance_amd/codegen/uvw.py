@@ -258,17 +258,18 @@ class UvwEmitter:
         return block
 
 
-def tp_module(low: Lowered, compute_units: int = 256):
+def tp_module(low: Lowered, compute_units: int = 256, kahan: bool = False):
+    """``kahan`` only affects the ordered segment sum used by the unfused convolution."""
     from .. import runtime as rt
 
-    if low.shared_weights:
+    if low.shared_weights and not kahan:
         from . import uvw_mfma
         if uvw_mfma.supported(low):
             return uvw_mfma.tp_module(low, compute_units)
     em = UvwEmitter(low)
     s = Src()
     s(prelude(low.ctype))
-    s(utility_kernels())
+    s(utility_kernels(kahan))
     blk_f = em.emit_forward(s)
     blk_b = em.emit_backward(s)
     max_blocks_b = compute_units * 2

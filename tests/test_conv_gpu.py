@@ -203,3 +203,52 @@ def test_conv_double_backward_runs():
     assert torch.autograd.gradcheck(lambda a, b, c: conv(a, b, c, rows, cols, perm), (X, Y, W), eps=1e-6, atol=1e-6)
     assert torch.autograd.gradgradcheck(lambda a, b, c: conv(a, b, c, rows, cols, perm), (X, Y, W), eps=1e-6,
                                         atol=1e-6)
+
+
+def _hub_graph(k):
+    """Node 0 receives from, and sends to, each of the nodes 1..k."""
+    spokes = np.arange(1, k + 1, dtype=np.int64)
+    rows = np.concatenate([np.zeros(k, dtype=np.int64), spokes])
+    cols = np.concatenate([spokes, np.zeros(k, dtype=np.int64)])
+    return CoordGraph(np.zeros((k + 1, 3)), rows, cols)
+
+
+KAHAN = [
+    ("cfg1", P.config1_single_uvu),
+    ("cfg2", P.config2_nequip_uvu),
+    ("mace-medium", lambda: P.mace_problems()[1]),
+    ("uvw", lambda: _fc(False)),
+]
+
+
+@pytest.mark.parametrize("name,make", KAHAN, ids=[c[0] for c in KAHAN])
+def test_kahan_summation(name, make):
+    """kahan=True gives the same result within tolerance, and on a node with thousands of
+    same-sign terms its fp32 sums (Z of the hub in forward, dX of the hub in backward) are
+    markedly closer to the float64 oracle than plain summation."""
+    problem = make()
+    k = 3000
+    g = _hub_graph(k)
+    n, E = k + 1, 2 * k
+    X, Y, W, G = _buffers(problem, n, E, seed=9)
+    ref = R.Problem.from_spec(problem)
+    z_ref = R.conv_forward(ref, X, Y, W, g.rows, g.cols)
+    dx_ref, dy_ref, dw_ref = R.conv_backward(ref, X, Y, W, G, g.rows, g.cols)
+    tr, tc, tp = (torch.tensor(a, device="cuda") for a in (g.rows, g.cols, g.transpose_perm))
+    hub_err = {}
+    for kahan in (False, True):
+        conv = oeq.TensorProductConv(problem, deterministic=True, kahan=kahan)
+        tX = torch.tensor(X, device="cuda", requires_grad=True)
+        tY = torch.tensor(Y, device="cuda", requires_grad=True)
+        tW = torch.tensor(W, device="cuda", requires_grad=True)
+        z = conv(tX, tY, tW, tr, tc, tp)
+        z.backward(torch.tensor(G, device="cuda"))
+        assert err(z, z_ref) <= 1e-5 and err(tX.grad, dx_ref) <= 1e-5
+        assert err(tY.grad, dy_ref) <= 1e-5 and err(tW.grad, dw_ref) <= 1e-5
+        hub_err[kahan] = (err(z[0], z_ref[0]), err(tX.grad[0], dx_ref[0]))
+    # uncompensated fp32 sums of 3000 terms lose a few bits; the compensated ones stay at rounding level
+    assert hub_err[True][0] <= 2e-7 and hub_err[True][1] <= 2e-7, hub_err
+    print(name, hub_err)
+    for plain, comp in zip(hub_err[False], hub_err[True]):
+        # narrow problems pack many rows per wave, which already splits the sum into short partial sums
+        assert comp <= plain and (plain <= 1.5e-7 or comp < 0.5 * plain), hub_err
