@@ -120,6 +120,25 @@ def nequip_problems():
     ]
 
 
+def diffdock_problems():
+    """Fully connected DiffDock score-model layers with per-row weights (problems.py:273-289)."""
+    feats = "10x1o + 10x1e + 48x0e + 48x0o"
+    return [
+        FCTPP(feats, "1x0e + 1x1o", feats, shared_weights=False, label="DiffDock-L=1"),
+        FCTPP(feats, "1x0e + 1x1o + 1x2e", feats, shared_weights=False, label="DiffDock-L=2"),
+    ]
+
+
+def e3tools_problems():
+    """e3tools convolution / transformer blocks (problems.py:398-419); the second shares its weights."""
+    return [
+        FCTPP("64x0e+16x1o", "1x0e+1x1o", "80x0e+16x1o", label="e3tools_conv", shared_weights=False,
+              internal_weights=False),
+        FCTPP("64x0e+16x1o", "1x0e+1x1o", "64x0e+16x1o", label="e3tools_transformer", shared_weights=True,
+              internal_weights=False),
+    ]
+
+
 # ---------------------------------------------------------------------------
 # The five benchmark configurations
 # ---------------------------------------------------------------------------
