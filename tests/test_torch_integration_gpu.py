@@ -90,3 +90,62 @@ def test_module_inside_a_model_moves_with_to():
     out = net(x, y, w)
     assert out.dtype == torch.float64 and out.shape == (10, 5)
     assert net.tp.config.irrep_dtype == np.float64
+
+
+def _module_and_inputs(kind):
+    """The reference's export fixtures (tests/export_test.py:18-86): 32x5e (x) 1x3e -> 32x5e, batch of
+    1000 rows or the 3-node / 4-edge toy graph."""
+    problem = oeq.TPProblem("32x5e", "1x3e", "32x5e", [(0, 0, 0, "uvu", True)], shared_weights=False,
+                            internal_weights=False)
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    if kind == "batch":
+        n = 1000
+        shapes = [(n, 352), (n, 7), (n, problem.weight_numel)]
+        return oeq.TensorProduct(problem), tuple(torch.rand(*s, device="cuda", generator=gen) for s in shapes)
+    rows = torch.tensor([0, 1, 1, 2], device="cuda")
+    cols = torch.tensor([1, 0, 2, 1], device="cuda")
+    X = torch.rand(3, 352, device="cuda", generator=gen)
+    Y = torch.rand(4, 7, device="cuda", generator=gen)
+    W = torch.rand(4, problem.weight_numel, device="cuda", generator=gen)
+    if kind == "conv_atomic":
+        return oeq.TensorProductConv(problem, deterministic=False), (X, Y, W, rows, cols)
+    return oeq.TensorProductConv(problem, deterministic=True), (X, Y, W, rows, cols, torch.argsort(cols, stable=True))
+
+
+KINDS = ["batch", "conv_det", "conv_atomic"]
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_save_load_compile_export(kind):
+    module, inputs = _module_and_inputs(kind)
+    expected = module(*inputs)
+    buf = io.BytesIO()
+    torch.save(module, buf)
+    buf.seek(0)
+    loaded = torch.load(buf, weights_only=True)
+    assert torch.allclose(loaded(*inputs), expected, atol=1e-5)
+    assert torch.allclose(torch.compile(module)(*inputs), expected, atol=1e-5)
+    exported = torch.export.export(module, args=inputs, strict=False)
+    assert torch.allclose(exported.module()(*inputs), expected, atol=1e-5)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_side_stream_matches_default_stream(kind):
+    """Kernels, scratch allocations and the per-call CSR build all follow torch's current stream."""
+    module, inputs = _module_and_inputs(kind)
+    ts = tuple(t.clone().requires_grad_(t.is_floating_point()) for t in inputs)
+    expected = module(*ts)
+    expected.sum().backward()
+    grads = [t.grad.clone() for t in ts[:3]]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    ts2 = tuple(t.detach().clone().requires_grad_(t.is_floating_point()) for t in inputs)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for _ in range(3):  # back-to-back calls reuse freed scratch blocks on this stream
+            z = module(*ts2)
+        z.sum().backward()
+    side.synchronize()
+    assert torch.allclose(z, expected, atol=1e-5)
+    for a, b in zip(grads, (t.grad for t in ts2[:3])):
+        assert torch.allclose(a, b / 1.0, atol=1e-4)
