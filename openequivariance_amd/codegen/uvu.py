@@ -51,6 +51,12 @@ class UvuEmitter:
         self.low = low
         self.ir_mul = low.ir_mul
         self.kahan = kahan  # conv forward: compensated (Kahan) summation over a receiver's edges
+        # Streaming hints, so that single-use data does not displace the gathered sender rows from the
+        # caches: bit 0 = per-row weights loaded non-temporally; bit 1 = per-row results (dW, dX terms)
+        # stored non-temporally; bit 2 = the sender-side reduction reads the dX terms non-temporally;
+        # bit 3 = output rows stored / output-gradient rows loaded non-temporally; bit 4 = X rows loaded
+        # non-temporally (batch kernels only: the convolution re-reads them).
+        self.nt = 0
         self.T = low.ctype
         self.words = 1 if low.elem_size == 4 else 2
         self.LPR = low.lanes_per_row
@@ -161,7 +167,7 @@ class UvuEmitter:
             s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sx + xoff{q}), (OEQ_LPTR)(&s_stage[wave][{q * 256}]), 16, 0, 0);")
         for q in range(st["nqw"]):
             s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sw + woff{q}), "
-              f"(OEQ_LPTR)(&s_stage[wave][{st['XF'] + q * 256}]), 16, 0, 0);")
+              f"(OEQ_LPTR)(&s_stage[wave][{st['XF'] + q * 256}]), 16, 0, {2 if self.nt & 1 else 0});")
         for j in range(low.L2):
             s(f"yn[{j}] = L2_in[({e}) * {low.L2} + {j}];")
         s.close()
@@ -281,7 +287,10 @@ class UvuEmitter:
             return f"yrow[{self._y_index(low.in2[p.i2], v, j)}]"
 
         def w(p: Path, v: str) -> str:
-            return f"((u < {low.in1[p.i1].mul}) ? wrow[{p.woff} + u * {low.in2[p.i2].mul} + ({v})] : T(0))"
+            idx = f"{p.woff} + u * {low.in2[p.i2].mul} + ({v})"
+            ld = f"__builtin_nontemporal_load(&wrow[{idx}])" if (self.nt & 1) and not low.shared_weights \
+                else f"wrow[{idx}]"
+            return f"((u < {low.in1[p.i1].mul}) ? {ld} : T(0))"
 
         return y, w
 
@@ -320,7 +329,8 @@ class UvuEmitter:
             base, st = self._lane_ptr(blk)
             s(f"const T* xp = {rowexpr} + {base};")
             for i in range(blk.d):
-                s(f"{dst}.b{b}[{i}] = xp[{i * st}];")
+                s(f"{dst}.b{b}[{i}] = " + (f"__builtin_nontemporal_load(xp + {i * st});" if self.nt & 16
+                                           else f"xp[{i * st}];"))
             s.close(" else {")
             s.level += 1
             for i in range(blk.d):
@@ -480,6 +490,8 @@ class UvuEmitter:
             for k in range(bo.d):
                 if atomic:
                     s(f"oeq_atomic_add(zp + {k * st}, a.o{io}[{k}]);")
+                elif self.nt & 8:
+                    s(f"__builtin_nontemporal_store(a.o{io}[{k}], zp + {k * st});")
                 else:
                     s(f"zp[{k * st}] = a.o{io}[{k}];")
             s.close()
@@ -784,7 +796,8 @@ class UvuEmitter:
             base, st = self._lane_ptr(bo)
             s(f"const T* gp = {rowexpr} + {base};")
             for k in range(bo.d):
-                s(f"{dst}.o{io}[{k}] = gp[{k * st}];")
+                s(f"{dst}.o{io}[{k}] = " + (f"__builtin_nontemporal_load(gp + {k * st});" if self.nt & 8
+                                            else f"gp[{k * st}];"))
             s.close(" else {")
             s.level += 1
             for k in range(bo.d):
@@ -808,7 +821,8 @@ class UvuEmitter:
                 base, st = self._lane_ptr(bo)
                 s(f"const T* gp = {g_on_demand_row} + {base};")
                 for k in range(bo.d):
-                    s(f"gk[{k}] = gp[{k * st}];")
+                    s(f"gk[{k}] = " + (f"__builtin_nontemporal_load(gp + {k * st});" if self.nt & 8
+                                       else f"gp[{k * st}];"))
                 s.close(" else {")
                 s.level += 1
                 for k in range(bo.d):
@@ -846,8 +860,9 @@ class UvuEmitter:
                 for j in js[1:]:
                     s(f"dwv += y{j} * h{j};")
                 if dw_mode == "store":
-                    s(f"if (u < {b1.mul}{' && ' + dw_guard if dw_guard else ''}) "
-                      f"dwrow[{p.woff} + u * {V} + ({v})] = dwv;")
+                    st = (f"__builtin_nontemporal_store(dwv, &dwrow[{p.woff} + u * {V} + ({v})]);" if self.nt & 2
+                          else f"dwrow[{p.woff} + u * {V} + ({v})] = dwv;")
+                    s(f"if (u < {b1.mul}{' && ' + dw_guard if dw_guard else ''}) {st}")
                 else:
                     s(f"dwacc[{base_slot} + {v}] += dwv;")
                 for j in js:
@@ -911,7 +926,7 @@ class UvuEmitter:
             s("__syncthreads();")
         s.close()
 
-    def _store_dx(self, s: Src, rowexpr: str, guard: str, atomic: bool = False):
+    def _store_dx(self, s: Src, rowexpr: str, guard: str, atomic: bool = False, nt: bool = False):
         low = self.low
         if atomic and self.tr_atomics:
             for b in self.used_in1:
@@ -926,6 +941,8 @@ class UvuEmitter:
             for i in range(blk.d):
                 if atomic:
                     s(f"oeq_atomic_add(dp + {i * st}, dx.b{b}[{i}]);")
+                elif nt:
+                    s(f"__builtin_nontemporal_store(dx.b{b}[{i}], dp + {i * st});")
                 else:
                     s(f"dp[{i * st}] = dx.b{b}[{i}];")
             s.close()
@@ -990,7 +1007,7 @@ class UvuEmitter:
         self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, g_on_demand_row="grow",
                         dw_mode="acc" if shared else "store", g_guard="live" if shared else None, dw_guard="live")
         s(f"T* dxrow = L1_grad + rowc * {low.L1};")
-        self._store_dx(s, "dxrow", "live")
+        self._store_dx(s, "dxrow", "live", nt=bool(self.nt & 2))
         self._zero_untouched_in1(s, "dxrow", "live")
         self._dy_finish(s, f"L2_grad + rowc * {low.L2}", "live")
         s.close()
@@ -1085,7 +1102,7 @@ class UvuEmitter:
                                     dw_mode="acc" if shared else "store")
                 if deterministic:
                     s(f"T* dxrow = dx_tmp + {e} * {low.L1};")
-                    self._store_dx(s, "dxrow", "true")
+                    self._store_dx(s, "dxrow", "true", nt=bool(self.nt & 2))
                     self._zero_untouched_in1(s, "dxrow", "true")
                 else:
                     s(f"T* dxrow = L1_grad + cols[{e}] * {low.L1};")
@@ -1135,8 +1152,9 @@ def tp_module(low: Lowered, compute_units: int = 256):
     # at 2 (forward) and 3 (backward); fp64 is left to the compiler
     f32 = low.elem_size == 4
     t = tuning(dict(tp_acc=48, tp_gf=max(1, 4 // low.n_chunks), tp_gb=max(1, 4 // low.n_chunks),
-                    tp_wf=2 if f32 else 0, tp_wb=(2 if low.n_chunks > 1 else 3) if f32 else 0))
+                    tp_wf=2 if f32 else 0, tp_wb=(2 if low.n_chunks > 1 else 3) if f32 else 0, tp_nt=0))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
+    em.nt = t["tp_nt"]
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels())
@@ -1167,11 +1185,12 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
 
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
     t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
-                    conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1))
+                    conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
     em = UvuEmitter(low, acc_budget_words=t["conv_acc"], kahan=kahan)
+    em.nt = t["conv_nt"]
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels(kahan))
@@ -1188,7 +1207,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, compute_units * 16),
     ]
     if deterministic:
-        s(fixup_backward_kernel(low.L1, kahan))
+        s(fixup_backward_kernel(low.L1, kahan, bool(em.nt & 4)))
         descs += [
             (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f, 0, xcd),
             (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b, 0, xcd),
