@@ -75,8 +75,22 @@ typedef enum {
     OEQ_ROLE_FILL_ZERO = 6,         /* clears a buffer (used instead of memset: capture-safe) */
     OEQ_ROLE_TP_BACKWARD_WREDUCE = 7,/* shared weights: second pass of the weight-gradient reduction */
     OEQ_ROLE_SEGMENT_SUM = 8,       /* ordered sum of rows over the segments of a sorted key list */
-    OEQ_ROLE_COUNT = 9
+    OEQ_ROLE_GROUP_COUNT = 9,       /* grouping an unsorted key list: histogram, */
+    OEQ_ROLE_GROUP_SCAN = 10,       /*   exclusive scan (one block), */
+    OEQ_ROLE_GROUP_SCATTER = 11,    /*   and scatter of the item indices into their key's segment */
+    OEQ_ROLE_COUNT = 12
 } oeq_role;
+
+/* How the convolution kernels of a set find the edges of a node (oeq_problem_dims.deterministic):
+ * the reference has the first two (loop_unroll_conv_atomic.cuh / loop_unroll_conv_det.cuh). */
+typedef enum {
+    OEQ_CONV_ATOMIC = 0,   /* any edge order; contiguous edge ranges per wave, float atomics at every change of node */
+    OEQ_CONV_SORTED = 1,   /* caller passes receiver-sorted edges (+ sender-major permutation for backward); CSR walk,
+                              fixed summation order, no atomics on node data */
+    OEQ_CONV_GROUPED = 2   /* any edge order; the library groups the edge indices by receiver (and by sender for
+                              backward) on the device, then runs the same CSR walk through that index; the order
+                              within a group, hence the rounding of the sums, may differ from run to run */
+} oeq_conv_mode;
 
 /* Several descriptors may name the same role: those kernels are launched back to back, in
  * descriptor order, with the same arguments and launch shape (that of the last descriptor). */
@@ -94,7 +108,7 @@ typedef struct {
     int64_t L1_dim, L2_dim, L3_dim, weight_numel;
     int32_t elem_size;          /* 4 = float, 8 = double (irreps and weights alike) */
     int32_t shared_weights;     /* weights are [weight_numel] instead of [rows, weight_numel] */
-    int32_t deterministic;      /* conv: receiver-sorted CSR mode */
+    int32_t deterministic;      /* conv: an oeq_conv_mode value */
     int32_t wpartial_per_block; /* shared weights: partial weight-gradient rows each block of the
                                    backward kernel writes (0 = none); the workspace holds
                                    max_blocks * wpartial_per_block rows of weight_numel elements */

@@ -161,15 +161,16 @@ class UvuEmitter:
     def _emit_stage_issue(self, s: Src, e: str):
         low, st = self.low, self.stage
         s.open("")
-        s(f"const T* sx = L1_in + cols[{e}] * {low.L1};")
-        s(f"const T* sw = W + ({e}) * {low.WN};")
+        s(f"const i64 eid = OEQ_EDGE({e});")
+        s(f"const T* sx = L1_in + cols[eid] * {low.L1};")
+        s(f"const T* sw = W + eid * {low.WN};")
         for q in range(st["nqx"]):
             s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sx + xoff{q}), (OEQ_LPTR)(&s_stage[wave][{q * 256}]), 16, 0, 0);")
         for q in range(st["nqw"]):
             s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sw + woff{q}), "
               f"(OEQ_LPTR)(&s_stage[wave][{st['XF'] + q * 256}]), 16, 0, {2 if self.nt & 1 else 0});")
         for j in range(low.L2):
-            s(f"yn[{j}] = L2_in[({e}) * {low.L2} + {j}];")
+            s(f"yn[{j}] = L2_in[eid * {low.L2} + {j}];")
         s.close()
 
     def _emit_stage_read(self, s: Src, buf: str):
@@ -229,9 +230,10 @@ class UvuEmitter:
     def _emit_stage3_issue(self, s: Src, buf: str, e: str):
         low, st = self.low, self.stage3
         s.open("")
-        s(f"const T* sx = L1_in + cols[{e}] * {low.L1};")
-        s(f"const T* sw = W + ({e}) * {low.WN};")
-        s(f"const T* sy = L2_in + ({e}) * {low.L2};")
+        s(f"const i64 eid = OEQ_EDGE({e});")
+        s(f"const T* sx = L1_in + cols[eid] * {low.L1};")
+        s(f"const T* sw = W + eid * {low.WN};")
+        s(f"const T* sy = L2_in + eid * {low.L2};")
         for q in range(st["nqx"]):
             n = min(64, st["nux"] - q * 64)
             guard = f"if (lane < {n}) " if n < 64 else ""
@@ -685,7 +687,7 @@ class UvuEmitter:
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void forward(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
             "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-            "const i64* __restrict__ rowptr)"
+            "const i64* __restrict__ rowptr, const i64* __restrict__ eperm)"
         )
         self._lane_prologue(s)
         if self.can_preload:
@@ -704,7 +706,7 @@ class UvuEmitter:
         def make_load(si):
             def load(buf, e):
                 if self.can_preload:
-                    s(f"load_edge_f{si}({buf}, {e}, L1_in, L2_in, W, cols, u);")
+                    s(f"load_edge_f{si}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u);")
             return load
 
         kahan = self.kahan and deterministic
@@ -724,9 +726,10 @@ class UvuEmitter:
                 s(f"fwd_seg{si}_pre({buf}, {acc});")
             else:
                 s.open("")
-                s(f"const T* xrow = L1_in + cols[{e}] * {low.L1};")
-                s(f"const T* yrow = L2_in + {e} * {low.L2};")
-                s(f"const T* wrow = W{'' if low.shared_weights else f' + {e} * {low.WN}'};")
+                s(f"const i64 eid = OEQ_EDGE({e});")
+                s(f"const T* xrow = L1_in + cols[eid] * {low.L1};")
+                s(f"const T* yrow = L2_in + eid * {low.L2};")
+                s(f"const T* wrow = W{'' if low.shared_weights else f' + eid * {low.WN}'};")
                 s("X_t x;")
                 self._load_x(s, "xrow", self.seg_in1[si])
                 s(f"fwd_seg{si}(x, yrow, wrow, u, {acc});")
@@ -767,7 +770,7 @@ class UvuEmitter:
 
                 def before_edge(e, si=si):
                     s.open("")
-                    s(f"const i64 row = rows[{e}];")
+                    s(f"const i64 row = rows[OEQ_EDGE({e})];")
                     s.open("if (row != cur)")
                     s.open("if (cur >= 0)")
                     s(f"T* zrow = L3_out + cur * {low.L3};")
@@ -1045,7 +1048,7 @@ class UvuEmitter:
             "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
             "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
             "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp)"
+            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm)"
         )
         self._lane_prologue(s)
         if self.NCH > 1:
@@ -1069,11 +1072,13 @@ class UvuEmitter:
 
         def load(buf, e):
             if self.can_preload:
-                s(f"load_edge_b({buf}, {e}, L1_in, L2_in, W, cols, u);")
+                s(f"load_edge_b({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u);")
 
         def make_compute(grow_expr_of):
-            def compute(buf, e):
+            def compute(buf, pos):
                 s.open("")
+                s(f"const i64 eid = OEQ_EDGE({pos});")
+                e = "eid"
                 if mode == 3:
                     s(f"const T* sb = &s_stage{buf}[wave][0];")
                     xname, yacc, wacc = self._acc_staged3("sb")
@@ -1177,48 +1182,71 @@ def tp_module(low: Lowered, compute_units: int = 256):
 
 
 def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kahan: bool = False):
-    """Source + launch descriptors for the fused convolution (forward, backward). ``kahan``
-    (deterministic mode only): compensated summation where rows are summed over edges, i.e. the
-    receiver's output in `forward` and the sender's gradient in `fixup_backward`, as in the
+    """Source + launch descriptors for the fused convolution (forward, backward).
+
+    ``deterministic``: the caller passes receiver-sorted edges and the sender-major permutation; the
+    kernels walk each node's edge segment (no atomics on node data, fixed summation order). Otherwise
+    the edge order is arbitrary and, by default, the library groups the edge indices by receiver and
+    by sender on the device and runs the same kernels through that index (``conv_sort=0`` in
+    ``OEQ_AMD_TUNE`` selects the kernels that walk contiguous edge ranges and flush with float atomics
+    instead, the scheme of the reference's templates/loop_unroll_conv_atomic.cuh).
+
+    ``kahan`` (deterministic mode only): compensated summation where rows are summed over edges, i.e.
+    the receiver's output in `forward` and the sender's gradient in `fixup_backward`, as in the
     reference (templates/loop_unroll_conv_det.cuh:70-94, 135-160, 227-271)."""
     from .. import runtime as rt
 
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
     t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
-                    conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15))
+                    conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
+                    conv_sort=1))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
+    if deterministic:
+        mode = rt.CONV_SORTED
+    else:
+        mode = rt.CONV_GROUPED if t["conv_sort"] else rt.CONV_ATOMIC
+    walk = mode != rt.CONV_ATOMIC  # kernels walk per-node edge segments
     em = UvuEmitter(low, acc_budget_words=t["conv_acc"], kahan=kahan)
     em.nt = t["conv_nt"]
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels(kahan))
+    # position in the walk -> edge index: through the library's grouping when there is one
+    s("#define OEQ_EDGE(j) (eperm ? eperm[(j)] : (j))")
     em.emit_structs(s)
     em.emit_forward_cores(s, preloaded=True)
     G_f = t["conv_gf"]
     G_b = 1 if em.NCH > 1 else t["conv_gb"]
     xcd = max(1, t["conv_xcd"])
-    blk_f = em.emit_conv_forward(s, G_f, deterministic, t["conv_pipe_f"], t["conv_wf"], xcd, bool(t["conv_tra"]))
+    blk_f = em.emit_conv_forward(s, G_f, walk, t["conv_pipe_f"], t["conv_wf"], xcd, bool(t["conv_tra"]))
     gres = None if t["conv_gres"] < 0 else bool(t["conv_gres"])
-    blk_b = em.emit_conv_backward(s, deterministic, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd, bool(t["conv_tra"]))
+    blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd, bool(t["conv_tra"]))
     descs = [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, compute_units * 16),
     ]
-    if deterministic:
+    if walk:
         s(fixup_backward_kernel(low.L1, kahan, bool(em.nt & 4)))
         descs += [
             (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f, 0, xcd),
             (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b, 0, xcd),
             (rt.ROLE_CONV_FIXUP_BACKWARD, "fixup_backward", 256, 1, 0),
         ]
+        if mode == rt.CONV_GROUPED:
+            descs += [
+                (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, compute_units * 16),
+                (rt.ROLE_GROUP_SCAN, "oeq_group_scan", 1024, 1, 1),
+                (rt.ROLE_GROUP_SCATTER, "oeq_group_scatter", 256, 256 * 4, compute_units * 16),
+            ]
     else:
-        # edge ranges: about 8 consecutive edges per wave group
+        # edge ranges: about conv_epw consecutive edges per wave group
+        epw = max(1, t["conv_epw"])
         descs += [
-            (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f * em.R * 8, compute_units * 32),
-            (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b * em.R * 8, compute_units * 32),
+            (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f * em.R * epw, compute_units * 32),
+            (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b * em.R * epw, compute_units * 32),
         ]
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
-                shared_weights=int(low.shared_weights), deterministic=int(deterministic), wpartial_per_block=0)
+                shared_weights=int(low.shared_weights), deterministic=mode, wpartial_per_block=0)
     return s.text(), dims, descs

@@ -154,6 +154,23 @@ struct oeq_kernels {
         void* args[] = {&n_items, &n_segments, &keys, &perm, &ptr};
         return launch(OEQ_ROLE_SEGMENT_PTR, n_items + 1, args, stream);
     }
+
+    // Counting sort of the item indices 0..n_items-1 by key: ptr[0..n_segments] = segment starts,
+    // perm = item indices grouped by key (unordered within a group); cursor is scratch of n_segments+1.
+    int group_by_key(int64_t n_items, int64_t n_segments, const int64_t* keys, int64_t* ptr, int64_t* cursor,
+                     int64_t* perm, void* stream) {
+        int rc = fill_zero(ptr, (size_t)(n_segments + 1) * sizeof(int64_t), stream);
+        if (rc) return rc;
+        void* cargs[] = {&n_items, &keys, &ptr};
+        rc = launch(OEQ_ROLE_GROUP_COUNT, n_items, cargs, stream);
+        if (rc) return rc;
+        int64_t n = n_segments + 1;
+        void* sargs[] = {&n, &ptr, &cursor};
+        rc = launch(OEQ_ROLE_GROUP_SCAN, 1, sargs, stream);
+        if (rc) return rc;
+        void* pargs[] = {&n_items, &keys, &cursor, &perm};
+        return launch(OEQ_ROLE_GROUP_SCATTER, n_items, pargs, stream);
+    }
 };
 
 extern "C" {
@@ -371,17 +388,22 @@ int oeq_tp_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in, void* 
 // fused graph convolution
 // ---------------------------------------------------------------------------
 
+// Workspace layouts. SORTED: forward [rowptr]; backward [rowptr | colptr | dx_tmp].
+// GROUPED: forward [rowptr | cursor | rperm]; backward [rowptr | colptr | cursor | rperm | sperm | dx_tmp].
+static size_t ptr_bytes_of(int64_t node_count) { return align_up((size_t)(node_count + 1) * sizeof(int64_t), 256); }
+static size_t perm_bytes_of(int64_t nnz) { return align_up((size_t)nnz * sizeof(int64_t), 256); }
+
 size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
-    (void)nnz;
-    if (!k || !k->dims.deterministic) return 0;
-    return align_up((size_t)(node_count + 1) * sizeof(int64_t), 256);
+    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
+    if (k->dims.deterministic == OEQ_CONV_SORTED) return ptr_bytes_of(node_count);
+    return 2 * ptr_bytes_of(node_count) + perm_bytes_of(nnz);
 }
 
 size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
-    if (!k || !k->dims.deterministic) return 0;
-    size_t ptr_bytes = align_up((size_t)(node_count + 1) * sizeof(int64_t), 256);
+    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
     size_t tmp_bytes = align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256);
-    return 2 * ptr_bytes + tmp_bytes;
+    if (k->dims.deterministic == OEQ_CONV_SORTED) return 2 * ptr_bytes_of(node_count) + tmp_bytes;
+    return 3 * ptr_bytes_of(node_count) + 2 * perm_bytes_of(nnz) + tmp_bytes;
 }
 
 int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
@@ -394,22 +416,30 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void
     const size_t out_bytes = (size_t)node_count * k->dims.L3_dim * k->dims.elem_size;
     if (nnz == 0) return k->fill_zero(L3_out, out_bytes, stream);
     if (!L1_in || !L2_in || !W || !rows || !cols) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL buffer");
-    int64_t* rowptr = nullptr;
+    int64_t *rowptr = nullptr, *rperm = nullptr;
+    const int mode = k->dims.deterministic;
     int rc;
-    if (k->dims.deterministic) {
+    if (mode != OEQ_CONV_ATOMIC) {
         size_t need = oeq_conv_forward_workspace_bytes(k, node_count, nnz);
         if (!workspace || workspace_bytes < need)
             return fail(OEQ_ERR_INVALID, "oeq_conv_forward: workspace too small (%zu < %zu bytes)", workspace_bytes,
                         need);
         rowptr = (int64_t*)workspace;
-        rc = k->segment_ptr(nnz, node_count, rows, nullptr, rowptr, stream);
+        if (mode == OEQ_CONV_SORTED) {
+            rc = k->segment_ptr(nnz, node_count, rows, nullptr, rowptr, stream);
+        } else {
+            const size_t pb = ptr_bytes_of(node_count);
+            int64_t* cursor = (int64_t*)((char*)workspace + pb);
+            rperm = (int64_t*)((char*)workspace + 2 * pb);
+            rc = k->group_by_key(nnz, node_count, rows, rowptr, cursor, rperm, stream);
+        }
         if (rc) return rc;
     } else {
         rc = k->fill_zero(L3_out, out_bytes, stream);
         if (rc) return rc;
     }
-    void* args[] = {&node_count, &nnz, &L1_in, &L2_in, &W, &L3_out, &rows, &cols, &rowptr};
-    return k->launch(OEQ_ROLE_CONV_FORWARD, k->dims.deterministic ? node_count : nnz, args, stream);
+    void* args[] = {&node_count, &nnz, &L1_in, &L2_in, &W, &L3_out, &rows, &cols, &rowptr, &rperm};
+    return k->launch(OEQ_ROLE_CONV_FORWARD, mode != OEQ_CONV_ATOMIC ? node_count : nnz, args, stream);
 }
 
 int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, void* L1_grad,
@@ -433,31 +463,46 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
     if (!L1_in || !L2_in || !L2_grad || !W || !W_grad || !L3_grad || !rows || !cols)
         return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL buffer");
 
-    int64_t *rowptr = nullptr, *colptr = nullptr;
+    int64_t *rowptr = nullptr, *colptr = nullptr, *rperm = nullptr;
+    const int64_t* sperm = transpose_perm;
     void* dx_tmp = nullptr;
-    if (k->dims.deterministic) {
-        if (!transpose_perm) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: deterministic mode needs transpose_perm");
+    const int mode = k->dims.deterministic;
+    if (mode != OEQ_CONV_ATOMIC) {
+        if (mode == OEQ_CONV_SORTED && !transpose_perm)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: deterministic mode needs transpose_perm");
         size_t need = oeq_conv_backward_workspace_bytes(k, node_count, nnz);
         if (!workspace || workspace_bytes < need)
             return fail(OEQ_ERR_INVALID, "oeq_conv_backward: workspace too small (%zu < %zu bytes)", workspace_bytes,
                         need);
-        size_t ptr_bytes = align_up((size_t)(node_count + 1) * sizeof(int64_t), 256);
+        const size_t pb = ptr_bytes_of(node_count), qb = perm_bytes_of(nnz);
         rowptr = (int64_t*)workspace;
-        colptr = (int64_t*)((char*)workspace + ptr_bytes);
-        dx_tmp = (char*)workspace + 2 * ptr_bytes;
-        rc = k->segment_ptr(nnz, node_count, rows, nullptr, rowptr, stream);
-        if (rc) return rc;
-        rc = k->segment_ptr(nnz, node_count, cols, transpose_perm, colptr, stream);
-        if (rc) return rc;
+        colptr = (int64_t*)((char*)workspace + pb);
+        if (mode == OEQ_CONV_SORTED) {
+            dx_tmp = (char*)workspace + 2 * pb;
+            rc = k->segment_ptr(nnz, node_count, rows, nullptr, rowptr, stream);
+            if (rc) return rc;
+            rc = k->segment_ptr(nnz, node_count, cols, transpose_perm, colptr, stream);
+            if (rc) return rc;
+        } else {
+            int64_t* cursor = (int64_t*)((char*)workspace + 2 * pb);
+            rperm = (int64_t*)((char*)workspace + 3 * pb);
+            int64_t* sp = (int64_t*)((char*)workspace + 3 * pb + qb);
+            dx_tmp = (char*)workspace + 3 * pb + 2 * qb;
+            rc = k->group_by_key(nnz, node_count, rows, rowptr, cursor, rperm, stream);
+            if (rc) return rc;
+            rc = k->group_by_key(nnz, node_count, cols, colptr, cursor, sp, stream);
+            if (rc) return rc;
+            sperm = sp;
+        }
     } else {
         rc = k->fill_zero(L1_grad, dx_bytes, stream);
         if (rc) return rc;
     }
     void* args[] = {&node_count, &nnz,  &L1_in, &L1_grad, &L2_in,  &L2_grad, &W,
-                    &W_grad,     &L3_grad, &rows, &cols,    &rowptr, &dx_tmp};
-    rc = k->launch(OEQ_ROLE_CONV_BACKWARD, k->dims.deterministic ? node_count : nnz, args, stream);
-    if (rc || !k->dims.deterministic) return rc;
-    void* fargs[] = {&node_count, &nnz, &dx_tmp, &L1_grad, &transpose_perm, &colptr};
+                    &W_grad,     &L3_grad, &rows, &cols,    &rowptr, &dx_tmp, &rperm};
+    rc = k->launch(OEQ_ROLE_CONV_BACKWARD, mode != OEQ_CONV_ATOMIC ? node_count : nnz, args, stream);
+    if (rc || mode == OEQ_CONV_ATOMIC) return rc;
+    void* fargs[] = {&node_count, &nnz, &dx_tmp, &L1_grad, &sperm, &colptr};
     return k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
 }
 

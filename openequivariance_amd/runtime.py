@@ -43,6 +43,11 @@ ROLE_SEGMENT_PTR = 5
 ROLE_FILL_ZERO = 6
 ROLE_TP_BACKWARD_WREDUCE = 7
 ROLE_SEGMENT_SUM = 8
+ROLE_GROUP_COUNT = 9
+ROLE_GROUP_SCAN = 10
+ROLE_GROUP_SCATTER = 11
+
+CONV_ATOMIC, CONV_SORTED, CONV_GROUPED = 0, 1, 2
 
 
 class OeqError(RuntimeError):

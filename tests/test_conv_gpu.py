@@ -252,3 +252,52 @@ def test_kahan_summation(name, make):
     for plain, comp in zip(hub_err[False], hub_err[True]):
         # narrow problems pack many rows per wave, which already splits the sum into short partial sums
         assert comp <= plain and (plain <= 1.5e-7 or comp < 0.5 * plain), hub_err
+
+
+@pytest.mark.parametrize("name,make", [("cfg2", P.config2_nequip_uvu), ("cfg5-f32", P.config5_mace_conv),
+                                       ("odd-shared", lambda: _odd(True))], ids=["cfg2", "cfg5-f32", "odd-shared"])
+def test_float_atomic_kernels(name, make, monkeypatch):
+    """deterministic=False normally groups the edges on the device and walks them per node; the
+    kernels that walk edge ranges and flush with float atomics stay selectable and must agree."""
+    monkeypatch.setenv("OEQ_AMD_TUNE", "conv_sort=0")
+    problem = make()
+    tol = tol_of(problem)
+    coords, rows, cols = _graph(40, 6, seed=2)
+    E = len(rows)
+    X, Y, W, G = _buffers(problem, 40, E, seed=77)
+    ref = R.Problem.from_spec(problem)
+    z_ref = R.conv_forward(ref, X, Y, W, rows, cols)
+    dx_ref, dy_ref, dw_ref = R.conv_backward(ref, X, Y, W, G, rows, cols)
+    conv = oeq.TensorProductConv(problem, deterministic=False)
+    from openequivariance_amd import runtime as rt
+    from openequivariance_amd._torch import ops
+    assert ops.get_entry(conv.kid).kernels().dims["deterministic"] == rt.CONV_ATOMIC
+    tX, tY, tW = (torch.tensor(a, device="cuda", requires_grad=True) for a in (X, Y, W))
+    z = conv(tX, tY, tW, torch.tensor(rows, device="cuda"), torch.tensor(cols, device="cuda"))
+    z.backward(torch.tensor(G, device="cuda"))
+    for got, want in ((z, z_ref), (tX.grad, dx_ref), (tY.grad, dy_ref), (tW.grad, dw_ref)):
+        assert err(got, want) <= tol
+
+
+def test_grouped_mode_handles_hubs_and_many_nodes():
+    """The device-side grouping (histogram, one-block scan, scatter) over more nodes than one scan
+    sweep covers, with isolated nodes and one hub that receives from and sends to 5000 nodes."""
+    problem = P.config1_single_uvu()
+    n = 20000
+    rng = np.random.default_rng(3)
+    hub = np.arange(1, 5001, dtype=np.int64)
+    rows = np.concatenate([np.zeros(5000, dtype=np.int64), hub, rng.integers(6000, n, size=30000)])
+    cols = np.concatenate([hub, np.zeros(5000, dtype=np.int64), rng.integers(6000, n, size=30000)])
+    order = rng.permutation(len(rows))
+    rows, cols = rows[order], cols[order]
+    E = len(rows)
+    X, Y, W, G = _buffers(problem, n, E, seed=5)
+    ref = R.Problem.from_spec(problem)
+    z_ref = R.conv_forward(ref, X, Y, W, rows, cols)
+    dx_ref, dy_ref, dw_ref = R.conv_backward(ref, X, Y, W, G, rows, cols)
+    conv = oeq.TensorProductConv(problem, deterministic=False)
+    tX, tY, tW = (torch.tensor(a, device="cuda", requires_grad=True) for a in (X, Y, W))
+    z = conv(tX, tY, tW, torch.tensor(rows, device="cuda"), torch.tensor(cols, device="cuda"))
+    z.backward(torch.tensor(G, device="cuda"))
+    for got, want in ((z, z_ref), (tX.grad, dx_ref), (tY.grad, dy_ref), (tW.grad, dw_ref)):
+        assert err(got, want) <= 1e-5
