@@ -85,10 +85,19 @@ def test_generated_conv_sources_compile_for_gfx950(make, det):
     src, dims, descs = build_conv_module(make(), det)
     blob = rt.compile_source(src)
     names = {d[1] for d in descs}
-    assert {"forward", "backward"} <= names and (("fixup_backward" in names) == det)
-    assert dims["deterministic"] == int(det)
+    assert {"forward", "backward", "fixup_backward"} <= names
+    assert ({"oeq_group_count", "oeq_group_scan", "oeq_group_scatter"} <= names) == (not det)
+    assert dims["deterministic"] == (rt.CONV_SORTED if det else rt.CONV_GROUPED)
     # generated code must not carry packed-FP32 arithmetic or anything CUDA-flavoured
     assert "__syncwarp" not in src and "cuda" not in src.lower()
+
+
+def test_float_atomics_conv_kernels_compile(monkeypatch):
+    from openequivariance_amd._torch.tensor_product_conv import build_conv_module
+    monkeypatch.setenv("OEQ_AMD_TUNE", "conv_sort=0")
+    src, dims, descs = build_conv_module(P.config5_mace_conv(), False)
+    assert dims["deterministic"] == rt.CONV_ATOMIC and "fixup_backward" not in {d[1] for d in descs}
+    assert "oeq_atomic_add" in src and len(rt.compile_source(src)) > 0
 
 
 def test_lowering_lane_mapping():
