@@ -970,7 +970,7 @@ class UvuEmitter:
         return [(p, self.wslot[p.index]) for p in self.low.paths]
 
     # ---------------------------------------------------------- TP backward
-    def emit_tp_backward(self, s: Src, G: int, waves_per_eu: int = 0):
+    def emit_tp_backward(self, s: Src, G: int, waves_per_eu: int = 0, g_resident: bool = False):
         low = self.low
         block = 64 * self.NCH * G
         shared = low.shared_weights
@@ -1007,8 +1007,16 @@ class UvuEmitter:
         # rows past the end of the batch are clamped duplicates: their gradients are
         # zeroed (shared weights) and none of their results is stored
         yacc, wacc = self._acc_pointer()
-        self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, g_on_demand_row="grow",
-                        dw_mode="acc" if shared else "store", g_guard="live" if shared else None, dw_guard="live")
+        if g_resident and not shared:
+            # the whole output-gradient slice is requested up front, together with X and W: one long
+            # burst of loads per row instead of a load-wait-compute round per path
+            s("G_t gr;")
+            self._load_g(s, "grow", self.used_out)
+            self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, dw_mode="store", dw_guard="live")
+        else:
+            self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, g_on_demand_row="grow",
+                            dw_mode="acc" if shared else "store", g_guard="live" if shared else None,
+                            dw_guard="live")
         s(f"T* dxrow = L1_grad + rowc * {low.L1};")
         self._store_dx(s, "dxrow", "live", nt=bool(self.nt & 2))
         self._zero_untouched_in1(s, "dxrow", "live")
@@ -1153,11 +1161,14 @@ def tp_module(low: Lowered, compute_units: int = 256):
     """Source + launch descriptors for the batch tensor product (forward, backward)."""
     from .. import runtime as rt
 
-    # occupancy hints measured on MI355X: wide (multi-chunk) fp32 rows run best at 2 waves/SIMD, narrow ones
-    # at 2 (forward) and 3 (backward); fp64 is left to the compiler
+    # Measured on MI355X. Forward: 2 waves/SIMD (fp32), fp64 left to the compiler. Backward: the row's whole
+    # output-gradient slice is requested up front with X and W (tp_gres); wide (multi-chunk) rows then run best
+    # with one row per block at 1 wave/SIMD (all 512 registers: 48 % -> 67 % of HBM peak at the MACE shape),
+    # narrow rows at 3 waves/SIMD.
     f32 = low.elem_size == 4
-    t = tuning(dict(tp_acc=48, tp_gf=max(1, 4 // low.n_chunks), tp_gb=max(1, 4 // low.n_chunks),
-                    tp_wf=2 if f32 else 0, tp_wb=(2 if low.n_chunks > 1 else 3) if f32 else 0, tp_nt=0))
+    wide = low.n_chunks > 1
+    t = tuning(dict(tp_acc=48, tp_gf=1 if wide else 4, tp_gb=1 if wide else 4,
+                    tp_wf=2 if f32 else 0, tp_wb=1 if wide else (3 if f32 else 0), tp_nt=0, tp_gres=1))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
     s = Src()
@@ -1167,7 +1178,7 @@ def tp_module(low: Lowered, compute_units: int = 256):
     em.emit_forward_cores(s, preloaded=False)
     G_f, G_b = t["tp_gf"], t["tp_gb"]
     blk_f = em.emit_tp_forward(s, G_f, t["tp_wf"])
-    blk_b = em.emit_tp_backward(s, G_b, t["tp_wb"])
+    blk_b = em.emit_tp_backward(s, G_b, t["tp_wb"], bool(t["tp_gres"]))
     max_blocks_b = compute_units * 8
     descs = [
         (rt.ROLE_TP_FORWARD, "forward", blk_f, G_f * em.R, 0),
