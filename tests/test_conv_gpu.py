@@ -301,3 +301,37 @@ def test_grouped_mode_handles_hubs_and_many_nodes():
     z.backward(torch.tensor(G, device="cuda"))
     for got, want in ((z, z_ref), (tX.grad, dx_ref), (tY.grad, dy_ref), (tW.grad, dw_ref)):
         assert err(got, want) <= 1e-5
+
+
+KNOBS = ["conv_pipe_f=0,conv_pipe_b=1", "conv_pipe_f=1,conv_pipe_b=2", "conv_pipe_f=3,conv_pipe_b=3",
+         "conv_xcd=1,conv_gres=0", "conv_nt=0,conv_acc=48", "conv_sort=0,conv_tra=0", "conv_sort=0,conv_pipe_f=3,conv_nt=0",
+         "conv_wf=0,conv_wb=0,conv_gf=1,conv_gb=1"]
+
+
+@pytest.mark.parametrize("knobs", KNOBS)
+def test_kernel_shape_knobs_keep_results(knobs, monkeypatch):
+    """Every alternative the OEQ_AMD_TUNE switches select (edge-loop pipelining variants, LDS staging,
+    XCD remap, register residency, streaming hints, output segmentation, float-atomics kernels with and
+    without the LDS transpose) computes the same convolution."""
+    monkeypatch.setenv("OEQ_AMD_TUNE", knobs)
+    for make in (P.config5_mace_conv, P.config2_nequip_uvu):
+        problem = make()
+        coords, rows, cols = _graph(36, 6, seed=4)
+        E = len(rows)
+        X, Y, W, G = _buffers(problem, 36, E, seed=21)
+        ref = R.Problem.from_spec(problem)
+        z_ref = R.conv_forward(ref, X, Y, W, rows, cols)
+        dx_ref, dy_ref, dw_ref = R.conv_backward(ref, X, Y, W, G, rows, cols)
+        g = CoordGraph(coords, rows, cols)
+        for det in (True, False):
+            conv = oeq.TensorProductConv(problem, deterministic=det)
+            tX = torch.tensor(X, device="cuda", requires_grad=True)
+            tY = torch.tensor(Y[g.order], device="cuda", requires_grad=True)
+            tW = torch.tensor(W[g.order], device="cuda", requires_grad=True)
+            perm = torch.tensor(g.transpose_perm, device="cuda") if det else None
+            z = conv(tX, tY, tW, torch.tensor(g.rows, device="cuda"), torch.tensor(g.cols, device="cuda"), perm)
+            z.backward(torch.tensor(G, device="cuda"))
+            assert err(z, z_ref) <= 1e-5, (knobs, det)
+            assert err(tX.grad, dx_ref) <= 1e-5, (knobs, det)
+            assert err(tY.grad.cpu().numpy(), dy_ref[g.order]) <= 1e-5, (knobs, det)
+            assert err(tW.grad.cpu().numpy(), dw_ref[g.order]) <= 1e-5, (knobs, det)

@@ -205,3 +205,22 @@ def test_runs_on_a_side_stream():
         z = tp(tx, ty, tw)
     side.synchronize()
     assert err(z, R.tp_forward(R.Problem.from_spec(problem), x, y, w)) <= 1e-5
+
+
+@pytest.mark.parametrize("knobs", ["tp_gres=0,tp_wb=2,tp_gb=2", "tp_nt=31,tp_acc=24", "tp_wf=0,tp_wb=0,tp_gf=2,tp_gb=2"])
+def test_kernel_shape_knobs_keep_results(knobs, monkeypatch):
+    """The alternatives selectable through OEQ_AMD_TUNE (gradient slice on demand, streaming hints,
+    output segmentation, occupancy and rows per block) compute the same tensor product."""
+    monkeypatch.setenv("OEQ_AMD_TUNE", knobs)
+    for make in (P.config3_mace_uvu, P.config2_nequip_uvu, lambda: _odd_uvu(True)):
+        problem = make()
+        x, y, w, g = tp_inputs(problem, 45, seed=6)
+        ref = R.Problem.from_spec(problem)
+        z_ref = R.tp_forward(ref, x, y, w)
+        grads_ref = R.tp_backward(ref, x, y, w, g)
+        tx, ty, tw = to_gpu(x, y, w, requires_grad=True)
+        z = oeq.TensorProduct(problem)(tx, ty, tw)
+        z.backward(torch.tensor(g, device="cuda"))
+        assert err(z, z_ref) <= 1e-5
+        for got, want in zip((tx.grad, ty.grad, tw.grad), grads_ref):
+            assert err(got, want) <= 1e-5, knobs
