@@ -57,6 +57,7 @@ class UvuEmitter:
         # bit 3 = output rows stored / output-gradient rows loaded non-temporally; bit 4 = X rows loaded
         # non-temporally (batch kernels only: the convolution re-reads them).
         self.nt = 0
+        self.sched_fence = False
         self.T = low.ctype
         self.words = 1 if low.elem_size == 4 else 2
         self.LPR = low.lanes_per_row
@@ -261,12 +262,43 @@ class UvuEmitter:
         return x, y, w
 
     def _lane_ptr(self, blk) -> Tuple[str, int]:
-        """(offset of channel ``u``'s first component within a row, stride between components) of a block:
-        [mul, 2l+1] rows keep a channel's components together, [2l+1, mul] rows keep a component's channels
-        together (then a wave's accesses are contiguous without any per-lane vector)."""
+        """(pointer-offset expression of channel ``u``'s first component within a row, stride between
+        components) of a block: [mul, 2l+1] rows keep a channel's components together, [2l+1, mul] rows keep
+        a component's channels together (then a wave's accesses are contiguous without any per-lane vector).
+        The expression is applied with :meth:`_ptr`."""
         if self.ir_mul:
-            return f"{blk.off} + u", blk.mul
-        return f"{blk.off} + u * {blk.d}", 1
+            return (blk.off, 1), blk.mul
+        return (blk.off, blk.d), 1
+
+    def _ptr(self, rowexpr: str, where, mul: Optional[int] = None) -> str:
+        """Pointer to element ``const + u * stride`` of a row. When a row fills the wave the row pointer is
+        wave-uniform and the lane part is a 32-bit byte offset shared by all blocks of the same stride.
+        With ``mul`` given and lanes beyond it, the lane index is clamped (loads stay in bounds and need no
+        branch; the caller discards their values)."""
+        const, stride = where
+        u = "u" if mul is None or self._full(mul) else f"(u < {mul} ? u : {mul - 1})"
+        if self.R == 1:
+            return f"oeq_at({rowexpr} + {const}, (unsigned){u} * {stride * self.low.elem_size}u)"
+        return f"({rowexpr} + {const} + {u} * {stride})"
+
+    def _full(self, mul: int) -> bool:
+        """Every lane's channel index (0 .. lanes_per_row * chunks - 1) is a channel of such a block."""
+        return mul == self.LPR * self.NCH
+
+    def _val(self, mul: int, loaded: str, extra: Optional[str] = None) -> str:
+        """A value loaded through a clamped pointer, zeroed for lanes without a channel (and when
+        ``extra`` is false)."""
+        conds = [c for c in (None if self._full(mul) else f"u < {mul}", extra) if c]
+        return f"oeq_sel({' && '.join(conds)}, {loaded})" if conds else loaded
+
+    def _store_cond(self, mul: int, *guards) -> Optional[str]:
+        conds = [g for g in guards if g and g != "true"]
+        if not self._full(mul):
+            conds.append(f"u < {mul}")
+        return " && ".join(conds) if conds else None
+
+    def _open_if(self, s: Src, cond: Optional[str]):
+        s.open(f"if ({cond})" if cond else "")
 
     def _y_index(self, b2, v: str, j: int) -> str:
         if self.ir_mul:
@@ -289,10 +321,10 @@ class UvuEmitter:
             return f"yrow[{self._y_index(low.in2[p.i2], v, j)}]"
 
         def w(p: Path, v: str) -> str:
-            idx = f"{p.woff} + u * {low.in2[p.i2].mul} + ({v})"
-            ld = f"__builtin_nontemporal_load(&wrow[{idx}])" if (self.nt & 1) and not low.shared_weights \
-                else f"wrow[{idx}]"
-            return f"((u < {low.in1[p.i1].mul}) ? {ld} : T(0))"
+            mul = low.in1[p.i1].mul
+            wp = self._ptr("wrow", (f"{p.woff} + ({v})", low.in2[p.i2].mul), mul)
+            ld = f"__builtin_nontemporal_load({wp})" if (self.nt & 1) and not low.shared_weights else f"*{wp}"
+            return self._val(mul, ld)
 
         return y, w
 
@@ -327,16 +359,12 @@ class UvuEmitter:
         low = self.low
         for b in blocks:
             blk = low.in1[b]
-            s.open(f"if (u < {blk.mul})")
+            s.open("")
             base, st = self._lane_ptr(blk)
-            s(f"const T* xp = {rowexpr} + {base};")
+            s(f"const T* xp = {self._ptr(rowexpr, base, blk.mul)};")
             for i in range(blk.d):
-                s(f"{dst}.b{b}[{i}] = " + (f"__builtin_nontemporal_load(xp + {i * st});" if self.nt & 16
-                                           else f"xp[{i * st}];"))
-            s.close(" else {")
-            s.level += 1
-            for i in range(blk.d):
-                s(f"{dst}.b{b}[{i}] = T(0);")
+                ld = f"__builtin_nontemporal_load(xp + {i * st})" if self.nt & 16 else f"xp[{i * st}]"
+                s(f"{dst}.b{b}[{i}] = {self._val(blk.mul, ld)};")
             s.close()
 
     def _for_v(self, s: Src, p: Path, body: Callable[[str], None]):
@@ -486,9 +514,9 @@ class UvuEmitter:
             return
         for io in self.segments[si]:
             bo = low.out[io]
-            s.open(f"if ({guard} && u < {bo.mul})")
+            self._open_if(s, self._store_cond(bo.mul, guard))
             base, st = self._lane_ptr(bo)
-            s(f"T* zp = {rowexpr} + {base};")
+            s(f"T* zp = {self._ptr(rowexpr, base)};")
             for k in range(bo.d):
                 if atomic:
                     s(f"oeq_atomic_add(zp + {k * st}, a.o{io}[{k}]);")
@@ -547,15 +575,23 @@ class UvuEmitter:
         s(f"const T* yrow = L2_in + rowc * {low.L2};")
         s(f"const T* wrow = W{'' if low.shared_weights else f' + rowc * {low.WN}'};")
         s(f"T* zrow = L3_out + rowc * {low.L3};")
+        # a row that fills the wave is live or not for the whole wave: one uniform branch around the body
+        # instead of a guard on every store
+        live = "live"
+        if self.R == 1:
+            s.open("if (live)")
+            live = "true"
         s("X_t x;")
         self._load_x(s, "xrow", self.used_in1)
         for si in range(len(self.segments)):
             s.open("")
             s(f"A{si}_t a; zero_seg{si}(a);")
             s(f"fwd_seg{si}(x, yrow, wrow, u, a);")
-            self._store_seg(s, si, "zrow", "live")
+            self._store_seg(s, si, "zrow", live)
             s.close()
-        self._zero_untouched_out(s, "zrow", "live")
+        self._zero_untouched_out(s, "zrow", live)
+        if self.R == 1:
+            s.close()
         s.close()
         s.close()
         return block
@@ -795,16 +831,12 @@ class UvuEmitter:
         low = self.low
         for io in ios:
             bo = low.out[io]
-            s.open(f"if (u < {bo.mul})")
+            s.open("")
             base, st = self._lane_ptr(bo)
-            s(f"const T* gp = {rowexpr} + {base};")
+            s(f"const T* gp = {self._ptr(rowexpr, base, bo.mul)};")
             for k in range(bo.d):
-                s(f"{dst}.o{io}[{k}] = " + (f"__builtin_nontemporal_load(gp + {k * st});" if self.nt & 8
-                                            else f"gp[{k * st}];"))
-            s.close(" else {")
-            s.level += 1
-            for k in range(bo.d):
-                s(f"{dst}.o{io}[{k}] = T(0);")
+                ld = f"__builtin_nontemporal_load(gp + {k * st})" if self.nt & 8 else f"gp[{k * st}]"
+                s(f"{dst}.o{io}[{k}] = {self._val(bo.mul, ld)};")
             s.close()
 
     def _bwd_paths(self, s: Src, *, xname: str, yacc, wacc, g_on_demand_row: Optional[str] = None,
@@ -820,16 +852,12 @@ class UvuEmitter:
             s.open("")
             if g_on_demand_row is not None:
                 s(f"T gk[{bo.d}];")
-                s.open(f"if (u < {bo.mul}{' && ' + g_guard if g_guard else ''})")
+                s.open("")
                 base, st = self._lane_ptr(bo)
-                s(f"const T* gp = {g_on_demand_row} + {base};")
+                s(f"const T* gp = {self._ptr(g_on_demand_row, base, bo.mul)};")
                 for k in range(bo.d):
-                    s(f"gk[{k}] = " + (f"__builtin_nontemporal_load(gp + {k * st});" if self.nt & 8
-                                       else f"gp[{k * st}];"))
-                s.close(" else {")
-                s.level += 1
-                for k in range(bo.d):
-                    s(f"gk[{k}] = T(0);")
+                    ld = f"__builtin_nontemporal_load(gp + {k * st})" if self.nt & 8 else f"gp[{k * st}]"
+                    s(f"gk[{k}] = {self._val(bo.mul, ld, g_guard)};")
                 s.close()
                 gname = lambda k: f"gk[{k}]"
             else:
@@ -862,16 +890,42 @@ class UvuEmitter:
                 s(f"T dwv = y{js[0]} * h{js[0]};")
                 for j in js[1:]:
                     s(f"dwv += y{j} * h{j};")
-                if dw_mode == "store":
-                    st = (f"__builtin_nontemporal_store(dwv, &dwrow[{p.woff} + u * {V} + ({v})]);" if self.nt & 2
-                          else f"dwrow[{p.woff} + u * {V} + ({v})] = dwv;")
-                    s(f"if (u < {b1.mul}{' && ' + dw_guard if dw_guard else ''}) {st}")
+                if dw_mode == "store" and self._dw_deferred(dw_guard):
+                    s(f"dwkeep[{base_slot} + {v}] = dwv;")
+                elif dw_mode == "store":
+                    dwp = self._ptr("dwrow", (f"{p.woff} + ({v})", V))
+                    st = (f"__builtin_nontemporal_store(dwv, {dwp});" if self.nt & 2 else f"*{dwp} = dwv;")
+                    cond = self._store_cond(b1.mul, dw_guard)
+                    s(f"if ({cond}) {st}" if cond else st)
                 else:
                     s(f"dwacc[{base_slot} + {v}] += dwv;")
                 for j in js:
                     s(f"dy[{self._y_index(b2, v, j)}] += wv * h{j};")
 
             self._for_v(s, p, body)
+            s.close()
+            if self.sched_fence and g_on_demand_row is not None:
+                # keep the scheduler from hoisting the next paths' gradient loads over this path:
+                # with many paths that costs more registers than a wave has
+                s("__builtin_amdgcn_sched_barrier(0);")
+
+    def _dw_deferred(self, dw_guard: Optional[str]) -> bool:
+        """Per-row weight gradients whose store needs a condition are kept in registers (``dwkeep``) and
+        stored after the last path: a conditional store inside the chain of paths splits it into many
+        basic blocks, and the compiler then moves the dY/dX accumulations to the end of the row, keeping
+        every path's operands alive until there (hundreds of registers for problems with many paths)."""
+        needs_cond = any(self._store_cond(self.low.in1[p.i1].mul, dw_guard) for p in self.low.paths)
+        return needs_cond and self.can_preload
+
+    def _flush_dwkeep(self, s: Src, dw_guard: Optional[str]):
+        low = self.low
+        for p in low.paths:
+            b1, V = low.in1[p.i1], low.in2[p.i2].mul
+            self._open_if(s, self._store_cond(b1.mul, dw_guard))
+            for v in range(V):
+                dwp = self._ptr("dwrow", (f"{p.woff} + {v}", V))
+                val = f"dwkeep[{self.wslot[p.index] + v}]"
+                s(f"__builtin_nontemporal_store({val}, {dwp});" if self.nt & 2 else f"*{dwp} = {val};")
             s.close()
 
     def _dy_reduce(self, s: Src):
@@ -938,9 +992,9 @@ class UvuEmitter:
             return
         for b in self.used_in1:
             blk = low.in1[b]
-            s.open(f"if ({guard} && u < {blk.mul})")
+            self._open_if(s, self._store_cond(blk.mul, guard))
             base, st = self._lane_ptr(blk)
-            s(f"T* dp = {rowexpr} + {base};")
+            s(f"T* dp = {self._ptr(rowexpr, base)};")
             for i in range(blk.d):
                 if atomic:
                     s(f"oeq_atomic_add(dp + {i * st}, dx.b{b}[{i}]);")
@@ -972,6 +1026,8 @@ class UvuEmitter:
     # ---------------------------------------------------------- TP backward
     def emit_tp_backward(self, s: Src, G: int, waves_per_eu: int = 0, g_resident: bool = False):
         low = self.low
+        if self.NCH > 1:
+            G = 1  # one row per block: the dY reduction across chunk waves uses block barriers
         block = 64 * self.NCH * G
         shared = low.shared_weights
         s.open(
@@ -999,28 +1055,41 @@ class UvuEmitter:
         s(f"const T* grow = L3_grad + rowc * {low.L3};")
         if not shared:
             s(f"T* dwrow = W_grad + rowc * {low.WN};")
+        # Rows past the end of the batch are clamped duplicates. A row that fills the wave is live or not
+        # for the whole wave (and, with one row per block, for the whole block, barriers included): one
+        # uniform branch around the body. Packed rows keep per-lane guards: gradients zeroed (shared
+        # weights) and no result stored.
+        live = "live"
+        if self.R == 1:
+            s.open("if (live)")
+            live = "true"
         s("X_t x, dx;")
         self._load_x(s, "xrow", self.used_in1)
         self._zero_x(s, "dx")
         s(f"T dy[{self.l2_pad}];")
         s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
-        # rows past the end of the batch are clamped duplicates: their gradients are
-        # zeroed (shared weights) and none of their results is stored
         yacc, wacc = self._acc_pointer()
+        deferred = not shared and self._dw_deferred(live)
+        if deferred:
+            s(f"T dwkeep[{self.n_wslots}];")
         if g_resident and not shared:
             # the whole output-gradient slice is requested up front, together with X and W: one long
             # burst of loads per row instead of a load-wait-compute round per path
             s("G_t gr;")
             self._load_g(s, "grow", self.used_out)
-            self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, dw_mode="store", dw_guard="live")
+            self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, dw_mode="store", dw_guard=live)
         else:
             self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, g_on_demand_row="grow",
-                            dw_mode="acc" if shared else "store", g_guard="live" if shared else None,
-                            dw_guard="live")
+                            dw_mode="acc" if shared else "store",
+                            g_guard="live" if shared and self.R > 1 else None, dw_guard=live)
+        if deferred:
+            self._flush_dwkeep(s, live)
         s(f"T* dxrow = L1_grad + rowc * {low.L1};")
-        self._store_dx(s, "dxrow", "live", nt=bool(self.nt & 2))
-        self._zero_untouched_in1(s, "dxrow", "live")
-        self._dy_finish(s, f"L2_grad + rowc * {low.L2}", "live")
+        self._store_dx(s, "dxrow", live, nt=bool(self.nt & 2))
+        self._zero_untouched_in1(s, "dxrow", live)
+        self._dy_finish(s, f"L2_grad + rowc * {low.L2}", live)
+        if self.R == 1:
+            s.close()
         s.close()
         if shared:
             # fold the R row groups of the wave, then every wave group writes one partial row
@@ -1107,12 +1176,17 @@ class UvuEmitter:
                 self._zero_x(s, "dx")
                 s(f"T dy[{self.l2_pad}];")
                 s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+                deferred = not shared and self._dw_deferred(None)
+                if deferred:
+                    s(f"T dwkeep[{self.n_wslots}];")
                 if resident:
                     self._bwd_paths(s, xname=xname, yacc=yacc, wacc=wacc, dw_mode="acc" if shared else "store")
                 else:
                     s(f"const T* grow = {grow_expr_of(e)};")
                     self._bwd_paths(s, xname=xname, yacc=yacc, wacc=wacc, g_on_demand_row="grow",
                                     dw_mode="acc" if shared else "store")
+                if deferred:
+                    self._flush_dwkeep(s, None)
                 if deterministic:
                     s(f"T* dxrow = dx_tmp + {e} * {low.L1};")
                     self._store_dx(s, "dxrow", "true", nt=bool(self.nt & 2))
@@ -1162,21 +1236,25 @@ def tp_module(low: Lowered, compute_units: int = 256):
     from .. import runtime as rt
 
     # Measured on MI355X. Forward: 2 waves/SIMD (fp32), fp64 left to the compiler. Backward: the row's whole
-    # output-gradient slice is requested up front with X and W (tp_gres); wide (multi-chunk) rows then run best
-    # with one row per block at 1 wave/SIMD (all 512 registers: 48 % -> 67 % of HBM peak at the MACE shape),
-    # narrow rows at 3 waves/SIMD.
+    # output-gradient slice is requested up front with X and W (one long burst of loads per row) at 2
+    # waves/SIMD; when that slice alone would take more than 256 registers per lane the gradients are
+    # loaded per path instead, with scheduling fences between paths, at 3 waves/SIMD.
     f32 = low.elem_size == 4
     wide = low.n_chunks > 1
+    g_words = sum(low.out[io].d for io in {p.io for p in low.paths}) * (1 if f32 else 2)
+    big = g_words > 256
     t = tuning(dict(tp_acc=48, tp_gf=1 if wide else 4, tp_gb=1 if wide else 4,
-                    tp_wf=2 if f32 else 0, tp_wb=1 if wide else (3 if f32 else 0), tp_nt=0, tp_gres=1))
+                    tp_wf=2 if f32 else 0, tp_wb=3 if big else 2, tp_nt=0, tp_gres=0 if big else 1,
+                    tp_sb=1 if big else 0))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
+    em.sched_fence = bool(t["tp_sb"])
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels())
     em.emit_structs(s)
     em.emit_forward_cores(s, preloaded=False)
-    G_f, G_b = t["tp_gf"], t["tp_gb"]
+    G_f, G_b = t["tp_gf"], (1 if em.NCH > 1 else t["tp_gb"])
     blk_f = em.emit_tp_forward(s, G_f, t["tp_wf"])
     blk_b = em.emit_tp_backward(s, G_b, t["tp_wb"], bool(t["tp_gres"]))
     max_blocks_b = compute_units * 8
