@@ -58,6 +58,9 @@ class UvuEmitter:
         # non-temporally (batch kernels only: the convolution re-reads them).
         self.nt = 0
         self.sched_fence = False
+        # plain stores of [64 x d] channel blocks go through the s_tr tile as well: bit 0 = forward outputs,
+        # bit 1 = backward dX (kernels that use it declare the tile)
+        self.tr_stores = 0
         self.T = low.ctype
         self.words = 1 if low.elem_size == 4 else 2
         self.LPR = low.lanes_per_row
@@ -505,6 +508,24 @@ class UvuEmitter:
         for t in range(d):
             s(f"oeq_atomic_add({rowexpr} + {off} + chunk * {64 * d} + {t * 64} + ul, s_tr[wave][{t * 64} + ul]);")
 
+    def _store_block_transposed(self, s: Src, rowexpr: str, off: int, d: int, val: Callable[[int], str],
+                                nt: bool = False):
+        """Store of one [64 x d] channel block through the wave-private LDS tile: every store instruction
+        of the wave then writes 64 consecutive elements. Per-lane stores of d contiguous values split into
+        16-byte and smaller pieces whose instructions each leave holes in the cache lines they touch."""
+        s("oeq_wave_sync();")
+        for k in range(d):
+            s(f"s_tr[wave][ul * {d} + {k}] = {val(k)};")
+        s("oeq_wave_sync();")
+        for t in range(d):
+            dst = f"{rowexpr} + {off} + chunk * {64 * d} + {t * 64} + ul"
+            s(f"__builtin_nontemporal_store(s_tr[wave][{t * 64} + ul], {dst});" if nt
+              else f"*({dst}) = s_tr[wave][{t * 64} + ul];")
+
+    def _can_transpose(self, blk, bit: int) -> bool:
+        return bool(self.tr_stores & bit) and self.R == 1 and not self.ir_mul and blk.d > 1 \
+            and self._full(blk.mul)
+
     def _store_seg(self, s: Src, si: int, rowexpr: str, guard: str, atomic: bool = False):
         low = self.low
         if atomic and self.tr_atomics:
@@ -514,6 +535,10 @@ class UvuEmitter:
             return
         for io in self.segments[si]:
             bo = low.out[io]
+            if not atomic and guard == "true" and self._can_transpose(bo, 1):
+                self._store_block_transposed(s, rowexpr, bo.off, bo.d, lambda k, io=io: f"a.o{io}[{k}]",
+                                             bool(self.nt & 8))
+                continue
             self._open_if(s, self._store_cond(bo.mul, guard))
             base, st = self._lane_ptr(bo)
             s(f"T* zp = {self._ptr(rowexpr, base)};")
@@ -566,6 +591,8 @@ class UvuEmitter:
             "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, T* __restrict__ L3_out)"
         )
         self._lane_prologue(s)
+        if self.tr_stores & 1 and self.R == 1:
+            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(b.d for b in low.out)}];")
         s(f"const i64 ngroups = (num_batch + {self.R - 1}) / {self.R};")
         s.open(f"for (i64 grp = (i64)blockIdx.x * {G} + g; grp < ngroups; grp += (i64)gridDim.x * {G})")
         s(f"const i64 row = grp * {self.R} + r;")
@@ -736,7 +763,7 @@ class UvuEmitter:
                 s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
             self._emit_stage3_offsets(s)
         self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave() and not self.ir_mul
-        if self.tr_atomics:
+        if self.tr_atomics or (self.tr_stores & 1 and self.R == 1):
             s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.out[io].d for io in self.used_out)}];")
 
         def make_load(si):
@@ -789,7 +816,7 @@ class UvuEmitter:
                             while m < 64:
                                 s(f"a.o{io}[{k}] += __shfl_xor(a.o{io}[{k}], {m});")
                                 m *= 2
-                self._store_seg(s, si, "zrow", "r == 0")
+                self._store_seg(s, si, "zrow", "r == 0" if self.R > 1 else "true")
                 s.close()
             self._zero_untouched_out(s, "zrow", "r == 0")
             s.close()
@@ -992,6 +1019,9 @@ class UvuEmitter:
             return
         for b in self.used_in1:
             blk = low.in1[b]
+            if not atomic and guard == "true" and self._can_transpose(blk, 2):
+                self._store_block_transposed(s, rowexpr, blk.off, blk.d, lambda i, b=b: f"dx.b{b}[{i}]", nt)
+                continue
             self._open_if(s, self._store_cond(blk.mul, guard))
             base, st = self._lane_ptr(blk)
             s(f"T* dp = {self._ptr(rowexpr, base)};")
@@ -1039,6 +1069,8 @@ class UvuEmitter:
         self._lane_prologue(s)
         if self.NCH > 1:
             s(f"__shared__ T s_dy[{G}][{self.NCH}][{self.l2_pad}];")
+        if self.tr_stores & 2 and self.R == 1:
+            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(b.d for b in low.in1)}];")
         if shared:
             s(f"T dwacc[{self.n_wslots}];")
             s(f"for (int t = 0; t < {self.n_wslots}; ++t) dwacc[t] = T(0);")
@@ -1143,7 +1175,7 @@ class UvuEmitter:
                 s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
             self._emit_stage3_offsets(s)
         self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave() and not self.ir_mul
-        if self.tr_atomics:
+        if self.tr_atomics or (self.tr_stores & 2 and self.R == 1):
             s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.in1[b].d for b in self.used_in1)}];")
         resident = deterministic and (self.g_resident if g_resident is None else g_resident)
 
@@ -1238,17 +1270,20 @@ def tp_module(low: Lowered, compute_units: int = 256):
     # Measured on MI355X. Forward: 2 waves/SIMD (fp32), fp64 left to the compiler. Backward: the row's whole
     # output-gradient slice is requested up front with X and W (one long burst of loads per row) at 2
     # waves/SIMD; when that slice alone would take more than 256 registers per lane the gradients are
-    # loaded per path instead, with scheduling fences between paths, at 3 waves/SIMD.
+    # loaded per path instead, with scheduling fences between paths, at 3 waves/SIMD. Forward outputs of
+    # full 64-channel blocks are stored through an LDS transpose (tp_trs bit 0): fp64 forward 45 % -> 66 %
+    # of HBM peak at the MACE shape, fp32 within noise; the same for dX (bit 1) measured neutral.
     f32 = low.elem_size == 4
     wide = low.n_chunks > 1
     g_words = sum(low.out[io].d for io in {p.io for p in low.paths}) * (1 if f32 else 2)
     big = g_words > 256
     t = tuning(dict(tp_acc=48, tp_gf=1 if wide else 4, tp_gb=1 if wide else 4,
                     tp_wf=2 if f32 else 0, tp_wb=3 if big else 2, tp_nt=0, tp_gres=0 if big else 1,
-                    tp_sb=1 if big else 0))
+                    tp_sb=1 if big else 0, tp_trs=1))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
     em.sched_fence = bool(t["tp_sb"])
+    em.tr_stores = t["tp_trs"]
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels())
@@ -1288,7 +1323,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
     t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
                     conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
-                    conv_sort=1))
+                    conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -1299,6 +1334,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     walk = mode != rt.CONV_ATOMIC  # kernels walk per-node edge segments
     em = UvuEmitter(low, acc_budget_words=t["conv_acc"], kahan=kahan)
     em.nt = t["conv_nt"]
+    em.tr_stores = t["conv_trs"]
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels(kahan))
