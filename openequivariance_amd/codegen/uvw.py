@@ -52,11 +52,11 @@ class UvwEmitter:
             out[n] = (names[key], c < 0)
         return out
 
-    def _row_loop_open(self, s: Src):
+    def _row_loop_open(self, s: Src, waves: int = WAVES_PER_BLOCK):
         s("const int lane = oeq_lane();")
         s("const int wave = oeq_wave();")
-        s(f"for (i64 base = (i64)blockIdx.x * {WAVES_PER_BLOCK}; base < num_batch; "
-          f"base += (i64)gridDim.x * {WAVES_PER_BLOCK}) {{")
+        s(f"for (i64 base = (i64)blockIdx.x * {waves}; base < num_batch; "
+          f"base += (i64)gridDim.x * {waves}) {{")
         s.level += 1
         s("const i64 row = base + wave;")
         s("const bool live = row < num_batch;")
@@ -109,10 +109,11 @@ class UvwEmitter:
                         started.add(k)
                     else:
                         s(f"t{k} {'-=' if neg else '+='} {q} * x[{i}];")
-                s("__syncthreads();")
+                # the tile is private to the wave (one row per wave): wave-level ordering is enough
+                s("oeq_wave_sync();")
                 for k in range(bo.d):
                     s(f"s_t[wave][{k}][lane] = {'t%d' % k if k in started else 'T(0)'};")
-                s("__syncthreads();")
+                s("oeq_wave_sync();")
                 s.close()
                 s(f"const int nu = ({b1.mul} - uc < 64) ? {b1.mul} - uc : 64;")
                 s(f"const T* wp = wrow + {p.woff} + ((i64)uc * {b2.mul} + v) * {bo.mul} + w;")
@@ -135,20 +136,57 @@ class UvwEmitter:
         return block
 
     # ------------------------------------------------------------ backward
+    TILE_BYTES = 12288  # per-wave LDS budget for one path's weight tile (larger blocks are accessed directly)
+
+    def _tile_plan(self, p: Path):
+        """Per-row weights of a path and one 64-channel chunk of u form a contiguous [rows, V, W] block.
+        Returns (max elements of such a block, vector width in elements for 16-byte copies) when it fits
+        the per-wave LDS tile, else None."""
+        low = self.low
+        if low.shared_weights:
+            return None
+        b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
+        per_u = b2.mul * bo.mul
+        rows = min(64, b1.mul)
+        elems = rows * per_u
+        if elems * low.elem_size > self.TILE_BYTES:
+            return None
+        vw = 16 // low.elem_size
+        chunk_starts = range(0, b1.mul, 64)
+        aligned = low.WN % vw == 0 and all((p.woff + uc * per_u) % vw == 0 and
+                                           (min(64, b1.mul - uc) * per_u) % vw == 0 for uc in chunk_starts)
+        return elems, (vw if aligned else 1)
+
     def emit_backward(self, s: Src):
         low = self.low
         shared = low.shared_weights
-        block = 64 * WAVES_PER_BLOCK
+        plans = {p.index: self._tile_plan(p) for p in low.paths}
+        tiled = [p for p in low.paths if plans[p.index]]
+        waves = WAVES_PER_BLOCK
+        if tiled:
+            tile_elems = (max(plans[p.index][0] for p in tiled) + 3) // 4 * 4
+            g_elems = max(low.out[p.io].mul * low.out[p.io].d for p in tiled)
+            vw = 16 // low.elem_size
+            s(f"struct __attribute__((aligned(16))) wvec_t {{ T v[{vw}]; }};")
+            # keep a block's LDS near 40 KB, so that four blocks (and at least four waves) share a CU
+            per_wave = (tile_elems + g_elems) * low.elem_size
+            waves = max(1, min(WAVES_PER_BLOCK, 40960 // per_wave))
+        self.backward_waves = waves
+        block = 64 * waves
         s.open(
             f'extern "C" __global__ __launch_bounds__({block}) void backward(i64 num_batch, '
             "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
             "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
             "const T* __restrict__ L3_grad, T* __restrict__ wpartial)"
         )
+        if tiled:
+            # one path's weights of the row, then (in place) its weight gradients; and that path's dZ block
+            s(f"__shared__ __attribute__((aligned(16))) T s_w[{waves}][{tile_elems}];")
+            s(f"__shared__ T s_g[{waves}][{g_elems}];")
         if shared:
             s(f"T* prow = wpartial + ((i64)blockIdx.x * {WAVES_PER_BLOCK} + oeq_wave()) * {low.WN};")
             s("bool first = true;")
-        self._row_loop_open(s)
+        self._row_loop_open(s, waves)
         s(f"const T* xrow = L1_in + rowc * {low.L1};")
         s(f"const T* yrow = L2_in + rowc * {low.L2};")
         s(f"const T* wrow = W{'' if shared else f' + rowc * {low.WN}'};")
@@ -170,55 +208,14 @@ class UvwEmitter:
             for p in paths:
                 b2, bo = low.in2[p.i2], low.out[p.io]
                 s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
-                s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
-                prods = self._products(s, p)
-                s(f"const i64 wbase = {p.woff} + ((i64)u * {b2.mul} + v) * {bo.mul};")
-                # G_k = sum_w W[u,v,w] * g[w,k]
-                for k in range(bo.d):
-                    s(f"T G{k} = T(0);")
-                s.open("if (uok)")
-                s.open(f"for (int w = 0; w < {bo.mul}; ++w)")
-                s("const T wv = wrow[wbase + w];")
-                for k in range(bo.d):
-                    s(f"G{k} += wv * grow[{bo.off} + w * {bo.d} + {k}];")
-                s.close()
-                s.close()
-                fstart = set()
-                for n, (i, j, k, c) in enumerate(p.nnz):
-                    q, neg = prods[n]
-                    s(f"dx[{i}] {'-=' if neg else '+='} {q} * G{k};")
-                    if k not in fstart:
-                        s(f"T f{k} = {'-' if neg else ''}{q} * x[{i}];")
-                        fstart.add(k)
-                    else:
-                        s(f"f{k} {'-=' if neg else '+='} {q} * x[{i}];")
-                pair = {}
-                for n, (i, j, k, c) in enumerate(p.nnz):
-                    if (i, k) not in pair:
-                        pair[(i, k)] = f"xg{len(pair)}"
-                        s(f"const T {pair[(i, k)]} = x[{i}] * G{k};")
-                    s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * {pair[(i, k)]};")
-                # dW[u,v,w] = sum_k f_k * g[w,k]
-                s.open(f"if (uok{' && live' if not shared else ''})")
-                s.open(f"for (int w = 0; w < {bo.mul}; ++w)")
-                terms = [f"f{k} * grow[{bo.off} + w * {bo.d} + {k}]" for k in sorted(fstart)]
-                s(f"T dwv = {terms[0]};")
-                for t in terms[1:]:
-                    s(f"dwv += {t};")
-                if shared:
-                    s("if (!live) dwv = T(0);")
-                    s("prow[wbase + w] = first ? dwv : prow[wbase + w] + dwv;")
+                if plans[p.index]:
+                    self._bwd_path_tiled(s, p, plans[p.index][1])
                 else:
-                    s("dwrow[wbase + w] = dwv;")
-                s.close()
-                s.close()
-                s.close()
+                    self._bwd_path_direct(s, p)
             s.open("if (live && uok)")
             for i in range(b1.d):
                 s(f"dxrow[{b1.off} + u * {b1.d} + {i}] = dx[{i}];")
             s.close()
-            if not paths:
-                pass
             s.close()
         if shared:
             s("first = false;")
@@ -257,6 +254,124 @@ class UvwEmitter:
         s.close()
         return block
 
+    def _cg_backward(self, s: Src, p: Path, prods, gname: str = "G"):
+        """dx, dy contributions of one (path, v) from G_k, and f_k = sum c x_i y_j (returns the k set)."""
+        b2 = self.low.in2[p.i2]
+        fstart = set()
+        for n, (i, j, k, c) in enumerate(p.nnz):
+            q, neg = prods[n]
+            s(f"dx[{i}] {'-=' if neg else '+='} {q} * {gname}{k};")
+            if k not in fstart:
+                s(f"T f{k} = {'-' if neg else ''}{q} * x[{i}];")
+                fstart.add(k)
+            else:
+                s(f"f{k} {'-=' if neg else '+='} {q} * x[{i}];")
+        pair = {}
+        for n, (i, j, k, c) in enumerate(p.nnz):
+            if (i, k) not in pair:
+                pair[(i, k)] = f"xg{len(pair)}"
+                s(f"const T {pair[(i, k)]} = x[{i}] * {gname}{k};")
+            s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * {pair[(i, k)]};")
+        return sorted(fstart)
+
+    def _bwd_path_direct(self, s: Src, p: Path):
+        """Weights read and weight gradients written straight from / to global memory, lane = u."""
+        low = self.low
+        shared = low.shared_weights
+        b2, bo = low.in2[p.i2], low.out[p.io]
+        s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
+        prods = self._products(s, p)
+        s(f"const i64 wbase = {p.woff} + ((i64)u * {b2.mul} + v) * {bo.mul};")
+        # G_k = sum_w W[u,v,w] * g[w,k]
+        for k in range(bo.d):
+            s(f"T G{k} = T(0);")
+        s.open("if (uok)")
+        s.open(f"for (int w = 0; w < {bo.mul}; ++w)")
+        s("const T wv = wrow[wbase + w];")
+        for k in range(bo.d):
+            s(f"G{k} += wv * grow[{bo.off} + w * {bo.d} + {k}];")
+        s.close()
+        s.close()
+        ks = self._cg_backward(s, p, prods)
+        # dW[u,v,w] = sum_k f_k * g[w,k]
+        s.open(f"if (uok{' && live' if not shared else ''})")
+        s.open(f"for (int w = 0; w < {bo.mul}; ++w)")
+        terms = [f"f{k} * grow[{bo.off} + w * {bo.d} + {k}]" for k in ks]
+        s(f"T dwv = {terms[0]};")
+        for t in terms[1:]:
+            s(f"dwv += {t};")
+        if shared:
+            s("if (!live) dwv = T(0);")
+            s("prow[wbase + w] = first ? dwv : prow[wbase + w] + dwv;")
+        else:
+            s("dwrow[wbase + w] = dwv;")
+        s.close()
+        s.close()
+        s.close()
+
+    def _bwd_path_tiled(self, s: Src, p: Path, vw: int):
+        """Per-row weights: the path's contiguous [rows, V, W] weight block of this u chunk is copied to
+        the wave's LDS tile with coalesced 16-byte accesses; lane u then walks its rows of the tile, the
+        weight gradients replace the weights in place and the tile is written back coalesced. Lane u
+        visits w in the rotated order (u + t) mod W, which spreads the lanes of a wave over the LDS banks
+        whatever the row stride; dZ of the path's output irrep is read from LDS in the same order."""
+        low = self.low
+        b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
+        V, Wn = b2.mul, bo.mul
+        per_u = V * Wn
+        s.open("")
+        s(f"const int nrows = ({b1.mul} - uc < 64) ? {b1.mul} - uc : 64;")
+        s(f"const int nel = nrows * {per_u};")
+        s(f"const i64 tbase = {p.woff} + (i64)uc * {per_u};")
+        s("T* tw = s_w[wave];")
+        s("T* tg = s_g[wave];")
+        s("oeq_wave_sync();  // the previous path's tile and dZ block are no longer read")
+        s(f"for (int t = lane; t < {Wn * bo.d}; t += 64) tg[t] = grow[{bo.off} + t];")
+        if vw > 1:
+            s(f"for (int t = lane * {vw}; t < nel; t += {64 * vw}) "
+              f"*(wvec_t*)(tw + t) = *(const wvec_t*)(wrow + tbase + t);")
+        else:
+            s("for (int t = lane; t < nel; t += 64) tw[t] = wrow[tbase + t];")
+        s("oeq_wave_sync();")
+        s(f"const int urow = uok ? lane : 0;  // lanes without a channel read row 0 and store nothing")
+        s(f"const int w0 = lane % {Wn};")
+        s.open(f"for (int v = 0; v < {V}; ++v)")
+        prods = self._products(s, p)
+        s(f"T* trow = tw + (urow * {V} + v) * {Wn};")
+        for k in range(bo.d):
+            s(f"T G{k} = T(0);")
+        s("int wr = w0;")
+        s("#pragma unroll 4")
+        s.open(f"for (int t = 0; t < {Wn}; ++t)")
+        s("const T wv = trow[wr];")
+        for k in range(bo.d):
+            s(f"G{k} += wv * tg[wr * {bo.d} + {k}];")
+        s(f"wr = (wr + 1 == {Wn}) ? 0 : wr + 1;")
+        s.close()
+        ks = self._cg_backward(s, p, prods)
+        s("wr = w0;")
+        s.open("if (uok)")
+        s("#pragma unroll 4")
+        s.open(f"for (int t = 0; t < {Wn}; ++t)")
+        terms = [f"f{k} * tg[wr * {bo.d} + {k}]" for k in ks]
+        s(f"T dwv = {terms[0]};")
+        for t in terms[1:]:
+            s(f"dwv += {t};")
+        s("trow[wr] = dwv;")
+        s(f"wr = (wr + 1 == {Wn}) ? 0 : wr + 1;")
+        s.close()
+        s.close()
+        s.close()
+        s("oeq_wave_sync();")
+        s.open("if (live)")
+        if vw > 1:
+            s(f"for (int t = lane * {vw}; t < nel; t += {64 * vw}) "
+              f"*(wvec_t*)(dwrow + tbase + t) = *(const wvec_t*)(tw + t);")
+        else:
+            s("for (int t = lane; t < nel; t += 64) dwrow[tbase + t] = tw[t];")
+        s.close()
+        s.close()
+
 
 def tp_module(low: Lowered, compute_units: int = 256, kahan: bool = False):
     """``kahan`` only affects the ordered segment sum used by the unfused convolution."""
@@ -275,7 +390,8 @@ def tp_module(low: Lowered, compute_units: int = 256, kahan: bool = False):
     max_blocks_b = compute_units * 2
     descs = [
         (rt.ROLE_TP_FORWARD, "forward", blk_f, WAVES_PER_BLOCK, compute_units * 16),
-        (rt.ROLE_TP_BACKWARD, "backward", blk_b, WAVES_PER_BLOCK, max_blocks_b if low.shared_weights else compute_units * 16),
+        (rt.ROLE_TP_BACKWARD, "backward", blk_b, em.backward_waves,
+         max_blocks_b if low.shared_weights else compute_units * 16),
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0),
     ]
