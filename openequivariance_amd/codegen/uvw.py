@@ -171,6 +171,14 @@ class UvwEmitter:
             # keep a block's LDS near 40 KB, so that four blocks (and at least four waves) share a CU
             per_wave = (tile_elems + g_elems) * low.elem_size
             waves = max(1, min(WAVES_PER_BLOCK, 40960 // per_wave))
+        # shared weights: each wave sums its rows' weight gradients in an LDS copy of the weight tensor
+        # (when that fits) and writes it out once, instead of a read-modify-write of global memory per row
+        self.shared_lds = False
+        if shared:
+            fit = 65536 // (low.WN * low.elem_size)
+            if fit >= 1:
+                self.shared_lds = True
+                waves = min(WAVES_PER_BLOCK, fit)
         self.backward_waves = waves
         block = 64 * waves
         s.open(
@@ -184,8 +192,13 @@ class UvwEmitter:
             s(f"__shared__ __attribute__((aligned(16))) T s_w[{waves}][{tile_elems}];")
             s(f"__shared__ T s_g[{waves}][{g_elems}];")
         if shared:
-            s(f"T* prow = wpartial + ((i64)blockIdx.x * {WAVES_PER_BLOCK} + oeq_wave()) * {low.WN};")
-            s("bool first = true;")
+            s(f"T* prow = wpartial + ((i64)blockIdx.x * {waves} + oeq_wave()) * {low.WN};")
+            if self.shared_lds:
+                s(f"__shared__ T s_dw[{waves}][{low.WN}];")
+                s(f"for (int t = oeq_lane(); t < {low.WN}; t += 64) s_dw[oeq_wave()][t] = T(0);")
+                s("oeq_wave_sync();")
+            else:
+                s("bool first = true;")
         self._row_loop_open(s, waves)
         s(f"const T* xrow = L1_in + rowc * {low.L1};")
         s(f"const T* yrow = L2_in + rowc * {low.L2};")
@@ -217,7 +230,7 @@ class UvwEmitter:
                 s(f"dxrow[{b1.off} + u * {b1.d} + {i}] = dx[{i}];")
             s.close()
             s.close()
-        if shared:
+        if shared and not self.shared_lds:
             s("first = false;")
         # dY: butterfly over the 64 lanes
         n = self.l2_pad
@@ -246,7 +259,10 @@ class UvwEmitter:
             s(f"if (dyidx + {j} < {low.L2}) L2_grad[rowc * {low.L2} + dyidx + {j}] = rv[{j}];")
         s.close()
         s.close()
-        if shared:
+        if shared and self.shared_lds:
+            s("oeq_wave_sync();")
+            s(f"for (int t = oeq_lane(); t < {low.WN}; t += 64) prow[t] = s_dw[oeq_wave()][t];")
+        elif shared:
             # a wave that saw no row still owns a partial row: clear it
             s.open("if (first)")
             s(f"for (int t = oeq_lane(); t < {low.WN}; t += 64) prow[t] = T(0);")
@@ -294,6 +310,23 @@ class UvwEmitter:
         s.close()
         ks = self._cg_backward(s, p, prods)
         # dW[u,v,w] = sum_k f_k * g[w,k]
+        if shared and self.shared_lds:
+            # lane u visits w in the rotated order (u + t) mod W: the lanes' LDS addresses then fall into
+            # different banks although their rows are a multiple of W apart
+            s.open("if (uok && live)")
+            s(f"int w = lane % {bo.mul};")
+            s(f"T* drow = s_dw[wave] + wbase;")
+            s.open(f"for (int t = 0; t < {bo.mul}; ++t)")
+            terms = [f"f{k} * grow[{bo.off} + w * {bo.d} + {k}]" for k in ks]
+            s(f"T dwv = {terms[0]};")
+            for t in terms[1:]:
+                s(f"dwv += {t};")
+            s("drow[w] += dwv;")
+            s(f"w = (w + 1 == {bo.mul}) ? 0 : w + 1;")
+            s.close()
+            s.close()
+            s.close()
+            return
         s.open(f"if (uok{' && live' if not shared else ''})")
         s.open(f"for (int w = 0; w < {bo.mul}; ++w)")
         terms = [f"f{k} * grow[{bo.off} + w * {bo.d} + {k}]" for k in ks]
@@ -387,7 +420,7 @@ def tp_module(low: Lowered, compute_units: int = 256, kahan: bool = False):
     s(utility_kernels(kahan))
     blk_f = em.emit_forward(s)
     blk_b = em.emit_backward(s)
-    max_blocks_b = compute_units * 2
+    max_blocks_b = compute_units * (3 if em.shared_lds else 2)
     descs = [
         (rt.ROLE_TP_FORWARD, "forward", blk_f, WAVES_PER_BLOCK, compute_units * 16),
         (rt.ROLE_TP_BACKWARD, "backward", blk_b, em.backward_waves,
@@ -397,5 +430,5 @@ def tp_module(low: Lowered, compute_units: int = 256, kahan: bool = False):
     ]
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
                 shared_weights=int(low.shared_weights), deterministic=0,
-                wpartial_per_block=WAVES_PER_BLOCK if low.shared_weights else 0)
+                wpartial_per_block=em.backward_waves if low.shared_weights else 0)
     return s.text(), dims, descs
