@@ -58,6 +58,8 @@ class UvuEmitter:
         # non-temporally (batch kernels only: the convolution re-reads them).
         self.nt = 0
         self.sched_fence = False
+        self.seg_waves = 1  # conv forward: waves per node that share its output segments between them
+        self.bwd_groups: Optional[List[List[int]]] = None  # conv backward: output blocks owned by each wave
         # plain stores of [64 x d] channel blocks go through the s_tr tile as well: bit 0 = forward outputs,
         # bit 1 = backward dX (kernels that use it declare the tile)
         self.tr_stores = 0
@@ -94,7 +96,7 @@ class UvuEmitter:
         self.n_wslots = n
         # operands of an edge can be fetched ahead into registers when every index is a constant
         self.can_preload = (
-            all(low.in2[p.i2].mul <= UNROLL_V_LIMIT for p in low.paths) and low.L2 <= 32 and self.n_wslots <= 64
+            all(low.in2[p.i2].mul <= UNROLL_V_LIMIT for p in low.paths) and low.L2 <= 32 and self.n_wslots <= 128
         )
 
         self.tr_atomics = False  # set by the conv kernels that declare the s_tr tile
@@ -561,11 +563,17 @@ class UvuEmitter:
               f"({rowexpr})[{bo.off} + t] = T(0);")
             s.close()
 
-    def _lane_prologue(self, s: Src):
+    def _lane_prologue(self, s: Src, seg_waves: int = 1):
+        """``seg_waves`` > 1: the waves of a node are (chunk, sg) pairs, ``sg`` naming the output segments
+        the wave owns."""
         s("const int lane = oeq_lane();")
         s("const int wave = oeq_wave();")
         s(f"const int chunk = wave % {self.NCH};")
-        s(f"const int g = wave / {self.NCH};")
+        if seg_waves > 1:
+            s(f"const int sg = (wave / {self.NCH}) % {seg_waves};")
+            s(f"const int g = wave / {self.NCH * seg_waves};")
+        else:
+            s(f"const int g = wave / {self.NCH};")
         if self.R > 1:
             s(f"const int r = lane / {self.LPR};")
             s(f"const int ul = lane % {self.LPR};")
@@ -743,7 +751,11 @@ class UvuEmitter:
     def emit_conv_forward(self, s: Src, G: int, deterministic: bool, pipelined: bool, waves_per_eu: int = 0,
                           xcd: int = 1, tr_atomics: bool = True):
         low = self.low
-        block = 64 * self.NCH * G
+        # With several output segments the waves of a node can each own some of them (their accumulators
+        # stay in registers) and walk the node's edges side by side, instead of one wave walking the edges
+        # once per segment.
+        segw = self.seg_waves if deterministic else 1
+        block = 64 * self.NCH * G * segw
         R = self.R
         mode = self._edge_mode(pipelined)
         s.open(
@@ -752,7 +764,7 @@ class UvuEmitter:
             "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, const i64* __restrict__ eperm)"
         )
-        self._lane_prologue(s)
+        self._lane_prologue(s, segw)
         if self.can_preload:
             s("E_t A, B;")
         if mode == 2:
@@ -764,7 +776,7 @@ class UvuEmitter:
             self._emit_stage3_offsets(s)
         self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave() and not self.ir_mul
         if self.tr_atomics or (self.tr_stores & 1 and self.R == 1):
-            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.out[io].d for io in self.used_out)}];")
+            s(f"__shared__ T s_tr[{self.NCH * G * segw}][{64 * max(low.out[io].d for io in self.used_out)}];")
 
         def make_load(si):
             def load(buf, e):
@@ -803,7 +815,7 @@ class UvuEmitter:
             s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
             s(f"T* zrow = L3_out + node * {low.L3};")
             for si in range(len(self.segments)):
-                s.open("")
+                s.open(f"if (sg == {si % segw})" if segw > 1 else "")
                 s(f"A{si}_t a; zero_seg{si}(a);")
                 if kahan:
                     s(f"A{si}_t c; zero_seg{si}(c);")
@@ -818,7 +830,7 @@ class UvuEmitter:
                                 m *= 2
                 self._store_seg(s, si, "zrow", "r == 0" if self.R > 1 else "true")
                 s.close()
-            self._zero_untouched_out(s, "zrow", "r == 0")
+            self._zero_untouched_out(s, "zrow", "r == 0 && sg == 0" if segw > 1 else "r == 0")
             s.close()
         else:
             # contiguous edge range per wave group; flush with atomics whenever the receiver changes
@@ -867,12 +879,13 @@ class UvuEmitter:
             s.close()
 
     def _bwd_paths(self, s: Src, *, xname: str, yacc, wacc, g_on_demand_row: Optional[str] = None,
-                   dw_mode: str = "store", g_guard: Optional[str] = None, dw_guard: Optional[str] = None):
+                   dw_mode: str = "store", g_guard: Optional[str] = None, dw_guard: Optional[str] = None,
+                   paths: Optional[List[Path]] = None):
         """Straight-line backward of all paths. In scope: ``xname`` (X_t), dx (X_t),
         dy[], u, and either gr (G_t, resident) or a row pointer to load output
         gradients from. dw_mode 'store': dwrow[...] = v; 'acc': dwacc[slot] += v."""
         low = self.low
-        for p in sorted(low.paths, key=lambda q: (q.io, q.index)):
+        for p in sorted(low.paths if paths is None else paths, key=lambda q: (q.io, q.index)):
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
             V = b2.mul
             s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
@@ -1142,6 +1155,132 @@ class UvuEmitter:
         return block
 
     # -------------------------------------------------------- conv backward
+    def plan_backward_groups(self, max_waves: int) -> Optional[List[List[int]]]:
+        """When a node's output gradient does not fit one wave's registers, share the output blocks (and
+        with them the paths) between several waves of the node so that each keeps its share resident.
+        Returns the blocks per wave, or None when that is not possible or not needed."""
+        low = self.low
+        if self.g_resident or low.shared_weights or not self.can_preload or self.R != 1:
+            return None
+        budget = max(1, 96 // self.words)  # leaves room for the edge operands, dX and dY beside it
+        sizes = [low.out[io].d for io in self.used_out]
+        n = -(-sum(sizes) // budget)
+        while n <= max_waves:
+            target = -(-sum(sizes) // n)
+            groups, cur, tot = [], [], 0
+            for io, d in zip(self.used_out, sizes):
+                if cur and tot + d > target and len(groups) < n - 1:
+                    groups.append(cur)
+                    cur, tot = [], 0
+                cur.append(io)
+                tot += d
+            groups.append(cur)
+            if all(sum(low.out[io].d for io in grp) <= budget for grp in groups):
+                return groups
+            n += 1
+        return None
+
+    def emit_conv_backward_split(self, s: Src, waves_per_eu: int = 0, xcd: int = 1) -> int:
+        """Deterministic-walk backward for problems whose output gradient exceeds one wave's registers:
+        the waves of a block all walk the edges of one node; wave ``sg`` keeps the gradient of its output
+        blocks resident and handles the paths into them (their dW is final); the partial dX and dY of an
+        edge are summed over the waves through LDS, in a fixed order."""
+        low = self.low
+        groups = self.bwd_groups
+        SW = len(groups)
+        block = 64 * self.NCH * SW
+        xoff, XW = {}, 0
+        for b in self.used_in1:
+            xoff[b] = XW
+            XW += low.in1[b].d
+        gpaths = [[p for p in low.paths if p.io in grp] for grp in groups]
+        gin1 = [sorted({p.i1 for p in ps}) for ps in gpaths]
+        for si in range(SW):
+            self._emit_load_edge(s, f"load_edge_b{si}", gin1[si], gpaths[si])
+        s.open(
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void backward(i64 node_count, i64 nnz, '
+            "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
+            "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
+            "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
+            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm)"
+        )
+        self._lane_prologue(s, SW)
+        if SW == 1:
+            s("const int sg = 0;")
+        s(f"__shared__ T s_dy[{SW * self.NCH}][{self.l2_pad}];")
+        s(f"__shared__ T s_dx[{SW}][{self.NCH}][{XW}][64];")
+        s("E_t A;")
+        self._node_loop_open(s, 1, xcd)
+        s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+        for si in range(SW):
+            s.open(f"if (sg == {si})")
+            s("G_t gr;")
+            self._load_g(s, f"L3_grad + node * {low.L3}", groups[si])
+            # every wave of the block runs the same number of edges, so the block barriers match up
+            s.open("for (i64 e = e0; e < e1; ++e)")
+            s("const i64 eid = OEQ_EDGE(e);")
+            s(f"load_edge_b{si}(A, eid, L1_in, L2_in, W, cols, u);")
+            yacc, wacc = self._acc_preloaded("A")
+            s(f"T* dwrow = W_grad + eid * {low.WN};")
+            s("X_t dx;")
+            self._zero_x(s, "dx")
+            s(f"T dy[{self.l2_pad}];")
+            s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+            deferred = self._dw_deferred(None)
+            if deferred:
+                s(f"T dwkeep[{self.n_wslots}];")
+            self._bwd_paths(s, xname="A.x", yacc=yacc, wacc=wacc, dw_mode="store", paths=gpaths[si])
+            if deferred:
+                low_paths, low.paths = low.paths, gpaths[si]
+                try:
+                    self._flush_dwkeep(s, None)
+                finally:
+                    low.paths = low_paths
+            for b in gin1[si]:
+                for i in range(low.in1[b].d):
+                    s(f"s_dx[{si}][chunk][{xoff[b] + i}][ul] = dx.b{b}[{i}];")
+            s.open("")
+            cur, dup = self._dy_reduce(s)
+            s.open(f"if ((ul & {dup}) == 0)")
+            for j in range(cur):
+                s(f"s_dy[{si} * {self.NCH} + chunk][dyidx + {j}] = rv[{j}];")
+            s.close()
+            s.close()
+            s("__syncthreads();")
+            # the used input blocks are shared out between the waves for the final sum and store
+            s(f"T* dxrow = dx_tmp + eid * {low.L1};")
+            for n, b in enumerate(self.used_in1):
+                if n % SW != si:
+                    continue
+                blk = low.in1[b]
+                contributors = [c for c in range(SW) if b in gin1[c]]
+                self._open_if(s, self._store_cond(blk.mul))
+                base, st = self._lane_ptr(blk)
+                s(f"T* dp = {self._ptr('dxrow', base)};")
+                for i in range(blk.d):
+                    terms = " + ".join(f"s_dx[{c}][chunk][{xoff[b] + i}][ul]" for c in contributors)
+                    val = f"({terms})" if contributors else "T(0)"
+                    if self.nt & 2:
+                        s(f"__builtin_nontemporal_store({val}, dp + {i * st});")
+                    else:
+                        s(f"dp[{i * st}] = {val};")
+                s.close()
+            if si == 0:
+                self._zero_untouched_in1(s, "dxrow", "true")
+                s.open(f"if (chunk == 0)")
+                s.open(f"for (int j = lane; j < {low.L2}; j += 64)")
+                s("T tot = s_dy[0][j];")
+                s(f"for (int cc = 1; cc < {SW * self.NCH}; ++cc) tot += s_dy[cc][j];")
+                s(f"L2_grad[eid * {low.L2} + j] = tot;")
+                s.close()
+                s.close()
+            s("__syncthreads();")
+            s.close()
+            s.close()
+        s.close()
+        s.close()
+        return block
+
     def emit_conv_backward(self, s: Src, deterministic: bool, G: int, pipelined: bool, waves_per_eu: int = 0,
                            g_resident: Optional[bool] = None, xcd: int = 1, tr_atomics: bool = True):
         low = self.low
@@ -1215,6 +1354,11 @@ class UvuEmitter:
                     self._bwd_paths(s, xname=xname, yacc=yacc, wacc=wacc, dw_mode="acc" if shared else "store")
                 else:
                     s(f"const T* grow = {grow_expr_of(e)};")
+                    if deterministic:
+                        # The receiver's gradient row is the same for all its edges: without this the compiler
+                        # hoists every load of it out of the edge loop, i.e. makes the whole row register
+                        # resident, which is exactly what did not fit.
+                        s(f'asm volatile("" : "+{"s" if self.R == 1 else "v"}"(grow));')
                     self._bwd_paths(s, xname=xname, yacc=yacc, wacc=wacc, g_on_demand_row="grow",
                                     dw_mode="acc" if shared else "store")
                 if deferred:
@@ -1323,7 +1467,8 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
     t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
                     conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
-                    conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0))
+                    conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
+                    conv_segw=4, conv_split=1))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -1333,8 +1478,37 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         mode = rt.CONV_GROUPED if t["conv_sort"] else rt.CONV_ATOMIC
     walk = mode != rt.CONV_ATOMIC  # kernels walk per-node edge segments
     em = UvuEmitter(low, acc_budget_words=t["conv_acc"], kahan=kahan)
+    if em.stage is None and em.can_preload and "conv_acc" not in os.environ.get("OEQ_AMD_TUNE", ""):
+        # Forward without LDS staging keeps two operand sets of an edge (X blocks, the weights of the
+        # output segment's paths, Y) beside the accumulators: shrink the segments until that fits, and
+        # give up the prefetch when even 48-word segments do not.
+        words = 1 if low.elem_size == 4 else 2
+
+        def plan(budget, sets):
+            e = UvuEmitter(low, acc_budget_words=budget, kahan=kahan)
+            need = max(sets * words * (sum(low.in1[b].d for b in e.seg_in1[si]) + low.L2 +
+                                       sum(low.in2[p.i2].mul for p in low.paths if p.io in seg))
+                       + words * sum(low.out[io].d for io in seg) for si, seg in enumerate(e.segments))
+            return e, need
+
+        budgets = (t["conv_acc"], 96, 64, 48)
+        for budget in budgets:
+            em, need = plan(budget, 2)
+            if need <= 170:
+                break
+        else:
+            t["conv_pipe_f"] = 0
+            for budget in budgets:
+                em, need = plan(budget, 1)
+                if need <= 190:
+                    break
     em.nt = t["conv_nt"]
+    if walk and len(em.segments) > 1 and t["conv_segw"] and em.stage is None and em.R == 1:
+        em.seg_waves = max(1, min(len(em.segments), t["conv_segw"], 8 // em.NCH))
+        t["conv_gf"] = max(1, min(t["conv_gf"], 8 // (em.NCH * em.seg_waves)))
     em.tr_stores = t["conv_trs"]
+    # output gradients that do not fit the register budget are loaded per path: fence the paths then
+    em.sched_fence = (not em.g_resident) if t["conv_sb"] < 0 else bool(t["conv_sb"])
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels(kahan))
@@ -1347,7 +1521,13 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     xcd = max(1, t["conv_xcd"])
     blk_f = em.emit_conv_forward(s, G_f, walk, t["conv_pipe_f"], t["conv_wf"], xcd, bool(t["conv_tra"]))
     gres = None if t["conv_gres"] < 0 else bool(t["conv_gres"])
-    blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd, bool(t["conv_tra"]))
+    em.bwd_groups = em.plan_backward_groups(8 // em.NCH) if (walk and t["conv_split"] and gres is None) else None
+    if em.bwd_groups:
+        G_b = 1
+        blk_b = em.emit_conv_backward_split(s, t["conv_wb"], xcd)
+    else:
+        blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd,
+                                      bool(t["conv_tra"]))
     descs = [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, compute_units * 16),

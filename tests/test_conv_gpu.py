@@ -55,6 +55,12 @@ CASES = [
     ("uvw", lambda: _fc(False), 40, 6),
     ("uvw-shared", lambda: _fc(True), 40, 6),
     ("uvw-cfg4-mfma", P.config4_uvw_shared, 30, 5),
+    # output gradient too large for one wave: forward shares the output segments, backward the output
+    # blocks, between several waves of a node (64 channels: one chunk; 128: two)
+    ("nequip-benzene", lambda: P.nequip_problems()[3], 30, 5),
+    ("benzene-128", lambda: P.ChannelwiseTPP(
+        "128x0o + 128x0e + 128x1o + 128x1e + 128x2o + 128x2e + 128x3o + 128x3e", "0e + 1o + 2e + 3o",
+        "128x0o + 128x0e + 128x1o + 128x1e + 128x2o + 128x2e + 128x3o + 128x3e", "benzene-128"), 24, 4),
 ]
 
 
