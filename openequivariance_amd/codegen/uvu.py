@@ -8,13 +8,23 @@ loop_unroll_conv_det.cuh:96-293) with a different decomposition:
 
 * lane <-> channel ``u``; the CG contraction of one channel is straight-line
   code with the sparse coefficients folded into constants; the operand shared
-  by all channels (the row's Y) is wave-uniform when a row fills a wave;
-* the convolution keeps the receiver's output (forward) or output gradient
-  (backward) in registers across all edges of that receiver (CSR walk), so Z and
-  dZ move once per node instead of once per edge, and the operands of the next
-  edge are fetched into a second register set while the current edge is computed;
+  by all channels (the row's Y) is wave-uniform when a row fills a wave, and so
+  is the row's base pointer: accesses are "uniform base + 32-bit lane offset";
+* a row's arithmetic is one basic block: lanes without a channel load through a
+  clamped index and drop the value, stores are unconditional where every lane
+  has a channel, and weight gradients that need a condition wait in registers
+  until the last path (a branch inside the chain of paths makes the compiler
+  postpone the dX/dY accumulations and keep every path's operands alive);
+* the convolution walks each receiver's edges (CSR order given by the caller,
+  or an edge index grouped by receiver on the device) and keeps the receiver's
+  output (forward) or output gradient (backward) in registers across them, so Z
+  and dZ move once per node instead of once per edge; the next edge's operands
+  arrive in an LDS staging buffer by direct global->LDS loads meanwhile;
+  problems too large for one wave's registers are shared between the waves of
+  the node's block by output segment / output block;
 * dY is accumulated per lane over all paths and reduced once per row with a
-  halving butterfly; nothing in deterministic mode uses atomics.
+  halving butterfly; no kernel of the walk uses atomics on node data (dX goes
+  through per-edge terms and a sender-ordered reduction).
 """
 
 from __future__ import annotations
