@@ -77,8 +77,9 @@ typedef enum {
     OEQ_ROLE_SEGMENT_SUM = 8,       /* ordered sum of rows over the segments of a sorted key list */
     OEQ_ROLE_GROUP_COUNT = 9,       /* grouping an unsorted key list: histogram, */
     OEQ_ROLE_GROUP_SCAN = 10,       /*   exclusive scan (one block), */
-    OEQ_ROLE_GROUP_SCATTER = 11,    /*   and scatter of the item indices into their key's segment */
-    OEQ_ROLE_COUNT = 12
+    OEQ_ROLE_GROUP_SCATTER = 11,    /*   scatter of the item indices into their key's segment, */
+    OEQ_ROLE_GROUP_ORDER = 12,      /*   and ascending order of the indices within each segment */
+    OEQ_ROLE_COUNT = 13
 } oeq_role;
 
 /* How the convolution kernels of a set find the edges of a node (oeq_problem_dims.deterministic):
@@ -88,8 +89,9 @@ typedef enum {
     OEQ_CONV_SORTED = 1,   /* caller passes receiver-sorted edges (+ sender-major permutation for backward); CSR walk,
                               fixed summation order, no atomics on node data */
     OEQ_CONV_GROUPED = 2   /* any edge order; the library groups the edge indices by receiver (and by sender for
-                              backward) on the device, then runs the same CSR walk through that index; the order
-                              within a group, hence the rounding of the sums, may differ from run to run */
+                              backward) on the device, ascending within a group, then runs the same CSR walk
+                              through that index: fixed summation order for a given edge list, no atomics on node
+                              data */
 } oeq_conv_mode;
 
 /* Several descriptors may name the same role: those kernels are launched back to back, in

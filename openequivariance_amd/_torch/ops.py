@@ -199,8 +199,10 @@ def _conv_checks(e: KernelEntry, L1_in, L2_in, W, rows, cols, perm, L3_grad=None
     check_tensor(cols, [nnz], torch.int64, "cols")
     if e.deterministic:
         check_tensor(perm, [nnz], torch.int64, "transpose perm")
-    elif torch.are_deterministic_algorithms_enabled():
-        # counterpart of at::globalContext().alertNotDeterministic (torch_core.hpp:448)
+    elif (torch.are_deterministic_algorithms_enabled() and not e.unfused
+          and e.kernels().dims["deterministic"] == rt.CONV_ATOMIC):
+        # counterpart of at::globalContext().alertNotDeterministic (torch_core.hpp:448); only the
+        # float-atomics kernels need it: the default grouped walk sums in a fixed order
         msg = ("OpenEquivariance_conv_atomic does not have a deterministic implementation, but you set "
                "'torch.use_deterministic_algorithms(True)'. Use TensorProductConv(..., deterministic=True).")
         if torch.is_deterministic_algorithms_warn_only_enabled():

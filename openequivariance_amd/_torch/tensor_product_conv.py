@@ -47,10 +47,10 @@ class TensorProductConv(torch.nn.Module):
 
     :param problem: specification of the tensor product.
     :param deterministic: ``False``: any edge order; the edge indices are grouped by receiver (and by
-           sender for backward) on the device at every call and the sums follow that grouping, whose
-           order within a node is not fixed, so results may differ in the last bits from run to run.
-           ``True``: receiver-sorted edges and ``sender_perm`` from the caller, fixed summation order
-           (bit-identical from run to run). *Default*: ``False``.
+           sender for backward) on the device at every call, ascending within a node, and the sums follow
+           that grouping (so this mode, too, gives the same bits from run to run for a given edge list).
+           ``True``: receiver-sorted edges and ``sender_perm`` from the caller, no grouping pass.
+           *Default*: ``False``.
     :param kahan: with ``deterministic=True``: Kahan-compensated summation over the edges of a node
            (receiver's output in forward, sender's gradient in backward). *Default*: ``False``.
     :param use_opaque: deprecated, ignored.

@@ -1554,6 +1554,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                 (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, compute_units * 16),
                 (rt.ROLE_GROUP_SCAN, "oeq_group_scan", 1024, 1, 1),
                 (rt.ROLE_GROUP_SCATTER, "oeq_group_scatter", 256, 256 * 4, compute_units * 16),
+                (rt.ROLE_GROUP_ORDER, "oeq_group_order", 256, 4, compute_units * 32),
             ]
     else:
         # edge ranges: about conv_epw consecutive edges per wave group

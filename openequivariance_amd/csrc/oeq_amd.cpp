@@ -156,9 +156,10 @@ struct oeq_kernels {
     }
 
     // Counting sort of the item indices 0..n_items-1 by key: ptr[0..n_segments] = segment starts,
-    // perm = item indices grouped by key (unordered within a group); cursor is scratch of n_segments+1.
+    // perm = item indices grouped by key, ascending within a group (so the result depends on the key
+    // list only); cursor (n_segments+1) and unordered (n_items) are scratch.
     int group_by_key(int64_t n_items, int64_t n_segments, const int64_t* keys, int64_t* ptr, int64_t* cursor,
-                     int64_t* perm, void* stream) {
+                     int64_t* unordered, int64_t* perm, void* stream) {
         int rc = fill_zero(ptr, (size_t)(n_segments + 1) * sizeof(int64_t), stream);
         if (rc) return rc;
         void* cargs[] = {&n_items, &keys, &ptr};
@@ -168,8 +169,11 @@ struct oeq_kernels {
         void* sargs[] = {&n, &ptr, &cursor};
         rc = launch(OEQ_ROLE_GROUP_SCAN, 1, sargs, stream);
         if (rc) return rc;
-        void* pargs[] = {&n_items, &keys, &cursor, &perm};
-        return launch(OEQ_ROLE_GROUP_SCATTER, n_items, pargs, stream);
+        void* pargs[] = {&n_items, &keys, &cursor, &unordered};
+        rc = launch(OEQ_ROLE_GROUP_SCATTER, n_items, pargs, stream);
+        if (rc) return rc;
+        void* oargs[] = {&n_segments, &ptr, &unordered, &perm};
+        return launch(OEQ_ROLE_GROUP_ORDER, n_segments, oargs, stream);
     }
 };
 
@@ -389,21 +393,22 @@ int oeq_tp_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in, void* 
 // ---------------------------------------------------------------------------
 
 // Workspace layouts. SORTED: forward [rowptr]; backward [rowptr | colptr | dx_tmp].
-// GROUPED: forward [rowptr | cursor | rperm]; backward [rowptr | colptr | cursor | rperm | sperm | dx_tmp].
+// GROUPED: forward [rowptr | cursor | rperm | scratch perm];
+//          backward [rowptr | colptr | cursor | rperm | sperm | scratch perm | dx_tmp].
 static size_t ptr_bytes_of(int64_t node_count) { return align_up((size_t)(node_count + 1) * sizeof(int64_t), 256); }
 static size_t perm_bytes_of(int64_t nnz) { return align_up((size_t)nnz * sizeof(int64_t), 256); }
 
 size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
     if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
     if (k->dims.deterministic == OEQ_CONV_SORTED) return ptr_bytes_of(node_count);
-    return 2 * ptr_bytes_of(node_count) + perm_bytes_of(nnz);
+    return 2 * ptr_bytes_of(node_count) + 2 * perm_bytes_of(nnz);
 }
 
 size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
     if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
     size_t tmp_bytes = align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256);
     if (k->dims.deterministic == OEQ_CONV_SORTED) return 2 * ptr_bytes_of(node_count) + tmp_bytes;
-    return 3 * ptr_bytes_of(node_count) + 2 * perm_bytes_of(nnz) + tmp_bytes;
+    return 3 * ptr_bytes_of(node_count) + 3 * perm_bytes_of(nnz) + tmp_bytes;
 }
 
 int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
@@ -431,7 +436,8 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void
             const size_t pb = ptr_bytes_of(node_count);
             int64_t* cursor = (int64_t*)((char*)workspace + pb);
             rperm = (int64_t*)((char*)workspace + 2 * pb);
-            rc = k->group_by_key(nnz, node_count, rows, rowptr, cursor, rperm, stream);
+            int64_t* scratch = (int64_t*)((char*)workspace + 2 * pb + perm_bytes_of(nnz));
+            rc = k->group_by_key(nnz, node_count, rows, rowptr, cursor, scratch, rperm, stream);
         }
         if (rc) return rc;
     } else {
@@ -487,10 +493,11 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
             int64_t* cursor = (int64_t*)((char*)workspace + 2 * pb);
             rperm = (int64_t*)((char*)workspace + 3 * pb);
             int64_t* sp = (int64_t*)((char*)workspace + 3 * pb + qb);
-            dx_tmp = (char*)workspace + 3 * pb + 2 * qb;
-            rc = k->group_by_key(nnz, node_count, rows, rowptr, cursor, rperm, stream);
+            int64_t* scratch = (int64_t*)((char*)workspace + 3 * pb + 2 * qb);
+            dx_tmp = (char*)workspace + 3 * pb + 3 * qb;
+            rc = k->group_by_key(nnz, node_count, rows, rowptr, cursor, scratch, rperm, stream);
             if (rc) return rc;
-            rc = k->group_by_key(nnz, node_count, cols, colptr, cursor, sp, stream);
+            rc = k->group_by_key(nnz, node_count, cols, colptr, cursor, scratch, sp, stream);
             if (rc) return rc;
             sperm = sp;
         }

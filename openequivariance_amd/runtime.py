@@ -46,6 +46,7 @@ ROLE_SEGMENT_SUM = 8
 ROLE_GROUP_COUNT = 9
 ROLE_GROUP_SCAN = 10
 ROLE_GROUP_SCATTER = 11
+ROLE_GROUP_ORDER = 12
 
 CONV_ATOMIC, CONV_SORTED, CONV_GROUPED = 0, 1, 2
 

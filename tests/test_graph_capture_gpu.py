@@ -88,25 +88,4 @@ def test_convolution_in_a_graph(deterministic):
         gen2 = torch.Generator(device="cuda").manual_seed(200 + seed)
         return [torch.randn(t.shape, device="cuda", generator=gen2) for t in (X, Y, W, G)]
 
-    if deterministic:
-        _replay_and_compare(step, [X, Y, W, G], new_values)
-    else:
-        # the grouping order inside a node is not fixed from run to run: compare within tolerance
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            step()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            captured = step()
-        for seed in range(4):
-            for t, v in zip([X, Y, W, G], new_values(seed)):
-                t.copy_(v)
-            expected = [o.clone() for o in step()]
-            graph.replay()
-            torch.cuda.synchronize()
-            for got, want in zip(captured, expected):
-                scale = float(want.abs().max())
-                assert float((got - want).abs().max()) <= 1e-5 * scale, seed
+    _replay_and_compare(step, [X, Y, W, G], new_values)

@@ -86,7 +86,7 @@ def test_generated_conv_sources_compile_for_gfx950(make, det):
     blob = rt.compile_source(src)
     names = {d[1] for d in descs}
     assert {"forward", "backward", "fixup_backward"} <= names
-    assert ({"oeq_group_count", "oeq_group_scan", "oeq_group_scatter"} <= names) == (not det)
+    assert ({"oeq_group_count", "oeq_group_scan", "oeq_group_scatter", "oeq_group_order"} <= names) == (not det)
     assert dims["deterministic"] == (rt.CONV_SORTED if det else rt.CONV_GROUPED)
     # generated code must not carry packed-FP32 arithmetic or anything CUDA-flavoured
     assert "__syncwarp" not in src and "cuda" not in src.lower()
