@@ -185,6 +185,14 @@ int oeq_segment_sum(oeq_kernels* k, int64_t n_segments, int64_t n_items, int64_t
                     void* workspace, size_t workspace_bytes, void* stream);
 size_t oeq_segment_sum_workspace_bytes(const oeq_kernels* k, int64_t n_segments);
 
+/* Same sum for keys in ANY order: the item indices are first grouped by key on the device (ascending
+ * within a key, so the summation order depends on the key list only), then summed as above. Replaces the
+ * same scatter_add_wrapper call where the reference relies on float atomics. */
+int oeq_grouped_sum(oeq_kernels* k, int64_t n_segments, int64_t n_items, int64_t row_len,
+                    const void* src, void* dst, const int64_t* keys,
+                    void* workspace, size_t workspace_bytes, void* stream);
+size_t oeq_grouped_sum_workspace_bytes(const oeq_kernels* k, int64_t n_segments, int64_t n_items);
+
 /* ---- per-kernel timing --------------------------------------------------- */
 /* Replaces GPUTimer (extension/backend/backend_hip.hpp:67-101). While enabled,
  * every kernel this set launches is bracketed by HIP events on the stream it is

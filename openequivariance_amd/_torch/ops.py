@@ -224,11 +224,17 @@ def _segment_sum(ks, src: torch.Tensor, n_segments: int, keys: torch.Tensor, per
 
 
 def _scatter_rows(e: KernelEntry, ks, src, n_segments, keys, perm):
-    """Sum edge rows into node rows: fixed order when deterministic, torch's atomic index_add_ otherwise
-    (the reference's unfused path, core/ConvolutionBase.py:292-301, is the latter)."""
+    """Sum edge rows into node rows in a fixed order: along the caller's sorted list when deterministic,
+    else after grouping the edge indices by key on the device (the reference's unfused path,
+    core/ConvolutionBase.py:292-301, uses a float-atomics scatter_add)."""
     if e.deterministic:
         return _segment_sum(ks, src, n_segments, keys, perm)
-    return src.new_zeros((n_segments, src.shape[1])).index_add_(0, keys, src)
+    dst = src.new_empty((n_segments, src.shape[1]))
+    nb = ks.grouped_sum_workspace_bytes(n_segments, src.shape[0])
+    ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=src.device)
+    ks.grouped_sum(n_segments, src.shape[0], src.shape[1], src.data_ptr(), dst.data_ptr(), keys.data_ptr(),
+                   ws.data_ptr(), nb, _stream())
+    return dst
 
 
 def _unfused_forward(e, ks, x, y, w, r, c, nodes, nnz):

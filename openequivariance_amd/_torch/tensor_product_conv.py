@@ -37,7 +37,11 @@ def build_conv_module(problem: TPProblem, deterministic: bool, kahan: bool = Fal
     cu = compute_units()
     src, dims, descs = uvw.tp_module(low, cu, kahan)
     descs = list(descs) + [(rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, cu * 16),
-                           (rt.ROLE_SEGMENT_SUM, "oeq_segment_sum", 256, 1, cu * 32)]
+                           (rt.ROLE_SEGMENT_SUM, "oeq_segment_sum", 256, 1, cu * 32),
+                           (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, cu * 16),
+                           (rt.ROLE_GROUP_SCAN, "oeq_group_scan", 1024, 1, 1),
+                           (rt.ROLE_GROUP_SCATTER, "oeq_group_scatter", 256, 256 * 4, cu * 16),
+                           (rt.ROLE_GROUP_ORDER, "oeq_group_order", 256, 4, cu * 32)]
     return src, dims, descs
 
 

@@ -310,6 +310,37 @@ int oeq_segment_sum(oeq_kernels* k, int64_t n_segments, int64_t n_items, int64_t
     return k->launch(OEQ_ROLE_SEGMENT_SUM, n_segments, args, stream);
 }
 
+size_t oeq_grouped_sum_workspace_bytes(const oeq_kernels* k, int64_t n_segments, int64_t n_items) {
+    (void)k;
+    // [ptr | cursor | perm | scratch perm]
+    return 2 * align_up((size_t)(n_segments + 1) * sizeof(int64_t), 256) +
+           2 * align_up((size_t)n_items * sizeof(int64_t), 256);
+}
+
+int oeq_grouped_sum(oeq_kernels* k, int64_t n_segments, int64_t n_items, int64_t row_len, const void* src, void* dst,
+                    const int64_t* keys, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_grouped_sum: NULL kernel set");
+    if (n_segments < 0 || n_items < 0 || row_len <= 0) return fail(OEQ_ERR_INVALID, "oeq_grouped_sum: bad size");
+    if (n_segments == 0) return OEQ_OK;
+    if (!dst) return fail(OEQ_ERR_INVALID, "oeq_grouped_sum: NULL dst");
+    if (n_items == 0) return k->fill_zero(dst, (size_t)n_segments * row_len * k->dims.elem_size, stream);
+    if (!src || !keys) return fail(OEQ_ERR_INVALID, "oeq_grouped_sum: NULL buffer");
+    size_t need = oeq_grouped_sum_workspace_bytes(k, n_segments, n_items);
+    if (!workspace || workspace_bytes < need)
+        return fail(OEQ_ERR_INVALID, "oeq_grouped_sum: workspace too small (%zu < %zu bytes)", workspace_bytes, need);
+    const size_t pb = align_up((size_t)(n_segments + 1) * sizeof(int64_t), 256);
+    const size_t qb = align_up((size_t)n_items * sizeof(int64_t), 256);
+    int64_t* ptr = (int64_t*)workspace;
+    int64_t* cursor = (int64_t*)((char*)workspace + pb);
+    int64_t* perm = (int64_t*)((char*)workspace + 2 * pb);
+    int64_t* scratch = (int64_t*)((char*)workspace + 2 * pb + qb);
+    int rc = k->group_by_key(n_items, n_segments, keys, ptr, cursor, scratch, perm, stream);
+    if (rc) return rc;
+    const int64_t* cperm = perm;
+    void* args[] = {&n_segments, &n_items, &row_len, &src, &dst, &cperm, &ptr};
+    return k->launch(OEQ_ROLE_SEGMENT_SUM, n_segments, args, stream);
+}
+
 int oeq_kernel_timing_enable(oeq_kernels* k, int enable) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_kernel_timing_enable: NULL kernel set");
     std::lock_guard<std::mutex> lock(k->mu);

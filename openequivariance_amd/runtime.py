@@ -131,6 +131,8 @@ EXPORTS = {
     "oeq_conv_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_segment_sum": (ctypes.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_segment_sum_workspace_bytes": (_SZ, [_P, _I64]),
+    "oeq_grouped_sum": (ctypes.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _P, _SZ, _P]),
+    "oeq_grouped_sum_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_kernel_timing_enable": (ctypes.c_int, [_P, ctypes.c_int]),
     "oeq_kernel_timing_collect": (ctypes.c_int, [_P, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
                                                  ctypes.POINTER(_I64)]),
@@ -272,6 +274,13 @@ class KernelSet:
     def segment_sum(self, n_segments, n_items, row_len, src, dst, keys, perm, ws, ws_bytes, stream):
         _check(self._lib.oeq_segment_sum(self.handle, n_segments, n_items, row_len, src, dst, keys, perm, ws,
                                          ws_bytes, stream), "oeq_segment_sum")
+
+    def grouped_sum_workspace_bytes(self, n_segments, n_items) -> int:
+        return self._lib.oeq_grouped_sum_workspace_bytes(self.handle, n_segments, n_items)
+
+    def grouped_sum(self, n_segments, n_items, row_len, src, dst, keys, ws, ws_bytes, stream):
+        _check(self._lib.oeq_grouped_sum(self.handle, n_segments, n_items, row_len, src, dst, keys, ws, ws_bytes,
+                                         stream), "oeq_grouped_sum")
 
     def conv_forward_workspace_bytes(self, nodes, nnz) -> int:
         return self._lib.oeq_conv_forward_workspace_bytes(self.handle, nodes, nnz)
