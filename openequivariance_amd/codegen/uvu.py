@@ -1212,7 +1212,8 @@ class UvuEmitter:
             "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
             "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
             "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm)"
+            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
+            "T* __restrict__ wpartial)"
         )
         self._lane_prologue(s, SW)
         if SW == 1:
@@ -1306,7 +1307,8 @@ class UvuEmitter:
             "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
             "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
             "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm)"
+            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
+            "T* __restrict__ wpartial)"
         )
         self._lane_prologue(s)
         if self.NCH > 1:
@@ -1401,14 +1403,31 @@ class UvuEmitter:
             s("const i64 ee = (eb + per < nnz) ? eb + per : nnz;")
             self._edge_loop(s, "eb + r", "ee", load, make_compute(lambda e: f"L3_grad + rows[{e}] * {low.L3}"),
                             mode)
-        if shared:
-            # shared weights: one atomic add per weight per wave (atomic mode only)
+        if shared and deterministic:
+            # shared weights, walk kernels: every wave group writes the sum over its nodes as one partial
+            # row (lane groups of packed rows folded first); the rows are added up in order afterwards
+            if self.R > 1:
+                s.open(f"for (int t = 0; t < {self.n_wslots}; ++t)")
+                m = self.LPR
+                while m < 64:
+                    s(f"dwacc[t] += __shfl_xor(dwacc[t], {m});")
+                    m *= 2
+                s.close()
+            s(f"T* prow = wpartial + ((i64)blockIdx.x * {G} + g) * {low.WN};")
+            for p, slot in self._dw_slots():
+                b1, V = low.in1[p.i1], low.in2[p.i2].mul
+                s.open(f"if (r == 0 && u < {b1.mul})")
+                s(f"for (int v = 0; v < {V}; ++v) prow[{p.woff} + u * {V} + v] = dwacc[{slot} + v];")
+                s.close()
+        elif shared:
+            # float-atomics kernels: one atomic add per weight per wave
             for p, slot in self._dw_slots():
                 b1, V = low.in1[p.i1], low.in2[p.i2].mul
                 s.open(f"if (u < {b1.mul})")
                 s(f"for (int v = 0; v < {V}; ++v) oeq_atomic_add(W_grad + {p.woff} + u * {V} + v, dwacc[{slot} + v]);")
                 s.close()
         s.close()
+        self.backward_groups_per_block = G
         return block
 
 
@@ -1529,6 +1548,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     G_f = t["conv_gf"]
     G_b = 1 if em.NCH > 1 else t["conv_gb"]
     xcd = max(1, t["conv_xcd"])
+    xcd_b = 1 if (walk and low.shared_weights) else xcd  # bounded grid: one partial dW row per wave group
     blk_f = em.emit_conv_forward(s, G_f, walk, t["conv_pipe_f"], t["conv_wf"], xcd, bool(t["conv_tra"]))
     gres = None if t["conv_gres"] < 0 else bool(t["conv_gres"])
     em.bwd_groups = em.plan_backward_groups(8 // em.NCH) if (walk and t["conv_split"] and gres is None) else None
@@ -1536,8 +1556,9 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         G_b = 1
         blk_b = em.emit_conv_backward_split(s, t["conv_wb"], xcd)
     else:
-        blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd,
+        blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd_b,
                                       bool(t["conv_tra"]))
+        G_b = em.backward_groups_per_block
     descs = [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, compute_units * 16),
@@ -1546,9 +1567,11 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         s(fixup_backward_kernel(low.L1, kahan, bool(em.nt & 4)))
         descs += [
             (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f, 0, xcd),
-            (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b, 0, xcd),
+            (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b, compute_units * 8 if low.shared_weights else 0, xcd_b),
             (rt.ROLE_CONV_FIXUP_BACKWARD, "fixup_backward", 256, 1, 0),
         ]
+        if low.shared_weights:
+            descs.append((rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0))
         if mode == rt.CONV_GROUPED:
             descs += [
                 (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, compute_units * 16),
@@ -1564,5 +1587,6 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b * em.R * epw, compute_units * 32),
         ]
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
-                shared_weights=int(low.shared_weights), deterministic=mode, wpartial_per_block=0)
+                shared_weights=int(low.shared_weights), deterministic=mode,
+                wpartial_per_block=G_b if (walk and low.shared_weights) else 0)
     return s.text(), dims, descs

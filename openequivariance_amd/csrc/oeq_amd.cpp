@@ -435,9 +435,17 @@ size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count
     return 2 * ptr_bytes_of(node_count) + 2 * perm_bytes_of(nnz);
 }
 
+// Shared weights, walk kernels: one partial weight-gradient row per wave group of the backward grid.
+static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t node_count) {
+    if (!k->dims.shared_weights || !k->dims.wpartial_per_block) return 0;
+    size_t rows = (size_t)k->grid_for(OEQ_ROLE_CONV_BACKWARD, node_count) * (size_t)k->dims.wpartial_per_block;
+    return align_up(rows * (size_t)k->dims.weight_numel * (size_t)k->dims.elem_size, 256);
+}
+
 size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
     if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
-    size_t tmp_bytes = align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256);
+    size_t tmp_bytes = align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256) +
+                       conv_wpartial_bytes(k, node_count);
     if (k->dims.deterministic == OEQ_CONV_SORTED) return 2 * ptr_bytes_of(node_count) + tmp_bytes;
     return 3 * ptr_bytes_of(node_count) + 3 * perm_bytes_of(nnz) + tmp_bytes;
 }
@@ -487,8 +495,11 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
     if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: negative size");
     const bool shared = k->dims.shared_weights != 0;
     const size_t es = (size_t)k->dims.elem_size;
+    // shared weights: the float-atomics kernels add into a cleared W_grad; the walk kernels write partial
+    // rows that are summed in order at the end (W_grad is cleared only when there is nothing to sum)
+    const bool wrows = shared && k->dims.deterministic != OEQ_CONV_ATOMIC && k->dims.wpartial_per_block > 0;
     int rc;
-    if (shared) {
+    if (shared && (!wrows || node_count == 0 || nnz == 0)) {
         if (!W_grad) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL W_grad");
         rc = k->fill_zero(W_grad, (size_t)k->dims.weight_numel * es, stream);
         if (rc) return rc;
@@ -502,7 +513,7 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
 
     int64_t *rowptr = nullptr, *colptr = nullptr, *rperm = nullptr;
     const int64_t* sperm = transpose_perm;
-    void* dx_tmp = nullptr;
+    void *dx_tmp = nullptr, *wpartial = nullptr;
     const int mode = k->dims.deterministic;
     if (mode != OEQ_CONV_ATOMIC) {
         if (mode == OEQ_CONV_SORTED && !transpose_perm)
@@ -532,16 +543,23 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
             if (rc) return rc;
             sperm = sp;
         }
+        if (wrows)
+            wpartial = (char*)dx_tmp + align_up((size_t)nnz * (size_t)k->dims.L1_dim * es, 256);
     } else {
         rc = k->fill_zero(L1_grad, dx_bytes, stream);
         if (rc) return rc;
     }
     void* args[] = {&node_count, &nnz,  &L1_in, &L1_grad, &L2_in,  &L2_grad, &W,
-                    &W_grad,     &L3_grad, &rows, &cols,    &rowptr, &dx_tmp, &rperm};
+                    &W_grad,     &L3_grad, &rows, &cols,    &rowptr, &dx_tmp, &rperm, &wpartial};
     rc = k->launch(OEQ_ROLE_CONV_BACKWARD, mode != OEQ_CONV_ATOMIC ? node_count : nnz, args, stream);
     if (rc || mode == OEQ_CONV_ATOMIC) return rc;
     void* fargs[] = {&node_count, &nnz, &dx_tmp, &L1_grad, &sperm, &colptr};
-    return k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
+    rc = k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
+    if (rc || !wrows) return rc;
+    int64_t n_partials = (int64_t)k->grid_for(OEQ_ROLE_CONV_BACKWARD, node_count) * k->dims.wpartial_per_block;
+    int64_t wn = k->dims.weight_numel;
+    void* rargs[] = {&n_partials, &wpartial, &W_grad, &wn};
+    return k->launch(OEQ_ROLE_TP_BACKWARD_WREDUCE, wn, rargs, stream);
 }
 
 }  // extern "C"
