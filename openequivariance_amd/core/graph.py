@@ -23,6 +23,17 @@ class CoordGraph:
         self.cols = cols[order]
         self.transpose_perm = np.lexsort((self.rows, self.cols)).astype(self.rows.dtype)
 
+    def save_npz(self, path) -> None:
+        """Write ``coords``, ``row``, ``col`` (the keys of the reference's graph files,
+        openequivariance/openequivariance/benchmark/ConvBenchmarkSuite.py:21-32) as an ``.npz`` archive."""
+        np.savez(path, coords=self.coords, row=self.rows, col=self.cols)
+
+    @classmethod
+    def from_npz(cls, path, name: str = "") -> "CoordGraph":
+        """Read a graph written by :meth:`save_npz` (plain arrays only: nothing is unpickled)."""
+        with np.load(path, allow_pickle=False) as z:
+            return cls(z["coords"], z["row"].astype(np.int64), z["col"].astype(np.int64), name)
+
 
 def periodic_radius_graph(n_nodes: int, mean_degree: float = 32.0, cutoff: float = 5.0, seed: int = 0):
     """Uniform points in a periodic cube sized so that the expected number of

@@ -98,3 +98,16 @@ def test_ops_reject_cpu_tensors():
     tp = oeq.TensorProduct(P.config1_single_uvu())
     with pytest.raises((RuntimeError, NotImplementedError)):
         tp(torch.zeros(2, 5), torch.zeros(2, 7), torch.zeros(2, 1))
+
+
+def test_graph_npz_round_trip(tmp_path):
+    from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
+    coords, rows, cols, _ = periodic_radius_graph(50, 6, 5.0, 1)
+    g = CoordGraph(coords, rows, cols, "toy")
+    g.save_npz(tmp_path / "g.npz")
+    h = CoordGraph.from_npz(tmp_path / "g.npz", "toy")
+    assert h.node_count == g.node_count and h.nnz == g.nnz
+    assert np.array_equal(h.rows, g.rows) and np.array_equal(h.cols, g.cols)
+    assert np.array_equal(h.transpose_perm, g.transpose_perm)
+    # rows are receiver-sorted and the permutation lists the edges sender-major
+    assert np.all(np.diff(h.rows) >= 0) and np.all(np.diff(h.cols[h.transpose_perm]) >= 0)
