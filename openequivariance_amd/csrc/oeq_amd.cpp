@@ -282,6 +282,10 @@ int oeq_kernels_create(const void* code, size_t code_size, const oeq_problem_dim
 
 void oeq_kernels_destroy(oeq_kernels* k) {
     if (!k) return;
+    for (auto& t : k->timed) {  // timings nobody collected
+        (void)hipEventDestroy(t.start);
+        (void)hipEventDestroy(t.stop);
+    }
     for (auto& s : k->slots)
         if (s.module) (void)hipModuleUnload(s.module);
     delete k;
