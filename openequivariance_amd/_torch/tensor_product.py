@@ -15,6 +15,7 @@ import torch
 from ..codegen.lower import lower
 from ..core.spec import TPProblem
 from . import ops
+from .benchmarking import TensorProductTiming
 from .utils import oeq_to_torch_dtype, torch_to_oeq_dtype, compute_units
 
 
@@ -27,7 +28,7 @@ def build_tp_module(problem: TPProblem):
     return uvw.tp_module(low, compute_units())
 
 
-class TensorProduct(torch.nn.Module):
+class TensorProduct(TensorProductTiming, torch.nn.Module):
     r"""Drop-in replacement for ``o3.TensorProduct`` from e3nn with per-problem
     HIP kernels. Supports 'uvu' and 'uvw' instructions with weights.
 

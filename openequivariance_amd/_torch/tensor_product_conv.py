@@ -21,6 +21,7 @@ import torch
 from ..codegen.lower import lower
 from ..core.spec import TPProblem
 from . import ops
+from .benchmarking import ConvolutionTiming
 from .utils import compute_units, oeq_to_torch_dtype, torch_to_oeq_dtype
 
 
@@ -45,7 +46,7 @@ def build_conv_module(problem: TPProblem, deterministic: bool, kahan: bool = Fal
     return src, dims, descs
 
 
-class TensorProductConv(torch.nn.Module):
+class TensorProductConv(ConvolutionTiming, torch.nn.Module):
     r"""Computes :math:`z_i = \sum_{(i,j,e)} W_e (x_j \otimes_{CG} y_e)` over the
     edges of a directed graph.
 

@@ -149,3 +149,24 @@ def test_side_stream_matches_default_stream(kind):
     assert torch.allclose(z, expected, atol=1e-5)
     for a, b in zip(grads, (t.grad for t in ts2[:3])):
         assert torch.allclose(a, b / 1.0, atol=1e-4)
+
+
+def test_benchmark_helpers():
+    """benchmark_forward / benchmark_backward keep the reference's call signatures and return one
+    positive sample per iteration; kernel-only time is below the time of the whole call."""
+    from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
+    problem = P.config2_nequip_uvu()
+    tp = oeq.TensorProduct(problem)
+    x, y, w, g = tp_inputs(problem, 20000, seed=1)
+    whole = tp.benchmark_forward(2, 4, x, y, g, w)
+    kernel = tp.benchmark_forward(2, 4, x, y, g, w, with_torch_overhead=False)
+    assert whole.shape == (4,) and np.all(whole > 0) and np.all(kernel > 0) and kernel.min() <= whole.max()
+    back = tp.benchmark_backward(2, 3, x, y, g, w, with_torch_overhead=False)
+    assert back.shape == (3,) and np.all(back > 0)
+    coords, rows, cols, _ = periodic_radius_graph(300, 12, 5.0, 0)
+    graph = CoordGraph(coords, rows, cols)
+    for det in (True, False):
+        conv = oeq.TensorProductConv(problem, deterministic=det)
+        for stats in (conv.benchmark_forward(1, 3, graph), conv.benchmark_backward(1, 3, graph)):
+            assert len(stats["time_millis"]) == 3 and min(stats["time_millis"]) > 0
+            assert stats["graph_adj_nnz"] == graph.nnz and min(stats["throughputs_gflops"]) > 0
