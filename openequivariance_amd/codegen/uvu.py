@@ -80,6 +80,13 @@ class UvuEmitter:
         self.NCH = low.n_chunks
         self.used_in1 = sorted({p.i1 for p in low.paths})
         self.used_out = sorted({p.io for p in low.paths})
+        # Blocks of different multiplicity in a row wider than a wave: chunk c only has channels of the blocks
+        # with mul > 64 c. The row bodies are then generated once per chunk (the chunk index is wave-uniform),
+        # each without the paths, loads and stores of the blocks it has no channel of; cur_chunk is the chunk
+        # being generated (None: one body for all chunks).
+        used_muls = {low.in1[b].mul for b in self.used_in1} | {low.out[io].mul for io in self.used_out}
+        self.chunk_split = self.R == 1 and self.NCH > 1 and any(m != 64 * self.NCH for m in used_muls)
+        self.cur_chunk: Optional[int] = None
         # output segments (register-resident accumulators of the conv forward)
         budget = max(1, acc_budget_words // self.words)
         self.segments: List[List[int]] = []
@@ -297,8 +304,44 @@ class UvuEmitter:
         return f"({rowexpr} + {const} + {u} * {stride})"
 
     def _full(self, mul: int) -> bool:
-        """Every lane's channel index (0 .. lanes_per_row * chunks - 1) is a channel of such a block."""
+        """Every lane's channel index is a channel of such a block (over all chunks, or in the chunk being
+        generated)."""
+        if self.cur_chunk is not None:
+            return mul >= 64 * (self.cur_chunk + 1)
         return mul == self.LPR * self.NCH
+
+    def _has(self, mul: int) -> bool:
+        """The chunk being generated has channels of a block of this multiplicity."""
+        return self.cur_chunk is None or mul > 64 * self.cur_chunk
+
+    def _paths(self, paths: Optional[List[Path]] = None) -> List[Path]:
+        base = self.low.paths if paths is None else paths
+        return [p for p in base if self._has(self.low.in1[p.i1].mul)]
+
+    def _in1_of(self, blocks: List[int]) -> List[int]:
+        return [b for b in blocks if self._has(self.low.in1[b].mul)]
+
+    def _out_of(self, ios: List[int]) -> List[int]:
+        return [io for io in ios if self._has(self.low.out[io].mul)]
+
+    def _sfx(self) -> str:
+        return "" if self.cur_chunk is None else f"_c{self.cur_chunk}"
+
+    def _per_chunk(self, s: Src, body: Callable[[], None], in_kernel: bool = True):
+        """Emit ``body`` once, or once per chunk (inside ``if (chunk == c)`` when in a kernel)."""
+        if not self.chunk_split:
+            body()
+            return
+        for c in range(self.NCH):
+            self.cur_chunk = c
+            try:
+                if in_kernel:
+                    s.open(f"if (chunk == {c})")
+                body()
+                if in_kernel:
+                    s.close()
+            finally:
+                self.cur_chunk = None
 
     def _val(self, mul: int, loaded: str, extra: Optional[str] = None) -> str:
         """A value loaded through a clamped pointer, zeroed for lanes without a channel (and when
@@ -372,7 +415,7 @@ class UvuEmitter:
 
     def _load_x(self, s: Src, rowexpr: str, blocks: List[int], dst: str = "x"):
         low = self.low
-        for b in blocks:
+        for b in self._in1_of(blocks):
             blk = low.in1[b]
             s.open("")
             base, st = self._lane_ptr(blk)
@@ -432,8 +475,10 @@ class UvuEmitter:
         """load_edge: fetch X[cols[e]] (the listed blocks), the weights of the
         listed paths and the edge's Y into an E_t."""
         low = self.low
+        paths = self._paths(paths)
         s.open(
-            f"OEQ_DEV void {name}(E_t& d, const i64 e, const T* __restrict__ L1_in, const T* __restrict__ L2_in, "
+            f"OEQ_DEV void {name}{self._sfx()}(E_t& d, const i64 e, const T* __restrict__ L1_in, "
+            "const T* __restrict__ L2_in, "
             "const T* __restrict__ W, const i64* __restrict__ cols, const int u)"
         )
         s("const i64 c = cols[e];")
@@ -455,19 +500,19 @@ class UvuEmitter:
         seg = self.segments[si]
         if preloaded == "lds":
             xname, yacc, wacc = self._acc_staged3("sb")
-            s.open(f"OEQ_DEV void fwd_seg{si}_lds(const T* sb, const int ul, A{si}_t& a)")
+            s.open(f"OEQ_DEV void fwd_seg{si}_lds{self._sfx()}(const T* sb, const int ul, A{si}_t& a)")
         elif preloaded:
             yacc, wacc = self._acc_preloaded("d")
-            s.open(f"OEQ_DEV void fwd_seg{si}_pre(const E_t& d, A{si}_t& a)")
+            s.open(f"OEQ_DEV void fwd_seg{si}_pre{self._sfx()}(const E_t& d, A{si}_t& a)")
             xname = "d.x"
         else:
             yacc, wacc = self._acc_pointer()
             s.open(
-                f"OEQ_DEV void fwd_seg{si}(const X_t& x, const T* __restrict__ yrow, "
+                f"OEQ_DEV void fwd_seg{si}{self._sfx()}(const X_t& x, const T* __restrict__ yrow, "
                 f"const T* __restrict__ wrow, const int u, A{si}_t& a)"
             )
             xname = "x"
-        for p in low.paths:
+        for p in self._paths():
             if p.io not in seg:
                 continue
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
@@ -491,14 +536,19 @@ class UvuEmitter:
         s.close()
 
     def emit_forward_cores(self, s: Src, preloaded: bool):
-        for si in range(len(self.segments)):
-            self._emit_fwd_seg(s, si, False)
-            if preloaded and self.can_preload:
-                paths = [p for p in self.low.paths if p.io in self.segments[si]]
-                self._emit_load_edge(s, f"load_edge_f{si}", self.seg_in1[si], paths)
-                self._emit_fwd_seg(s, si, True)
-            if preloaded and self.stage3 is not None:
-                self._emit_fwd_seg(s, si, "lds")
+        def emit():
+            for si in range(len(self.segments)):
+                self._emit_fwd_seg(s, si, False)
+                if preloaded and self.can_preload:
+                    paths = [p for p in self.low.paths if p.io in self.segments[si]]
+                    self._emit_load_edge(s, f"load_edge_f{si}", self.seg_in1[si], paths)
+                    self._emit_fwd_seg(s, si, True)
+                if preloaded and self.stage3 is not None:
+                    self._emit_fwd_seg(s, si, "lds")
+
+        self._per_chunk(s, emit, in_kernel=False)
+        if self.chunk_split:
+            emit()  # chunk-agnostic versions, used by the float-atomics kernels
 
     def _regular_wave(self) -> bool:
         """Every used block is exactly 64 channels per wave-chunk and a row fills the wave."""
@@ -541,11 +591,11 @@ class UvuEmitter:
     def _store_seg(self, s: Src, si: int, rowexpr: str, guard: str, atomic: bool = False):
         low = self.low
         if atomic and self.tr_atomics:
-            for io in self.segments[si]:
+            for io in self._out_of(self.segments[si]):
                 bo = low.out[io]
                 self._atomic_block_transposed(s, rowexpr, bo.off, bo.d, lambda k, io=io: f"a.o{io}[{k}]")
             return
-        for io in self.segments[si]:
+        for io in self._out_of(self.segments[si]):
             bo = low.out[io]
             if not atomic and guard == "true" and self._can_transpose(bo, 1):
                 self._store_block_transposed(s, rowexpr, bo.off, bo.d, lambda k, io=io: f"a.o{io}[{k}]",
@@ -626,14 +676,17 @@ class UvuEmitter:
         if self.R == 1:
             s.open("if (live)")
             live = "true"
-        s("X_t x;")
-        self._load_x(s, "xrow", self.used_in1)
-        for si in range(len(self.segments)):
-            s.open("")
-            s(f"A{si}_t a; zero_seg{si}(a);")
-            s(f"fwd_seg{si}(x, yrow, wrow, u, a);")
-            self._store_seg(s, si, "zrow", live)
-            s.close()
+        def row_body():
+            s("X_t x;")
+            self._load_x(s, "xrow", self.used_in1)
+            for si in range(len(self.segments)):
+                s.open("")
+                s(f"A{si}_t a; zero_seg{si}(a);")
+                s(f"fwd_seg{si}{self._sfx()}(x, yrow, wrow, u, a);")
+                self._store_seg(s, si, "zrow", live)
+                s.close()
+
+        self._per_chunk(s, row_body)
         self._zero_untouched_out(s, "zrow", live)
         if self.R == 1:
             s.close()
@@ -648,11 +701,17 @@ class UvuEmitter:
         sets (A, B); the next edge's loads are issued before the current edge is
         computed. ``load(buf, e)`` / ``compute(buf, e)`` emit code."""
         R = self.R
+        # The compiler takes a direct global->LDS load to write only the bytes at the pointer it is given,
+        # not the 64 lanes' worth behind it, so it would move reads of the staging buffer across the load
+        # or across the wait for it. The empty asm statements pin them: no memory access crosses one.
+        fence = 'asm volatile("" ::: "memory");'
+
         def vmcnt(n: int) -> str:
             # s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt = simm16[3:0] | simm16[15:14] << 4)
-            return f"__builtin_amdgcn_s_waitcnt({(n & 15) | 0x0F70 | ((n >> 4) << 14)}); /* vmcnt({n}) */"
+            return f"__builtin_amdgcn_s_waitcnt({(n & 15) | 0x0F70 | ((n >> 4) << 14)}); /* vmcnt({n}) */ {fence}"
 
-        lgkm0 = "__builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): LDS reads retired before the buffer is refilled"
+        # lgkmcnt(0): LDS reads retired before the buffer is refilled
+        lgkm0 = f"{fence} __builtin_amdgcn_s_waitcnt(0xC07F); {fence}"
         if pipelined == 3:
             # Two LDS buffers per wave, loads one edge ahead. Stores and atomics of the loop body share
             # the vector-memory counter, so the wait before an edge is for everything outstanding.
@@ -791,7 +850,7 @@ class UvuEmitter:
         def make_load(si):
             def load(buf, e):
                 if self.can_preload:
-                    s(f"load_edge_f{si}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u);")
+                    s(f"load_edge_f{si}{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u);")
             return load
 
         kahan = self.kahan and deterministic
@@ -806,9 +865,9 @@ class UvuEmitter:
 
         def inner(si, buf, e):
             if mode == 3:
-                s(f"fwd_seg{si}_lds(&s_stage{buf}[wave][0], ul, {acc});")
+                s(f"fwd_seg{si}_lds{self._sfx()}(&s_stage{buf}[wave][0], ul, {acc});")
             elif self.can_preload:
-                s(f"fwd_seg{si}_pre({buf}, {acc});")
+                s(f"fwd_seg{si}_pre{self._sfx()}({buf}, {acc});")
             else:
                 s.open("")
                 s(f"const i64 eid = OEQ_EDGE({e});")
@@ -817,7 +876,7 @@ class UvuEmitter:
                 s(f"const T* wrow = W{'' if low.shared_weights else f' + eid * {low.WN}'};")
                 s("X_t x;")
                 self._load_x(s, "xrow", self.seg_in1[si])
-                s(f"fwd_seg{si}(x, yrow, wrow, u, {acc});")
+                s(f"fwd_seg{si}{self._sfx()}(x, yrow, wrow, u, {acc});")
                 s.close()
 
         if deterministic:
@@ -826,19 +885,25 @@ class UvuEmitter:
             s(f"T* zrow = L3_out + node * {low.L3};")
             for si in range(len(self.segments)):
                 s.open(f"if (sg == {si % segw})" if segw > 1 else "")
-                s(f"A{si}_t a; zero_seg{si}(a);")
-                if kahan:
-                    s(f"A{si}_t c; zero_seg{si}(c);")
-                self._edge_loop(s, "e0 + r", "e1", make_load(si), make_compute(si), mode)
-                if R > 1:
-                    # fold the R lane groups (fixed order) into group 0
-                    for io in self.segments[si]:
-                        for k in range(low.out[io].d):
-                            m = self.LPR
-                            while m < 64:
-                                s(f"a.o{io}[{k}] += __shfl_xor(a.o{io}[{k}], {m});")
-                                m *= 2
-                self._store_seg(s, si, "zrow", "r == 0" if self.R > 1 else "true")
+
+                def node_body(si=si):
+                    if self.cur_chunk is not None and not self._out_of(self.segments[si]):
+                        return  # this chunk has no channel of the segment's blocks
+                    s(f"A{si}_t a; zero_seg{si}(a);")
+                    if kahan:
+                        s(f"A{si}_t c; zero_seg{si}(c);")
+                    self._edge_loop(s, "e0 + r", "e1", make_load(si), make_compute(si), mode)
+                    if R > 1:
+                        # fold the R lane groups (fixed order) into group 0
+                        for io in self.segments[si]:
+                            for k in range(low.out[io].d):
+                                m = self.LPR
+                                while m < 64:
+                                    s(f"a.o{io}[{k}] += __shfl_xor(a.o{io}[{k}], {m});")
+                                    m *= 2
+                    self._store_seg(s, si, "zrow", "r == 0" if self.R > 1 else "true")
+
+                self._per_chunk(s, node_body)
                 s.close()
             self._zero_untouched_out(s, "zrow", "r == 0 && sg == 0" if segw > 1 else "r == 0")
             s.close()
@@ -878,7 +943,7 @@ class UvuEmitter:
     # ------------------------------------------------------- backward pieces
     def _load_g(self, s: Src, rowexpr: str, ios: List[int], dst: str = "gr"):
         low = self.low
-        for io in ios:
+        for io in self._out_of(ios):
             bo = low.out[io]
             s.open("")
             base, st = self._lane_ptr(bo)
@@ -895,7 +960,7 @@ class UvuEmitter:
         dy[], u, and either gr (G_t, resident) or a row pointer to load output
         gradients from. dw_mode 'store': dwrow[...] = v; 'acc': dwacc[slot] += v."""
         low = self.low
-        for p in sorted(low.paths if paths is None else paths, key=lambda q: (q.io, q.index)):
+        for p in sorted(self._paths(paths), key=lambda q: (q.io, q.index)):
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
             V = b2.mul
             s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
@@ -964,12 +1029,12 @@ class UvuEmitter:
         stored after the last path: a conditional store inside the chain of paths splits it into many
         basic blocks, and the compiler then moves the dY/dX accumulations to the end of the row, keeping
         every path's operands alive until there (hundreds of registers for problems with many paths)."""
-        needs_cond = any(self._store_cond(self.low.in1[p.i1].mul, dw_guard) for p in self.low.paths)
+        needs_cond = any(self._store_cond(self.low.in1[p.i1].mul, dw_guard) for p in self._paths())
         return needs_cond and self.can_preload
 
     def _flush_dwkeep(self, s: Src, dw_guard: Optional[str]):
         low = self.low
-        for p in low.paths:
+        for p in self._paths():
             b1, V = low.in1[p.i1], low.in2[p.i2].mul
             self._open_if(s, self._store_cond(b1.mul, dw_guard))
             for v in range(V):
@@ -1036,11 +1101,11 @@ class UvuEmitter:
     def _store_dx(self, s: Src, rowexpr: str, guard: str, atomic: bool = False, nt: bool = False):
         low = self.low
         if atomic and self.tr_atomics:
-            for b in self.used_in1:
+            for b in self._in1_of(self.used_in1):
                 blk = low.in1[b]
                 self._atomic_block_transposed(s, rowexpr, blk.off, blk.d, lambda i, b=b: f"dx.b{b}[{i}]")
             return
-        for b in self.used_in1:
+        for b in self._in1_of(self.used_in1):
             blk = low.in1[b]
             if not atomic and guard == "true" and self._can_transpose(blk, 2):
                 self._store_block_transposed(s, rowexpr, blk.off, blk.d, lambda i, b=b: f"dx.b{b}[{i}]", nt)
@@ -1069,7 +1134,7 @@ class UvuEmitter:
             s.close()
 
     def _zero_x(self, s: Src, name: str):
-        for b in self.used_in1:
+        for b in self._in1_of(self.used_in1):
             for i in range(self.low.in1[b].d):
                 s(f"{name}.b{b}[{i}] = T(0);")
 
@@ -1118,31 +1183,35 @@ class UvuEmitter:
         if self.R == 1:
             s.open("if (live)")
             live = "true"
-        s("X_t x, dx;")
-        self._load_x(s, "xrow", self.used_in1)
-        self._zero_x(s, "dx")
-        s(f"T dy[{self.l2_pad}];")
-        s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
-        yacc, wacc = self._acc_pointer()
-        deferred = not shared and self._dw_deferred(live)
-        if deferred:
-            s(f"T dwkeep[{self.n_wslots}];")
-        if g_resident and not shared:
-            # the whole output-gradient slice is requested up front, together with X and W: one long
-            # burst of loads per row instead of a load-wait-compute round per path
-            s("G_t gr;")
-            self._load_g(s, "grow", self.used_out)
-            self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, dw_mode="store", dw_guard=live)
-        else:
-            self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, g_on_demand_row="grow",
-                            dw_mode="acc" if shared else "store",
-                            g_guard="live" if shared and self.R > 1 else None, dw_guard=live)
-        if deferred:
-            self._flush_dwkeep(s, live)
-        s(f"T* dxrow = L1_grad + rowc * {low.L1};")
-        self._store_dx(s, "dxrow", live, nt=bool(self.nt & 2))
-        self._zero_untouched_in1(s, "dxrow", live)
-        self._dy_finish(s, f"L2_grad + rowc * {low.L2}", live)
+        def row_body():
+            s("X_t x, dx;")
+            self._load_x(s, "xrow", self.used_in1)
+            self._zero_x(s, "dx")
+            s(f"T dy[{self.l2_pad}];")
+            s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+            yacc, wacc = self._acc_pointer()
+            deferred = not shared and self._dw_deferred(live)
+            if deferred:
+                s(f"T dwkeep[{self.n_wslots}];")
+            if g_resident and not shared:
+                # the whole output-gradient slice is requested up front, together with X and W: one long
+                # burst of loads per row instead of a load-wait-compute round per path
+                s("G_t gr;")
+                self._load_g(s, "grow", self.used_out)
+                self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, dw_mode="store", dw_guard=live)
+            else:
+                self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, g_on_demand_row="grow",
+                                dw_mode="acc" if shared else "store",
+                                g_guard="live" if shared and self.R > 1 else None, dw_guard=live)
+            if deferred:
+                self._flush_dwkeep(s, live)
+            s(f"T* dxrow = L1_grad + rowc * {low.L1};")
+            self._store_dx(s, "dxrow", live, nt=bool(self.nt & 2))
+            self._zero_untouched_in1(s, "dxrow", live)
+            # every chunk's body ends with the same block barriers of the dY reduction
+            self._dy_finish(s, f"L2_grad + rowc * {low.L2}", live)
+
+        self._per_chunk(s, row_body)
         if self.R == 1:
             s.close()
         s.close()
@@ -1165,16 +1234,33 @@ class UvuEmitter:
         return block
 
     # -------------------------------------------------------- conv backward
+    def ragged(self) -> bool:
+        """Some used block has lanes without a channel (guards, clamped loads, deferred dW stores)."""
+        low = self.low
+        full = self.LPR * self.NCH
+        return any(low.in1[b].mul != full for b in self.used_in1) or any(low.out[io].mul != full
+                                                                          for io in self.used_out)
+
+    def backward_words(self, g_resident: bool) -> int:
+        """Rough count of 32-bit registers a lane needs in a backward row / edge body."""
+        low = self.low
+        x = sum(low.in1[b].d for b in self.used_in1)
+        g = sum(low.out[io].d for io in self.used_out) if g_resident else 8
+        w = self.n_wslots * (2 if self.ragged() else 1)  # weights, and weight gradients waiting for their store
+        return self.words * (g + 2 * x + self.l2_pad + w + low.L2) + 40
+
     def plan_backward_groups(self, max_waves: int) -> Optional[List[List[int]]]:
         """When a node's output gradient does not fit one wave's registers, share the output blocks (and
         with them the paths) between several waves of the node so that each keeps its share resident.
         Returns the blocks per wave, or None when that is not possible or not needed."""
         low = self.low
-        if self.g_resident or low.shared_weights or not self.can_preload or self.R != 1:
+        fits = self.g_resident and self.backward_words(True) <= 240
+        if fits or low.shared_weights or not self.can_preload or self.R != 1:
             return None
-        budget = max(1, 96 // self.words)  # leaves room for the edge operands, dX and dY beside it
+        # room for the edge operands, dX, dY (and deferred dW) beside the wave's share of the gradient
+        budget = max(1, (96 if not self.ragged() else 64) // self.words)
         sizes = [low.out[io].d for io in self.used_out]
-        n = -(-sum(sizes) // budget)
+        n = max(2 if self.g_resident else 1, -(-sum(sizes) // budget))
         while n <= max_waves:
             target = -(-sum(sizes) // n)
             groups, cur, tot = [], [], 0
@@ -1206,7 +1292,8 @@ class UvuEmitter:
         gpaths = [[p for p in low.paths if p.io in grp] for grp in groups]
         gin1 = [sorted({p.i1 for p in ps}) for ps in gpaths]
         for si in range(SW):
-            self._emit_load_edge(s, f"load_edge_b{si}", gin1[si], gpaths[si])
+            self._per_chunk(s, lambda si=si: self._emit_load_edge(s, f"load_edge_b{si}", gin1[si], gpaths[si]),
+                            in_kernel=False)
         s.open(
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void backward(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
@@ -1225,68 +1312,72 @@ class UvuEmitter:
         s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
         for si in range(SW):
             s.open(f"if (sg == {si})")
-            s("G_t gr;")
-            self._load_g(s, f"L3_grad + node * {low.L3}", groups[si])
-            # every wave of the block runs the same number of edges, so the block barriers match up
-            s.open("for (i64 e = e0; e < e1; ++e)")
-            s("const i64 eid = OEQ_EDGE(e);")
-            s(f"load_edge_b{si}(A, eid, L1_in, L2_in, W, cols, u);")
-            yacc, wacc = self._acc_preloaded("A")
-            s(f"T* dwrow = W_grad + eid * {low.WN};")
-            s("X_t dx;")
-            self._zero_x(s, "dx")
-            s(f"T dy[{self.l2_pad}];")
-            s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
-            deferred = self._dw_deferred(None)
-            if deferred:
-                s(f"T dwkeep[{self.n_wslots}];")
-            self._bwd_paths(s, xname="A.x", yacc=yacc, wacc=wacc, dw_mode="store", paths=gpaths[si])
-            if deferred:
-                low_paths, low.paths = low.paths, gpaths[si]
-                try:
-                    self._flush_dwkeep(s, None)
-                finally:
-                    low.paths = low_paths
-            for b in gin1[si]:
-                for i in range(low.in1[b].d):
-                    s(f"s_dx[{si}][chunk][{xoff[b] + i}][ul] = dx.b{b}[{i}];")
-            s.open("")
-            cur, dup = self._dy_reduce(s)
-            s.open(f"if ((ul & {dup}) == 0)")
-            for j in range(cur):
-                s(f"s_dy[{si} * {self.NCH} + chunk][dyidx + {j}] = rv[{j}];")
-            s.close()
-            s.close()
-            s("__syncthreads();")
-            # the used input blocks are shared out between the waves for the final sum and store
-            s(f"T* dxrow = dx_tmp + eid * {low.L1};")
-            for n, b in enumerate(self.used_in1):
-                if n % SW != si:
-                    continue
-                blk = low.in1[b]
-                contributors = [c for c in range(SW) if b in gin1[c]]
-                self._open_if(s, self._store_cond(blk.mul))
-                base, st = self._lane_ptr(blk)
-                s(f"T* dp = {self._ptr('dxrow', base)};")
-                for i in range(blk.d):
-                    terms = " + ".join(f"s_dx[{c}][chunk][{xoff[b] + i}][ul]" for c in contributors)
-                    val = f"({terms})" if contributors else "T(0)"
-                    if self.nt & 2:
-                        s(f"__builtin_nontemporal_store({val}, dp + {i * st});")
-                    else:
-                        s(f"dp[{i * st}] = {val};")
-                s.close()
-            if si == 0:
-                self._zero_untouched_in1(s, "dxrow", "true")
-                s.open(f"if (chunk == 0)")
-                s.open(f"for (int j = lane; j < {low.L2}; j += 64)")
-                s("T tot = s_dy[0][j];")
-                s(f"for (int cc = 1; cc < {SW * self.NCH}; ++cc) tot += s_dy[cc][j];")
-                s(f"L2_grad[eid * {low.L2} + j] = tot;")
+
+            def sg_body(si=si):
+                s("G_t gr;")
+                self._load_g(s, f"L3_grad + node * {low.L3}", groups[si])
+                # every wave of the block runs the same number of edges, so the block barriers match up
+                s.open("for (i64 e = e0; e < e1; ++e)")
+                s("const i64 eid = OEQ_EDGE(e);")
+                s(f"load_edge_b{si}{self._sfx()}(A, eid, L1_in, L2_in, W, cols, u);")
+                yacc, wacc = self._acc_preloaded("A")
+                s(f"T* dwrow = W_grad + eid * {low.WN};")
+                s("X_t dx;")
+                self._zero_x(s, "dx")
+                s(f"T dy[{self.l2_pad}];")
+                s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+                deferred = self._dw_deferred(None)
+                if deferred:
+                    s(f"T dwkeep[{self.n_wslots}];")
+                self._bwd_paths(s, xname="A.x", yacc=yacc, wacc=wacc, dw_mode="store", paths=gpaths[si])
+                if deferred:
+                    low_paths, low.paths = low.paths, gpaths[si]
+                    try:
+                        self._flush_dwkeep(s, None)
+                    finally:
+                        low.paths = low_paths
+                for b in self._in1_of(gin1[si]):
+                    for i in range(low.in1[b].d):
+                        s(f"s_dx[{si}][chunk][{xoff[b] + i}][ul] = dx.b{b}[{i}];")
+                s.open("")
+                cur, dup = self._dy_reduce(s)
+                s.open(f"if ((ul & {dup}) == 0)")
+                for j in range(cur):
+                    s(f"s_dy[{si} * {self.NCH} + chunk][dyidx + {j}] = rv[{j}];")
                 s.close()
                 s.close()
-            s("__syncthreads();")
-            s.close()
+                s("__syncthreads();")
+                # the used input blocks are shared out between the waves for the final sum and store
+                s(f"T* dxrow = dx_tmp + eid * {low.L1};")
+                for n, b in enumerate(self.used_in1):
+                    if n % SW != si or not self._has(low.in1[b].mul):
+                        continue
+                    blk = low.in1[b]
+                    contributors = [c for c in range(SW) if b in gin1[c]]
+                    self._open_if(s, self._store_cond(blk.mul))
+                    base, st = self._lane_ptr(blk)
+                    s(f"T* dp = {self._ptr('dxrow', base)};")
+                    for i in range(blk.d):
+                        terms = " + ".join(f"s_dx[{c}][chunk][{xoff[b] + i}][ul]" for c in contributors)
+                        val = f"({terms})" if contributors else "T(0)"
+                        if self.nt & 2:
+                            s(f"__builtin_nontemporal_store({val}, dp + {i * st});")
+                        else:
+                            s(f"dp[{i * st}] = {val};")
+                    s.close()
+                if si == 0:
+                    self._zero_untouched_in1(s, "dxrow", "true")
+                    s.open(f"if (chunk == 0)")
+                    s.open(f"for (int j = lane; j < {low.L2}; j += 64)")
+                    s("T tot = s_dy[0][j];")
+                    s(f"for (int cc = 1; cc < {SW * self.NCH}; ++cc) tot += s_dy[cc][j];")
+                    s(f"L2_grad[eid * {low.L2} + j] = tot;")
+                    s.close()
+                    s.close()
+                s("__syncthreads();")
+                s.close()
+
+            self._per_chunk(s, sg_body)
             s.close()
         s.close()
         s.close()
@@ -1302,6 +1393,9 @@ class UvuEmitter:
         mode = self._edge_mode(pipelined)
         if self.can_preload:
             self._emit_load_edge(s, "load_edge_b", self.used_in1, low.paths)
+            if self.chunk_split and deterministic:
+                self._per_chunk(s, lambda: self._emit_load_edge(s, "load_edge_b", self.used_in1, low.paths),
+                                in_kernel=False)
         s.open(
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void backward(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
@@ -1332,7 +1426,7 @@ class UvuEmitter:
 
         def load(buf, e):
             if self.can_preload:
-                s(f"load_edge_b({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u);")
+                s(f"load_edge_b{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u);")
 
         def make_compute(grow_expr_of):
             def compute(buf, pos):
@@ -1389,12 +1483,17 @@ class UvuEmitter:
         if deterministic:
             self._node_loop_open(s, G, xcd)
             s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
-            if resident:
-                s("G_t gr;")
-                self._load_g(s, f"L3_grad + node * {low.L3}", self.used_out)
-            # with more than one chunk all waves of the block walk the same edges, so the
-            # block barriers of the dY reduction are reached uniformly
-            self._edge_loop(s, "e0 + r", "e1", load, make_compute(lambda e: f"L3_grad + node * {low.L3}"), mode)
+
+            def node_body():
+                if resident:
+                    s("G_t gr;")
+                    self._load_g(s, f"L3_grad + node * {low.L3}", self.used_out)
+                # with more than one chunk all waves of the block walk the same edges, so the
+                # block barriers of the dY reduction are reached uniformly (also across per-chunk bodies)
+                self._edge_loop(s, "e0 + r", "e1", load, make_compute(lambda e: f"L3_grad + node * {low.L3}"),
+                                mode)
+
+            self._per_chunk(s, node_body)
             s.close()
         else:
             s(f"const i64 ngrp = (i64)gridDim.x * {G};")
@@ -1449,10 +1548,12 @@ def tp_module(low: Lowered, compute_units: int = 256):
     f32 = low.elem_size == 4
     wide = low.n_chunks > 1
     g_words = sum(low.out[io].d for io in {p.io for p in low.paths}) * (1 if f32 else 2)
+    probe = UvuEmitter(low)
     big = g_words > 256
+    on_demand = big or probe.backward_words(True) > (250 if f32 else 420)
     t = tuning(dict(tp_acc=48, tp_gf=1 if wide else 4, tp_gb=1 if wide else 4,
-                    tp_wf=2 if f32 else 0, tp_wb=3 if big else 2, tp_nt=0, tp_gres=0 if big else 1,
-                    tp_sb=1 if big else 0, tp_trs=1))
+                    tp_wf=2 if f32 else 0, tp_wb=3 if big else 2, tp_nt=0, tp_gres=0 if on_demand else 1,
+                    tp_sb=1 if on_demand else 0, tp_trs=1))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
     em.sched_fence = bool(t["tp_sb"])
@@ -1518,7 +1619,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             need = max(sets * words * (sum(low.in1[b].d for b in e.seg_in1[si]) + low.L2 +
                                        sum(low.in2[p.i2].mul for p in low.paths if p.io in seg))
                        + words * sum(low.out[io].d for io in seg) for si, seg in enumerate(e.segments))
-            return e, need
+            return e, need + (40 if e.ragged() else 0)  # clamped indices and select masks of ragged blocks
 
         budgets = (t["conv_acc"], 96, 64, 48)
         for budget in budgets:

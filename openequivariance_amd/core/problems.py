@@ -120,6 +120,41 @@ def nequip_problems():
     ]
 
 
+def tetris_poly_problems():
+    """The two fully connected products of e3nn's tetris polynomial example (problems.py:253-270);
+    default (shared) weights."""
+    return [
+        FCTPP("1x0e + 1x1o + 1x2e + 1x3o", "1x0e + 1x1o + 1x2e + 1x3o", "64x0e + 24x1e + 24x1o + 16x2e + 16x2o",
+              label="tetris-poly-1"),
+        FCTPP("64x0e + 24x1e + 24x1o + 16x2e + 16x2o", "1x0e + 1x1o + 1x2e", "0o + 6x0e", label="tetris-poly-2"),
+    ]
+
+
+def nequix_problems():
+    """NequiX MP-1 layers: mixed multiplicities per irrep, one with 89 channels (problems.py:351-372)."""
+    sh = "1x0e+1x1o+1x2e+1x3o"
+    mid = "128x0e+64x1o+32x2e+32x3o"
+    return [
+        CTPP("89x0e", sh, "89x0e+89x1o+89x2e+89x3o", "nequix-mp-1-first_layer"),
+        CTPP(mid, sh, "128x0e+128x1o+128x2e+128x3o+64x1o+64x0e+64x2e+64x1o+64x3o+64x2e+32x2e+32x1o+32x3o+32x0e+32x2e"
+                      "+32x1o+32x3o+32x3o+32x2e+32x1o+32x3o+32x0e+32x2e", "nequix-mp-1-main_layers"),
+        CTPP(mid, sh, "128x0e+64x0e+32x0e+32x0e", "nequix-mp-1-last_layer"),
+    ]
+
+
+def seven_net_problems():
+    """SevenNet l3i5 layers, even-parity harmonics (problems.py:375-395)."""
+    sh = "1x0e+1x1e+1x2e+1x3e"
+    mid = "128x0e+64x1e+32x2e+32x3e"
+    return [
+        CTPP("128x0e", sh, "128x0e+128x1e+128x2e+128x3e", "SevenNet_l3i5-first-layer"),
+        CTPP(mid, sh, "128x0e+64x0e+32x0e+32x0e+128x1e+64x1e+64x1e+64x1e+32x1e+32x1e+32x1e+32x1e+32x1e+128x2e+64x2e"
+                      "+64x2e+64x2e+32x2e+32x2e+32x2e+32x2e+32x2e+32x2e+32x2e+128x3e+64x3e+64x3e+32x3e+32x3e+32x3e"
+                      "+32x3e+32x3e+32x3e+32x3e", "SevenNet_l3i5-main-layers"),
+        CTPP(mid, sh, "128x0e+64x0e+32x0e+32x0e", "SevenNet_l3i5-last-layer"),
+    ]
+
+
 def diffdock_problems():
     """Fully connected DiffDock score-model layers with per-row weights (problems.py:273-289)."""
     feats = "10x1o + 10x1e + 48x0e + 48x0o"

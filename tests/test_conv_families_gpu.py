@@ -37,6 +37,7 @@ def _cases():
                 dtype = np.float64 if (n + q) % 4 == 3 else np.float32
                 out.append(_single(mode, m, irs[(2 * n + q) % len(irs)], dtype))
     out += P.mace_problems() + P.diffdock_problems() + P.e3tools_problems()
+    out += P.nequix_problems() + P.seven_net_problems()  # a different multiplicity per irrep
     shared = P.mace_problems()[0].clone()
     shared.shared_weights = True
     shared.label = "mace-large-shared"

@@ -27,6 +27,12 @@ def _odd_uvw(shared):
                          internal_weights=False, label="odd-uvw")
 
 
+def _as_f64(problem):
+    q = problem.clone()
+    q.irrep_dtype, q.weight_dtype = np.float64, np.float64
+    return q
+
+
 CASES = [
     ("cfg1-b1000", P.config1_single_uvu, 1000),
     ("cfg1-b37", P.config1_single_uvu, 37),
@@ -49,6 +55,15 @@ CASES = [
     ("uvu-mul2-big", lambda: P.SingleInstruction("4x1e", "12x1e", "4x1e", "uvu"), 40),
     ("uvw-unshared", lambda: P.FullyConnectedTPProblem("16x0e+16x1o", "1x0e+1x1o", "16x0e+16x1o",
                                                       shared_weights=False, internal_weights=False), 33),
+    # production layers with a different multiplicity per irrep (rows wider than a wave: the chunks of a
+    # row then run different code), one with 89 channels
+    ("nequix-first", lambda: P.nequix_problems()[0], 53),
+    ("nequix-main", lambda: P.nequix_problems()[1], 53),
+    ("nequix-last", lambda: P.nequix_problems()[2], 53),
+    ("sevennet-main", lambda: P.seven_net_problems()[1], 53),
+    ("sevennet-main-f64", lambda: _as_f64(P.seven_net_problems()[1]), 29),
+    ("tetris-1", lambda: P.tetris_poly_problems()[0], 53),
+    ("tetris-2", lambda: P.tetris_poly_problems()[1], 53),
     ("odd-uvw", lambda: _odd_uvw(False), 21),
     ("odd-uvw-shared", lambda: _odd_uvw(True), 21),
 ]
