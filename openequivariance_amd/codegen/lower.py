@@ -149,13 +149,52 @@ def lower(problem: TPProblem) -> Lowered:
         WN=problem.weight_numel, label=problem.label,
     )
     low.ir_mul = problem.layout == "ir_mul"
+    _lane_mapping(low)
+    if mode == "uvu" and not low.ir_mul and 1 < low.n_chunks <= 4 and \
+            any(in1[p.i1].mul != 64 * low.n_chunks for p in paths):
+        low = _fold_wide_blocks(low)
+    return low
+
+
+def _lane_mapping(low: Lowered) -> None:
+    in1, paths = low.in1, low.paths
     used_mul = [in1[p.i1].mul for p in paths]
     low.max_u = max(used_mul)
     low.lanes_per_row = 64 if low.max_u > 32 else _pow2ceil(low.max_u)
     low.rows_per_wave = 64 // low.lanes_per_row
     low.n_chunks = (low.max_u + 63) // 64
     low.total_nnz = sum(len(p.nnz) for p in paths)
-    return low
+
+
+def _fold_wide_blocks(low: Lowered) -> Lowered:
+    """'uvu' rows wider than a wave whose irreps have different multiplicities (128x0e+64x1o+32x2e,
+    89x0e, ...): cut every block into pieces of at most 64 channels and every path into the paths
+    between matching pieces. In the [mul, 2l+1] layout a piece is just a block that starts further into
+    the row, and its weights start ``64 * mul_v`` further into the path's weights, so the result is an
+    ordinary problem with at most 64 channels per block: one wave then owns the whole row and walks the
+    pieces one after the other, where waves that each owned one 64-channel slice of every block would
+    mostly have idle lanes or nothing to do."""
+    def cut(blocks: List[Block]):
+        pieces, index = [], {}
+        for b, blk in enumerate(blocks):
+            for c in range((blk.mul + 63) // 64):
+                index[(b, c)] = len(pieces)
+                pieces.append(Block(blk.off + c * 64 * blk.d, min(64, blk.mul - c * 64), blk.l))
+        return pieces, index
+
+    in1, index1 = cut(low.in1)
+    out, index3 = cut(low.out)
+    paths = []
+    for p in low.paths:
+        v_mul = low.in2[p.i2].mul
+        for c in range((low.in1[p.i1].mul + 63) // 64):
+            paths.append(Path(len(paths), index1[(p.i1, c)], p.i2, index3[(p.io, c)], p.woff + c * 64 * v_mul,
+                              p.coeff, p.nnz, p.l))
+    folded = Lowered(mode=low.mode, ctype=low.ctype, elem_size=low.elem_size, shared_weights=low.shared_weights,
+                     in1=in1, in2=low.in2, out=out, paths=paths, L1=low.L1, L2=low.L2, L3=low.L3, WN=low.WN,
+                     label=low.label)
+    _lane_mapping(folded)
+    return folded
 
 
 def float_literal(v: float, ctype: str) -> str:

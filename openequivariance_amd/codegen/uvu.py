@@ -30,7 +30,7 @@ loop_unroll_conv_det.cuh:96-293) with a different decomposition:
 from __future__ import annotations
 
 import os
-from typing import Callable, Dict, List, Optional, Tuple
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 from .common import Src, fixup_backward_kernel, prelude, utility_kernels
 from .lower import Lowered, Path, float_literal
@@ -68,6 +68,7 @@ class UvuEmitter:
         # non-temporally (batch kernels only: the convolution re-reads them).
         self.nt = 0
         self.sched_fence = False
+        self.fence_words = 0  # gradient registers between two scheduling fences (0: a fence after every path)
         self.seg_waves = 1  # conv forward: waves per node that share its output segments between them
         self.bwd_groups: Optional[List[List[int]]] = None  # conv backward: output blocks owned by each wave
         # plain stores of [64 x d] channel blocks go through the s_tr tile as well: bit 0 = forward outputs,
@@ -355,7 +356,14 @@ class UvuEmitter:
             conds.append(f"u < {mul}")
         return " && ".join(conds) if conds else None
 
-    def _open_if(self, s: Src, cond: Optional[str]):
+    def _open_if(self, s: Src, cond: Optional[str], values: Sequence[str] = ()):
+        """Open the block of a (possibly conditional) store of ``values``. Values that only a
+        conditional store uses are first passed through an empty asm statement: the compiler would
+        otherwise move the whole chain of operations that computes them into the conditional block,
+        and with it keep every operand of that chain alive until there."""
+        if cond:
+            for v in values:
+                s(f'asm volatile("" : "+v"({v}));')
         s.open(f"if ({cond})" if cond else "")
 
     def _y_index(self, b2, v: str, j: int) -> str:
@@ -601,7 +609,7 @@ class UvuEmitter:
                 self._store_block_transposed(s, rowexpr, bo.off, bo.d, lambda k, io=io: f"a.o{io}[{k}]",
                                              bool(self.nt & 8))
                 continue
-            self._open_if(s, self._store_cond(bo.mul, guard))
+            self._open_if(s, self._store_cond(bo.mul, guard), [f"a.o{io}[{k}]" for k in range(bo.d)])
             base, st = self._lane_ptr(bo)
             s(f"T* zp = {self._ptr(rowexpr, base)};")
             for k in range(bo.d):
@@ -960,7 +968,9 @@ class UvuEmitter:
         dy[], u, and either gr (G_t, resident) or a row pointer to load output
         gradients from. dw_mode 'store': dwrow[...] = v; 'acc': dwacc[slot] += v."""
         low = self.low
-        for p in sorted(self._paths(paths), key=lambda q: (q.io, q.index)):
+        ordered = sorted(self._paths(paths), key=lambda q: (q.io, q.index))
+        since_fence = 0
+        for n_path, p in enumerate(ordered):
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
             V = b2.mul
             s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
@@ -1020,9 +1030,15 @@ class UvuEmitter:
             self._for_v(s, p, body)
             s.close()
             if self.sched_fence and g_on_demand_row is not None:
-                # keep the scheduler from hoisting the next paths' gradient loads over this path:
-                # with many paths that costs more registers than a wave has
-                s("__builtin_amdgcn_sched_barrier(0);")
+                # keep the scheduler from hoisting all later paths' gradient loads over this path (with
+                # many paths that costs more registers than a wave has): a fence after every run of
+                # paths whose gradients take about ``fence_words`` registers, so that each run's loads
+                # still go out together
+                since_fence += bo.d * self.words
+                nxt = ordered[n_path + 1] if n_path + 1 < len(ordered) else None
+                if nxt is None or since_fence + low.out[nxt.io].d * self.words > self.fence_words:
+                    s("__builtin_amdgcn_sched_barrier(0);")
+                    since_fence = 0
 
     def _dw_deferred(self, dw_guard: Optional[str]) -> bool:
         """Per-row weight gradients whose store needs a condition are kept in registers (``dwkeep``) and
@@ -1032,11 +1048,26 @@ class UvuEmitter:
         needs_cond = any(self._store_cond(self.low.in1[p.i1].mul, dw_guard) for p in self._paths())
         return needs_cond and self.can_preload
 
+    def _pin_gradients(self, s: Src, blocks: List[int], deferred: bool, paths: Optional[List[Path]] = None):
+        """After the last path of a row / edge: pass every gradient accumulator through an empty asm
+        statement. What follows (conditional stores, the dY reduction) has branches, and the compiler
+        would otherwise move the accumulation chains below them, keeping every path's operands alive
+        until there."""
+        low = self.low
+        vals = [f"dx.b{b}[{i}]" for b in self._in1_of(blocks) for i in range(low.in1[b].d)]
+        vals += [f"dy[{t}]" for t in range(self.l2_pad)]
+        if deferred:
+            for p in self._paths(paths):
+                vals += [f"dwkeep[{self.wslot[p.index] + v}]" for v in range(low.in2[p.i2].mul)]
+        for v in vals:
+            s(f'asm volatile("" : "+v"({v}));')
+
     def _flush_dwkeep(self, s: Src, dw_guard: Optional[str]):
         low = self.low
         for p in self._paths():
             b1, V = low.in1[p.i1], low.in2[p.i2].mul
-            self._open_if(s, self._store_cond(b1.mul, dw_guard))
+            self._open_if(s, self._store_cond(b1.mul, dw_guard),
+                          [f"dwkeep[{self.wslot[p.index] + v}]" for v in range(V)])
             for v in range(V):
                 dwp = self._ptr("dwrow", (f"{p.woff} + {v}", V))
                 val = f"dwkeep[{self.wslot[p.index] + v}]"
@@ -1110,7 +1141,7 @@ class UvuEmitter:
             if not atomic and guard == "true" and self._can_transpose(blk, 2):
                 self._store_block_transposed(s, rowexpr, blk.off, blk.d, lambda i, b=b: f"dx.b{b}[{i}]", nt)
                 continue
-            self._open_if(s, self._store_cond(blk.mul, guard))
+            self._open_if(s, self._store_cond(blk.mul, guard), [f"dx.b{b}[{i}]" for i in range(blk.d)])
             base, st = self._lane_ptr(blk)
             s(f"T* dp = {self._ptr(rowexpr, base)};")
             for i in range(blk.d):
@@ -1203,6 +1234,7 @@ class UvuEmitter:
                 self._bwd_paths(s, xname="x", yacc=yacc, wacc=wacc, g_on_demand_row="grow",
                                 dw_mode="acc" if shared else "store",
                                 g_guard="live" if shared and self.R > 1 else None, dw_guard=live)
+            self._pin_gradients(s, self.used_in1, deferred)
             if deferred:
                 self._flush_dwkeep(s, live)
             s(f"T* dxrow = L1_grad + rowc * {low.L1};")
@@ -1330,6 +1362,7 @@ class UvuEmitter:
                 if deferred:
                     s(f"T dwkeep[{self.n_wslots}];")
                 self._bwd_paths(s, xname="A.x", yacc=yacc, wacc=wacc, dw_mode="store", paths=gpaths[si])
+                self._pin_gradients(s, gin1[si], deferred, gpaths[si])
                 if deferred:
                     low_paths, low.paths = low.paths, gpaths[si]
                     try:
@@ -1467,6 +1500,7 @@ class UvuEmitter:
                         s(f'asm volatile("" : "+{"s" if self.R == 1 else "v"}"(grow));')
                     self._bwd_paths(s, xname=xname, yacc=yacc, wacc=wacc, g_on_demand_row="grow",
                                     dw_mode="acc" if shared else "store")
+                self._pin_gradients(s, self.used_in1, deferred)
                 if deferred:
                     self._flush_dwkeep(s, None)
                 if deterministic:
@@ -1553,10 +1587,11 @@ def tp_module(low: Lowered, compute_units: int = 256):
     on_demand = big or probe.backward_words(True) > (250 if f32 else 420)
     t = tuning(dict(tp_acc=48, tp_gf=1 if wide else 4, tp_gb=1 if wide else 4,
                     tp_wf=2 if f32 else 0, tp_wb=3 if big else 2, tp_nt=0, tp_gres=0 if on_demand else 1,
-                    tp_sb=1 if on_demand else 0, tp_trs=1))
+                    tp_sb=1 if on_demand else 0, tp_trs=1, tp_fw=0))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
     em.sched_fence = bool(t["tp_sb"])
+    em.fence_words = t["tp_fw"]
     em.tr_stores = t["tp_trs"]
     s = Src()
     s(prelude(low.ctype))
