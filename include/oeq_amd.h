@@ -79,7 +79,9 @@ typedef enum {
     OEQ_ROLE_GROUP_SCAN = 10,       /*   exclusive scan (one block), */
     OEQ_ROLE_GROUP_SCATTER = 11,    /*   scatter of the item indices into their key's segment, */
     OEQ_ROLE_GROUP_ORDER = 12,      /*   and ascending order of the indices within each segment */
-    OEQ_ROLE_COUNT = 13
+    OEQ_ROLE_DOUBLE_BACKWARD_A = 13,/* second order: gradient w.r.t. the output gradient (forward-shaped) */
+    OEQ_ROLE_DOUBLE_BACKWARD_B = 14,/* second order: gradients w.r.t. X, Y, W (backward-shaped) */
+    OEQ_ROLE_COUNT = 15
 } oeq_role;
 
 /* How the convolution kernels of a set find the edges of a node (oeq_problem_dims.deterministic):
@@ -172,6 +174,32 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz,
                       const int64_t* transpose_perm,
                       void* workspace, size_t workspace_bytes, void* stream);
 size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
+
+/* ---- second-order ('double backward') kernels ---------------------------- */
+/* Gradient of the backward pass: given the operands of oeq_tp_backward (L1_in, L2_in, W, L3_grad) and
+ * cotangents L1_dgrad, L2_dgrad, W_dgrad of its three results, writes the gradients with respect to
+ * L1_in, L2_in, W and L3_grad (all four fully overwritten). Replaces JITTPImpl::double_backward
+ * (extension/tensorproducts.hpp:97-111) as called by jit_tp_double_backward
+ * (extension/torch_core.hpp:357-420). Only kernel sets for which oeq_has_double_backward() is non-zero
+ * carry these kernels ('uvu' problems with per-row weights); for the others the same result is composed
+ * from oeq_tp_forward / oeq_tp_backward calls by the caller. */
+int oeq_has_double_backward(const oeq_kernels* k);
+int oeq_tp_double_backward(oeq_kernels* k, int64_t num_batch,
+                           const void* L1_in, const void* L2_in, const void* W, const void* L3_grad,
+                           const void* L1_dgrad, const void* L2_dgrad, const void* W_dgrad,
+                           void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad, void* stream);
+
+/* The same for the fused convolution; replaces JITConvImpl::double_backward
+ * (extension/convolution.hpp:138-178) as called by jit_conv_double_backward
+ * (extension/torch_core.hpp:544-625). Index arguments and workspace
+ * (oeq_conv_backward_workspace_bytes() bytes) are those of oeq_conv_backward. Not available for
+ * OEQ_CONV_ATOMIC kernel sets. */
+int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz,
+                             const void* L1_in, const void* L2_in, const void* W, const void* L3_grad,
+                             const void* L1_dgrad, const void* L2_dgrad, const void* W_dgrad,
+                             void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad,
+                             const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm,
+                             void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- ordered segment sum -------------------------------------------------- */
 /* dst[s, :] = sum, in list order, of src[item, :] over the items whose key is s, for s < n_segments.

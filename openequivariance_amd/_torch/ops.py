@@ -164,19 +164,96 @@ def _tp_bwd_setup(ctx, inputs, output):
     ctx.save_for_backward(inputs[0], inputs[1], inputs[2], inputs[3])
 
 
+def _sum2(a, b):
+    """a + b where either may be missing; in place on ``a`` (a fresh kernel output nothing else holds)
+    when no graph is being recorded, which saves a pass over a weight-sized tensor."""
+    if a is None or b is None:
+        return b if a is None else a
+    return a + b if torch.is_grad_enabled() else a.add_(b)
+
+
+def _second_order(forward, backward, x, y, w, g, ddx, ddy, ddw):
+    """Gradients of ``backward(x, y, w, g) -> (dx, dy, dw)`` contracted with (ddx, ddy, ddw). The
+    tensor product is linear in each of x, y, w and g, so every term is the forward or backward
+    kernel applied with one operand replaced by its cotangent (the reference has two dedicated
+    kernels for this, double_backward_A/B in templates/loop_unroll_batch.cuh:148-317). Terms of
+    cotangents autograd did not ask for (None) are skipped."""
+    dx = dy = dw = gg = None
+    if ddy is not None:
+        dx1, _, dw1 = backward(x, ddy, w, g)
+        dx, dw = dx1, dw1
+        gg = forward(x, ddy, w)
+    if ddw is not None:
+        dx2, dy2, _ = backward(x, y, ddw, g)
+        dx, dy = _sum2(dx, dx2), dy2
+        gg = _sum2(gg, forward(x, y, ddw))
+    if ddx is not None:
+        _, dy3, dw3 = backward(ddx, y, w, g)
+        dy, dw = _sum2(dy, dy3), _sum2(dw, dw3)
+        gg = _sum2(gg, forward(ddx, y, w))
+    return dx, dy, dw, gg
+
+
+# The fused second-order kernels are used when no graph is being recorded for a third derivative (then
+# the composition of differentiable first-order ops is needed) and at least two of the three cotangents
+# are present (a missing one is passed as zeros; with a single cotangent the two first-order calls of
+# the composition read less). Tests switch this off to compare the two routes.
+FUSED_DOUBLE_BACKWARD = True
+
+
+def _use_fused(kid, ddx, ddy, ddw) -> bool:
+    if not FUSED_DOUBLE_BACKWARD or torch.is_grad_enabled():
+        return False
+    if sum(t is not None for t in (ddx, ddy, ddw)) < 2:
+        return False
+    e = get_entry(kid)
+    return not e.unfused and e.kernels().has_double_backward()
+
+
 def _zeros_if_none(t, like):
     return torch.zeros_like(like) if t is None else t
+
+
+@torch.library.custom_op("oeq_amd::tp_double_backward", mutates_args=(), device_types="cuda")
+def tp_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_grad: torch.Tensor,
+                       L1_dgrad: torch.Tensor, L2_dgrad: torch.Tensor, W_dgrad: torch.Tensor,
+                       kid: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(L1_grad, L2_grad, W_grad, L3_dgrad): the op of the reference's jit_tp_double_backward
+    (extension/torch_core.hpp:357-420)."""
+    e = get_entry(kid)
+    n = L1_in.shape[0] if L1_in.dim() > 0 else -1
+    for t, name in ((L1_in, "L1_in"), (L1_dgrad, "L1_dgrad")):
+        check_tensor(t, [n, e.L1], e.dtype, name)
+    for t, name in ((L2_in, "L2_in"), (L2_dgrad, "L2_dgrad")):
+        check_tensor(t, [n, e.L2], e.dtype, name)
+    for t, name in ((W, "W"), (W_dgrad, "W_dgrad")):
+        check_tensor(t, _wshape(e, n), e.dtype, name)
+    check_tensor(L3_grad, [n, e.L3], e.dtype, "L3_grad")
+    x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
+    a, b, c = L1_dgrad.contiguous(), L2_dgrad.contiguous(), W_dgrad.contiguous()
+    dx, dy, dw, gg = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w), torch.empty_like(g)
+    with torch.cuda.device(x.device):
+        e.kernels().tp_double_backward(n, x.data_ptr(), y.data_ptr(), w.data_ptr(), g.data_ptr(), a.data_ptr(),
+                                       b.data_ptr(), c.data_ptr(), dx.data_ptr(), dy.data_ptr(), dw.data_ptr(),
+                                       gg.data_ptr(), _stream())
+    return dx, dy, dw, gg
+
+
+@tp_double_backward.register_fake
+def _(L1_in, L2_in, W, L3_grad, L1_dgrad, L2_dgrad, W_dgrad, kid):
+    return torch.empty_like(L1_in), torch.empty_like(L2_in), torch.empty_like(W), torch.empty_like(L3_grad)
 
 
 def _tp_bwd_backward(ctx, ddx, ddy, ddw):
     x, y, w, g = ctx.saved_tensors
     kid = ctx.kid
-    ddx, ddy, ddw = _zeros_if_none(ddx, x), _zeros_if_none(ddy, y), _zeros_if_none(ddw, w)
-    dx1, _, dw1 = tp_backward(x, ddy, w, g, kid)
-    dx2, dy2, _ = tp_backward(x, y, ddw, g, kid)
-    _, dy3, dw3 = tp_backward(ddx, y, w, g, kid)
-    gg = tp_forward(ddx, y, w, kid) + tp_forward(x, ddy, w, kid) + tp_forward(x, y, ddw, kid)
-    return dx1 + dx2, dy2 + dy3, dw1 + dw3, gg, None
+    if _use_fused(kid, ddx, ddy, ddw):
+        dx, dy, dw, gg = tp_double_backward(x, y, w, g, _zeros_if_none(ddx, x), _zeros_if_none(ddy, y),
+                                            _zeros_if_none(ddw, w), kid)
+        return dx, dy, dw, gg, None
+    dx, dy, dw, gg = _second_order(lambda a, b, c: tp_forward(a, b, c, kid),
+                                   lambda a, b, c, d: tp_backward(a, b, c, d, kid), x, y, w, g, ddx, ddy, ddw)
+    return dx, dy, dw, gg, None
 
 
 tp_backward.register_autograd(_tp_bwd_backward, setup_context=_tp_bwd_setup)
@@ -326,16 +403,47 @@ def _conv_bwd_setup(ctx, inputs, output):
     ctx.save_for_backward(*inputs[:7])
 
 
+@torch.library.custom_op("oeq_amd::conv_double_backward", mutates_args=(), device_types="cuda")
+def conv_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_grad: torch.Tensor,
+                         L1_dgrad: torch.Tensor, L2_dgrad: torch.Tensor, W_dgrad: torch.Tensor,
+                         rows: torch.Tensor, cols: torch.Tensor, transpose_perm: torch.Tensor,
+                         kid: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(L1_grad, L2_grad, W_grad, L3_dgrad): the op of the reference's jit_conv_double_backward
+    (extension/torch_core.hpp:544-625)."""
+    e = get_entry(kid)
+    nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm, L3_grad)
+    _conv_checks(e, L1_dgrad, L2_dgrad, W_dgrad, rows, cols, transpose_perm)
+    x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
+    a, b, c = L1_dgrad.contiguous(), L2_dgrad.contiguous(), W_dgrad.contiguous()
+    r, cc, p = rows.contiguous(), cols.contiguous(), transpose_perm.contiguous()
+    dx, dy, dw, gg = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w), torch.empty_like(g)
+    with torch.cuda.device(x.device):
+        ks = e.kernels()
+        nb = ks.conv_backward_workspace_bytes(nodes, nnz)
+        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
+        ks.conv_double_backward(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), g.data_ptr(), a.data_ptr(),
+                                b.data_ptr(), c.data_ptr(), dx.data_ptr(), dy.data_ptr(), dw.data_ptr(),
+                                gg.data_ptr(), r.data_ptr(), cc.data_ptr(), p.data_ptr() if e.deterministic else 0,
+                                ws.data_ptr() if nb else 0, nb, _stream())
+    return dx, dy, dw, gg
+
+
+@conv_double_backward.register_fake
+def _(L1_in, L2_in, W, L3_grad, L1_dgrad, L2_dgrad, W_dgrad, rows, cols, transpose_perm, kid):
+    return torch.empty_like(L1_in), torch.empty_like(L2_in), torch.empty_like(W), torch.empty_like(L3_grad)
+
+
 def _conv_bwd_backward(ctx, ddx, ddy, ddw):
     x, y, w, g, rows, cols, perm = ctx.saved_tensors
     kid = ctx.kid
-    ddx, ddy, ddw = _zeros_if_none(ddx, x), _zeros_if_none(ddy, y), _zeros_if_none(ddw, w)
-    dx1, _, dw1 = conv_backward(x, ddy, w, g, rows, cols, perm, kid)
-    dx2, dy2, _ = conv_backward(x, y, ddw, g, rows, cols, perm, kid)
-    _, dy3, dw3 = conv_backward(ddx, y, w, g, rows, cols, perm, kid)
-    gg = (conv_forward(ddx, y, w, rows, cols, perm, kid) + conv_forward(x, ddy, w, rows, cols, perm, kid)
-          + conv_forward(x, y, ddw, rows, cols, perm, kid))
-    return dx1 + dx2, dy2 + dy3, dw1 + dw3, gg, None, None, None, None
+    if _use_fused(kid, ddx, ddy, ddw):
+        dx, dy, dw, gg = conv_double_backward(x, y, w, g, _zeros_if_none(ddx, x), _zeros_if_none(ddy, y),
+                                              _zeros_if_none(ddw, w), rows, cols, perm, kid)
+        return dx, dy, dw, gg, None, None, None, None
+    dx, dy, dw, gg = _second_order(lambda a, b, c: conv_forward(a, b, c, rows, cols, perm, kid),
+                                   lambda a, b, c, d: conv_backward(a, b, c, d, rows, cols, perm, kid),
+                                   x, y, w, g, ddx, ddy, ddw)
+    return dx, dy, dw, gg, None, None, None, None
 
 
 conv_backward.register_autograd(_conv_bwd_backward, setup_context=_conv_bwd_setup)

@@ -1587,7 +1587,8 @@ def tp_module(low: Lowered, compute_units: int = 256):
     on_demand = big or probe.backward_words(True) > (250 if f32 else 420)
     t = tuning(dict(tp_acc=48, tp_gf=1 if wide else 4, tp_gb=1 if wide else 4,
                     tp_wf=2 if f32 else 0, tp_wb=3 if big else 2, tp_nt=0, tp_gres=0 if on_demand else 1,
-                    tp_sb=1 if on_demand else 0, tp_trs=1, tp_fw=0))
+                    tp_sb=1 if on_demand else 0, tp_trs=1, tp_fw=0,
+                    tp_dd=1, dd_wa=2, dd_wb=2))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
     em.sched_fence = bool(t["tp_sb"])
@@ -1608,6 +1609,9 @@ def tp_module(low: Lowered, compute_units: int = 256):
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0),
     ]
+    from . import uvu_double
+    if t["tp_dd"] and uvu_double.supported(low):
+        descs += uvu_double.add_tp_kernels(s, low, em, t)
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
                 shared_weights=int(low.shared_weights), deterministic=0,
                 wpartial_per_block=G_b if low.shared_weights else 0)
@@ -1633,7 +1637,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
                     conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
-                    conv_segw=4, conv_split=1))
+                    conv_segw=4, conv_split=1, conv_dd=1, dd_acc=112, dd_g=2, dd_wa=2, dd_wb=2))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -1708,6 +1712,9 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         ]
         if low.shared_weights:
             descs.append((rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0))
+        from . import uvu_double
+        if t["conv_dd"] and uvu_double.supported(low) and not kahan:
+            descs += uvu_double.add_conv_kernels(s, low, em, t, xcd)
         if mode == rt.CONV_GROUPED:
             descs += [
                 (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, compute_units * 16),

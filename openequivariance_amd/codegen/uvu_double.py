@@ -1,0 +1,495 @@
+"""HIP source generator for the second-order ('double backward') kernels of 'uvu' problems.
+
+The first backward pass maps (X, Y, W, dZ) to (dX, dY, dW). Differentiating it once more, with
+cotangents (A, B, C) for (dX, dY, dW), gives, because the tensor product ``F`` is linear in each
+operand,
+
+    d/d(dZ) = F(A, Y, W) + F(X, B, W) + F(X, Y, C)                         (kernel ``double_backward_a``)
+    d/dX    = dX-part of backward(., B, W; dZ) + backward(., Y, C; dZ)
+    d/dY    = dY-part of backward(A, ., W; dZ) + backward(X, ., C; dZ)     (kernel ``double_backward_b``)
+    d/dW    = dW-part of backward(A, Y, .; dZ) + backward(X, B, .; dZ)
+
+The reference computes the same two groups with its kernels ``double_backward_A`` /
+``double_backward_B`` (openequivariance/openequivariance/templates/loop_unroll_batch.cuh:148-317,
+templates/loop_unroll_conv_det.cuh, wired in extension/torch_core.hpp:357-420 and 544-625). Here each
+kernel reads every operand once: per path the CG products of Y and of B are formed side by side, and
+the weights W and C are streamed together, where composing the first-order kernels would make three
+passes over the weight-sized tensors for each group.
+
+Work decomposition is that of the first-order kernels (lane = channel, a wave or a group of chunk
+waves per row / per receiver node, register-resident accumulators over a node's edges, per-edge dX
+terms reduced by the sender-ordered second pass). Per-row weights only.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+from .common import Src
+from .lower import Lowered, Path
+from .uvu import UvuEmitter
+
+
+def supported(low: Lowered) -> bool:
+    return low.mode == "uvu" and not low.shared_weights
+
+
+class DoubleEmitter(UvuEmitter):
+    """Adds ``double_backward_a`` / ``double_backward_b`` (batch and convolution flavours) to a module
+    whose structs (X_t, G_t) the base emitter has already written."""
+
+    # ------------------------------------------------------------ operands
+    def _y_of(self, row: str):
+        def y(p: Path, v: str, j: int) -> str:
+            return f"{row}[{self._y_index(self.low.in2[p.i2], v, j)}]"
+        return y
+
+    def _w_of(self, row: str):
+        low = self.low
+
+        def w(p: Path, v: str) -> str:
+            mul = low.in1[p.i1].mul
+            wp = self._ptr(row, (f"{p.woff} + ({v})", low.in2[p.i2].mul), mul)
+            ld = f"__builtin_nontemporal_load({wp})" if self.nt & 1 else f"*{wp}"
+            return self._val(mul, ld)
+        return w
+
+    def _two_products(self, s: Src, p: Path, v: str) -> Dict[int, Tuple[str, str, bool]]:
+        """|c| * y_j and |c| * b_j for the distinct (|c|, j) of a path: nnz index -> (qy, qb, negative)."""
+        yacc, bacc = self._y_of("yrow"), self._y_of("brow")
+        for j in sorted({j for _, j, _, _ in p.nnz}):
+            s(f"const T y{j} = {yacc(p, v, j)};")
+            s(f"const T b{j} = {bacc(p, v, j)};")
+        names: Dict[Tuple[str, int], int] = {}
+        out = {}
+        for n, (i, j, k, c) in enumerate(p.nnz):
+            key = (self.lit(abs(c)), j)
+            if key not in names:
+                names[key] = len(names)
+                s(f"const T q{names[key]} = T({key[0]}) * y{j};")
+                s(f"const T r{names[key]} = T({key[0]}) * b{j};")
+            out[n] = (f"q{names[key]}", f"r{names[key]}", c < 0)
+        return out
+
+    # ------------------------------------------------------------ kernel A cores
+    def emit_double_cores(self, s: Src):
+        """dda_seg<i>: adds one row's / one edge's three forward terms to the accumulators of segment i."""
+        low = self.low
+
+        def emit():
+            for si, seg in enumerate(self.segments):
+                s.open(
+                    f"OEQ_DEV void dda_seg{si}{self._sfx()}(const X_t& x, const X_t& xa, const T* __restrict__ yrow, "
+                    "const T* __restrict__ brow, const T* __restrict__ wrow, const T* __restrict__ crow, "
+                    f"const int u, D{si}_t& a)"
+                )
+                wacc, cacc = self._w_of("wrow"), self._w_of("crow")
+                for p in self._paths():
+                    if p.io not in seg:
+                        continue
+                    s(f"// path {p.index}")
+
+                    def body(v, p=p):
+                        prods = self._two_products(s, p, v)
+                        started = set()
+                        for n, (i, j, k, c) in enumerate(p.nnz):
+                            qy, qb, neg = prods[n]
+                            xi, ai = f"x.b{p.i1}[{i}]", f"xa.b{p.i1}[{i}]"
+                            sign = "-" if neg else ""
+                            if k not in started:
+                                s(f"T t{k} = {sign}{qy} * {ai}; T s{k} = {sign}{qy} * {xi};")
+                                started.add(k)
+                            else:
+                                op = "-=" if neg else "+="
+                                s(f"t{k} {op} {qy} * {ai}; s{k} {op} {qy} * {xi};")
+                            s(f"t{k} {'-=' if neg else '+='} {qb} * {xi};")
+                        s(f"const T wv = {wacc(p, v)};")
+                        s(f"const T cv = {cacc(p, v)};")
+                        for k in sorted(started):
+                            s(f"a.o{p.io}[{k}] += wv * t{k} + cv * s{k};")
+
+                    self._for_v(s, p, body)
+                s.close()
+
+        self._per_chunk(s, emit, in_kernel=False)
+
+    # ------------------------------------------------------------ kernel B paths
+    def _ddb_paths(self, s: Src, g_on_demand_row: Optional[str], fence: bool, deferred: bool,
+                   dw_guard: Optional[str]):
+        """Straight-line second-order backward of all paths. In scope: x, xa (X_t), dx (X_t), dy[],
+        yrow, brow, wrow, crow, dwrow, u, and gr (G_t) or the row pointer named ``g_on_demand_row``."""
+        low = self.low
+        wacc, cacc = self._w_of("wrow"), self._w_of("crow")
+        ordered = sorted(self._paths(), key=lambda q: (q.io, q.index))
+        since_fence = 0
+        for n_path, p in enumerate(ordered):
+            b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
+            V = b2.mul
+            s(f"// path {p.index}")
+            s.open("")
+            if g_on_demand_row is not None:
+                s(f"T gk[{bo.d}];")
+                s.open("")
+                base, st = self._lane_ptr(bo)
+                s(f"const T* gp = {self._ptr(g_on_demand_row, base, bo.mul)};")
+                for k in range(bo.d):
+                    s(f"gk[{k}] = {self._val(bo.mul, f'gp[{k * st}]')};")
+                s.close()
+                gname = lambda k: f"gk[{k}]"
+            else:
+                gname = lambda k, io=p.io: f"gr.o{io}[{k}]"
+            base_slot = self.wslot[p.index]
+
+            def body(v, p=p, b1=b1, b2=b2, V=V, gname=gname, base_slot=base_slot):
+                prods = self._two_products(s, p, v)
+                s(f"const T wv = {wacc(p, v)};")
+                s(f"const T cv = {cacc(p, v)};")
+                ks = sorted({k for _, _, k, _ in p.nnz})
+                js = sorted({j for _, j, _, _ in p.nnz})
+                for k in ks:
+                    s(f"const T gw{k} = {gname(k)} * wv; const T gc{k} = {gname(k)} * cv;")
+                # d/dX: (|c| b_j)(g_k w) + (|c| y_j)(g_k c)
+                for n, (i, j, k, c) in enumerate(p.nnz):
+                    qy, qb, neg = prods[n]
+                    op = "-=" if neg else "+="
+                    s(f"dx.b{p.i1}[{i}] {op} {qb} * gw{k}; dx.b{p.i1}[{i}] {op} {qy} * gc{k};")
+                # h_j = sum_ik c x_i g_k, ha_j = sum_ik c a_i g_k
+                pair, hstart = {}, set()
+                for n, (i, j, k, c) in enumerate(p.nnz):
+                    if (i, k) not in pair:
+                        pair[(i, k)] = len(pair)
+                        s(f"const T xg{pair[(i, k)]} = x.b{p.i1}[{i}] * {gname(k)}; "
+                          f"const T ag{pair[(i, k)]} = xa.b{p.i1}[{i}] * {gname(k)};")
+                    m = pair[(i, k)]
+                    if j not in hstart:
+                        s(f"T h{j} = T({self.lit(c)}) * xg{m}; T ha{j} = T({self.lit(c)}) * ag{m};")
+                        hstart.add(j)
+                    else:
+                        s(f"h{j} += T({self.lit(c)}) * xg{m}; ha{j} += T({self.lit(c)}) * ag{m};")
+                # d/dW = sum_j b_j h_j + y_j ha_j ; d/dY_j = c h_j + w ha_j
+                s(f"T dwv = b{js[0]} * h{js[0]};")
+                s(f"dwv += y{js[0]} * ha{js[0]};")
+                for j in js[1:]:
+                    s(f"dwv += b{j} * h{j}; dwv += y{j} * ha{j};")
+                if deferred:
+                    s(f"dwkeep[{base_slot} + {v}] = dwv;")
+                else:
+                    dwp = self._ptr("dwrow", (f"{p.woff} + ({v})", V))
+                    st = (f"__builtin_nontemporal_store(dwv, {dwp});" if self.nt & 2 else f"*{dwp} = dwv;")
+                    cond = self._store_cond(b1.mul, dw_guard)
+                    s(f"if ({cond}) {st}" if cond else st)
+                for j in js:
+                    s(f"dy[{self._y_index(b2, v, j)}] += cv * h{j}; dy[{self._y_index(b2, v, j)}] += wv * ha{j};")
+
+            self._for_v(s, p, body)
+            s.close()
+            if fence and g_on_demand_row is not None:
+                since_fence += bo.d * self.words
+                nxt = ordered[n_path + 1] if n_path + 1 < len(ordered) else None
+                if nxt is None or since_fence + low.out[nxt.io].d * self.words > self.fence_words:
+                    s("__builtin_amdgcn_sched_barrier(0);")
+                    since_fence = 0
+
+    def double_b_resident(self) -> bool:
+        """The row's / node's output-gradient slice stays in registers beside X, A, dX and dY."""
+        low = self.low
+        x = sum(low.in1[b].d for b in self.used_in1)
+        g = sum(low.out[io].d for io in self.used_out)
+        return self.words * (g + 3 * x + self.l2_pad) + 48 <= 232
+
+    # ------------------------------------------------------------ batch kernels
+    def emit_tp_double_a(self, s: Src, G: int, waves_per_eu: int = 0):
+        low = self.low
+        block = 64 * self.NCH * G
+        s.open(
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_a(i64 num_batch, '
+            "const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
+            "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
+            "T* __restrict__ L3_dgrad)"
+        )
+        self._lane_prologue(s)
+        if self.tr_stores & 1 and self.R == 1:
+            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(b.d for b in low.out)}];")
+        s(f"const i64 ngroups = (num_batch + {self.R - 1}) / {self.R};")
+        s.open(f"for (i64 grp = (i64)blockIdx.x * {G} + g; grp < ngroups; grp += (i64)gridDim.x * {G})")
+        s(f"const i64 row = grp * {self.R} + r;")
+        s("const bool live = row < num_batch;")
+        s("const i64 rowc = live ? row : num_batch - 1;")
+        s(f"const T* xrow = L1_in + rowc * {low.L1};")
+        s(f"const T* arow = L1_dgrad + rowc * {low.L1};")
+        s(f"const T* yrow = L2_in + rowc * {low.L2};")
+        s(f"const T* brow = L2_dgrad + rowc * {low.L2};")
+        s(f"const T* wrow = W + rowc * {low.WN};")
+        s(f"const T* crow = W_dgrad + rowc * {low.WN};")
+        s(f"T* zrow = L3_dgrad + rowc * {low.L3};")
+        live = "live"
+        if self.R == 1:
+            s.open("if (live)")
+            live = "true"
+
+        def row_body():
+            s("X_t x, xa;")
+            self._load_x(s, "xrow", self.used_in1)
+            self._load_x(s, "arow", self.used_in1, "xa")
+            for si in range(len(self.segments)):
+                if self.cur_chunk is not None and not self._out_of(self.segments[si]):
+                    continue
+                s.open("")
+                s(f"D{si}_t a; zero_dseg{si}(a);")
+                s(f"dda_seg{si}{self._sfx()}(x, xa, yrow, brow, wrow, crow, u, a);")
+                self._store_seg(s, si, "zrow", live)
+                s.close()
+
+        self._per_chunk(s, row_body)
+        self._zero_untouched_out(s, "zrow", live)
+        if self.R == 1:
+            s.close()
+        s.close()
+        s.close()
+        return block
+
+    def emit_tp_double_b(self, s: Src, G: int, waves_per_eu: int = 0):
+        low = self.low
+        if self.NCH > 1:
+            G = 1  # the dY reduction across chunk waves uses block barriers
+        block = 64 * self.NCH * G
+        s.open(
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_b(i64 num_batch, '
+            "const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
+            "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
+            "const T* __restrict__ L3_grad, T* __restrict__ L1_grad, T* __restrict__ L2_grad, T* __restrict__ W_grad)"
+        )
+        self._lane_prologue(s)
+        if self.NCH > 1:
+            s(f"__shared__ T s_dy[{G}][{self.NCH}][{self.l2_pad}];")
+        if self.tr_stores & 2 and self.R == 1:
+            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(b.d for b in low.in1)}];")
+        s(f"const i64 ngroups = (num_batch + {self.R - 1}) / {self.R};")
+        s.open(f"for (i64 base = (i64)blockIdx.x * {G}; base < ngroups; base += (i64)gridDim.x * {G})")
+        s("const i64 grp = base + g;")
+        s(f"const i64 row = grp * {self.R} + r;")
+        s("const bool live = row < num_batch;")
+        s("const i64 rowc = live ? row : num_batch - 1;")
+        s(f"const T* xrow = L1_in + rowc * {low.L1};")
+        s(f"const T* arow = L1_dgrad + rowc * {low.L1};")
+        s(f"const T* yrow = L2_in + rowc * {low.L2};")
+        s(f"const T* brow = L2_dgrad + rowc * {low.L2};")
+        s(f"const T* wrow = W + rowc * {low.WN};")
+        s(f"const T* crow = W_dgrad + rowc * {low.WN};")
+        s(f"const T* grow = L3_grad + rowc * {low.L3};")
+        s(f"T* dwrow = W_grad + rowc * {low.WN};")
+        live = "live"
+        if self.R == 1:
+            s.open("if (live)")
+            live = "true"
+        resident = self.double_b_resident()
+
+        def row_body():
+            s("X_t x, xa, dx;")
+            self._load_x(s, "xrow", self.used_in1)
+            self._load_x(s, "arow", self.used_in1, "xa")
+            self._zero_x(s, "dx")
+            s(f"T dy[{self.l2_pad}];")
+            s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+            deferred = self._dw_deferred(live)
+            if deferred:
+                s(f"T dwkeep[{self.n_wslots}];")
+            if resident:
+                s("G_t gr;")
+                self._load_g(s, "grow", self.used_out)
+                self._ddb_paths(s, None, False, deferred, live)
+            else:
+                self._ddb_paths(s, "grow", True, deferred, live)
+            self._pin_gradients(s, self.used_in1, deferred)
+            if deferred:
+                self._flush_dwkeep(s, live)
+            s(f"T* dxrow = L1_grad + rowc * {low.L1};")
+            self._store_dx(s, "dxrow", live, nt=bool(self.nt & 2))
+            self._zero_untouched_in1(s, "dxrow", live)
+            self._dy_finish(s, f"L2_grad + rowc * {low.L2}", live)
+
+        self._per_chunk(s, row_body)
+        if self.R == 1:
+            s.close()
+        s.close()
+        s.close()
+        return block
+
+    # ------------------------------------------------------------ convolution kernels
+    _CONV_OPERANDS = (
+        "const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
+        "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
+    )
+
+    def _edge_rows(self, s: Src, e: str):
+        low = self.low
+        s(f"const i64 eid = OEQ_EDGE({e});")
+        s("const i64 sender = cols[eid];")
+        s(f"const T* xrow = L1_in + sender * {low.L1};")
+        s(f"const T* arow = L1_dgrad + sender * {low.L1};")
+        s(f"const T* yrow = L2_in + eid * {low.L2};")
+        s(f"const T* brow = L2_dgrad + eid * {low.L2};")
+        s(f"const T* wrow = W + eid * {low.WN};")
+        s(f"const T* crow = W_dgrad + eid * {low.WN};")
+
+    def emit_conv_double_a(self, s: Src, G: int, waves_per_eu: int = 0, xcd: int = 1):
+        """Receiver-major walk: the node's accumulators stay in registers over its edges."""
+        low = self.low
+        block = 64 * self.NCH * G
+        s.open(
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_a(i64 node_count, '
+            f"i64 nnz, {self._CONV_OPERANDS}T* __restrict__ L3_dgrad, const i64* __restrict__ rows, "
+            "const i64* __restrict__ cols, const i64* __restrict__ rowptr, const i64* __restrict__ eperm)"
+        )
+        self._lane_prologue(s)
+        if self.tr_stores & 1 and self.R == 1:
+            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.out[io].d for io in self.used_out)}];")
+        self._node_loop_open(s, G, xcd)
+        s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+        s(f"T* zrow = L3_dgrad + node * {low.L3};")
+        for si in range(len(self.segments)):
+            s.open("")
+
+            def node_body(si=si):
+                if self.cur_chunk is not None and not self._out_of(self.segments[si]):
+                    return
+                s(f"D{si}_t a; zero_dseg{si}(a);")
+                s.open(f"for (i64 e = e0 + r; e < e1; e += {self.R})")
+                self._edge_rows(s, "e")
+                s("X_t x, xa;")
+                self._load_x(s, "xrow", self.seg_in1[si])
+                self._load_x(s, "arow", self.seg_in1[si], "xa")
+                s(f"dda_seg{si}{self._sfx()}(x, xa, yrow, brow, wrow, crow, u, a);")
+                s.close()
+                if self.R > 1:
+                    for io in self.segments[si]:
+                        for k in range(low.out[io].d):
+                            m = self.LPR
+                            while m < 64:
+                                s(f"a.o{io}[{k}] += __shfl_xor(a.o{io}[{k}], {m});")
+                                m *= 2
+                self._store_seg(s, si, "zrow", "r == 0" if self.R > 1 else "true")
+
+            self._per_chunk(s, node_body)
+            s.close()
+        self._zero_untouched_out(s, "zrow", "r == 0")
+        s.close()
+        s.close()
+        return block
+
+    def emit_conv_double_b(self, s: Src, G: int, waves_per_eu: int = 0, xcd: int = 1):
+        """Receiver-major walk with the node's output-gradient slice in registers (when it fits); the
+        per-edge d/dX terms go to ``dx_tmp`` for the sender-ordered reduction, as in the first-order
+        backward kernel."""
+        low = self.low
+        if self.NCH > 1:
+            G = 1
+        block = 64 * self.NCH * G
+        s.open(
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_b(i64 node_count, '
+            f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
+            "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
+            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm)"
+        )
+        self._lane_prologue(s)
+        if self.NCH > 1:
+            s(f"__shared__ T s_dy[{G}][{self.NCH}][{self.l2_pad}];")
+        if self.tr_stores & 2 and self.R == 1:
+            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.in1[b].d for b in self.used_in1)}];")
+        resident = self.double_b_resident()
+        self._node_loop_open(s, G, xcd)
+        s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+
+        def node_body():
+            if resident:
+                s("G_t gr;")
+                self._load_g(s, f"L3_grad + node * {low.L3}", self.used_out)
+            # with more than one chunk every wave of the block walks the same edges: the block barriers
+            # of the dY reduction are reached uniformly
+            s.open(f"for (i64 e = e0 + r; e < e1; e += {self.R})")
+            self._edge_rows(s, "e")
+            s(f"T* dwrow = W_grad + eid * {low.WN};")
+            s("X_t x, xa, dx;")
+            self._load_x(s, "xrow", self.used_in1)
+            self._load_x(s, "arow", self.used_in1, "xa")
+            self._zero_x(s, "dx")
+            s(f"T dy[{self.l2_pad}];")
+            s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+            deferred = self._dw_deferred(None)
+            if deferred:
+                s(f"T dwkeep[{self.n_wslots}];")
+            if resident:
+                self._ddb_paths(s, None, False, deferred, None)
+            else:
+                s(f"const T* grow = L3_grad + node * {low.L3};")
+                # without this the compiler hoists the loads of the node's gradient row out of the edge
+                # loop, i.e. makes it register resident after all
+                s(f'asm volatile("" : "+{"s" if self.R == 1 else "v"}"(grow));')
+                self._ddb_paths(s, "grow", True, deferred, None)
+            self._pin_gradients(s, self.used_in1, deferred)
+            if deferred:
+                self._flush_dwkeep(s, None)
+            s(f"T* dxrow = dx_tmp + eid * {low.L1};")
+            self._store_dx(s, "dxrow", "true", nt=bool(self.nt & 2))
+            self._zero_untouched_in1(s, "dxrow", "true")
+            self._dy_finish(s, f"L2_grad + eid * {low.L2}", "true")
+            s.close()
+
+        self._per_chunk(s, node_body)
+        s.close()
+        s.close()
+        return block
+
+
+def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict) -> List[tuple]:
+    """Append the batch double-backward kernels to a module; returns their launch descriptors."""
+    from .. import runtime as rt
+
+    em = DoubleEmitter(low, acc_budget_words=64)
+    em.nt = base.nt
+    em.tr_stores = base.tr_stores
+    em.fence_words = 48
+    # the accumulator structs of this emitter's (smaller) segments
+    _emit_segment_structs(s, em, "D")
+    em.emit_double_cores(s)
+    wide = low.n_chunks > 1
+    G = 1 if wide else 4
+    blk_a = em.emit_tp_double_a(s, G, tune.get("dd_wa", 2))
+    blk_b = em.emit_tp_double_b(s, G, tune.get("dd_wb", 2))
+    G_b = 1 if em.NCH > 1 else G
+    return [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_a", blk_a, G * em.R, 0),
+            (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_b", blk_b, G_b * em.R, 0)]
+
+
+def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: int) -> List[tuple]:
+    """Append the convolution double-backward kernels (receiver-major walk) to a module."""
+    from .. import runtime as rt
+
+    em = DoubleEmitter(low, acc_budget_words=tune.get("dd_acc", 112))
+    em.nt = base.nt
+    em.tr_stores = base.tr_stores
+    em.fence_words = 0
+    _emit_segment_structs(s, em, "D")
+    em.emit_double_cores(s)
+    G = max(1, tune.get("dd_g", 2) // em.NCH) if em.R == 1 else 4
+    blk_a = em.emit_conv_double_a(s, G, tune.get("dd_wa", 2), xcd)
+    blk_b = em.emit_conv_double_b(s, G, tune.get("dd_wb", 2), xcd)
+    G_b = 1 if em.NCH > 1 else G
+    return [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_a", blk_a, G, 0, xcd),
+            (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_b", blk_b, G_b, 0, xcd)]
+
+
+def _emit_segment_structs(s: Src, em: DoubleEmitter, prefix: str):
+    """This emitter's output segments can differ from the first-order kernels': its accumulator
+    structs get their own names (D<i>_t, zero_dseg<i>)."""
+    low = em.low
+    for si, seg in enumerate(em.segments):
+        s(f"struct {prefix}{si}_t {{")
+        for io in seg:
+            s(f"    T o{io}[{low.out[io].d}];")
+        s("};")
+        s.open(f"OEQ_DEV void zero_{prefix.lower()}seg{si}({prefix}{si}_t& a)")
+        for io in seg:
+            for k in range(low.out[io].d):
+                s(f"a.o{io}[{k}] = T(0);")
+        s.close()

@@ -454,6 +454,47 @@ size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_coun
     return 3 * ptr_bytes_of(node_count) + 3 * perm_bytes_of(nnz) + tmp_bytes;
 }
 
+// What the walk kernels of a backward-type call need besides the operands: CSR pointers over receivers and
+// over senders, the walk orders (GROUPED mode: built here; SORTED mode: the caller's lists), and the
+// buffer of per-edge dX terms. Everything lives in the caller's workspace (layouts above).
+struct WalkIndex {
+    int64_t *rowptr = nullptr, *colptr = nullptr, *rperm = nullptr;
+    const int64_t* sperm = nullptr;
+    void* dx_tmp = nullptr;
+};
+
+static int walk_index(oeq_kernels* k, const char* who, int64_t node_count, int64_t nnz, const int64_t* rows,
+                      const int64_t* cols, const int64_t* transpose_perm, void* workspace, size_t workspace_bytes,
+                      void* stream, WalkIndex* ix) {
+    const int mode = k->dims.deterministic;
+    if (mode == OEQ_CONV_SORTED && !transpose_perm)
+        return fail(OEQ_ERR_INVALID, "%s: deterministic mode needs transpose_perm", who);
+    size_t need = oeq_conv_backward_workspace_bytes(k, node_count, nnz);
+    if (!workspace || workspace_bytes < need)
+        return fail(OEQ_ERR_INVALID, "%s: workspace too small (%zu < %zu bytes)", who, workspace_bytes, need);
+    const size_t pb = ptr_bytes_of(node_count), qb = perm_bytes_of(nnz);
+    ix->rowptr = (int64_t*)workspace;
+    ix->colptr = (int64_t*)((char*)workspace + pb);
+    ix->sperm = transpose_perm;
+    int rc;
+    if (mode == OEQ_CONV_SORTED) {
+        ix->dx_tmp = (char*)workspace + 2 * pb;
+        rc = k->segment_ptr(nnz, node_count, rows, nullptr, ix->rowptr, stream);
+        if (rc) return rc;
+        return k->segment_ptr(nnz, node_count, cols, transpose_perm, ix->colptr, stream);
+    }
+    int64_t* cursor = (int64_t*)((char*)workspace + 2 * pb);
+    ix->rperm = (int64_t*)((char*)workspace + 3 * pb);
+    int64_t* sp = (int64_t*)((char*)workspace + 3 * pb + qb);
+    int64_t* scratch = (int64_t*)((char*)workspace + 3 * pb + 2 * qb);
+    ix->dx_tmp = (char*)workspace + 3 * pb + 3 * qb;
+    rc = k->group_by_key(nnz, node_count, rows, ix->rowptr, cursor, scratch, ix->rperm, stream);
+    if (rc) return rc;
+    rc = k->group_by_key(nnz, node_count, cols, ix->colptr, cursor, scratch, sp, stream);
+    ix->sperm = sp;
+    return rc;
+}
+
 int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
                      const void* W, void* L3_out, const int64_t* rows, const int64_t* cols, void* workspace,
                      size_t workspace_bytes, void* stream) {
@@ -520,33 +561,11 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
     void *dx_tmp = nullptr, *wpartial = nullptr;
     const int mode = k->dims.deterministic;
     if (mode != OEQ_CONV_ATOMIC) {
-        if (mode == OEQ_CONV_SORTED && !transpose_perm)
-            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: deterministic mode needs transpose_perm");
-        size_t need = oeq_conv_backward_workspace_bytes(k, node_count, nnz);
-        if (!workspace || workspace_bytes < need)
-            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: workspace too small (%zu < %zu bytes)", workspace_bytes,
-                        need);
-        const size_t pb = ptr_bytes_of(node_count), qb = perm_bytes_of(nnz);
-        rowptr = (int64_t*)workspace;
-        colptr = (int64_t*)((char*)workspace + pb);
-        if (mode == OEQ_CONV_SORTED) {
-            dx_tmp = (char*)workspace + 2 * pb;
-            rc = k->segment_ptr(nnz, node_count, rows, nullptr, rowptr, stream);
-            if (rc) return rc;
-            rc = k->segment_ptr(nnz, node_count, cols, transpose_perm, colptr, stream);
-            if (rc) return rc;
-        } else {
-            int64_t* cursor = (int64_t*)((char*)workspace + 2 * pb);
-            rperm = (int64_t*)((char*)workspace + 3 * pb);
-            int64_t* sp = (int64_t*)((char*)workspace + 3 * pb + qb);
-            int64_t* scratch = (int64_t*)((char*)workspace + 3 * pb + 2 * qb);
-            dx_tmp = (char*)workspace + 3 * pb + 3 * qb;
-            rc = k->group_by_key(nnz, node_count, rows, rowptr, cursor, scratch, rperm, stream);
-            if (rc) return rc;
-            rc = k->group_by_key(nnz, node_count, cols, colptr, cursor, scratch, sp, stream);
-            if (rc) return rc;
-            sperm = sp;
-        }
+        WalkIndex ix;
+        rc = walk_index(k, "oeq_conv_backward", node_count, nnz, rows, cols, transpose_perm, workspace,
+                        workspace_bytes, stream, &ix);
+        if (rc) return rc;
+        rowptr = ix.rowptr, colptr = ix.colptr, rperm = ix.rperm, sperm = ix.sperm, dx_tmp = ix.dx_tmp;
         if (wrows)
             wpartial = (char*)dx_tmp + align_up((size_t)nnz * (size_t)k->dims.L1_dim * es, 256);
     } else {
@@ -564,6 +583,68 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
     int64_t wn = k->dims.weight_numel;
     void* rargs[] = {&n_partials, &wpartial, &W_grad, &wn};
     return k->launch(OEQ_ROLE_TP_BACKWARD_WREDUCE, wn, rargs, stream);
+}
+
+// ---------------------------------------------------------------------------
+// second-order kernels
+// ---------------------------------------------------------------------------
+
+int oeq_has_double_backward(const oeq_kernels* k) {
+    return k && k->roles[OEQ_ROLE_DOUBLE_BACKWARD_A].present && k->roles[OEQ_ROLE_DOUBLE_BACKWARD_B].present;
+}
+
+int oeq_tp_double_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in, const void* L2_in, const void* W,
+                           const void* L3_grad, const void* L1_dgrad, const void* L2_dgrad, const void* W_dgrad,
+                           void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: NULL kernel set");
+    if (!oeq_has_double_backward(k))
+        return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: this kernel set has no second-order kernels");
+    if (num_batch < 0) return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: negative batch");
+    if (num_batch == 0) return OEQ_OK;
+    if (!L1_in || !L2_in || !W || !L3_grad || !L1_dgrad || !L2_dgrad || !W_dgrad || !L1_grad || !L2_grad || !W_grad ||
+        !L3_dgrad)
+        return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: NULL buffer");
+    void* a[] = {&num_batch, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_dgrad};
+    int rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_A, num_batch, a, stream);
+    if (rc) return rc;
+    void* b[] = {&num_batch, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_grad, &L1_grad, &L2_grad, &W_grad};
+    return k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, num_batch, b, stream);
+}
+
+int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
+                             const void* W, const void* L3_grad, const void* L1_dgrad, const void* L2_dgrad,
+                             const void* W_dgrad, void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad,
+                             const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL kernel set");
+    if (!oeq_has_double_backward(k) || k->dims.deterministic == OEQ_CONV_ATOMIC)
+        return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: this kernel set has no second-order kernels");
+    if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: negative size");
+    if (node_count == 0) return OEQ_OK;
+    if (!L1_grad || !L3_dgrad) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL output");
+    const size_t es = (size_t)k->dims.elem_size;
+    if (nnz == 0) {
+        int rc = k->fill_zero(L1_grad, (size_t)node_count * k->dims.L1_dim * es, stream);
+        if (rc) return rc;
+        return k->fill_zero(L3_dgrad, (size_t)node_count * k->dims.L3_dim * es, stream);
+    }
+    if (!L1_in || !L2_in || !W || !L3_grad || !L1_dgrad || !L2_dgrad || !W_dgrad || !L2_grad || !W_grad || !rows ||
+        !cols)
+        return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL buffer");
+    WalkIndex ix;
+    int rc = walk_index(k, "oeq_conv_double_backward", node_count, nnz, rows, cols, transpose_perm, workspace,
+                        workspace_bytes, stream, &ix);
+    if (rc) return rc;
+    void* a[] = {&node_count, &nnz, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_dgrad,
+                 &rows,       &cols, &ix.rowptr, &ix.rperm};
+    rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_A, node_count, a, stream);
+    if (rc) return rc;
+    void* b[] = {&node_count, &nnz,     &L1_in,  &L1_dgrad, &L2_in, &L2_dgrad,  &W,         &W_dgrad,
+                 &L3_grad,    &L2_grad, &W_grad, &rows,     &cols,  &ix.rowptr, &ix.dx_tmp, &ix.rperm};
+    rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count, b, stream);
+    if (rc) return rc;
+    void* fargs[] = {&node_count, &nnz, &ix.dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};
+    return k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
 }
 
 }  // extern "C"

@@ -47,6 +47,8 @@ ROLE_GROUP_COUNT = 9
 ROLE_GROUP_SCAN = 10
 ROLE_GROUP_SCATTER = 11
 ROLE_GROUP_ORDER = 12
+ROLE_DOUBLE_BACKWARD_A = 13
+ROLE_DOUBLE_BACKWARD_B = 14
 
 CONV_ATOMIC, CONV_SORTED, CONV_GROUPED = 0, 1, 2
 
@@ -129,6 +131,9 @@ EXPORTS = {
     "oeq_conv_forward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_backward": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_conv_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_has_double_backward": (ctypes.c_int, [_P]),
+    "oeq_tp_double_backward": (ctypes.c_int, [_P, _I64] + [_P] * 12),
+    "oeq_conv_double_backward": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 15 + [_SZ, _P]),
     "oeq_segment_sum": (ctypes.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_segment_sum_workspace_bytes": (_SZ, [_P, _I64]),
     "oeq_grouped_sum": (ctypes.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _P, _SZ, _P]),
@@ -291,6 +296,18 @@ class KernelSet:
     def conv_forward(self, nodes, nnz, x, y, w, out, rows, cols, ws, ws_bytes, stream):
         _check(self._lib.oeq_conv_forward(self.handle, nodes, nnz, x, y, w, out, rows, cols, ws, ws_bytes, stream),
                "oeq_conv_forward")
+
+    def has_double_backward(self) -> bool:
+        return bool(self._lib.oeq_has_double_backward(self.handle))
+
+    def tp_double_backward(self, n, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg, stream):
+        _check(self._lib.oeq_tp_double_backward(self.handle, n, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg, stream),
+               "oeq_tp_double_backward")
+
+    def conv_double_backward(self, nodes, nnz, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg, rows, cols, perm, ws,
+                             ws_bytes, stream):
+        _check(self._lib.oeq_conv_double_backward(self.handle, nodes, nnz, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg,
+                                                  rows, cols, perm, ws, ws_bytes, stream), "oeq_conv_double_backward")
 
     def conv_backward(self, nodes, nnz, x, dx, y, dy, w, dw, g, rows, cols, perm, ws, ws_bytes, stream):
         _check(self._lib.oeq_conv_backward(self.handle, nodes, nnz, x, dx, y, dy, w, dw, g, rows, cols, perm, ws,

@@ -1,0 +1,173 @@
+"""The fused second-order kernels (`double_backward_a` / `double_backward_b`) against the composition of
+first-order kernels, which tests/test_higher_derivatives_gpu.py checks against float64 autograd through the
+CPU restatement. Also through autograd: the force-training pattern (gradient of a function of the first
+gradients) with the fused route switched on and off."""
+
+import numpy as np
+import pytest
+import torch
+
+import openequivariance_amd as oeq
+from openequivariance_amd._torch import ops
+from openequivariance_amd.core import problems as P
+from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
+from oracle import e3nn_ref as R
+from gpu_util import tol_of
+
+pytestmark = pytest.mark.gpu
+
+
+def _f64(problem):
+    q = problem.clone()
+    q.irrep_dtype, q.weight_dtype = np.float64, np.float64
+    return q
+
+
+def _ir_mul(problem):
+    q = problem.clone()
+    q.layout = "ir_mul"
+    return q
+
+
+def _odd():
+    # packed rows (5 channels), mul2 > 1, a block no instruction reads and one no instruction writes
+    return oeq.TPProblem("5x1e+3x2e+2x0e", "2x1e+1x0e", "5x1e+3x2e+5x0e+4x1o",
+                         [(0, 0, 0, "uvu", True), (0, 1, 0, "uvu", True), (1, 0, 1, "uvu", True),
+                          (0, 0, 2, "uvu", True)], shared_weights=False, internal_weights=False)
+
+
+CASES = [
+    ("cfg1", P.config1_single_uvu, 1000),
+    ("odd", _odd, 333),
+    ("odd-f64", lambda: _f64(_odd()), 333),
+    ("cfg2", P.config2_nequip_uvu, 257),
+    ("cfg2-f64", lambda: _f64(P.config2_nequip_uvu()), 129),
+    ("cfg2-ir_mul", lambda: _ir_mul(P.config2_nequip_uvu()), 129),
+    ("cfg3", P.config3_mace_uvu, 67),
+    ("cfg3-f64", lambda: _f64(P.config3_mace_uvu()), 33),
+    ("lips", lambda: P.nequip_problems()[0], 129),
+    ("benzene", lambda: P.nequip_problems()[3], 33),
+    ("nequix-first", lambda: P.nequix_problems()[0], 65),
+    ("sevennet-main", lambda: P.seven_net_problems()[1], 65),
+    ("mace-large-ir_mul", lambda: _ir_mul(P.mace_problems()[0]), 33),
+]
+
+
+def _rand(rng, shape, dt):
+    return torch.tensor(rng.uniform(-1, 1, size=shape).astype(dt), device="cuda")
+
+
+def _check(names, fused, composed, tol):
+    for name, a, b in zip(names, fused, composed):
+        e = R.normalized_error(a.cpu().numpy(), b.cpu().numpy())
+        assert e <= tol, (name, e)
+
+
+@pytest.mark.parametrize("name,make,batch", CASES, ids=[c[0] for c in CASES])
+def test_tp_fused_matches_composition(name, make, batch):
+    problem = make()
+    tp = oeq.TensorProduct(problem)
+    e = ops.get_entry(tp.kid)
+    assert e.kernels().has_double_backward()
+    dt = np.dtype(problem.irrep_dtype)
+    rng = np.random.default_rng(5)
+    x, a = (_rand(rng, (batch, e.L1), dt) for _ in range(2))
+    y, b = (_rand(rng, (batch, e.L2), dt) for _ in range(2))
+    w, c = (_rand(rng, (batch, e.WN), dt) for _ in range(2))
+    g = _rand(rng, (batch, e.L3), dt)
+    fused = ops.tp_double_backward(x, y, w, g, a, b, c, tp.kid)
+    composed = ops._second_order(lambda p, q, r: ops.tp_forward(p, q, r, tp.kid),
+                                 lambda p, q, r, s: ops.tp_backward(p, q, r, s, tp.kid), x, y, w, g, a, b, c)
+    _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
+
+
+def _graph(n=60):
+    coords, rows, cols, _ = periodic_radius_graph(n, 8.0, 3.2, seed=3)
+    return CoordGraph(coords, rows, cols)
+
+
+CONV_CASES = [c for c in CASES if c[0] not in ("cfg1",)] + [("cfg1", P.config1_single_uvu, 0)]
+
+
+@pytest.mark.parametrize("det", [True, False], ids=["sorted", "grouped"])
+@pytest.mark.parametrize("name,make,batch", CONV_CASES, ids=[c[0] for c in CONV_CASES])
+def test_conv_fused_matches_composition(name, make, batch, det):
+    problem = make()
+    gph = _graph()
+    n, E = gph.coords.shape[0], gph.nnz
+    conv = oeq.TensorProductConv(problem, deterministic=det)
+    e = ops.get_entry(conv.kid)
+    assert e.kernels().has_double_backward()
+    dt = np.dtype(problem.irrep_dtype)
+    rng = np.random.default_rng(6)
+    if det:
+        rows, cols, perm = gph.rows, gph.cols, gph.transpose_perm
+    else:
+        order = rng.permutation(E)
+        rows, cols, perm = gph.rows[order], gph.cols[order], np.zeros(0, np.int64)
+    tr, tc, tp = (torch.tensor(v, device="cuda") for v in (rows, cols, perm))
+    x, a = (_rand(rng, (n, e.L1), dt) for _ in range(2))
+    y, b = (_rand(rng, (E, e.L2), dt) for _ in range(2))
+    w, c = (_rand(rng, (E, e.WN), dt) for _ in range(2))
+    g = _rand(rng, (n, e.L3), dt)
+    fused = ops.conv_double_backward(x, y, w, g, a, b, c, tr, tc, tp, conv.kid)
+    composed = ops._second_order(lambda p, q, r: ops.conv_forward(p, q, r, tr, tc, tp, conv.kid),
+                                 lambda p, q, r, s: ops.conv_backward(p, q, r, s, tr, tc, tp, conv.kid),
+                                 x, y, w, g, a, b, c)
+    _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
+
+
+def test_conv_fused_isolated_nodes_and_empty():
+    """Nodes without edges get zero rows; an empty edge list gives zero node gradients."""
+    problem = P.config2_nequip_uvu()
+    conv = oeq.TensorProductConv(problem, deterministic=True)
+    e = ops.get_entry(conv.kid)
+    rng = np.random.default_rng(7)
+    n = 9
+    rows = np.array([1, 1, 4, 4, 4, 7], np.int64)
+    cols = np.array([4, 7, 1, 4, 8, 1], np.int64)
+    perm = np.argsort(cols, kind="stable").astype(np.int64)
+    for E, (r_, c_, p_) in ((6, (rows, cols, perm)), (0, (rows[:0], cols[:0], perm[:0]))):
+        tr, tc, tp = (torch.tensor(v, device="cuda") for v in (r_, c_, p_))
+        x, a = (_rand(rng, (n, e.L1), np.float32) for _ in range(2))
+        y, b = (_rand(rng, (E, e.L2), np.float32) for _ in range(2))
+        w, c = (_rand(rng, (E, e.WN), np.float32) for _ in range(2))
+        g = _rand(rng, (n, e.L3), np.float32)
+        fused = ops.conv_double_backward(x, y, w, g, a, b, c, tr, tc, tp, conv.kid)
+        composed = ops._second_order(lambda p, q, r: ops.conv_forward(p, q, r, tr, tc, tp, conv.kid),
+                                     lambda p, q, r, s: ops.conv_backward(p, q, r, s, tr, tc, tp, conv.kid),
+                                     x, y, w, g, a, b, c)
+        if E:
+            _check(("dx", "dy", "dw", "gg"), fused, composed, 1e-5)
+            assert float(fused[3][0].abs().max()) == 0.0  # node 0 receives nothing
+        else:
+            assert float(fused[0].abs().max()) == 0.0 and float(fused[3].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("which", ["tp", "conv"])
+def test_force_training_pattern(which, monkeypatch):
+    """loss = f(first gradients); its gradient w.r.t. the inputs with the fused kernels equals the
+    one with the composed first-order kernels."""
+    problem = P.config2_nequip_uvu()
+    rng = np.random.default_rng(8)
+    gph = _graph(40)
+    n, E = gph.coords.shape[0], gph.nnz
+    if which == "tp":
+        mod = oeq.TensorProduct(problem)
+        rows_n, extra = E, ()
+    else:
+        mod = oeq.TensorProductConv(problem, deterministic=True)
+        rows_n, extra = n, tuple(torch.tensor(v, device="cuda") for v in (gph.rows, gph.cols, gph.transpose_perm))
+    e = ops.get_entry(mod.kid)
+    base = [_rand(rng, (rows_n, e.L1), np.float32), _rand(rng, (E, e.L2), np.float32),
+            _rand(rng, (E, e.WN), np.float32)]
+    g = _rand(rng, (rows_n, e.L3), np.float32)
+    results = []
+    for fused in (True, False):
+        monkeypatch.setattr(ops, "FUSED_DOUBLE_BACKWARD", fused)
+        ts = [t.clone().requires_grad_(True) for t in base]
+        z = mod(*ts, *extra)
+        first = torch.autograd.grad(z, ts, g, create_graph=True)
+        loss = sum((t ** 2).sum() for t in first)
+        results.append([t.detach() for t in torch.autograd.grad(loss, ts)])
+    _check(("x", "y", "w"), results[0], results[1], 1e-5)
