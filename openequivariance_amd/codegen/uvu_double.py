@@ -115,12 +115,12 @@ class DoubleEmitter(UvuEmitter):
 
     # ------------------------------------------------------------ kernel B paths
     def _ddb_paths(self, s: Src, g_on_demand_row: Optional[str], fence: bool, deferred: bool,
-                   dw_guard: Optional[str]):
+                   dw_guard: Optional[str], paths: Optional[List[Path]] = None):
         """Straight-line second-order backward of all paths. In scope: x, xa (X_t), dx (X_t), dy[],
         yrow, brow, wrow, crow, dwrow, u, and gr (G_t) or the row pointer named ``g_on_demand_row``."""
         low = self.low
         wacc, cacc = self._w_of("wrow"), self._w_of("crow")
-        ordered = sorted(self._paths(), key=lambda q: (q.io, q.index))
+        ordered = sorted(self._paths(paths), key=lambda q: (q.io, q.index))
         since_fence = 0
         for n_path, p in enumerate(ordered):
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
@@ -146,26 +146,28 @@ class DoubleEmitter(UvuEmitter):
                 s(f"const T cv = {cacc(p, v)};")
                 ks = sorted({k for _, _, k, _ in p.nnz})
                 js = sorted({j for _, j, _, _ in p.nnz})
+                # One output component k at a time, so that what is derived from g_k (its products with the
+                # weights and with the X / A components) is dead before the next k: in any other order
+                # these temporaries, two sets of them here, cost more registers than the operands.
+                #   d/dX_i += (|c| b_j)(g_k w) + (|c| y_j)(g_k c)
+                #   h_j = sum_ik c x_i g_k,  ha_j = sum_ik c a_i g_k
+                for j in js:
+                    s(f"T h{j} = T(0), ha{j} = T(0);")
                 for k in ks:
-                    s(f"const T gw{k} = {gname(k)} * wv; const T gc{k} = {gname(k)} * cv;")
-                # d/dX: (|c| b_j)(g_k w) + (|c| y_j)(g_k c)
-                for n, (i, j, k, c) in enumerate(p.nnz):
-                    qy, qb, neg = prods[n]
-                    op = "-=" if neg else "+="
-                    s(f"dx.b{p.i1}[{i}] {op} {qb} * gw{k}; dx.b{p.i1}[{i}] {op} {qy} * gc{k};")
-                # h_j = sum_ik c x_i g_k, ha_j = sum_ik c a_i g_k
-                pair, hstart = {}, set()
-                for n, (i, j, k, c) in enumerate(p.nnz):
-                    if (i, k) not in pair:
-                        pair[(i, k)] = len(pair)
-                        s(f"const T xg{pair[(i, k)]} = x.b{p.i1}[{i}] * {gname(k)}; "
-                          f"const T ag{pair[(i, k)]} = xa.b{p.i1}[{i}] * {gname(k)};")
-                    m = pair[(i, k)]
-                    if j not in hstart:
-                        s(f"T h{j} = T({self.lit(c)}) * xg{m}; T ha{j} = T({self.lit(c)}) * ag{m};")
-                        hstart.add(j)
-                    else:
-                        s(f"h{j} += T({self.lit(c)}) * xg{m}; ha{j} += T({self.lit(c)}) * ag{m};")
+                    s.open("")
+                    s(f"const T gw = {gname(k)} * wv; const T gc = {gname(k)} * cv;")
+                    of_k = [(n, t) for n, t in enumerate(p.nnz) if t[2] == k]
+                    for n, (i, j, _, c) in of_k:
+                        qy, qb, neg = prods[n]
+                        op = "-=" if neg else "+="
+                        s(f"dx.b{p.i1}[{i}] {op} {qb} * gw; dx.b{p.i1}[{i}] {op} {qy} * gc;")
+                    for i in sorted({t[0] for _, t in of_k}):
+                        s(f"{{ const T xg = x.b{p.i1}[{i}] * {gname(k)}; const T ag = xa.b{p.i1}[{i}] * {gname(k)};")
+                        for n, (i2, j, _, c) in of_k:
+                            if i2 == i:
+                                s(f"  h{j} += T({self.lit(c)}) * xg; ha{j} += T({self.lit(c)}) * ag;")
+                        s("}")
+                    s.close()
                 # d/dW = sum_j b_j h_j + y_j ha_j ; d/dY_j = c h_j + w ha_j
                 s(f"T dwv = b{js[0]} * h{js[0]};")
                 s(f"dwv += y{js[0]} * ha{js[0]};")
@@ -189,13 +191,23 @@ class DoubleEmitter(UvuEmitter):
                 if nxt is None or since_fence + low.out[nxt.io].d * self.words > self.fence_words:
                     s("__builtin_amdgcn_sched_barrier(0);")
                     since_fence = 0
+            elif self.fence_paths and (n_path + 1) % self.fence_paths == 0 and n_path + 1 < len(ordered):
+                # resident gradients: the scheduler would still request every path's W and C values up
+                # front, two registers per path on top of X, A, dX, dY and the gradient slice
+                s("__builtin_amdgcn_sched_barrier(0);")
+
+    fence_paths = 0   # resident gradients: a scheduling fence after every so many paths (0: none)
+    force_resident: Optional[bool] = None
 
     def double_b_resident(self) -> bool:
         """The row's / node's output-gradient slice stays in registers beside X, A, dX and dY."""
         low = self.low
+        if self.force_resident is not None:
+            return self.force_resident
         x = sum(low.in1[b].d for b in self.used_in1)
         g = sum(low.out[io].d for io in self.used_out)
-        return self.words * (g + 3 * x + self.l2_pad) + 48 <= 232
+        # X, A, dX, dY, the gradient slice, and the W and C values of every path (requested up front)
+        return self.words * (g + 3 * x + self.l2_pad + 2 * self.n_wslots) + 40 <= 232
 
     # ------------------------------------------------------------ batch kernels
     def emit_tp_double_a(self, s: Src, G: int, waves_per_eu: int = 0):
@@ -441,6 +453,142 @@ class DoubleEmitter(UvuEmitter):
         return block
 
 
+    # ---- kernel B with a node's output blocks shared between several waves ------------------------
+    def plan_double_groups(self, max_waves: int) -> Optional[List[List[int]]]:
+        """Output blocks per wave when one wave cannot keep X, A, dX, dY, the node's gradient slice and
+        the in-flight W / C values of all paths in registers: None when one wave can (or when the
+        kernel shape does not allow the split)."""
+        low = self.low
+        if self.R != 1 or not self.can_preload:
+            return None
+        x = sum(low.in1[b].d for b in self.used_in1)
+        fixed = self.words * (3 * x + self.l2_pad) + 40
+        sizes = [low.out[io].d for io in self.used_out]
+        per_path = {io: sum(2 * low.in2[p.i2].mul for p in low.paths if p.io == io) for io in self.used_out}
+
+        def need(grp):
+            return fixed + self.words * sum(low.out[io].d + per_path[io] for io in grp)
+
+        if need(self.used_out) <= 200:
+            return None
+        # the waves exchange their dX terms through LDS: [waves][chunks][X components][64 lanes]
+        lds_per_wave = self.NCH * x * 64 * low.elem_size
+        max_waves = min(max_waves, 60000 // lds_per_wave)
+        n = 2
+        while n <= max_waves:
+            target = -(-sum(sizes) // n)
+            groups, cur, tot = [], [], 0
+            for io, d in zip(self.used_out, sizes):
+                if cur and tot + d > target and len(groups) < n - 1:
+                    groups.append(cur)
+                    cur, tot = [], 0
+                cur.append(io)
+                tot += d
+            groups.append(cur)
+            if all(need(grp) <= 200 for grp in groups) or n == max_waves:
+                return groups
+            n += 1
+        return None
+
+    def emit_conv_double_b_split(self, s: Src, groups: List[List[int]], waves_per_eu: int = 0, xcd: int = 1) -> int:
+        """All waves of a block walk the edges of one node; wave ``sg`` keeps the gradient of its output
+        blocks resident and handles the paths into them (their d/dW is final); an edge's partial d/dX and
+        d/dY are summed over the waves through LDS in a fixed order."""
+        low = self.low
+        SW = len(groups)
+        block = 64 * self.NCH * SW
+        xoff, XW = {}, 0
+        for b in self.used_in1:
+            xoff[b] = XW
+            XW += low.in1[b].d
+        gpaths = [[p for p in low.paths if p.io in grp] for grp in groups]
+        gin1 = [sorted({p.i1 for p in ps}) for ps in gpaths]
+        s.open(
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_b(i64 node_count, '
+            f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
+            "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
+            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm)"
+        )
+        self._lane_prologue(s, SW)
+        s(f"__shared__ T s_dy[{SW * self.NCH}][{self.l2_pad}];")
+        s(f"__shared__ T s_dx[{SW}][{self.NCH}][{XW}][64];")
+        self._node_loop_open(s, 1, xcd)
+        s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+        for si in range(SW):
+            s.open(f"if (sg == {si})")
+
+            def sg_body(si=si):
+                s("G_t gr;")
+                self._load_g(s, f"L3_grad + node * {low.L3}", groups[si])
+                # every wave of the block runs the same number of edges, so the block barriers match up
+                s.open("for (i64 e = e0; e < e1; ++e)")
+                self._edge_rows(s, "e")
+                s(f"T* dwrow = W_grad + eid * {low.WN};")
+                s("X_t x, xa, dx;")
+                self._load_x(s, "xrow", gin1[si])
+                self._load_x(s, "arow", gin1[si], "xa")
+                self._zero_x(s, "dx")
+                s(f"T dy[{self.l2_pad}];")
+                s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+                deferred = self._dw_deferred(None)
+                if deferred:
+                    s(f"T dwkeep[{self.n_wslots}];")
+                self._ddb_paths(s, None, False, deferred, None, gpaths[si])
+                self._pin_gradients(s, gin1[si], deferred, gpaths[si])
+                if deferred:
+                    low_paths, low.paths = low.paths, gpaths[si]
+                    try:
+                        self._flush_dwkeep(s, None)
+                    finally:
+                        low.paths = low_paths
+                for b in self._in1_of(gin1[si]):
+                    for i in range(low.in1[b].d):
+                        s(f"s_dx[{si}][chunk][{xoff[b] + i}][ul] = dx.b{b}[{i}];")
+                s.open("")
+                cur, dup = self._dy_reduce(s)
+                s.open(f"if ((ul & {dup}) == 0)")
+                for j in range(cur):
+                    s(f"s_dy[{si} * {self.NCH} + chunk][dyidx + {j}] = rv[{j}];")
+                s.close()
+                s.close()
+                s("__syncthreads();")
+                # the used input blocks are shared out between the waves for the final sum and store
+                s(f"T* dxrow = dx_tmp + eid * {low.L1};")
+                for n, b in enumerate(self.used_in1):
+                    if n % SW != si or not self._has(low.in1[b].mul):
+                        continue
+                    blk = low.in1[b]
+                    contributors = [c for c in range(SW) if b in gin1[c]]
+                    self._open_if(s, self._store_cond(blk.mul))
+                    base, st = self._lane_ptr(blk)
+                    s(f"T* dp = {self._ptr('dxrow', base)};")
+                    for i in range(blk.d):
+                        terms = " + ".join(f"s_dx[{c}][chunk][{xoff[b] + i}][ul]" for c in contributors)
+                        val = f"({terms})" if contributors else "T(0)"
+                        if self.nt & 2:
+                            s(f"__builtin_nontemporal_store({val}, dp + {i * st});")
+                        else:
+                            s(f"dp[{i * st}] = {val};")
+                    s.close()
+                if si == 0:
+                    self._zero_untouched_in1(s, "dxrow", "true")
+                    s.open("if (chunk == 0)")
+                    s.open(f"for (int j = lane; j < {low.L2}; j += 64)")
+                    s("T tot = s_dy[0][j];")
+                    s(f"for (int cc = 1; cc < {SW * self.NCH}; ++cc) tot += s_dy[cc][j];")
+                    s(f"L2_grad[eid * {low.L2} + j] = tot;")
+                    s.close()
+                    s.close()
+                s("__syncthreads();")
+                s.close()
+
+            self._per_chunk(s, sg_body)
+            s.close()
+        s.close()
+        s.close()
+        return block
+
+
 def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict) -> List[tuple]:
     """Append the batch double-backward kernels to a module; returns their launch descriptors."""
     from .. import runtime as rt
@@ -468,13 +616,21 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     em = DoubleEmitter(low, acc_budget_words=tune.get("dd_acc", 112))
     em.nt = base.nt
     em.tr_stores = base.tr_stores
-    em.fence_words = 0
+    em.fence_words = tune.get("dd_fw", 32)
+    em.fence_paths = tune.get("dd_fp", 0)
+    if tune.get("dd_gres", -1) >= 0:
+        em.force_resident = bool(tune["dd_gres"])
     _emit_segment_structs(s, em, "D")
     em.emit_double_cores(s)
     G = max(1, tune.get("dd_g", 2) // em.NCH) if em.R == 1 else 4
     blk_a = em.emit_conv_double_a(s, G, tune.get("dd_wa", 2), xcd)
-    blk_b = em.emit_conv_double_b(s, G, tune.get("dd_wb", 2), xcd)
-    G_b = 1 if em.NCH > 1 else G
+    groups = em.plan_double_groups(8 // em.NCH) if tune.get("dd_split", 1) else None
+    if groups:
+        blk_b = em.emit_conv_double_b_split(s, groups, tune.get("dd_wb", 2), xcd)
+        G_b = 1
+    else:
+        blk_b = em.emit_conv_double_b(s, G, tune.get("dd_wb", 2), xcd)
+        G_b = 1 if em.NCH > 1 else G
     return [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_a", blk_a, G, 0, xcd),
             (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_b", blk_b, G_b, 0, xcd)]
 
