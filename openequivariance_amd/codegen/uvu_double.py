@@ -344,23 +344,26 @@ class DoubleEmitter(UvuEmitter):
         s(f"const T* wrow = W + eid * {low.WN};")
         s(f"const T* crow = W_dgrad + eid * {low.WN};")
 
-    def emit_conv_double_a(self, s: Src, G: int, waves_per_eu: int = 0, xcd: int = 1):
-        """Receiver-major walk: the node's accumulators stay in registers over its edges."""
+    def emit_conv_double_a(self, s: Src, G: int, waves_per_eu: int = 0, xcd: int = 1, segw: int = 1):
+        """Receiver-major walk: the node's accumulators stay in registers over its edges. With ``segw``
+        > 1 the output segments of a node are shared between that many waves, which walk its edges side
+        by side (fewer registers per wave, more waves in flight)."""
         low = self.low
-        block = 64 * self.NCH * G
+        segw = max(1, min(segw, len(self.segments))) if self.R == 1 else 1
+        block = 64 * self.NCH * G * segw
         s.open(
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_a(i64 node_count, '
             f"i64 nnz, {self._CONV_OPERANDS}T* __restrict__ L3_dgrad, const i64* __restrict__ rows, "
             "const i64* __restrict__ cols, const i64* __restrict__ rowptr, const i64* __restrict__ eperm)"
         )
-        self._lane_prologue(s)
+        self._lane_prologue(s, segw)
         if self.tr_stores & 1 and self.R == 1:
-            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.out[io].d for io in self.used_out)}];")
+            s(f"__shared__ T s_tr[{self.NCH * G * segw}][{64 * max(low.out[io].d for io in self.used_out)}];")
         self._node_loop_open(s, G, xcd)
         s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
         s(f"T* zrow = L3_dgrad + node * {low.L3};")
         for si in range(len(self.segments)):
-            s.open("")
+            s.open(f"if (sg == {si % segw})" if segw > 1 else "")
 
             def node_body(si=si):
                 if self.cur_chunk is not None and not self._out_of(self.segments[si]):
@@ -384,7 +387,7 @@ class DoubleEmitter(UvuEmitter):
 
             self._per_chunk(s, node_body)
             s.close()
-        self._zero_untouched_out(s, "zrow", "r == 0")
+        self._zero_untouched_out(s, "zrow", "r == 0 && sg == 0" if segw > 1 else "r == 0")
         s.close()
         s.close()
         return block
@@ -623,7 +626,9 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     _emit_segment_structs(s, em, "D")
     em.emit_double_cores(s)
     G = max(1, tune.get("dd_g", 2) // em.NCH) if em.R == 1 else 4
-    blk_a = em.emit_conv_double_a(s, G, tune.get("dd_wa", 2), xcd)
+    segw = min(len(em.segments), max(1, tune.get("dd_segw", 4)), 8 // em.NCH) if em.R == 1 else 1
+    G_a = max(1, min(G, 8 // (em.NCH * segw)))
+    blk_a = em.emit_conv_double_a(s, G_a, tune.get("dd_wa", 2), xcd, segw)
     groups = em.plan_double_groups(8 // em.NCH) if tune.get("dd_split", 1) else None
     if groups:
         blk_b = em.emit_conv_double_b_split(s, groups, tune.get("dd_wb", 2), xcd)
@@ -631,7 +636,7 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     else:
         blk_b = em.emit_conv_double_b(s, G, tune.get("dd_wb", 2), xcd)
         G_b = 1 if em.NCH > 1 else G
-    return [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_a", blk_a, G, 0, xcd),
+    return [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_a", blk_a, G_a, 0, xcd),
             (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_b", blk_b, G_b, 0, xcd)]
 
 
