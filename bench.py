@@ -36,6 +36,8 @@ def parse():
     ap.add_argument("--no-atomic", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the side measurements (spatially ordered nodes, batch tensor-product configs)")
+    ap.add_argument("--with-double", action="store_true",
+                    help="with --no-extras: still run the second-order (double backward) side measurement")
     ap.add_argument("--only-tp", default=None, metavar="N",
                     help="run only the batched tensor-product side measurement for config N (1, 2, 3, 3d, 4) "
                          "and print its row; used for per-kernel profiles")
@@ -315,6 +317,38 @@ def main():
             "hbm_roofline_frac": (fwd_bytes + bwd_bytes) / (ms_sp * 1e-3) / 1e9 / HBM_PEAK_GBS,
         }
         del Ys, trs, tcs, tps
+
+    # Second-order kernels at the same shape (the backward of the backward, as in force training):
+    # the fused pair against the composition of three forward and three backward calls.
+    if (not args.no_extras or args.with_double) and ks.has_double_backward():
+        from openequivariance_amd import runtime as rt
+        A_, B_, C_ = torch.randn_like(X), torch.randn_like(Y), torch.randn_like(W)
+
+        def step_dd():
+            ops.conv_double_backward(X, Y, W, G, A_, B_, C_, tr, tc, tp, kid)
+
+        def step_composed():
+            with torch.no_grad():
+                ops._second_order(lambda p, q, r: ops.conv_forward(p, q, r, tr, tc, tp, kid),
+                                  lambda p, q, r, s: ops.conv_backward(p, q, r, s, tr, tc, tp, kid),
+                                  X, Y, W, G, A_, B_, C_)
+
+        ms_dd = time_steps(step_dd, max(3, args.steps // 4), 2)
+        ks.timing_enable(True)
+        step_dd()
+        torch.cuda.synchronize()
+        split = {name: ks.timing_collect(role)[0] for name, role in
+                 (("double_backward_a", rt.ROLE_DOUBLE_BACKWARD_A), ("double_backward_b", rt.ROLE_DOUBLE_BACKWARD_B),
+                  ("fixup_backward", rt.ROLE_CONV_FIXUP_BACKWARD))}
+        ks.timing_enable(False)
+        ms_cmp = time_steps(step_composed, 2, 1)
+        dd_bytes = 4 * (E * 3 * (L2 + WN) + N * (3 * L1 + 2 * L3))
+        extras["double_backward"] = {
+            "fused_ms": ms_dd, "composed_first_order_ms": ms_cmp, "kernel_ms": split,
+            "hbm_roofline_frac": dd_bytes / (ms_dd * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "algorithmic_bytes_per_edge": dd_bytes / E,
+        }
+        del A_, B_, C_
 
     cpu = None
     if args.cpu_receivers > 0:

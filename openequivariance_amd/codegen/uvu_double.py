@@ -115,9 +115,11 @@ class DoubleEmitter(UvuEmitter):
 
     # ------------------------------------------------------------ kernel B paths
     def _ddb_paths(self, s: Src, g_on_demand_row: Optional[str], fence: bool, deferred: bool,
-                   dw_guard: Optional[str], paths: Optional[List[Path]] = None):
+                   dw_guard: Optional[str], paths: Optional[List[Path]] = None, fwd_acc: bool = False):
         """Straight-line second-order backward of all paths. In scope: x, xa (X_t), dx (X_t), dy[],
-        yrow, brow, wrow, crow, dwrow, u, and gr (G_t) or the row pointer named ``g_on_demand_row``."""
+        yrow, brow, wrow, crow, dwrow, u, and gr (G_t) or the row pointer named ``g_on_demand_row``.
+        ``fwd_acc``: the three forward terms of kernel A are added to ``a`` (G_t) as well, from the same
+        operand registers."""
         low = self.low
         wacc, cacc = self._w_of("wrow"), self._w_of("crow")
         ordered = sorted(self._paths(paths), key=lambda q: (q.io, q.index))
@@ -182,6 +184,19 @@ class DoubleEmitter(UvuEmitter):
                     s(f"if ({cond}) {st}" if cond else st)
                 for j in js:
                     s(f"dy[{self._y_index(b2, v, j)}] += cv * h{j}; dy[{self._y_index(b2, v, j)}] += wv * ha{j};")
+                if fwd_acc:
+                    for k in ks:
+                        s.open("")
+                        s("T ft = T(0), fs = T(0);")
+                        for n, (i, j, k2, c) in enumerate(p.nnz):
+                            if k2 != k:
+                                continue
+                            qy, qb, neg = prods[n]
+                            op = "-=" if neg else "+="
+                            xi, ai = f"x.b{p.i1}[{i}]", f"xa.b{p.i1}[{i}]"
+                            s(f"ft {op} {qy} * {ai}; ft {op} {qb} * {xi}; fs {op} {qy} * {xi};")
+                        s(f"a.o{p.io}[{k}] += wv * ft + cv * fs;")
+                        s.close()
 
             self._for_v(s, p, body)
             s.close()
@@ -404,14 +419,16 @@ class DoubleEmitter(UvuEmitter):
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_b(i64 node_count, '
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm)"
+            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
+            "T* __restrict__ L3_dgrad)"
         )
         self._lane_prologue(s)
         if self.NCH > 1:
             s(f"__shared__ T s_dy[{G}][{self.NCH}][{self.l2_pad}];")
-        if self.tr_stores & 2 and self.R == 1:
-            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.in1[b].d for b in self.used_in1)}];")
-        resident = self.double_b_resident()
+        if (self.tr_stores & 2 or (self.merged and self.tr_stores & 1)) and self.R == 1:
+            dmax = max([low.in1[b].d for b in self.used_in1] + [low.out[io].d for io in self.used_out])
+            s(f"__shared__ T s_tr[{self.NCH * G}][{64 * dmax}];")
+        resident = self.double_b_resident() or self.merged
         self._node_loop_open(s, G, xcd)
         s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
 
@@ -419,6 +436,11 @@ class DoubleEmitter(UvuEmitter):
             if resident:
                 s("G_t gr;")
                 self._load_g(s, f"L3_grad + node * {low.L3}", self.used_out)
+            if self.merged:
+                s("G_t a;")
+                for io in self._out_of(self.used_out):
+                    for k in range(low.out[io].d):
+                        s(f"a.o{io}[{k}] = T(0);")
             # with more than one chunk every wave of the block walks the same edges: the block barriers
             # of the dY reduction are reached uniformly
             s.open(f"for (i64 e = e0 + r; e < e1; e += {self.R})")
@@ -434,7 +456,7 @@ class DoubleEmitter(UvuEmitter):
             if deferred:
                 s(f"T dwkeep[{self.n_wslots}];")
             if resident:
-                self._ddb_paths(s, None, False, deferred, None)
+                self._ddb_paths(s, None, False, deferred, None, fwd_acc=self.merged)
             else:
                 s(f"const T* grow = L3_grad + node * {low.L3};")
                 # without this the compiler hoists the loads of the node's gradient row out of the edge
@@ -449,14 +471,38 @@ class DoubleEmitter(UvuEmitter):
             self._zero_untouched_in1(s, "dxrow", "true")
             self._dy_finish(s, f"L2_grad + eid * {low.L2}", "true")
             s.close()
+            if self.merged:
+                if self.R > 1:  # fold the lane groups of packed rows (fixed order) into group 0
+                    for io in self._out_of(self.used_out):
+                        for k in range(low.out[io].d):
+                            m = self.LPR
+                            while m < 64:
+                                s(f"a.o{io}[{k}] += __shfl_xor(a.o{io}[{k}], {m});")
+                                m *= 2
+                segments, self.segments = self.segments, [self.used_out]
+                try:
+                    self._store_seg(s, 0, f"(L3_dgrad + node * {low.L3})", "r == 0" if self.R > 1 else "true")
+                finally:
+                    self.segments = segments
 
         self._per_chunk(s, node_body)
+        if self.merged:
+            self._zero_untouched_out(s, f"(L3_dgrad + node * {low.L3})", "r == 0")
         s.close()
         s.close()
         return block
 
 
     # ---- kernel B with a node's output blocks shared between several waves ------------------------
+    merged = False     # kernel B also accumulates and writes kernel A's result (no separate kernel A)
+    need_limit = 200   # register estimate above which a node's output blocks are shared between waves
+
+    def merged_fits_one_wave(self) -> bool:
+        low = self.low
+        x = sum(low.in1[b].d for b in self.used_in1)
+        g = sum(low.out[io].d for io in self.used_out)
+        return self.words * (2 * g + 3 * x + self.l2_pad + 2 * self.n_wslots) + 40 <= 232
+
     def plan_double_groups(self, max_waves: int) -> Optional[List[List[int]]]:
         """Output blocks per wave when one wave cannot keep X, A, dX, dY, the node's gradient slice and
         the in-flight W / C values of all paths in registers: None when one wave can (or when the
@@ -470,9 +516,9 @@ class DoubleEmitter(UvuEmitter):
         per_path = {io: sum(2 * low.in2[p.i2].mul for p in low.paths if p.io == io) for io in self.used_out}
 
         def need(grp):
-            return fixed + self.words * sum(low.out[io].d + per_path[io] for io in grp)
+            return fixed + self.words * sum(low.out[io].d * (2 if self.merged else 1) + per_path[io] for io in grp)
 
-        if need(self.used_out) <= 200:
+        if need(self.used_out) <= self.need_limit:
             return None
         # the waves exchange their dX terms through LDS: [waves][chunks][X components][64 lanes]
         lds_per_wave = self.NCH * x * 64 * low.elem_size
@@ -488,7 +534,7 @@ class DoubleEmitter(UvuEmitter):
                 cur.append(io)
                 tot += d
             groups.append(cur)
-            if all(need(grp) <= 200 for grp in groups) or n == max_waves:
+            if all(need(grp) <= self.need_limit for grp in groups) or n == max_waves:
                 return groups
             n += 1
         return None
@@ -510,11 +556,14 @@ class DoubleEmitter(UvuEmitter):
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_b(i64 node_count, '
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm)"
+            "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
+            "T* __restrict__ L3_dgrad)"
         )
         self._lane_prologue(s, SW)
         s(f"__shared__ T s_dy[{SW * self.NCH}][{self.l2_pad}];")
         s(f"__shared__ T s_dx[{SW}][{self.NCH}][{XW}][64];")
+        if self.merged and self.tr_stores & 1:
+            s(f"__shared__ T s_tr[{self.NCH * SW}][{64 * max(low.out[io].d for io in self.used_out)}];")
         self._node_loop_open(s, 1, xcd)
         s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
         for si in range(SW):
@@ -523,6 +572,11 @@ class DoubleEmitter(UvuEmitter):
             def sg_body(si=si):
                 s("G_t gr;")
                 self._load_g(s, f"L3_grad + node * {low.L3}", groups[si])
+                if self.merged:
+                    s("G_t a;")
+                    for io in self._out_of(groups[si]):
+                        for k in range(low.out[io].d):
+                            s(f"a.o{io}[{k}] = T(0);")
                 # every wave of the block runs the same number of edges, so the block barriers match up
                 s.open("for (i64 e = e0; e < e1; ++e)")
                 self._edge_rows(s, "e")
@@ -536,7 +590,7 @@ class DoubleEmitter(UvuEmitter):
                 deferred = self._dw_deferred(None)
                 if deferred:
                     s(f"T dwkeep[{self.n_wslots}];")
-                self._ddb_paths(s, None, False, deferred, None, gpaths[si])
+                self._ddb_paths(s, None, False, deferred, None, gpaths[si], fwd_acc=self.merged)
                 self._pin_gradients(s, gin1[si], deferred, gpaths[si])
                 if deferred:
                     low_paths, low.paths = low.paths, gpaths[si]
@@ -584,9 +638,17 @@ class DoubleEmitter(UvuEmitter):
                     s.close()
                 s("__syncthreads();")
                 s.close()
+                if self.merged:
+                    segments, self.segments = self.segments, groups
+                    try:
+                        self._store_seg(s, si, f"(L3_dgrad + node * {low.L3})", "true")
+                    finally:
+                        self.segments = segments
 
             self._per_chunk(s, sg_body)
             s.close()
+        if self.merged:
+            self._zero_untouched_out(s, f"(L3_dgrad + node * {low.L3})", "sg == 0")
         s.close()
         s.close()
         return block
@@ -626,18 +688,28 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     _emit_segment_structs(s, em, "D")
     em.emit_double_cores(s)
     G = max(1, tune.get("dd_g", 2) // em.NCH) if em.R == 1 else 4
-    segw = min(len(em.segments), max(1, tune.get("dd_segw", 4)), 8 // em.NCH) if em.R == 1 else 1
-    G_a = max(1, min(G, 8 // (em.NCH * segw)))
-    blk_a = em.emit_conv_double_a(s, G_a, tune.get("dd_wa", 2), xcd, segw)
+    em.need_limit = tune.get("dd_need", 200)
+    # dd_merge=1: one kernel for both results (W, C and the gathered X, A rows are then read once instead of
+    # twice). Measured slower on MI355X for every shape tried (MACE shape 37 - 85 ms against 33 ms for the
+    # pair): its accumulators on top of kernel B's state spill whatever the split, so it is off by default.
+    em.merged = bool(tune.get("dd_merge", 0))
     groups = em.plan_double_groups(8 // em.NCH) if tune.get("dd_split", 1) else None
+    if em.merged and not groups and not em.merged_fits_one_wave():
+        em.merged = False
+        groups = em.plan_double_groups(8 // em.NCH) if tune.get("dd_split", 1) else None
+    descs = []
+    if not em.merged:
+        segw = min(len(em.segments), max(1, tune.get("dd_segw", 4)), 8 // em.NCH) if em.R == 1 else 1
+        G_a = max(1, min(G, 8 // (em.NCH * segw)))
+        blk_a = em.emit_conv_double_a(s, G_a, tune.get("dd_wa", 2), xcd, segw)
+        descs.append((rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_a", blk_a, G_a, 0, xcd))
     if groups:
         blk_b = em.emit_conv_double_b_split(s, groups, tune.get("dd_wb", 2), xcd)
         G_b = 1
     else:
         blk_b = em.emit_conv_double_b(s, G, tune.get("dd_wb", 2), xcd)
         G_b = 1 if em.NCH > 1 else G
-    return [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_a", blk_a, G_a, 0, xcd),
-            (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_b", blk_b, G_b, 0, xcd)]
+    return descs + [(rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_b", blk_b, G_b, 0, xcd)]
 
 
 def _emit_segment_structs(s: Src, em: DoubleEmitter, prefix: str):

@@ -589,15 +589,14 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
 // second-order kernels
 // ---------------------------------------------------------------------------
 
-int oeq_has_double_backward(const oeq_kernels* k) {
-    return k && k->roles[OEQ_ROLE_DOUBLE_BACKWARD_A].present && k->roles[OEQ_ROLE_DOUBLE_BACKWARD_B].present;
-}
+// Kernel B alone is a complete set when it also produces kernel A's result (convolution, merged form).
+int oeq_has_double_backward(const oeq_kernels* k) { return k && k->roles[OEQ_ROLE_DOUBLE_BACKWARD_B].present; }
 
 int oeq_tp_double_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in, const void* L2_in, const void* W,
                            const void* L3_grad, const void* L1_dgrad, const void* L2_dgrad, const void* W_dgrad,
                            void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad, void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: NULL kernel set");
-    if (!oeq_has_double_backward(k))
+    if (!oeq_has_double_backward(k) || !k->roles[OEQ_ROLE_DOUBLE_BACKWARD_A].present)
         return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: this kernel set has no second-order kernels");
     if (num_batch < 0) return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: negative batch");
     if (num_batch == 0) return OEQ_OK;
@@ -637,10 +636,12 @@ int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, co
     if (rc) return rc;
     void* a[] = {&node_count, &nnz, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_dgrad,
                  &rows,       &cols, &ix.rowptr, &ix.rperm};
-    rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_A, node_count, a, stream);
-    if (rc) return rc;
-    void* b[] = {&node_count, &nnz,     &L1_in,  &L1_dgrad, &L2_in, &L2_dgrad,  &W,         &W_dgrad,
-                 &L3_grad,    &L2_grad, &W_grad, &rows,     &cols,  &ix.rowptr, &ix.dx_tmp, &ix.rperm};
+    if (k->roles[OEQ_ROLE_DOUBLE_BACKWARD_A].present) {
+        rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_A, node_count, a, stream);
+        if (rc) return rc;
+    }
+    void* b[] = {&node_count, &nnz,     &L1_in,  &L1_dgrad, &L2_in, &L2_dgrad,  &W,         &W_dgrad, &L3_grad,
+                 &L2_grad,    &W_grad,  &rows,   &cols,     &ix.rowptr, &ix.dx_tmp, &ix.rperm, &L3_dgrad};
     rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count, b, stream);
     if (rc) return rc;
     void* fargs[] = {&node_count, &nnz, &ix.dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};

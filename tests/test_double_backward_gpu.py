@@ -117,6 +117,13 @@ def test_conv_fused_matches_composition(name, make, batch, det):
     _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
 
 
+def test_conv_single_kernel_variant(monkeypatch):
+    """The optional single-kernel form (both results from one walk; OEQ_AMD_TUNE=dd_merge=1)."""
+    monkeypatch.setenv("OEQ_AMD_TUNE", "dd_merge=1")
+    for name, make in (("odd", _odd), ("cfg2", P.config2_nequip_uvu), ("cfg3", P.config3_mace_uvu)):
+        test_conv_fused_matches_composition(name, make, 0, True)
+
+
 def test_conv_fused_isolated_nodes_and_empty():
     """Nodes without edges get zero rows; an empty edge list gives zero node gradients."""
     problem = P.config2_nequip_uvu()
