@@ -1714,7 +1714,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         if low.shared_weights:
             descs.append((rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0))
         from . import uvu_double
-        if t["conv_dd"] and uvu_double.supported(low) and not kahan:
+        if t["conv_dd"] and uvu_double.supported(low, conv=True) and not kahan:
             descs += uvu_double.add_conv_kernels(s, low, em, t, xcd)
         if mode == rt.CONV_GROUPED:
             descs += [

@@ -30,8 +30,18 @@ from .lower import Lowered, Path
 from .uvu import UvuEmitter
 
 
-def supported(low: Lowered) -> bool:
-    return low.mode == "uvu" and not low.shared_weights
+# Convolution: above this many paths (after folding of wide rows) the kernels' register needs (two
+# operand sets per path in flight beside X, A, dX, dY and the gradient slice) make them spill so much that
+# they no longer beat the composition of first-order kernels (measured: SevenNet main layer, 38 paths,
+# 63 - 80 ms against 66 ms; NequIP benzene, 68 paths, 155 - 175 ms against 118 ms; NequiX main layer, 27
+# paths, 28 against 35 ms). The batch kernels are 3 - 4 times faster than the composition for all of them.
+CONV_MAX_PATHS = 32
+
+
+def supported(low: Lowered, conv: bool = False) -> bool:
+    if low.mode != "uvu" or low.shared_weights:
+        return False
+    return not conv or len(low.paths) <= CONV_MAX_PATHS
 
 
 class DoubleEmitter(UvuEmitter):

@@ -9,6 +9,7 @@ import torch
 
 import openequivariance_amd as oeq
 from openequivariance_amd._torch import ops
+from openequivariance_amd.codegen import uvu_double
 from openequivariance_amd.core import problems as P
 from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
 from oracle import e3nn_ref as R
@@ -91,10 +92,13 @@ CONV_CASES = [c for c in CASES if c[0] not in ("cfg1",)] + [("cfg1", P.config1_s
 
 @pytest.mark.parametrize("det", [True, False], ids=["sorted", "grouped"])
 @pytest.mark.parametrize("name,make,batch", CONV_CASES, ids=[c[0] for c in CONV_CASES])
-def test_conv_fused_matches_composition(name, make, batch, det):
+def test_conv_fused_matches_composition(name, make, batch, det, monkeypatch):
     problem = make()
     gph = _graph()
     n, E = gph.coords.shape[0], gph.nnz
+    if name in ("benzene", "sevennet-main"):
+        # more paths than the fused convolution kernels are built for by default
+        monkeypatch.setattr(uvu_double, "CONV_MAX_PATHS", 1000)
     conv = oeq.TensorProductConv(problem, deterministic=det)
     e = ops.get_entry(conv.kid)
     assert e.kernels().has_double_backward()
@@ -121,7 +125,7 @@ def test_conv_single_kernel_variant(monkeypatch):
     """The optional single-kernel form (both results from one walk; OEQ_AMD_TUNE=dd_merge=1)."""
     monkeypatch.setenv("OEQ_AMD_TUNE", "dd_merge=1")
     for name, make in (("odd", _odd), ("cfg2", P.config2_nequip_uvu), ("cfg3", P.config3_mace_uvu)):
-        test_conv_fused_matches_composition(name, make, 0, True)
+        test_conv_fused_matches_composition(name, make, 0, True, monkeypatch)
 
 
 def test_conv_fused_isolated_nodes_and_empty():
@@ -149,6 +153,14 @@ def test_conv_fused_isolated_nodes_and_empty():
             assert float(fused[3][0].abs().max()) == 0.0  # node 0 receives nothing
         else:
             assert float(fused[0].abs().max()) == 0.0 and float(fused[3].abs().max()) == 0.0
+
+
+def test_many_path_convolutions_use_the_composition():
+    from openequivariance_amd.codegen.lower import lower
+    assert not uvu_double.supported(lower(P.seven_net_problems()[1]), conv=True)
+    assert uvu_double.supported(lower(P.seven_net_problems()[1]))
+    conv = oeq.TensorProductConv(P.seven_net_problems()[1], deterministic=True)
+    assert not ops.get_entry(conv.kid).kernels().has_double_backward()
 
 
 @pytest.mark.parametrize("which", ["tp", "conv"])
