@@ -5,7 +5,8 @@
 //   <dir>/bundle.txt    problem dims, kernel descriptors, batch size
 //   <dir>/{x,y,w,g}.bin inputs, <dir>/{z,dx,dy,dw}.bin expected results (raw little-endian floats)
 // compiles the source with oeq_jit_compile, runs oeq_tp_forward / oeq_tp_backward on plain
-// hipMalloc'ed buffers and compares with the expected values (max normalised error).
+// hipMalloc'ed buffers and compares with the expected values (max normalised error); when the set has
+// second-order kernels, oeq_tp_double_backward is checked against sums of first-order calls.
 //
 // Build: hipcc -O2 -std=c++17 -Iinclude tests/cabi/cabi_roundtrip.cpp -o tests/cabi/cabi_roundtrip \
 //        -Lopenequivariance_amd -loeq_amd -Wl,-rpath,'$ORIGIN/../../openequivariance_amd'
@@ -124,7 +125,49 @@ int main(int argc, char** argv) {
     const double e[4] = {normalized_error(z, z_ref), normalized_error(dx, dx_ref), normalized_error(dy, dy_ref),
                          normalized_error(dw, dw_ref)};
     std::printf("errors z=%.3g dx=%.3g dy=%.3g dw=%.3g\n", e[0], e[1], e[2], e[3]);
+    double e2[2] = {0, 0};
+    if (oeq_has_double_backward(k)) {
+        // Second-order kernels against the first-order entry points, with the first-order gradients as
+        // cotangents (A, B, C) = (dX, dY, dW): d/d(dZ) = F(A,Y,W) + F(X,B,W) + F(X,Y,C) and
+        // d/dX = dX-part of backward(X,B,W;dZ) + dX-part of backward(X,Y,C;dZ).
+        float *hX, *hY, *hW, *hG, *tZ, *tX, *tY, *tW;
+        CHECK_HIP(hipMalloc(&hX, bytes(x)));
+        CHECK_HIP(hipMalloc(&hY, bytes(y)));
+        CHECK_HIP(hipMalloc(&hW, bytes(w)));
+        CHECK_HIP(hipMalloc(&hG, bytes(g)));
+        CHECK_HIP(hipMalloc(&tZ, bytes(g)));
+        CHECK_HIP(hipMalloc(&tX, bytes(x)));
+        CHECK_HIP(hipMalloc(&tY, bytes(y)));
+        CHECK_HIP(hipMalloc(&tW, bytes(w)));
+        CHECK_OEQ(oeq_tp_double_backward(k, batch, dX, dY, dW, dG, gX, gY, gW, hX, hY, hW, hG, stream));
+        CHECK_HIP(hipStreamSynchronize(stream));
+        std::vector<float> gg(g.size()), ddx(x.size()), gg_ref(g.size(), 0.f), ddx_ref(x.size(), 0.f), t(g.size()),
+            tx(x.size());
+        CHECK_HIP(hipMemcpy(gg.data(), hG, bytes(gg), hipMemcpyDeviceToHost));
+        CHECK_HIP(hipMemcpy(ddx.data(), hX, bytes(ddx), hipMemcpyDeviceToHost));
+        const float* fw[3][3] = {{gX, dY, dW}, {dX, gY, dW}, {dX, dY, gW}};
+        for (auto& o : fw) {
+            CHECK_OEQ(oeq_tp_forward(k, batch, o[0], o[1], o[2], tZ, stream));
+            CHECK_HIP(hipStreamSynchronize(stream));
+            CHECK_HIP(hipMemcpy(t.data(), tZ, bytes(t), hipMemcpyDeviceToHost));
+            for (size_t i = 0; i < t.size(); ++i) gg_ref[i] += t[i];
+        }
+        const float* bw[2][2] = {{gY, dW}, {dY, gW}};
+        for (auto& o : bw) {
+            CHECK_OEQ(oeq_tp_backward(k, batch, dX, tX, o[0], tY, o[1], tW, dG, ws, ws_bytes, stream));
+            CHECK_HIP(hipStreamSynchronize(stream));
+            CHECK_HIP(hipMemcpy(tx.data(), tX, bytes(tx), hipMemcpyDeviceToHost));
+            for (size_t i = 0; i < tx.size(); ++i) ddx_ref[i] += tx[i];
+        }
+        e2[0] = normalized_error(gg, gg_ref);
+        e2[1] = normalized_error(ddx, ddx_ref);
+        std::printf("second order: d/d(dZ)=%.3g d/dX=%.3g\n", e2[0], e2[1]);
+    } else {
+        std::printf("second order: no fused kernels in this set\n");
+    }
     oeq_kernels_destroy(k);
+    for (double v : e2)
+        if (!(v <= 1e-5)) { std::printf("FAILED\n"); return 6; }
     for (double v : e)
         if (!(v <= 1e-5)) { std::printf("FAILED\n"); return 5; }
     std::printf("OK\n");
