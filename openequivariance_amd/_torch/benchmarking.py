@@ -1,6 +1,6 @@
 """Timing helpers on the two modules, with the call signatures of the reference's
-``benchmark_forward`` / ``benchmark_backward``
-(openequivariance/openequivariance/core/TensorProductBase.py:69-124,
+``benchmark_forward`` / ``benchmark_backward`` / ``benchmark_double_backward``
+(openequivariance/openequivariance/core/TensorProductBase.py:69-175,
 core/ConvolutionBase.py:134-290, core/utils.py:152-205).
 
 ``with_torch_overhead=True`` times the whole op call with events on torch's current
@@ -75,6 +75,37 @@ class TensorProductTiming:
         return time_call(lambda: z.backward(gradient=g, retain_graph=True, inputs=[x, y, w]), num_warmup, num_iter,
                          x.device, entry, (rt.ROLE_TP_BACKWARD, rt.ROLE_TP_BACKWARD_WREDUCE))
 
+    def benchmark_double_backward(self, num_warmup, num_iter, L1_in, L2_in, weights, weights_grad,
+                                  with_torch_overhead=True,
+                                  kernel_names=("double_backward_a", "double_backward_b")) -> np.ndarray:
+        """Time of the gradient of a scalar function of the three first-order gradients with respect to
+        X, Y, W and the output gradient (the reference's protocol, TensorProductBase.py:126-175; as
+        there, the output gradient is the forward result and ``weights_grad`` is accepted for
+        signature compatibility only)."""
+        x, y, w = (torch.as_tensor(a).to("cuda").detach().requires_grad_(True) for a in (L1_in, L2_in, weights))
+        z = self.forward(x, y, w)
+        g = z.clone().detach().requires_grad_(True)
+        first = torch.autograd.grad(z, [x, y, w], g, create_graph=True, retain_graph=True)
+        dummy = sum(torch.norm(t) for t in first)
+        dummy_grad = torch.ones_like(dummy)
+        entry = None if with_torch_overhead else ops.get_entry(self.kid)
+        roles = (rt.ROLE_DOUBLE_BACKWARD_A, rt.ROLE_DOUBLE_BACKWARD_B, rt.ROLE_TP_FORWARD, rt.ROLE_TP_BACKWARD,
+                 rt.ROLE_TP_BACKWARD_WREDUCE)
+        return time_call(lambda: torch.autograd.grad(dummy, [x, y, w, g], dummy_grad, retain_graph=True),
+                         num_warmup, num_iter, x.device, entry, roles)
+
+    def double_backward(self, in1, in2, out_grad, weights, weights_dgrad, in1_dgrad, in2_dgrad):
+        """(in1_grad, in2_grad, weights_grad, out_dgrad) as numpy arrays: the second-order map evaluated
+        through autograd, the role of the reference's ``double_backward_cpu``
+        (_torch/NPDoubleBackwardMixin.py:17-59)."""
+        dev = "cuda"
+        x, y, w, g = (torch.tensor(np.asarray(a), device=dev, requires_grad=True)
+                      for a in (in1, in2, weights, out_grad))
+        cot = [torch.tensor(np.asarray(a), device=dev) for a in (in1_dgrad, in2_dgrad, weights_dgrad)]
+        first = torch.autograd.grad(self.forward(x, y, w), [x, y, w], g, create_graph=True, retain_graph=True)
+        second = torch.autograd.grad(first, [x, y, w, g], cot)
+        return tuple(t.detach().cpu().numpy() for t in second)
+
 
 class ConvolutionTiming:
     """Mixin for ``TensorProductConv``; ``graph`` is a ``CoordGraph``."""
@@ -125,3 +156,26 @@ class ConvolutionTiming:
         t = time_call(lambda: z.backward(gradient=G, retain_graph=True, inputs=[X, Y, W]), num_warmup, num_iter,
                       X.device)
         return self._stats("backward", t, graph, num_warmup, num_iter, prng_seed)
+
+    def benchmark_double_backward(self, num_warmup, num_iter, graph, prng_seed=12345,
+                                  kernel_names=("double_backward_a", "double_backward_b")):
+        """Same protocol as the batch module's: gradient of the sum of the norms of (dX, dY, dW) with
+        respect to X, Y, W and the output gradient."""
+        X, Y, W, G = self._random_buffers(graph, prng_seed)
+        X, Y, W, G = (t.requires_grad_(True) for t in (X, Y, W, G))
+        rows, cols, perm = self._graph_tensors(graph)
+        z = self.forward(X, Y, W, rows, cols, perm)
+        first = torch.autograd.grad(z, [X, Y, W], G, create_graph=True, retain_graph=True)
+        dummy = sum(torch.norm(t) for t in first)
+        t = time_call(lambda: torch.autograd.grad(dummy, [X, Y, W, G], retain_graph=True), num_warmup, num_iter,
+                      X.device)
+        low = self._low
+        wn = 0 if low.shared_weights else low.WN
+        stats = self._stats("backward", t, graph, num_warmup, num_iter, prng_seed)
+        data = (3 * graph.nnz * (low.L2 + wn) + graph.node_count * (3 * low.L1 + 2 * low.L3)) * low.elem_size
+        tt = np.asarray(t, dtype=np.float64)
+        stats.update(direction="double_backward", data_per_tp=data / max(1, graph.nnz),
+                     bandwidth_gbps=[float(v) for v in data / (tt * 1e6)])
+        stats.pop("throughputs_gflops", None)
+        stats.pop("flops_per_tp", None)
+        return stats

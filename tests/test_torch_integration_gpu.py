@@ -163,6 +163,15 @@ def test_benchmark_helpers():
     assert whole.shape == (4,) and np.all(whole > 0) and np.all(kernel > 0) and kernel.min() <= whole.max()
     back = tp.benchmark_backward(2, 3, x, y, g, w, with_torch_overhead=False)
     assert back.shape == (3,) and np.all(back > 0)
+    dd_whole = tp.benchmark_double_backward(1, 3, x, y, w, w)
+    dd_kernel = tp.benchmark_double_backward(1, 3, x, y, w, w, with_torch_overhead=False)
+    assert dd_whole.shape == (3,) and np.all(dd_kernel > 0) and dd_kernel.min() <= dd_whole.max()
+    # the second-order map as numpy arrays, against the first-order kernels by linearity in dZ:
+    # with zero cotangents for dY and dW, d/d(dZ) = F(A, Y, W)
+    a = np.random.default_rng(3).uniform(size=x.shape).astype(np.float32)
+    second = tp.double_backward(x, y, g, w, np.zeros_like(w), a, np.zeros_like(y))
+    f_a = tp(*to_gpu(a, y, w)).cpu().numpy()
+    assert err(second[3], f_a) <= 1e-5
     coords, rows, cols, _ = periodic_radius_graph(300, 12, 5.0, 0)
     graph = CoordGraph(coords, rows, cols)
     for det in (True, False):
@@ -170,3 +179,5 @@ def test_benchmark_helpers():
         for stats in (conv.benchmark_forward(1, 3, graph), conv.benchmark_backward(1, 3, graph)):
             assert len(stats["time_millis"]) == 3 and min(stats["time_millis"]) > 0
             assert stats["graph_adj_nnz"] == graph.nnz and min(stats["throughputs_gflops"]) > 0
+        stats = conv.benchmark_double_backward(1, 2, graph)
+        assert stats["direction"] == "double_backward" and min(stats["time_millis"]) > 0
