@@ -1648,7 +1648,23 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         mode = rt.CONV_GROUPED if t["conv_sort"] else rt.CONV_ATOMIC
     walk = mode != rt.CONV_ATOMIC  # kernels walk per-node edge segments
     em = UvuEmitter(low, acc_budget_words=t["conv_acc"], kahan=kahan)
-    if em.stage is None and em.can_preload and "conv_acc" not in os.environ.get("OEQ_AMD_TUNE", ""):
+    # fp64 with rows that fill the wave: when everything a node needs (accumulators or gradient slice, one
+    # operand set) fits the 512 registers a lane has at one wave per SIMD, that beats walking the edges once
+    # per output segment / sharing the node between waves (MACE shape, fp64: forward 18.4 -> 12.5 ms,
+    # backward 42.1 -> 26.4 ms). The same plan loses for every fp32 problem tried.
+    user_tune = os.environ.get("OEQ_AMD_TUNE", "")
+    wide64 = low.elem_size == 8 and em.R == 1 and not kahan and walk and not low.shared_weights
+    if wide64 and "conv_acc" not in user_tune and "conv_wf" not in user_tune:
+        x_all = sum(low.in1[b].d for b in em.used_in1)
+        need_f = 2 * (sum(low.out[io].d for io in em.used_out) + x_all + em.n_wslots + low.L2) + 40
+        if len(em.segments) > 1 and need_f <= 480:
+            t["conv_acc"], t["conv_wf"] = 1 << 20, 1
+            t["conv_trs"] &= ~1
+            em = UvuEmitter(low, acc_budget_words=t["conv_acc"], kahan=kahan)
+    if wide64 and not any(k in user_tune for k in ("conv_wb", "conv_gres", "conv_split")):
+        if 240 < em.backward_words(True) <= 480:
+            t["conv_wb"], t["conv_gres"], t["conv_split"] = 1, 1, 0
+    if em.stage is None and em.can_preload and "conv_acc" not in user_tune and t["conv_acc"] < (1 << 20):
         # Forward without LDS staging keeps two operand sets of an edge (X blocks, the weights of the
         # output segment's paths, Y) beside the accumulators: shrink the segments until that fits, and
         # give up the prefetch when even 48-word segments do not.
