@@ -37,8 +37,16 @@ def _odd():
                           (0, 0, 2, "uvu", True)], shared_weights=False, internal_weights=False)
 
 
+def _wide_v():
+    # more second-operand channels than the emitters unroll: the v loop stays a loop
+    return oeq.TPProblem("4x1e+7x0e", "12x1e+10x0e", "4x0e+4x1e+7x1e",
+                         [(0, 0, 0, "uvu", True), (0, 1, 1, "uvu", True), (1, 0, 2, "uvu", True)],
+                         shared_weights=False, internal_weights=False)
+
+
 CASES = [
     ("cfg1", P.config1_single_uvu, 1000),
+    ("wide-v", _wide_v, 211),
     ("odd", _odd, 333),
     ("odd-f64", lambda: _f64(_odd()), 333),
     ("cfg2", P.config2_nequip_uvu, 257),
