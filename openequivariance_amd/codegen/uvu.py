@@ -71,6 +71,7 @@ class UvuEmitter:
         self.fence_words = 0  # gradient registers between two scheduling fences (0: a fence after every path)
         self.seg_waves = 1  # conv forward: waves per node that share its output segments between them
         self.bwd_groups: Optional[List[List[int]]] = None  # conv backward: output blocks owned by each wave
+        self.group_budget = 0  # gradient words per wave when a node is shared between waves (0: default)
         # plain stores of [64 x d] channel blocks go through the s_tr tile as well: bit 0 = forward outputs,
         # bit 1 = backward dX (kernels that use it declare the tile)
         self.tr_stores = 0
@@ -1290,7 +1291,7 @@ class UvuEmitter:
         if fits or low.shared_weights or not self.can_preload or self.R != 1:
             return None
         # room for the edge operands, dX, dY (and deferred dW) beside the wave's share of the gradient
-        budget = max(1, (96 if not self.ragged() else 64) // self.words)
+        budget = max(1, (self.group_budget or (96 if not self.ragged() else 64)) // self.words)
         sizes = [low.out[io].d for io in self.used_out]
         n = max(2 if self.g_resident else 1, -(-sum(sizes) // budget))
         while n <= max_waves:
@@ -1638,7 +1639,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=112, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
-                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200))
+                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -1708,9 +1709,15 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     xcd_b = 1 if (walk and low.shared_weights) else xcd  # bounded grid: one partial dW row per wave group
     blk_f = em.emit_conv_forward(s, G_f, walk, t["conv_pipe_f"], t["conv_wf"], xcd, bool(t["conv_tra"]))
     gres = None if t["conv_gres"] < 0 else bool(t["conv_gres"])
+    em.group_budget = t["conv_gbud"]
     em.bwd_groups = em.plan_backward_groups(8 // em.NCH) if (walk and t["conv_split"] and gres is None) else None
     if em.bwd_groups:
         G_b = 1
+        wpb = em.NCH * len(em.bwd_groups)
+        if 8 % wpb and 12 % wpb == 0 and "conv_wb" not in user_tune:
+            # blocks of 3 waves leave a quarter of the wave slots empty at 2 waves per SIMD (8 per CU); at 3
+            # per SIMD they fill them (SevenNet main layer: 14.6 -> 10.1 ms)
+            t["conv_wb"] = 3
         blk_b = em.emit_conv_backward_split(s, t["conv_wb"], xcd)
     else:
         blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd_b,
