@@ -1588,7 +1588,7 @@ def tp_module(low: Lowered, compute_units: int = 256):
     on_demand = big or probe.backward_words(True) > (250 if f32 else 420)
     t = tuning(dict(tp_acc=48, tp_gf=1 if wide else 4, tp_gb=1 if wide else 4,
                     tp_wf=2 if f32 else 0, tp_wb=3 if big else 2, tp_nt=0, tp_gres=0 if on_demand else 1,
-                    tp_sb=1 if on_demand else 0, tp_trs=1, tp_fw=0,
+                    tp_sb=1 if on_demand else 0, tp_trs=1, tp_fw=64,
                     tp_dd=1, dd_wa=2, dd_wb=2))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
