@@ -1,7 +1,11 @@
 """Timing helpers on the two modules, with the call signatures of the reference's
 ``benchmark_forward`` / ``benchmark_backward`` / ``benchmark_double_backward``
 (openequivariance/openequivariance/core/TensorProductBase.py:69-175,
-core/ConvolutionBase.py:134-290, core/utils.py:152-205).
+core/ConvolutionBase.py:134-290, core/utils.py:152-205), and the numpy-in / numpy-out
+helpers its correctness harness drives (``forward_cpu``, ``backward_cpu``,
+``double_backward_cpu``: _torch/TensorProduct.py:138-178, _torch/TensorProductConv.py:209-275,
+_torch/NPDoubleBackwardMixin.py). Despite their names the latter run on the GPU: "cpu" says where
+the caller's arrays live.
 
 ``with_torch_overhead=True`` times the whole op call with events on torch's current
 stream; ``False`` returns the device time of the kernels alone, taken with HIP events
@@ -94,10 +98,18 @@ class TensorProductTiming:
         return time_call(lambda: torch.autograd.grad(dummy, [x, y, w, g], dummy_grad, retain_graph=True),
                          num_warmup, num_iter, x.device, entry, roles)
 
-    def double_backward(self, in1, in2, out_grad, weights, weights_dgrad, in1_dgrad, in2_dgrad):
+    def forward_cpu(self, L1_in, L2_in, L3_out, weights) -> None:
+        x, y, w = (torch.tensor(np.asarray(a), device="cuda") for a in (L1_in, L2_in, weights))
+        L3_out[:] = self.forward(x, y, w).cpu().numpy()
+
+    def backward_cpu(self, L1_in, L1_grad, L2_in, L2_grad, L3_grad, weights, weights_grad) -> None:
+        x, y, w = (torch.tensor(np.asarray(a), device="cuda", requires_grad=True) for a in (L1_in, L2_in, weights))
+        self.forward(x, y, w).backward(gradient=torch.tensor(np.asarray(L3_grad), device="cuda"))
+        L1_grad[:], L2_grad[:], weights_grad[:] = (t.grad.cpu().numpy() for t in (x, y, w))
+
+    def double_backward_cpu(self, in1, in2, out_grad, weights, weights_dgrad, in1_dgrad, in2_dgrad):
         """(in1_grad, in2_grad, weights_grad, out_dgrad) as numpy arrays: the second-order map evaluated
-        through autograd, the role of the reference's ``double_backward_cpu``
-        (_torch/NPDoubleBackwardMixin.py:17-59)."""
+        through autograd (_torch/NPDoubleBackwardMixin.py:17-59 of the reference)."""
         dev = "cuda"
         x, y, w, g = (torch.tensor(np.asarray(a), device=dev, requires_grad=True)
                       for a in (in1, in2, weights, out_grad))
@@ -105,6 +117,8 @@ class TensorProductTiming:
         first = torch.autograd.grad(self.forward(x, y, w), [x, y, w], g, create_graph=True, retain_graph=True)
         second = torch.autograd.grad(first, [x, y, w, g], cot)
         return tuple(t.detach().cpu().numpy() for t in second)
+
+    double_backward = double_backward_cpu
 
 
 class ConvolutionTiming:
@@ -141,6 +155,27 @@ class ConvolutionTiming:
             "throughputs_gflops": [float(v) for v in flops * graph.nnz / (t * 1e6)],
             "bandwidth_gbps": [float(v) for v in data / (t * 1e6)],
         }
+
+    def forward_cpu(self, L1_in, L2_in, weights, L3_out, graph) -> None:
+        x, y, w = (torch.tensor(np.asarray(a), device="cuda") for a in (L1_in, L2_in, weights))
+        L3_out[:] = self.forward(x, y, w, *self._graph_tensors(graph)).cpu().numpy()
+
+    def backward_cpu(self, L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, graph) -> None:
+        x, y, w = (torch.tensor(np.asarray(a), device="cuda", requires_grad=True) for a in (L1_in, L2_in, weights))
+        z = self.forward(x, y, w, *self._graph_tensors(graph))
+        z.backward(gradient=torch.tensor(np.asarray(L3_grad), device="cuda"))
+        L1_grad[:], L2_grad[:], weights_grad[:] = (t.grad.cpu().numpy() for t in (x, y, w))
+
+    def double_backward_cpu(self, in1, in2, out_grad, weights, weights_dgrad, in1_dgrad, in2_dgrad, graph):
+        """(in1_grad, in2_grad, weights_grad, out_dgrad) as numpy arrays
+        (_torch/NPDoubleBackwardMixin.py:145-193 of the reference)."""
+        x, y, w, g = (torch.tensor(np.asarray(a), device="cuda", requires_grad=True)
+                      for a in (in1, in2, weights, out_grad))
+        cot = [torch.tensor(np.asarray(a), device="cuda") for a in (in1_dgrad, in2_dgrad, weights_dgrad)]
+        z = self.forward(x, y, w, *self._graph_tensors(graph))
+        first = torch.autograd.grad(z, [x, y, w], g, create_graph=True, retain_graph=True)
+        second = torch.autograd.grad(first, [x, y, w, g], cot)
+        return tuple(t.detach().cpu().numpy() for t in second)
 
     def benchmark_forward(self, num_warmup, num_iter, graph, prng_seed=12345, kernel_names=("forward",)):
         X, Y, W, _ = self._random_buffers(graph, prng_seed)

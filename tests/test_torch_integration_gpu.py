@@ -171,7 +171,7 @@ def test_benchmark_helpers():
     # the second-order map as numpy arrays, against the first-order kernels by linearity in dZ:
     # with zero cotangents for dY and dW, d/d(dZ) = F(A, Y, W)
     a = np.random.default_rng(3).uniform(size=x.shape).astype(np.float32)
-    second = tp.double_backward(x, y, g, w, np.zeros_like(w), a, np.zeros_like(y))
+    second = tp.double_backward_cpu(x, y, g, w, np.zeros_like(w), a, np.zeros_like(y))
     f_a = tp(*to_gpu(a, y, w)).cpu().numpy()
     assert err(second[3], f_a) <= 1e-5
     coords, rows, cols, _ = periodic_radius_graph(300, 12, 5.0, 0)
@@ -183,3 +183,38 @@ def test_benchmark_helpers():
             assert stats["graph_adj_nnz"] == graph.nnz and min(stats["throughputs_gflops"]) > 0
         stats = conv.benchmark_double_backward(1, 2, graph)
         assert stats["direction"] == "double_backward" and min(stats["time_millis"]) > 0
+
+
+def test_numpy_interface():
+    """forward_cpu / backward_cpu / double_backward_cpu: numpy arrays in, results written into (or
+    returned as) numpy arrays, as the reference's correctness harness calls them."""
+    from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
+    problem = P.config2_nequip_uvu()
+    ref = R.Problem.from_spec(problem)
+    x, y, w, g = tp_inputs(problem, 300, seed=2)
+    tp = oeq.TensorProduct(problem)
+    z, dx, dy, dw = np.zeros_like(g), np.zeros_like(x), np.zeros_like(y), np.zeros_like(w)
+    tp.forward_cpu(x, y, z, w)
+    tp.backward_cpu(x, dx, y, dy, g, w, dw)
+    for got, want in zip((z, dx, dy, dw), (R.tp_forward(ref, x, y, w),) + tuple(R.tp_backward(ref, x, y, w, g))):
+        assert err(got, want) <= 1e-5
+    coords, rows, cols, _ = periodic_radius_graph(50, 8.0, 4.0, 1)
+    graph = CoordGraph(coords, rows, cols)
+    rng = np.random.default_rng(4)
+    X = rng.uniform(size=(50, problem.irreps_in1.dim)).astype(np.float32)
+    Y = rng.uniform(size=(graph.nnz, problem.irreps_in2.dim)).astype(np.float32)
+    W = rng.uniform(size=(graph.nnz, problem.weight_numel)).astype(np.float32)
+    G = rng.uniform(size=(50, problem.irreps_out.dim)).astype(np.float32)
+    for det in (True, False):
+        conv = oeq.TensorProductConv(problem, deterministic=det)
+        Z, dX, dY, dW = np.zeros_like(G), np.zeros_like(X), np.zeros_like(Y), np.zeros_like(W)
+        conv.forward_cpu(X, Y, W, Z, graph)
+        conv.backward_cpu(X, dX, Y, dY, W, dW, G, graph)
+        want = (R.conv_forward(ref, X, Y, W, graph.rows, graph.cols),) + tuple(
+            R.conv_backward(ref, X, Y, W, G, graph.rows, graph.cols))
+        for got, w_ in zip((Z, dX, dY, dW), want):
+            assert err(got, w_) <= 1e-5
+        # second order with only the X cotangent: d/d(dZ) is the forward pass applied to it
+        A = rng.uniform(size=X.shape).astype(np.float32)
+        second = conv.double_backward_cpu(X, Y, G, W, np.zeros_like(W), A, np.zeros_like(Y), graph)
+        assert err(second[3], R.conv_forward(ref, A, Y, W, graph.rows, graph.cols)) <= 1e-5
