@@ -338,7 +338,7 @@ def main():
         step_dd()
         torch.cuda.synchronize()
         split = {name: ks.timing_collect(role)[0] for name, role in
-                 (("double_backward_a", rt.ROLE_DOUBLE_BACKWARD_A), ("double_backward_b", rt.ROLE_DOUBLE_BACKWARD_B),
+                 (("double_backward_A", rt.ROLE_DOUBLE_BACKWARD_A), ("double_backward_B", rt.ROLE_DOUBLE_BACKWARD_B),
                   ("fixup_backward", rt.ROLE_CONV_FIXUP_BACKWARD))}
         ks.timing_enable(False)
         ms_cmp = time_steps(step_composed, 2, 1)

@@ -81,7 +81,7 @@ class TensorProductTiming:
 
     def benchmark_double_backward(self, num_warmup, num_iter, L1_in, L2_in, weights, weights_grad,
                                   with_torch_overhead=True,
-                                  kernel_names=("double_backward_a", "double_backward_b")) -> np.ndarray:
+                                  kernel_names=("double_backward_A", "double_backward_B")) -> np.ndarray:
         """Time of the gradient of a scalar function of the three first-order gradients with respect to
         X, Y, W and the output gradient (the reference's protocol, TensorProductBase.py:126-175; as
         there, the output gradient is the forward result and ``weights_grad`` is accepted for
@@ -193,7 +193,7 @@ class ConvolutionTiming:
         return self._stats("backward", t, graph, num_warmup, num_iter, prng_seed)
 
     def benchmark_double_backward(self, num_warmup, num_iter, graph, prng_seed=12345,
-                                  kernel_names=("double_backward_a", "double_backward_b")):
+                                  kernel_names=("double_backward_A", "double_backward_B")):
         """Same protocol as the batch module's: gradient of the sum of the norms of (dX, dY, dW) with
         respect to X, Y, W and the output gradient."""
         X, Y, W, G = self._random_buffers(graph, prng_seed)

@@ -4,9 +4,9 @@ The first backward pass maps (X, Y, W, dZ) to (dX, dY, dW). Differentiating it o
 cotangents (A, B, C) for (dX, dY, dW), gives, because the tensor product ``F`` is linear in each
 operand,
 
-    d/d(dZ) = F(A, Y, W) + F(X, B, W) + F(X, Y, C)                         (kernel ``double_backward_a``)
+    d/d(dZ) = F(A, Y, W) + F(X, B, W) + F(X, Y, C)                         (kernel ``double_backward_A``)
     d/dX    = dX-part of backward(., B, W; dZ) + backward(., Y, C; dZ)
-    d/dY    = dY-part of backward(A, ., W; dZ) + backward(X, ., C; dZ)     (kernel ``double_backward_b``)
+    d/dY    = dY-part of backward(A, ., W; dZ) + backward(X, ., C; dZ)     (kernel ``double_backward_B``)
     d/dW    = dW-part of backward(A, Y, .; dZ) + backward(X, B, .; dZ)
 
 The reference computes the same two groups with its kernels ``double_backward_A`` /
@@ -45,7 +45,7 @@ def supported(low: Lowered, conv: bool = False) -> bool:
 
 
 class DoubleEmitter(UvuEmitter):
-    """Adds ``double_backward_a`` / ``double_backward_b`` (batch and convolution flavours) to a module
+    """Adds ``double_backward_A`` / ``double_backward_B`` (batch and convolution flavours) to a module
     whose structs (X_t, G_t) the base emitter has already written."""
 
     # ------------------------------------------------------------ operands
@@ -239,7 +239,7 @@ class DoubleEmitter(UvuEmitter):
         low = self.low
         block = 64 * self.NCH * G
         s.open(
-            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_a(i64 num_batch, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_A(i64 num_batch, '
             "const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
             "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
             "T* __restrict__ L3_dgrad)"
@@ -291,7 +291,7 @@ class DoubleEmitter(UvuEmitter):
             G = 1  # the dY reduction across chunk waves uses block barriers
         block = 64 * self.NCH * G
         s.open(
-            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_b(i64 num_batch, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_B(i64 num_batch, '
             "const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
             "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
             "const T* __restrict__ L3_grad, T* __restrict__ L1_grad, T* __restrict__ L2_grad, T* __restrict__ W_grad)"
@@ -377,7 +377,7 @@ class DoubleEmitter(UvuEmitter):
         segw = max(1, min(segw, len(self.segments))) if self.R == 1 else 1
         block = 64 * self.NCH * G * segw
         s.open(
-            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_a(i64 node_count, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_A(i64 node_count, '
             f"i64 nnz, {self._CONV_OPERANDS}T* __restrict__ L3_dgrad, const i64* __restrict__ rows, "
             "const i64* __restrict__ cols, const i64* __restrict__ rowptr, const i64* __restrict__ eperm)"
         )
@@ -426,7 +426,7 @@ class DoubleEmitter(UvuEmitter):
             G = 1
         block = 64 * self.NCH * G
         s.open(
-            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_b(i64 node_count, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_B(i64 node_count, '
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
@@ -563,7 +563,7 @@ class DoubleEmitter(UvuEmitter):
         gpaths = [[p for p in low.paths if p.io in grp] for grp in groups]
         gin1 = [sorted({p.i1 for p in ps}) for ps in gpaths]
         s.open(
-            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_b(i64 node_count, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_B(i64 node_count, '
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
@@ -680,8 +680,8 @@ def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict) -> List[t
     blk_a = em.emit_tp_double_a(s, G, tune.get("dd_wa", 2))
     blk_b = em.emit_tp_double_b(s, G, tune.get("dd_wb", 2))
     G_b = 1 if em.NCH > 1 else G
-    return [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_a", blk_a, G * em.R, 0),
-            (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_b", blk_b, G_b * em.R, 0)]
+    return [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_A", blk_a, G * em.R, 0),
+            (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_b, G_b * em.R, 0)]
 
 
 def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: int) -> List[tuple]:
@@ -712,14 +712,14 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
         segw = min(len(em.segments), max(1, tune.get("dd_segw", 4)), 8 // em.NCH) if em.R == 1 else 1
         G_a = max(1, min(G, 8 // (em.NCH * segw)))
         blk_a = em.emit_conv_double_a(s, G_a, tune.get("dd_wa", 2), xcd, segw)
-        descs.append((rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_a", blk_a, G_a, 0, xcd))
+        descs.append((rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_A", blk_a, G_a, 0, xcd))
     if groups:
         blk_b = em.emit_conv_double_b_split(s, groups, tune.get("dd_wb", 2), xcd)
         G_b = 1
     else:
         blk_b = em.emit_conv_double_b(s, G, tune.get("dd_wb", 2), xcd)
         G_b = 1 if em.NCH > 1 else G
-    return descs + [(rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_b", blk_b, G_b, 0, xcd)]
+    return descs + [(rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_b, G_b, 0, xcd)]
 
 
 def _emit_segment_structs(s: Src, em: DoubleEmitter, prefix: str):

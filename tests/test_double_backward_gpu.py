@@ -1,4 +1,4 @@
-"""The fused second-order kernels (`double_backward_a` / `double_backward_b`) against the composition of
+"""The fused second-order kernels (`double_backward_A` / `double_backward_B`) against the composition of
 first-order kernels, which tests/test_higher_derivatives_gpu.py checks against float64 autograd through the
 CPU restatement. Also through autograd: the force-training pattern (gradient of a function of the first
 gradients) with the fused route switched on and off."""
