@@ -170,7 +170,8 @@ def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
-              "use --gpus 1. See DESIGN.md for how the path would shard.", file=sys.stderr)
+              "use --gpus 1. (Sharding would split the receivers into contiguous blocks with a halo "
+              "exchange of sender rows; it is not built.)", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
