@@ -38,6 +38,11 @@ def _cases():
                 out.append(_single(mode, m, irs[(2 * n + q) % len(irs)], dtype))
     out += P.mace_problems() + P.diffdock_problems() + P.e3tools_problems()
     out += P.nequix_problems() + P.seven_net_problems()  # a different multiplicity per irrep
+    # ... with an input block no instruction reads and an output block no instruction writes
+    out.append(oeq.TPProblem("100x0e+70x1o+40x2e+96x1e", "1x0e+2x1o", "100x0e+70x1o+100x1o+40x1o+33x2e",
+                             [(0, 0, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 1, 2, "uvu", True),
+                              (2, 1, 3, "uvu", True, 0.7)], shared_weights=False, internal_weights=False,
+                             label="folded-gaps"))
     shared = P.mace_problems()[0].clone()
     shared.shared_weights = True
     shared.label = "mace-large-shared"

@@ -37,6 +37,13 @@ def _odd():
                           (0, 0, 2, "uvu", True)], shared_weights=False, internal_weights=False)
 
 
+def _folded():
+    # wide row with a different multiplicity per irrep, unread input block, unwritten output block
+    return oeq.TPProblem("100x0e+70x1o+40x2e+96x1e", "1x0e+2x1o", "100x0e+70x1o+100x1o+40x1o+33x2e",
+                         [(0, 0, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 1, 2, "uvu", True),
+                          (2, 1, 3, "uvu", True, 0.7)], shared_weights=False, internal_weights=False)
+
+
 def _wide_v():
     # more second-operand channels than the emitters unroll: the v loop stays a loop
     return oeq.TPProblem("4x1e+7x0e", "12x1e+10x0e", "4x0e+4x1e+7x1e",
@@ -47,6 +54,7 @@ def _wide_v():
 CASES = [
     ("cfg1", P.config1_single_uvu, 1000),
     ("wide-v", _wide_v, 211),
+    ("folded-gaps", _folded, 61),
     ("odd", _odd, 333),
     ("odd-f64", lambda: _f64(_odd()), 333),
     ("cfg2", P.config2_nequip_uvu, 257),

@@ -27,6 +27,15 @@ def _odd_uvw(shared):
                          internal_weights=False, label="odd-uvw")
 
 
+def _folded_with_gaps():
+    # a row wider than a wave with a different multiplicity per irrep (folded into 64-channel pieces), one
+    # input block no instruction reads, one output block no instruction writes, second operand with mul 2
+    return oeq.TPProblem("100x0e+70x1o+40x2e+96x1e", "1x0e+2x1o", "100x0e+70x1o+100x1o+40x1o+33x2e",
+                         [(0, 0, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 1, 2, "uvu", True),
+                          (2, 1, 3, "uvu", True, 0.7)], shared_weights=False, internal_weights=False,
+                         label="folded-gaps")
+
+
 def _as_f64(problem):
     q = problem.clone()
     q.irrep_dtype, q.weight_dtype = np.float64, np.float64
@@ -57,6 +66,8 @@ CASES = [
                                                       shared_weights=False, internal_weights=False), 33),
     # production layers with a different multiplicity per irrep (rows wider than a wave: the chunks of a
     # row then run different code), one with 89 channels
+    ("folded-gaps", _folded_with_gaps, 61),
+    ("folded-gaps-f64", lambda: _as_f64(_folded_with_gaps()), 37),
     ("nequix-first", lambda: P.nequix_problems()[0], 53),
     ("nequix-main", lambda: P.nequix_problems()[1], 53),
     ("nequix-last", lambda: P.nequix_problems()[2], 53),
