@@ -31,6 +31,9 @@ def _pow2ceil(n: int) -> int:
 class UvwEmitter:
     def __init__(self, low: Lowered):
         assert low.mode == "uvw"
+        from .uvu import tuning
+        self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576))
+        self.TILE_BYTES = self.tune["uvw_tile"]
         self.low = low
         self.T = low.ctype
         self.l2_pad = _pow2ceil(low.L2)
@@ -136,7 +139,9 @@ class UvwEmitter:
         return block
 
     # ------------------------------------------------------------ backward
-    TILE_BYTES = 12288  # per-wave LDS budget for one path's weight tile (larger blocks are accessed directly)
+    # TILE_BYTES (set from the uvw_tile knob): per-wave LDS budget for one path's weight tile; larger
+    # blocks are accessed directly. 24 KB takes in [64 x 80] blocks (e3tools convolution: 44 % -> 59 % of
+    # HBM peak); with the loads of the next tile in flight during a step, fewer waves per CU no longer hurt.
 
     def _tile_plan(self, p: Path):
         """Per-row weights of a path and one 64-channel chunk of u form a contiguous [rows, V, W] block.
@@ -164,12 +169,13 @@ class UvwEmitter:
         tiled = [p for p in low.paths if plans[p.index]]
         waves = WAVES_PER_BLOCK
         if tiled:
-            tile_elems = (max(plans[p.index][0] for p in tiled) + 3) // 4 * 4
-            g_elems = max(low.out[p.io].mul * low.out[p.io].d for p in tiled)
+            # rows of the tile start an odd number of elements apart: lanes reading the same column of
+            # their rows hit different banks
+            tile_elems = (max(min(64, low.in1[p.i1].mul) * self._row_stride(p) for p in tiled) + 3) // 4 * 4
             vw = 16 // low.elem_size
             s(f"struct __attribute__((aligned(16))) wvec_t {{ T v[{vw}]; }};")
             # keep a block's LDS near 40 KB, so that four blocks (and at least four waves) share a CU
-            per_wave = (tile_elems + g_elems) * low.elem_size
+            per_wave = tile_elems * low.elem_size
             waves = max(1, min(WAVES_PER_BLOCK, 40960 // per_wave))
         # shared weights: each wave sums its rows' weight gradients in an LDS copy of the weight tensor
         # (when that fits) and writes it out once, instead of a read-modify-write of global memory per row
@@ -188,9 +194,8 @@ class UvwEmitter:
             "const T* __restrict__ L3_grad, T* __restrict__ wpartial)"
         )
         if tiled:
-            # one path's weights of the row, then (in place) its weight gradients; and that path's dZ block
+            # one path's weights of the row, then (in place) its weight gradients
             s(f"__shared__ __attribute__((aligned(16))) T s_w[{waves}][{tile_elems}];")
-            s(f"__shared__ T s_g[{waves}][{g_elems}];")
         if shared:
             s(f"T* prow = wpartial + ((i64)blockIdx.x * {waves} + oeq_wave()) * {low.WN};")
             if self.shared_lds:
@@ -199,6 +204,11 @@ class UvwEmitter:
                 s("oeq_wave_sync();")
             else:
                 s("bool first = true;")
+        if tiled:
+            steps0 = [(i1, c, p) for i1, b1 in enumerate(low.in1) for c in range((b1.mul + 63) // 64)
+                      for p in low.paths if p.i1 == i1 and plans[p.index]]
+            nv_max = max(self._pad_vectors(st[2], st[1] * 64, plans[st[2].index][1]) for st in steps0)
+            s(f"wvec_t pf[{nv_max}];  // the next weight tile on its way from global memory to LDS")
         self._row_loop_open(s, waves)
         s(f"const T* xrow = L1_in + rowc * {low.L1};")
         s(f"const T* yrow = L2_in + rowc * {low.L2};")
@@ -209,27 +219,46 @@ class UvwEmitter:
             s(f"T* dwrow = W_grad + rowc * {low.WN};")
         s(f"T dy[{self.l2_pad}];")
         s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
+        pipelined = bool(tiled)
+        if pipelined:
+            # Every (input block, 64-channel chunk, path) is a step known at generation time. The weight
+            # tile of the next tiled step is requested from global memory into registers (pf) before the
+            # current step computes, and written to LDS when that step is done: one exposed memory latency
+            # per row instead of one per path.
+            steps = [(i1, c, p) for i1, b1 in enumerate(low.in1) for c in range((b1.mul + 63) // 64)
+                     for p in low.paths if p.i1 == i1]
+            tsteps = [st for st in steps if plans[st[2].index]]
+            self._pad_issue(s, tsteps[0][2], tsteps[0][1] * 64, plans[tsteps[0][2].index][1])
         for i1, b1 in enumerate(low.in1):
             paths = [p for p in low.paths if p.i1 == i1]
             s(f"// ---- in1[{i1}]: {b1.mul} x l={b1.l}")
-            s.open(f"for (int uc = 0; uc < {b1.mul}; uc += 64)")
-            s("const int u = uc + lane;")
-            s(f"const bool uok = u < {b1.mul};")
-            s(f"T x[{b1.d}], dx[{b1.d}];")
-            for i in range(b1.d):
-                s(f"x[{i}] = uok ? xrow[{b1.off} + u * {b1.d} + {i}] : T(0); dx[{i}] = T(0);")
-            for p in paths:
-                b2, bo = low.in2[p.i2], low.out[p.io]
-                s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
-                if plans[p.index]:
-                    self._bwd_path_tiled(s, p, plans[p.index][1])
+            chunks = range((b1.mul + 63) // 64) if pipelined else [None]
+            for c in chunks:
+                if c is None:
+                    s.open(f"for (int uc = 0; uc < {b1.mul}; uc += 64)")
                 else:
-                    self._bwd_path_direct(s, p)
-            s.open("if (live && uok)")
-            for i in range(b1.d):
-                s(f"dxrow[{b1.off} + u * {b1.d} + {i}] = dx[{i}];")
-            s.close()
-            s.close()
+                    s.open("")
+                    s(f"const int uc = {c * 64};")
+                s("const int u = uc + lane;")
+                s(f"const bool uok = u < {b1.mul};")
+                s(f"T x[{b1.d}], dx[{b1.d}];")
+                for i in range(b1.d):
+                    s(f"x[{i}] = uok ? xrow[{b1.off} + u * {b1.d} + {i}] : T(0); dx[{i}] = T(0);")
+                for p in paths:
+                    b2, bo = low.in2[p.i2], low.out[p.io]
+                    s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
+                    if plans[p.index] and pipelined:
+                        k = tsteps.index((i1, c, p))
+                        nxt = tsteps[k + 1] if k + 1 < len(tsteps) else None
+                        self._bwd_path_padded(s, p, plans[p.index][1], c * 64,
+                                              (nxt[2], nxt[1] * 64, plans[nxt[2].index][1]) if nxt else None)
+                    else:
+                        self._bwd_path_direct(s, p)
+                s.open("if (live && uok)")
+                for i in range(b1.d):
+                    s(f"dxrow[{b1.off} + u * {b1.d} + {i}] = dx[{i}];")
+                s.close()
+                s.close()
         if shared and not self.shared_lds:
             s("first = false;")
         # dY: butterfly over the 64 lanes
@@ -342,66 +371,111 @@ class UvwEmitter:
         s.close()
         s.close()
 
-    def _bwd_path_tiled(self, s: Src, p: Path, vw: int):
-        """Per-row weights: the path's contiguous [rows, V, W] weight block of this u chunk is copied to
-        the wave's LDS tile with coalesced 16-byte accesses; lane u then walks its rows of the tile, the
-        weight gradients replace the weights in place and the tile is written back coalesced. Lane u
-        visits w in the rotated order (u + t) mod W, which spreads the lanes of a wave over the LDS banks
-        whatever the row stride; dZ of the path's output irrep is read from LDS in the same order."""
+    def _row_stride(self, p: Path) -> int:
+        per_u = self.low.in2[p.i2].mul * self.low.out[p.io].mul
+        return per_u | 1
+
+    def _pad_geometry(self, p: Path, uc: int, vw: int):
+        low = self.low
+        b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
+        per_u = b2.mul * bo.mul
+        nrows = min(64, b1.mul - uc)
+        return per_u, nrows * per_u, p.woff + uc * per_u, self._row_stride(p)
+
+    def _pad_vectors(self, p: Path, uc: int, vw: int) -> int:
+        _, nel, _, _ = self._pad_geometry(p, uc, vw)
+        return -(-nel // (64 * vw))
+
+    def _pad_issue(self, s: Src, p: Path, uc: int, vw: int):
+        """Request this lane's share of a step's contiguous weight block (coalesced 16-byte reads)."""
+        per_u, nel, tbase, _ = self._pad_geometry(p, uc, vw)
+        for q in range(self._pad_vectors(p, uc, vw)):
+            t = f"(lane + {64 * q}) * {vw}"
+            guard = "" if (64 * q + 64) * vw <= nel else f"if ({t} < {nel}) "
+            if vw > 1:
+                s(f"{guard}pf[{q}] = *(const wvec_t*)(wrow + {tbase} + {t});")
+            else:
+                s(f"{guard}pf[{q}].v[0] = wrow[{tbase} + {t}];")
+
+    def _pad_commit(self, s: Src, p: Path, uc: int, vw: int):
+        """Registers -> padded LDS tile (row r of the block starts at r * S)."""
+        per_u, nel, _, S = self._pad_geometry(p, uc, vw)
+        for q in range(self._pad_vectors(p, uc, vw)):
+            t = f"(lane + {64 * q}) * {vw}"
+            s.open("" if (64 * q + 64) * vw <= nel else f"if ({t} < {nel})")
+            s(f"const int t = {t};")
+            if per_u % vw == 0:
+                s(f"const int tr = t / {per_u};")
+                s(f"T* dst = tw + tr * {S - per_u} + t;")
+                for i in range(vw):
+                    s(f"dst[{i}] = pf[{q}].v[{i}];")
+            else:  # a vector can straddle two rows
+                for i in range(vw):
+                    s(f"tw[(t + {i}) / {per_u} * {S - per_u} + t + {i}] = pf[{q}].v[{i}];")
+            s.close()
+
+    def _bwd_path_padded(self, s: Src, p: Path, vw: int, uc: int, nxt):
+        """One step of the pipelined per-row-weight backward. The step's weights are in ``pf``; they go
+        to the wave's LDS tile, whose rows start an odd number of elements apart: lane u can then walk
+        its row front to back (all lanes at the same column) without bank conflicts and with addresses
+        that are constants within the unrolled loops. dZ of the path's output irrep is the same for every
+        lane: it is read through the scalar cache and enters the multiply-adds as scalar operands. Weight
+        gradients replace the weights in the tile, which is copied out coalesced. ``nxt``: the next tiled
+        step, whose weights are requested as soon as ``pf`` is free."""
         low = self.low
         b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
         V, Wn = b2.mul, bo.mul
-        per_u = V * Wn
+        per_u, nel, tbase, S = self._pad_geometry(p, uc, vw)
+        unroll = max(1, self.tune["uvw_unroll"])
         s.open("")
-        s(f"const int nrows = ({b1.mul} - uc < 64) ? {b1.mul} - uc : 64;")
-        s(f"const int nel = nrows * {per_u};")
-        s(f"const i64 tbase = {p.woff} + (i64)uc * {per_u};")
         s("T* tw = s_w[wave];")
-        s("T* tg = s_g[wave];")
-        s("oeq_wave_sync();  // the previous path's tile and dZ block are no longer read")
-        s(f"for (int t = lane; t < {Wn * bo.d}; t += 64) tg[t] = grow[{bo.off} + t];")
-        if vw > 1:
-            s(f"for (int t = lane * {vw}; t < nel; t += {64 * vw}) "
-              f"*(wvec_t*)(tw + t) = *(const wvec_t*)(wrow + tbase + t);")
-        else:
-            s("for (int t = lane; t < nel; t += 64) tw[t] = wrow[tbase + t];")
+        s(f"const T* gq = grow + {bo.off};  // wave-uniform")
+        s("oeq_wave_sync();  // the previous step's tile is no longer read")
+        self._pad_commit(s, p, uc, vw)
+        if nxt is not None:
+            self._pad_issue(s, *nxt)
         s("oeq_wave_sync();")
-        s(f"const int urow = uok ? lane : 0;  // lanes without a channel read row 0 and store nothing")
-        s(f"const int w0 = lane % {Wn};")
+        s("const int urow = uok ? lane : 0;  // lanes without a channel read row 0 and store nothing")
         s.open(f"for (int v = 0; v < {V}; ++v)")
         prods = self._products(s, p)
-        s(f"T* trow = tw + (urow * {V} + v) * {Wn};")
+        s(f"T* trow = tw + urow * {S} + v * {Wn};")
         for k in range(bo.d):
             s(f"T G{k} = T(0);")
-        s("int wr = w0;")
-        s("#pragma unroll 4")
-        s.open(f"for (int t = 0; t < {Wn}; ++t)")
-        s("const T wv = trow[wr];")
+        s(f"#pragma unroll {unroll}")
+        s.open(f"for (int w = 0; w < {Wn}; ++w)")
+        s("const T wv = trow[w];")
         for k in range(bo.d):
-            s(f"G{k} += wv * tg[wr * {bo.d} + {k}];")
-        s(f"wr = (wr + 1 == {Wn}) ? 0 : wr + 1;")
+            s(f"G{k} += wv * gq[w * {bo.d} + {k}];")
         s.close()
         ks = self._cg_backward(s, p, prods)
-        s("wr = w0;")
         s.open("if (uok)")
-        s("#pragma unroll 4")
-        s.open(f"for (int t = 0; t < {Wn}; ++t)")
-        terms = [f"f{k} * tg[wr * {bo.d} + {k}]" for k in ks]
+        s(f"#pragma unroll {unroll}")
+        s.open(f"for (int w = 0; w < {Wn}; ++w)")
+        terms = [f"f{k} * gq[w * {bo.d} + {k}]" for k in ks]
         s(f"T dwv = {terms[0]};")
         for t in terms[1:]:
             s(f"dwv += {t};")
-        s("trow[wr] = dwv;")
-        s(f"wr = (wr + 1 == {Wn}) ? 0 : wr + 1;")
+        s("trow[w] = dwv;")
         s.close()
         s.close()
         s.close()
         s("oeq_wave_sync();")
         s.open("if (live)")
-        if vw > 1:
-            s(f"for (int t = lane * {vw}; t < nel; t += {64 * vw}) "
-              f"*(wvec_t*)(dwrow + tbase + t) = *(const wvec_t*)(tw + t);")
-        else:
-            s("for (int t = lane; t < nel; t += 64) dwrow[tbase + t] = tw[t];")
+        for q in range(self._pad_vectors(p, uc, vw)):
+            t = f"(lane + {64 * q}) * {vw}"
+            s.open("" if (64 * q + 64) * vw <= nel else f"if ({t} < {nel})")
+            s(f"const int t = {t};")
+            if vw > 1:
+                s("wvec_t val;")
+                for i in range(vw):
+                    if per_u % vw == 0:
+                        s(f"val.v[{i}] = tw[t / {per_u} * {S - per_u} + t + {i}];")
+                    else:
+                        s(f"val.v[{i}] = tw[(t + {i}) / {per_u} * {S - per_u} + t + {i}];")
+                s(f"*(wvec_t*)(dwrow + {tbase} + t) = val;")
+            else:
+                s(f"dwrow[{tbase} + t] = tw[t / {per_u} * {S - per_u} + t];")
+            s.close()
         s.close()
         s.close()
 
