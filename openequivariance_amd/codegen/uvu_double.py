@@ -41,7 +41,8 @@ CONV_MAX_PATHS = 32
 def supported(low: Lowered, conv: bool = False) -> bool:
     if low.mode != "uvu" or low.shared_weights:
         return False
-    return not conv or len(low.paths) <= CONV_MAX_PATHS
+    from .uvu import tuning
+    return not conv or len(low.paths) <= tuning(dict(dd_maxp=CONV_MAX_PATHS))["dd_maxp"]
 
 
 class DoubleEmitter(UvuEmitter):
