@@ -39,7 +39,7 @@ def parse():
     ap.add_argument("--with-double", action="store_true",
                     help="with --no-extras: still run the second-order (double backward) side measurement")
     ap.add_argument("--only-tp", default=None, metavar="N",
-                    help="run only the batched tensor-product side measurement for config N (1, 2, 3, 3d, 4) "
+                    help="run only the batched tensor-product side measurement for config N (1, 2, 3, 3d, 4, dd) "
                          "and print its row; used for per-kernel profiles")
     return ap.parse_args()
 
@@ -131,9 +131,10 @@ def tp_config_table(dev, only=None):
 
     cases = [("cfg1 single uvu f32", P.config1_single_uvu(), 100000), ("cfg2 nequip uvu f32", P.config2_nequip_uvu(), 200000),
              ("cfg3 mace uvu f32", P.config3_mace_uvu(), 500000), ("cfg3 mace uvu f64", P.config3_mace_uvu(np.float64), 500000),
-             ("cfg4 uvw shared f32 (MFMA)", P.config4_uvw_shared(), 262144)]
+             ("cfg4 uvw shared f32 (MFMA)", P.config4_uvw_shared(), 262144),
+             ("DiffDock L=1 uvw per-row weights f32", P.diffdock_problems()[0], 100000)]
     if only is not None:
-        cases = [cases[["1", "2", "3", "3d", "4"].index(only)]]
+        cases = [cases[["1", "2", "3", "3d", "4", "dd"].index(only)]]
     table = []
     for name, prob, B in cases:
         low = lower(prob)
@@ -154,7 +155,7 @@ def tp_config_table(dev, only=None):
                "fwd_rows_per_s": B / tf * 1e3, "bwd_rows_per_s": B / tb * 1e3,
                "fwd_gflops": B * low.flops("forward") / tf / 1e6, "bwd_gflops": B * low.flops("backward") / tb / 1e6,
                "fwd_hbm_frac": fb / tf / 1e6 / HBM_PEAK_GBS, "bwd_hbm_frac": bb / tb / 1e6 / HBM_PEAK_GBS}
-        if low.mode == "uvw":
+        if low.mode == "uvw" and prob.shared_weights:
             dense = sum(2 * low.in1[p.i1].mul * low.in2[p.i2].mul * low.out[p.io].mul * low.out[p.io].d for p in low.paths)
             row["fwd_dense_tflops"] = B * dense / tf / 1e9
             row["bwd_dense_tflops"] = 2 * B * dense / tb / 1e9
