@@ -69,6 +69,7 @@ class UvuEmitter:
         self.nt = 0
         self.sched_fence = False
         self.fence_words = 0  # gradient registers between two scheduling fences (0: a fence after every path)
+        self.prefetch_runs = False  # request the next run's gradients and weights while a run computes
         self.seg_waves = 1  # conv forward: waves per node that share its output segments between them
         self.bwd_groups: Optional[List[List[int]]] = None  # conv backward: output blocks owned by each wave
         self.group_budget = 0  # gradient words per wave when a node is shared between waves (0: default)
@@ -971,12 +972,51 @@ class UvuEmitter:
         low = self.low
         ordered = sorted(self._paths(paths), key=lambda q: (q.io, q.index))
         since_fence = 0
+        # On-demand gradients with fences: the paths between two fences form a run. With prefetch_runs the
+        # gradient (and weight) values of run k+1 are requested at the start of run k, into variables named
+        # per path, so that a run computes while the next one's loads are in flight; without it every run
+        # starts with an exposed memory round trip.
+        prefetch = (self.prefetch_runs and self.sched_fence and g_on_demand_row is not None
+                    and all(low.in2[q.i2].mul <= UNROLL_V_LIMIT for q in ordered))
+        runs: List[List[Path]] = []
+        if prefetch:
+            cur, words = [], 0
+            for q in ordered:
+                dq = low.out[q.io].d * self.words
+                if cur and words + dq > self.fence_words:
+                    runs.append(cur)
+                    cur, words = [], 0
+                cur.append(q)
+                words += dq
+            runs.append(cur)
+
+        def emit_run_loads(run):
+            for q in run:
+                bo_q = low.out[q.io]
+                s(f"T gk{q.index}[{bo_q.d}];")
+                s.open("")
+                base, st = self._lane_ptr(bo_q)
+                s(f"const T* gp = {self._ptr(g_on_demand_row, base, bo_q.mul)};")
+                for k in range(bo_q.d):
+                    ld = f"__builtin_nontemporal_load(gp + {k * st})" if self.nt & 8 else f"gp[{k * st}]"
+                    s(f"gk{q.index}[{k}] = {self._val(bo_q.mul, ld, g_guard)};")
+                s.close()
+                for v in range(low.in2[q.i2].mul):
+                    s(f"const T wv{q.index}_{v} = {wacc(q, str(v))};")
+
+        run_of = {q.index: ri for ri, run in enumerate(runs) for q in run}
+        if prefetch:
+            emit_run_loads(runs[0])
         for n_path, p in enumerate(ordered):
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
             V = b2.mul
             s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
+            if prefetch and runs[run_of[p.index]][0] is p and run_of[p.index] + 1 < len(runs):
+                emit_run_loads(runs[run_of[p.index] + 1])
             s.open("")
-            if g_on_demand_row is not None:
+            if prefetch:
+                gname = lambda k, idx=p.index: f"gk{idx}[{k}]"
+            elif g_on_demand_row is not None:
                 s(f"T gk[{bo.d}];")
                 s.open("")
                 base, st = self._lane_ptr(bo)
@@ -992,7 +1032,7 @@ class UvuEmitter:
 
             def body(v, p=p, b1=b1, b2=b2, V=V, gname=gname, base_slot=base_slot):
                 prods = self._products(s, p, v, yacc)
-                s(f"const T wv = {wacc(p, v)};")
+                s(f"const T wv = {f'wv{p.index}_{v}' if prefetch else wacc(p, v)};")
                 ks = sorted({k for _, _, k, _ in p.nnz})
                 js = sorted({j for _, j, _, _ in p.nnz})
                 # dX: dx_i += (|c| y_j) * (g_k w)
@@ -1030,7 +1070,10 @@ class UvuEmitter:
 
             self._for_v(s, p, body)
             s.close()
-            if self.sched_fence and g_on_demand_row is not None:
+            if prefetch:
+                if runs[run_of[p.index]][-1] is p:
+                    s("__builtin_amdgcn_sched_barrier(0);")
+            elif self.sched_fence and g_on_demand_row is not None:
                 # keep the scheduler from hoisting all later paths' gradient loads over this path (with
                 # many paths that costs more registers than a wave has): a fence after every run of
                 # paths whose gradients take about ``fence_words`` registers, so that each run's loads
@@ -1586,14 +1629,18 @@ def tp_module(low: Lowered, compute_units: int = 256):
     probe = UvuEmitter(low)
     big = g_words > 256
     on_demand = big or probe.backward_words(True) > (250 if f32 else 420)
+    # the next run's gradients can be requested ahead when every path's v loop is unrolled
+    pf_ok = all(low.in2[p.i2].mul <= UNROLL_V_LIMIT for p in low.paths)
     t = tuning(dict(tp_acc=48, tp_gf=1 if wide else 4, tp_gb=1 if wide else 4,
-                    tp_wf=2 if f32 else 0, tp_wb=3 if big else 2, tp_nt=0, tp_gres=0 if on_demand else 1,
-                    tp_sb=1 if on_demand else 0, tp_trs=1, tp_fw=64,
+                    tp_wf=2 if f32 else 0, tp_wb=3 if (big and not pf_ok) else 2, tp_nt=0,
+                    tp_gres=0 if on_demand else 1,
+                    tp_sb=1 if on_demand else 0, tp_trs=1, tp_fw=64, tp_pf=1,
                     tp_dd=1, dd_wa=2, dd_wb=2))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
     em.sched_fence = bool(t["tp_sb"])
     em.fence_words = t["tp_fw"]
+    em.prefetch_runs = bool(t["tp_pf"])
     em.tr_stores = t["tp_trs"]
     s = Src()
     s(prelude(low.ctype))
@@ -1639,7 +1686,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=112, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
-                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0))
+                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fw=0, conv_pf=0))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -1696,6 +1743,8 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     em.tr_stores = t["conv_trs"]
     # output gradients that do not fit the register budget are loaded per path: fence the paths then
     em.sched_fence = (not em.g_resident) if t["conv_sb"] < 0 else bool(t["conv_sb"])
+    em.fence_words = t["conv_fw"]
+    em.prefetch_runs = bool(t["conv_pf"])
     s = Src()
     s(prelude(low.ctype))
     s(utility_kernels(kahan))
