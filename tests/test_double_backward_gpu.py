@@ -171,6 +171,34 @@ def test_conv_fused_isolated_nodes_and_empty():
             assert float(fused[0].abs().max()) == 0.0 and float(fused[3].abs().max()) == 0.0
 
 
+def test_edge_cases_and_refusals():
+    """Empty batch: nothing launched, empty results. Kernel sets without second-order kernels (shared
+    weights) refuse the fused entry point loudly; autograd then composes first-order kernels instead."""
+    problem = P.config2_nequip_uvu()
+    tp = oeq.TensorProduct(problem)
+    e = ops.get_entry(tp.kid)
+    empty = [torch.zeros((0, n), device="cuda") for n in (e.L1, e.L2, e.WN, e.L3, e.L1, e.L2, e.WN)]
+    out = ops.tp_double_backward(*empty, tp.kid)
+    assert [tuple(t.shape) for t in out] == [(0, e.L1), (0, e.L2), (0, e.WN), (0, e.L3)]
+    shared = problem.clone()
+    shared.shared_weights = True
+    tps = oeq.TensorProduct(shared)
+    es = ops.get_entry(tps.kid)
+    assert not es.kernels().has_double_backward()
+    rng = np.random.default_rng(1)
+    x, a = (_rand(rng, (9, es.L1), np.float32) for _ in range(2))
+    y, b = (_rand(rng, (9, es.L2), np.float32) for _ in range(2))
+    w, c = (_rand(rng, (es.WN,), np.float32) for _ in range(2))
+    g = _rand(rng, (9, es.L3), np.float32)
+    with pytest.raises(RuntimeError, match="no second-order kernels"):
+        ops.tp_double_backward(x, y, w, g, a, b, c, tps.kid)
+    # through autograd the shared-weight problem still differentiates twice (composition)
+    ts = [t.clone().requires_grad_(True) for t in (x, y, w)]
+    first = torch.autograd.grad(tps(*ts), ts, g, create_graph=True)
+    second = torch.autograd.grad(sum((t ** 2).sum() for t in first), ts)
+    assert all(torch.isfinite(t).all() for t in second)
+
+
 def test_many_path_convolutions_use_the_composition():
     from openequivariance_amd.codegen.lower import lower
     assert not uvu_double.supported(lower(P.seven_net_problems()[1]), conv=True)
