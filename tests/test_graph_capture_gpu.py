@@ -1,4 +1,4 @@
-"""The ops can be recorded into a HIP graph (torch.cuda.graph): every launch goes to the
+"""The ops (first- and second-order) can be recorded into a HIP graph (torch.cuda.graph): every launch goes to the
 capturing stream, buffers are cleared by a fill kernel rather than a memset node, and scratch
 comes from torch's capture-aware allocator. Each graph is replayed several times with new
 input values and eager work in between, and every replay is compared with the eager result."""
@@ -56,7 +56,10 @@ def test_tensor_product_in_a_graph(make):
     def step():
         z = ops.tp_forward(x, y, w, tp.kid)
         dx, dy, dw = ops.tp_backward(x, y, w, g, tp.kid)
-        return [z, dx, dy, dw]
+        out = [z, dx, dy, dw]
+        if ops.get_entry(tp.kid).kernels().has_double_backward():  # fused second-order kernels
+            out += list(ops.tp_double_backward(x, y, w, g, dx, dy, dw, tp.kid))
+        return out
 
     def new_values(seed):
         gen2 = torch.Generator(device="cuda").manual_seed(100 + seed)
@@ -82,7 +85,8 @@ def test_convolution_in_a_graph(deterministic):
     def step():
         z = ops.conv_forward(X, Y, W, tr, tc, tp, conv.kid)
         dx, dy, dw = ops.conv_backward(X, Y, W, G, tr, tc, tp, conv.kid)
-        return [z, dx, dy, dw]
+        second = ops.conv_double_backward(X, Y, W, G, dx, dy, dw, tr, tc, tp, conv.kid)
+        return [z, dx, dy, dw] + list(second)
 
     def new_values(seed):
         gen2 = torch.Generator(device="cuda").manual_seed(200 + seed)
