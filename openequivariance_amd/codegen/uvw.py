@@ -151,6 +151,8 @@ class UvwEmitter:
         if low.shared_weights:
             return None
         b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
+        if b1.mul == 1:
+            return None  # one input channel: handled with lanes = output channels instead
         per_u = b2.mul * bo.mul
         rows = min(64, b1.mul)
         elems = rows * per_u
@@ -252,6 +254,8 @@ class UvwEmitter:
                         nxt = tsteps[k + 1] if k + 1 < len(tsteps) else None
                         self._bwd_path_padded(s, p, plans[p.index][1], c * 64,
                                               (nxt[2], nxt[1] * 64, plans[nxt[2].index][1]) if nxt else None)
+                    elif b1.mul == 1:
+                        self._bwd_path_single_u(s, p)
                     else:
                         self._bwd_path_direct(s, p)
                 s.open("if (live && uok)")
@@ -318,6 +322,81 @@ class UvwEmitter:
                 s(f"const T {pair[(i, k)]} = x[{i}] * {gname}{k};")
             s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * {pair[(i, k)]};")
         return sorted(fstart)
+
+    def _bwd_path_single_u(self, s: Src, p: Path):
+        """A path whose first operand has one channel (spherical harmonics of an edge, say): lanes are the
+        output channels w instead of u, of which there is only one. G_k = sum_w W[w] g[w,k] is a wave
+        reduction, the weight gradient dW[w] = sum_k f_k g[w,k] is one value per lane (coalesced), and
+        the dX / dY terms are wave-uniform: lane 0 (the lane that owns u = 0 in the surrounding code)
+        adds them to its accumulators."""
+        low = self.low
+        shared = low.shared_weights
+        b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
+        Wn, d3 = bo.mul, bo.d
+        nchunk = (Wn + 63) // 64
+        s.open("")
+        s(f"T xu[{b1.d}];")
+        for i in range(b1.d):
+            s(f"xu[{i}] = xrow[{b1.off} + {i}];")
+        s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
+        prods = self._products(s, p)
+        s(f"const int wbase = {p.woff} + v * {Wn};")
+        for k in range(d3):
+            s(f"T G{k} = T(0);")
+        if nchunk == 1:
+            s(f"T gv[{d3}];")
+        for c in range(nchunk):
+            s.open("")
+            s(f"const int w = {c * 64} + lane;")
+            s(f"const bool wok = w < {Wn};")
+            s(f"const int wc = wok ? w : {Wn - 1};")
+            s("const T wv = wok ? wrow[wbase + wc] : T(0);")
+            for k in range(d3):
+                ld = f"grow[{bo.off} + wc * {d3} + {k}]"
+                if nchunk == 1:
+                    s(f"gv[{k}] = wok ? {ld} : T(0);")
+                    s(f"G{k} += wv * gv[{k}];")
+                else:
+                    s(f"G{k} += wv * {ld};")
+            s.close()
+        for k in range(d3):
+            for m in (32, 16, 8, 4, 2, 1):
+                s(f"G{k} += __shfl_xor(G{k}, {m});")
+        # wave-uniform from here on; only lane 0 (uok) keeps the dX / dY terms
+        fstart = set()
+        for n, (i, j, k, c) in enumerate(p.nnz):
+            q, neg = prods[n]
+            if k not in fstart:
+                s(f"T f{k} = {'-' if neg else ''}{q} * xu[{i}];")
+                fstart.add(k)
+            else:
+                s(f"f{k} {'-=' if neg else '+='} {q} * xu[{i}];")
+        s.open("if (uok)")
+        for n, (i, j, k, c) in enumerate(p.nnz):
+            q, neg = prods[n]
+            s(f"dx[{i}] {'-=' if neg else '+='} {q} * G{k};")
+            s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * (xu[{i}] * G{k});")
+        s.close()
+        ks = sorted(fstart)
+        for c in range(nchunk):
+            s.open("")
+            s(f"const int w = {c * 64} + lane;")
+            s(f"const bool wok = w < {Wn};")
+            s(f"const int wc = wok ? w : {Wn - 1};")
+            gk = (lambda k: f"gv[{k}]") if nchunk == 1 else (lambda k: f"grow[{bo.off} + wc * {d3} + {k}]")
+            s(f"T dwv = f{ks[0]} * {gk(ks[0])};")
+            for k in ks[1:]:
+                s(f"dwv += f{k} * {gk(k)};")
+            if shared and self.shared_lds:
+                s("if (wok && live) s_dw[wave][wbase + w] += dwv;")
+            elif shared:
+                s("if (!live) dwv = T(0);")
+                s("if (wok) prow[wbase + w] = first ? dwv : prow[wbase + w] + dwv;")
+            else:
+                s("if (wok && live) dwrow[wbase + w] = dwv;")
+            s.close()
+        s.close()
+        s.close()
 
     def _bwd_path_direct(self, s: Src, p: Path):
         """Weights read and weight gradients written straight from / to global memory, lane = u."""

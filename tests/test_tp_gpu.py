@@ -27,6 +27,14 @@ def _odd_uvw(shared):
                          internal_weights=False, label="odd-uvw")
 
 
+def _single_channel_uvw(shared):
+    # first operand with one channel per irrep (lanes = output channels in backward), outputs wider than a wave
+    return oeq.TPProblem("1x1o+1x0e+1x2e", "1x1o+2x0e", "70x1o+24x0e+130x1e+3x2e",
+                         [(0, 1, 0, "uvw", True), (1, 1, 1, "uvw", True), (0, 0, 2, "uvw", True),
+                          (2, 1, 3, "uvw", True), (1, 0, 0, "uvw", True, 0.5)], shared_weights=shared,
+                         internal_weights=False, label="single-channel-uvw")
+
+
 def _folded_with_gaps():
     # a row wider than a wave with a different multiplicity per irrep (folded into 64-channel pieces), one
     # input block no instruction reads, one output block no instruction writes, second operand with mul 2
@@ -66,6 +74,9 @@ CASES = [
                                                       shared_weights=False, internal_weights=False), 33),
     # production layers with a different multiplicity per irrep (rows wider than a wave: the chunks of a
     # row then run different code), one with 89 channels
+    ("single-channel-uvw", lambda: _single_channel_uvw(False), 45),
+    ("single-channel-uvw-shared", lambda: _single_channel_uvw(True), 45),
+    ("single-channel-uvw-f64", lambda: _as_f64(_single_channel_uvw(False)), 23),
     ("folded-gaps", _folded_with_gaps, 61),
     ("folded-gaps-f64", lambda: _as_f64(_folded_with_gaps()), 37),
     ("nequix-first", lambda: P.nequix_problems()[0], 53),
