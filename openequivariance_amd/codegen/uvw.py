@@ -32,7 +32,7 @@ class UvwEmitter:
     def __init__(self, low: Lowered):
         assert low.mode == "uvw"
         from .uvu import tuning
-        self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576))
+        self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576, uvw_regdw=1))
         self.TILE_BYTES = self.tune["uvw_tile"]
         self.low = low
         self.T = low.ctype
@@ -182,15 +182,33 @@ class UvwEmitter:
         # shared weights: each wave sums its rows' weight gradients in an LDS copy of the weight tensor
         # (when that fits) and writes it out once, instead of a read-modify-write of global memory per row
         self.shared_lds = False
+        self.reg_dw = False
         if shared:
+            # Small shared weight tensors with at most 64 input channels per path: lane u keeps its rows
+            # dW[u, :, :] of every path in registers over all the rows the wave handles (no read-modify-write
+            # of LDS per row), and reads W from one padded LDS copy per block with constant offsets.
+            dw_regs = sum(low.in2[p.i2].mul * low.out[p.io].mul for p in low.paths) * (low.elem_size // 4)
+            self.wsh_base, off = {}, 0
+            for p in low.paths:
+                self.wsh_base[p.index] = off
+                off += low.in1[p.i1].mul * self._row_stride(p)
+            self.wsh_elems = off
+            if (self.tune["uvw_regdw"] and dw_regs <= 176 and all(1 < low.in1[p.i1].mul <= 64 for p in low.paths)
+                    and off * low.elem_size <= 49152):
+                self.reg_dw = True
+                waves = WAVES_PER_BLOCK
+        if shared and not self.reg_dw:
             fit = 65536 // (low.WN * low.elem_size)
             if fit >= 1:
                 self.shared_lds = True
                 waves = min(WAVES_PER_BLOCK, fit)
         self.backward_waves = waves
         block = 64 * waves
+        # register-resident weight gradients: left to one wave per SIMD with up to 512 registers (e3tools
+        # transformer block: 0.29 ms against 0.57 ms with spills at 256; uvw_regdw=2 selects the latter)
+        attr = " __attribute__((amdgpu_waves_per_eu(2, 2)))" if (self.reg_dw and self.tune["uvw_regdw"] == 2) else ""
         s.open(
-            f'extern "C" __global__ __launch_bounds__({block}) void backward(i64 num_batch, '
+            f'extern "C" __global__ __launch_bounds__({block}){attr} void backward(i64 num_batch, '
             "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
             "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
             "const T* __restrict__ L3_grad, T* __restrict__ wpartial)"
@@ -200,7 +218,16 @@ class UvwEmitter:
             s(f"__shared__ __attribute__((aligned(16))) T s_w[{waves}][{tile_elems}];")
         if shared:
             s(f"T* prow = wpartial + ((i64)blockIdx.x * {waves} + oeq_wave()) * {low.WN};")
-            if self.shared_lds:
+            if self.reg_dw:
+                s(f"__shared__ T s_wsh[{self.wsh_elems}];")
+                for p in low.paths:
+                    per_u, S = low.in2[p.i2].mul * low.out[p.io].mul, self._row_stride(p)
+                    s(f"for (int t = threadIdx.x; t < {low.in1[p.i1].mul * per_u}; t += {block}) "
+                      f"s_wsh[{self.wsh_base[p.index]} + t / {per_u} * {S - per_u} + t] = W[{p.woff} + t];")
+                    s(f"T dwr{p.index}[{per_u}];")
+                    s(f"for (int t = 0; t < {per_u}; ++t) dwr{p.index}[t] = T(0);")
+                s("__syncthreads();")
+            elif self.shared_lds:
                 s(f"__shared__ T s_dw[{waves}][{low.WN}];")
                 s(f"for (int t = oeq_lane(); t < {low.WN}; t += 64) s_dw[oeq_wave()][t] = T(0);")
                 s("oeq_wave_sync();")
@@ -254,6 +281,8 @@ class UvwEmitter:
                         nxt = tsteps[k + 1] if k + 1 < len(tsteps) else None
                         self._bwd_path_padded(s, p, plans[p.index][1], c * 64,
                                               (nxt[2], nxt[1] * 64, plans[nxt[2].index][1]) if nxt else None)
+                    elif self.reg_dw:
+                        self._bwd_path_regdw(s, p)
                     elif b1.mul == 1:
                         self._bwd_path_single_u(s, p)
                     else:
@@ -263,7 +292,7 @@ class UvwEmitter:
                     s(f"dxrow[{b1.off} + u * {b1.d} + {i}] = dx[{i}];")
                 s.close()
                 s.close()
-        if shared and not self.shared_lds:
+        if shared and not self.shared_lds and not self.reg_dw:
             s("first = false;")
         # dY: butterfly over the 64 lanes
         n = self.l2_pad
@@ -292,7 +321,15 @@ class UvwEmitter:
             s(f"if (dyidx + {j} < {low.L2}) L2_grad[rowc * {low.L2} + dyidx + {j}] = rv[{j}];")
         s.close()
         s.close()
-        if shared and self.shared_lds:
+        if shared and self.reg_dw:
+            # lane u owns rows [u, :, :] of every path's weight gradient
+            for p in low.paths:
+                per_u = low.in2[p.i2].mul * low.out[p.io].mul
+                s.open(f"if (oeq_lane() < {low.in1[p.i1].mul})")
+                for t in range(per_u):
+                    s(f"prow[{p.woff} + oeq_lane() * {per_u} + {t}] = dwr{p.index}[{t}];")
+                s.close()
+        elif shared and self.shared_lds:
             s("oeq_wave_sync();")
             s(f"for (int t = oeq_lane(); t < {low.WN}; t += 64) prow[t] = s_dw[oeq_wave()][t];")
         elif shared:
@@ -322,6 +359,35 @@ class UvwEmitter:
                 s(f"const T {pair[(i, k)]} = x[{i}] * {gname}{k};")
             s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * {pair[(i, k)]};")
         return sorted(fstart)
+
+    def _bwd_path_regdw(self, s: Src, p: Path):
+        """Shared weights, lane = u, weight gradients in registers (``dwr<path>``) over all rows of the
+        wave; W from the block's padded LDS copy (rows an odd number of elements apart: no bank
+        conflicts, constant offsets), dZ of the output irrep through the scalar cache."""
+        low = self.low
+        b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
+        V, Wn, d3 = b2.mul, bo.mul, bo.d
+        S = self._row_stride(p)
+        s.open("")
+        s(f"const T* gq = grow + {bo.off};  // wave-uniform")
+        s(f"const T* wl = s_wsh + {self.wsh_base[p.index]} + (uok ? u : 0) * {S};")
+        for vv in range(V):
+            s.open("")
+            s(f"const int v = {vv};")
+            prods = self._products(s, p)
+            for k in range(d3):
+                s(f"T G{k} = T(0);")
+            for w in range(Wn):
+                s(f"{{ const T wv = wl[{vv * Wn + w}]; " +
+                  " ".join(f"G{k} += wv * gq[{w * d3 + k}];" for k in range(d3)) + " }")
+            ks = self._cg_backward(s, p, prods)
+            s.open("if (uok && live)")
+            for w in range(Wn):
+                terms = " + ".join(f"f{k} * gq[{w * d3 + k}]" for k in ks)
+                s(f"dwr{p.index}[{vv * Wn + w}] += {terms};")
+            s.close()
+            s.close()
+        s.close()
 
     def _bwd_path_single_u(self, s: Src, p: Path):
         """A path whose first operand has one channel (spherical harmonics of an edge, say): lanes are the
