@@ -9,7 +9,6 @@ kernels read weights in e3nn order directly).
 
 from __future__ import annotations
 
-import numpy as np
 import torch
 
 from ..codegen.lower import lower

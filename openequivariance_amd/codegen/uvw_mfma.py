@@ -42,7 +42,7 @@ D[m][n]: n = l % 16, m = 4 * (l / 16) + i for the i-th of 4 result registers.
 
 from __future__ import annotations
 
-from typing import Dict, List, Tuple
+from typing import List
 
 from .common import Src, prelude, utility_kernels
 from .lower import Lowered, Path, float_literal

@@ -11,7 +11,7 @@ from typing import Optional
 
 import numpy as np
 
-from .spec import Irrep, Irreps, TPProblem
+from .spec import Irreps, TPProblem
 
 
 class FullyConnectedTPProblem(TPProblem):

@@ -13,7 +13,7 @@ import collections
 import copy
 import itertools
 import math
-from typing import Any, List, NamedTuple, Optional, Tuple
+from typing import List, NamedTuple, Optional, Tuple
 
 import numpy as np
 

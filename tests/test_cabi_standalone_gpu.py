@@ -2,7 +2,6 @@
 kernel-set creation, forward and backward on plain hipMalloc'ed buffers, no Python or torch in that
 process. This test only writes the kernel bundle and the oracle's expected values, then runs it."""
 
-import os
 import subprocess
 from pathlib import Path
 

@@ -3,7 +3,6 @@ capturing stream, buffers are cleared by a fill kernel rather than a memset node
 comes from torch's capture-aware allocator. Each graph is replayed several times with new
 input values and eager work in between, and every replay is compared with the eager result."""
 
-import numpy as np
 import pytest
 import torch
 

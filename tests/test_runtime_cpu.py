@@ -2,7 +2,6 @@
 generated sources for gfx950 with no GPU present and reports errors through
 return codes. No kernel is launched here."""
 
-import ctypes
 import os
 import re
 
