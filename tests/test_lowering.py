@@ -1,0 +1,82 @@
+"""Planner invariants that need no GPU: folding of wide rows with mixed multiplicities, which kernel
+sets carry the fused second-order kernels, and that the generated sources compile for gfx950."""
+
+import numpy as np
+import pytest
+
+import openequivariance_amd as oeq
+from openequivariance_amd import runtime as rt
+from openequivariance_amd.codegen import lower as L
+from openequivariance_amd.codegen import uvu_double
+from openequivariance_amd.core import problems as P
+
+
+def _unfolded(problem):
+    """The tables before folding (what lower() would return for a row that needs none)."""
+    low = L.lower(problem)
+    in1, in2, out = (L._blocks(ir) for ir in (problem.irreps_in1, problem.irreps_in2, problem.irreps_out))
+    return low, in1, in2, out
+
+
+@pytest.mark.parametrize("problem", P.nequix_problems() + P.seven_net_problems(), ids=lambda p: p.label)
+def test_folding_preserves_the_problem(problem):
+    low, in1, in2, out = _unfolded(problem)
+    wide = max(in1[i.i_in1].mul for i in problem.instructions) > 64
+    ragged = any(in1[i.i_in1].mul != 64 * ((max(b.mul for b in in1) + 63) // 64) for i in problem.instructions)
+    assert (low.n_chunks == 1) == (not wide or ragged)
+    assert (low.L1, low.L2, low.L3, low.WN) == (problem.irreps_in1.dim, problem.irreps_in2.dim,
+                                                problem.irreps_out.dim, problem.weight_numel)
+    # pieces tile their blocks exactly: same elements, at most 64 channels each
+    for pieces, blocks in ((low.in1, in1), (low.out, out)):
+        covered = sorted((b.off, b.off + b.mul * b.d) for b in pieces)
+        assert covered[0][0] == 0 and covered[-1][1] == sum(b.mul * b.d for b in blocks)
+        assert all(a[1] == b[0] for a, b in zip(covered, covered[1:]))
+        if low.n_chunks == 1 and wide:
+            assert max(b.mul for b in pieces) <= 64
+    # every weight belongs to exactly one folded path
+    spans = sorted((p.woff, p.woff + low.in1[p.i1].mul * low.in2[p.i2].mul) for p in low.paths)
+    assert spans[0][0] == 0 and spans[-1][1] == low.WN and all(a[1] == b[0] for a, b in zip(spans, spans[1:]))
+    # same arithmetic: the reference's FLOP count does not change
+    plain = sum(3 * len(p.nnz) * low.in1[p.i1].mul * low.in2[p.i2].mul + low.out[p.io].mul * low.out[p.io].d
+                for p in low.paths)
+    assert low.flops("forward") == plain
+    assert sum(low.in1[p.i1].mul for p in low.paths) == sum(in1[i.i_in1].mul for i in problem.instructions)
+
+
+def test_uniform_wide_rows_are_not_folded():
+    low = L.lower(P.config3_mace_uvu())
+    assert low.n_chunks == 2 and len(low.paths) == 23 and max(b.mul for b in low.in1) == 128
+    ir_mul = P.seven_net_problems()[1].clone()
+    ir_mul.layout = "ir_mul"
+    assert L.lower(ir_mul).n_chunks == 2  # pieces of a component-major block are not contiguous
+
+
+def test_which_sets_carry_fused_second_order_kernels():
+    assert uvu_double.supported(L.lower(P.config3_mace_uvu()))
+    assert uvu_double.supported(L.lower(P.config3_mace_uvu()), conv=True)
+    seven = L.lower(P.seven_net_problems()[1])
+    assert uvu_double.supported(seven) and not uvu_double.supported(seven, conv=True)  # 38 paths
+    shared = P.config2_nequip_uvu().clone()
+    shared.shared_weights = True
+    assert not uvu_double.supported(L.lower(shared))
+    assert not uvu_double.supported(L.lower(P.config4_uvw_shared()))
+
+
+@pytest.mark.parametrize("make,conv", [(lambda: P.nequix_problems()[1], False), (lambda: P.seven_net_problems()[0], True),
+                                       (lambda: P.config2_nequip_uvu(np.float64), True),
+                                       (lambda: P.diffdock_problems()[0], False), (lambda: P.tetris_poly_problems()[0], False),
+                                       (lambda: P.e3tools_problems()[1], False)],
+                         ids=["nequix-main-tp", "sevennet-first-conv", "cfg2-f64-conv", "diffdock-tp", "tetris-tp",
+                              "e3tools-transformer-tp"])
+def test_generated_sources_compile_for_gfx950(make, conv):
+    from openequivariance_amd._torch.tensor_product import build_tp_module
+    from openequivariance_amd._torch.tensor_product_conv import build_conv_module
+    problem = make()
+    src, dims, descs = build_conv_module(problem, True) if conv else build_tp_module(problem)
+    blob = rt.compile_source(src, use_disk_cache=False)
+    assert blob[:4] == b"\x7fELF"
+    names = {d[1] for d in descs}
+    assert {"forward", "backward"} <= names
+    if problem.instructions[0].connection_mode == "uvu":
+        assert {"double_backward_A", "double_backward_B"} <= names
+        assert {d[0] for d in descs} >= {rt.ROLE_DOUBLE_BACKWARD_A, rt.ROLE_DOUBLE_BACKWARD_B}
