@@ -49,6 +49,9 @@ class Block:
     off: int
     mul: int
     l: int
+    # [2l+1, mul] layout only: distance between two components of a channel when it is not ``mul`` (a
+    # piece of a wider block keeps the stride of the block it was cut from)
+    cstride: int = 0
 
     @property
     def d(self) -> int:
@@ -150,8 +153,7 @@ def lower(problem: TPProblem) -> Lowered:
     )
     low.ir_mul = problem.layout == "ir_mul"
     _lane_mapping(low)
-    if mode == "uvu" and not low.ir_mul and 1 < low.n_chunks <= 4 and \
-            any(in1[p.i1].mul != 64 * low.n_chunks for p in paths):
+    if mode == "uvu" and 1 < low.n_chunks <= 4 and any(in1[p.i1].mul != 64 * low.n_chunks for p in paths):
         low = _fold_wide_blocks(low)
     return low
 
@@ -170,20 +172,31 @@ def _fold_wide_blocks(low: Lowered) -> Lowered:
     """'uvu' rows wider than a wave whose irreps have different multiplicities (128x0e+64x1o+32x2e,
     89x0e, ...): cut every block into pieces of at most 64 channels and every path into the paths
     between matching pieces. In the [mul, 2l+1] layout a piece is just a block that starts further into
-    the row, and its weights start ``64 * mul_v`` further into the path's weights, so the result is an
-    ordinary problem with at most 64 channels per block: one wave then owns the whole row and walks the
+    the row (in the [2l+1, mul] layout: 64 channels further into each component, with the components
+    still ``mul`` apart), and its weights start ``64 * mul_v`` further into the path's weights, so the
+    result is an ordinary problem with at most 64 channels per block: one wave then owns the whole row and walks the
     pieces one after the other, where waves that each owned one 64-channel slice of every block would
     mostly have idle lanes or nothing to do."""
-    def cut(blocks: List[Block]):
+    def cut(blocks: List[Block], used):
         pieces, index = [], {}
         for b, blk in enumerate(blocks):
+            if low.ir_mul and b not in used:
+                # [2l+1, mul] layout: the channels of a piece are not one contiguous range; a block no path
+                # touches (it is only cleared) stays whole
+                index[(b, 0)] = len(pieces)
+                pieces.append(blk)
+                continue
             for c in range((blk.mul + 63) // 64):
                 index[(b, c)] = len(pieces)
-                pieces.append(Block(blk.off + c * 64 * blk.d, min(64, blk.mul - c * 64), blk.l))
+                n = min(64, blk.mul - c * 64)
+                if low.ir_mul:  # component i of channel u sits at off + i * mul + u
+                    pieces.append(Block(blk.off + c * 64, n, blk.l, cstride=blk.mul))
+                else:
+                    pieces.append(Block(blk.off + c * 64 * blk.d, n, blk.l))
         return pieces, index
 
-    in1, index1 = cut(low.in1)
-    out, index3 = cut(low.out)
+    in1, index1 = cut(low.in1, {p.i1 for p in low.paths})
+    out, index3 = cut(low.out, {p.io for p in low.paths})
     paths = []
     for p in low.paths:
         v_mul = low.in2[p.i2].mul
@@ -193,6 +206,7 @@ def _fold_wide_blocks(low: Lowered) -> Lowered:
     folded = Lowered(mode=low.mode, ctype=low.ctype, elem_size=low.elem_size, shared_weights=low.shared_weights,
                      in1=in1, in2=low.in2, out=out, paths=paths, L1=low.L1, L2=low.L2, L3=low.L3, WN=low.WN,
                      label=low.label)
+    folded.ir_mul = low.ir_mul
     _lane_mapping(folded)
     return folded
 

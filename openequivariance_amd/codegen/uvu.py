@@ -292,7 +292,7 @@ class UvuEmitter:
         a component's channels together (then a wave's accesses are contiguous without any per-lane vector).
         The expression is applied with :meth:`_ptr`."""
         if self.ir_mul:
-            return (blk.off, 1), blk.mul
+            return (blk.off, 1), (blk.cstride or blk.mul)
         return (blk.off, blk.d), 1
 
     def _ptr(self, rowexpr: str, where, mul: Optional[int] = None) -> str:

@@ -37,6 +37,14 @@ PROBLEMS = [
     ("13x5e", lambda: _single(13)),
     ("multi-v", lambda: _multi_v(False)),
     ("multi-v-shared", lambda: _multi_v(True)),
+    # wide rows with a different multiplicity per irrep: folded into 64-channel pieces whose components
+    # stay a whole block's multiplicity apart
+    ("nequix-first", lambda: P.nequix_problems()[0]),
+    ("sevennet-main", lambda: P.seven_net_problems()[1]),
+    ("folded-gaps", lambda: oeq.TPProblem(
+        "100x0e+70x1o+40x2e+96x1e", "1x0e+2x1o", "100x0e+70x1o+100x1o+40x1o+33x2e",
+        [(0, 0, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 1, 2, "uvu", True), (2, 1, 3, "uvu", True, 0.7)],
+        shared_weights=False, internal_weights=False, label="folded-gaps")),
 ]
 
 

@@ -46,9 +46,17 @@ def test_folding_preserves_the_problem(problem):
 def test_uniform_wide_rows_are_not_folded():
     low = L.lower(P.config3_mace_uvu())
     assert low.n_chunks == 2 and len(low.paths) == 23 and max(b.mul for b in low.in1) == 128
-    ir_mul = P.seven_net_problems()[1].clone()
-    ir_mul.layout = "ir_mul"
-    assert L.lower(ir_mul).n_chunks == 2  # pieces of a component-major block are not contiguous
+
+
+def test_folding_in_component_major_layout():
+    problem = P.seven_net_problems()[1].clone()
+    problem.layout = "ir_mul"
+    low = L.lower(problem)
+    assert low.ir_mul and low.n_chunks == 1 and max(b.mul for b in low.in1) <= 64
+    whole = L._blocks(problem.irreps_in1)
+    # the two pieces of 128x0e: 64 channels apart, components a whole block's multiplicity apart
+    first, second = [b for b in low.in1 if whole[0].off <= b.off < whole[0].off + whole[0].mul * whole[0].d][:2]
+    assert (second.off - first.off, first.cstride, second.cstride) == (64, 128, 128)
 
 
 def test_which_sets_carry_fused_second_order_kernels():
