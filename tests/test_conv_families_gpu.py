@@ -43,6 +43,11 @@ def _cases():
                              [(0, 0, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 1, 2, "uvu", True),
                               (2, 1, 3, "uvu", True, 0.7)], shared_weights=False, internal_weights=False,
                              label="folded-gaps"))
+    # wider than four waves and ragged: chunk waves with bodies specialised per chunk
+    out.append(oeq.TPProblem("300x0e+70x1o+20x2e", "1x0e+1x1o", "300x0e+70x1o+300x1o+20x1o",
+                             [(0, 0, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 1, 2, "uvu", True),
+                              (2, 1, 3, "uvu", True)], shared_weights=False, internal_weights=False,
+                             label="very-wide-ragged"))
     shared = P.mace_problems()[0].clone()
     shared.shared_weights = True
     shared.label = "mace-large-shared"

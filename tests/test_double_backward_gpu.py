@@ -55,6 +55,10 @@ CASES = [
     ("cfg1", P.config1_single_uvu, 1000),
     ("wide-v", _wide_v, 211),
     ("folded-gaps", _folded, 61),
+    ("very-wide-ragged", lambda: oeq.TPProblem(
+        "300x0e+70x1o+20x2e", "1x0e+1x1o", "300x0e+70x1o+300x1o+20x1o",
+        [(0, 0, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 1, 2, "uvu", True), (2, 1, 3, "uvu", True)],
+        shared_weights=False, internal_weights=False), 37),
     ("odd", _odd, 333),
     ("odd-f64", lambda: _f64(_odd()), 333),
     ("cfg2", P.config2_nequip_uvu, 257),

@@ -35,6 +35,15 @@ def _single_channel_uvw(shared):
                          internal_weights=False, label="single-channel-uvw")
 
 
+def _very_wide_ragged():
+    # wider than four waves with a different multiplicity per irrep: not folded, the chunk waves run
+    # bodies specialised per chunk
+    return oeq.TPProblem("300x0e+70x1o+20x2e", "1x0e+1x1o", "300x0e+70x1o+300x1o+20x1o",
+                         [(0, 0, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 1, 2, "uvu", True),
+                          (2, 1, 3, "uvu", True)], shared_weights=False, internal_weights=False,
+                         label="very-wide-ragged")
+
+
 def _folded_with_gaps():
     # a row wider than a wave with a different multiplicity per irrep (folded into 64-channel pieces), one
     # input block no instruction reads, one output block no instruction writes, second operand with mul 2
@@ -77,6 +86,7 @@ CASES = [
     ("single-channel-uvw", lambda: _single_channel_uvw(False), 45),
     ("single-channel-uvw-shared", lambda: _single_channel_uvw(True), 45),
     ("single-channel-uvw-f64", lambda: _as_f64(_single_channel_uvw(False)), 23),
+    ("very-wide-ragged", _very_wide_ragged, 37),
     ("folded-gaps", _folded_with_gaps, 61),
     ("folded-gaps-f64", lambda: _as_f64(_folded_with_gaps()), 37),
     ("nequix-first", lambda: P.nequix_problems()[0], 53),
