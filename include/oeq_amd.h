@@ -81,7 +81,8 @@ typedef enum {
     OEQ_ROLE_GROUP_ORDER = 12,      /*   and ascending order of the indices within each segment */
     OEQ_ROLE_DOUBLE_BACKWARD_A = 13,/* second order: gradient w.r.t. the output gradient (forward-shaped) */
     OEQ_ROLE_DOUBLE_BACKWARD_B = 14,/* second order: gradients w.r.t. X, Y, W (backward-shaped) */
-    OEQ_ROLE_COUNT = 15
+    OEQ_ROLE_ORDER_HOP = 15,        /* convolution walk order: one hop of the node clustering */
+    OEQ_ROLE_COUNT = 16
 } oeq_role;
 
 /* How the convolution kernels of a set find the edges of a node (oeq_problem_dims.deterministic):
@@ -95,6 +96,17 @@ typedef enum {
                               through that index: fixed summation order for a given edge list, no atomics on node
                               data */
 } oeq_conv_mode;
+
+/* What the receiver walk of the convolution backward does with the per-edge terms of the gradient
+ * with respect to the sender rows (oeq_problem_dims.dx_mode). The reference's deterministic backward
+ * walks sender-sorted edges instead and re-reads the receiver's gradient row per edge
+ * (loop_unroll_conv_det.cuh:187-293). */
+typedef enum {
+    OEQ_DX_TERMS = 0,    /* terms go to scratch; fixup_backward sums them per sender in sender-major order */
+    OEQ_DX_ATOMIC = 1,   /* terms are added into the cleared sender rows with float atomics (not bit-reproducible) */
+    OEQ_DX_ARRIVAL = 2   /* terms go to scratch; the wave that delivers the last term of a sender sums that
+                            sender's terms in sender-major order (same bits as OEQ_DX_TERMS, no second kernel) */
+} oeq_dx_mode;
 
 /* Several descriptors may name the same role: those kernels are launched back to back, in
  * descriptor order, with the same arguments and launch shape (that of the last descriptor). */
@@ -116,6 +128,13 @@ typedef struct {
     int32_t wpartial_per_block; /* shared weights: partial weight-gradient rows each block of the
                                    backward kernel writes (0 = none); the workspace holds
                                    max_blocks * wpartial_per_block rows of weight_numel elements */
+    int32_t dx_mode;            /* conv backward, walk modes: an oeq_dx_mode value */
+    int32_t n_chunks;           /* conv backward, OEQ_DX_ARRIVAL: arrival counters per sender node
+                                   (one per 64-channel chunk of a row) */
+    int32_t order_hops;         /* conv, walk modes: > 0 = at every call the nodes are clustered by the
+                                   highest-priority node within this many edges and walked cluster by cluster,
+                                   so that nodes sharing senders run side by side and the gathered sender rows
+                                   are served by the L2; 0 = nodes are walked by index */
 } oeq_problem_dims;
 
 int oeq_kernels_create(const void* code, size_t code_size,
@@ -191,15 +210,15 @@ int oeq_tp_double_backward(oeq_kernels* k, int64_t num_batch,
 
 /* The same for the fused convolution; replaces JITConvImpl::double_backward
  * (extension/convolution.hpp:138-178) as called by jit_conv_double_backward
- * (extension/torch_core.hpp:544-625). Index arguments and workspace
- * (oeq_conv_backward_workspace_bytes() bytes) are those of oeq_conv_backward. Not available for
- * OEQ_CONV_ATOMIC kernel sets. */
+ * (extension/torch_core.hpp:544-625). Index arguments are those of oeq_conv_backward; the workspace must
+ * hold oeq_conv_double_backward_workspace_bytes() bytes. Not available for OEQ_CONV_ATOMIC kernel sets. */
 int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz,
                              const void* L1_in, const void* L2_in, const void* W, const void* L3_grad,
                              const void* L1_dgrad, const void* L2_dgrad, const void* W_dgrad,
                              void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad,
                              const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm,
                              void* workspace, size_t workspace_bytes, void* stream);
+size_t oeq_conv_double_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
 
 /* ---- ordered segment sum -------------------------------------------------- */
 /* dst[s, :] = sum, in list order, of src[item, :] over the items whose key is s, for s < n_segments.

@@ -277,9 +277,11 @@ def _conv_checks(e: KernelEntry, L1_in, L2_in, W, rows, cols, perm, L3_grad=None
     if e.deterministic:
         check_tensor(perm, [nnz], torch.int64, "transpose perm")
     elif (torch.are_deterministic_algorithms_enabled() and not e.unfused
-          and e.kernels().dims["deterministic"] == rt.CONV_ATOMIC):
-        # counterpart of at::globalContext().alertNotDeterministic (torch_core.hpp:448); only the
-        # float-atomics kernels need it: the default grouped walk sums in a fixed order
+          and (e.kernels().dims["deterministic"] == rt.CONV_ATOMIC
+               or (L3_grad is not None and e.kernels().dims.get("dx_mode", 0) == rt.DX_ATOMIC))):
+        # counterpart of at::globalContext().alertNotDeterministic (torch_core.hpp:448) for the calls that
+        # use float atomics: the backward of deterministic=False (sender gradients), and both directions
+        # of the float-atomics kernels. The grouped forward sums in a fixed order and needs no alert.
         msg = ("OpenEquivariance_conv_atomic does not have a deterministic implementation, but you set "
                "'torch.use_deterministic_algorithms(True)'. Use TensorProductConv(..., deterministic=True).")
         if torch.is_deterministic_algorithms_warn_only_enabled():
@@ -419,7 +421,7 @@ def conv_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tens
     dx, dy, dw, gg = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w), torch.empty_like(g)
     with torch.cuda.device(x.device):
         ks = e.kernels()
-        nb = ks.conv_backward_workspace_bytes(nodes, nnz)
+        nb = ks.conv_double_backward_workspace_bytes(nodes, nnz)
         ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
         ks.conv_double_backward(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), g.data_ptr(), a.data_ptr(),
                                 b.data_ptr(), c.data_ptr(), dx.data_ptr(), dy.data_ptr(), dw.data_ptr(),

@@ -120,6 +120,16 @@ class UvuEmitter:
         )
 
         self.tr_atomics = False  # set by the conv kernels that declare the s_tr tile
+        # Products |c| * y_j of a CG coefficient and a component of the row's second operand are the
+        # same for every channel. With ``use_q`` the lanes of a wave compute them once per edge, one
+        # product per lane and 64-entry slab, into a wave-private LDS table that the contraction reads
+        # back as broadcasts, instead of every lane forming every product in the vector ALU (a third of
+        # the forward's and an eighth of the backward's vector instructions at the MACE shape).
+        self.use_q = False
+        self.q_pin = True
+        self.q_ahead = (64, 64)  # multiply-adds between the request of a path's products and their use (fwd, bwd)
+        self.q_entries: List[Tuple[int, float]] = []  # table slot -> (index into the Y row, coefficient)
+        self.q_slot: Dict[Tuple[int, int, str, int], int] = {}  # (path, v, |c| literal, j) -> slot
         self.stage = self._stage_layout()
         self.stage3 = self._stage3_layout()
 
@@ -195,8 +205,12 @@ class UvuEmitter:
         for q in range(st["nqw"]):
             s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sw + woff{q}), "
               f"(OEQ_LPTR)(&s_stage[wave][{st['XF'] + q * 256}]), 16, 0, {2 if self.nt & 1 else 0});")
-        for j in range(low.L2):
-            s(f"yn[{j}] = L2_in[eid * {low.L2} + {j}];")
+        if self.use_q:
+            for r in range(self.q_slabs):
+                s(f"yn[{r}] = L2_in[eid * {low.L2} + qt.j[{r}]];")
+        else:
+            for j in range(low.L2):
+                s(f"yn[{j}] = L2_in[eid * {low.L2} + {j}];")
         s.close()
 
     def _emit_stage_read(self, s: Src, buf: str):
@@ -207,8 +221,12 @@ class UvuEmitter:
                 s(f"{buf}.x.b{b}[{i}] = s_stage[wave][{self._stage_x(blk, st['xl'][b], i)}];")
         for p in low.paths:
             s(f"{buf}.w[{self.wslot[p.index]}] = s_stage[wave][{st['XF'] + p.index * 64} + ul];")
-        for j in range(low.L2):
-            s(f"{buf}.y[{j}] = yn[{j}];")
+        if self.use_q:
+            for r in range(self.q_slabs):
+                s(f"{buf}.yq[{r}] = yn[{r}];")
+        else:
+            for j in range(low.L2):
+                s(f"{buf}.y[{j}] = yn[{j}];")
 
     # ---- double-buffered staging: X, W and Y of an edge live only in LDS ------------
     def _stage3_layout(self):
@@ -408,9 +426,107 @@ class UvuEmitter:
 
         return y, w
 
+    def _qarg(self) -> str:
+        return ", qt" if self.use_q else ""
+
+    def q_supported(self) -> bool:
+        """The product table needs the second operand to be the same for the whole wave (a row that
+        fills the wave) and every index a generation-time constant."""
+        return self.R == 1 and self.can_preload
+
+    def build_q_table(self):
+        """Slots 0..L2-1 hold the raw Y row, the rest the distinct products of every (path, v) in path
+        order (so the slots a path reads are contiguous and can be fetched as 16-byte vectors)."""
+        low = self.low
+        self.q_entries = [(j, 1.0) for j in range(low.L2)]
+        self.q_slot = {}
+        for p in low.paths:
+            b2 = low.in2[p.i2]
+            for v in range(b2.mul):
+                for (i, j, k, c) in p.nnz:
+                    key = (p.index, v, self.lit(abs(c)), j)
+                    if key not in self.q_slot:
+                        self.q_slot[key] = len(self.q_entries)
+                        yidx = b2.off + (j * b2.mul + v if self.ir_mul else v * b2.d + j)
+                        self.q_entries.append((yidx, abs(c)))
+        self.q_slabs = -(-len(self.q_entries) // 64)
+        self.q_floats = self.q_slabs * 64
+
+    def emit_q_tables(self, s: Src):
+        """Module-scope constants: for table slot t, which Y component it multiplies and by what."""
+        pad = self.q_floats - len(self.q_entries)
+        js = [j for j, _ in self.q_entries] + [0] * pad
+        cs = [self.lit(c) for _, c in self.q_entries] + [self.lit(0.0)] * pad
+        s(f"__device__ const int OEQ_QJ[{self.q_floats}] = {{{', '.join(map(str, js))}}};")
+        s(f"__device__ const T OEQ_QC[{self.q_floats}] = {{{', '.join(f'T({c})' for c in cs)}}};")
+        s(f"struct __attribute__((aligned({4 * self.low.elem_size}))) oeq_q4 {{ T v[4]; }};")
+        s(f"struct Q_t {{ int j[{self.q_slabs}]; T c[{self.q_slabs}]; }};")
+
+    def _emit_q_prologue(self, s: Src, waves: int):
+        s(f"__shared__ __attribute__((aligned(16))) T s_q[{waves}][{self.q_floats}];")
+        s("Q_t qt;")
+        for r in range(self.q_slabs):
+            s(f"qt.j[{r}] = OEQ_QJ[{r * 64} + lane]; qt.c[{r}] = OEQ_QC[{r * 64} + lane];")
+        s("T* const sq = &s_q[wave][0];")
+
+    def _emit_q_build(self, s: Src, src: str):
+        """Fill the wave's table from the Y values its lanes fetched (``src[r]``). The wave-scope fences
+        keep the table reads of the previous edge above the writes and those of this edge below."""
+        s("oeq_wave_sync();")
+        for r in range(self.q_slabs):
+            s(f"sq[{r * 64} + lane] = qt.c[{r}] * {src}[{r}];")
+        s("oeq_wave_sync();")
+
+    def _q_slots_of(self, p: Path, v: int) -> List[int]:
+        return [self.q_slot[(p.index, v, self.lit(abs(c)), j)] for (i, j, k, c) in p.nnz]
+
+    def _q_fetch_plan(self, ordered: List[Path], ahead: int = 64):
+        """Which table vectors to request before each path of ``ordered``: those of the paths that
+        start within the next ``ahead`` multiply-adds (and were not requested yet), so that a path's
+        products have arrived by the time its first instruction needs them. Returns a list, per path,
+        of vector indices; the caller declares them at the scope of the whole contraction."""
+        low = self.low
+        groups = []
+        for p in ordered:
+            gs = set()
+            for v in range(low.in2[p.i2].mul):
+                sl = self._q_slots_of(p, v)
+                gs |= set(range(min(sl) // 4, max(sl) // 4 + 1))
+            groups.append(sorted(gs))
+        plan, declared, reach = [], set(), 0
+        for k in range(len(ordered)):
+            work, m = 0, k
+            want = []
+            while m < len(ordered) and (m == k or work < ahead):
+                want += [g for g in groups[m] if g not in declared and g not in want]
+                work += len(ordered[m].nnz) * low.in2[ordered[m].i2].mul
+                m += 1
+            declared |= set(want)
+            plan.append(want)
+        return plan
+
+    def _emit_q_fetch(self, s: Src, want: List[int]):
+        for g in want:
+            s(f"const oeq_q4 qg{g} = *(const oeq_q4*)(sq + {4 * g});")
+        if want and self.q_pin:
+            # keep the requests here: the scheduler would otherwise sink them to their first use
+            s("__builtin_amdgcn_sched_barrier(0);")
+
+    def _emit_q_raw_y(self, s: Src):
+        """The raw Y row (table slots 0..L2-1), for the contractions that use it beside the products."""
+        for g in range(-(-self.low.L2 // 4)):
+            s(f"const oeq_q4 qy{g} = *(const oeq_q4*)(sq + {4 * g});")
+
     def _products(self, s: Src, p: Path, v: str, yacc) -> Dict[int, Tuple[str, bool]]:
         """Emit the distinct |c|*y_j products of a path. Returns nnz index ->
         (operand name, negative)."""
+        if self.use_q:
+            b2 = self.low.in2[p.i2]
+            for j in sorted({j for _, j, _, _ in p.nnz}):
+                yidx = b2.off + (j * b2.mul + int(v) if self.ir_mul else int(v) * b2.d + j)
+                s(f"const T y{j} = qy{yidx // 4}.v[{yidx % 4}];")
+            slots = self._q_slots_of(p, int(v))
+            return {n: (f"qg{t // 4}.v[{t % 4}]", p.nnz[n][3] < 0) for n, t in enumerate(slots)}
         for j in sorted({j for _, j, _, _ in p.nnz}):
             s(f"const T y{j} = {yacc(p, v, j)};")
         names: Dict[Tuple[str, int], str] = {}
@@ -459,7 +575,12 @@ class UvuEmitter:
         for io in self.used_out:
             s(f"    T o{io}[{low.out[io].d}];")
         s("};")
-        if self.can_preload:
+        if self.can_preload and self.q_entries:
+            # y: the edge's Y row; yq: the Y values this lane multiplies for the wave's product table
+            # (a kernel uses one of the two)
+            self.emit_q_tables(s)
+            s(f"struct E_t {{ X_t x; T w[{self.n_wslots}]; T y[{low.L2}]; T yq[{self.q_slabs}]; }};")
+        elif self.can_preload:
             s(f"struct E_t {{ X_t x; T w[{self.n_wslots}]; T y[{low.L2}]; }};")
         for si, seg in enumerate(self.segments):
             s(f"struct A{si}_t {{")
@@ -489,7 +610,7 @@ class UvuEmitter:
         s.open(
             f"OEQ_DEV void {name}{self._sfx()}(E_t& d, const i64 e, const T* __restrict__ L1_in, "
             "const T* __restrict__ L2_in, "
-            "const T* __restrict__ W, const i64* __restrict__ cols, const int u)"
+            f"const T* __restrict__ W, const i64* __restrict__ cols, const int u{', const Q_t& qt' if self.use_q else ''})"
         )
         s("const i64 c = cols[e];")
         s(f"const T* xrow = L1_in + c * {low.L1};")
@@ -500,12 +621,23 @@ class UvuEmitter:
             for v in range(low.in2[p.i2].mul):
                 s(f"d.w[{self.wslot[p.index] + v}] = {wptr(p, str(v))};")
         self._load_x(s, "xrow", in1_blocks, "d.x")
-        for j in range(low.L2):
-            s(f"d.y[{j}] = yrow[{j}];")
+        if self.use_q:
+            for r in range(self.q_slabs):
+                s(f"d.yq[{r}] = yrow[qt.j[{r}]];")
+        else:
+            for j in range(low.L2):
+                s(f"d.y[{j}] = yrow[{j}];")
         s.close()
 
     # --------------------------------------------------------- forward cores
     def _emit_fwd_seg(self, s: Src, si: int, preloaded):
+        if self.use_q and preloaded is not True:
+            # only the register-operand variant reads the product table
+            self.use_q = False
+            try:
+                return self._emit_fwd_seg(s, si, preloaded)
+            finally:
+                self.use_q = True
         low = self.low
         seg = self.segments[si]
         if preloaded == "lds":
@@ -513,7 +645,8 @@ class UvuEmitter:
             s.open(f"OEQ_DEV void fwd_seg{si}_lds{self._sfx()}(const T* sb, const int ul, A{si}_t& a)")
         elif preloaded:
             yacc, wacc = self._acc_preloaded("d")
-            s.open(f"OEQ_DEV void fwd_seg{si}_pre{self._sfx()}(const E_t& d, A{si}_t& a)")
+            s.open(f"OEQ_DEV void fwd_seg{si}_pre{self._sfx()}(const E_t& d, {'const T* sq, ' if self.use_q else ''}"
+                   f"A{si}_t& a)")
             xname = "d.x"
         else:
             yacc, wacc = self._acc_pointer()
@@ -522,11 +655,15 @@ class UvuEmitter:
                 f"const T* __restrict__ wrow, const int u, A{si}_t& a)"
             )
             xname = "x"
-        for p in self._paths():
-            if p.io not in seg:
-                continue
+        seg_paths = [p for p in self._paths() if p.io in seg]
+        if self.use_q:
+            qplan = self._q_fetch_plan(seg_paths, self.q_ahead[0])
+            self._emit_q_raw_y(s)
+        for n_p, p in enumerate(seg_paths):
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
             s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l}) in1[{p.i1}] x in2[{p.i2}] -> out[{p.io}], nnz={len(p.nnz)}")
+            if self.use_q:
+                self._emit_q_fetch(s, qplan[n_p])
 
             def body(v, p=p):
                 prods = self._products(s, p, v, yacc)
@@ -754,7 +891,7 @@ class UvuEmitter:
             return
         if pipelined == 2:
             # one LDS buffer per wave, copied to registers before the next edge's loads are issued
-            s(f"T yn[{self.low.L2}];")
+            s(f"T yn[{self.q_slabs if self.use_q else self.low.L2}];")
             s(f"i64 e = {first};")
             s.open(f"if (e < {last})")
             self._emit_stage_issue(s, "e")
@@ -807,7 +944,7 @@ class UvuEmitter:
     def _edge_mode(self, pipelined: int) -> int:
         """0: load, then compute; 1: next edge's operands prefetched into a second register set;
         2: next edge's operands prefetched into the wave's LDS staging buffer."""
-        if pipelined == 3 and self.stage3 is not None:
+        if pipelined == 3 and self.stage3 is not None and not self.use_q:
             return 3
         if pipelined >= 2 and self.stage is not None:
             return 2
@@ -820,12 +957,16 @@ class UvuEmitter:
         round-robin; with ``xcd`` > 1 (grid a multiple of it) block ids are remapped
         so that each XCD walks one contiguous range of nodes and neighbouring
         receivers share their senders' rows through that XCD's L2."""
+        # ``order`` (may be NULL) lists the nodes in the order in which they are to be walked: nodes that
+        # share senders next to each other, so that the blocks resident on one XCD gather from a small set
+        # of sender rows (the library derives it from the graph at every call).
         if xcd > 1:
             s(f"const i64 vper = (i64)gridDim.x / {xcd};")
             s(f"const i64 vblk = ((i64)blockIdx.x % {xcd}) * vper + (i64)blockIdx.x / {xcd};")
-            s.open(f"for (i64 node = vblk * {G} + g; node < node_count; node += node_count + 1)")
+            s.open(f"for (i64 vnode = vblk * {G} + g; vnode < node_count; vnode += node_count + 1)")
         else:
-            s.open(f"for (i64 node = (i64)blockIdx.x * {G} + g; node < node_count; node += (i64)gridDim.x * {G})")
+            s.open(f"for (i64 vnode = (i64)blockIdx.x * {G} + g; vnode < node_count; vnode += (i64)gridDim.x * {G})")
+        s("const i64 node = order ? order[vnode] : vnode;")
 
     def emit_conv_forward(self, s: Src, G: int, deterministic: bool, pipelined: bool, waves_per_eu: int = 0,
                           xcd: int = 1, tr_atomics: bool = True):
@@ -841,9 +982,11 @@ class UvuEmitter:
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void forward(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
             "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-            "const i64* __restrict__ rowptr, const i64* __restrict__ eperm)"
+            "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order)"
         )
         self._lane_prologue(s, segw)
+        if self.use_q:
+            self._emit_q_prologue(s, block // 64)
         if self.can_preload:
             s("E_t A, B;")
         if mode == 2:
@@ -860,7 +1003,7 @@ class UvuEmitter:
         def make_load(si):
             def load(buf, e):
                 if self.can_preload:
-                    s(f"load_edge_f{si}{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u);")
+                    s(f"load_edge_f{si}{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u{self._qarg()});")
             return load
 
         kahan = self.kahan and deterministic
@@ -877,7 +1020,9 @@ class UvuEmitter:
             if mode == 3:
                 s(f"fwd_seg{si}_lds{self._sfx()}(&s_stage{buf}[wave][0], ul, {acc});")
             elif self.can_preload:
-                s(f"fwd_seg{si}_pre{self._sfx()}({buf}, {acc});")
+                if self.use_q:
+                    self._emit_q_build(s, f"{buf}.yq")
+                s(f"fwd_seg{si}_pre{self._sfx()}({buf}, {'sq, ' if self.use_q else ''}{acc});")
             else:
                 s.open("")
                 s(f"const i64 eid = OEQ_EDGE({e});")
@@ -1007,10 +1152,15 @@ class UvuEmitter:
         run_of = {q.index: ri for ri, run in enumerate(runs) for q in run}
         if prefetch:
             emit_run_loads(runs[0])
+        if self.use_q:
+            qplan = self._q_fetch_plan(ordered, self.q_ahead[1])
+            self._emit_q_raw_y(s)
         for n_path, p in enumerate(ordered):
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
             V = b2.mul
             s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
+            if self.use_q:
+                self._emit_q_fetch(s, qplan[n_path])
             if prefetch and runs[run_of[p.index]][0] is p and run_of[p.index] + 1 < len(runs):
                 emit_run_loads(runs[run_of[p.index] + 1])
             s.open("")
@@ -1197,6 +1347,76 @@ class UvuEmitter:
                     s(f"dp[{i * st}] = dx.b{b}[{i}];")
             s.close()
 
+    def _term_slots(self):
+        """Position of (input block, component) in a wave's lane-major slice of a per-edge dX term row:
+        value (b, i) of lane ``ul`` sits at ``chunk * 64 * n + slot * 64 + ul`` (n = number of slots), so
+        every store or load instruction of the wave covers 64 consecutive elements."""
+        slots, n = {}, 0
+        for b in self.used_in1:
+            for i in range(self.low.in1[b].d):
+                slots[(b, i)] = n
+                n += 1
+        return slots, n
+
+    def _term_ptr(self, rowexpr: str, slot: int, n: int) -> str:
+        return f"oeq_at({rowexpr} + chunk * {64 * n} + {slot * 64}, (unsigned)ul * {self.low.elem_size}u)"
+
+    def _store_terms(self, s: Src, rowexpr: str):
+        slots, n = self._term_slots()
+        for (b, i), slot in slots.items():
+            ptr = self._term_ptr(rowexpr, slot, n)
+            s(f"*{ptr} = dx.b{b}[{i}];")
+
+    def _load_terms(self, s: Src, rowexpr: str, dst: str):
+        slots, n = self._term_slots()
+        for (b, i), slot in slots.items():
+            ptr = self._term_ptr(rowexpr, slot, n)
+            s(f"{dst}.b{b}[{i}] = *{ptr};")
+
+    def _arrivals(self, s: Src):
+        """After a wave has stored the dX terms of its node's edges: make them visible to the device,
+        count one arrival per edge at the edge's sender (one counter per sender and channel chunk), and
+        for every sender whose count is now complete sum its terms in ``sperm`` order and write its row.
+        The last arrival is whichever wave happens to come last; the sum it forms does not depend on that."""
+        low = self.low
+        s("__threadfence();")  # release: this wave's terms before its arrivals
+        s.open("for (i64 eb = e0; eb < e1; eb += 64)")
+        s("const i64 ea = eb + lane;")
+        s("i64 sn = 0; bool last = false;")
+        s.open("if (ea < e1)")
+        s("sn = cols[OEQ_EDGE(ea)];")
+        s(f"const int seen = __hip_atomic_fetch_add(arrivals + sn * {self.NCH} + chunk, 1, __ATOMIC_RELAXED, "
+          "__HIP_MEMORY_SCOPE_AGENT) + 1;")
+        s("last = seen == (int)(colptr[sn + 1] - colptr[sn]);")
+        s.close()
+        s("unsigned long long todo = __ballot(last);")
+        s.open("while (todo)")
+        s("const int src_lane = __ffsll((long long)todo) - 1;")
+        s("todo &= todo - 1;")
+        s("const i64 snd = ((i64)__builtin_amdgcn_readlane((int)(sn >> 32), src_lane) << 32) | "
+          "(unsigned)__builtin_amdgcn_readlane((int)sn, src_lane);")
+        s("__threadfence();")  # acquire: the other waves' terms after their arrivals
+        s("X_t tot;")
+        self._zero_x(s, "tot")
+        s("const i64 j0 = colptr[snd], j1 = colptr[snd + 1];")
+        # the additions stay in list order; unrolling only lets several rows be in flight at a time
+        s("#pragma unroll 4")
+        s.open("for (i64 j = j0; j < j1; ++j)")
+        s(f"const T* trow = dx_tmp + sperm[j] * {low.L1};")
+        s("X_t t;")
+        self._load_terms(s, "trow", "t")
+        for b in self._in1_of(self.used_in1):
+            for i in range(low.in1[b].d):
+                s(f"tot.b{b}[{i}] += t.b{b}[{i}];")
+        s.close()
+        s(f"T* orow = L1_grad + snd * {low.L1};")
+        s.open("")
+        s("X_t& dx = tot;")
+        self._store_dx(s, "orow", "true")
+        s.close()
+        s.close()
+        s.close()
+
     def _zero_untouched_in1(self, s: Src, rowexpr: str, guard: str):
         low = self.low
         for b in range(len(low.in1)):
@@ -1376,9 +1596,12 @@ class UvuEmitter:
             "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
             "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
-            "T* __restrict__ wpartial)"
+            "T* __restrict__ wpartial, const i64* __restrict__ colptr, const i64* __restrict__ sperm, "
+            "int* __restrict__ arrivals, const i64* __restrict__ order)"
         )
         self._lane_prologue(s, SW)
+        if self.use_q:
+            self._emit_q_prologue(s, block // 64)
         if SW == 1:
             s("const int sg = 0;")
         s(f"__shared__ T s_dy[{SW * self.NCH}][{self.l2_pad}];")
@@ -1395,8 +1618,10 @@ class UvuEmitter:
                 # every wave of the block runs the same number of edges, so the block barriers match up
                 s.open("for (i64 e = e0; e < e1; ++e)")
                 s("const i64 eid = OEQ_EDGE(e);")
-                s(f"load_edge_b{si}{self._sfx()}(A, eid, L1_in, L2_in, W, cols, u);")
+                s(f"load_edge_b{si}{self._sfx()}(A, eid, L1_in, L2_in, W, cols, u{self._qarg()});")
                 yacc, wacc = self._acc_preloaded("A")
+                if self.use_q:
+                    self._emit_q_build(s, "A.yq")
                 s(f"T* dwrow = W_grad + eid * {low.WN};")
                 s("X_t dx;")
                 self._zero_x(s, "dx")
@@ -1460,8 +1685,20 @@ class UvuEmitter:
         s.close()
         return block
 
+    DX_TERMS, DX_ATOMIC, DX_ARRIVAL = 0, 1, 2
+
     def emit_conv_backward(self, s: Src, deterministic: bool, G: int, pipelined: bool, waves_per_eu: int = 0,
-                           g_resident: Optional[bool] = None, xcd: int = 1, tr_atomics: bool = True):
+                           g_resident: Optional[bool] = None, xcd: int = 1, tr_atomics: bool = True,
+                           dx_mode: int = 0):
+        """``deterministic``: the kernel walks each receiver's edge segment. What happens to the per-edge
+        dX terms of the walk is ``dx_mode``: DX_TERMS writes them to ``dx_tmp`` for the sender-ordered
+        reduction of ``fixup_backward``; DX_ATOMIC adds them into the (cleared) sender rows with float
+        atomics; DX_ARRIVAL writes them to ``dx_tmp`` and counts, per sender and channel chunk, the terms
+        that have arrived: the wave that delivers a sender's last term sums that sender's terms in the
+        order of ``sperm`` and writes the row, so the reduction needs no kernel of its own and stays
+        bit-identical to ``fixup_backward``. (At the MACE shape the walk kernel is bound by its memory
+        traffic, the in-kernel reduction adds the same 13 GB of reads to it, and the sum comes out slower
+        than the separate kernel: 15.0 against 14.6 ms. Hence opt-in, ``conv_dxm=2``.)"""
         low = self.low
         shared = low.shared_weights
         if self.NCH > 1:
@@ -1479,9 +1716,12 @@ class UvuEmitter:
             "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
             "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
-            "T* __restrict__ wpartial)"
+            "T* __restrict__ wpartial, const i64* __restrict__ colptr, const i64* __restrict__ sperm, "
+            "int* __restrict__ arrivals, const i64* __restrict__ order)"
         )
         self._lane_prologue(s)
+        if self.use_q:
+            self._emit_q_prologue(s, block // 64)
         if self.NCH > 1:
             s(f"__shared__ T s_dy[{G}][{self.NCH}][{self.l2_pad}];")
         if shared:
@@ -1496,14 +1736,17 @@ class UvuEmitter:
             for b in "AB":
                 s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
             self._emit_stage3_offsets(s)
-        self.tr_atomics = (not deterministic) and tr_atomics and self._regular_wave() and not self.ir_mul
+        dx_atomic = (not deterministic) or dx_mode == self.DX_ATOMIC
+        self.tr_atomics = dx_atomic and tr_atomics and self._regular_wave() and not self.ir_mul
         if self.tr_atomics or (self.tr_stores & 2 and self.R == 1):
             s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.in1[b].d for b in self.used_in1)}];")
         resident = deterministic and (self.g_resident if g_resident is None else g_resident)
+        if dx_mode == self.DX_ARRIVAL:
+            assert deterministic and self.R == 1, "arrival counting needs the receiver walk and rows that fill a wave"
 
         def load(buf, e):
             if self.can_preload:
-                s(f"load_edge_b{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u);")
+                s(f"load_edge_b{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u{self._qarg()});")
 
         def make_compute(grow_expr_of):
             def compute(buf, pos):
@@ -1516,6 +1759,8 @@ class UvuEmitter:
                 elif self.can_preload:
                     yacc, wacc = self._acc_preloaded(buf)
                     xname = f"{buf}.x"
+                    if self.use_q:
+                        self._emit_q_build(s, f"{buf}.yq")
                 else:
                     yacc, wacc = self._acc_pointer()
                     xname = "x"
@@ -1547,10 +1792,14 @@ class UvuEmitter:
                 self._pin_gradients(s, self.used_in1, deferred)
                 if deferred:
                     self._flush_dwkeep(s, None)
-                if deterministic:
+                if not dx_atomic:
                     s(f"T* dxrow = dx_tmp + {e} * {low.L1};")
-                    self._store_dx(s, "dxrow", "true", nt=bool(self.nt & 2))
-                    self._zero_untouched_in1(s, "dxrow", "true")
+                    # terms the arrival scheme re-reads soon are stored plainly, so that they stay cached
+                    if dx_mode == self.DX_ARRIVAL:
+                        self._store_terms(s, "dxrow")
+                    else:
+                        self._store_dx(s, "dxrow", "true", nt=bool(self.nt & 2))
+                        self._zero_untouched_in1(s, "dxrow", "true")
                 else:
                     s(f"T* dxrow = L1_grad + cols[{e}] * {low.L1};")
                     self._store_dx(s, "dxrow", "true", atomic=True)
@@ -1570,6 +1819,8 @@ class UvuEmitter:
                 # block barriers of the dY reduction are reached uniformly (also across per-chunk bodies)
                 self._edge_loop(s, "e0 + r", "e1", load, make_compute(lambda e: f"L3_grad + node * {low.L3}"),
                                 mode)
+                if dx_mode == self.DX_ARRIVAL:
+                    self._arrivals(s)
 
             self._per_chunk(s, node_body)
             s.close()
@@ -1686,7 +1937,8 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=112, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
-                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fw=0, conv_pf=0))
+                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fw=0, conv_pf=0,
+                    conv_dxm=-1, conv_q=1, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -1737,6 +1989,14 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                 if need <= 190:
                     break
     em.nt = t["conv_nt"]
+    q_fwd = q_bwd = False
+    if t["conv_q"] and em.q_supported():
+        # bit 0: forward, bit 1: backward. Backward gains nothing at the MACE shape (it is bound by its
+        # memory traffic, and the table's vectors compete with the resident gradient slice for registers)
+        q_fwd, q_bwd = bool(t["conv_q"] & 1), bool(t["conv_q"] & 2)
+        em.q_pin = bool(t["conv_qpin"])
+        em.q_ahead = (t["conv_qaf"], t["conv_qab"])
+        em.build_q_table()
     if walk and len(em.segments) > 1 and t["conv_segw"] and em.stage is None and em.R == 1:
         em.seg_waves = max(1, min(len(em.segments), t["conv_segw"], 8 // em.NCH))
         t["conv_gf"] = max(1, min(t["conv_gf"], 8 // (em.NCH * em.seg_waves)))
@@ -1751,13 +2011,16 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     # position in the walk -> edge index: through the library's grouping when there is one
     s("#define OEQ_EDGE(j) (eperm ? eperm[(j)] : (j))")
     em.emit_structs(s)
+    em.use_q = q_fwd
     em.emit_forward_cores(s, preloaded=True)
     G_f = t["conv_gf"]
     G_b = 1 if em.NCH > 1 else t["conv_gb"]
     xcd = max(1, t["conv_xcd"])
     xcd_b = 1 if (walk and low.shared_weights) else xcd  # bounded grid: one partial dW row per wave group
     blk_f = em.emit_conv_forward(s, G_f, walk, t["conv_pipe_f"], t["conv_wf"], xcd, bool(t["conv_tra"]))
+    em.use_q = q_bwd
     gres = None if t["conv_gres"] < 0 else bool(t["conv_gres"])
+    dx_mode = 0
     em.group_budget = t["conv_gbud"]
     em.bwd_groups = em.plan_backward_groups(8 // em.NCH) if (walk and t["conv_split"] and gres is None) else None
     if em.bwd_groups:
@@ -1769,8 +2032,17 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             t["conv_wb"] = 3
         blk_b = em.emit_conv_backward_split(s, t["conv_wb"], xcd)
     else:
+        # what becomes of the walk's per-edge dX terms (UvuEmitter.emit_conv_backward)
+        if walk and not kahan:
+            # deterministic=False may use float atomics, and adding the terms straight into the sender
+            # rows saves their round trip through scratch memory and the second kernel; the caller-sorted
+            # mode promises the same bits on every run and keeps the ordered reduction
+            dx_mode = t["conv_dxm"] if t["conv_dxm"] >= 0 else (em.DX_ATOMIC if mode == rt.CONV_GROUPED
+                                                                  else em.DX_TERMS)
+            if dx_mode == em.DX_ARRIVAL and em.R != 1:
+                dx_mode = em.DX_TERMS
         blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd_b,
-                                      bool(t["conv_tra"]))
+                                      bool(t["conv_tra"]), dx_mode)
         G_b = em.backward_groups_per_block
     descs = [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
@@ -1788,13 +2060,14 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         from . import uvu_double
         if t["conv_dd"] and uvu_double.supported(low, conv=True) and not kahan:
             descs += uvu_double.add_conv_kernels(s, low, em, t, xcd)
-        if mode == rt.CONV_GROUPED:
-            descs += [
-                (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, compute_units * 16),
-                (rt.ROLE_GROUP_SCAN, "oeq_group_scan", 1024, 1, 1),
-                (rt.ROLE_GROUP_SCATTER, "oeq_group_scatter", 256, 256 * 4, compute_units * 16),
-                (rt.ROLE_GROUP_ORDER, "oeq_group_order", 256, 4, compute_units * 32),
-            ]
+        # counting sort: of the edge indices by node (GROUPED mode) and of the nodes by cluster (walk order)
+        descs += [
+            (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, compute_units * 16),
+            (rt.ROLE_GROUP_SCAN, "oeq_group_scan", 1024, 1, 1),
+            (rt.ROLE_GROUP_SCATTER, "oeq_group_scatter", 256, 256 * 4, compute_units * 16),
+            (rt.ROLE_GROUP_ORDER, "oeq_group_order", 256, 4, compute_units * 32),
+            (rt.ROLE_ORDER_HOP, "oeq_order_hop", 256, 256, compute_units * 16),
+        ]
     else:
         # edge ranges: about conv_epw consecutive edges per wave group
         epw = max(1, t["conv_epw"])
@@ -1804,5 +2077,6 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         ]
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
                 shared_weights=int(low.shared_weights), deterministic=mode,
-                wpartial_per_block=G_b if (walk and low.shared_weights) else 0)
+                wpartial_per_block=G_b if (walk and low.shared_weights) else 0, dx_mode=dx_mode,
+                n_chunks=em.NCH, order_hops=max(0, t["conv_hops"]) if walk else 0)
     return s.text(), dims, descs

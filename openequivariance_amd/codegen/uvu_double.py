@@ -380,7 +380,8 @@ class DoubleEmitter(UvuEmitter):
         s.open(
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_A(i64 node_count, '
             f"i64 nnz, {self._CONV_OPERANDS}T* __restrict__ L3_dgrad, const i64* __restrict__ rows, "
-            "const i64* __restrict__ cols, const i64* __restrict__ rowptr, const i64* __restrict__ eperm)"
+            "const i64* __restrict__ cols, const i64* __restrict__ rowptr, const i64* __restrict__ eperm, "
+            "const i64* __restrict__ order)"
         )
         self._lane_prologue(s, segw)
         if self.tr_stores & 1 and self.R == 1:
@@ -431,7 +432,7 @@ class DoubleEmitter(UvuEmitter):
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
-            "T* __restrict__ L3_dgrad)"
+            "T* __restrict__ L3_dgrad, const i64* __restrict__ order)"
         )
         self._lane_prologue(s)
         if self.NCH > 1:
@@ -568,7 +569,7 @@ class DoubleEmitter(UvuEmitter):
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
-            "T* __restrict__ L3_dgrad)"
+            "T* __restrict__ L3_dgrad, const i64* __restrict__ order)"
         )
         self._lane_prologue(s, SW)
         s(f"__shared__ T s_dy[{SW * self.NCH}][{self.l2_pad}];")

@@ -10,6 +10,7 @@
 #include <hip/hiprtc.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -72,7 +73,7 @@ struct oeq_kernels {
     RoleInfo roles[OEQ_ROLE_COUNT];
     std::mutex mu;
     DeviceSlot slots[kMaxDevices];
-    bool timing = false;
+    std::atomic<bool> timing{false};
     std::vector<TimedLaunch> timed;
 
     // Resolve the function for `role` on the current device (loading the code
@@ -122,7 +123,7 @@ struct oeq_kernels {
         int rc = functions(role, &fns);
         if (rc) return rc;
         unsigned grid = grid_for(role, units);
-        if (!timing) {
+        if (!timing.load(std::memory_order_relaxed)) {
             for (hipFunction_t fn : *fns)
                 HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, roles[role].block, 1, 1, 0, (hipStream_t)stream, args,
                                               nullptr));
@@ -155,6 +156,23 @@ struct oeq_kernels {
         return launch(OEQ_ROLE_SEGMENT_PTR, n_items + 1, args, stream);
     }
 
+    // Item indices grouped by key, in no particular order within a group: ptr[0..n_segments] = group
+    // starts, perm = the grouped indices; cursor (n_segments+1) is scratch.
+    int group_unordered(int64_t n_items, int64_t n_segments, const int64_t* keys, int64_t* ptr, int64_t* cursor,
+                        int64_t* perm, void* stream) {
+        int rc = fill_zero(ptr, (size_t)(n_segments + 1) * sizeof(int64_t), stream);
+        if (rc) return rc;
+        void* cargs[] = {&n_items, &keys, &ptr};
+        rc = launch(OEQ_ROLE_GROUP_COUNT, n_items, cargs, stream);
+        if (rc) return rc;
+        int64_t n = n_segments + 1;
+        void* sargs[] = {&n, &ptr, &cursor};
+        rc = launch(OEQ_ROLE_GROUP_SCAN, 1, sargs, stream);
+        if (rc) return rc;
+        void* pargs[] = {&n_items, &keys, &cursor, &perm};
+        return launch(OEQ_ROLE_GROUP_SCATTER, n_items, pargs, stream);
+    }
+
     // Counting sort of the item indices 0..n_items-1 by key: ptr[0..n_segments] = segment starts,
     // perm = item indices grouped by key, ascending within a group (so the result depends on the key
     // list only); cursor (n_segments+1) and unordered (n_items) are scratch.
@@ -180,7 +198,7 @@ struct oeq_kernels {
 extern "C" {
 
 const char* oeq_last_error(void) { return g_error.c_str(); }
-int oeq_abi_version(void) { return 1; }
+int oeq_abi_version(void) { return 2; }
 
 int oeq_get_device_props(int device, oeq_device_props* out) {
     if (!out) return fail(OEQ_ERR_INVALID, "oeq_get_device_props: out is NULL");
@@ -347,8 +365,7 @@ int oeq_grouped_sum(oeq_kernels* k, int64_t n_segments, int64_t n_items, int64_t
 
 int oeq_kernel_timing_enable(oeq_kernels* k, int enable) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_kernel_timing_enable: NULL kernel set");
-    std::lock_guard<std::mutex> lock(k->mu);
-    k->timing = enable != 0;
+    k->timing.store(enable != 0, std::memory_order_relaxed);
     return OEQ_OK;
 }
 
@@ -427,17 +444,10 @@ int oeq_tp_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in, void* 
 // fused graph convolution
 // ---------------------------------------------------------------------------
 
-// Workspace layouts. SORTED: forward [rowptr]; backward [rowptr | colptr | dx_tmp].
-// GROUPED: forward [rowptr | cursor | rperm | scratch perm];
-//          backward [rowptr | colptr | cursor | rperm | sperm | scratch perm | dx_tmp].
+// Workspace of the walk modes: one layout for every convolution entry point (pieces a call does not need
+// are left out).
 static size_t ptr_bytes_of(int64_t node_count) { return align_up((size_t)(node_count + 1) * sizeof(int64_t), 256); }
 static size_t perm_bytes_of(int64_t nnz) { return align_up((size_t)nnz * sizeof(int64_t), 256); }
-
-size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
-    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
-    if (k->dims.deterministic == OEQ_CONV_SORTED) return ptr_bytes_of(node_count);
-    return 2 * ptr_bytes_of(node_count) + 2 * perm_bytes_of(nnz);
-}
 
 // Shared weights, walk kernels: one partial weight-gradient row per wave group of the backward grid.
 static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t node_count) {
@@ -446,53 +456,125 @@ static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t node_count) {
     return align_up(rows * (size_t)k->dims.weight_numel * (size_t)k->dims.elem_size, 256);
 }
 
-size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
-    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
-    size_t tmp_bytes = align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256) +
-                       conv_wpartial_bytes(k, node_count);
-    if (k->dims.deterministic == OEQ_CONV_SORTED) return 2 * ptr_bytes_of(node_count) + tmp_bytes;
-    return 3 * ptr_bytes_of(node_count) + 3 * perm_bytes_of(nnz) + tmp_bytes;
+// Byte offsets of the pieces of a call's workspace (SIZE_MAX: piece not present).
+// `terms`: the per-edge dX terms and the sender-side index that their reduction walks;
+// `arrivals`: the per-sender arrival counters of OEQ_DX_ARRIVAL; `wpartial`: partial weight-gradient rows.
+struct WalkLayout {
+    size_t rowptr = SIZE_MAX, colptr = SIZE_MAX, cursor = SIZE_MAX, rperm = SIZE_MAX, sperm = SIZE_MAX,
+           scratch = SIZE_MAX, key_a = SIZE_MAX, key_b = SIZE_MAX, optr = SIZE_MAX, ocursor = SIZE_MAX,
+           order = SIZE_MAX, arrivals = SIZE_MAX, dx_tmp = SIZE_MAX, wpartial = SIZE_MAX, total = 0;
+};
+
+static WalkLayout walk_layout(const oeq_kernels* k, int64_t node_count, int64_t nnz, bool terms, bool arrivals,
+                              bool wpartial) {
+    WalkLayout w;
+    const size_t pb = ptr_bytes_of(node_count), qb = perm_bytes_of(nnz);
+    auto take = [&w](size_t bytes) { size_t at = w.total; w.total += bytes; return at; };
+    w.rowptr = take(pb);
+    if (terms) w.colptr = take(pb);
+    if (k->dims.deterministic == OEQ_CONV_GROUPED) {
+        w.cursor = take(pb);
+        w.rperm = take(qb);
+        if (terms) w.sperm = take(qb);
+        w.scratch = take(qb);
+    }
+    if (k->dims.order_hops > 0 && k->roles[OEQ_ROLE_ORDER_HOP].present) {
+        w.key_a = take(pb);
+        w.key_b = take(pb);
+        w.optr = take(pb);
+        w.ocursor = take(pb);
+        w.order = take(pb);
+    }
+    if (arrivals)
+        w.arrivals = take(align_up((size_t)node_count * (size_t)std::max(1, k->dims.n_chunks) * sizeof(int32_t), 256));
+    if (terms) w.dx_tmp = take(align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256));
+    if (wpartial)
+        if (size_t wp = conv_wpartial_bytes(k, node_count)) w.wpartial = take(wp);
+    return w;
 }
 
-// What the walk kernels of a backward-type call need besides the operands: CSR pointers over receivers and
-// over senders, the walk orders (GROUPED mode: built here; SORTED mode: the caller's lists), and the
-// buffer of per-edge dX terms. Everything lives in the caller's workspace (layouts above).
+size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
+    return walk_layout(k, node_count, nnz, false, false, false).total;
+}
+
+static WalkLayout backward_layout(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    return walk_layout(k, node_count, nnz, k->dims.dx_mode != OEQ_DX_ATOMIC, k->dims.dx_mode == OEQ_DX_ARRIVAL,
+                       true);
+}
+
+size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
+    return backward_layout(k, node_count, nnz).total;
+}
+
+// the second-order kernels always go through the per-edge terms and fixup_backward
+size_t oeq_conv_double_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
+    return walk_layout(k, node_count, nnz, true, false, false).total;
+}
+
+// What the walk kernels of a backward-type call need besides the operands: CSR pointers over receivers and,
+// when the per-edge terms are kept, over senders; the walk orders (GROUPED mode: built here; SORTED mode: the
+// caller's lists); the buffer of per-edge dX terms. Everything lives in the caller's workspace.
 struct WalkIndex {
     int64_t *rowptr = nullptr, *colptr = nullptr, *rperm = nullptr;
     const int64_t* sperm = nullptr;
-    void* dx_tmp = nullptr;
+    void *dx_tmp = nullptr, *wpartial = nullptr;
+    int32_t* arrivals = nullptr;
+    int64_t* order = nullptr;  // the order in which the walk kernels visit the nodes (NULL: by index)
 };
 
-static int walk_index(oeq_kernels* k, const char* who, int64_t node_count, int64_t nnz, const int64_t* rows,
-                      const int64_t* cols, const int64_t* transpose_perm, void* workspace, size_t workspace_bytes,
-                      void* stream, WalkIndex* ix) {
+static int walk_index(oeq_kernels* k, const char* who, const WalkLayout& w, int64_t node_count, int64_t nnz,
+                      const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* workspace,
+                      size_t workspace_bytes, void* stream, WalkIndex* ix) {
     const int mode = k->dims.deterministic;
-    if (mode == OEQ_CONV_SORTED && !transpose_perm)
+    const bool terms = w.dx_tmp != SIZE_MAX;
+    if (mode == OEQ_CONV_SORTED && terms && !transpose_perm)
         return fail(OEQ_ERR_INVALID, "%s: deterministic mode needs transpose_perm", who);
-    size_t need = oeq_conv_backward_workspace_bytes(k, node_count, nnz);
-    if (!workspace || workspace_bytes < need)
-        return fail(OEQ_ERR_INVALID, "%s: workspace too small (%zu < %zu bytes)", who, workspace_bytes, need);
-    const size_t pb = ptr_bytes_of(node_count), qb = perm_bytes_of(nnz);
-    ix->rowptr = (int64_t*)workspace;
-    ix->colptr = (int64_t*)((char*)workspace + pb);
+    if (!workspace || workspace_bytes < w.total)
+        return fail(OEQ_ERR_INVALID, "%s: workspace too small (%zu < %zu bytes)", who, workspace_bytes, w.total);
+    char* base = (char*)workspace;
+    auto at = [base](size_t off) -> char* { return off == SIZE_MAX ? nullptr : base + off; };
+    ix->rowptr = (int64_t*)at(w.rowptr);
+    ix->colptr = (int64_t*)at(w.colptr);
+    ix->dx_tmp = at(w.dx_tmp);
+    ix->wpartial = at(w.wpartial);
+    ix->arrivals = (int32_t*)at(w.arrivals);
     ix->sperm = transpose_perm;
     int rc;
     if (mode == OEQ_CONV_SORTED) {
-        ix->dx_tmp = (char*)workspace + 2 * pb;
         rc = k->segment_ptr(nnz, node_count, rows, nullptr, ix->rowptr, stream);
-        if (rc) return rc;
-        return k->segment_ptr(nnz, node_count, cols, transpose_perm, ix->colptr, stream);
+        if (!rc && terms) rc = k->segment_ptr(nnz, node_count, cols, transpose_perm, ix->colptr, stream);
+    } else {
+        int64_t* cursor = (int64_t*)at(w.cursor);
+        int64_t* scratch = (int64_t*)at(w.scratch);
+        ix->rperm = (int64_t*)at(w.rperm);
+        rc = k->group_by_key(nnz, node_count, rows, ix->rowptr, cursor, scratch, ix->rperm, stream);
+        if (!rc && terms) {
+            int64_t* sp = (int64_t*)at(w.sperm);
+            rc = k->group_by_key(nnz, node_count, cols, ix->colptr, cursor, scratch, sp, stream);
+            ix->sperm = sp;
+        }
     }
-    int64_t* cursor = (int64_t*)((char*)workspace + 2 * pb);
-    ix->rperm = (int64_t*)((char*)workspace + 3 * pb);
-    int64_t* sp = (int64_t*)((char*)workspace + 3 * pb + qb);
-    int64_t* scratch = (int64_t*)((char*)workspace + 3 * pb + 2 * qb);
-    ix->dx_tmp = (char*)workspace + 3 * pb + 3 * qb;
-    rc = k->group_by_key(nnz, node_count, rows, ix->rowptr, cursor, scratch, ix->rperm, stream);
-    if (rc) return rc;
-    rc = k->group_by_key(nnz, node_count, cols, ix->colptr, cursor, scratch, sp, stream);
-    ix->sperm = sp;
-    return rc;
+    if (rc || w.order == SIZE_MAX) return rc;
+    // Walk order: cluster the nodes by the highest-priority node within `order_hops` edges, then list them
+    // cluster by cluster (a counting sort by cluster key; the order inside a cluster is whatever the
+    // scatter's atomics give, which changes which nodes run side by side but no result).
+    int64_t* keys[2] = {(int64_t*)at(w.key_a), (int64_t*)at(w.key_b)};
+    const int64_t* key_in = nullptr;
+    const int64_t* cperm = ix->rperm;
+    for (int h = 0; h < k->dims.order_hops; ++h) {
+        int64_t* key_out = keys[h & 1];
+        void* hargs[] = {&node_count, &ix->rowptr, &cols, &cperm, &key_in, &key_out};
+        rc = k->launch(OEQ_ROLE_ORDER_HOP, node_count, hargs, stream);
+        if (rc) return rc;
+        key_in = key_out;
+    }
+    int64_t* optr = (int64_t*)at(w.optr);
+    int64_t* ocursor = (int64_t*)at(w.ocursor);
+    ix->order = (int64_t*)at(w.order);
+    return k->group_unordered(node_count, node_count, key_in, optr, ocursor, ix->order, stream);
 }
 
 int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
@@ -505,30 +587,18 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void
     const size_t out_bytes = (size_t)node_count * k->dims.L3_dim * k->dims.elem_size;
     if (nnz == 0) return k->fill_zero(L3_out, out_bytes, stream);
     if (!L1_in || !L2_in || !W || !rows || !cols) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL buffer");
-    int64_t *rowptr = nullptr, *rperm = nullptr;
+    WalkIndex ix;
     const int mode = k->dims.deterministic;
     int rc;
     if (mode != OEQ_CONV_ATOMIC) {
-        size_t need = oeq_conv_forward_workspace_bytes(k, node_count, nnz);
-        if (!workspace || workspace_bytes < need)
-            return fail(OEQ_ERR_INVALID, "oeq_conv_forward: workspace too small (%zu < %zu bytes)", workspace_bytes,
-                        need);
-        rowptr = (int64_t*)workspace;
-        if (mode == OEQ_CONV_SORTED) {
-            rc = k->segment_ptr(nnz, node_count, rows, nullptr, rowptr, stream);
-        } else {
-            const size_t pb = ptr_bytes_of(node_count);
-            int64_t* cursor = (int64_t*)((char*)workspace + pb);
-            rperm = (int64_t*)((char*)workspace + 2 * pb);
-            int64_t* scratch = (int64_t*)((char*)workspace + 2 * pb + perm_bytes_of(nnz));
-            rc = k->group_by_key(nnz, node_count, rows, rowptr, cursor, scratch, rperm, stream);
-        }
+        rc = walk_index(k, "oeq_conv_forward", walk_layout(k, node_count, nnz, false, false, false), node_count, nnz,
+                        rows, cols, nullptr, workspace, workspace_bytes, stream, &ix);
         if (rc) return rc;
     } else {
         rc = k->fill_zero(L3_out, out_bytes, stream);
         if (rc) return rc;
     }
-    void* args[] = {&node_count, &nnz, &L1_in, &L2_in, &W, &L3_out, &rows, &cols, &rowptr, &rperm};
+    void* args[] = {&node_count, &nnz, &L1_in, &L2_in, &W, &L3_out, &rows, &cols, &ix.rowptr, &ix.rperm, &ix.order};
     return k->launch(OEQ_ROLE_CONV_FORWARD, mode != OEQ_CONV_ATOMIC ? node_count : nnz, args, stream);
 }
 
@@ -556,32 +626,37 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
     if (!L1_in || !L2_in || !L2_grad || !W || !W_grad || !L3_grad || !rows || !cols)
         return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL buffer");
 
-    int64_t *rowptr = nullptr, *colptr = nullptr, *rperm = nullptr;
-    const int64_t* sperm = transpose_perm;
-    void *dx_tmp = nullptr, *wpartial = nullptr;
+    WalkIndex ix;
     const int mode = k->dims.deterministic;
+    const int dx_mode = mode == OEQ_CONV_ATOMIC ? (int)OEQ_DX_ATOMIC : k->dims.dx_mode;
     if (mode != OEQ_CONV_ATOMIC) {
-        WalkIndex ix;
-        rc = walk_index(k, "oeq_conv_backward", node_count, nnz, rows, cols, transpose_perm, workspace,
-                        workspace_bytes, stream, &ix);
+        rc = walk_index(k, "oeq_conv_backward", backward_layout(k, node_count, nnz), node_count, nnz, rows, cols,
+                        transpose_perm, workspace, workspace_bytes, stream, &ix);
         if (rc) return rc;
-        rowptr = ix.rowptr, colptr = ix.colptr, rperm = ix.rperm, sperm = ix.sperm, dx_tmp = ix.dx_tmp;
-        if (wrows)
-            wpartial = (char*)dx_tmp + align_up((size_t)nnz * (size_t)k->dims.L1_dim * es, 256);
-    } else {
+    }
+    if (dx_mode != OEQ_DX_TERMS) {
+        // atomics accumulate into the rows; the arrival scheme never visits a node that sends nothing
         rc = k->fill_zero(L1_grad, dx_bytes, stream);
         if (rc) return rc;
     }
-    void* args[] = {&node_count, &nnz,  &L1_in, &L1_grad, &L2_in,  &L2_grad, &W,
-                    &W_grad,     &L3_grad, &rows, &cols,    &rowptr, &dx_tmp, &rperm, &wpartial};
+    if (dx_mode == OEQ_DX_ARRIVAL) {
+        rc = k->fill_zero(ix.arrivals, (size_t)node_count * (size_t)std::max(1, k->dims.n_chunks) * sizeof(int32_t),
+                          stream);
+        if (rc) return rc;
+    }
+    void* args[] = {&node_count, &nnz,     &L1_in, &L1_grad, &L2_in,     &L2_grad,   &W,          &W_grad,   &L3_grad,
+                    &rows,       &cols,    &ix.rowptr, &ix.dx_tmp, &ix.rperm, &ix.wpartial, &ix.colptr, &ix.sperm,
+                    &ix.arrivals, &ix.order};
     rc = k->launch(OEQ_ROLE_CONV_BACKWARD, mode != OEQ_CONV_ATOMIC ? node_count : nnz, args, stream);
     if (rc || mode == OEQ_CONV_ATOMIC) return rc;
-    void* fargs[] = {&node_count, &nnz, &dx_tmp, &L1_grad, &sperm, &colptr};
-    rc = k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
+    if (dx_mode == OEQ_DX_TERMS) {
+        void* fargs[] = {&node_count, &nnz, &ix.dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};
+        rc = k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
+    }
     if (rc || !wrows) return rc;
     int64_t n_partials = (int64_t)k->grid_for(OEQ_ROLE_CONV_BACKWARD, node_count) * k->dims.wpartial_per_block;
     int64_t wn = k->dims.weight_numel;
-    void* rargs[] = {&n_partials, &wpartial, &W_grad, &wn};
+    void* rargs[] = {&n_partials, &ix.wpartial, &W_grad, &wn};
     return k->launch(OEQ_ROLE_TP_BACKWARD_WREDUCE, wn, rargs, stream);
 }
 
@@ -631,17 +706,17 @@ int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, co
         !cols)
         return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL buffer");
     WalkIndex ix;
-    int rc = walk_index(k, "oeq_conv_double_backward", node_count, nnz, rows, cols, transpose_perm, workspace,
-                        workspace_bytes, stream, &ix);
+    int rc = walk_index(k, "oeq_conv_double_backward", walk_layout(k, node_count, nnz, true, false, false), node_count,
+                        nnz, rows, cols, transpose_perm, workspace, workspace_bytes, stream, &ix);
     if (rc) return rc;
     void* a[] = {&node_count, &nnz, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_dgrad,
-                 &rows,       &cols, &ix.rowptr, &ix.rperm};
+                 &rows,       &cols, &ix.rowptr, &ix.rperm, &ix.order};
     if (k->roles[OEQ_ROLE_DOUBLE_BACKWARD_A].present) {
         rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_A, node_count, a, stream);
         if (rc) return rc;
     }
     void* b[] = {&node_count, &nnz,     &L1_in,  &L1_dgrad, &L2_in, &L2_dgrad,  &W,         &W_dgrad, &L3_grad,
-                 &L2_grad,    &W_grad,  &rows,   &cols,     &ix.rowptr, &ix.dx_tmp, &ix.rperm, &L3_dgrad};
+                 &L2_grad,    &W_grad,  &rows,   &cols,     &ix.rowptr, &ix.dx_tmp, &ix.rperm, &L3_dgrad, &ix.order};
     rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count, b, stream);
     if (rc) return rc;
     void* fargs[] = {&node_count, &nnz, &ix.dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};

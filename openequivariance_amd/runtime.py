@@ -49,8 +49,11 @@ ROLE_GROUP_SCATTER = 11
 ROLE_GROUP_ORDER = 12
 ROLE_DOUBLE_BACKWARD_A = 13
 ROLE_DOUBLE_BACKWARD_B = 14
+ROLE_ORDER_HOP = 15
 
 CONV_ATOMIC, CONV_SORTED, CONV_GROUPED = 0, 1, 2
+DX_TERMS, DX_ATOMIC, DX_ARRIVAL = 0, 1, 2
+ABI_VERSION = 2
 
 
 class OeqError(RuntimeError):
@@ -92,6 +95,9 @@ class _ProblemDims(ctypes.Structure):
         ("shared_weights", ctypes.c_int32),
         ("deterministic", ctypes.c_int32),
         ("wpartial_per_block", ctypes.c_int32),
+        ("dx_mode", ctypes.c_int32),
+        ("n_chunks", ctypes.c_int32),
+        ("order_hops", ctypes.c_int32),
     ]
 
 
@@ -131,6 +137,7 @@ EXPORTS = {
     "oeq_conv_forward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_backward": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_conv_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_conv_double_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_has_double_backward": (ctypes.c_int, [_P]),
     "oeq_tp_double_backward": (ctypes.c_int, [_P, _I64] + [_P] * 12),
     "oeq_conv_double_backward": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 15 + [_SZ, _P]),
@@ -150,15 +157,31 @@ def lib_path() -> Path:
     return _LIB_PATH
 
 
+def _stale() -> bool:
+    """The built library is older than the sources it is made from."""
+    built = _LIB_PATH.stat().st_mtime
+    return any(src.exists() and src.stat().st_mtime > built for src in (_SRC_PATH, _INCLUDE_DIR / "oeq_amd.h"))
+
+
 def load_library():
-    """Load liboeq_amd.so (building it first only if no built file exists)."""
+    """Load liboeq_amd.so. It is built first when no built file exists or the file is older than its
+    sources; a library whose ABI version is not the one this module binds is refused (kernel argument
+    lists are positional, so a mismatch would mean wrong pointers on the GPU rather than an error)."""
     global _lib
     with _lib_lock:
         if _lib is not None:
             return _lib
-        if not _LIB_PATH.exists():
+        if not _LIB_PATH.exists() or _stale():
             build_library()
         lib = ctypes.CDLL(str(_LIB_PATH))
+        try:
+            lib.oeq_abi_version.restype = ctypes.c_int
+            found = lib.oeq_abi_version()
+        except AttributeError:
+            found = None
+        if found != ABI_VERSION:
+            raise OeqError(f"{_LIB_PATH} has ABI version {found}, this package needs {ABI_VERSION}: "
+                           "rebuild it (python -c 'import __graft_entry__ as g; g.build()' at the repository root)")
         for name, (res, args) in EXPORTS.items():
             fn = getattr(lib, name)
             fn.restype = res
@@ -292,6 +315,9 @@ class KernelSet:
 
     def conv_backward_workspace_bytes(self, nodes, nnz) -> int:
         return self._lib.oeq_conv_backward_workspace_bytes(self.handle, nodes, nnz)
+
+    def conv_double_backward_workspace_bytes(self, nodes, nnz) -> int:
+        return self._lib.oeq_conv_double_backward_workspace_bytes(self.handle, nodes, nnz)
 
     def conv_forward(self, nodes, nnz, x, y, w, out, rows, cols, ws, ws_bytes, stream):
         _check(self._lib.oeq_conv_forward(self.handle, nodes, nnz, x, y, w, out, rows, cols, ws, ws_bytes, stream),

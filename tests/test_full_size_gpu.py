@@ -116,13 +116,14 @@ def test_cfg5_full_graph():
                              G[tr[te]].cpu().numpy())
     assert err(dx[s], gx.sum(0)) <= 1e-5
     # deterministic=False: on the sorted list the device-side grouping reproduces the caller's order (same
-    # bits); on shuffled edges it agrees to tolerance and is itself reproducible
+    # bits for the output and the per-edge gradients; the sender gradient is accumulated with float atomics
+    # and agrees to tolerance); on shuffled edges it agrees to tolerance and the forward is reproducible
     perm = torch.randperm(E, device="cuda", generator=gen)
     at = oeq.TensorProductConv(problem, deterministic=False)
     dummy = torch.zeros(1, dtype=torch.int64, device="cuda")
     assert torch.equal(ops.conv_forward(X, Y, W, tr, tc, dummy, at.kid), z)
     dxs, dys, dws = ops.conv_backward(X, Y, W, G, tr, tc, dummy, at.kid)
-    assert torch.equal(dxs, dx) and torch.equal(dys, dy) and torch.equal(dws, dw)
+    assert _rel(dxs, dx) <= 1e-5 and torch.equal(dys, dy) and torch.equal(dws, dw)
     del dxs, dys, dws
     Yp, Wp, rp, cp = Y[perm].contiguous(), W[perm].contiguous(), tr[perm].contiguous(), tc[perm].contiguous()
     za = ops.conv_forward(X, Yp, Wp, rp, cp, dummy, at.kid)

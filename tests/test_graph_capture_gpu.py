@@ -14,7 +14,8 @@ from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
 pytestmark = pytest.mark.gpu
 
 
-def _replay_and_compare(eager_fn, static_inputs, make_new_values):
+def _replay_and_compare(eager_fn, static_inputs, make_new_values, tol=0.0):
+    """``tol`` > 0: outputs that depend on float atomics are compared by max normalised error."""
     # warm-up on a side stream (compiles and loads the kernels, primes the allocator)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -36,7 +37,10 @@ def _replay_and_compare(eager_fn, static_inputs, make_new_values):
         graph.replay()
         torch.cuda.synchronize()
         for got, want in zip(captured, expected):
-            assert torch.equal(got, want), seed
+            if tol:
+                assert torch.isfinite(got).all() and (got - want).abs().max() <= tol * want.abs().max(), seed
+            else:
+                assert torch.equal(got, want), seed
         (static_inputs[0] * 2).sum().item()  # unrelated eager work between replays
 
 
@@ -91,4 +95,5 @@ def test_convolution_in_a_graph(deterministic):
         gen2 = torch.Generator(device="cuda").manual_seed(200 + seed)
         return [torch.randn(t.shape, device="cuda", generator=gen2) for t in (X, Y, W, G)]
 
-    _replay_and_compare(step, [X, Y, W, G], new_values)
+    # deterministic=False accumulates the sender gradient with float atomics (and what is derived from it here)
+    _replay_and_compare(step, [X, Y, W, G], new_values, tol=0.0 if deterministic else 2e-5)

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/oeq_amd.h but not exported"
     assert set(names) == set(rt.EXPORTS), "ctypes table and header disagree"
-    assert lib.oeq_abi_version() == 1
+    assert lib.oeq_abi_version() == rt.ABI_VERSION
 
 
 def test_compile_error_is_reported_not_fatal():
@@ -85,7 +85,8 @@ def test_generated_conv_sources_compile_for_gfx950(make, det):
     blob = rt.compile_source(src)
     names = {d[1] for d in descs}
     assert {"forward", "backward", "fixup_backward"} <= names
-    assert ({"oeq_group_count", "oeq_group_scan", "oeq_group_scatter", "oeq_group_order"} <= names) == (not det)
+    # the counting-sort kernels serve the edge grouping (deterministic=False) and, in both modes, the walk order
+    assert {"oeq_group_count", "oeq_group_scan", "oeq_group_scatter", "oeq_group_order", "oeq_order_hop"} <= names
     assert dims["deterministic"] == (rt.CONV_SORTED if det else rt.CONV_GROUPED)
     # generated code must not carry packed-FP32 arithmetic or anything CUDA-flavoured
     assert "__syncwarp" not in src and "cuda" not in src.lower()
