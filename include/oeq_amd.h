@@ -180,6 +180,23 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz,
                      void* workspace, size_t workspace_bytes, void* stream);
 size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
 
+/* oeq_conv_forward for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc. It has no counterpart in the reference (whose convolution always takes a
+ * caller-allocated workspace tensor). Same operands and result as oeq_conv_forward; the index scratch
+ * (CSR pointers, edge grouping, walk order) lives in a device array inside the library instead of a
+ * caller workspace, and the call itself allocates nothing (no hipMalloc / hipFree, no event or module
+ * creation): the kernel set must already be loaded on the current device, i.e. oeq_conv_forward has run on
+ * it once. Limits: the scratch needed, oeq_conv_forward_workspace_bytes(), must not exceed
+ * oeq_static_scratch_bytes() (32 MiB: e.g. 1.9 M edges over 50 000 nodes with deterministic=False, 4 M
+ * nodes in deterministic mode); larger calls are refused with OEQ_ERR_INVALID. Every call on a GPU uses
+ * that GPU's one array: calls that overlap in time on one GPU (two streams, two threads) race and must be
+ * serialised by the caller. Per-kernel timing (oeq_kernel_timing_enable) is not applied to these calls. */
+int oeq_conv_forward_static(oeq_kernels* k, int64_t node_count, int64_t nnz,
+                            const void* L1_in, const void* L2_in, const void* W,
+                            void* L3_out, const int64_t* rows, const int64_t* cols,
+                            void* stream);
+size_t oeq_static_scratch_bytes(void);
+
 /* Replaces JITConvImpl::backward (extension/convolution.hpp:109-136) as called
  * by jit_conv_backward (extension/torch_core.hpp:478-542). Deterministic mode
  * additionally needs transpose_perm [nnz]: the permutation listing the

@@ -1,8 +1,9 @@
 // liboeq_amd.so: host runtime behind the C ABI declared in include/oeq_amd.h.
 //
-// Host-only translation unit: compiles HIP source with hiprtc, loads the code
-// object once per device, and enqueues the generated kernels on the caller's
-// stream. The kernel argument lists used here are the contract the Python
+// Compiles HIP source with hiprtc, loads the code object once per device, and
+// enqueues the generated kernels on the caller's stream. The only device-side
+// object of this translation unit is the scratch array of the allocation-free
+// entry point (oeq_conv_forward_static). The kernel argument lists used here are the contract the Python
 // code generator (openequivariance_amd/codegen) emits against.
 #include "oeq_amd.h"
 
@@ -118,12 +119,23 @@ struct oeq_kernels {
         return (unsigned)blocks;
     }
 
+    // Set by the allocation-free entry point for the duration of its call (on its thread): launches then
+    // create no timing events.
+    static thread_local bool no_events;
+
+    bool loaded_on_current_device() {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
+        std::lock_guard<std::mutex> lock(mu);
+        return slots[dev].module != nullptr;
+    }
+
     int launch(int role, int64_t units, void** args, void* stream) {
         const std::vector<hipFunction_t>* fns = nullptr;
         int rc = functions(role, &fns);
         if (rc) return rc;
         unsigned grid = grid_for(role, units);
-        if (!timing.load(std::memory_order_relaxed)) {
+        if (no_events || !timing.load(std::memory_order_relaxed)) {
             for (hipFunction_t fn : *fns)
                 HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, roles[role].block, 1, 1, 0, (hipStream_t)stream, args,
                                               nullptr));
@@ -194,6 +206,38 @@ struct oeq_kernels {
         return launch(OEQ_ROLE_GROUP_ORDER, n_segments, oargs, stream);
     }
 };
+
+thread_local bool oeq_kernels::no_events = false;
+
+// ---------------------------------------------------------------------------
+// scratch memory of the allocation-free entry point
+// ---------------------------------------------------------------------------
+
+// One copy per GPU, held until the process ends. In host code the array's name is only a handle for
+// hipGetSymbolAddress: the address kernels and fills work on is resolved once per device (with that device
+// current) and kept in g_scratch_ptr.
+#define OEQ_STATIC_SCRATCH_BYTES (32u << 20)
+static __device__ __align__(256) unsigned char scratch[OEQ_STATIC_SCRATCH_BYTES];
+
+namespace {
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mu;
+
+int static_scratch(void** out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(OEQ_ERR_INVALID, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(OEQ_ERR_HIP, "hipGetSymbolAddress returned a NULL address for the scratch array");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return OEQ_OK;
+}
+}  // namespace
 
 extern "C" {
 
@@ -600,6 +644,32 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void
     }
     void* args[] = {&node_count, &nnz, &L1_in, &L2_in, &W, &L3_out, &rows, &cols, &ix.rowptr, &ix.rperm, &ix.order};
     return k->launch(OEQ_ROLE_CONV_FORWARD, mode != OEQ_CONV_ATOMIC ? node_count : nnz, args, stream);
+}
+
+size_t oeq_static_scratch_bytes(void) { return OEQ_STATIC_SCRATCH_BYTES; }
+
+int oeq_conv_forward_static(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
+                            const void* W, void* L3_out, const int64_t* rows, const int64_t* cols, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_forward_static: NULL kernel set");
+    if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_forward_static: negative size");
+    const size_t need = oeq_conv_forward_workspace_bytes(k, node_count, nnz);
+    if (need > OEQ_STATIC_SCRATCH_BYTES)
+        return fail(OEQ_ERR_INVALID,
+                    "oeq_conv_forward_static: %lld nodes and %lld edges need %zu bytes of index scratch, the static "
+                    "buffer holds %u; use oeq_conv_forward with a caller-provided workspace",
+                    (long long)node_count, (long long)nnz, need, (unsigned)OEQ_STATIC_SCRATCH_BYTES);
+    // loading a code object allocates device memory: that has to have happened before
+    if (!k->loaded_on_current_device())
+        return fail(OEQ_ERR_INVALID,
+                    "oeq_conv_forward_static: the kernels are not loaded on this device yet; run oeq_conv_forward "
+                    "once on it first");
+    void* ws = nullptr;
+    int rc = static_scratch(&ws);
+    if (rc) return rc;
+    oeq_kernels::no_events = true;
+    rc = oeq_conv_forward(k, node_count, nnz, L1_in, L2_in, W, L3_out, rows, cols, ws, OEQ_STATIC_SCRATCH_BYTES, stream);
+    oeq_kernels::no_events = false;
+    return rc;
 }
 
 int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, void* L1_grad,

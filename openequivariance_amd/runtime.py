@@ -103,8 +103,11 @@ class _ProblemDims(ctypes.Structure):
 
 def build_library(verbose: bool = False) -> Path:
     """Compile csrc/oeq_amd.cpp into liboeq_amd.so next to this file."""
+    # the library carries one device-side object (the scratch array of oeq_conv_forward_static), so it is
+    # compiled for the target architecture, with the device flags every kernel here is compiled with
     cmd = [
-        "hipcc", "-O2", "-std=c++17", "-shared", "-fPIC", f"-I{_INCLUDE_DIR}",
+        "hipcc", "-O2", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={DEFAULT_ARCH}",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", f"-I{_INCLUDE_DIR}",
         str(_SRC_PATH), "-o", str(_LIB_PATH), "-lhiprtc",
     ]
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -135,6 +138,8 @@ EXPORTS = {
     "oeq_tp_backward_workspace_bytes": (_SZ, [_P, _I64]),
     "oeq_conv_forward": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_conv_forward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_conv_forward_static": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]),
+    "oeq_static_scratch_bytes": (_SZ, []),
     "oeq_conv_backward": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_conv_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_double_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
@@ -322,6 +327,11 @@ class KernelSet:
     def conv_forward(self, nodes, nnz, x, y, w, out, rows, cols, ws, ws_bytes, stream):
         _check(self._lib.oeq_conv_forward(self.handle, nodes, nnz, x, y, w, out, rows, cols, ws, ws_bytes, stream),
                "oeq_conv_forward")
+
+    def conv_forward_static(self, nodes, nnz, x, y, w, out, rows, cols, stream):
+        """oeq_conv_forward with the library's static scratch array instead of a workspace; allocates nothing."""
+        _check(self._lib.oeq_conv_forward_static(self.handle, nodes, nnz, x, y, w, out, rows, cols, stream),
+               "oeq_conv_forward_static")
 
     def has_double_backward(self) -> bool:
         return bool(self._lib.oeq_has_double_backward(self.handle))
