@@ -95,8 +95,7 @@ def test_conv_matches_oracle(name, make, n_nodes, deg):
         z.backward(torch.tensor(G, device="cuda"))
         assert err(tX.grad, dx_ref) <= tol, (name, det)
         assert err(tY.grad, dy_ref[order]) <= tol, (name, det)
-        wtol = tol * (np.sqrt(E) if problem.shared_weights else 1.0)
-        assert err(tW.grad, dw_ref if problem.shared_weights else dw_ref[order]) <= wtol, (name, det)
+        assert err(tW.grad, dw_ref if problem.shared_weights else dw_ref[order]) <= tol, (name, det)
 
 
 def test_reference_toy_graph():

@@ -238,3 +238,77 @@ def test_force_training_pattern(which, monkeypatch):
         loss = sum((t ** 2).sum() for t in first)
         results.append([t.detach() for t in torch.autograd.grad(loss, ts)])
     _check(("x", "y", "w"), results[0], results[1], 1e-5)
+
+
+# ---------------------------------------------------------------------------
+# the fused kernels directly against float64 autograd through the CPU restatement
+# ---------------------------------------------------------------------------
+
+def _oracle_second_order(fn, x, y, w, g, a, b, c):
+    """Gradients of <a, dx> + <b, dy> + <c, dw> with respect to (x, y, w, g), where (dx, dy, dw) is the
+    backward of z = fn(x, y, w) for the output gradient g; float64 autograd on the host."""
+    t = [torch.tensor(v.double().cpu().numpy(), requires_grad=True) for v in (x, y, w, g)]
+    cot = [torch.tensor(v.double().cpu().numpy()) for v in (a, b, c)]
+    z = fn(*t[:3])
+    first = torch.autograd.grad(z, t[:3], t[3], create_graph=True)
+    s = sum((p * q).sum() for p, q in zip(cot, first))
+    return [v.numpy() for v in torch.autograd.grad(s, t)]
+
+
+ORACLE_TP = [("cfg1", P.config1_single_uvu, 64), ("cfg2", P.config2_nequip_uvu, 33), ("cfg3", P.config3_mace_uvu, 9),
+             ("cfg3-f64", lambda: _f64(P.config3_mace_uvu()), 5), ("folded-gaps", _folded, 17), ("odd", _odd, 40)]
+
+
+@pytest.mark.parametrize("name,make,batch", ORACLE_TP, ids=[c[0] for c in ORACLE_TP])
+def test_tp_fused_matches_float64_autograd(name, make, batch):
+    from oracle.torch_ref import TorchTP
+    problem = make()
+    tp = oeq.TensorProduct(problem)
+    e = ops.get_entry(tp.kid)
+    assert e.kernels().has_double_backward()
+    dt = np.dtype(problem.irrep_dtype)
+    rng = np.random.default_rng(15)
+    x, a = (_rand(rng, (batch, e.L1), dt) for _ in range(2))
+    y, b = (_rand(rng, (batch, e.L2), dt) for _ in range(2))
+    w, c = (_rand(rng, (batch, e.WN), dt) for _ in range(2))
+    g = _rand(rng, (batch, e.L3), dt)
+    fused = ops.tp_double_backward(x, y, w, g, a, b, c, tp.kid)
+    want = _oracle_second_order(TorchTP(R.Problem.from_spec(problem), torch.float64), x, y, w, g, a, b, c)
+    for nm, got, ref in zip(("dx", "dy", "dw", "gg"), fused, want):
+        err = R.normalized_error(got.cpu().numpy(), ref)
+        assert err <= tol_of(problem), (nm, err)
+
+
+ORACLE_CONV = [("cfg2", P.config2_nequip_uvu), ("cfg5", P.config5_mace_conv),
+               ("cfg5-f64", lambda: _f64(P.config5_mace_conv())), ("folded-gaps", _folded), ("odd", _odd)]
+
+
+@pytest.mark.parametrize("det", [True, False], ids=["sorted", "grouped"])
+@pytest.mark.parametrize("name,make", ORACLE_CONV, ids=[c[0] for c in ORACLE_CONV])
+def test_conv_fused_matches_float64_autograd(name, make, det):
+    from oracle.torch_ref import TorchConv
+    problem = make()
+    gph = _graph(24)
+    n, E = gph.coords.shape[0], gph.nnz
+    conv = oeq.TensorProductConv(problem, deterministic=det)
+    e = ops.get_entry(conv.kid)
+    assert e.kernels().has_double_backward()
+    dt = np.dtype(problem.irrep_dtype)
+    rng = np.random.default_rng(16)
+    if det:
+        rows, cols, perm = gph.rows, gph.cols, gph.transpose_perm
+    else:
+        order = rng.permutation(E)
+        rows, cols, perm = gph.rows[order], gph.cols[order], np.zeros(0, np.int64)
+    tr, tc, tp = (torch.tensor(v, device="cuda") for v in (rows, cols, perm))
+    x, a = (_rand(rng, (n, e.L1), dt) for _ in range(2))
+    y, b = (_rand(rng, (E, e.L2), dt) for _ in range(2))
+    w, c = (_rand(rng, (E, e.WN), dt) for _ in range(2))
+    g = _rand(rng, (n, e.L3), dt)
+    fused = ops.conv_double_backward(x, y, w, g, a, b, c, tr, tc, tp, conv.kid)
+    oracle = TorchConv(R.Problem.from_spec(problem), torch.float64)
+    want = _oracle_second_order(lambda p, q, r: oracle(p, q, r, torch.tensor(rows), torch.tensor(cols)),
+                                x, y, w, g, a, b, c)
+    for nm, got, ref in zip(("dx", "dy", "dw", "gg"), fused, want):
+        err = R.normalized_error(got.cpu().numpy(), ref)
+        assert err <= tol_of(problem), (nm, err)

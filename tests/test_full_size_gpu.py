@@ -42,6 +42,60 @@ def test_cfg2_full_batch():
     assert torch.isfinite(z).all() and torch.isfinite(x.grad).all()
 
 
+def test_cfg1_full_batch():
+    """Config 1 at its scaled-up size: 100 000 rows, uniform[0,1) inputs from seed 0, every row against the
+    oracle (the problem is small enough for that)."""
+    problem = P.config1_single_uvu()
+    B = 100000
+    rng = np.random.default_rng(0)
+    x, y, w, g = (rng.uniform(size=(B, d)).astype(np.float32) for d in (5, 7, 1, 5))
+    tx, ty, tw = (torch.tensor(a, device="cuda", requires_grad=True) for a in (x, y, w))
+    tp = oeq.TensorProduct(problem)
+    z = tp(tx, ty, tw)
+    z.backward(torch.tensor(g, device="cuda"))
+    ref = R.Problem.from_spec(problem)
+    assert err(z, R.tp_forward(ref, x, y, w)) <= 1e-5
+    for got, want in zip((tx.grad, ty.grad, tw.grad), R.tp_backward(ref, x, y, w, g)):
+        assert err(got, want) <= 1e-5
+    assert torch.equal(tp(2.0 * tx, ty, 0.25 * tw), 0.5 * z)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_cfg3_full_batch(dtype):
+    """Config 3 at its full size, 500 000 rows, in both precisions: a sample of rows (first, last, both sides
+    of the boundaries between the blocks of a grid-sized sweep) against the oracle, exact scaling by powers of
+    two, linearity in the output gradient, same bits on a second run."""
+    problem = P.config3_mace_uvu(dtype)
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    B = 500000
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(B, 2048, device="cuda", generator=gen, dtype=tdt)
+    v = torch.randn(B, 3, device="cuda", generator=gen, dtype=torch.float64)
+    y = torch.tensor(spherical_harmonics(3, v.cpu().numpy()).astype(dtype), device="cuda")
+    w = torch.randn(B, 2944, device="cuda", generator=gen, dtype=tdt)
+    g = torch.randn(B, 12672, device="cuda", generator=gen, dtype=tdt)
+    tp = oeq.TensorProduct(problem)
+    ops = torch.ops.oeq_amd
+    z = ops.tp_forward(x, y, w, tp.kid)
+    idx = torch.tensor([0, 1, 2, 2047, 2048, 2049, 250000, 499998, B - 1], device="cuda")
+    ref = R.Problem.from_spec(problem)
+    xs, ys, ws, gs = (t[idx].cpu().numpy() for t in (x, y, w, g))
+    assert err(z[idx], R.tp_forward(ref, xs, ys, ws)) <= tol
+    assert torch.isfinite(z).all()
+    assert torch.equal(ops.tp_forward(4.0 * x, y, 0.5 * w, tp.kid), 2.0 * z)
+    del z
+    dx, dy, dw = ops.tp_backward(x, y, w, g, tp.kid)
+    rx, ry, rw = R.tp_backward(ref, xs, ys, ws, gs)
+    assert err(dx[idx], rx) <= tol and err(dy[idx], ry) <= tol and err(dw[idx], rw) <= tol
+    dx2, dy2, dw2 = ops.tp_backward(x, y, w, g, tp.kid)
+    assert torch.equal(dx, dx2) and torch.equal(dy, dy2) and torch.equal(dw, dw2)
+    del dx2, dy2, dw2
+    # linear in the output gradient (a power of two scales exactly)
+    sx, sy, sw = ops.tp_backward(x, y, w, 2.0 * g, tp.kid)
+    assert torch.equal(sx, 2.0 * dx) and torch.equal(sy, 2.0 * dy) and torch.equal(sw, 2.0 * dw)
+
+
 def test_cfg4_full_batch_mfma():
     problem = P.config4_uvw_shared()
     B = 262144

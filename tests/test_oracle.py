@@ -274,3 +274,46 @@ def test_sorted_graph_matches_coordgraph():
     # both directions present, no self loops, minimum-image vectors within the cutoff
     assert set(zip(rows.tolist(), cols.tolist())) == set(zip(cols.tolist(), rows.tolist()))
     assert np.all(rows != cols) and np.all(np.linalg.norm(vec, axis=1) < 5.0)
+
+
+# ------------------------------------------------------------ torch restatement (second-order checker, CPU baseline)
+
+@pytest.mark.parametrize("case", TINY)
+def test_torch_restatement_matches_numpy_oracle(case):
+    """oracle/torch_ref.py is the checker of every second/third-derivative test and what bench.py times as
+    the CPU baseline: its forward equals the brute-force loops, its autograd gradients equal the hand-written
+    backward of the numpy oracle, for per-row and shared weights, 'uvu' and 'uvw'."""
+    import torch
+    from oracle.torch_ref import TorchTP
+
+    a, b, o, ins, shared = case
+    prob = R.Problem(a, b, o, ins, shared)
+    rng = np.random.default_rng(11)
+    x, y, w = _rand(prob, 4, rng)
+    g = rng.normal(size=(4, prob.dims[2]))
+    tx, ty, tw = (torch.tensor(v, dtype=torch.float64, requires_grad=True) for v in (x, y, w))
+    z = TorchTP(prob, torch.float64)(tx, ty, tw)
+    np.testing.assert_allclose(z.detach().numpy(), R.tp_forward_loops(prob, x, y, w), atol=1e-13)
+    z.backward(torch.tensor(g))
+    for got, want in zip((tx.grad, ty.grad, tw.grad), R.tp_backward(prob, x, y, w, g)):
+        np.testing.assert_allclose(got.numpy(), want, atol=1e-12)
+
+
+@pytest.mark.parametrize("make", [P.config1_single_uvu, P.config2_nequip_uvu, P.config4_uvw_shared])
+def test_torch_restatement_conv_matches_numpy_oracle(make):
+    import torch
+    from oracle.torch_ref import TorchConv
+
+    prob = R.Problem.from_spec(make())
+    rng = np.random.default_rng(12)
+    n, E = 7, 19
+    rows, cols = rng.integers(0, n, size=E), rng.integers(0, n, size=E)
+    X, Y = rng.normal(size=(n, prob.dims[0])), rng.normal(size=(E, prob.dims[1]))
+    W = rng.normal(size=(prob.weight_numel,) if prob.shared_weights else (E, prob.weight_numel))
+    G = rng.normal(size=(n, prob.dims[2]))
+    tX, tY, tW = (torch.tensor(v, dtype=torch.float64, requires_grad=True) for v in (X, Y, W))
+    Z = TorchConv(prob, torch.float64)(tX, tY, tW, torch.tensor(rows), torch.tensor(cols))
+    np.testing.assert_allclose(Z.detach().numpy(), R.conv_forward(prob, X, Y, W, rows, cols), atol=1e-12)
+    Z.backward(torch.tensor(G))
+    for got, want in zip((tX.grad, tY.grad, tW.grad), R.conv_backward(prob, X, Y, W, G, rows, cols)):
+        np.testing.assert_allclose(got.numpy(), want, atol=1e-11)

@@ -118,9 +118,9 @@ def test_forward_backward_match_oracle(name, make, B):
     z.backward(tg)
     assert err(tx.grad, dx_ref) <= tol
     assert err(ty.grad, dy_ref) <= tol
-    # a shared weight gradient sums `B` terms: allow the accumulated rounding of that sum
-    wtol = tol * (max(1.0, np.sqrt(B)) if problem.shared_weights else 1.0)
-    assert err(tw.grad, dw_ref) <= wtol
+    # a shared weight gradient sums `B` same-sign terms (the inputs are uniform[0,1)); it still has to meet
+    # the tolerance of every other result
+    assert err(tw.grad, dw_ref) <= tol
 
 
 def test_same_precision_reference_is_not_closer_by_accident():
