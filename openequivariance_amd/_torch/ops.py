@@ -264,6 +264,42 @@ tp_backward.register_autograd(_tp_bwd_backward, setup_context=_tp_bwd_setup)
 # ---------------------------------------------------------------------------
 
 
+# Edge-list validation before any kernel is launched: ``CHECK_INDICES = True`` here, or
+# OEQ_AMD_CHECK_INDICES=1 in the environment. Off by default, like in the reference (which checks
+# shapes, dtypes and devices only, torch_core.hpp:109-134): the check synchronises with the device.
+# Without it a corrupt edge list cannot make the kernels read or write outside their operands (every
+# index is forced into range on the device), but the sums it gives are then meaningless.
+CHECK_INDICES = False
+
+
+def check_edge_list(nodes: int, rows: torch.Tensor, cols: torch.Tensor, perm: Optional[torch.Tensor],
+                    deterministic: bool):
+    """RuntimeError unless 0 <= rows, cols < nodes and, for the caller-sorted mode, rows is non-decreasing
+    and perm is a permutation of the edges that lists them by non-decreasing sender."""
+    nnz = rows.shape[0]
+    if nnz == 0:
+        return
+    for name, t in (("rows", rows), ("cols", cols)):
+        lo, hi = int(t.min()), int(t.max())
+        if lo < 0 or hi >= nodes:
+            raise RuntimeError(f"Index out of range in tensor '{name}': values span [{lo}, {hi}], "
+                               f"the graph has {nodes} nodes")
+    if deterministic:
+        if nnz > 1 and bool((rows[1:] < rows[:-1]).any()):
+            raise RuntimeError("Tensor 'rows' is not sorted: deterministic=True needs the edges sorted by receiver")
+        lo, hi = int(perm.min()), int(perm.max())
+        if lo < 0 or hi >= nnz or int(torch.bincount(perm, minlength=nnz).max()) != 1:
+            raise RuntimeError("Tensor 'transpose perm' is not a permutation of the edges")
+        by_sender = cols[perm]
+        if nnz > 1 and bool((by_sender[1:] < by_sender[:-1]).any()):
+            raise RuntimeError("Tensor 'transpose perm' does not list the edges by sender")
+
+
+def _check_indices_enabled() -> bool:
+    import os
+    return CHECK_INDICES or os.environ.get("OEQ_AMD_CHECK_INDICES", "0") not in ("", "0")
+
+
 def _conv_checks(e: KernelEntry, L1_in, L2_in, W, rows, cols, perm, L3_grad=None):
     nodes = L1_in.shape[0] if L1_in.dim() > 0 else -1
     nnz = rows.shape[0] if rows.dim() > 0 else -1
@@ -276,6 +312,10 @@ def _conv_checks(e: KernelEntry, L1_in, L2_in, W, rows, cols, perm, L3_grad=None
     check_tensor(cols, [nnz], torch.int64, "cols")
     if e.deterministic:
         check_tensor(perm, [nnz], torch.int64, "transpose perm")
+    if _check_indices_enabled():
+        check_edge_list(nodes, rows, cols, perm if e.deterministic else None, bool(e.deterministic))
+    if e.deterministic:
+        pass
     elif (torch.are_deterministic_algorithms_enabled() and not e.unfused
           and (e.kernels().dims["deterministic"] == rt.CONV_ATOMIC
                or (L3_grad is not None and e.kernels().dims.get("dx_mode", 0) == rt.DX_ATOMIC))):

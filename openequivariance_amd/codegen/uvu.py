@@ -198,7 +198,7 @@ class UvuEmitter:
         low, st = self.low, self.stage
         s.open("")
         s(f"const i64 eid = OEQ_EDGE({e});")
-        s(f"const T* sx = L1_in + cols[eid] * {low.L1};")
+        s(f"const T* sx = L1_in + oeq_idx(cols[eid], node_count) * {low.L1};")
         s(f"const T* sw = W + eid * {low.WN};")
         for q in range(st["nqx"]):
             s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sx + xoff{q}), (OEQ_LPTR)(&s_stage[wave][{q * 256}]), 16, 0, 0);")
@@ -275,7 +275,7 @@ class UvuEmitter:
         low, st = self.low, self.stage3
         s.open("")
         s(f"const i64 eid = OEQ_EDGE({e});")
-        s(f"const T* sx = L1_in + cols[eid] * {low.L1};")
+        s(f"const T* sx = L1_in + oeq_idx(cols[eid], node_count) * {low.L1};")
         s(f"const T* sw = W + eid * {low.WN};")
         s(f"const T* sy = L2_in + eid * {low.L2};")
         for q in range(st["nqx"]):
@@ -610,9 +610,10 @@ class UvuEmitter:
         s.open(
             f"OEQ_DEV void {name}{self._sfx()}(E_t& d, const i64 e, const T* __restrict__ L1_in, "
             "const T* __restrict__ L2_in, "
-            f"const T* __restrict__ W, const i64* __restrict__ cols, const int u{', const Q_t& qt' if self.use_q else ''})"
+f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, const int u"
+            f"{', const Q_t& qt' if self.use_q else ''})"
         )
-        s("const i64 c = cols[e];")
+        s("const i64 c = oeq_idx(cols[e], node_count);")
         s(f"const T* xrow = L1_in + c * {low.L1};")
         s(f"const T* yrow = L2_in + e * {low.L2};")
         s(f"const T* wrow = W{'' if low.shared_weights else f' + e * {low.WN}'};")
@@ -1003,7 +1004,7 @@ class UvuEmitter:
         def make_load(si):
             def load(buf, e):
                 if self.can_preload:
-                    s(f"load_edge_f{si}{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u{self._qarg()});")
+                    s(f"load_edge_f{si}{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, node_count, u{self._qarg()});")
             return load
 
         kahan = self.kahan and deterministic
@@ -1026,7 +1027,7 @@ class UvuEmitter:
             else:
                 s.open("")
                 s(f"const i64 eid = OEQ_EDGE({e});")
-                s(f"const T* xrow = L1_in + cols[eid] * {low.L1};")
+                s(f"const T* xrow = L1_in + oeq_idx(cols[eid], node_count) * {low.L1};")
                 s(f"const T* yrow = L2_in + eid * {low.L2};")
                 s(f"const T* wrow = W{'' if low.shared_weights else f' + eid * {low.WN}'};")
                 s("X_t x;")
@@ -1036,7 +1037,7 @@ class UvuEmitter:
 
         if deterministic:
             self._node_loop_open(s, G, xcd)
-            s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+            s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
             s(f"T* zrow = L3_out + node * {low.L3};")
             for si in range(len(self.segments)):
                 s.open(f"if (sg == {si % segw})" if segw > 1 else "")
@@ -1075,7 +1076,7 @@ class UvuEmitter:
 
                 def before_edge(e, si=si):
                     s.open("")
-                    s(f"const i64 row = rows[OEQ_EDGE({e})];")
+                    s(f"const i64 row = oeq_idx(rows[OEQ_EDGE({e})], node_count);")
                     s.open("if (row != cur)")
                     s.open("if (cur >= 0)")
                     s(f"T* zrow = L3_out + cur * {low.L3};")
@@ -1384,7 +1385,7 @@ class UvuEmitter:
         s("const i64 ea = eb + lane;")
         s("i64 sn = 0; bool last = false;")
         s.open("if (ea < e1)")
-        s("sn = cols[OEQ_EDGE(ea)];")
+        s("sn = oeq_idx(cols[OEQ_EDGE(ea)], node_count);")
         s(f"const int seen = __hip_atomic_fetch_add(arrivals + sn * {self.NCH} + chunk, 1, __ATOMIC_RELAXED, "
           "__HIP_MEMORY_SCOPE_AGENT) + 1;")
         s("last = seen == (int)(colptr[sn + 1] - colptr[sn]);")
@@ -1398,11 +1399,11 @@ class UvuEmitter:
         s("__threadfence();")  # acquire: the other waves' terms after their arrivals
         s("X_t tot;")
         self._zero_x(s, "tot")
-        s("const i64 j0 = colptr[snd], j1 = colptr[snd + 1];")
+        s("const i64 j0 = oeq_pos(colptr[snd], nnz), j1 = oeq_pos(colptr[snd + 1], nnz);")
         # the additions stay in list order; unrolling only lets several rows be in flight at a time
         s("#pragma unroll 4")
         s.open("for (i64 j = j0; j < j1; ++j)")
-        s(f"const T* trow = dx_tmp + sperm[j] * {low.L1};")
+        s(f"const T* trow = dx_tmp + oeq_idx(sperm[j], nnz) * {low.L1};")
         s("X_t t;")
         self._load_terms(s, "trow", "t")
         for b in self._in1_of(self.used_in1):
@@ -1608,7 +1609,7 @@ class UvuEmitter:
         s(f"__shared__ T s_dx[{SW}][{self.NCH}][{XW}][64];")
         s("E_t A;")
         self._node_loop_open(s, 1, xcd)
-        s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+        s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
         for si in range(SW):
             s.open(f"if (sg == {si})")
 
@@ -1618,7 +1619,7 @@ class UvuEmitter:
                 # every wave of the block runs the same number of edges, so the block barriers match up
                 s.open("for (i64 e = e0; e < e1; ++e)")
                 s("const i64 eid = OEQ_EDGE(e);")
-                s(f"load_edge_b{si}{self._sfx()}(A, eid, L1_in, L2_in, W, cols, u{self._qarg()});")
+                s(f"load_edge_b{si}{self._sfx()}(A, eid, L1_in, L2_in, W, cols, node_count, u{self._qarg()});")
                 yacc, wacc = self._acc_preloaded("A")
                 if self.use_q:
                     self._emit_q_build(s, "A.yq")
@@ -1746,7 +1747,7 @@ class UvuEmitter:
 
         def load(buf, e):
             if self.can_preload:
-                s(f"load_edge_b{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, u{self._qarg()});")
+                s(f"load_edge_b{self._sfx()}({buf}, OEQ_EDGE({e}), L1_in, L2_in, W, cols, node_count, u{self._qarg()});")
 
         def make_compute(grow_expr_of):
             def compute(buf, pos):
@@ -1764,7 +1765,7 @@ class UvuEmitter:
                 else:
                     yacc, wacc = self._acc_pointer()
                     xname = "x"
-                    s(f"const T* xrow = L1_in + cols[{e}] * {low.L1};")
+                    s(f"const T* xrow = L1_in + oeq_idx(cols[{e}], node_count) * {low.L1};")
                     s(f"const T* yrow = L2_in + {e} * {low.L2};")
                     s(f"const T* wrow = W{'' if shared else f' + {e} * {low.WN}'};")
                     s("X_t x;")
@@ -1801,7 +1802,7 @@ class UvuEmitter:
                         self._store_dx(s, "dxrow", "true", nt=bool(self.nt & 2))
                         self._zero_untouched_in1(s, "dxrow", "true")
                 else:
-                    s(f"T* dxrow = L1_grad + cols[{e}] * {low.L1};")
+                    s(f"T* dxrow = L1_grad + oeq_idx(cols[{e}], node_count) * {low.L1};")
                     self._store_dx(s, "dxrow", "true", atomic=True)
                 self._dy_finish(s, f"L2_grad + {e} * {low.L2}", "true")
                 s.close()
@@ -1809,7 +1810,7 @@ class UvuEmitter:
 
         if deterministic:
             self._node_loop_open(s, G, xcd)
-            s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+            s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
 
             def node_body():
                 if resident:
@@ -1829,7 +1830,7 @@ class UvuEmitter:
             s("const i64 per = (nnz + ngrp - 1) / ngrp;")
             s(f"const i64 eb = ((i64)blockIdx.x * {G} + g) * per;")
             s("const i64 ee = (eb + per < nnz) ? eb + per : nnz;")
-            self._edge_loop(s, "eb + r", "ee", load, make_compute(lambda e: f"L3_grad + rows[{e}] * {low.L3}"),
+            self._edge_loop(s, "eb + r", "ee", load, make_compute(lambda e: f"L3_grad + oeq_idx(rows[{e}], node_count) * {low.L3}"),
                             mode)
         if shared and deterministic:
             # shared weights, walk kernels: every wave group writes the sum over its nodes as one partial

@@ -362,7 +362,7 @@ class DoubleEmitter(UvuEmitter):
     def _edge_rows(self, s: Src, e: str):
         low = self.low
         s(f"const i64 eid = OEQ_EDGE({e});")
-        s("const i64 sender = cols[eid];")
+        s("const i64 sender = oeq_idx(cols[eid], node_count);")
         s(f"const T* xrow = L1_in + sender * {low.L1};")
         s(f"const T* arow = L1_dgrad + sender * {low.L1};")
         s(f"const T* yrow = L2_in + eid * {low.L2};")
@@ -387,7 +387,7 @@ class DoubleEmitter(UvuEmitter):
         if self.tr_stores & 1 and self.R == 1:
             s(f"__shared__ T s_tr[{self.NCH * G * segw}][{64 * max(low.out[io].d for io in self.used_out)}];")
         self._node_loop_open(s, G, xcd)
-        s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+        s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
         s(f"T* zrow = L3_dgrad + node * {low.L3};")
         for si in range(len(self.segments)):
             s.open(f"if (sg == {si % segw})" if segw > 1 else "")
@@ -442,7 +442,7 @@ class DoubleEmitter(UvuEmitter):
             s(f"__shared__ T s_tr[{self.NCH * G}][{64 * dmax}];")
         resident = self.double_b_resident() or self.merged
         self._node_loop_open(s, G, xcd)
-        s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+        s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
 
         def node_body():
             if resident:
@@ -577,7 +577,7 @@ class DoubleEmitter(UvuEmitter):
         if self.merged and self.tr_stores & 1:
             s(f"__shared__ T s_tr[{self.NCH * SW}][{64 * max(low.out[io].d for io in self.used_out)}];")
         self._node_loop_open(s, 1, xcd)
-        s("const i64 e0 = rowptr[node], e1 = rowptr[node + 1];")
+        s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
         for si in range(SW):
             s.open(f"if (sg == {si})")
 

@@ -174,14 +174,14 @@ struct oeq_kernels {
                         int64_t* perm, void* stream) {
         int rc = fill_zero(ptr, (size_t)(n_segments + 1) * sizeof(int64_t), stream);
         if (rc) return rc;
-        void* cargs[] = {&n_items, &keys, &ptr};
+        void* cargs[] = {&n_items, &keys, &ptr, &n_segments};
         rc = launch(OEQ_ROLE_GROUP_COUNT, n_items, cargs, stream);
         if (rc) return rc;
         int64_t n = n_segments + 1;
         void* sargs[] = {&n, &ptr, &cursor};
         rc = launch(OEQ_ROLE_GROUP_SCAN, 1, sargs, stream);
         if (rc) return rc;
-        void* pargs[] = {&n_items, &keys, &cursor, &perm};
+        void* pargs[] = {&n_items, &keys, &cursor, &perm, &n_segments};
         return launch(OEQ_ROLE_GROUP_SCATTER, n_items, pargs, stream);
     }
 
@@ -192,14 +192,14 @@ struct oeq_kernels {
                      int64_t* unordered, int64_t* perm, void* stream) {
         int rc = fill_zero(ptr, (size_t)(n_segments + 1) * sizeof(int64_t), stream);
         if (rc) return rc;
-        void* cargs[] = {&n_items, &keys, &ptr};
+        void* cargs[] = {&n_items, &keys, &ptr, &n_segments};
         rc = launch(OEQ_ROLE_GROUP_COUNT, n_items, cargs, stream);
         if (rc) return rc;
         int64_t n = n_segments + 1;
         void* sargs[] = {&n, &ptr, &cursor};
         rc = launch(OEQ_ROLE_GROUP_SCAN, 1, sargs, stream);
         if (rc) return rc;
-        void* pargs[] = {&n_items, &keys, &cursor, &unordered};
+        void* pargs[] = {&n_items, &keys, &cursor, &unordered, &n_segments};
         rc = launch(OEQ_ROLE_GROUP_SCATTER, n_items, pargs, stream);
         if (rc) return rc;
         void* oargs[] = {&n_segments, &ptr, &unordered, &perm};
@@ -610,7 +610,7 @@ static int walk_index(oeq_kernels* k, const char* who, const WalkLayout& w, int6
     const int64_t* cperm = ix->rperm;
     for (int h = 0; h < k->dims.order_hops; ++h) {
         int64_t* key_out = keys[h & 1];
-        void* hargs[] = {&node_count, &ix->rowptr, &cols, &cperm, &key_in, &key_out};
+        void* hargs[] = {&node_count, &nnz, &ix->rowptr, &cols, &cperm, &key_in, &key_out};
         rc = k->launch(OEQ_ROLE_ORDER_HOP, node_count, hargs, stream);
         if (rc) return rc;
         key_in = key_out;

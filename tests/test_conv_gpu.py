@@ -216,6 +216,48 @@ def test_conv_input_validation():
         conv(X, Y, W, rows.cpu(), cols, perm)
 
 
+def test_edge_list_validation(monkeypatch):
+    """With the edge-list check switched on, a corrupt list is reported before any kernel is launched; with it
+    off (the default, as in the reference) the kernels force every index into range, so the same lists give
+    meaningless but finite-sized work and no access outside the operands."""
+    from openequivariance_amd._torch import ops
+    problem = P.config1_single_uvu()
+    X, Y, W = torch.rand(3, 5, device="cuda"), torch.rand(4, 7, device="cuda"), torch.rand(4, 1, device="cuda")
+    rows = torch.tensor([0, 1, 1, 2], device="cuda")
+    cols = torch.tensor([1, 0, 2, 1], device="cuda")
+    perm = torch.argsort(cols, stable=True)
+    det = oeq.TensorProductConv(problem, deterministic=True)
+    grp = oeq.TensorProductConv(problem, deterministic=False)
+    bad_lists = [
+        ("out of range in tensor 'cols'", det, rows, torch.tensor([1, 0, 3, 1], device="cuda"), perm),
+        ("out of range in tensor 'rows'", grp, torch.tensor([0, -1, 1, 2], device="cuda"), cols, None),
+        ("'rows' is not sorted", det, torch.tensor([1, 0, 1, 2], device="cuda"), cols, perm),
+        ("not a permutation", det, rows, cols, torch.tensor([1, 1, 3, 2], device="cuda")),
+        ("not a permutation", det, rows, cols, torch.tensor([1, 0, 4, 2], device="cuda")),
+        ("does not list the edges by sender", det, rows, cols, torch.tensor([0, 1, 2, 3], device="cuda")),
+    ]
+    monkeypatch.setattr(ops, "CHECK_INDICES", True)
+    det(X, Y, W, rows, cols, perm)
+    grp(X, Y, W, rows, cols)
+    for msg, conv, r, c, p in bad_lists:
+        with pytest.raises(RuntimeError, match=msg):
+            conv(X, Y, W, r, c, p)
+    monkeypatch.setattr(ops, "CHECK_INDICES", False)
+    monkeypatch.setenv("OEQ_AMD_CHECK_INDICES", "1")
+    with pytest.raises(RuntimeError, match="out of range"):
+        grp(X, Y, W, rows, torch.tensor([1, 0, 2, 7], device="cuda"))
+    monkeypatch.setenv("OEQ_AMD_CHECK_INDICES", "0")
+    # unchecked: indices are forced into range on the device; the calls complete and touch only their operands
+    guard = torch.full((64,), 7.0, device="cuda")
+    for msg, conv, r, c, p in bad_lists:
+        Xg, Yg, Wg = (t.clone().requires_grad_(True) for t in (X, Y, W))
+        z = conv(Xg, Yg, Wg, r, c, p)
+        z.sum().backward()
+        torch.cuda.synchronize()
+        assert z.shape == (3, 5) and Xg.grad.shape == (3, 5)
+    assert bool((guard == 7.0).all())
+
+
 def test_conv_double_backward_runs():
     problem = P.config1_single_uvu(np.float64)
     conv = oeq.TensorProductConv(problem, deterministic=True)
