@@ -58,6 +58,12 @@ class UvuEmitter:
     def __init__(self, low: Lowered, *, acc_budget_words: int = 128, g_resident_words: int = 128,
                  kahan: bool = False):
         assert low.mode == "uvu"
+        if low.n_chunks > 16:
+            # one wave per 64-channel chunk of a row, all in one block: 1024 threads is the block limit
+            widest = max(b.mul for b in list(low.in1) + list(low.out))
+            raise ValueError(f"'uvu' kernels handle at most 1024 channels per irrep block (16 chunks of 64); this "
+                             f"problem has a block of multiplicity {widest}. Split the block into several irreps "
+                             "of at most 1024 channels each (with one instruction per piece).")
         self.low = low
         self.ir_mul = low.ir_mul
         self.kahan = kahan  # conv forward: compensated (Kahan) summation over a receiver's edges

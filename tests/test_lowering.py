@@ -88,3 +88,18 @@ def test_generated_sources_compile_for_gfx950(make, conv):
     if problem.instructions[0].connection_mode == "uvu":
         assert {"double_backward_A", "double_backward_B"} <= names
         assert {d[0] for d in descs} >= {rt.ROLE_DOUBLE_BACKWARD_A, rt.ROLE_DOUBLE_BACKWARD_B}
+
+
+@pytest.mark.parametrize("mul", [1088, 2048])
+def test_blocks_wider_than_1024_channels_fail_with_a_message(mul):
+    """One wave per 64-channel chunk and one block per row: 1024 channels is the limit, and exceeding it is
+    reported when the kernels are generated, not as a bad launch descriptor later."""
+    import openequivariance_amd as oeq
+    from openequivariance_amd._torch.tensor_product import build_tp_module
+    from openequivariance_amd._torch.tensor_product_conv import build_conv_module
+    problem = oeq.TPProblem(f"{mul}x1o", "1x1o", f"{mul}x0e", [(0, 0, 0, "uvu", True)], shared_weights=False,
+                            internal_weights=False)
+    with pytest.raises(ValueError, match="at most 1024 channels"):
+        build_tp_module(problem)
+    with pytest.raises(ValueError, match="at most 1024 channels"):
+        build_conv_module(problem, True)
