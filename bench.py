@@ -5,8 +5,12 @@ One step = forward + backward of ``TensorProductConv`` (deterministic mode) on a
 synthetic periodic radius graph: N = 50000 nodes, mean degree ~32 (E ~ 1.6 M),
 X = 128x{0e,1o,2e,3o}, Y = spherical harmonics lmax 3, 23 'uvu' paths, fp32.
 All inputs are resident in HBM before the timed region starts. The default
-``deterministic=False`` mode on shuffled edges (device-side grouping, and the
-float-atomics kernels for comparison) is timed beside it and reported in ``modes``.
+``deterministic=False`` mode on shuffled edges (device-side grouping, sender
+gradients by float atomics; and the reference-style float-atomics kernels for
+comparison) is timed beside it and reported in ``modes``. Next to the HBM
+roofline the record carries the vector-ALU bound of the step (the kernels are
+compiled without packed FP32 instructions) and the stream ceilings measured on
+the same GPU by ./hbm_stream.
 
 Prints ONE JSON line (rank 0). ``value`` = edges per second of the whole step.
 """
@@ -22,6 +26,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+FP32_VECTOR_PEAK_TFLOPS = 157.3  # published; reached with packed FP32 instructions, which this build does not use
 
 
 def parse():
@@ -115,12 +120,17 @@ def tp_config_table(dev, only=None):
     from openequivariance_amd.codegen.lower import lower
     from openequivariance_amd.core import problems as P
 
+    # 512 MiB written before every timed call: twice the 256 MB Infinity Cache, so no operand of the call is
+    # still cached from the previous iteration (the reference flushes 100 MB, backend_hip.hpp:88-95)
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+
     def med(fn, warm=3, it=10):
         for _ in range(warm):
             fn()
         torch.cuda.synchronize()
         ts = []
         for _ in range(it):
+            flush.zero_()
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a.record()
             fn()
@@ -164,7 +174,21 @@ def tp_config_table(dev, only=None):
         table.append(row)
         del x, y, w, g
         torch.cuda.empty_cache()
+    del flush
     return table
+
+
+def hbm_ceilings():
+    """Read-only / write-only / copy stream rates of this GPU (./hbm_stream, built by __graft_entry__.build())."""
+    import subprocess
+    exe = os.path.join(ROOT, "hbm_stream")
+    if not os.path.exists(exe):
+        return None
+    try:
+        res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+        return json.loads(res.stdout.strip().splitlines()[-1]) if res.returncode == 0 else None
+    except Exception:
+        return None
 
 
 def main():
@@ -246,6 +270,26 @@ def main():
         "traffic": None,
         "algorithmic_bytes_per_launch": bwd_kernel_bytes, "avg_kernel_ms": avg["backward"],
         "launches_timed": kt["backward"][1],
+    }
+    # The same fraction per op, with the kernels an op cannot do without counted in: the backward op is
+    # `backward` + `fixup_backward` (+ the index kernels) and moves bwd_bytes; forward moves fwd_bytes.
+    index_ms = avg["oeq_segment_ptr"] * (kt["oeq_segment_ptr"][1] / max(1, kt["backward"][1]))
+    bwd_op_ms = avg["backward"] + avg["fixup_backward"]
+    roofline["ops"] = {
+        "forward": {"algorithmic_bytes": fwd_bytes, "kernel_ms": avg["forward"],
+                    "frac": fwd_bytes / (avg["forward"] * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "backward_op": {"algorithmic_bytes": bwd_bytes, "kernel_ms": bwd_op_ms, "kernels": ["backward", "fixup_backward"],
+                        "frac": bwd_bytes / (bwd_op_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "index_kernels_ms_per_step": index_ms,
+    }
+    # Both bounds of the step (time at 100 % of each peak). The arithmetic is ordinary v_fma_f32: every HIP
+    # file of this build is compiled without packed FP32 instructions, which halves the usable vector rate, so
+    # the step is bounded by its arithmetic before it is bounded by HBM.
+    step_flops = (fwd_flops + bwd_flops) * E
+    roofline["bounds_ms"] = {
+        "hbm_at_8_TBps": (fwd_bytes + bwd_bytes) / HBM_PEAK_GBS / 1e6,
+        "fp32_vector_at_published_peak": step_flops / (FP32_VECTOR_PEAK_TFLOPS * 1e9),
+        "fp32_vector_without_packed_instructions": step_flops / (FP32_VECTOR_PEAK_TFLOPS / 2 * 1e9),
     }
 
     modes = {
@@ -369,6 +413,7 @@ def main():
             tr = json.load(f)
         if tr.get("edges") == E:
             roofline["traffic"] = tr["backward_bytes_per_launch"]
+            roofline["traffic_per_kernel"] = tr.get("per_kernel")
 
     out = {
         "metric": "fused conv fwd+bwd edges/s at MACE shape (deterministic mode)",
@@ -386,6 +431,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "modes": modes,
+        "hbm_stream_ceilings": None if args.no_extras else hbm_ceilings(),
     }
     out.update(extras)
     print(json.dumps(out))

@@ -1,0 +1,117 @@
+// Stream ceilings of the GPU's memory system, measured with plain kernels: what a read-only, a write-only
+// and a copy kernel reach, as sequential sweeps and as one 384 KB chunk per block (the shape of the
+// convolution's per-node edge data). bench.py runs this program (built by __graft_entry__.build()) and
+// puts its JSON line into the bench record; profiles/hbm_ceiling.md summarises it.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <numeric>
+#include <random>
+#include <vector>
+
+typedef float __attribute__((ext_vector_type(4))) f4;
+
+#define CHECK(x)                                                                        \
+    do {                                                                                \
+        hipError_t e_ = (x);                                                            \
+        if (e_ != hipSuccess) {                                                         \
+            std::fprintf(stderr, "%s failed: %s\n", #x, hipGetErrorString(e_));         \
+            return 1;                                                                   \
+        }                                                                               \
+    } while (0)
+
+__global__ __launch_bounds__(256) void read_sweep(const f4* __restrict__ p, size_t n, float* out) {
+    f4 acc = {0, 0, 0, 0};
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) acc += __builtin_nontemporal_load(p + i);
+    if (acc.x + acc.y + acc.z + acc.w == 123.456f) *out = 1.f;
+}
+
+__global__ __launch_bounds__(256) void write_sweep(f4* __restrict__ p, size_t n) {
+    const f4 v = {1, 2, 3, 4};
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) __builtin_nontemporal_store(v, p + i);
+}
+
+__global__ __launch_bounds__(256) void copy_sweep(const f4* __restrict__ a, f4* __restrict__ b, size_t n) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(a + i), b + i);
+}
+
+// one chunk per block, chunks taken in the order `perm` gives
+template <int WRITE>
+__global__ __launch_bounds__(128) void chunks(const f4* __restrict__ a, f4* __restrict__ b, const int* __restrict__ perm,
+                                              int chunk_f4, float* out) {
+    const long c = perm[blockIdx.x];
+    const f4* src = a + c * chunk_f4;
+    f4* dst = b + c * chunk_f4;
+    f4 acc = {0, 0, 0, 0};
+    for (int i = threadIdx.x; i < chunk_f4; i += 128) {
+        const f4 v = __builtin_nontemporal_load(src + i);
+        if (WRITE) __builtin_nontemporal_store(v, dst + i);
+        else acc += v;
+    }
+    if (!WRITE && acc.x + acc.y + acc.z + acc.w == 123.456f) *out = 1.f;
+}
+
+template <typename F>
+static float median_ms(F launch, int iters = 7) {
+    hipEvent_t a, b;
+    (void)hipEventCreate(&a);
+    (void)hipEventCreate(&b);
+    launch();
+    launch();
+    (void)hipDeviceSynchronize();
+    std::vector<float> ts;
+    for (int i = 0; i < iters; ++i) {
+        (void)hipEventRecord(a);
+        launch();
+        (void)hipEventRecord(b);
+        (void)hipEventSynchronize(b);
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, a, b);
+        ts.push_back(ms);
+    }
+    std::sort(ts.begin(), ts.end());
+    return ts[ts.size() / 2];
+}
+
+int main() {
+    const int n_chunks = 21000, chunk_bytes = 384 * 1024;  // 8.26 GB per buffer
+    const int chunk_f4 = chunk_bytes / 16;
+    const size_t bytes = (size_t)n_chunks * chunk_bytes, n = bytes / 16;
+    f4 *a = nullptr, *b = nullptr;
+    float* out = nullptr;
+    int* dperm = nullptr;
+    CHECK(hipMalloc(&a, bytes));
+    CHECK(hipMalloc(&b, bytes));
+    CHECK(hipMalloc(&out, 4));
+    CHECK(hipMalloc(&dperm, n_chunks * sizeof(int)));
+    CHECK(hipMemset(a, 1, bytes));
+    CHECK(hipMemset(b, 0, bytes));
+    const double gb = bytes / 1e9;
+    double best_r = 0, best_w = 0, best_c = 0;
+    for (int grid : {1024, 2048, 4096, 8192, 32768}) {
+        best_r = std::max(best_r, gb / median_ms([&] { read_sweep<<<grid, 256>>>(a, n, out); }) * 1e3);
+        best_w = std::max(best_w, gb / median_ms([&] { write_sweep<<<grid, 256>>>(b, n); }) * 1e3);
+        best_c = std::max(best_c, 2 * gb / median_ms([&] { copy_sweep<<<grid, 256>>>(a, b, n); }) * 1e3);
+    }
+    std::vector<int> perm(n_chunks);
+    std::iota(perm.begin(), perm.end(), 0);
+    CHECK(hipMemcpy(dperm, perm.data(), n_chunks * sizeof(int), hipMemcpyHostToDevice));
+    const double seq_r = gb / median_ms([&] { chunks<0><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
+    const double seq_c = 2 * gb / median_ms([&] { chunks<1><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
+    std::mt19937 gen(1);
+    std::shuffle(perm.begin(), perm.end(), gen);
+    CHECK(hipMemcpy(dperm, perm.data(), n_chunks * sizeof(int), hipMemcpyHostToDevice));
+    const double sc_r = gb / median_ms([&] { chunks<0><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
+    const double sc_c = 2 * gb / median_ms([&] { chunks<1><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
+    const double memcpy_c = 2 * gb / median_ms([&] { (void)hipMemcpyAsync(b, a, bytes, hipMemcpyDeviceToDevice, 0); }) * 1e3;
+    std::printf("{\"unit\": \"GB/s\", \"buffer_gb\": %.2f, \"read_sweep\": %.0f, \"write_sweep\": %.0f, \"copy_sweep\": %.0f, "
+                "\"read_chunks_sequential\": %.0f, \"copy_chunks_sequential\": %.0f, \"read_chunks_scattered\": %.0f, "
+                "\"copy_chunks_scattered\": %.0f, \"hipMemcpy_d2d\": %.0f}\n",
+                gb, best_r, best_w, best_c, seq_r, seq_c, sc_r, sc_c, memcpy_c);
+    return 0;
+}

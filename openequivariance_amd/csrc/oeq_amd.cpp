@@ -488,6 +488,15 @@ int oeq_tp_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in, void* 
 // fused graph convolution
 // ---------------------------------------------------------------------------
 
+// The generated kernels force every node and edge index into range with 32-bit arithmetic.
+static int check_graph_size(const char* who, int64_t node_count, int64_t nnz) {
+    if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "%s: negative size", who);
+    if (node_count > 0x7fffffffLL || nnz > 0x7fffffffLL)
+        return fail(OEQ_ERR_INVALID, "%s: %lld nodes / %lld edges; at most 2^31 - 1 of each are supported", who,
+                    (long long)node_count, (long long)nnz);
+    return OEQ_OK;
+}
+
 // Workspace of the walk modes: one layout for every convolution entry point (pieces a call does not need
 // are left out).
 static size_t ptr_bytes_of(int64_t node_count) { return align_up((size_t)(node_count + 1) * sizeof(int64_t), 256); }
@@ -625,7 +634,7 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void
                      const void* W, void* L3_out, const int64_t* rows, const int64_t* cols, void* workspace,
                      size_t workspace_bytes, void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL kernel set");
-    if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: negative size");
+    if (int bad = check_graph_size("oeq_conv_forward", node_count, nnz)) return bad;
     if (node_count == 0) return OEQ_OK;
     if (!L3_out) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL L3_out");
     const size_t out_bytes = (size_t)node_count * k->dims.L3_dim * k->dims.elem_size;
@@ -677,7 +686,7 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
                       const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* workspace,
                       size_t workspace_bytes, void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL kernel set");
-    if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: negative size");
+    if (int bad = check_graph_size("oeq_conv_backward", node_count, nnz)) return bad;
     const bool shared = k->dims.shared_weights != 0;
     const size_t es = (size_t)k->dims.elem_size;
     // shared weights: the float-atomics kernels add into a cleared W_grad; the walk kernels write partial
@@ -763,7 +772,7 @@ int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, co
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL kernel set");
     if (!oeq_has_double_backward(k) || k->dims.deterministic == OEQ_CONV_ATOMIC)
         return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: this kernel set has no second-order kernels");
-    if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: negative size");
+    if (int bad = check_graph_size("oeq_conv_double_backward", node_count, nnz)) return bad;
     if (node_count == 0) return OEQ_OK;
     if (!L1_grad || !L3_dgrad) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL output");
     const size_t es = (size_t)k->dims.elem_size;
