@@ -301,6 +301,18 @@ def main():
         }
     }
 
+    # The ops keep the index derived from an edge list (CSR pointers, walk order) between calls on the same
+    # tensors, as the layers of a model and their backward passes are; the same step with that cache off,
+    # i.e. the index rebuilt by every forward and every backward:
+    cache_entries, ops.INDEX_CACHE_ENTRIES = ops.INDEX_CACHE_ENTRIES, 0
+    try:
+        ms_cold = time_steps(step_det, max(3, args.steps // 2), 1)
+    finally:
+        ops.INDEX_CACHE_ENTRIES = cache_entries
+    modes["deterministic_index_rebuilt_every_call"] = {
+        "ms_per_step": ms_cold, "edges_per_s": E / (ms_cold * 1e-3),
+        "hbm_roofline_frac": (fwd_bytes + bwd_bytes) / (ms_cold * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
     # ---- deterministic=False (the API default): any edge order --------------------
     if not args.no_atomic:
         perm = torch.randperm(E, device=dev, generator=gen)
@@ -320,6 +332,12 @@ def main():
             ops.conv_backward(X, Ya, Wa, G, ra, ca, dummy, conv_a.kid)
 
         modes["nondeterministic_shuffled_edges"] = mode_entry(time_steps(step_unsorted, args.steps, 1), args.steps)
+        cache_entries, ops.INDEX_CACHE_ENTRIES = ops.INDEX_CACHE_ENTRIES, 0
+        try:
+            modes["nondeterministic_shuffled_edges_index_rebuilt_every_call"] = mode_entry(
+                time_steps(step_unsorted, max(3, args.steps // 2), 1), max(3, args.steps // 2))
+        finally:
+            ops.INDEX_CACHE_ENTRIES = cache_entries
 
         # the float-atomics kernels (edge ranges, flush at every change of receiver), same shuffled edges
         saved = os.environ.get("OEQ_AMD_TUNE")

@@ -211,6 +211,45 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz,
                       void* workspace, size_t workspace_bytes, void* stream);
 size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
 
+/* ---- the index of an edge list, built once and used by several calls --------------------------------- */
+/* Every walk-mode convolution call first derives an index from (rows, cols): CSR pointers over receivers,
+ * in OEQ_CONV_GROUPED mode the edge ids grouped by receiver, the walk order of the nodes and, with
+ * `sender_side` != 0, the same over senders (needed by the calls that reduce per-edge sender-gradient terms:
+ * oeq_conv_backward unless oeq_problem_dims.dx_mode is OEQ_DX_ATOMIC, and oeq_conv_double_backward). The entry
+ * points above build it into the front of their workspace at every call. A caller that runs several
+ * convolutions over one edge list (forward and backward of every layer of a model) builds it once with
+ * oeq_conv_index_build and passes it to the *_indexed variants, which take the same operands, `index` /
+ * `index_bytes` / `index_sender_side` as given to the build, and a scratch buffer of
+ * oeq_conv_backward_scratch_bytes() / oeq_conv_double_backward_scratch_bytes() (forward needs none).
+ * The reference keeps the corresponding state (its workspace tensor and, for the deterministic mode, the
+ * caller's transpose_perm) in the Python module (_torch/TensorProductConv.py:187-193). The index is read-only
+ * after the build, so calls on several streams may share it once the build has completed; it is tied to the
+ * kernel set's mode, node_count, nnz and the contents of rows / cols (/ transpose_perm). For OEQ_CONV_ATOMIC
+ * kernel sets there is no index (size 0; pass NULL). */
+size_t oeq_conv_index_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz, int sender_side);
+int oeq_conv_index_build(oeq_kernels* k, int64_t node_count, int64_t nnz,
+                         const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm,
+                         int sender_side, void* index, size_t index_bytes, void* stream);
+int oeq_conv_forward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz,
+                             const void* L1_in, const void* L2_in, const void* W, void* L3_out,
+                             const int64_t* rows, const int64_t* cols,
+                             const void* index, size_t index_bytes, int index_sender_side, void* stream);
+int oeq_conv_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz,
+                              const void* L1_in, void* L1_grad, const void* L2_in, void* L2_grad,
+                              const void* W, void* W_grad, const void* L3_grad,
+                              const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm,
+                              const void* index, size_t index_bytes, int index_sender_side,
+                              void* scratch, size_t scratch_bytes, void* stream);
+size_t oeq_conv_backward_scratch_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
+int oeq_conv_double_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz,
+                                     const void* L1_in, const void* L2_in, const void* W, const void* L3_grad,
+                                     const void* L1_dgrad, const void* L2_dgrad, const void* W_dgrad,
+                                     void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad,
+                                     const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm,
+                                     const void* index, size_t index_bytes,
+                                     void* scratch, size_t scratch_bytes, void* stream);
+size_t oeq_conv_double_backward_scratch_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
+
 /* ---- second-order ('double backward') kernels ---------------------------- */
 /* Gradient of the backward pass: given the operands of oeq_tp_backward (L1_in, L2_in, W, L3_grad) and
  * cotangents L1_dgrad, L2_dgrad, W_dgrad of its three results, writes the gradients with respect to

@@ -332,6 +332,58 @@ def _conv_checks(e: KernelEntry, L1_in, L2_in, W, rows, cols, perm, L3_grad=None
     return nodes, nnz
 
 
+# ---------------------------------------------------------------------------
+# index of an edge list, kept between calls
+# ---------------------------------------------------------------------------
+
+# A walk-mode convolution first derives an index from the edge list (CSR pointers, edge grouping, walk
+# order; include/oeq_amd.h, oeq_conv_index_build). The layers of a model, and the forward and backward of
+# each, usually run over the same edge tensors, so the ops keep the last few indices and reuse one when a
+# call brings the same tensors (same storage, same version counters, i.e. not written to since), on the same
+# stream, for a kernel set that indexes the same way. The cache holds references to the edge tensors, so
+# their memory cannot be handed to different data while an entry exists. 0 switches the cache off.
+INDEX_CACHE_ENTRIES = 4
+_index_cache: List[dict] = []
+_index_cache_lock = threading.Lock()
+
+
+def clear_index_cache():
+    with _index_cache_lock:
+        _index_cache.clear()
+
+
+def _conv_index(ks, nodes: int, nnz: int, r: torch.Tensor, c: torch.Tensor, p: Optional[torch.Tensor],
+                need_sender_side: bool):
+    """(index tensor, sender_side flag) for the edge list; built now unless a valid one is cached."""
+    dims = ks.dims
+    stream = _stream()
+    grouped = dims["deterministic"] == rt.CONV_GROUPED
+    # the sender side is cheap to add when the caller brings the sender-major permutation, costly when the
+    # library has to group the edges by sender itself: then only the calls that need it build it
+    sender_side = need_sender_side or (not grouped and p is not None and p.numel() == nnz)
+    key = (dims["deterministic"], dims.get("order_hops", 0), nodes, nnz, r.data_ptr(), c.data_ptr(),
+           p.data_ptr() if (p is not None and not grouped) else 0, stream, r.device.index)
+    versions = (r._version, c._version, p._version if (p is not None and not grouped) else 0)
+    caching = INDEX_CACHE_ENTRIES > 0 and not torch.cuda.is_current_stream_capturing()
+    if caching:
+        with _index_cache_lock:
+            for i, ent in enumerate(_index_cache):
+                if ent["key"] == key and ent["versions"] == versions and (ent["sender_side"] or not sender_side):
+                    _index_cache.append(_index_cache.pop(i))
+                    return ent["index"], ent["sender_side"]
+    nb = ks.conv_index_bytes(nodes, nnz, sender_side)
+    index = torch.empty(max(nb, 1), dtype=torch.uint8, device=r.device)
+    ks.conv_index_build(nodes, nnz, r.data_ptr(), c.data_ptr(), p.data_ptr() if (p is not None and not grouped) else 0,
+                        sender_side, index.data_ptr(), nb, stream)
+    if caching:
+        with _index_cache_lock:
+            _index_cache[:] = [ent for ent in _index_cache if ent["key"] != key]
+            _index_cache.append({"key": key, "versions": versions, "sender_side": sender_side, "index": index,
+                                 "refs": (r, c, p)})
+            del _index_cache[:-INDEX_CACHE_ENTRIES]
+    return index, sender_side
+
+
 def _segment_sum(ks, src: torch.Tensor, n_segments: int, keys: torch.Tensor, perm: Optional[torch.Tensor]):
     """Ordered sum of the rows of ``src`` over runs of equal ``keys`` (read through ``perm`` if given)."""
     dst = src.new_empty((n_segments, src.shape[1]))
@@ -386,10 +438,14 @@ def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows
     out = x.new_empty((nodes, e.L3))
     with torch.cuda.device(x.device):
         ks = e.kernels()
-        nb = ks.conv_forward_workspace_bytes(nodes, nnz)
-        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
-        ks.conv_forward(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), r.data_ptr(),
-                        c.data_ptr(), ws.data_ptr() if nb else 0, nb, _stream())
+        if ks.dims["deterministic"] == rt.CONV_ATOMIC or nodes == 0 or nnz == 0:
+            ks.conv_forward(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), r.data_ptr(),
+                            c.data_ptr(), 0, 0, _stream())
+        else:
+            perm = transpose_perm.contiguous() if e.deterministic else None
+            index, side = _conv_index(ks, nodes, nnz, r, c, perm, False)
+            ks.conv_forward_indexed(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), r.data_ptr(),
+                                    c.data_ptr(), index.data_ptr(), index.numel(), side, _stream())
     return out
 
 
@@ -413,11 +469,18 @@ def conv_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_
     dx, dy, dw = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w)
     with torch.cuda.device(x.device):
         ks = e.kernels()
-        nb = ks.conv_backward_workspace_bytes(nodes, nnz)
-        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
-        ks.conv_backward(nodes, nnz, x.data_ptr(), dx.data_ptr(), y.data_ptr(), dy.data_ptr(), w.data_ptr(),
-                         dw.data_ptr(), g.data_ptr(), r.data_ptr(), c.data_ptr(),
-                         p.data_ptr() if e.deterministic else 0, ws.data_ptr() if nb else 0, nb, _stream())
+        pp = p.data_ptr() if e.deterministic else 0
+        if ks.dims["deterministic"] == rt.CONV_ATOMIC or nodes == 0 or nnz == 0:
+            ks.conv_backward(nodes, nnz, x.data_ptr(), dx.data_ptr(), y.data_ptr(), dy.data_ptr(), w.data_ptr(),
+                             dw.data_ptr(), g.data_ptr(), r.data_ptr(), c.data_ptr(), pp, 0, 0, _stream())
+        else:
+            terms = ks.dims.get("dx_mode", 0) != rt.DX_ATOMIC
+            index, side = _conv_index(ks, nodes, nnz, r, c, p if e.deterministic else None, terms)
+            nb = ks.conv_backward_scratch_bytes(nodes, nnz)
+            ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
+            ks.conv_backward_indexed(nodes, nnz, x.data_ptr(), dx.data_ptr(), y.data_ptr(), dy.data_ptr(), w.data_ptr(),
+                                     dw.data_ptr(), g.data_ptr(), r.data_ptr(), c.data_ptr(), pp, index.data_ptr(),
+                                     index.numel(), side, ws.data_ptr() if nb else 0, nb, _stream())
     return dx, dy, dw
 
 
@@ -461,12 +524,19 @@ def conv_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tens
     dx, dy, dw, gg = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w), torch.empty_like(g)
     with torch.cuda.device(x.device):
         ks = e.kernels()
-        nb = ks.conv_double_backward_workspace_bytes(nodes, nnz)
-        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
-        ks.conv_double_backward(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), g.data_ptr(), a.data_ptr(),
-                                b.data_ptr(), c.data_ptr(), dx.data_ptr(), dy.data_ptr(), dw.data_ptr(),
-                                gg.data_ptr(), r.data_ptr(), cc.data_ptr(), p.data_ptr() if e.deterministic else 0,
-                                ws.data_ptr() if nb else 0, nb, _stream())
+        pp = p.data_ptr() if e.deterministic else 0
+        if nodes == 0 or nnz == 0:
+            ks.conv_double_backward(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), g.data_ptr(), a.data_ptr(),
+                                    b.data_ptr(), c.data_ptr(), dx.data_ptr(), dy.data_ptr(), dw.data_ptr(),
+                                    gg.data_ptr(), r.data_ptr(), cc.data_ptr(), pp, 0, 0, _stream())
+        else:
+            index, _side = _conv_index(ks, nodes, nnz, r, cc, p if e.deterministic else None, True)
+            nb = ks.conv_double_backward_scratch_bytes(nodes, nnz)
+            ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
+            ks.conv_double_backward_indexed(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), g.data_ptr(),
+                                            a.data_ptr(), b.data_ptr(), c.data_ptr(), dx.data_ptr(), dy.data_ptr(),
+                                            dw.data_ptr(), gg.data_ptr(), r.data_ptr(), cc.data_ptr(), pp,
+                                            index.data_ptr(), index.numel(), ws.data_ptr() if nb else 0, nb, _stream())
     return dx, dy, dw, gg
 
 

@@ -242,7 +242,7 @@ int static_scratch(void** out) {
 extern "C" {
 
 const char* oeq_last_error(void) { return g_error.c_str(); }
-int oeq_abi_version(void) { return 2; }
+int oeq_abi_version(void) { return 3; }
 
 int oeq_get_device_props(int device, oeq_device_props* out) {
     if (!out) return fail(OEQ_ERR_INVALID, "oeq_get_device_props: out is NULL");
@@ -497,47 +497,62 @@ static int check_graph_size(const char* who, int64_t node_count, int64_t nnz) {
     return OEQ_OK;
 }
 
-// Workspace of the walk modes: one layout for every convolution entry point (pieces a call does not need
-// are left out).
+// Shared weights, walk kernels: one partial weight-gradient row per wave group of the backward grid.
 static size_t ptr_bytes_of(int64_t node_count) { return align_up((size_t)(node_count + 1) * sizeof(int64_t), 256); }
 static size_t perm_bytes_of(int64_t nnz) { return align_up((size_t)nnz * sizeof(int64_t), 256); }
 
-// Shared weights, walk kernels: one partial weight-gradient row per wave group of the backward grid.
 static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t node_count) {
     if (!k->dims.shared_weights || !k->dims.wpartial_per_block) return 0;
     size_t rows = (size_t)k->grid_for(OEQ_ROLE_CONV_BACKWARD, node_count) * (size_t)k->dims.wpartial_per_block;
     return align_up(rows * (size_t)k->dims.weight_numel * (size_t)k->dims.elem_size, 256);
 }
 
-// Byte offsets of the pieces of a call's workspace (SIZE_MAX: piece not present).
-// `terms`: the per-edge dX terms and the sender-side index that their reduction walks;
-// `arrivals`: the per-sender arrival counters of OEQ_DX_ARRIVAL; `wpartial`: partial weight-gradient rows.
-struct WalkLayout {
-    size_t rowptr = SIZE_MAX, colptr = SIZE_MAX, cursor = SIZE_MAX, rperm = SIZE_MAX, sperm = SIZE_MAX,
-           scratch = SIZE_MAX, key_a = SIZE_MAX, key_b = SIZE_MAX, optr = SIZE_MAX, ocursor = SIZE_MAX,
-           order = SIZE_MAX, arrivals = SIZE_MAX, dx_tmp = SIZE_MAX, wpartial = SIZE_MAX, total = 0;
+// The index of an edge list: what the walk kernels derive from (rows, cols) alone. Receiver side: CSR
+// pointers, in GROUPED mode the edge ids grouped by receiver, and the walk order of the nodes. Sender side
+// (for the calls that reduce per-edge dX terms): CSR pointers over senders and, in GROUPED mode, the edge ids
+// grouped by sender. Byte offsets into the index buffer (SIZE_MAX: piece not present); the pieces after
+// `keep` are temporaries of the build.
+struct IndexLayout {
+    size_t rowptr = SIZE_MAX, colptr = SIZE_MAX, rperm = SIZE_MAX, sperm = SIZE_MAX, order = SIZE_MAX, keep = 0,
+           cursor = SIZE_MAX, scratch = SIZE_MAX, key_a = SIZE_MAX, key_b = SIZE_MAX, optr = SIZE_MAX,
+           ocursor = SIZE_MAX, total = 0;
 };
 
-static WalkLayout walk_layout(const oeq_kernels* k, int64_t node_count, int64_t nnz, bool terms, bool arrivals,
-                              bool wpartial) {
-    WalkLayout w;
+static IndexLayout index_layout(const oeq_kernels* k, int64_t node_count, int64_t nnz, bool sender_side) {
+    IndexLayout w;
     const size_t pb = ptr_bytes_of(node_count), qb = perm_bytes_of(nnz);
+    const bool grouped = k->dims.deterministic == OEQ_CONV_GROUPED;
+    const bool ordered = k->dims.order_hops > 0 && k->roles[OEQ_ROLE_ORDER_HOP].present;
     auto take = [&w](size_t bytes) { size_t at = w.total; w.total += bytes; return at; };
     w.rowptr = take(pb);
-    if (terms) w.colptr = take(pb);
-    if (k->dims.deterministic == OEQ_CONV_GROUPED) {
+    if (sender_side) w.colptr = take(pb);
+    if (grouped) w.rperm = take(qb);
+    if (grouped && sender_side) w.sperm = take(qb);
+    if (ordered) w.order = take(pb);
+    w.keep = w.total;
+    if (grouped) {
         w.cursor = take(pb);
-        w.rperm = take(qb);
-        if (terms) w.sperm = take(qb);
         w.scratch = take(qb);
     }
-    if (k->dims.order_hops > 0 && k->roles[OEQ_ROLE_ORDER_HOP].present) {
+    if (ordered) {
         w.key_a = take(pb);
         w.key_b = take(pb);
         w.optr = take(pb);
         w.ocursor = take(pb);
-        w.order = take(pb);
     }
+    return w;
+}
+
+// What a call needs besides operands and index: `terms` = the per-edge dX terms, `arrivals` = the per-sender
+// arrival counters of OEQ_DX_ARRIVAL, `wpartial` = partial weight-gradient rows (shared weights).
+struct ScratchLayout {
+    size_t arrivals = SIZE_MAX, dx_tmp = SIZE_MAX, wpartial = SIZE_MAX, total = 0;
+};
+
+static ScratchLayout scratch_layout(const oeq_kernels* k, int64_t node_count, int64_t nnz, bool terms, bool arrivals,
+                                    bool wpartial) {
+    ScratchLayout w;
+    auto take = [&w](size_t bytes) { size_t at = w.total; w.total += bytes; return at; };
     if (arrivals)
         w.arrivals = take(align_up((size_t)node_count * (size_t)std::max(1, k->dims.n_chunks) * sizeof(int32_t), 256));
     if (terms) w.dx_tmp = take(align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256));
@@ -546,93 +561,121 @@ static WalkLayout walk_layout(const oeq_kernels* k, int64_t node_count, int64_t 
     return w;
 }
 
-size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
-    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
-    return walk_layout(k, node_count, nnz, false, false, false).total;
-}
-
-static WalkLayout backward_layout(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
-    return walk_layout(k, node_count, nnz, k->dims.dx_mode != OEQ_DX_ATOMIC, k->dims.dx_mode == OEQ_DX_ARRIVAL,
-                       true);
-}
-
-size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
-    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
-    return backward_layout(k, node_count, nnz).total;
-}
-
-// the second-order kernels always go through the per-edge terms and fixup_backward
-size_t oeq_conv_double_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
-    if (!k || k->dims.deterministic == OEQ_CONV_ATOMIC) return 0;
-    return walk_layout(k, node_count, nnz, true, false, false).total;
-}
-
-// What the walk kernels of a backward-type call need besides the operands: CSR pointers over receivers and,
-// when the per-edge terms are kept, over senders; the walk orders (GROUPED mode: built here; SORTED mode: the
-// caller's lists); the buffer of per-edge dX terms. Everything lives in the caller's workspace.
 struct WalkIndex {
     int64_t *rowptr = nullptr, *colptr = nullptr, *rperm = nullptr;
     const int64_t* sperm = nullptr;
-    void *dx_tmp = nullptr, *wpartial = nullptr;
-    int32_t* arrivals = nullptr;
     int64_t* order = nullptr;  // the order in which the walk kernels visit the nodes (NULL: by index)
 };
 
-static int walk_index(oeq_kernels* k, const char* who, const WalkLayout& w, int64_t node_count, int64_t nnz,
-                      const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* workspace,
-                      size_t workspace_bytes, void* stream, WalkIndex* ix) {
-    const int mode = k->dims.deterministic;
-    const bool terms = w.dx_tmp != SIZE_MAX;
-    if (mode == OEQ_CONV_SORTED && terms && !transpose_perm)
+struct WalkScratch {
+    void *dx_tmp = nullptr, *wpartial = nullptr;
+    int32_t* arrivals = nullptr;
+};
+
+static char* at_offset(const void* base, size_t off) { return off == SIZE_MAX ? nullptr : (char*)base + off; }
+
+// Pointers into a built index buffer.
+static int bind_index(const oeq_kernels* k, const char* who, const IndexLayout& w, const void* index,
+                      size_t index_bytes, const int64_t* transpose_perm, WalkIndex* ix) {
+    if (!index || index_bytes < w.keep)
+        return fail(OEQ_ERR_INVALID, "%s: index buffer too small (%zu < %zu bytes)", who, index_bytes, w.keep);
+    if (k->dims.deterministic == OEQ_CONV_SORTED && w.colptr != SIZE_MAX && !transpose_perm)
         return fail(OEQ_ERR_INVALID, "%s: deterministic mode needs transpose_perm", who);
-    if (!workspace || workspace_bytes < w.total)
-        return fail(OEQ_ERR_INVALID, "%s: workspace too small (%zu < %zu bytes)", who, workspace_bytes, w.total);
-    char* base = (char*)workspace;
-    auto at = [base](size_t off) -> char* { return off == SIZE_MAX ? nullptr : base + off; };
-    ix->rowptr = (int64_t*)at(w.rowptr);
-    ix->colptr = (int64_t*)at(w.colptr);
-    ix->dx_tmp = at(w.dx_tmp);
-    ix->wpartial = at(w.wpartial);
-    ix->arrivals = (int32_t*)at(w.arrivals);
-    ix->sperm = transpose_perm;
-    int rc;
-    if (mode == OEQ_CONV_SORTED) {
-        rc = k->segment_ptr(nnz, node_count, rows, nullptr, ix->rowptr, stream);
-        if (!rc && terms) rc = k->segment_ptr(nnz, node_count, cols, transpose_perm, ix->colptr, stream);
+    ix->rowptr = (int64_t*)at_offset(index, w.rowptr);
+    ix->colptr = (int64_t*)at_offset(index, w.colptr);
+    ix->rperm = (int64_t*)at_offset(index, w.rperm);
+    ix->sperm = w.sperm != SIZE_MAX ? (const int64_t*)at_offset(index, w.sperm) : transpose_perm;
+    ix->order = (int64_t*)at_offset(index, w.order);
+    return OEQ_OK;
+}
+
+static int build_index(oeq_kernels* k, const char* who, const IndexLayout& w, int64_t node_count, int64_t nnz,
+                       const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* index,
+                       size_t index_bytes, void* stream) {
+    if (!rows || !cols) return fail(OEQ_ERR_INVALID, "%s: NULL edge list", who);
+    if (!index || index_bytes < w.total)
+        return fail(OEQ_ERR_INVALID, "%s: workspace too small (%zu < %zu bytes)", who, index_bytes, w.total);
+    WalkIndex ix;
+    int rc = bind_index(k, who, w, index, index_bytes, transpose_perm, &ix);
+    if (rc) return rc;
+    const bool sender_side = w.colptr != SIZE_MAX;
+    if (k->dims.deterministic == OEQ_CONV_SORTED) {
+        rc = k->segment_ptr(nnz, node_count, rows, nullptr, ix.rowptr, stream);
+        if (!rc && sender_side) rc = k->segment_ptr(nnz, node_count, cols, transpose_perm, ix.colptr, stream);
     } else {
-        int64_t* cursor = (int64_t*)at(w.cursor);
-        int64_t* scratch = (int64_t*)at(w.scratch);
-        ix->rperm = (int64_t*)at(w.rperm);
-        rc = k->group_by_key(nnz, node_count, rows, ix->rowptr, cursor, scratch, ix->rperm, stream);
-        if (!rc && terms) {
-            int64_t* sp = (int64_t*)at(w.sperm);
-            rc = k->group_by_key(nnz, node_count, cols, ix->colptr, cursor, scratch, sp, stream);
-            ix->sperm = sp;
-        }
+        int64_t* cursor = (int64_t*)at_offset(index, w.cursor);
+        int64_t* scratch = (int64_t*)at_offset(index, w.scratch);
+        rc = k->group_by_key(nnz, node_count, rows, ix.rowptr, cursor, scratch, ix.rperm, stream);
+        if (!rc && sender_side)
+            rc = k->group_by_key(nnz, node_count, cols, ix.colptr, cursor, scratch, (int64_t*)ix.sperm, stream);
     }
-    if (rc || w.order == SIZE_MAX) return rc;
+    if (rc || !ix.order) return rc;
     // Walk order: cluster the nodes by the highest-priority node within `order_hops` edges, then list them
     // cluster by cluster (a counting sort by cluster key; the order inside a cluster is whatever the
     // scatter's atomics give, which changes which nodes run side by side but no result).
-    int64_t* keys[2] = {(int64_t*)at(w.key_a), (int64_t*)at(w.key_b)};
+    int64_t* keys[2] = {(int64_t*)at_offset(index, w.key_a), (int64_t*)at_offset(index, w.key_b)};
     const int64_t* key_in = nullptr;
-    const int64_t* cperm = ix->rperm;
+    const int64_t* cperm = ix.rperm;
     for (int h = 0; h < k->dims.order_hops; ++h) {
         int64_t* key_out = keys[h & 1];
-        void* hargs[] = {&node_count, &nnz, &ix->rowptr, &cols, &cperm, &key_in, &key_out};
+        void* hargs[] = {&node_count, &nnz, &ix.rowptr, &cols, &cperm, &key_in, &key_out};
         rc = k->launch(OEQ_ROLE_ORDER_HOP, node_count, hargs, stream);
         if (rc) return rc;
         key_in = key_out;
     }
-    int64_t* optr = (int64_t*)at(w.optr);
-    int64_t* ocursor = (int64_t*)at(w.ocursor);
-    ix->order = (int64_t*)at(w.order);
-    return k->group_unordered(node_count, node_count, key_in, optr, ocursor, ix->order, stream);
+    return k->group_unordered(node_count, node_count, key_in, (int64_t*)at_offset(index, w.optr),
+                              (int64_t*)at_offset(index, w.ocursor), ix.order, stream);
 }
 
-int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
-                     const void* W, void* L3_out, const int64_t* rows, const int64_t* cols, void* workspace,
-                     size_t workspace_bytes, void* stream) {
+static bool walk_mode(const oeq_kernels* k) { return k->dims.deterministic != OEQ_CONV_ATOMIC; }
+static bool backward_terms(const oeq_kernels* k) { return k->dims.dx_mode != OEQ_DX_ATOMIC; }
+
+size_t oeq_conv_index_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz, int sender_side) {
+    if (!k || !walk_mode(k) || node_count < 0 || nnz < 0) return 0;
+    return index_layout(k, node_count, nnz, sender_side != 0).total;
+}
+
+int oeq_conv_index_build(oeq_kernels* k, int64_t node_count, int64_t nnz, const int64_t* rows, const int64_t* cols,
+                         const int64_t* transpose_perm, int sender_side, void* index, size_t index_bytes,
+                         void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_index_build: NULL kernel set");
+    if (int bad = check_graph_size("oeq_conv_index_build", node_count, nnz)) return bad;
+    if (!walk_mode(k) || node_count == 0 || nnz == 0) return OEQ_OK;  // nothing to index
+    if (sender_side && k->dims.deterministic == OEQ_CONV_SORTED && !transpose_perm)
+        return fail(OEQ_ERR_INVALID, "oeq_conv_index_build: deterministic mode needs transpose_perm");
+    return build_index(k, "oeq_conv_index_build", index_layout(k, node_count, nnz, sender_side != 0), node_count, nnz,
+                       rows, cols, transpose_perm, index, index_bytes, stream);
+}
+
+size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    return oeq_conv_index_bytes(k, node_count, nnz, 0);
+}
+
+size_t oeq_conv_backward_scratch_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    if (!k || !walk_mode(k)) return 0;
+    return scratch_layout(k, node_count, nnz, backward_terms(k), k->dims.dx_mode == OEQ_DX_ARRIVAL, true).total;
+}
+
+size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    if (!k || !walk_mode(k)) return 0;
+    return oeq_conv_index_bytes(k, node_count, nnz, backward_terms(k)) +
+           oeq_conv_backward_scratch_bytes(k, node_count, nnz);
+}
+
+// the second-order kernels always go through the per-edge terms and fixup_backward
+size_t oeq_conv_double_backward_scratch_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    if (!k || !walk_mode(k)) return 0;
+    return scratch_layout(k, node_count, nnz, true, false, false).total;
+}
+
+size_t oeq_conv_double_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    if (!k || !walk_mode(k)) return 0;
+    return oeq_conv_index_bytes(k, node_count, nnz, 1) + oeq_conv_double_backward_scratch_bytes(k, node_count, nnz);
+}
+
+int oeq_conv_forward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
+                             const void* W, void* L3_out, const int64_t* rows, const int64_t* cols, const void* index,
+                             size_t index_bytes, int index_sender_side, void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL kernel set");
     if (int bad = check_graph_size("oeq_conv_forward", node_count, nnz)) return bad;
     if (node_count == 0) return OEQ_OK;
@@ -641,18 +684,37 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void
     if (nnz == 0) return k->fill_zero(L3_out, out_bytes, stream);
     if (!L1_in || !L2_in || !W || !rows || !cols) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL buffer");
     WalkIndex ix;
-    const int mode = k->dims.deterministic;
     int rc;
-    if (mode != OEQ_CONV_ATOMIC) {
-        rc = walk_index(k, "oeq_conv_forward", walk_layout(k, node_count, nnz, false, false, false), node_count, nnz,
-                        rows, cols, nullptr, workspace, workspace_bytes, stream, &ix);
+    if (walk_mode(k)) {
+        // the forward reads the receiver side only; the caller's perm stands in where the layout wants one
+        rc = bind_index(k, "oeq_conv_forward", index_layout(k, node_count, nnz, index_sender_side != 0), index,
+                        index_bytes, rows, &ix);
         if (rc) return rc;
     } else {
         rc = k->fill_zero(L3_out, out_bytes, stream);
         if (rc) return rc;
     }
     void* args[] = {&node_count, &nnz, &L1_in, &L2_in, &W, &L3_out, &rows, &cols, &ix.rowptr, &ix.rperm, &ix.order};
-    return k->launch(OEQ_ROLE_CONV_FORWARD, mode != OEQ_CONV_ATOMIC ? node_count : nnz, args, stream);
+    return k->launch(OEQ_ROLE_CONV_FORWARD, walk_mode(k) ? node_count : nnz, args, stream);
+}
+
+int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
+                     const void* W, void* L3_out, const int64_t* rows, const int64_t* cols, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL kernel set");
+    if (int bad = check_graph_size("oeq_conv_forward", node_count, nnz)) return bad;
+    size_t index_bytes = 0;
+    if (walk_mode(k) && node_count > 0 && nnz > 0) {
+        if (!L3_out) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL L3_out");
+        if (!L1_in || !L2_in || !W || !rows || !cols) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL buffer");
+        const IndexLayout w = index_layout(k, node_count, nnz, false);
+        int rc = build_index(k, "oeq_conv_forward", w, node_count, nnz, rows, cols, nullptr, workspace,
+                             workspace_bytes, stream);
+        if (rc) return rc;
+        index_bytes = w.total;
+    }
+    return oeq_conv_forward_indexed(k, node_count, nnz, L1_in, L2_in, W, L3_out, rows, cols, workspace, index_bytes, 0,
+                                    stream);
 }
 
 size_t oeq_static_scratch_bytes(void) { return OEQ_STATIC_SCRATCH_BYTES; }
@@ -681,17 +743,18 @@ int oeq_conv_forward_static(oeq_kernels* k, int64_t node_count, int64_t nnz, con
     return rc;
 }
 
-int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, void* L1_grad,
-                      const void* L2_in, void* L2_grad, const void* W, void* W_grad, const void* L3_grad,
-                      const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* workspace,
-                      size_t workspace_bytes, void* stream) {
+int oeq_conv_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, void* L1_grad,
+                              const void* L2_in, void* L2_grad, const void* W, void* W_grad, const void* L3_grad,
+                              const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm,
+                              const void* index, size_t index_bytes, int index_sender_side, void* scratch,
+                              size_t scratch_bytes, void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL kernel set");
     if (int bad = check_graph_size("oeq_conv_backward", node_count, nnz)) return bad;
     const bool shared = k->dims.shared_weights != 0;
     const size_t es = (size_t)k->dims.elem_size;
     // shared weights: the float-atomics kernels add into a cleared W_grad; the walk kernels write partial
     // rows that are summed in order at the end (W_grad is cleared only when there is nothing to sum)
-    const bool wrows = shared && k->dims.deterministic != OEQ_CONV_ATOMIC && k->dims.wpartial_per_block > 0;
+    const bool wrows = shared && walk_mode(k) && k->dims.wpartial_per_block > 0;
     int rc;
     if (shared && (!wrows || node_count == 0 || nnz == 0)) {
         if (!W_grad) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL W_grad");
@@ -706,12 +769,24 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
         return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL buffer");
 
     WalkIndex ix;
-    const int mode = k->dims.deterministic;
-    const int dx_mode = mode == OEQ_CONV_ATOMIC ? (int)OEQ_DX_ATOMIC : k->dims.dx_mode;
-    if (mode != OEQ_CONV_ATOMIC) {
-        rc = walk_index(k, "oeq_conv_backward", backward_layout(k, node_count, nnz), node_count, nnz, rows, cols,
-                        transpose_perm, workspace, workspace_bytes, stream, &ix);
+    WalkScratch sc;
+    const int dx_mode = walk_mode(k) ? k->dims.dx_mode : (int)OEQ_DX_ATOMIC;
+    if (walk_mode(k)) {
+        if (backward_terms(k) && !index_sender_side)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: this kernel set needs an index built with the sender side");
+        rc = bind_index(k, "oeq_conv_backward", index_layout(k, node_count, nnz, index_sender_side != 0), index,
+                        index_bytes, transpose_perm ? transpose_perm : rows, &ix);
         if (rc) return rc;
+        if (backward_terms(k) && k->dims.deterministic == OEQ_CONV_SORTED && !transpose_perm)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: deterministic mode needs transpose_perm");
+        const ScratchLayout w =
+            scratch_layout(k, node_count, nnz, backward_terms(k), dx_mode == OEQ_DX_ARRIVAL, true);
+        if (w.total && (!scratch || scratch_bytes < w.total))
+            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: workspace too small (%zu < %zu bytes of scratch)",
+                        scratch_bytes, w.total);
+        sc.dx_tmp = at_offset(scratch, w.dx_tmp);
+        sc.wpartial = at_offset(scratch, w.wpartial);
+        sc.arrivals = (int32_t*)at_offset(scratch, w.arrivals);
     }
     if (dx_mode != OEQ_DX_TERMS) {
         // atomics accumulate into the rows; the arrival scheme never visits a node that sends nothing
@@ -719,24 +794,54 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
         if (rc) return rc;
     }
     if (dx_mode == OEQ_DX_ARRIVAL) {
-        rc = k->fill_zero(ix.arrivals, (size_t)node_count * (size_t)std::max(1, k->dims.n_chunks) * sizeof(int32_t),
+        rc = k->fill_zero(sc.arrivals, (size_t)node_count * (size_t)std::max(1, k->dims.n_chunks) * sizeof(int32_t),
                           stream);
         if (rc) return rc;
     }
     void* args[] = {&node_count, &nnz,     &L1_in, &L1_grad, &L2_in,     &L2_grad,   &W,          &W_grad,   &L3_grad,
-                    &rows,       &cols,    &ix.rowptr, &ix.dx_tmp, &ix.rperm, &ix.wpartial, &ix.colptr, &ix.sperm,
-                    &ix.arrivals, &ix.order};
-    rc = k->launch(OEQ_ROLE_CONV_BACKWARD, mode != OEQ_CONV_ATOMIC ? node_count : nnz, args, stream);
-    if (rc || mode == OEQ_CONV_ATOMIC) return rc;
+                    &rows,       &cols,    &ix.rowptr, &sc.dx_tmp, &ix.rperm, &sc.wpartial, &ix.colptr, &ix.sperm,
+                    &sc.arrivals, &ix.order};
+    rc = k->launch(OEQ_ROLE_CONV_BACKWARD, walk_mode(k) ? node_count : nnz, args, stream);
+    if (rc || !walk_mode(k)) return rc;
     if (dx_mode == OEQ_DX_TERMS) {
-        void* fargs[] = {&node_count, &nnz, &ix.dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};
+        void* fargs[] = {&node_count, &nnz, &sc.dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};
         rc = k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
     }
     if (rc || !wrows) return rc;
     int64_t n_partials = (int64_t)k->grid_for(OEQ_ROLE_CONV_BACKWARD, node_count) * k->dims.wpartial_per_block;
     int64_t wn = k->dims.weight_numel;
-    void* rargs[] = {&n_partials, &ix.wpartial, &W_grad, &wn};
+    void* rargs[] = {&n_partials, &sc.wpartial, &W_grad, &wn};
     return k->launch(OEQ_ROLE_TP_BACKWARD_WREDUCE, wn, rargs, stream);
+}
+
+int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, void* L1_grad,
+                      const void* L2_in, void* L2_grad, const void* W, void* W_grad, const void* L3_grad,
+                      const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL kernel set");
+    if (int bad = check_graph_size("oeq_conv_backward", node_count, nnz)) return bad;
+    size_t index_bytes = 0;
+    const bool sender_side = walk_mode(k) && backward_terms(k);
+    if (walk_mode(k) && node_count > 0 && nnz > 0) {
+        if (!L1_grad) return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL L1_grad");
+        if (!L1_in || !L2_in || !L2_grad || !W || !W_grad || !L3_grad || !rows || !cols)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: NULL buffer");
+        if (sender_side && k->dims.deterministic == OEQ_CONV_SORTED && !transpose_perm)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: deterministic mode needs transpose_perm");
+        const IndexLayout w = index_layout(k, node_count, nnz, sender_side);
+        const size_t need = w.total + oeq_conv_backward_scratch_bytes(k, node_count, nnz);
+        if (!workspace || workspace_bytes < need)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_backward: workspace too small (%zu < %zu bytes)", workspace_bytes,
+                        need);
+        int rc = build_index(k, "oeq_conv_backward", w, node_count, nnz, rows, cols, transpose_perm, workspace, w.total,
+                             stream);
+        if (rc) return rc;
+        index_bytes = w.total;
+    }
+    return oeq_conv_backward_indexed(k, node_count, nnz, L1_in, L1_grad, L2_in, L2_grad, W, W_grad, L3_grad, rows, cols,
+                                     transpose_perm, workspace, index_bytes, sender_side,
+                                     workspace ? (char*)workspace + index_bytes : nullptr,
+                                     workspace_bytes > index_bytes ? workspace_bytes - index_bytes : 0, stream);
 }
 
 // ---------------------------------------------------------------------------
@@ -764,13 +869,14 @@ int oeq_tp_double_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in,
     return k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, num_batch, b, stream);
 }
 
-int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
-                             const void* W, const void* L3_grad, const void* L1_dgrad, const void* L2_dgrad,
-                             const void* W_dgrad, void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad,
-                             const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* workspace,
-                             size_t workspace_bytes, void* stream) {
+int oeq_conv_double_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in,
+                                     const void* L2_in, const void* W, const void* L3_grad, const void* L1_dgrad,
+                                     const void* L2_dgrad, const void* W_dgrad, void* L1_grad, void* L2_grad,
+                                     void* W_grad, void* L3_dgrad, const int64_t* rows, const int64_t* cols,
+                                     const int64_t* transpose_perm, const void* index, size_t index_bytes,
+                                     void* scratch, size_t scratch_bytes, void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL kernel set");
-    if (!oeq_has_double_backward(k) || k->dims.deterministic == OEQ_CONV_ATOMIC)
+    if (!oeq_has_double_backward(k) || !walk_mode(k))
         return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: this kernel set has no second-order kernels");
     if (int bad = check_graph_size("oeq_conv_double_backward", node_count, nnz)) return bad;
     if (node_count == 0) return OEQ_OK;
@@ -785,9 +891,14 @@ int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, co
         !cols)
         return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL buffer");
     WalkIndex ix;
-    int rc = walk_index(k, "oeq_conv_double_backward", walk_layout(k, node_count, nnz, true, false, false), node_count,
-                        nnz, rows, cols, transpose_perm, workspace, workspace_bytes, stream, &ix);
+    int rc = bind_index(k, "oeq_conv_double_backward", index_layout(k, node_count, nnz, true), index, index_bytes,
+                        transpose_perm, &ix);
     if (rc) return rc;
+    const ScratchLayout w = scratch_layout(k, node_count, nnz, true, false, false);
+    if (!scratch || scratch_bytes < w.total)
+        return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: workspace too small (%zu < %zu bytes of scratch)",
+                    scratch_bytes, w.total);
+    void* dx_tmp = at_offset(scratch, w.dx_tmp);
     void* a[] = {&node_count, &nnz, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_dgrad,
                  &rows,       &cols, &ix.rowptr, &ix.rperm, &ix.order};
     if (k->roles[OEQ_ROLE_DOUBLE_BACKWARD_A].present) {
@@ -795,11 +906,41 @@ int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, co
         if (rc) return rc;
     }
     void* b[] = {&node_count, &nnz,     &L1_in,  &L1_dgrad, &L2_in, &L2_dgrad,  &W,         &W_dgrad, &L3_grad,
-                 &L2_grad,    &W_grad,  &rows,   &cols,     &ix.rowptr, &ix.dx_tmp, &ix.rperm, &L3_dgrad, &ix.order};
+                 &L2_grad,    &W_grad,  &rows,   &cols,     &ix.rowptr, &dx_tmp, &ix.rperm, &L3_dgrad, &ix.order};
     rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count, b, stream);
     if (rc) return rc;
-    void* fargs[] = {&node_count, &nnz, &ix.dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};
+    void* fargs[] = {&node_count, &nnz, &dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};
     return k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
+}
+
+int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
+                             const void* W, const void* L3_grad, const void* L1_dgrad, const void* L2_dgrad,
+                             const void* W_dgrad, void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad,
+                             const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+    if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL kernel set");
+    if (!oeq_has_double_backward(k) || !walk_mode(k))
+        return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: this kernel set has no second-order kernels");
+    if (int bad = check_graph_size("oeq_conv_double_backward", node_count, nnz)) return bad;
+    size_t index_bytes = 0;
+    if (node_count > 0 && nnz > 0) {
+        if (!rows || !cols) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL buffer");
+        if (k->dims.deterministic == OEQ_CONV_SORTED && !transpose_perm)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: deterministic mode needs transpose_perm");
+        const IndexLayout w = index_layout(k, node_count, nnz, true);
+        const size_t need = w.total + oeq_conv_double_backward_scratch_bytes(k, node_count, nnz);
+        if (!workspace || workspace_bytes < need)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: workspace too small (%zu < %zu bytes)",
+                        workspace_bytes, need);
+        int rc = build_index(k, "oeq_conv_double_backward", w, node_count, nnz, rows, cols, transpose_perm, workspace,
+                             w.total, stream);
+        if (rc) return rc;
+        index_bytes = w.total;
+    }
+    return oeq_conv_double_backward_indexed(k, node_count, nnz, L1_in, L2_in, W, L3_grad, L1_dgrad, L2_dgrad, W_dgrad,
+                                            L1_grad, L2_grad, W_grad, L3_dgrad, rows, cols, transpose_perm, workspace,
+                                            index_bytes, workspace ? (char*)workspace + index_bytes : nullptr,
+                                            workspace_bytes > index_bytes ? workspace_bytes - index_bytes : 0, stream);
 }
 
 }  // extern "C"

@@ -53,7 +53,7 @@ ROLE_ORDER_HOP = 15
 
 CONV_ATOMIC, CONV_SORTED, CONV_GROUPED = 0, 1, 2
 DX_TERMS, DX_ATOMIC, DX_ARRIVAL = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class OeqError(RuntimeError):
@@ -143,6 +143,13 @@ EXPORTS = {
     "oeq_conv_backward": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_conv_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_double_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_conv_index_bytes": (_SZ, [_P, _I64, _I64, ctypes.c_int]),
+    "oeq_conv_index_build": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, ctypes.c_int, _P, _SZ, _P]),
+    "oeq_conv_forward_indexed": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _SZ, ctypes.c_int, _P]),
+    "oeq_conv_backward_indexed": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 10 + [_P, _SZ, ctypes.c_int, _P, _SZ, _P]),
+    "oeq_conv_backward_scratch_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_conv_double_backward_indexed": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 14 + [_P, _SZ, _P, _SZ, _P]),
+    "oeq_conv_double_backward_scratch_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_has_double_backward": (ctypes.c_int, [_P]),
     "oeq_tp_double_backward": (ctypes.c_int, [_P, _I64] + [_P] * 12),
     "oeq_conv_double_backward": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 15 + [_SZ, _P]),
@@ -332,6 +339,36 @@ class KernelSet:
         """oeq_conv_forward with the library's static scratch array instead of a workspace; allocates nothing."""
         _check(self._lib.oeq_conv_forward_static(self.handle, nodes, nnz, x, y, w, out, rows, cols, stream),
                "oeq_conv_forward_static")
+
+    # ---- index of an edge list, built once and shared by several calls
+    def conv_index_bytes(self, nodes, nnz, sender_side: bool) -> int:
+        return self._lib.oeq_conv_index_bytes(self.handle, nodes, nnz, int(sender_side))
+
+    def conv_index_build(self, nodes, nnz, rows, cols, perm, sender_side: bool, index, index_bytes, stream):
+        _check(self._lib.oeq_conv_index_build(self.handle, nodes, nnz, rows, cols, perm, int(sender_side), index,
+                                              index_bytes, stream), "oeq_conv_index_build")
+
+    def conv_forward_indexed(self, nodes, nnz, x, y, w, out, rows, cols, index, index_bytes, sender_side, stream):
+        _check(self._lib.oeq_conv_forward_indexed(self.handle, nodes, nnz, x, y, w, out, rows, cols, index, index_bytes,
+                                                  int(sender_side), stream), "oeq_conv_forward_indexed")
+
+    def conv_backward_scratch_bytes(self, nodes, nnz) -> int:
+        return self._lib.oeq_conv_backward_scratch_bytes(self.handle, nodes, nnz)
+
+    def conv_backward_indexed(self, nodes, nnz, x, dx, y, dy, w, dw, g, rows, cols, perm, index, index_bytes,
+                              sender_side, scratch, scratch_bytes, stream):
+        _check(self._lib.oeq_conv_backward_indexed(self.handle, nodes, nnz, x, dx, y, dy, w, dw, g, rows, cols, perm,
+                                                   index, index_bytes, int(sender_side), scratch, scratch_bytes,
+                                                   stream), "oeq_conv_backward_indexed")
+
+    def conv_double_backward_scratch_bytes(self, nodes, nnz) -> int:
+        return self._lib.oeq_conv_double_backward_scratch_bytes(self.handle, nodes, nnz)
+
+    def conv_double_backward_indexed(self, nodes, nnz, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg, rows, cols, perm,
+                                     index, index_bytes, scratch, scratch_bytes, stream):
+        _check(self._lib.oeq_conv_double_backward_indexed(self.handle, nodes, nnz, x, y, w, g, ddx, ddy, ddw, dx, dy, dw,
+                                                          gg, rows, cols, perm, index, index_bytes, scratch,
+                                                          scratch_bytes, stream), "oeq_conv_double_backward_indexed")
 
     def has_double_backward(self) -> bool:
         return bool(self._lib.oeq_has_double_backward(self.handle))

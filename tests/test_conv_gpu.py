@@ -450,3 +450,58 @@ def test_sender_gradient_modes():
     assert (dx - base[1]).abs().max() <= 1e-5 * base[1].abs().max()
     assert ops.get_entry(oeq.TensorProductConv(problem, deterministic=True).kid).kernels().dims["dx_mode"] == rt.DX_TERMS
     assert ops.get_entry(oeq.TensorProductConv(problem, deterministic=False).kid).kernels().dims["dx_mode"] == rt.DX_ATOMIC
+
+
+def test_edge_list_index_is_reused_and_invalidated():
+    """The ops keep the index of the last few edge lists: a second call over the same tensors builds nothing,
+    a call after the tensors were written to (or with other tensors of the same contents) builds again, and the
+    results are the same bits as with the cache switched off."""
+    from openequivariance_amd._torch import ops
+    problem = P.config2_nequip_uvu()
+    coords, rows, cols = _graph(80, 8, seed=9)
+    g = CoordGraph(coords, rows, cols)
+    E = g.nnz
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    X = torch.randn(80, problem.irreps_in1.dim, device="cuda", generator=gen)
+    Y = torch.randn(E, problem.irreps_in2.dim, device="cuda", generator=gen)
+    W = torch.randn(E, problem.weight_numel, device="cuda", generator=gen)
+    G = torch.randn(80, problem.irreps_out.dim, device="cuda", generator=gen)
+    for det in (True, False):
+        conv = oeq.TensorProductConv(problem, deterministic=det)
+        tr, tc, tp = (torch.tensor(a, device="cuda") for a in (g.rows, g.cols, g.transpose_perm))
+        builds = []
+        ks = ops.get_entry(conv.kid).kernels()
+        real = ks.conv_index_build
+        ks.conv_index_build = lambda *a, **k: (builds.append(1), real(*a, **k))[1]
+        try:
+            ops.clear_index_cache()
+            z1 = ops.conv_forward(X, Y, W, tr, tc, tp, conv.kid)
+            first = len(builds)
+            assert first == 1
+            z2 = ops.conv_forward(X, Y, W, tr, tc, tp, conv.kid)
+            g1 = ops.conv_backward(X, Y, W, G, tr, tc, tp, conv.kid)
+            assert len(builds) == first, "same tensors, same stream: the index is reused"
+            assert torch.equal(z1, z2)
+            # written to in place (same values): the version counter moves, the index is rebuilt
+            tc.add_(0)
+            z3 = ops.conv_forward(X, Y, W, tr, tc, tp, conv.kid)
+            assert len(builds) == first + 1 and torch.equal(z3, z1)
+            # a different edge list in the same storage must not be served the old index
+            flipped = torch.tensor(g.cols[::-1].copy(), device="cuda")
+            tc.copy_(flipped)
+            tp2 = torch.tensor(np.lexsort((g.rows, g.cols[::-1])), device="cuda")
+            z4 = ops.conv_forward(X, Y, W, tr, tc, tp2, conv.kid)
+            monkey_off = ops.INDEX_CACHE_ENTRIES
+            ops.INDEX_CACHE_ENTRIES = 0
+            try:
+                z5 = ops.conv_forward(X, Y, W, tr, tc, tp2, conv.kid)
+                tc.copy_(torch.tensor(g.cols, device="cuda"))
+                g2 = ops.conv_backward(X, Y, W, G, tr, tc, tp, conv.kid)
+            finally:
+                ops.INDEX_CACHE_ENTRIES = monkey_off
+            assert torch.equal(z4, z5) and not torch.equal(z4, z1)
+            assert torch.equal(g1[1], g2[1]) and torch.equal(g1[2], g2[2])
+            assert (g1[0] - g2[0]).abs().max() <= 1e-5 * g2[0].abs().max()
+        finally:
+            ks.conv_index_build = real
+            ops.clear_index_cache()
