@@ -2,12 +2,19 @@
 // and a copy kernel reach, as sequential sweeps and as one 384 KB chunk per block (the shape of the
 // convolution's per-node edge data). bench.py runs this program (built by __graft_entry__.build()) and
 // puts its JSON line into the bench record; profiles/hbm_ceiling.md summarises it.
+//
+// `./hbm_stream accumulate` instead runs three kernels that add 8.6 GB worth of values into a buffer small
+// enough to stay in the L2 caches: float atomics from all blocks on one 512 KB buffer, float atomics with each
+// XCD's blocks on their own 512 KB slice, and plain read-modify-write of 1024 private 16 KB slices. Under
+// rocprofv3 --pmc WRITE_SIZE / FETCH_SIZE they show where such updates are carried out: in the L2 (traffic =
+// the buffer, once) or on the memory side (traffic = every update).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
 #include <cstdio>
 #include <numeric>
 #include <random>
+#include <string>
 #include <vector>
 
 typedef float __attribute__((ext_vector_type(4))) f4;
@@ -56,6 +63,50 @@ __global__ __launch_bounds__(128) void chunks(const f4* __restrict__ a, f4* __re
     if (!WRITE && acc.x + acc.y + acc.z + acc.w == 123.456f) *out = 1.f;
 }
 
+__global__ __launch_bounds__(256) void atomics_shared(float* p, int n_floats, int rounds) {
+    for (int r = 0; r < rounds; ++r)
+        for (int i = threadIdx.x; i < n_floats; i += 256) unsafeAtomicAdd(p + i, 1.0f);
+}
+
+__global__ __launch_bounds__(256) void atomics_per_xcd(float* p, int n_floats, int rounds) {
+    float* q = p + (size_t)(blockIdx.x % 8) * n_floats;  // workgroups go to the XCDs round-robin
+    for (int r = 0; r < rounds; ++r)
+        for (int i = threadIdx.x; i < n_floats; i += 256) unsafeAtomicAdd(q + i, 1.0f);
+}
+
+__global__ __launch_bounds__(256) void rmw_private(float* p, int n_floats, int rounds) {
+    float* q = p + (size_t)blockIdx.x * n_floats;
+    for (int r = 0; r < rounds; ++r)
+        for (int i = threadIdx.x; i < n_floats; i += 256) q[i] += 1.0f;
+}
+
+static int accumulate_modes() {
+    const int n = 128 * 1024;         // 512 KB of floats: the shared buffer, and each of the 8 per-XCD slices
+    const int n_private = 4096;       // 16 KB of floats per block in the third kernel
+    const int blocks = 1024;
+    // the largest footprint of the three kernels: 8 slices of n floats, or one private slice per block
+    const size_t bytes = sizeof(float) * std::max((size_t)8 * n, (size_t)blocks * n_private);
+    float* p = nullptr;
+    CHECK(hipMalloc(&p, bytes));
+    CHECK(hipMemset(p, 0, bytes));
+    hipEvent_t a, b;
+    (void)hipEventCreate(&a);
+    (void)hipEventCreate(&b);
+    const char* names[3] = {"atomics_shared", "atomics_per_xcd", "rmw_private"};
+    for (int mode = 0; mode < 3; ++mode) {
+        (void)hipEventRecord(a);
+        if (mode == 0) atomics_shared<<<blocks, 256>>>(p, n, 16);
+        if (mode == 1) atomics_per_xcd<<<blocks, 256>>>(p, n, 16);
+        if (mode == 2) rmw_private<<<blocks, 256>>>(p, n_private, 512);
+        (void)hipEventRecord(b);
+        (void)hipEventSynchronize(b);
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, a, b);
+        std::printf("%s: %.3f ms for 8.59 GB of updates (%.0f GB/s)\n", names[mode], ms, 8589.9 / ms);
+    }
+    return 0;
+}
+
 template <typename F>
 static float median_ms(F launch, int iters = 7) {
     hipEvent_t a, b;
@@ -78,7 +129,8 @@ static float median_ms(F launch, int iters = 7) {
     return ts[ts.size() / 2];
 }
 
-int main() {
+int main(int argc, char** argv) {
+    if (argc > 1 && std::string(argv[1]) == "accumulate") return accumulate_modes();
     const int n_chunks = 21000, chunk_bytes = 384 * 1024;  // 8.26 GB per buffer
     const int chunk_f4 = chunk_bytes / 16;
     const size_t bytes = (size_t)n_chunks * chunk_bytes, n = bytes / 16;
