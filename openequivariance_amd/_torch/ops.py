@@ -443,7 +443,10 @@ def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows
                             c.data_ptr(), 0, 0, _stream())
         else:
             perm = transpose_perm.contiguous() if e.deterministic else None
-            index, side = _conv_index(ks, nodes, nnz, r, c, perm, False)
+            # the forward walk needs the receiver side only; where the backward pass will want the edges grouped
+            # by sender as well, both are built now, so that one index serves the whole step
+            both = ks.dims["deterministic"] == rt.CONV_GROUPED and ks.dims.get("dx_mode", 0) != rt.DX_ATOMIC
+            index, side = _conv_index(ks, nodes, nnz, r, c, perm, both)
             ks.conv_forward_indexed(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), r.data_ptr(),
                                     c.data_ptr(), index.data_ptr(), index.numel(), side, _stream())
     return out

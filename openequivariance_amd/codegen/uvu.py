@@ -73,6 +73,7 @@ class UvuEmitter:
         # bit 3 = output rows stored / output-gradient rows loaded non-temporally; bit 4 = X rows loaded
         # non-temporally (batch kernels only: the convolution re-reads them).
         self.nt = 0
+        self.mask_loads = False  # zero X and W values in lanes without a channel (see _operand)
         self.sched_fence = False
         self.fence_words = 0  # gradient registers between two scheduling fences (0: a fence after every path)
         self.prefetch_runs = False  # request the next run's gradients and weights while a run computes
@@ -330,6 +331,15 @@ class UvuEmitter:
             return f"oeq_at({rowexpr} + {const}, (unsigned){u} * {stride * self.low.elem_size}u)"
         return f"({rowexpr} + {const} + {u} * {stride})"
 
+    def _gptr(self, rowexpr: str, where, mul: int) -> str:
+        """Pointer through which a lane reads its channel of an output-gradient block. Lanes without a
+        channel are pointed at a row of zeros: every sum across lanes has a factor from the output
+        gradient, so this is what keeps their terms out of it, and the loaded values need no select
+        (a select after each load has made the compiler wait for the loads one by one)."""
+        if self._full(mul):
+            return self._ptr(rowexpr, where, mul)
+        return f"(u < {mul} ? {self._ptr(rowexpr, where)} : (const T*)oeq_zero_row)"
+
     def _full(self, mul: int) -> bool:
         """Every lane's channel index is a channel of such a block (over all chunks, or in the chunk being
         generated)."""
@@ -376,6 +386,18 @@ class UvuEmitter:
         conds = [c for c in (None if self._full(mul) else f"u < {mul}", extra) if c]
         return f"oeq_sel({' && '.join(conds)}, {loaded})" if conds else loaded
 
+    @staticmethod
+    def _guarded(loaded: str, guard: Optional[str]) -> str:
+        return f"oeq_sel({guard}, {loaded})" if guard else loaded
+
+    def _operand(self, mul: int, loaded: str) -> str:
+        """A per-row operand (X or W value) loaded through a clamped pointer. Lanes without a channel
+        read the block's last channel and keep that value: nothing they compute is stored, and every sum
+        across lanes (the gradients with respect to Y) has a factor from the output gradient, which
+        ``_val`` zeroes for them. Leaving the select off the loads lets the compiler issue them back to
+        back; with it, chains of load, wait, select through one register have been seen."""
+        return self._val(mul, loaded) if self.mask_loads else loaded
+
     def _store_cond(self, mul: int, *guards) -> Optional[str]:
         conds = [g for g in guards if g and g != "true"]
         if not self._full(mul):
@@ -416,7 +438,7 @@ class UvuEmitter:
             mul = low.in1[p.i1].mul
             wp = self._ptr("wrow", (f"{p.woff} + ({v})", low.in2[p.i2].mul), mul)
             ld = f"__builtin_nontemporal_load({wp})" if (self.nt & 1) and not low.shared_weights else f"*{wp}"
-            return self._val(mul, ld)
+            return self._operand(mul, ld)
 
         return y, w
 
@@ -554,7 +576,7 @@ class UvuEmitter:
             s(f"const T* xp = {self._ptr(rowexpr, base, blk.mul)};")
             for i in range(blk.d):
                 ld = f"__builtin_nontemporal_load(xp + {i * st})" if self.nt & 16 else f"xp[{i * st}]"
-                s(f"{dst}.b{b}[{i}] = {self._val(blk.mul, ld)};")
+                s(f"{dst}.b{b}[{i}] = {self._operand(blk.mul, ld)};")
             s.close()
 
     def _for_v(self, s: Src, p: Path, body: Callable[[str], None]):
@@ -581,6 +603,11 @@ class UvuEmitter:
         for io in self.used_out:
             s(f"    T o{io}[{low.out[io].d}];")
         s("};")
+        partial = [low.out[io] for io in self.used_out if low.out[io].mul % (self.LPR * self.NCH)]
+        if partial:
+            # what lanes without a channel read in place of an output-gradient block (see _gptr)
+            extent = max((b.d - 1) * self._lane_ptr(b)[1] + 1 for b in partial)
+            s(f"__device__ const T oeq_zero_row[{extent}] = {{}};")
         if self.can_preload and self.q_entries:
             # y: the edge's Y row; yq: the Y values this lane multiplies for the wave's product table
             # (a kernel uses one of the two)
@@ -1109,10 +1136,10 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             bo = low.out[io]
             s.open("")
             base, st = self._lane_ptr(bo)
-            s(f"const T* gp = {self._ptr(rowexpr, base, bo.mul)};")
+            s(f"const T* gp = {self._gptr(rowexpr, base, bo.mul)};")
             for k in range(bo.d):
                 ld = f"__builtin_nontemporal_load(gp + {k * st})" if self.nt & 8 else f"gp[{k * st}]"
-                s(f"{dst}.o{io}[{k}] = {self._val(bo.mul, ld)};")
+                s(f"{dst}.o{io}[{k}] = {ld};")
             s.close()
 
     def _bwd_paths(self, s: Src, *, xname: str, yacc, wacc, g_on_demand_row: Optional[str] = None,
@@ -1148,10 +1175,10 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
                 s(f"T gk{q.index}[{bo_q.d}];")
                 s.open("")
                 base, st = self._lane_ptr(bo_q)
-                s(f"const T* gp = {self._ptr(g_on_demand_row, base, bo_q.mul)};")
+                s(f"const T* gp = {self._gptr(g_on_demand_row, base, bo_q.mul)};")
                 for k in range(bo_q.d):
                     ld = f"__builtin_nontemporal_load(gp + {k * st})" if self.nt & 8 else f"gp[{k * st}]"
-                    s(f"gk{q.index}[{k}] = {self._val(bo_q.mul, ld, g_guard)};")
+                    s(f"gk{q.index}[{k}] = {self._guarded(ld, g_guard)};")
                 s.close()
                 for v in range(low.in2[q.i2].mul):
                     s(f"const T wv{q.index}_{v} = {wacc(q, str(v))};")
@@ -1177,10 +1204,10 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
                 s(f"T gk[{bo.d}];")
                 s.open("")
                 base, st = self._lane_ptr(bo)
-                s(f"const T* gp = {self._ptr(g_on_demand_row, base, bo.mul)};")
+                s(f"const T* gp = {self._gptr(g_on_demand_row, base, bo.mul)};")
                 for k in range(bo.d):
                     ld = f"__builtin_nontemporal_load(gp + {k * st})" if self.nt & 8 else f"gp[{k * st}]"
-                    s(f"gk[{k}] = {self._val(bo.mul, ld, g_guard)};")
+                    s(f"gk[{k}] = {self._guarded(ld, g_guard)};")
                 s.close()
                 gname = lambda k: f"gk[{k}]"
             else:
@@ -1893,9 +1920,10 @@ def tp_module(low: Lowered, compute_units: int = 256):
                     tp_wf=2 if f32 else 0, tp_wb=3 if (big and not pf_ok) else 2, tp_nt=0,
                     tp_gres=0 if on_demand else 1,
                     tp_sb=1 if on_demand else 0, tp_trs=1, tp_fw=64, tp_pf=1,
-                    tp_dd=1, dd_wa=2, dd_wb=2))
+                    tp_dd=1, dd_wa=2, dd_wb=2, tp_mask=0))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
+    em.mask_loads = bool(t["tp_mask"])
     em.sched_fence = bool(t["tp_sb"])
     em.fence_words = t["tp_fw"]
     em.prefetch_runs = bool(t["tp_pf"])
@@ -1945,7 +1973,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=112, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
                     dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fw=0, conv_pf=0,
-                    conv_dxm=-1, conv_q=1, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24))
+                    conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -1996,6 +2024,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                 if need <= 190:
                     break
     em.nt = t["conv_nt"]
+    em.mask_loads = bool(t["tp_mask"])
     q_fwd = q_bwd = False
     if t["conv_q"] and em.q_supported():
         # bit 0: forward, bit 1: backward. Backward gains nothing at the MACE shape (it is bound by its
@@ -2044,8 +2073,12 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             # deterministic=False may use float atomics, and adding the terms straight into the sender
             # rows saves their round trip through scratch memory and the second kernel; the caller-sorted
             # mode promises the same bits on every run and keeps the ordered reduction
-            dx_mode = t["conv_dxm"] if t["conv_dxm"] >= 0 else (em.DX_ATOMIC if mode == rt.CONV_GROUPED
-                                                                  else em.DX_TERMS)
+            # (only where a row fills the wave and the atomics go through the LDS transpose, 64 consecutive
+            # floats per instruction: per-lane atomics of packed or ragged rows are several times slower than
+            # the ordered reduction)
+            coalesced = bool(t["conv_tra"]) and em._regular_wave() and not em.ir_mul
+            dx_mode = t["conv_dxm"] if t["conv_dxm"] >= 0 else (
+                em.DX_ATOMIC if (mode == rt.CONV_GROUPED and coalesced) else em.DX_TERMS)
             if dx_mode == em.DX_ARRIVAL and em.R != 1:
                 dx_mode = em.DX_TERMS
         blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd_b,

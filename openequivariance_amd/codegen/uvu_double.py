@@ -62,7 +62,7 @@ class DoubleEmitter(UvuEmitter):
             mul = low.in1[p.i1].mul
             wp = self._ptr(row, (f"{p.woff} + ({v})", low.in2[p.i2].mul), mul)
             ld = f"__builtin_nontemporal_load({wp})" if self.nt & 1 else f"*{wp}"
-            return self._val(mul, ld)
+            return self._operand(mul, ld)
         return w
 
     def _two_products(self, s: Src, p: Path, v: str) -> Dict[int, Tuple[str, str, bool]]:
@@ -144,9 +144,9 @@ class DoubleEmitter(UvuEmitter):
                 s(f"T gk[{bo.d}];")
                 s.open("")
                 base, st = self._lane_ptr(bo)
-                s(f"const T* gp = {self._ptr(g_on_demand_row, base, bo.mul)};")
+                s(f"const T* gp = {self._gptr(g_on_demand_row, base, bo.mul)};")
                 for k in range(bo.d):
-                    s(f"gk[{k}] = {self._val(bo.mul, f'gp[{k * st}]')};")
+                    s(f"gk[{k}] = gp[{k * st}];")
                 s.close()
                 gname = lambda k: f"gk[{k}]"
             else:
@@ -672,6 +672,7 @@ def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict) -> List[t
 
     em = DoubleEmitter(low, acc_budget_words=64)
     em.nt = base.nt
+    em.mask_loads = base.mask_loads
     em.tr_stores = base.tr_stores
     em.fence_words = 48
     # the accumulator structs of this emitter's (smaller) segments
@@ -692,6 +693,7 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
 
     em = DoubleEmitter(low, acc_budget_words=tune.get("dd_acc", 112))
     em.nt = base.nt
+    em.mask_loads = base.mask_loads
     em.tr_stores = base.tr_stores
     em.fence_words = tune.get("dd_fw", 32)
     em.fence_paths = tune.get("dd_fp", 0)

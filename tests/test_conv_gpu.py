@@ -374,9 +374,10 @@ KNOBS = ["conv_pipe_f=0,conv_pipe_b=1", "conv_pipe_f=1,conv_pipe_b=2", "conv_pip
          "conv_xcd=1,conv_gres=0", "conv_nt=0,conv_acc=48", "conv_sort=0,conv_tra=0", "conv_sort=0,conv_pipe_f=3,conv_nt=0",
          "conv_wf=0,conv_wb=0,conv_gf=1,conv_gb=1",
          # sender gradients: ordered reduction / float atomics / arrival counting; walk order off, 1 and 3 hops;
-         # wave-shared product table off, and on in both directions
-         "conv_dxm=0,conv_hops=0,conv_q=0", "conv_dxm=1,conv_hops=1", "conv_dxm=2,conv_hops=3,conv_q=3",
-         "conv_q=2,conv_qaf=16,conv_qab=200,conv_qpin=0"]
+         # wave-shared product table forward only, backward only and in both directions; lanes without a
+         # channel zeroed after each load
+         "conv_dxm=0,conv_hops=0,conv_q=1", "conv_dxm=1,conv_hops=1", "conv_dxm=2,conv_hops=3,conv_q=3",
+         "conv_q=2,conv_qaf=16,conv_qab=200,conv_qpin=0", "tp_mask=1"]
 
 
 @pytest.mark.parametrize("knobs", KNOBS)
