@@ -25,16 +25,28 @@ from .benchmarking import ConvolutionTiming
 from .utils import compute_units, oeq_to_torch_dtype, torch_to_oeq_dtype
 
 
+def fused(low) -> bool:
+    """Whether the convolution of this problem runs as fused kernels: every 'uvu' problem, and 'uvw'
+    problems with per-edge weights (``OEQ_AMD_TUNE=conv_fuse_uvw=0`` sends those through the unfused path)."""
+    if low.mode == "uvu":
+        return True
+    from ..codegen import uvw
+    from ..codegen.uvu import tuning
+    return uvw.conv_supported(low) and bool(tuning(dict(conv_fuse_uvw=1))["conv_fuse_uvw"])
+
+
 def build_conv_module(problem: TPProblem, deterministic: bool, kahan: bool = False):
     low = lower(problem)
     if low.mode == "uvu":
         from ..codegen import uvu
         return uvu.conv_module(low, deterministic, compute_units(), kahan)
-    # 'uvw': no fused kernel; the batch kernels run on gathered rows and an ordered segment sum (or torch's
-    # index_add_ in atomic mode) scatters the result, like the reference's unfused convolution
-    # (core/ConvolutionBase.py:292-301, _torch/TensorProductConv.py:595-640).
     from .. import runtime as rt
     from ..codegen import uvw
+    if fused(low):
+        return uvw.conv_module(low, deterministic, compute_units(), kahan)
+    # 'uvw' with shared weights: no fused kernel; the batch kernels run on gathered rows and an ordered
+    # segment sum scatters the result, like the reference's unfused convolution
+    # (core/ConvolutionBase.py:292-301, _torch/TensorProductConv.py:595-640).
     cu = compute_units()
     src, dims, descs = uvw.tp_module(low, cu, kahan)
     descs = list(descs) + [(rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, cu * 16),
@@ -86,7 +98,7 @@ class TensorProductConv(ConvolutionTiming, torch.nn.Module):
         entry = ops.KernelEntry(
             lambda p=problem, d=deterministic, k=kahan: build_conv_module(p, d, k), low.L1, low.L2, low.L3, low.WN,
             low.shared_weights, oeq_to_torch_dtype(problem.irrep_dtype), deterministic=deterministic,
-            unfused=low.mode != "uvu",
+            unfused=not fused(low),
         )
         self.kid = ops.register_entry(entry)
         self._dummy_perm = None

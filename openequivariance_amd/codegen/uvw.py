@@ -32,7 +32,7 @@ class UvwEmitter:
     def __init__(self, low: Lowered):
         assert low.mode == "uvw"
         from .uvu import tuning
-        self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576, uvw_regdw=1))
+        self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576, uvw_regdw=1, conv_hops=2, conv_fuse_uvw=1))
         self.TILE_BYTES = self.tune["uvw_tile"]
         self.low = low
         self.T = low.ctype
@@ -66,6 +66,55 @@ class UvwEmitter:
         s("const i64 rowc = live ? row : num_batch - 1;")
 
     # ------------------------------------------------------------- forward
+    def _forward_block(self, s: Src, io: int, acc: str = "acc"):
+        """Adds the contribution of one row (xrow, yrow, wrow) to the channels w = wc + lane of output block
+        ``io``: the CG contraction with lanes = u goes to the wave's LDS tile, the channel mix reads it
+        back as broadcasts with lanes = w."""
+        low = self.low
+        bo = low.out[io]
+        for p in [q for q in low.paths if q.io == io]:
+            b1, b2 = low.in1[p.i1], low.in2[p.i2]
+            s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l}) {b1.mul}x{b2.mul}->{bo.mul}")
+            s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
+            s.open(f"for (int uc = 0; uc < {b1.mul}; uc += 64)")
+            s.open("")
+            s("const int u = uc + lane;")
+            s(f"T x[{b1.d}];")
+            s.open(f"if (u < {b1.mul})")
+            for i in range(b1.d):
+                s(f"x[{i}] = xrow[{b1.off} + u * {b1.d} + {i}];")
+            s.close(" else {")
+            s.level += 1
+            for i in range(b1.d):
+                s(f"x[{i}] = T(0);")
+            s.close()
+            prods = self._products(s, p)
+            started = set()
+            for n, (i, j, k, c) in enumerate(p.nnz):
+                q, neg = prods[n]
+                if k not in started:
+                    s(f"T t{k} = {'-' if neg else ''}{q} * x[{i}];")
+                    started.add(k)
+                else:
+                    s(f"t{k} {'-=' if neg else '+='} {q} * x[{i}];")
+            # the tile is private to the wave (one row per wave): wave-level ordering is enough
+            s("oeq_wave_sync();")
+            for k in range(bo.d):
+                s(f"s_t[wave][{k}][lane] = {'t%d' % k if k in started else 'T(0)'};")
+            s("oeq_wave_sync();")
+            s.close()
+            s(f"const int nu = ({b1.mul} - uc < 64) ? {b1.mul} - uc : 64;")
+            s(f"const T* wp = wrow + {p.woff} + ((i64)uc * {b2.mul} + v) * {bo.mul} + w;")
+            s.open(f"if (w < {bo.mul})")
+            s.open("for (int uu = 0; uu < nu; ++uu)")
+            s(f"const T wv = wp[(i64)uu * {b2.mul * bo.mul}];")
+            for k in range(bo.d):
+                s(f"{acc}[{k}] += wv * s_t[wave][{k}][uu];")
+            s.close()
+            s.close()
+            s.close()
+            s.close()
+
     def emit_forward(self, s: Src):
         low = self.low
         block = 64 * WAVES_PER_BLOCK
@@ -80,55 +129,13 @@ class UvwEmitter:
         s(f"const T* wrow = W{'' if low.shared_weights else f' + rowc * {low.WN}'};")
         s(f"T* zrow = L3_out + rowc * {low.L3};")
         for io, bo in enumerate(low.out):
-            paths = [p for p in low.paths if p.io == io]
             s(f"// ---- out[{io}]: {bo.mul} x l={bo.l}")
             s.open(f"for (int wc = 0; wc < {bo.mul}; wc += 64)")
             s("const int w = wc + lane;")
             s(f"T acc[{bo.d}];")
             for k in range(bo.d):
                 s(f"acc[{k}] = T(0);")
-            for p in paths:
-                b1, b2 = low.in1[p.i1], low.in2[p.i2]
-                s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l}) {b1.mul}x{b2.mul}->{bo.mul}")
-                s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
-                s.open(f"for (int uc = 0; uc < {b1.mul}; uc += 64)")
-                s.open("")
-                s("const int u = uc + lane;")
-                s(f"T x[{b1.d}];")
-                s.open(f"if (u < {b1.mul})")
-                for i in range(b1.d):
-                    s(f"x[{i}] = xrow[{b1.off} + u * {b1.d} + {i}];")
-                s.close(" else {")
-                s.level += 1
-                for i in range(b1.d):
-                    s(f"x[{i}] = T(0);")
-                s.close()
-                prods = self._products(s, p)
-                started = set()
-                for n, (i, j, k, c) in enumerate(p.nnz):
-                    q, neg = prods[n]
-                    if k not in started:
-                        s(f"T t{k} = {'-' if neg else ''}{q} * x[{i}];")
-                        started.add(k)
-                    else:
-                        s(f"t{k} {'-=' if neg else '+='} {q} * x[{i}];")
-                # the tile is private to the wave (one row per wave): wave-level ordering is enough
-                s("oeq_wave_sync();")
-                for k in range(bo.d):
-                    s(f"s_t[wave][{k}][lane] = {'t%d' % k if k in started else 'T(0)'};")
-                s("oeq_wave_sync();")
-                s.close()
-                s(f"const int nu = ({b1.mul} - uc < 64) ? {b1.mul} - uc : 64;")
-                s(f"const T* wp = wrow + {p.woff} + ((i64)uc * {b2.mul} + v) * {bo.mul} + w;")
-                s.open(f"if (w < {bo.mul})")
-                s.open("for (int uu = 0; uu < nu; ++uu)")
-                s(f"const T wv = wp[(i64)uu * {b2.mul * bo.mul}];")
-                for k in range(bo.d):
-                    s(f"acc[{k}] += wv * s_t[wave][{k}][uu];")
-                s.close()
-                s.close()
-                s.close()
-                s.close()
+            self._forward_block(s, io)
             s.open(f"if (live && w < {bo.mul})")
             for k in range(bo.d):
                 s(f"zrow[{bo.off} + w * {bo.d} + {k}] = acc[{k}];")
@@ -137,6 +144,83 @@ class UvwEmitter:
         s.close()
         s.close()
         return block
+
+    def emit_conv_forward(self, s: Src, kahan: bool = False):
+        """Fused convolution, forward: the waves of a block share a receiver node's output segments (64
+        channels of one output block each, lanes = w) and each keeps its segments in registers over the
+        node's edges, whose senders' rows, Y rows and weight rows it reads in place: no gathered copy of X
+        and no per-edge message tensor. The nodes are taken in the walk order of the index, the edges of a
+        node in list order (so the sums do not depend on scheduling); with ``kahan`` each edge's message is
+        added with a compensation term. Returns (block size, nodes per block)."""
+        low = self.low
+        assert not low.shared_weights
+        segs = [(io, wc) for io, bo in enumerate(low.out) for wc in range(0, bo.mul, 64)
+                if any(p.io == io for p in low.paths)]
+        empty = [io for io in range(len(low.out)) if not any(p.io == io for p in low.paths)]
+        wpn = max(1, min(WAVES_PER_BLOCK, len(segs)))  # waves per node
+        G = WAVES_PER_BLOCK // wpn
+        block = 64 * wpn * G
+        s.open(
+            f'extern "C" __global__ __launch_bounds__({block}) void forward(i64 node_count, i64 nnz, '
+            "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
+            "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
+            "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order)"
+        )
+        s(f"__shared__ T s_t[{wpn * G}][{self.max_d3}][64];")
+        s("const int lane = oeq_lane();")
+        s("const int wave = oeq_wave();")
+        s(f"const int g = wave / {wpn}, sg = wave % {wpn};")
+        s.open(f"for (i64 base = (i64)blockIdx.x * {G}; base < node_count; base += (i64)gridDim.x * {G})")
+        s("const i64 vnode = base + g;")
+        s("const bool live = vnode < node_count;")
+        s("const i64 vc = live ? vnode : node_count - 1;")
+        s("const i64 node = order ? oeq_idx(order[vc], node_count) : vc;")
+        s("const i64 e0 = oeq_pos(rowptr[node], nnz);")
+        s("const i64 e1 = live ? oeq_pos(rowptr[node + 1], nnz) : e0;")
+        s(f"T* zrow = L3_out + node * {low.L3};")
+        for io in empty:
+            # an output block no path writes: zeros
+            bo = low.out[io]
+            s.open("if (live && sg == 0)")
+            s(f"for (int t = lane; t < {bo.mul * bo.d}; t += 64) zrow[{bo.off} + t] = T(0);")
+            s.close()
+        for si, (io, wc) in enumerate(segs):
+            bo = low.out[io]
+            s(f"// ---- out[{io}]: {bo.mul} x l={bo.l}, channels {wc}..")
+            s.open(f"if (sg == {si % wpn})")
+            s(f"const int wc = {wc};")
+            s("const int w = wc + lane;")
+            s(f"T acc[{bo.d}];")
+            for k in range(bo.d):
+                s(f"acc[{k}] = T(0);")
+            if kahan:
+                s(f"T comp[{bo.d}];")
+                for k in range(bo.d):
+                    s(f"comp[{k}] = T(0);")
+            s.open("for (i64 pos = e0; pos < e1; ++pos)")
+            s("const i64 e = oeq_idx(OEQ_EDGE(pos), nnz);")
+            s(f"const T* xrow = L1_in + oeq_idx(cols[e], node_count) * {low.L1};")
+            s(f"const T* yrow = L2_in + e * {low.L2};")
+            s(f"const T* wrow = W + e * {low.WN};")
+            if kahan:
+                s(f"T msg[{bo.d}];")
+                for k in range(bo.d):
+                    s(f"msg[{k}] = T(0);")
+                self._forward_block(s, io, "msg")
+                for k in range(bo.d):
+                    s(f"{{ const T y = msg[{k}] - comp[{k}]; const T t = acc[{k}] + y; "
+                      f"comp[{k}] = (t - acc[{k}]) - y; acc[{k}] = t; }}")
+            else:
+                self._forward_block(s, io)
+            s.close()
+            s.open(f"if (live && w < {bo.mul})")
+            for k in range(bo.d):
+                s(f"zrow[{bo.off} + w * {bo.d} + {k}] = acc[{k}];")
+            s.close()
+            s.close()
+        s.close()
+        s.close()
+        return block, G
 
     # ------------------------------------------------------------ backward
     # TILE_BYTES (set from the uvw_tile knob): per-wave LDS budget for one path's weight tile; larger
@@ -164,9 +248,14 @@ class UvwEmitter:
                                            (min(64, b1.mul - uc) * per_u) % vw == 0 for uc in chunk_starts)
         return elems, (vw if aligned else 1)
 
-    def emit_backward(self, s: Src):
+    def emit_backward(self, s: Src, conv: bool = False):
+        """``conv``: the fused convolution's backward. An edge is a row: X comes from the sender's row,
+        the output gradient from the receiver's, the X gradient goes to the edge's row of ``dx_tmp``
+        (summed per sender, in the order of the sender-major list, by ``fixup_backward``); per-row
+        weights only. The edges need no order here, so the kernel strides over the edge list as it is."""
         low = self.low
         shared = low.shared_weights
+        assert not (conv and shared)
         plans = {p.index: self._tile_plan(p) for p in low.paths}
         tiled = [p for p in low.paths if plans[p.index]]
         waves = WAVES_PER_BLOCK
@@ -207,12 +296,24 @@ class UvwEmitter:
         # register-resident weight gradients: left to one wave per SIMD with up to 512 registers (e3tools
         # transformer block: 0.29 ms against 0.57 ms with spills at 256; uvw_regdw=2 selects the latter)
         attr = " __attribute__((amdgpu_waves_per_eu(2, 2)))" if (self.reg_dw and self.tune["uvw_regdw"] == 2) else ""
-        s.open(
-            f'extern "C" __global__ __launch_bounds__({block}){attr} void backward(i64 num_batch, '
-            "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
-            "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
-            "const T* __restrict__ L3_grad, T* __restrict__ wpartial)"
-        )
+        if conv:
+            s.open(
+                f'extern "C" __global__ __launch_bounds__({block}){attr} void backward(i64 node_count, i64 nnz, '
+                "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
+                "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
+                "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
+                "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
+                "T* __restrict__ wpartial, const i64* __restrict__ colptr, const i64* __restrict__ sperm, "
+                "int* __restrict__ arrivals, const i64* __restrict__ order)"
+            )
+            s("const i64 num_batch = nnz;")
+        else:
+            s.open(
+                f'extern "C" __global__ __launch_bounds__({block}){attr} void backward(i64 num_batch, '
+                "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
+                "T* __restrict__ L2_grad, const T* __restrict__ W, T* __restrict__ W_grad, "
+                "const T* __restrict__ L3_grad, T* __restrict__ wpartial)"
+            )
         if tiled:
             # one path's weights of the row, then (in place) its weight gradients
             s(f"__shared__ __attribute__((aligned(16))) T s_w[{waves}][{tile_elems}];")
@@ -239,11 +340,16 @@ class UvwEmitter:
             nv_max = max(self._pad_vectors(st[2], st[1] * 64, plans[st[2].index][1]) for st in steps0)
             s(f"wvec_t pf[{nv_max}];  // the next weight tile on its way from global memory to LDS")
         self._row_loop_open(s, waves)
-        s(f"const T* xrow = L1_in + rowc * {low.L1};")
+        if conv:
+            s(f"const T* xrow = L1_in + oeq_idx(cols[rowc], node_count) * {low.L1};")
+            s(f"const T* grow = L3_grad + oeq_idx(rows[rowc], node_count) * {low.L3};")
+            s(f"T* dxrow = dx_tmp + rowc * {low.L1};")
+        else:
+            s(f"const T* xrow = L1_in + rowc * {low.L1};")
+            s(f"const T* grow = L3_grad + rowc * {low.L3};")
+            s(f"T* dxrow = L1_grad + rowc * {low.L1};")
         s(f"const T* yrow = L2_in + rowc * {low.L2};")
         s(f"const T* wrow = W{'' if shared else f' + rowc * {low.WN}'};")
-        s(f"const T* grow = L3_grad + rowc * {low.L3};")
-        s(f"T* dxrow = L1_grad + rowc * {low.L1};")
         if not shared:
             s(f"T* dwrow = W_grad + rowc * {low.WN};")
         s(f"T dy[{self.l2_pad}];")
@@ -623,6 +729,51 @@ class UvwEmitter:
             s.close()
         s.close()
         s.close()
+
+
+def conv_supported(low: Lowered) -> bool:
+    """Problems the fused 'uvw' convolution kernels cover: per-row (per-edge) weights."""
+    return low.mode == "uvw" and not low.shared_weights
+
+
+def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kahan: bool = False):
+    """Source + launch descriptors of the fused 'uvw' convolution (per-edge weights; replaces the
+    reference's 'uvw' branch inside its convolution templates, templates/loop_unroll_conv_atomic.cuh:52-180
+    and loop_unroll_conv_det.cuh:187-293). Same kernel roles, argument lists and index as the 'uvu'
+    convolution: a receiver walk for the forward pass, per-edge gradients plus the ordered sender-side
+    sum for the backward pass. ``deterministic``: the caller brings receiver-sorted edges and the
+    sender-major permutation; otherwise the library groups the edge ids on the device first."""
+    from .. import runtime as rt
+    from .common import fixup_backward_kernel
+
+    assert conv_supported(low)
+    em = UvwEmitter(low)
+    s = Src()
+    s(prelude(low.ctype))
+    s(utility_kernels(kahan))
+    s("#define OEQ_EDGE(j) (eperm ? eperm[(j)] : (j))")
+    blk_f, G_f = em.emit_conv_forward(s, kahan)
+    blk_b = em.emit_backward(s, conv=True)
+    s(fixup_backward_kernel(low.L1, kahan, True))
+    cu = compute_units
+    descs = [
+        (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, cu * 16),
+        (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, cu * 16),
+        (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f, cu * 32),
+        # strides over the edges: the grid need not follow the node count it is derived from
+        (rt.ROLE_CONV_BACKWARD, "backward", blk_b, 1, cu * 16),
+        (rt.ROLE_CONV_FIXUP_BACKWARD, "fixup_backward", 256, 1, 0),
+        (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, cu * 16),
+        (rt.ROLE_GROUP_SCAN, "oeq_group_scan", 1024, 1, 1),
+        (rt.ROLE_GROUP_SCATTER, "oeq_group_scatter", 256, 256 * 4, cu * 16),
+        (rt.ROLE_GROUP_ORDER, "oeq_group_order", 256, 4, cu * 32),
+        (rt.ROLE_ORDER_HOP, "oeq_order_hop", 256, 256, cu * 16),
+    ]
+    t = em.tune
+    dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
+                shared_weights=0, deterministic=rt.CONV_SORTED if deterministic else rt.CONV_GROUPED,
+                wpartial_per_block=0, dx_mode=rt.DX_TERMS, n_chunks=1, order_hops=max(0, t["conv_hops"]))
+    return s.text(), dims, descs
 
 
 def tp_module(low: Lowered, compute_units: int = 256, kahan: bool = False):

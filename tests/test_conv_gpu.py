@@ -43,6 +43,12 @@ def _fc(shared):
                                      internal_weights=False, label="fc-uvw")
 
 
+def _as_f64(problem):
+    out = problem.clone()
+    out.irrep_dtype = out.weight_dtype = np.float64
+    return out
+
+
 CASES = [
     ("cfg1", P.config1_single_uvu, 40, 6),
     ("cfg2", P.config2_nequip_uvu, 60, 8),
@@ -51,8 +57,12 @@ CASES = [
     ("mace-large", lambda: P.mace_problems()[0], 40, 6),
     ("odd", lambda: _odd(False), 40, 6),
     ("odd-shared", lambda: _odd(True), 40, 6),
-    # 'uvw' problems: no fused kernel, batch kernels on gathered rows + ordered segment sum / index_add_
+    # 'uvw' problems with per-edge weights: fused kernels (receiver walk forward, per-edge backward + ordered
+    # sender-side sum); with shared weights: batch kernels on gathered rows + ordered segment sum
     ("uvw", lambda: _fc(False), 40, 6),
+    ("uvw-diffdock", lambda: P.diffdock_problems()[0], 40, 6),
+    ("uvw-diffdock-f64", lambda: _as_f64(P.diffdock_problems()[1]), 30, 5),
+    ("uvw-e3tools-conv", lambda: P.e3tools_problems()[0], 40, 6),
     ("uvw-shared", lambda: _fc(True), 40, 6),
     ("uvw-cfg4-mfma", P.config4_uvw_shared, 30, 5),
     # output gradient too large for one wave: forward shares the output segments, backward the output
@@ -96,6 +106,44 @@ def test_conv_matches_oracle(name, make, n_nodes, deg):
         assert err(tX.grad, dx_ref) <= tol, (name, det)
         assert err(tY.grad, dy_ref[order]) <= tol, (name, det)
         assert err(tW.grad, dw_ref if problem.shared_weights else dw_ref[order]) <= tol, (name, det)
+
+
+def test_uvw_fused_matches_unfused(monkeypatch):
+    """'uvw' with per-edge weights runs as fused kernels; the unfused path (gathered rows, batch kernels,
+    segment sums) stays selectable. Both agree, in both modes, and the fused deterministic mode gives the
+    same bits on every run."""
+    from openequivariance_amd._torch import ops
+    problem = P.diffdock_problems()[0]
+    coords, rows, cols = _graph(200, 10, seed=4)
+    g = CoordGraph(coords, rows, cols)
+    E = g.nnz
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    X = torch.randn(200, problem.irreps_in1.dim, device="cuda", generator=gen)
+    Y = torch.randn(E, problem.irreps_in2.dim, device="cuda", generator=gen)
+    W = torch.randn(E, problem.weight_numel, device="cuda", generator=gen)
+    G = torch.randn(200, problem.irreps_out.dim, device="cuda", generator=gen)
+    tr, tc, tp = (torch.tensor(a, device="cuda") for a in (g.rows, g.cols, g.transpose_perm))
+    out = {}
+    for fuse in (1, 0):
+        monkeypatch.setenv("OEQ_AMD_TUNE", f"conv_fuse_uvw={fuse}")
+        for det in (True, False):
+            conv = oeq.TensorProductConv(problem, deterministic=det)
+            e = ops.get_entry(conv.kid)
+            assert e.unfused == (fuse == 0)
+            runs = []
+            for _ in range(3):
+                z = ops.conv_forward(X, Y, W, tr, tc, tp, conv.kid)
+                runs.append((z,) + tuple(ops.conv_backward(X, Y, W, G, tr, tc, tp, conv.kid)))
+            for later in runs[1:]:
+                for a, b in zip(runs[0], later):
+                    assert torch.equal(a, b), (fuse, det)
+            out[(fuse, det)] = runs[0]
+    for det in (True, False):
+        for a, b in zip(out[(1, det)], out[(0, det)]):
+            assert (a - b).abs().max() <= 2e-6 * b.abs().max(), det
+    # the grouped mode orders a node's edges by edge id, which is the order of the sorted list here
+    for a, b in zip(out[(1, True)], out[(1, False)]):
+        assert torch.equal(a, b)
 
 
 def test_reference_toy_graph():
