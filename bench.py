@@ -178,6 +178,66 @@ def tp_config_table(dev, only=None):
     return table
 
 
+def uvw_conv_table(dev, nodes=12000):
+    """Side measurement: the fused 'uvw' convolution with per-edge weights (DiffDock, e3tools) on a graph of
+    the headline's density, forward and backward, beside the unfused path (gathered rows, batch kernels,
+    segment sums) that it replaces. Bytes = every operand once (W and dW dominate: 27-30 KB per edge)."""
+    import numpy as np
+    import torch
+
+    import openequivariance_amd as oeq
+    from openequivariance_amd._torch import ops
+    from openequivariance_amd.codegen.lower import lower
+    from openequivariance_amd.core import problems as P
+    from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
+
+    coords, rows, cols, _vec = periodic_radius_graph(nodes, 32.0 * (nodes / 50000) ** (1 / 3), 5.0, 0)
+    g = CoordGraph(coords, rows, cols)
+    E = g.nnz
+    tr, tc, tp = (torch.tensor(a, device=dev) for a in (g.rows, g.cols, g.transpose_perm))
+
+    def med(fn, warm=2, it=7):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(it):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b))
+        return float(np.median(ts))
+
+    table = []
+    saved = os.environ.get("OEQ_AMD_TUNE")
+    try:
+        for prob in (P.diffdock_problems()[0], P.e3tools_problems()[0]):
+            low = lower(prob)
+            X, Y = torch.randn(nodes, low.L1, device=dev), torch.randn(E, low.L2, device=dev)
+            W, G = torch.randn(E, low.WN, device=dev), torch.randn(nodes, low.L3, device=dev)
+            fb = 4 * (E * (low.WN + low.L2 + low.L1) + nodes * low.L3)
+            bb = 4 * (E * (2 * low.WN + 2 * low.L2 + low.L1) + nodes * (low.L3 + low.L1))
+            row = {"config": prob.label, "nodes": nodes, "edges": E, "mode": "deterministic"}
+            for key, fuse in (("fused", 1), ("unfused", 0)):
+                os.environ["OEQ_AMD_TUNE"] = ((saved + ",") if saved else "") + f"conv_fuse_uvw={fuse}"
+                kid = oeq.TensorProductConv(prob, deterministic=True).kid
+                tf = med(lambda: ops.conv_forward(X, Y, W, tr, tc, tp, kid))
+                tb = med(lambda: ops.conv_backward(X, Y, W, G, tr, tc, tp, kid))
+                row[key] = {"fwd_ms": tf, "bwd_ms": tb, "fwd_hbm_frac": fb / tf / 1e6 / HBM_PEAK_GBS,
+                            "bwd_hbm_frac": bb / tb / 1e6 / HBM_PEAK_GBS}
+            table.append(row)
+            del X, Y, W, G
+            torch.cuda.empty_cache()
+    finally:
+        if saved is None:
+            os.environ.pop("OEQ_AMD_TUNE", None)
+        else:
+            os.environ["OEQ_AMD_TUNE"] = saved
+    return table
+
+
 def hbm_ceilings():
     """Read-only / write-only / copy stream rates of this GPU (./hbm_stream, built by __graft_entry__.build())."""
     import subprocess
@@ -422,6 +482,7 @@ def main():
         del X, W, G, Y
         torch.cuda.empty_cache()
         extras["tp_configs"] = tp_config_table(dev)
+        extras["uvw_conv"] = uvw_conv_table(dev)
 
     traffic_path = os.path.join(ROOT, "profiles", "conv_cfg5_traffic.json")
     if os.path.exists(traffic_path):
