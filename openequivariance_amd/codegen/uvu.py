@@ -1941,7 +1941,7 @@ def tp_module(low: Lowered, compute_units: int = 256):
         (rt.ROLE_TP_FORWARD, "forward", blk_f, G_f * em.R, 0),
         (rt.ROLE_TP_BACKWARD, "backward", blk_b, G_b * em.R, max_blocks_b if low.shared_weights else 0),
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
-        (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0),
+        (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 64, 0),
     ]
     from . import uvu_double
     if t["tp_dd"] and uvu_double.supported(low):
@@ -2096,7 +2096,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             (rt.ROLE_CONV_FIXUP_BACKWARD, "fixup_backward", 256, 1, 0),
         ]
         if low.shared_weights:
-            descs.append((rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0))
+            descs.append((rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 64, 0))
         from . import uvu_double
         if t["conv_dd"] and uvu_double.supported(low, conv=True) and not kahan:
             descs += uvu_double.add_conv_kernels(s, low, em, t, xcd)

@@ -796,7 +796,7 @@ def tp_module(low: Lowered, compute_units: int = 256, kahan: bool = False):
         (rt.ROLE_TP_BACKWARD, "backward", blk_b, em.backward_waves,
          max_blocks_b if low.shared_weights else compute_units * 16),
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
-        (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0),
+        (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 64, 0),
     ]
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
                 shared_weights=int(low.shared_weights), deterministic=0,

@@ -70,13 +70,14 @@ class MfmaEmitter:
         self.low = low
         self.max_d3 = max(low.out[p.io].d for p in low.paths)
         self.max_d1 = max(low.in1[p.i1].d for p in low.paths)
-        self.gstride = low.L3 + 1
-        while self.gstride % 32 != 1:
-            self.gstride += 1
+        # Row stride of the dZ tile in LDS: 4 mod 32 words. Rows then start on 16-byte boundaries (the tile is
+        # filled with 16-byte stores), and the 32 lanes of a half-wave that read one column of 16 rows, at two
+        # k-steps d words apart (d odd), fall into 32 different banks.
+        self.gstride = self._tile_stride(low.L3)
         # order in which the forward / dW sweeps visit the paths: grouped by output block
         self.fwd_order: List[Path] = [p for io in range(len(low.out)) for p in low.paths if p.io == io]
         from .uvu import tuning
-        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2))
+        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2, uvw_pipe=1, uvw_regs=300, uvw_dma=0))
 
     def lit(self, v):
         return float_literal(v, "float")
@@ -144,37 +145,63 @@ class MfmaEmitter:
         s(f"s_y[r][c] = (row0 + r < num_batch) ? L2_in[(row0 + r) * {low.L2} + c] : T(0);")
         s.close()
 
-    def _stage_g(self, s: Src, col0: int = 0, ncols: int = None):
+    @staticmethod
+    def _tile_stride(ncols: int) -> int:
+        """Row stride (words) of an LDS tile with ncols columns: 4 mod 32 when rows can start on 16-byte
+        boundaries (see ``gstride``), else 1 mod 32."""
+        want = 4 if ncols % 4 == 0 else 1
+        stride = ncols + want
+        while stride % 32 != want:
+            stride += 1
+        return stride
+
+    def _stage_g(self, s: Src, col0: int = 0, ncols: int = None, local: bool = False):
         """dZ tile (columns col0 .. col0+ncols) -> LDS, rows past the batch zeroed. All loads of a
-        thread are issued before the first LDS store, so their latencies overlap."""
+        thread are issued before the first LDS store, so their latencies overlap. ``local``: s_g holds
+        only those columns (column c of the row at index c - col0)."""
         low = self.low
         ncols = low.L3 if ncols is None else ncols
+        dst0 = 0 if local else col0
         nthreads = 64 * WAVES
         if low.L3 % 4 == 0 and col0 % 4 == 0 and ncols % 4 == 0:
-            nvec = RT * ncols // 4
-            iters = (nvec + nthreads - 1) // nthreads
+            # each wave moves its 4 rows, 64 lanes x 16 bytes at a time: every address is affine in the lane id
+            rpw, nc4 = RT // WAVES, ncols // 4
+            J = (nc4 + 63) // 64
             s.open("")
-            s(f"float4 gv[{iters}];")
-            s("#pragma unroll")
-            s.open(f"for (int it = 0; it < {iters}; ++it)")
-            s(f"const int t = tid + it * {nthreads};")
-            s(f"const int r = t / {ncols // 4}, c = {col0} + (t % {ncols // 4}) * 4;")
-            s(f"gv[it] = (t < {nvec} && row0 + r < num_batch) ? "
-              f"*(const float4*)(L3_grad + (row0 + r) * {low.L3} + c) : make_float4(0.f, 0.f, 0.f, 0.f);")
-            s.close()
-            s("#pragma unroll")
-            s.open(f"for (int it = 0; it < {iters}; ++it)")
-            s(f"const int t = tid + it * {nthreads};")
-            s(f"const int r = t / {ncols // 4}, c = {col0} + (t % {ncols // 4}) * 4;")
-            s.open(f"if (t < {nvec})")
-            s("s_g[r][c] = gv[it].x; s_g[r][c + 1] = gv[it].y; s_g[r][c + 2] = gv[it].z; s_g[r][c + 3] = gv[it].w;")
-            s.close()
-            s.close()
+            s(f"float4 gv[{rpw * J}];")
+            for phase in ("load", "store"):
+                for rr in range(rpw):
+                    for j in range(J):
+                        part = (j + 1) * 64 > nc4
+                        c4 = f"(lane + {64 * j})"
+                        r = f"(wave * {rpw} + {rr})"
+                        if phase == "load":
+                            cond = f"row0 + {r} < num_batch" + (f" && {c4} < {nc4}" if part else "")
+                            s(f"gv[{rr * J + j}] = ({cond}) ? *(const float4*)(L3_grad + (row0 + {r}) * {low.L3} + "
+                              f"{col0} + 4 * {c4}) : make_float4(0.f, 0.f, 0.f, 0.f);")
+                        else:
+                            guard = f"if ({c4} < {nc4}) " if part else ""
+                            s(f"{guard}*(float4*)&s_g[{r}][{dst0} + 4 * {c4}] = gv[{rr * J + j}];")
             s.close()
         else:
             s.open(f"for (int t = tid; t < {RT * ncols}; t += {nthreads})")
-            s(f"const int r = t / {ncols}, c = {col0} + t % {ncols};")
-            s(f"s_g[r][c] = (row0 + r < num_batch) ? L3_grad[(row0 + r) * {low.L3} + c] : T(0);")
+            s(f"const int r = t / {ncols}, c = t % {ncols};")
+            s(f"s_g[r][{dst0} + c] = (row0 + r < num_batch) ? L3_grad[(row0 + r) * {low.L3} + {col0} + c] : T(0);")
+            s.close()
+
+    def _dma_g(self, s: Src, tile: str, buf: str):
+        """Request the dZ rows of a tile into s_g[buf] with direct global->LDS loads (each wave its 4 rows,
+        64 lanes x 16 bytes per instruction, landing side by side in LDS). Rows past the end of the batch
+        repeat the last row: what is computed from them is never stored."""
+        low = self.low
+        rpw, nc4 = RT // WAVES, low.L3 // 4
+        for rr in range(rpw):
+            s.open("")
+            s(f"i64 grow = {tile} * {RT} + wave * {rpw} + {rr}; if (grow >= num_batch) grow = num_batch - 1;")
+            for j in range((nc4 + 63) // 64):
+                guard = f"if (lane + {64 * j} < {nc4}) " if (j + 1) * 64 > nc4 else ""
+                s(f"{guard}__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(L3_grad + grow * {low.L3} + 4 * (lane + {64 * j})), "
+                  f"(OEQ_LPTR)(&s_g[{buf}][wave * {rpw} + {rr}][{256 * j}]), 16, 0, 0);")
             s.close()
 
     def _load_x_rows(self, s: Src, dst: str, p: Path):
@@ -197,6 +224,130 @@ class MfmaEmitter:
         s(f"cg_fwd{p.index}({xsrc}[rr], s_y[r], t);")
         for k in range(bo.d):
             s(f"s_T[{buf}][{k}][lane][r] = t[{k}];")
+        s.close()
+
+    def _dx_paths(self, s: Src, paths: List[Path]):
+        """G = dZ W^T of every path on the matrix cores, then the CG part on the vector ALU (in scope:
+        x, dx, dy, s_g, s_y, wreg<path>). ``uvw_pipe`` = 0: path after path, operand order left to the
+        compiler. 1: the A operands (dZ values from LDS) are fetched one chunk of 4 k-steps ahead of the
+        multiplies that use them, and nothing moves across a chunk boundary: without that the compiler
+        hoists the LDS reads of several paths, runs out of registers and spills the weight slices. 2: as 1,
+        and the CG part of the previous path (one of its four rows per chunk) sits between the multiplies of
+        the current one, so that the vector ALU works while the matrix core does."""
+        low = self.low
+        pipe = self.tune["uvw_pipe"]
+        CH = 4
+        if pipe == 0:
+            for p in paths:
+                bo = low.out[p.io]
+                s(f"// path {p.index}")
+                s.open("")
+                # G[k] = sum_w dZ[(r,k), w] * W[u, w]   (A = dZ tile, B = W^T slice in registers)
+                s(f"v4f G[{bo.d}];")
+                for k in range(bo.d):
+                    s(f"G[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+                s("#pragma unroll")
+                s.open("for (int st = 0; st < 16; ++st)")
+                for k in range(bo.d):
+                    s(f"G[{k}] = {MFMA}({self.g_at('l16', f'{bo.off} + (4 * st + lq) * {bo.d} + {k}')}, wreg{p.index}[st], G[{k}], 0, 0, 0);")
+                s.close()
+                s("#pragma unroll")
+                s.open("for (int i = 0; i < 4; ++i)")
+                s(f"T Gk[{bo.d}];")
+                for k in range(bo.d):
+                    s(f"Gk[{k}] = G[{k}][i];")
+                s(f"cg_bwd{p.index}(x[i], s_y[4 * lq + i], Gk, dx[i], dy[i]);")
+                s.close()
+                s.close()
+            return
+        maxd = max(low.out[p.io].d for p in paths)
+        s(f"T opa[{CH * maxd}], opb[{CH * maxd}];  // A operands of the current and the next chunk")
+        if self.lds_w:
+            s(f"T wla[{CH}], wlb[{CH}];  // B operands of a path whose weight slice is kept in LDS")
+        s(f"v4f Ga[{maxd}], Gb[{maxd}];")
+        segs = [(n, c) for n in range(len(paths)) for c in range(16 // CH)]
+
+        def reads(seg, buf):
+            n, c = seg
+            bo = low.out[paths[n].io]
+            for q in range(CH):
+                for k in range(bo.d):
+                    s(f"{buf}[{q * bo.d + k}] = {self.g_at('l16', f'{bo.off} + ({4 * (c * CH + q)} + lq) * {bo.d} + {k}')};")
+            if paths[n].index in self.lds_w:
+                slot = self.lds_w.index(paths[n].index)
+                for q in range(CH):
+                    s(f"{'wla' if buf == 'opa' else 'wlb'}[{q}] = s_wl[{slot}][{c * CH + q}][tid];")
+
+        def cg_row(n, i):
+            p = paths[n]
+            bo = low.out[p.io]
+            G = "Ga" if n % 2 == 0 else "Gb"
+            s.open("")
+            s(f"T Gk[{bo.d}];")
+            for k in range(bo.d):
+                s(f"Gk[{k}] = {G}[{k}][{i}];")
+            s(f"cg_bwd{p.index}(x[{i}], s_y[4 * lq + {i}], Gk, dx[{i}], dy[{i}]);")
+            s.close()
+
+        reads(segs[0], "opa")
+        for t, (n, c) in enumerate(segs):
+            p = paths[n]
+            bo = low.out[p.io]
+            cur, nxt = ("opa", "opb") if t % 2 == 0 else ("opb", "opa")
+            G = "Ga" if n % 2 == 0 else "Gb"
+            if c == 0:
+                s(f"// path {p.index}")
+                for k in range(bo.d):
+                    s(f"{G}[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+            if t + 1 < len(segs):
+                reads(segs[t + 1], nxt)
+            for q in range(CH):
+                wop = (f"{'wla' if cur == 'opa' else 'wlb'}[{q}]" if p.index in self.lds_w
+                       else f"wreg{p.index}[{c * CH + q}]")
+                for k in range(bo.d):
+                    s(f"{G}[{k}] = {MFMA}({cur}[{q * bo.d + k}], {wop}, {G}[{k}], 0, 0, 0);")
+            if pipe >= 2 and n > 0:
+                cg_row(n - 1, c)
+            if pipe == 3 and n > 0:
+                # one multiply, then its share of the vector instructions of the row's CG part
+                valu = max(1, int(3.4 * len(paths[n - 1].nnz)) // (CH * bo.d))
+                for _ in range(CH * bo.d):
+                    s("__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);")
+                    s(f"__builtin_amdgcn_sched_group_barrier(0x002, {valu}, 0);")
+            s("__builtin_amdgcn_sched_barrier(0);")
+            if pipe == 1 and c == 16 // CH - 1:
+                for i in range(4):
+                    cg_row(n, i)
+        if pipe >= 2:
+            for i in range(4):
+                cg_row(len(paths) - 1, i)
+
+    def _reduce_dy(self, s: Src):
+        """Sum of dy[i][j] (4 rows x L2 values per lane) over the 16 lanes of a lane group, into
+        s_dy[wave][row][j]. Each step pairs every lane with one partner through a DPP lane permutation
+        (mirror of the 16, mirror of each 8, mirror of each quad, neighbour); a lane keeps one half of its
+        values and adds the partner's copies of that half, so the count of values halves with the count of
+        lanes that hold them: 45 permuted adds instead of four per value."""
+        low = self.low
+        n = 4 * low.L2
+        cur = (n + 15) // 16 * 16
+        s.open("")
+        s(f"T rv[{cur}];")
+        for o in range(cur):
+            s(f"rv[{o}] = {f'dy[{o // low.L2}][{o % low.L2}]' if o < n else 'T(0)'};")
+        s("int at = 0;  // index of rv[0] in the lane group's value list")
+        for ctrl, bit in (("0x140", 8), ("0x141", 4), ("0x1B", 2), ("0xB1", 1)):
+            half = cur // 2
+            s.open("")
+            s(f"const bool hi = (l16 & {bit}) != 0;")
+            for j in range(half):
+                s(f"{{ const T keep = hi ? rv[{j + half}] : rv[{j}]; const T send = hi ? rv[{j}] : rv[{j + half}]; "
+                  f"rv[{j}] = keep + oeq_dpp<{ctrl}>(send); }}")
+            s(f"at += hi ? {half} : 0;")
+            s.close()
+            cur = half
+        for t in range(cur):
+            s(f"if (at + {t} < {n}) (&s_dy[wave][4 * lq][0])[at + {t}] = rv[{t}];")
         s.close()
 
     # ------------------------------------------------------------- forward
@@ -314,16 +465,44 @@ class MfmaEmitter:
                 s.close()
                 s.close()
                 continue
-            s(f"__shared__ T s_g[{RT}][{self.gstride}];")
+            # the dZ tile: staged through registers, or (uvw_dma) written by direct global->LDS loads into one of
+            # two buffers while the other tile is worked on
+            dma = bool(self.tune["uvw_dma"]) and low.L3 % 4 == 0
+            self.g_at = (lambda row, col: f"sg[{row} * {self.gstride} + {col}]") if dma else (
+                lambda row, col: f"s_g[{row}][{col}]")
+            s(f"__shared__ __attribute__((aligned(16))) T s_g[{'2][' if dma else ''}{RT}][{self.gstride}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             s(f"__shared__ T s_dy[{WAVES}][{RT}][{low.L2}];")
             self._prologue(s)
             s("const int u = wave * 16 + l16;  // channel of this lane in the MFMA result layout")
-            self._load_wreg(s, paths, transposed=True)
+            # Registers per lane: 16 per resident weight slice, the 4 rows' x / dx / dy, G and the operand
+            # chunks. Where that exceeds the budget of two waves per SIMD, the slices of the paths with the
+            # fewest multiplies are kept in LDS instead (read like the A operands, one chunk ahead): spilled
+            # slices would come back from scratch memory in the middle of the multiply sequence.
+            need = lambda n: 16 * n + 4 * (self.max_d1 + b1.d + low.L2) + 6 * max(low.out[p.io].d for p in paths) + 48
+            by_cost = sorted(paths, key=lambda p: (low.out[p.io].d, p.index))
+            self.lds_w = []
+            if self.tune["uvw_pipe"]:
+                while len(paths) - len(self.lds_w) > 1 and need(len(paths) - len(self.lds_w)) > self.tune["uvw_regs"]:
+                    self.lds_w.append(by_cost[len(self.lds_w)].index)
+            if self.lds_w:
+                s(f"__shared__ T s_wl[{len(self.lds_w)}][16][{64 * WAVES}];")
+            self._load_wreg(s, [p for p in paths if p.index not in self.lds_w], transposed=True)
+            for n, pi in enumerate(self.lds_w):
+                woff = next(p.woff for p in paths if p.index == pi)
+                s("#pragma unroll")
+                s(f"for (int st = 0; st < 16; ++st) s_wl[{n}][st][tid] = W[{woff} + u * 64 + 4 * st + lq];")
+            if dma:
+                s("int buf = 0;")
+                s("if ((i64)blockIdx.x < ntiles) {")
+                s.level += 1
+                self._dma_g(s, "(i64)blockIdx.x", "0")
+                s.close()
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
             s(f"const i64 row0 = tile * {RT};")
             s("__syncthreads();")
-            self._stage_g(s)
+            if not dma:
+                self._stage_g(s)
             self._stage_y(s)
             # X of the lane's 4 (row, channel) pairs: issued before the barrier and the MFMA loop
             s(f"T x[4][{self.max_d1}], dx[4][{b1.d}], dy[4][{low.L2}];")
@@ -335,28 +514,20 @@ class MfmaEmitter:
                 s(f"x[i][{c}] = xp[{c}]; dx[i][{c}] = T(0);")
             s(f"for (int j = 0; j < {low.L2}; ++j) dy[i][j] = T(0);")
             s.close()
-            s("__syncthreads();")
-            for p in paths:
-                b2, bo = low.in2[p.i2], low.out[p.io]
-                s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
-                s.open("")
-                # G[k] = sum_w dZ[(r,k), w] * W[u, w]   (A = dZ tile, B = W^T slice in registers)
-                s(f"v4f G[{bo.d}];")
-                for k in range(bo.d):
-                    s(f"G[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
-                s("#pragma unroll")
-                s.open("for (int st = 0; st < 16; ++st)")
-                for k in range(bo.d):
-                    s(f"G[{k}] = {MFMA}(s_g[l16][{bo.off} + (4 * st + lq) * {bo.d} + {k}], wreg{p.index}[st], G[{k}], 0, 0, 0);")
+            if dma:
+                # this wave's loads of the tile have landed; after the barrier, everybody's have, and nobody
+                # reads the other buffer any more: the next tile may be requested into it
+                fence = 'asm volatile("" ::: "memory");'
+                s(f"{fence} __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0) */ {fence}")
+                s("__syncthreads();")
+                s.open("if (tile + gridDim.x < ntiles)")
+                self._dma_g(s, "(tile + gridDim.x)", "(buf ^ 1)")
                 s.close()
-                s("#pragma unroll")
-                s.open("for (int i = 0; i < 4; ++i)")
-                s(f"T Gk[{bo.d}];")
-                for k in range(bo.d):
-                    s(f"Gk[{k}] = G[{k}][i];")
-                s(f"cg_bwd{p.index}(x[i], s_y[4 * lq + i], Gk, dx[i], dy[i]);")
-                s.close()
-                s.close()
+                s(f"const T* sg = &s_g[buf][0][0];")
+                s(fence)
+            else:
+                s("__syncthreads();")
+            self._dx_paths(s, paths)
             s("#pragma unroll")
             s.open("for (int i = 0; i < 4; ++i)")
             s("const i64 row = row0 + 4 * lq + i;")
@@ -367,20 +538,15 @@ class MfmaEmitter:
             s.close()
             s.close()
             # dY: sum over the 16 channels of the lane group, then over the 4 waves through LDS
-            s.open("for (int i = 0; i < 4; ++i)")
-            s.open(f"for (int j = 0; j < {low.L2}; ++j)")
-            s("T v = dy[i][j];")
-            for m in (1, 2, 4, 8):
-                s(f"v += __shfl_xor(v, {m});")
-            s("if (l16 == 0) s_dy[wave][4 * lq + i][j] = v;")
-            s.close()
-            s.close()
+            self._reduce_dy(s)
             s("__syncthreads();")
             s.open(f"for (int t = tid; t < {RT * low.L2}; t += {64 * WAVES})")
             s(f"const int r = t / {low.L2}, c = t % {low.L2};")
             s("const T tot = ((s_dy[0][r][c] + s_dy[1][r][c]) + s_dy[2][r][c]) + s_dy[3][r][c];")
             s(f"if (row0 + r < num_batch) L2_grad[(row0 + r) * {low.L2} + c] {'=' if first_dy else '+='} tot;")
             s.close()
+            if dma:
+                s("buf ^= 1;")
             s.close()
             s.close()
             first_dy = False
@@ -394,7 +560,8 @@ class MfmaEmitter:
             names.append(name)
             s(f"// ======== dW of the paths into out[{io}]")
             self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_ww"])
-            s(f"__shared__ T s_g[{RT}][{self.gstride}];")
+            # only this irrep's columns of the dZ tile are needed (and kept)
+            s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self._tile_stride(bo.mul * bo.d)}];")
             s(f"__shared__ T s_T[2][{bo.d}][64][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             self._prologue(s)
@@ -408,8 +575,7 @@ class MfmaEmitter:
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
             s(f"const i64 row0 = tile * {RT};")
             s("__syncthreads();")
-            # only this irrep's columns of the dZ tile are needed
-            self._stage_g(s, bo.off, bo.mul * bo.d)
+            self._stage_g(s, bo.off, bo.mul * bo.d, local=True)
             self._stage_y(s)
             self._load_x_rows(s, "xa", order[0])
             s("__syncthreads();")
@@ -429,7 +595,7 @@ class MfmaEmitter:
                 s("const int kk = kq >> 4, rr = kq & 15;")
                 s(f"const T a = s_T[{buf}][kk][u][rr];")
                 for nn in range(4):
-                    s(f"dw{p.index}[{nn}] = {MFMA}(a, s_g[rr][{bo.off} + ({16 * nn} + l16) * {bo.d} + kk], dw{p.index}[{nn}], 0, 0, 0);")
+                    s(f"dw{p.index}[{nn}] = {MFMA}(a, s_g[rr][({16 * nn} + l16) * {bo.d} + kk], dw{p.index}[{nn}], 0, 0, 0);")
                 s.close()
                 cur, nxt = nxt, cur
             s.close()
@@ -450,6 +616,10 @@ def tp_module(low: Lowered, compute_units: int = 256):
     s = Src()
     s(prelude(low.ctype))
     s("typedef float v4f __attribute__((ext_vector_type(4)));")
+    # value of the lane that a DPP control word pairs this lane with (row_mirror 0x140, row_half_mirror 0x141,
+    # quad_perm otherwise)
+    s("template <int CTRL> OEQ_DEV float oeq_dpp(float v) { return __builtin_bit_cast(float, "
+      "__builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true)); }")
     s(utility_kernels())
     em._emit_path_fns(s)
     fwd_names = em.emit_forward(s)
@@ -459,7 +629,7 @@ def tp_module(low: Lowered, compute_units: int = 256):
     descs += [(rt.ROLE_TP_BACKWARD, n, 64 * WAVES, RT, max_blocks) for n in bwd_names]
     descs += [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
-        (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 256, 0),
+        (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 64, 0),
     ]
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
                 shared_weights=1, deterministic=0, wpartial_per_block=1)
