@@ -782,7 +782,8 @@ def tp_module(low: Lowered, compute_units: int = 256, kahan: bool = False):
 
     if low.shared_weights and not kahan:
         from . import uvw_mfma
-        if uvw_mfma.supported(low):
+        from .uvu import tuning
+        if uvw_mfma.supported(low) and tuning(dict(uvw_mfma=1))["uvw_mfma"]:
             return uvw_mfma.tp_module(low, compute_units)
     em = UvwEmitter(low)
     s = Src()

@@ -9,10 +9,17 @@ reference does this mix with a scalar-FMA warp matmul on 32-wide chunks
 (openequivariance/openequivariance/templates/wmm.cuh:1-87,
 loop_unroll_tp.cuh:55-84, 217-272).
 
-Work decomposition: a block of 4 waves owns a tile of 16 batch rows at a time;
-wave ``w`` owns output channels (forward) or input channels (backward)
-``16w .. 16w+15`` of every 64-channel block. Forward and backward are each a
-short sequence of kernels launched back to back with the same arguments:
+Work decomposition: irrep blocks are cut into pieces of at most 64 channels
+(multiplicities are multiples of 16), a path into one sub-path per pair of
+pieces with its own 64 x 64 (or smaller) corner of the path's weight matrix. A
+block of 4 waves owns a tile of 16 batch rows at a time; wave ``w`` owns output
+channels (forward) or input channels (backward) ``16w .. 16w+15`` of a piece
+(waves beyond a narrow piece's channels sit out the multiplies). Forward and
+backward are each a short sequence of kernels launched back to back with the
+same arguments; with pieces on both sides a kernel takes one piece and the
+sub-paths that meet it from the k-th piece of the other side, and all but the
+first kernel of a piece add to what is already there (a tile is always handled
+by the same thread of the same block, so the order of these additions is fixed):
 
 * forward, one kernel per output irrep: the wave's slices of the weight
   matrices of the paths feeding that irrep stay in registers in MFMA B-operand
@@ -42,6 +49,7 @@ D[m][n]: n = l % 16, m = 4 * (l / 16) + i for the i-th of 4 result registers.
 
 from __future__ import annotations
 
+from dataclasses import dataclass
 from typing import List
 
 from .common import Src, prelude, utility_kernels
@@ -50,34 +58,110 @@ from .lower import Lowered, Path, float_literal
 RT = 16          # rows per tile
 WAVES = 4        # waves per block
 TPAD = RT + 1    # padded row stride of the T tile in LDS (bank spread)
+PIECE = 64       # channels per piece of an irrep block
 MFMA = "__builtin_amdgcn_mfma_f32_16x16x4f32"
 
 
+@dataclass
+class VBlock:
+    """A piece (at most 64 channels) of an irrep block."""
+    off: int
+    mul: int
+    l: int
+    orig: int     # index of the block it was cut from
+    chunk: int    # which piece of that block
+
+    @property
+    def d(self) -> int:
+        return 2 * self.l + 1
+
+
+@dataclass
+class VPath:
+    """The part of a path between one piece of its input block and one piece of its output block: a
+    U x Wn corner of the path's weight matrix, whose rows are ``ld`` words apart."""
+    index: int
+    p: Path
+    vi: int
+    vo: int
+    U: int
+    Wn: int
+    woff: int
+    ld: int
+    ub: int
+    wb: int
+
+
+def _pieces(blocks) -> List[VBlock]:
+    out = []
+    for i, b in enumerate(blocks):
+        for c in range((b.mul + PIECE - 1) // PIECE):
+            out.append(VBlock(b.off + c * PIECE * b.d, min(PIECE, b.mul - c * PIECE), b.l, i, c))
+    return out
+
+
+def _split(low: Lowered):
+    vin, vout = _pieces(low.in1), _pieces(low.out)
+    vpaths = []
+    for p in low.paths:
+        wtot = low.out[p.io].mul
+        for vi, a in enumerate(vin):
+            if a.orig != p.i1:
+                continue
+            for vo, o in enumerate(vout):
+                if o.orig != p.io:
+                    continue
+                vpaths.append(VPath(len(vpaths), p, vi, vo, a.mul, o.mul,
+                                    p.woff + a.chunk * PIECE * wtot + o.chunk * PIECE, wtot, a.chunk, o.chunk))
+    return vin, vout, vpaths
+
+
+def _groups(vpaths: List[VPath], side: str, n_blocks: int):
+    """Kernels of one pass: for every piece on ``side`` ('vo' or 'vi') its sub-paths grouped by the piece
+    index on the other side. Returns [(piece, [sub-paths], first kernel of that piece?)]; a piece without
+    paths gets one entry with an empty list."""
+    other = "ub" if side == "vo" else "wb"
+    out = []
+    for b in range(n_blocks):
+        mine = [vp for vp in vpaths if getattr(vp, side) == b]
+        keys = sorted({getattr(vp, other) for vp in mine})
+        if not keys:
+            out.append((b, [], True))
+        for n, key in enumerate(keys):
+            out.append((b, [vp for vp in mine if getattr(vp, other) == key], n == 0))
+    return out
+
+
 def supported(low: Lowered) -> bool:
-    if low.mode != "uvw" or not low.shared_weights or low.ctype != "float":
+    if low.mode != "uvw" or not low.shared_weights or low.ctype != "float" or low.ir_mul:
         return False
-    if low.L3 > 2048 or low.L2 > 32:
+    if low.L3 > 1152 or low.L2 > 32:
         return False
     for p in low.paths:
         a, b, o = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
-        if b.mul != 1 or a.mul != 64 or o.mul != 64:
+        if b.mul != 1 or a.mul % 16 or o.mul % 16:
             return False
-    return 16 * len(low.paths) <= 192
+    # register budget of the widest kernel of each pass: 16-channel k-steps of resident weight slices
+    # (forward, dX: a few slices may move to LDS there) and 16 x 16 dW tiles
+    vin, vout, vpaths = _split(low)
+    fwd = max((sum(vp.U // 4 for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
+    dxk = max((sum(vp.Wn // 4 for vp in g) for _, g, _ in _groups(vpaths, "vi", len(vin))), default=0)
+    dwk = max((sum(4 * (vp.Wn // 16) for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
+    return fwd <= 80 and dxk <= 112 and dwk <= 80
 
 
 class MfmaEmitter:
     def __init__(self, low: Lowered):
         self.low = low
+        self.vin, self.vout, self.vpaths = _split(low)
         self.max_d3 = max(low.out[p.io].d for p in low.paths)
         self.max_d1 = max(low.in1[p.i1].d for p in low.paths)
         # Row stride of the dZ tile in LDS: 4 mod 32 words. Rows then start on 16-byte boundaries (the tile is
         # filled with 16-byte stores), and the 32 lanes of a half-wave that read one column of 16 rows, at two
         # k-steps d words apart (d odd), fall into 32 different banks.
         self.gstride = self._tile_stride(low.L3)
-        # order in which the forward / dW sweeps visit the paths: grouped by output block
-        self.fwd_order: List[Path] = [p for io in range(len(low.out)) for p in low.paths if p.io == io]
         from .uvu import tuning
-        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2, uvw_pipe=1, uvw_regs=300, uvw_dma=0))
+        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2, uvw_pipe=1, uvw_regs=220, uvw_dma=0))
 
     def lit(self, v):
         return float_literal(v, "float")
@@ -204,72 +288,76 @@ class MfmaEmitter:
                   f"(OEQ_LPTR)(&s_g[{buf}][wave * {rpw} + {rr}][{256 * j}]), 16, 0, 0);")
             s.close()
 
-    def _load_x_rows(self, s: Src, dst: str, p: Path):
-        """X of the wave's 4 rows for path p, lanes = channel u (T-compute layout)."""
+    def _load_x_rows(self, s: Src, dst: str, vp: VPath):
+        """X of the wave's 4 rows for a sub-path, lanes = channel u of its input piece (T-compute layout);
+        lanes beyond the piece read its last channel (their T values are never multiplied)."""
         low = self.low
-        b1 = low.in1[p.i1]
+        a = self.vin[vp.vi]
+        lane = "lane" if a.mul == 64 else f"(lane < {a.mul} ? lane : {a.mul - 1})"
         s.open(f"for (int rr = 0; rr < {RT // WAVES}; ++rr)")
         s(f"i64 row = row0 + wave * {RT // WAVES} + rr; if (row >= num_batch) row = num_batch - 1;")
-        s(f"const T* xp = L1_in + row * {low.L1} + {b1.off} + lane * {b1.d};")
-        for i in range(b1.d):
+        s(f"const T* xp = L1_in + row * {low.L1} + {a.off} + {lane} * {a.d};")
+        for i in range(a.d):
             s(f"{dst}[rr][{i}] = xp[{i}];")
         s.close()
 
-    def _t_compute(self, s: Src, p: Path, xsrc: str, buf: str):
-        low = self.low
-        bo = low.out[p.io]
+    def _t_compute(self, s: Src, vp: VPath, xsrc: str, buf: str):
+        d3 = self.vout[vp.vo].d
         s.open(f"for (int rr = 0; rr < {RT // WAVES}; ++rr)")
         s(f"const int r = wave * {RT // WAVES} + rr;")
-        s(f"T t[{bo.d}];")
-        s(f"cg_fwd{p.index}({xsrc}[rr], s_y[r], t);")
-        for k in range(bo.d):
+        s(f"T t[{d3}];")
+        s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y[r], t);")
+        for k in range(d3):
             s(f"s_T[{buf}][{k}][lane][r] = t[{k}];")
         s.close()
 
-    def _dx_paths(self, s: Src, paths: List[Path]):
-        """G = dZ W^T of every path on the matrix cores, then the CG part on the vector ALU (in scope:
+    def _dx_paths(self, s: Src, paths: List[VPath]):
+        """G = dZ W^T of every sub-path on the matrix cores, then its CG part on the vector ALU (in scope:
         x, dx, dy, s_g, s_y, wreg<path>). ``uvw_pipe`` = 0: path after path, operand order left to the
         compiler. 1: the A operands (dZ values from LDS) are fetched one chunk of 4 k-steps ahead of the
-        multiplies that use them, and nothing moves across a chunk boundary: without that the compiler
-        hoists the LDS reads of several paths, runs out of registers and spills the weight slices. 2: as 1,
-        and the CG part of the previous path (one of its four rows per chunk) sits between the multiplies of
-        the current one, so that the vector ALU works while the matrix core does."""
-        low = self.low
+        multiplies that use them, and nothing moves across a chunk boundary: left alone, the compiler hoists
+        the LDS reads of several paths and spills the weight slices."""
         pipe = self.tune["uvw_pipe"]
         CH = 4
+
+        def cg_rows(vp, G):
+            d3 = self.vout[vp.vo].d
+            s("#pragma unroll")
+            s.open("for (int i = 0; i < 4; ++i)")
+            s(f"T Gk[{d3}];")
+            for k in range(d3):
+                s(f"Gk[{k}] = {G}[{k}][i];")
+            s(f"cg_bwd{vp.p.index}(x[i], s_y[4 * lq + i], Gk, dx[i], dy[i]);")
+            s.close()
+
         if pipe == 0:
-            for p in paths:
-                bo = low.out[p.io]
-                s(f"// path {p.index}")
+            for vp in paths:
+                bo = self.vout[vp.vo]
+                s(f"// path {vp.p.index}, output piece {vp.wb}")
                 s.open("")
                 # G[k] = sum_w dZ[(r,k), w] * W[u, w]   (A = dZ tile, B = W^T slice in registers)
                 s(f"v4f G[{bo.d}];")
                 for k in range(bo.d):
                     s(f"G[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
                 s("#pragma unroll")
-                s.open("for (int st = 0; st < 16; ++st)")
+                s.open(f"for (int st = 0; st < {vp.Wn // 4}; ++st)")
                 for k in range(bo.d):
-                    s(f"G[{k}] = {MFMA}({self.g_at('l16', f'{bo.off} + (4 * st + lq) * {bo.d} + {k}')}, wreg{p.index}[st], G[{k}], 0, 0, 0);")
+                    s(f"G[{k}] = {MFMA}({self.g_at('l16', f'{bo.off} + (4 * st + lq) * {bo.d} + {k}')}, "
+                      f"wreg{vp.index}[st], G[{k}], 0, 0, 0);")
                 s.close()
-                s("#pragma unroll")
-                s.open("for (int i = 0; i < 4; ++i)")
-                s(f"T Gk[{bo.d}];")
-                for k in range(bo.d):
-                    s(f"Gk[{k}] = G[{k}][i];")
-                s(f"cg_bwd{p.index}(x[i], s_y[4 * lq + i], Gk, dx[i], dy[i]);")
-                s.close()
+                cg_rows(vp, "G")
                 s.close()
             return
-        maxd = max(low.out[p.io].d for p in paths)
+        maxd = max(self.vout[vp.vo].d for vp in paths)
         s(f"T opa[{CH * maxd}], opb[{CH * maxd}];  // A operands of the current and the next chunk")
         if self.lds_w:
             s(f"T wla[{CH}], wlb[{CH}];  // B operands of a path whose weight slice is kept in LDS")
-        s(f"v4f Ga[{maxd}], Gb[{maxd}];")
-        segs = [(n, c) for n in range(len(paths)) for c in range(16 // CH)]
+        s(f"v4f G[{maxd}];")
+        segs = [(n, c) for n, vp in enumerate(paths) for c in range(vp.Wn // (4 * CH))]
 
         def reads(seg, buf):
             n, c = seg
-            bo = low.out[paths[n].io]
+            bo = self.vout[paths[n].vo]
             for q in range(CH):
                 for k in range(bo.d):
                     s(f"{buf}[{q * bo.d + k}] = {self.g_at('l16', f'{bo.off} + ({4 * (c * CH + q)} + lq) * {bo.d} + {k}')};")
@@ -278,49 +366,25 @@ class MfmaEmitter:
                 for q in range(CH):
                     s(f"{'wla' if buf == 'opa' else 'wlb'}[{q}] = s_wl[{slot}][{c * CH + q}][tid];")
 
-        def cg_row(n, i):
-            p = paths[n]
-            bo = low.out[p.io]
-            G = "Ga" if n % 2 == 0 else "Gb"
-            s.open("")
-            s(f"T Gk[{bo.d}];")
-            for k in range(bo.d):
-                s(f"Gk[{k}] = {G}[{k}][{i}];")
-            s(f"cg_bwd{p.index}(x[{i}], s_y[4 * lq + {i}], Gk, dx[{i}], dy[{i}]);")
-            s.close()
-
         reads(segs[0], "opa")
         for t, (n, c) in enumerate(segs):
-            p = paths[n]
-            bo = low.out[p.io]
+            vp = paths[n]
+            bo = self.vout[vp.vo]
             cur, nxt = ("opa", "opb") if t % 2 == 0 else ("opb", "opa")
-            G = "Ga" if n % 2 == 0 else "Gb"
             if c == 0:
-                s(f"// path {p.index}")
+                s(f"// path {vp.p.index}, output piece {vp.wb}")
                 for k in range(bo.d):
-                    s(f"{G}[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+                    s(f"G[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
             if t + 1 < len(segs):
                 reads(segs[t + 1], nxt)
             for q in range(CH):
-                wop = (f"{'wla' if cur == 'opa' else 'wlb'}[{q}]" if p.index in self.lds_w
-                       else f"wreg{p.index}[{c * CH + q}]")
+                wop = (f"{'wla' if cur == 'opa' else 'wlb'}[{q}]" if vp.index in self.lds_w
+                       else f"wreg{vp.index}[{c * CH + q}]")
                 for k in range(bo.d):
-                    s(f"{G}[{k}] = {MFMA}({cur}[{q * bo.d + k}], {wop}, {G}[{k}], 0, 0, 0);")
-            if pipe >= 2 and n > 0:
-                cg_row(n - 1, c)
-            if pipe == 3 and n > 0:
-                # one multiply, then its share of the vector instructions of the row's CG part
-                valu = max(1, int(3.4 * len(paths[n - 1].nnz)) // (CH * bo.d))
-                for _ in range(CH * bo.d):
-                    s("__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);")
-                    s(f"__builtin_amdgcn_sched_group_barrier(0x002, {valu}, 0);")
+                    s(f"G[{k}] = {MFMA}({cur}[{q * bo.d + k}], {wop}, G[{k}], 0, 0, 0);")
             s("__builtin_amdgcn_sched_barrier(0);")
-            if pipe == 1 and c == 16 // CH - 1:
-                for i in range(4):
-                    cg_row(n, i)
-        if pipe >= 2:
-            for i in range(4):
-                cg_row(len(paths) - 1, i)
+            if c == vp.Wn // (4 * CH) - 1:
+                cg_rows(vp, "G")
 
     def _reduce_dy(self, s: Src):
         """Sum of dy[i][j] (4 rows x L2 values per lane) over the 16 lanes of a lane group, into
@@ -351,15 +415,21 @@ class MfmaEmitter:
         s.close()
 
     # ------------------------------------------------------------- forward
-    def _load_wreg(self, s: Src, paths: List[Path], transposed: bool):
-        for p in paths:
-            s(f"T wreg{p.index}[16];")
+    def _load_wreg(self, s: Src, vps: List[VPath], transposed: bool):
+        """Weight slices in MFMA B-operand layout, 1 register per 4 k-steps... per k-step of 4: forward
+        B[k = u' = 4 st + lq][n = l16] = W[u'][w = 16 wave + l16] (U / 4 registers); backward (transposed)
+        B[k = w = 4 st + lq][n = l16] = W[u][w] (Wn / 4 registers). Waves without channels in the piece load
+        nothing (``act`` is in scope)."""
+        for vp in vps:
+            n = (vp.Wn if transposed else vp.U) // 4
+            s(f"T wreg{vp.index}[{n}];")
             s("#pragma unroll")
-            if transposed:  # B[k = w = 4 st + lq][n = l16] = W_p[u][w]
-                s(f"for (int st = 0; st < 16; ++st) wreg{p.index}[st] = W[{p.woff} + u * 64 + 4 * st + lq];")
-            else:           # B[k = u' = 4 st + lq][n = l16] = W_p[u'][w = 16 wave + l16]
-                s(f"for (int st = 0; st < 16; ++st) wreg{p.index}[st] = "
-                  f"W[{p.woff} + (4 * st + lq) * 64 + wave * 16 + l16];")
+            if transposed:
+                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = act ? "
+                  f"W[{vp.woff} + u * {vp.ld} + 4 * st + lq] : T(0);")
+            else:
+                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = act ? "
+                  f"W[{vp.woff} + (4 * st + lq) * {vp.ld} + wave * 16 + l16] : T(0);")
 
     FWD_SIG = ("(i64 num_batch, const T* __restrict__ L1_in, const T* __restrict__ L2_in, "
                "const T* __restrict__ W, T* __restrict__ L3_out)")
@@ -373,32 +443,37 @@ class MfmaEmitter:
             attr += f" __attribute__((amdgpu_waves_per_eu({waves_per_eu}, {waves_per_eu})))"
         s.open(f'extern "C" __global__ {attr} void {name}{sig}')
 
+    def _zero_kernel(self, s: Src, ptr: str, row_len: int, blk: VBlock):
+        """A piece that no path touches: zeros."""
+        self._prologue(s)
+        s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
+        s(f"const i64 row0 = tile * {RT};")
+        s.open(f"for (int t = tid; t < {RT * blk.mul * blk.d}; t += {64 * WAVES})")
+        s(f"const int r = t / {blk.mul * blk.d}, c = t % {blk.mul * blk.d};")
+        s(f"if (row0 + r < num_batch) {ptr}[(row0 + r) * {row_len} + {blk.off} + c] = T(0);")
+        s.close()
+        s.close()
+        s.close()
+
     def emit_forward(self, s: Src) -> List[str]:
-        """One kernel per output irrep (launched back to back), so that only the weights of the
-        paths feeding that irrep (16 registers each) are resident and register allocation is per
-        irrep. Returns the kernel names in launch order."""
+        """One kernel per piece of an output irrep and piece index of the input side (launched back to
+        back), so that only the weight slices of the sub-paths it multiplies are resident and register
+        allocation is per kernel. Returns the kernel names in launch order."""
         low = self.low
         names = []
-        for io, bo in enumerate(low.out):
-            order = [p for p in low.paths if p.io == io]
-            name = "forward" if not names else f"forward_o{io}"
+        for vo, order, first in _groups(self.vpaths, "vo", len(self.vout)):
+            bo = self.vout[vo]
+            name = "forward" if not names else f"forward_o{vo}_{order[0].ub if order else 0}"
             names.append(name)
-            s(f"// ======== out[{io}]: {bo.mul} x l={bo.l}")
+            s(f"// ======== out piece {vo}: {bo.mul} x l={bo.l} at {bo.off}")
             self._kernel_open(s, name, self.FWD_SIG, self.tune["uvw_wf"])
             if not order:
-                self._prologue(s)
-                s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
-                s(f"const i64 row0 = tile * {RT};")
-                s.open(f"for (int t = tid; t < {RT * bo.mul * bo.d}; t += {64 * WAVES})")
-                s(f"const int r = t / {bo.mul * bo.d}, c = t % {bo.mul * bo.d};")
-                s(f"if (row0 + r < num_batch) L3_out[(row0 + r) * {low.L3} + {bo.off} + c] = T(0);")
-                s.close()
-                s.close()
-                s.close()
+                self._zero_kernel(s, "L3_out", low.L3, bo)
                 continue
             s(f"__shared__ T s_T[2][{bo.d}][64][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             self._prologue(s)
+            s(f"const bool act = wave * 16 < {bo.mul};  // this wave has output channels in the piece")
             s(f"T xa[{RT // WAVES}][{self.max_d1}], xb[{RT // WAVES}][{self.max_d1}];")
             self._load_wreg(s, order, transposed=False)
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
@@ -411,27 +486,30 @@ class MfmaEmitter:
             for k in range(bo.d):
                 s(f"acc[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
             cur, nxt = "xa", "xb"
-            for n, p in enumerate(order):
+            for n, vp in enumerate(order):
                 buf = n % 2
-                s(f"// path {p.index}: l=({low.in1[p.i1].l},{low.in2[p.i2].l},{bo.l})")
-                self._t_compute(s, p, cur, str(buf))
+                p = vp.p
+                s(f"// path {p.index}: l=({low.in1[p.i1].l},{low.in2[p.i2].l},{bo.l}), input piece {vp.ub}")
+                self._t_compute(s, vp, cur, str(buf))
                 if n + 1 < len(order):
                     self._load_x_rows(s, nxt, order[n + 1])
                 s("__syncthreads();")
+                s.open("if (act)")
                 s("#pragma unroll")
-                s.open("for (int st = 0; st < 16; ++st)")
+                s.open(f"for (int st = 0; st < {vp.U // 4}; ++st)")
                 for k in range(bo.d):
-                    s(f"acc[{k}] = {MFMA}(s_T[{buf}][{k}][4 * st + lq][l16], wreg{p.index}[st], acc[{k}], 0, 0, 0);")
+                    s(f"acc[{k}] = {MFMA}(s_T[{buf}][{k}][4 * st + lq][l16], wreg{vp.index}[st], acc[{k}], 0, 0, 0);")
+                s.close()
                 s.close()
                 cur, nxt = nxt, cur
             # D layout: rows 4*lq + i, column (channel) l16 of the wave's slice
             s("#pragma unroll")
             s.open("for (int i = 0; i < 4; ++i)")
             s("const i64 row = row0 + 4 * lq + i;")
-            s.open("if (row < num_batch)")
+            s.open("if (act && row < num_batch)")
             s(f"T* zp = L3_out + row * {low.L3} + {bo.off} + (wave * 16 + l16) * {bo.d};")
             for k in range(bo.d):
-                s(f"zp[{k}] = acc[{k}][i];")
+                s(f"zp[{k}] {'=' if first else '+='} acc[{k}][i];")
             s.close()
             s.close()
             s.close()
@@ -440,30 +518,22 @@ class MfmaEmitter:
 
     # ------------------------------------------------------------ backward
     def emit_backward(self, s: Src) -> List[str]:
-        """One kernel per input irrep (dX of that irrep and the dY contributions of its paths) and
-        one per output irrep (dW of the paths feeding it), launched back to back. A tile is always
-        handled by the same block and thread, so the dY contributions of successive kernels are
-        added in a fixed order with plain read-modify-writes. Returns the kernel names."""
+        """Kernels per piece of an input irrep (dX of the piece and the dY contributions of its sub-paths)
+        and per piece of an output irrep (dW of the sub-paths feeding it), launched back to back. A tile is
+        always handled by the same block and thread, so what successive kernels add to dY (and to dX, with
+        several output pieces) arrives in a fixed order with plain read-modify-writes. Returns the names."""
         low = self.low
         names = []
         # ---------------- dX, dY ------------------------------------------------
         first_dy = True
-        for i1, b1 in enumerate(low.in1):
-            paths = [p for p in low.paths if p.i1 == i1]
-            name = "backward" if not names else f"backward_x{i1}"
+        for vi, paths, first in _groups(self.vpaths, "vi", len(self.vin)):
+            b1 = self.vin[vi]
+            name = "backward" if not names else f"backward_x{vi}_{paths[0].wb if paths else 0}"
             names.append(name)
-            s(f"// ======== in1[{i1}]: {b1.mul} x l={b1.l}")
+            s(f"// ======== in1 piece {vi}: {b1.mul} x l={b1.l} at {b1.off}")
             self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_wx"])
             if not paths:
-                self._prologue(s)
-                s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
-                s(f"const i64 row0 = tile * {RT};")
-                s.open(f"for (int t = tid; t < {RT * b1.mul * b1.d}; t += {64 * WAVES})")
-                s(f"const int r = t / {b1.mul * b1.d}, c = t % {b1.mul * b1.d};")
-                s(f"if (row0 + r < num_batch) L1_grad[(row0 + r) * {low.L1} + {b1.off} + c] = T(0);")
-                s.close()
-                s.close()
-                s.close()
+                self._zero_kernel(s, "L1_grad", low.L1, b1)
                 continue
             # the dZ tile: staged through registers, or (uvw_dma) written by direct global->LDS loads into one of
             # two buffers while the other tile is worked on
@@ -474,24 +544,28 @@ class MfmaEmitter:
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             s(f"__shared__ T s_dy[{WAVES}][{RT}][{low.L2}];")
             self._prologue(s)
-            s("const int u = wave * 16 + l16;  // channel of this lane in the MFMA result layout")
-            # Registers per lane: 16 per resident weight slice, the 4 rows' x / dx / dy, G and the operand
-            # chunks. Where that exceeds the budget of two waves per SIMD, the slices of the paths with the
-            # fewest multiplies are kept in LDS instead (read like the A operands, one chunk ahead): spilled
-            # slices would come back from scratch memory in the middle of the multiply sequence.
-            need = lambda n: 16 * n + 4 * (self.max_d1 + b1.d + low.L2) + 6 * max(low.out[p.io].d for p in paths) + 48
-            by_cost = sorted(paths, key=lambda p: (low.out[p.io].d, p.index))
+            s(f"const bool act = wave * 16 < {b1.mul};  // this wave has input channels in the piece")
+            s("const int u = act ? wave * 16 + l16 : 0;  // channel of this lane in the MFMA result layout")
+            # Registers per lane: one per 4 k-steps of a resident weight slice, the 4 rows' x / dx / dy, G and
+            # the operand chunks. Where that exceeds the budget of two waves per SIMD, the slices of the paths
+            # with the fewest multiplies are kept in LDS instead (read like the A operands, one chunk ahead):
+            # spilled slices would come back from scratch memory in the middle of the multiply sequence.
+            fixed = 4 * (self.max_d1 + b1.d + low.L2) + 6 * max(self.vout[vp.vo].d for vp in paths) + 48
+            by_cost = sorted(paths, key=lambda vp: (self.vout[vp.vo].d, vp.index))
             self.lds_w = []
             if self.tune["uvw_pipe"]:
-                while len(paths) - len(self.lds_w) > 1 and need(len(paths) - len(self.lds_w)) > self.tune["uvw_regs"]:
+                resident = lambda: sum(vp.Wn // 4 for vp in paths if vp.index not in self.lds_w)
+                while len(paths) - len(self.lds_w) > 1 and len(self.lds_w) < 3 and \
+                        resident() + fixed > self.tune["uvw_regs"]:
                     self.lds_w.append(by_cost[len(self.lds_w)].index)
             if self.lds_w:
                 s(f"__shared__ T s_wl[{len(self.lds_w)}][16][{64 * WAVES}];")
-            self._load_wreg(s, [p for p in paths if p.index not in self.lds_w], transposed=True)
+            self._load_wreg(s, [vp for vp in paths if vp.index not in self.lds_w], transposed=True)
             for n, pi in enumerate(self.lds_w):
-                woff = next(p.woff for p in paths if p.index == pi)
+                vp = next(q for q in paths if q.index == pi)
                 s("#pragma unroll")
-                s(f"for (int st = 0; st < 16; ++st) s_wl[{n}][st][tid] = W[{woff} + u * 64 + 4 * st + lq];")
+                s(f"for (int st = 0; st < {vp.Wn // 4}; ++st) s_wl[{n}][st][tid] = "
+                  f"act ? W[{vp.woff} + u * {vp.ld} + 4 * st + lq] : T(0);")
             if dma:
                 s("int buf = 0;")
                 s("if ((i64)blockIdx.x < ntiles) {")
@@ -527,6 +601,7 @@ class MfmaEmitter:
                 s(fence)
             else:
                 s("__syncthreads();")
+            s.open("if (act)")
             self._dx_paths(s, paths)
             s("#pragma unroll")
             s.open("for (int i = 0; i < 4; ++i)")
@@ -534,7 +609,8 @@ class MfmaEmitter:
             s.open("if (row < num_batch)")
             s(f"T* dp = L1_grad + row * {low.L1} + {b1.off} + u * {b1.d};")
             for c in range(b1.d):
-                s(f"dp[{c}] = dx[i][{c}];")
+                s(f"dp[{c}] {'=' if first else '+='} dx[i][{c}];")
+            s.close()
             s.close()
             s.close()
             # dY: sum over the 16 channels of the lane group, then over the 4 waves through LDS
@@ -550,17 +626,19 @@ class MfmaEmitter:
             s.close()
             s.close()
             first_dy = False
+        if first_dy:
+            raise AssertionError("no path")
 
         # ---------------- dW ----------------------------------------------------
-        for io, bo in enumerate(low.out):
-            order = [p for p in low.paths if p.io == io]
+        for vo, order, _first in _groups(self.vpaths, "vo", len(self.vout)):
             if not order:
                 continue
-            name = f"backward_w{io}"
+            bo = self.vout[vo]
+            name = f"backward_w{vo}_{order[0].ub}"
             names.append(name)
-            s(f"// ======== dW of the paths into out[{io}]")
+            s(f"// ======== dW of the sub-paths into out piece {vo} from input pieces {order[0].ub}")
             self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_ww"])
-            # only this irrep's columns of the dZ tile are needed (and kept)
+            # only this piece's columns of the dZ tile are needed (and kept)
             s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self._tile_stride(bo.mul * bo.d)}];")
             s(f"__shared__ T s_T[2][{bo.d}][64][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
@@ -568,10 +646,11 @@ class MfmaEmitter:
             s("const int u = wave * 16 + l16;")
             s(f"T* prow = wpartial + (i64)blockIdx.x * {low.WN};")
             s(f"T xa[{RT // WAVES}][{self.max_d1}], xb[{RT // WAVES}][{self.max_d1}];")
-            # dw{p}[n]: D tile rows = channels u of the wave's slice, columns = w in 16 n .. 16 n + 15
-            for p in order:
-                s(f"v4f dw{p.index}[4];")
-                s(f"for (int n = 0; n < 4; ++n) dw{p.index}[n] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+            # dw<path>[n]: D tile rows = channels u of the wave's slice, columns = w in 16 n .. 16 n + 15
+            ntile = bo.mul // 16
+            for vp in order:
+                s(f"v4f dw{vp.index}[{ntile}];")
+                s(f"for (int n = 0; n < {ntile}; ++n) dw{vp.index}[n] = v4f{{0.f, 0.f, 0.f, 0.f}};")
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
             s(f"const i64 row0 = tile * {RT};")
             s("__syncthreads();")
@@ -580,31 +659,35 @@ class MfmaEmitter:
             self._load_x_rows(s, "xa", order[0])
             s("__syncthreads();")
             cur, nxt = "xa", "xb"
-            for n, p in enumerate(order):
-                b1, b2 = low.in1[p.i1], low.in2[p.i2]
+            for n, vp in enumerate(order):
+                p = vp.p
                 buf = n % 2
-                s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
-                self._t_compute(s, p, cur, str(buf))
+                s(f"// path {p.index}: l=({low.in1[p.i1].l},{low.in2[p.i2].l},{bo.l})")
+                self._t_compute(s, vp, cur, str(buf))
                 if n + 1 < len(order):
                     self._load_x_rows(s, nxt, order[n + 1])
                 s("__syncthreads();")
                 # dW[u, w] += sum_(k,r) T[(k,r), u] * dZ[(k,r), w]   (A = T^T, B = dZ tile)
+                s.open(f"if (wave * 16 < {vp.U})")
                 s("#pragma unroll")
                 s.open(f"for (int st = 0; st < {4 * bo.d}; ++st)")
                 s("const int kq = 4 * st + lq;")
                 s("const int kk = kq >> 4, rr = kq & 15;")
                 s(f"const T a = s_T[{buf}][kk][u][rr];")
-                for nn in range(4):
-                    s(f"dw{p.index}[{nn}] = {MFMA}(a, s_g[rr][({16 * nn} + l16) * {bo.d} + kk], dw{p.index}[{nn}], 0, 0, 0);")
+                for nn in range(ntile):
+                    s(f"dw{vp.index}[{nn}] = {MFMA}(a, s_g[rr][({16 * nn} + l16) * {bo.d} + kk], dw{vp.index}[{nn}], 0, 0, 0);")
+                s.close()
                 s.close()
                 cur, nxt = nxt, cur
             s.close()
-            for p in order:
-                for nn in range(4):
+            for vp in order:
+                s.open(f"if (wave * 16 < {vp.U})")
+                for nn in range(ntile):
                     s("#pragma unroll")
                     s.open("for (int i = 0; i < 4; ++i)")
-                    s(f"prow[{p.woff} + (wave * 16 + 4 * lq + i) * 64 + {16 * nn} + l16] = dw{p.index}[{nn}][i];")
+                    s(f"prow[{vp.woff} + (wave * 16 + 4 * lq + i) * {vp.ld} + {16 * nn} + l16] = dw{vp.index}[{nn}][i];")
                     s.close()
+                s.close()
             s.close()
         return names
 

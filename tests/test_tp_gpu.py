@@ -53,6 +53,11 @@ def _folded_with_gaps():
                          label="folded-gaps")
 
 
+def _fc_shared(in1, in2, out):
+    return P.FullyConnectedTPProblem(in1, in2, out, shared_weights=True, internal_weights=False,
+                                     label=f"fc-shared {in1}")
+
+
 def _as_f64(problem):
     q = problem.clone()
     q.irrep_dtype, q.weight_dtype = np.float64, np.float64
@@ -98,7 +103,18 @@ CASES = [
     ("tetris-2", lambda: P.tetris_poly_problems()[1], 53),
     ("odd-uvw", lambda: _odd_uvw(False), 21),
     ("odd-uvw-shared", lambda: _odd_uvw(True), 21),
+    # shared-weight 'uvw' on the matrix cores: 32 channels (half the waves sit out the multiplies), 128 channels
+    # (two pieces per irrep, four sub-paths per path, later kernels add to the first one's rows), a different
+    # multiplicity per irrep, an input irrep no path reads and an output irrep no path writes
+    ("mfma-32", lambda: _fc_shared("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e"), 75),
+    ("mfma-128", lambda: _fc_shared("128x0e+128x1o", "1x0e+1x1o", "128x0e+128x1o"), 45),
+    ("mfma-mixed", lambda: _fc_shared("64x0e+32x1o+16x2e", "1x0e+1x1o", "48x0e+80x1o+16x2e"), 50),
+    ("mfma-gaps", lambda: oeq.TPProblem(
+        "32x0e+16x1o+48x2e", "1x0e+1x1o", "32x0e+16x1e+64x1o",
+        [(0, 0, 0, "uvw", True), (0, 1, 2, "uvw", True), (1, 0, 2, "uvw", True, 0.6), (1, 1, 0, "uvw", True)],
+        shared_weights=True, internal_weights=False, label="mfma-gaps"), 50),
 ]
+MFMA_CASES = {"cfg4-shared", "mfma-32", "mfma-128", "mfma-mixed", "mfma-gaps"}
 
 
 @pytest.mark.parametrize("name,make,B", CASES, ids=[c[0] for c in CASES])
@@ -110,6 +126,10 @@ def test_forward_backward_match_oracle(name, make, B):
     z_ref = R.tp_forward(ref, x, y, w)
     dx_ref, dy_ref, dw_ref = R.tp_backward(ref, x, y, w, g)
     tp = oeq.TensorProduct(problem)
+    if name in MFMA_CASES:
+        from openequivariance_amd.codegen import uvw_mfma
+        from openequivariance_amd.codegen.lower import lower
+        assert uvw_mfma.supported(lower(problem)), "this case is meant to run on the MFMA kernels"
     tx, ty, tw = to_gpu(x, y, w, requires_grad=True)
     (tg,) = to_gpu(g)
     z = tp(tx, ty, tw)
