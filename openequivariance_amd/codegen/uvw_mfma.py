@@ -161,7 +161,8 @@ class MfmaEmitter:
         # k-steps d words apart (d odd), fall into 32 different banks.
         self.gstride = self._tile_stride(low.L3)
         from .uvu import tuning
-        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2, uvw_pipe=1, uvw_regs=220, uvw_dma=0))
+        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2, uvw_pipe=1, uvw_regs=220, uvw_dma=0,
+                                uvw_merge=1, uvw_fregs=232, uvw_wregs=232))
 
     def lit(self, v):
         return float_literal(v, "float")
@@ -415,7 +416,7 @@ class MfmaEmitter:
         s.close()
 
     # ------------------------------------------------------------- forward
-    def _load_wreg(self, s: Src, vps: List[VPath], transposed: bool):
+    def _load_wreg(self, s: Src, vps: List[VPath], transposed: bool, act: str = "act"):
         """Weight slices in MFMA B-operand layout, 1 register per 4 k-steps... per k-step of 4: forward
         B[k = u' = 4 st + lq][n = l16] = W[u'][w = 16 wave + l16] (U / 4 registers); backward (transposed)
         B[k = w = 4 st + lq][n = l16] = W[u][w] (Wn / 4 registers). Waves without channels in the piece load
@@ -425,10 +426,10 @@ class MfmaEmitter:
             s(f"T wreg{vp.index}[{n}];")
             s("#pragma unroll")
             if transposed:
-                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = act ? "
+                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = {act} ? "
                   f"W[{vp.woff} + u * {vp.ld} + 4 * st + lq] : T(0);")
             else:
-                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = act ? "
+                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = {act} ? "
                   f"W[{vp.woff} + (4 * st + lq) * {vp.ld} + wave * 16 + l16] : T(0);")
 
     FWD_SIG = ("(i64 num_batch, const T* __restrict__ L1_in, const T* __restrict__ L2_in, "
@@ -455,63 +456,91 @@ class MfmaEmitter:
         s.close()
         s.close()
 
+    def _merge(self, groups, cost, limit):
+        """Consecutive (piece, sub-paths, first) groups that share a kernel: a group joins the kernel before
+        it while the kernel's estimated registers stay within ``limit``. Kernels of narrow output irreps
+        (l = 0: one multiply per k-step) are dominated by what every kernel pays per tile - staging, barriers,
+        the X loads - so they ride along with a neighbour. Groups without paths stay alone."""
+        kernels = []
+        for g in groups:
+            prev = kernels[-1][-1] if kernels else None
+            # only neighbours in the row share a kernel (one dZ tile then covers their columns)
+            adjacent = prev is not None and prev[0] != g[0] and \
+                self.vout[prev[0]].off + self.vout[prev[0]].mul * self.vout[prev[0]].d == self.vout[g[0]].off
+            if adjacent and g[1] and prev[1] and self.tune["uvw_merge"] and cost(kernels[-1] + [g]) <= limit:
+                kernels[-1].append(g)
+            else:
+                kernels.append([g])
+        return kernels
+
     def emit_forward(self, s: Src) -> List[str]:
-        """One kernel per piece of an output irrep and piece index of the input side (launched back to
-        back), so that only the weight slices of the sub-paths it multiplies are resident and register
-        allocation is per kernel. Returns the kernel names in launch order."""
+        """Kernels per piece of an output irrep and piece index of the input side (launched back to back;
+        pieces with few paths share a kernel), so that only the weight slices of the sub-paths it multiplies
+        are resident and register allocation is per kernel. Returns the kernel names in launch order."""
         low = self.low
         names = []
-        for vo, order, first in _groups(self.vpaths, "vo", len(self.vout)):
-            bo = self.vout[vo]
-            name = "forward" if not names else f"forward_o{vo}_{order[0].ub if order else 0}"
+        cost = lambda ker: (sum(vp.U // 4 for g in ker for vp in g[1]) + sum(4 * self.vout[g[0]].d for g in ker)
+                            + 2 * (RT // WAVES) * self.max_d1 + 64)
+        for ker in self._merge(_groups(self.vpaths, "vo", len(self.vout)), cost, self.tune["uvw_fregs"]):
+            vo0, order0, _ = ker[0]
+            name = "forward" if not names else f"forward_o{vo0}_{order0[0].ub if order0 else 0}"
             names.append(name)
-            s(f"// ======== out piece {vo}: {bo.mul} x l={bo.l} at {bo.off}")
+            s("// ======== out pieces " + ", ".join(f"{vo}: {self.vout[vo].mul} x l={self.vout[vo].l}" for vo, _, _ in ker))
             self._kernel_open(s, name, self.FWD_SIG, self.tune["uvw_wf"])
-            if not order:
-                self._zero_kernel(s, "L3_out", low.L3, bo)
+            if not order0:
+                self._zero_kernel(s, "L3_out", low.L3, self.vout[vo0])
                 continue
-            s(f"__shared__ T s_T[2][{bo.d}][64][{TPAD}];")
+            maxd = max(self.vout[vo].d for vo, _, _ in ker)
+            s(f"__shared__ T s_T[2][{maxd}][64][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             self._prologue(s)
-            s(f"const bool act = wave * 16 < {bo.mul};  // this wave has output channels in the piece")
             s(f"T xa[{RT // WAVES}][{self.max_d1}], xb[{RT // WAVES}][{self.max_d1}];")
-            self._load_wreg(s, order, transposed=False)
+            for vo, order, _ in ker:
+                s(f"const bool act{vo} = wave * 16 < {self.vout[vo].mul};  // this wave has output channels in the piece")
+            order_all = [vp for _, order, _ in ker for vp in order]
+            for vo, order, _ in ker:
+                self._load_wreg(s, order, transposed=False, act=f"act{vo}")
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
             s(f"const i64 row0 = tile * {RT};")
             s("__syncthreads();  // all reads of the previous tile's LDS data are done")
             self._stage_y(s)
-            self._load_x_rows(s, "xa", order[0])
+            self._load_x_rows(s, "xa", order_all[0])
             s("__syncthreads();")
-            s(f"v4f acc[{bo.d}];")
-            for k in range(bo.d):
-                s(f"acc[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+            for vo, _, _ in ker:
+                s(f"v4f acc{vo}[{self.vout[vo].d}];")
+                for k in range(self.vout[vo].d):
+                    s(f"acc{vo}[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
             cur, nxt = "xa", "xb"
-            for n, vp in enumerate(order):
+            for n, vp in enumerate(order_all):
                 buf = n % 2
                 p = vp.p
+                bo = self.vout[vp.vo]
                 s(f"// path {p.index}: l=({low.in1[p.i1].l},{low.in2[p.i2].l},{bo.l}), input piece {vp.ub}")
                 self._t_compute(s, vp, cur, str(buf))
-                if n + 1 < len(order):
-                    self._load_x_rows(s, nxt, order[n + 1])
+                if n + 1 < len(order_all):
+                    self._load_x_rows(s, nxt, order_all[n + 1])
                 s("__syncthreads();")
-                s.open("if (act)")
+                s.open(f"if (act{vp.vo})")
                 s("#pragma unroll")
                 s.open(f"for (int st = 0; st < {vp.U // 4}; ++st)")
                 for k in range(bo.d):
-                    s(f"acc[{k}] = {MFMA}(s_T[{buf}][{k}][4 * st + lq][l16], wreg{vp.index}[st], acc[{k}], 0, 0, 0);")
+                    s(f"acc{vp.vo}[{k}] = {MFMA}(s_T[{buf}][{k}][4 * st + lq][l16], wreg{vp.index}[st], "
+                      f"acc{vp.vo}[{k}], 0, 0, 0);")
                 s.close()
                 s.close()
                 cur, nxt = nxt, cur
             # D layout: rows 4*lq + i, column (channel) l16 of the wave's slice
-            s("#pragma unroll")
-            s.open("for (int i = 0; i < 4; ++i)")
-            s("const i64 row = row0 + 4 * lq + i;")
-            s.open("if (act && row < num_batch)")
-            s(f"T* zp = L3_out + row * {low.L3} + {bo.off} + (wave * 16 + l16) * {bo.d};")
-            for k in range(bo.d):
-                s(f"zp[{k}] {'=' if first else '+='} acc[{k}][i];")
-            s.close()
-            s.close()
+            for vo, _, first in ker:
+                bo = self.vout[vo]
+                s("#pragma unroll")
+                s.open("for (int i = 0; i < 4; ++i)")
+                s("const i64 row = row0 + 4 * lq + i;")
+                s.open(f"if (act{vo} && row < num_batch)")
+                s(f"T* zp = L3_out + row * {low.L3} + {bo.off} + (wave * 16 + l16) * {bo.d};")
+                for k in range(bo.d):
+                    s(f"zp[{k}] {'=' if first else '+='} acc{vo}[{k}][i];")
+                s.close()
+                s.close()
             s.close()
             s.close()
         return names
@@ -630,42 +659,51 @@ class MfmaEmitter:
             raise AssertionError("no path")
 
         # ---------------- dW ----------------------------------------------------
-        for vo, order, _first in _groups(self.vpaths, "vo", len(self.vout)):
-            if not order:
-                continue
-            bo = self.vout[vo]
-            name = f"backward_w{vo}_{order[0].ub}"
+        cost = lambda ker: (sum(4 * (vp.Wn // 16) for g in ker for vp in g[1]) + 2 * (RT // WAVES) * self.max_d1
+                            + 4 * max(self.vout[g[0]].mul // 16 for g in ker) + 64)
+        groups = [g for g in _groups(self.vpaths, "vo", len(self.vout)) if g[1]]
+        for ker in self._merge(groups, cost, self.tune["uvw_wregs"]):
+            # pieces that share a kernel must be neighbours in the row: one dZ tile covers their columns
+            pieces = [self.vout[vo] for vo, _, _ in ker]
+            if any(a.off + a.mul * a.d != b.off for a, b in zip(pieces, pieces[1:])):
+                raise AssertionError("merged output pieces are not contiguous")
+            order_all = [vp for _, order, _ in ker for vp in order]
+            col0 = pieces[0].off
+            ncols = pieces[-1].off + pieces[-1].mul * pieces[-1].d - col0
+            maxd = max(b.d for b in pieces)
+            name = f"backward_w{ker[0][0]}_{order_all[0].ub}"
             names.append(name)
-            s(f"// ======== dW of the sub-paths into out piece {vo} from input pieces {order[0].ub}")
+            s("// ======== dW of the sub-paths into out pieces " + ", ".join(str(vo) for vo, _, _ in ker))
             self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_ww"])
-            # only this piece's columns of the dZ tile are needed (and kept)
-            s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self._tile_stride(bo.mul * bo.d)}];")
-            s(f"__shared__ T s_T[2][{bo.d}][64][{TPAD}];")
+            # only these pieces' columns of the dZ tile are needed (and kept)
+            s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self._tile_stride(ncols)}];")
+            s(f"__shared__ T s_T[2][{maxd}][64][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             self._prologue(s)
             s("const int u = wave * 16 + l16;")
             s(f"T* prow = wpartial + (i64)blockIdx.x * {low.WN};")
             s(f"T xa[{RT // WAVES}][{self.max_d1}], xb[{RT // WAVES}][{self.max_d1}];")
             # dw<path>[n]: D tile rows = channels u of the wave's slice, columns = w in 16 n .. 16 n + 15
-            ntile = bo.mul // 16
-            for vp in order:
+            for vp in order_all:
+                ntile = vp.Wn // 16
                 s(f"v4f dw{vp.index}[{ntile}];")
                 s(f"for (int n = 0; n < {ntile}; ++n) dw{vp.index}[n] = v4f{{0.f, 0.f, 0.f, 0.f}};")
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
             s(f"const i64 row0 = tile * {RT};")
             s("__syncthreads();")
-            self._stage_g(s, bo.off, bo.mul * bo.d, local=True)
+            self._stage_g(s, col0, ncols, local=True)
             self._stage_y(s)
-            self._load_x_rows(s, "xa", order[0])
+            self._load_x_rows(s, "xa", order_all[0])
             s("__syncthreads();")
             cur, nxt = "xa", "xb"
-            for n, vp in enumerate(order):
+            for n, vp in enumerate(order_all):
                 p = vp.p
+                bo = self.vout[vp.vo]
                 buf = n % 2
                 s(f"// path {p.index}: l=({low.in1[p.i1].l},{low.in2[p.i2].l},{bo.l})")
                 self._t_compute(s, vp, cur, str(buf))
-                if n + 1 < len(order):
-                    self._load_x_rows(s, nxt, order[n + 1])
+                if n + 1 < len(order_all):
+                    self._load_x_rows(s, nxt, order_all[n + 1])
                 s("__syncthreads();")
                 # dW[u, w] += sum_(k,r) T[(k,r), u] * dZ[(k,r), w]   (A = T^T, B = dZ tile)
                 s.open(f"if (wave * 16 < {vp.U})")
@@ -674,15 +712,16 @@ class MfmaEmitter:
                 s("const int kq = 4 * st + lq;")
                 s("const int kk = kq >> 4, rr = kq & 15;")
                 s(f"const T a = s_T[{buf}][kk][u][rr];")
-                for nn in range(ntile):
-                    s(f"dw{vp.index}[{nn}] = {MFMA}(a, s_g[rr][({16 * nn} + l16) * {bo.d} + kk], dw{vp.index}[{nn}], 0, 0, 0);")
+                for nn in range(vp.Wn // 16):
+                    s(f"dw{vp.index}[{nn}] = {MFMA}(a, s_g[rr][{bo.off - col0} + ({16 * nn} + l16) * {bo.d} + kk], "
+                      f"dw{vp.index}[{nn}], 0, 0, 0);")
                 s.close()
                 s.close()
                 cur, nxt = nxt, cur
             s.close()
-            for vp in order:
+            for vp in order_all:
                 s.open(f"if (wave * 16 < {vp.U})")
-                for nn in range(ntile):
+                for nn in range(vp.Wn // 16):
                     s("#pragma unroll")
                     s.open("for (int i = 0; i < 4; ++i)")
                     s(f"prow[{vp.woff} + (wave * 16 + 4 * lq + i) * {vp.ld} + {16 * nn} + l16] = dw{vp.index}[{nn}][i];")
