@@ -162,7 +162,7 @@ class MfmaEmitter:
         self.gstride = self._tile_stride(low.L3)
         from .uvu import tuning
         self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2, uvw_pipe=1, uvw_regs=220, uvw_dma=0,
-                                uvw_merge=1, uvw_fregs=232, uvw_wregs=232))
+                                uvw_merge=1, uvw_fregs=232, uvw_wregs=232, uvw_xregs=215))
 
     def lit(self, v):
         return float_literal(v, "float")
@@ -312,7 +312,7 @@ class MfmaEmitter:
             s(f"s_T[{buf}][{k}][lane][r] = t[{k}];")
         s.close()
 
-    def _dx_paths(self, s: Src, paths: List[VPath]):
+    def _dx_paths(self, s: Src, paths: List[VPath], x: str = "x", dx: str = "dx"):
         """G = dZ W^T of every sub-path on the matrix cores, then its CG part on the vector ALU (in scope:
         x, dx, dy, s_g, s_y, wreg<path>). ``uvw_pipe`` = 0: path after path, operand order left to the
         compiler. 1: the A operands (dZ values from LDS) are fetched one chunk of 4 k-steps ahead of the
@@ -328,7 +328,7 @@ class MfmaEmitter:
             s(f"T Gk[{d3}];")
             for k in range(d3):
                 s(f"Gk[{k}] = {G}[{k}][i];")
-            s(f"cg_bwd{vp.p.index}(x[i], s_y[4 * lq + i], Gk, dx[i], dy[i]);")
+            s(f"cg_bwd{vp.p.index}({x}[i], s_y[4 * lq + i], Gk, {dx}[i], dy[i]);")
             s.close()
 
         if pipe == 0:
@@ -416,7 +416,7 @@ class MfmaEmitter:
         s.close()
 
     # ------------------------------------------------------------- forward
-    def _load_wreg(self, s: Src, vps: List[VPath], transposed: bool, act: str = "act"):
+    def _load_wreg(self, s: Src, vps: List[VPath], transposed: bool, act: str = "act", u: str = "u"):
         """Weight slices in MFMA B-operand layout, 1 register per 4 k-steps... per k-step of 4: forward
         B[k = u' = 4 st + lq][n = l16] = W[u'][w = 16 wave + l16] (U / 4 registers); backward (transposed)
         B[k = w = 4 st + lq][n = l16] = W[u][w] (Wn / 4 registers). Waves without channels in the piece load
@@ -427,7 +427,7 @@ class MfmaEmitter:
             s("#pragma unroll")
             if transposed:
                 s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = {act} ? "
-                  f"W[{vp.woff} + u * {vp.ld} + 4 * st + lq] : T(0);")
+                  f"W[{vp.woff} + {u} * {vp.ld} + 4 * st + lq] : T(0);")
             else:
                 s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = {act} ? "
                   f"W[{vp.woff} + (4 * st + lq) * {vp.ld} + wave * 16 + l16] : T(0);")
@@ -456,7 +456,7 @@ class MfmaEmitter:
         s.close()
         s.close()
 
-    def _merge(self, groups, cost, limit):
+    def _merge(self, groups, cost, limit, blocks):
         """Consecutive (piece, sub-paths, first) groups that share a kernel: a group joins the kernel before
         it while the kernel's estimated registers stay within ``limit``. Kernels of narrow output irreps
         (l = 0: one multiply per k-step) are dominated by what every kernel pays per tile - staging, barriers,
@@ -466,7 +466,7 @@ class MfmaEmitter:
             prev = kernels[-1][-1] if kernels else None
             # only neighbours in the row share a kernel (one dZ tile then covers their columns)
             adjacent = prev is not None and prev[0] != g[0] and \
-                self.vout[prev[0]].off + self.vout[prev[0]].mul * self.vout[prev[0]].d == self.vout[g[0]].off
+                blocks[prev[0]].off + blocks[prev[0]].mul * blocks[prev[0]].d == blocks[g[0]].off
             if adjacent and g[1] and prev[1] and self.tune["uvw_merge"] and cost(kernels[-1] + [g]) <= limit:
                 kernels[-1].append(g)
             else:
@@ -481,7 +481,7 @@ class MfmaEmitter:
         names = []
         cost = lambda ker: (sum(vp.U // 4 for g in ker for vp in g[1]) + sum(4 * self.vout[g[0]].d for g in ker)
                             + 2 * (RT // WAVES) * self.max_d1 + 64)
-        for ker in self._merge(_groups(self.vpaths, "vo", len(self.vout)), cost, self.tune["uvw_fregs"]):
+        for ker in self._merge(_groups(self.vpaths, "vo", len(self.vout)), cost, self.tune["uvw_fregs"], self.vout):
             vo0, order0, _ = ker[0]
             name = "forward" if not names else f"forward_o{vo0}_{order0[0].ub if order0 else 0}"
             names.append(name)
@@ -555,15 +555,21 @@ class MfmaEmitter:
         names = []
         # ---------------- dX, dY ------------------------------------------------
         first_dy = True
-        for vi, paths, first in _groups(self.vpaths, "vi", len(self.vin)):
-            b1 = self.vin[vi]
-            name = "backward" if not names else f"backward_x{vi}_{paths[0].wb if paths else 0}"
+        # registers per lane: one per 4 k-steps of a resident weight slice, the 4 rows' x / dx per piece, dy, G
+        # and the operand chunks
+        fixed = lambda ker: (sum(8 * self.vin[g[0]].d for g in ker) + 4 * low.L2
+                             + 6 * max(self.vout[vp.vo].d for g in ker for vp in g[1]) + 48)
+        cost = lambda ker: sum(vp.Wn // 4 for g in ker for vp in g[1]) + fixed(ker)
+        for ker in self._merge(_groups(self.vpaths, "vi", len(self.vin)), cost, self.tune["uvw_xregs"], self.vin):
+            vi0, paths0, _ = ker[0]
+            name = "backward" if not names else f"backward_x{vi0}_{paths0[0].wb if paths0 else 0}"
             names.append(name)
-            s(f"// ======== in1 piece {vi}: {b1.mul} x l={b1.l} at {b1.off}")
+            s("// ======== in1 pieces " + ", ".join(f"{vi}: {self.vin[vi].mul} x l={self.vin[vi].l}" for vi, _, _ in ker))
             self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_wx"])
-            if not paths:
-                self._zero_kernel(s, "L1_grad", low.L1, b1)
+            if not paths0:
+                self._zero_kernel(s, "L1_grad", low.L1, self.vin[vi0])
                 continue
+            paths_all = [vp for _, ps, _ in ker for vp in ps]
             # the dZ tile: staged through registers, or (uvw_dma) written by direct global->LDS loads into one of
             # two buffers while the other tile is worked on
             dma = bool(self.tune["uvw_dma"]) and low.L3 % 4 == 0
@@ -573,28 +579,29 @@ class MfmaEmitter:
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             s(f"__shared__ T s_dy[{WAVES}][{RT}][{low.L2}];")
             self._prologue(s)
-            s(f"const bool act = wave * 16 < {b1.mul};  // this wave has input channels in the piece")
-            s("const int u = act ? wave * 16 + l16 : 0;  // channel of this lane in the MFMA result layout")
-            # Registers per lane: one per 4 k-steps of a resident weight slice, the 4 rows' x / dx / dy, G and
-            # the operand chunks. Where that exceeds the budget of two waves per SIMD, the slices of the paths
-            # with the fewest multiplies are kept in LDS instead (read like the A operands, one chunk ahead):
-            # spilled slices would come back from scratch memory in the middle of the multiply sequence.
-            fixed = 4 * (self.max_d1 + b1.d + low.L2) + 6 * max(self.vout[vp.vo].d for vp in paths) + 48
-            by_cost = sorted(paths, key=lambda vp: (self.vout[vp.vo].d, vp.index))
+            for vi, _, _ in ker:
+                s(f"const bool act{vi} = wave * 16 < {self.vin[vi].mul};  // this wave has input channels in the piece")
+                s(f"const int u{vi} = act{vi} ? wave * 16 + l16 : 0;  // channel of this lane in the MFMA result layout")
+            # Where the registers exceed the budget of two waves per SIMD, the weight slices of the paths with
+            # the fewest multiplies are kept in LDS instead (read like the A operands, one chunk ahead): spilled
+            # slices would come back from scratch memory in the middle of the multiply sequence.
+            by_cost = sorted(paths_all, key=lambda vp: (self.vout[vp.vo].d, vp.index))
             self.lds_w = []
             if self.tune["uvw_pipe"]:
-                resident = lambda: sum(vp.Wn // 4 for vp in paths if vp.index not in self.lds_w)
-                while len(paths) - len(self.lds_w) > 1 and len(self.lds_w) < 3 and \
-                        resident() + fixed > self.tune["uvw_regs"]:
+                resident = lambda: sum(vp.Wn // 4 for vp in paths_all if vp.index not in self.lds_w)
+                while len(paths_all) - len(self.lds_w) > 1 and len(self.lds_w) < 3 and \
+                        resident() + fixed(ker) > self.tune["uvw_regs"]:
                     self.lds_w.append(by_cost[len(self.lds_w)].index)
             if self.lds_w:
                 s(f"__shared__ T s_wl[{len(self.lds_w)}][16][{64 * WAVES}];")
-            self._load_wreg(s, [vp for vp in paths if vp.index not in self.lds_w], transposed=True)
+            for vi, ps, _ in ker:
+                self._load_wreg(s, [vp for vp in ps if vp.index not in self.lds_w], transposed=True,
+                                act=f"act{vi}", u=f"u{vi}")
             for n, pi in enumerate(self.lds_w):
-                vp = next(q for q in paths if q.index == pi)
+                vp = next(q for q in paths_all if q.index == pi)
                 s("#pragma unroll")
                 s(f"for (int st = 0; st < {vp.Wn // 4}; ++st) s_wl[{n}][st][tid] = "
-                  f"act ? W[{vp.woff} + u * {vp.ld} + 4 * st + lq] : T(0);")
+                  f"act{vp.vi} ? W[{vp.woff} + u{vp.vi} * {vp.ld} + 4 * st + lq] : T(0);")
             if dma:
                 s("int buf = 0;")
                 s("if ((i64)blockIdx.x < ntiles) {")
@@ -608,13 +615,19 @@ class MfmaEmitter:
                 self._stage_g(s)
             self._stage_y(s)
             # X of the lane's 4 (row, channel) pairs: issued before the barrier and the MFMA loop
-            s(f"T x[4][{self.max_d1}], dx[4][{b1.d}], dy[4][{low.L2}];")
+            s(f"T dy[4][{low.L2}];")
+            for vi, _, _ in ker:
+                s(f"T x{vi}[4][{self.max_d1}], dx{vi}[4][{self.vin[vi].d}];")
             s("#pragma unroll")
             s.open("for (int i = 0; i < 4; ++i)")
             s("i64 row = row0 + 4 * lq + i; if (row >= num_batch) row = num_batch - 1;")
-            s(f"const T* xp = L1_in + row * {low.L1} + {b1.off} + u * {b1.d};")
-            for c in range(b1.d):
-                s(f"x[i][{c}] = xp[{c}]; dx[i][{c}] = T(0);")
+            for vi, _, _ in ker:
+                b1 = self.vin[vi]
+                s.open("")
+                s(f"const T* xp = L1_in + row * {low.L1} + {b1.off} + u{vi} * {b1.d};")
+                for c in range(b1.d):
+                    s(f"x{vi}[i][{c}] = xp[{c}]; dx{vi}[i][{c}] = T(0);")
+                s.close()
             s(f"for (int j = 0; j < {low.L2}; ++j) dy[i][j] = T(0);")
             s.close()
             if dma:
@@ -630,18 +643,20 @@ class MfmaEmitter:
                 s(fence)
             else:
                 s("__syncthreads();")
-            s.open("if (act)")
-            self._dx_paths(s, paths)
-            s("#pragma unroll")
-            s.open("for (int i = 0; i < 4; ++i)")
-            s("const i64 row = row0 + 4 * lq + i;")
-            s.open("if (row < num_batch)")
-            s(f"T* dp = L1_grad + row * {low.L1} + {b1.off} + u * {b1.d};")
-            for c in range(b1.d):
-                s(f"dp[{c}] {'=' if first else '+='} dx[i][{c}];")
-            s.close()
-            s.close()
-            s.close()
+            for vi, ps, first in ker:
+                b1 = self.vin[vi]
+                s.open(f"if (act{vi})")
+                self._dx_paths(s, ps, f"x{vi}", f"dx{vi}")
+                s("#pragma unroll")
+                s.open("for (int i = 0; i < 4; ++i)")
+                s("const i64 row = row0 + 4 * lq + i;")
+                s.open("if (row < num_batch)")
+                s(f"T* dp = L1_grad + row * {low.L1} + {b1.off} + u{vi} * {b1.d};")
+                for c in range(b1.d):
+                    s(f"dp[{c}] {'=' if first else '+='} dx{vi}[i][{c}];")
+                s.close()
+                s.close()
+                s.close()
             # dY: sum over the 16 channels of the lane group, then over the 4 waves through LDS
             self._reduce_dy(s)
             s("__syncthreads();")
@@ -662,7 +677,7 @@ class MfmaEmitter:
         cost = lambda ker: (sum(4 * (vp.Wn // 16) for g in ker for vp in g[1]) + 2 * (RT // WAVES) * self.max_d1
                             + 4 * max(self.vout[g[0]].mul // 16 for g in ker) + 64)
         groups = [g for g in _groups(self.vpaths, "vo", len(self.vout)) if g[1]]
-        for ker in self._merge(groups, cost, self.tune["uvw_wregs"]):
+        for ker in self._merge(groups, cost, self.tune["uvw_wregs"], self.vout):
             # pieces that share a kernel must be neighbours in the row: one dZ tile covers their columns
             pieces = [self.vout[vo] for vo, _, _ in ker]
             if any(a.off + a.mul * a.d != b.off for a, b in zip(pieces, pieces[1:])):
