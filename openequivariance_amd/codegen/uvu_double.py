@@ -35,7 +35,7 @@ from .uvu import UvuEmitter
 # they no longer beat the composition of first-order kernels (measured: SevenNet main layer, 38 paths,
 # 63 - 80 ms against 66 ms; NequIP benzene, 68 paths, 155 - 175 ms against 118 ms; NequiX main layer, 27
 # paths, 28 against 35 ms). The batch kernels are 3 - 4 times faster than the composition for all of them.
-CONV_MAX_PATHS = 32
+CONV_MAX_PATHS = 96
 
 
 def supported(low: Lowered, conv: bool = False) -> bool:
@@ -691,7 +691,30 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     """Append the convolution double-backward kernels (receiver-major walk) to a module."""
     from .. import runtime as rt
 
-    em = DoubleEmitter(low, acc_budget_words=tune.get("dd_acc", 112))
+    def kernel_a_need(e: DoubleEmitter) -> int:
+        """Registers kernel A needs for its widest output segment: the accumulators, X and A of the input
+        blocks the segment's paths read, one W and one C value per path."""
+        worst = 0
+        for si, seg in enumerate(e.segments):
+            acc = sum(low.out[io].d for io in seg)
+            xin = sum(low.in1[b].d for b in e.seg_in1[si])
+            wc = sum(2 * low.in2[p.i2].mul for p in low.paths if p.io in seg)
+            worst = max(worst, e.words * (acc + 2 * xin + wc))
+        return worst
+
+    # Output segment size of kernel A: 112 accumulator words where the widest segment then fits (the MACE
+    # shape: one segment, 177 words); problems with many paths per output block (SevenNet, NequIP benzene)
+    # spill there, up to 149 registers, and take the largest budget that leaves the widest segment under
+    # 160 words - with the spills the fused pair was slower than composing first-order kernels.
+    if tune.get("dd_acc", 0) > 0:
+        em = DoubleEmitter(low, acc_budget_words=tune["dd_acc"])
+    else:
+        em = DoubleEmitter(low, acc_budget_words=112)
+        if kernel_a_need(em) > 200:
+            for budget in (80, 64, 48, 32):
+                em = DoubleEmitter(low, acc_budget_words=budget)
+                if kernel_a_need(em) <= 160:
+                    break
     em.nt = base.nt
     em.mask_loads = base.mask_loads
     em.tr_stores = base.tr_stores
