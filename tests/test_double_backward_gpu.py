@@ -203,10 +203,17 @@ def test_edge_cases_and_refusals():
     assert all(torch.isfinite(t).all() for t in second)
 
 
-def test_many_path_convolutions_use_the_composition():
+def test_path_limit_of_the_fused_convolution_kernels(monkeypatch):
+    """Convolutions with up to 96 paths get fused second-order kernels (SevenNet main layer: 38, NequIP
+    benzene: 68); beyond the limit (lowered here through its knob) the kernel set has none and autograd
+    composes first-order kernels."""
     from openequivariance_amd.codegen.lower import lower
-    assert not uvu_double.supported(lower(P.seven_net_problems()[1]), conv=True)
-    assert uvu_double.supported(lower(P.seven_net_problems()[1]))
+    low = lower(P.seven_net_problems()[1])
+    assert uvu_double.supported(low, conv=True) and uvu_double.supported(low)
+    conv = oeq.TensorProductConv(P.seven_net_problems()[1], deterministic=True)
+    assert ops.get_entry(conv.kid).kernels().has_double_backward()
+    monkeypatch.setenv("OEQ_AMD_TUNE", "dd_maxp=32")
+    assert not uvu_double.supported(low, conv=True)
     conv = oeq.TensorProductConv(P.seven_net_problems()[1], deterministic=True)
     assert not ops.get_entry(conv.kid).kernels().has_double_backward()
 
@@ -280,7 +287,9 @@ def test_tp_fused_matches_float64_autograd(name, make, batch):
 
 
 ORACLE_CONV = [("cfg2", P.config2_nequip_uvu), ("cfg5", P.config5_mace_conv),
-               ("cfg5-f64", lambda: _f64(P.config5_mace_conv())), ("folded-gaps", _folded), ("odd", _odd)]
+               ("cfg5-f64", lambda: _f64(P.config5_mace_conv())), ("folded-gaps", _folded), ("odd", _odd),
+               # many paths per output block: kernel A walks smaller output segments (38 and 68 paths)
+               ("sevennet-main", lambda: P.seven_net_problems()[1]), ("nequip-benzene", lambda: P.nequip_problems()[3])]
 
 
 @pytest.mark.parametrize("det", [True, False], ids=["sorted", "grouped"])
