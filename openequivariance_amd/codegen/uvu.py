@@ -74,6 +74,7 @@ class UvuEmitter:
         # non-temporally (batch kernels only: the convolution re-reads them).
         self.nt = 0
         self.mask_loads = False  # zero X and W values in lanes without a channel (see _operand)
+        self.forms = True  # per path, put the CG coefficient on the factor with the fewest distinct products
         self.sched_fence = False
         self.fence_words = 0  # gradient registers between two scheduling fences (0: a fence after every path)
         self.prefetch_runs = False  # request the next run's gradients and weights while a run computes
@@ -567,6 +568,41 @@ class UvuEmitter:
             out[n] = (names[key], c < 0)
         return out
 
+    def _form_counts(self, p: Path):
+        """Distinct (|c|, j), (|c|, i), (|c|, k) pairs and distinct |c| of a path: what it costs to carry
+        the coefficient on the Y value, on the X value, on the output, and to fold the weight into it."""
+        mag = lambda c: self.lit(abs(c))
+        cj = len({(mag(c), j) for _, j, _, c in p.nnz})
+        ci = len({(mag(c), i) for i, _, _, c in p.nnz})
+        ck = len({(mag(c), k) for _, _, k, c in p.nnz})
+        nc = len({mag(c) for _, _, _, c in p.nnz})
+        return cj, ci, ck, nc
+
+    def _y_values(self, s: Src, p: Path, v: str, yacc):
+        for j in sorted({j for _, j, _, _ in p.nnz}):
+            s(f"const T y{j} = {yacc(p, v, j)};")
+
+    def _scaled(self, s: Src, p: Path, which: int, operand, prefix: str, weight: Optional[str] = None):
+        """Emit the distinct products |c| * operand(index) of a path, index = component ``which`` of an
+        nnz entry (0: i, 1: j, 2: k); with ``weight`` the coefficient is |c| * weight, formed once per
+        distinct |c|. Returns nnz index -> (name, negative)."""
+        cw = {}
+        if weight is not None:
+            for _, _, _, c in p.nnz:
+                m = self.lit(abs(c))
+                if m not in cw:
+                    cw[m] = f"cw{len(cw)}"
+                    s(f"const T {cw[m]} = T({m}) * {weight};")
+        names, out = {}, {}
+        for n, ent in enumerate(p.nnz):
+            key = (self.lit(abs(ent[3])), ent[which])
+            if key not in names:
+                names[key] = f"{prefix}{len(names)}"
+                coef = cw[key[0]] if weight is not None else f"T({key[0]})"
+                s(f"const T {names[key]} = {coef} * {operand(ent[which])};")
+            out[n] = (names[key], ent[3] < 0)
+        return out
+
     def _load_x(self, s: Src, rowexpr: str, blocks: List[int], dst: str = "x"):
         low = self.low
         for b in self._in1_of(blocks):
@@ -699,16 +735,50 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             if self.use_q:
                 self._emit_q_fetch(s, qplan[n_p])
 
-            def body(v, p=p):
-                prods = self._products(s, p, v, yacc)
+            def body(v, p=p, bo=bo):
+                # The coefficient of a term rides on whichever factor has the fewest distinct (|c|, index)
+                # pairs in this path: the Y value, the X value, or - summing the +-x_i*y_j of equal |c| first -
+                # the output, where it is folded into the weight (no separate scaling of the outputs then).
+                cj, ci, ck, nc = self._form_counts(p)
+                n = len(p.nnz)
+                form = 0
+                if self.forms and not self.use_q:
+                    costs = [cj + n + bo.d, ci + n + bo.d, n + nc + ck]
+                    form = costs.index(min(costs))
+                if form == 2:
+                    self._y_values(s, p, v, yacc)
+                    sums = {}
+                    for i, j, k, c in p.nnz:
+                        key = (self.lit(abs(c)), k)
+                        term = f"{self._xv(xname, p.i1, i)} * y{j}"
+                        if key not in sums:
+                            sums[key] = f"s{len(sums)}"
+                            s(f"T {sums[key]} = {'-' if c < 0 else ''}{term};")
+                        else:
+                            s(f"{sums[key]} {'-=' if c < 0 else '+='} {term};")
+                    s(f"const T wv = {wacc(p, v)};")
+                    cw = {}
+                    for (m, k), name in sums.items():
+                        if m not in cw:
+                            cw[m] = f"cw{len(cw)}"
+                            s(f"const T {cw[m]} = T({m}) * wv;")
+                        s(f"a.o{p.io}[{k}] += {cw[m]} * {name};")
+                    return
+                if form == 1:
+                    self._y_values(s, p, v, yacc)
+                    prods = self._scaled(s, p, 0, lambda i: self._xv(xname, p.i1, i), "qx")
+                    other = lambda i, j: f"y{j}"
+                else:
+                    prods = self._products(s, p, v, yacc)
+                    other = lambda i, j: self._xv(xname, p.i1, i)
                 started = set()
-                for n, (i, j, k, c) in enumerate(p.nnz):
-                    q, neg = prods[n]
+                for n_, (i, j, k, c) in enumerate(p.nnz):
+                    q, neg = prods[n_]
                     if k not in started:
-                        s(f"T t{k} = {'-' if neg else ''}{q} * {self._xv(xname, p.i1, i)};")
+                        s(f"T t{k} = {'-' if neg else ''}{q} * {other(i, j)};")
                         started.add(k)
                     else:
-                        s(f"t{k} {'-=' if neg else '+='} {q} * {self._xv(xname, p.i1, i)};")
+                        s(f"t{k} {'-=' if neg else '+='} {q} * {other(i, j)};")
                 s(f"const T wv = {wacc(p, v)};")
                 for k in sorted(started):
                     s(f"a.o{p.io}[{k}] += wv * t{k};")
@@ -1215,16 +1285,62 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             base_slot = self.wslot[p.index]
 
             def body(v, p=p, b1=b1, b2=b2, V=V, gname=gname, base_slot=base_slot):
-                prods = self._products(s, p, v, yacc)
-                s(f"const T wv = {f'wv{p.index}_{v}' if prefetch else wacc(p, v)};")
                 ks = sorted({k for _, _, k, _ in p.nnz})
                 js = sorted({j for _, j, _, _ in p.nnz})
-                # dX: dx_i += (|c| y_j) * (g_k w)
-                for k in ks:
-                    s(f"const T gw{k} = {gname(k)} * wv;")
-                for n, (i, j, k, c) in enumerate(p.nnz):
-                    q, neg = prods[n]
-                    s(f"dx.b{p.i1}[{i}] {'-=' if neg else '+='} {q} * gw{k};")
+                # dX: dx_i += c * y_j * g_k * w. As in the forward pass the coefficient rides on the factor
+                # with the fewest distinct (|c|, index) pairs - Y, the weighted gradient, or (after summing the
+                # +-y_j*g_k of equal |c|) the result - and the weight on the gradient values or on the coefficient.
+                cj, ci, ck, nc = self._form_counts(p)
+                nz = len(p.nnz)
+                form = 0
+                if self.forms and not self.use_q:
+                    costs = [cj + min(len(ks), nc) + nz, ck + min(len(ks), nc) + nz, nz + nc + ci]
+                    form = costs.index(min(costs))
+                    if form < 2 and nc < len(ks):
+                        form += 3  # weight folded into the coefficient instead of into the gradient values
+                wv_expr = f"wv{p.index}_{v}" if prefetch else wacc(p, v)
+                if form == 0:
+                    prods = self._products(s, p, v, yacc)
+                    s(f"const T wv = {wv_expr};")
+                    for k in ks:
+                        s(f"const T gw{k} = {gname(k)} * wv;")
+                    for n, (i, j, k, c) in enumerate(p.nnz):
+                        q, neg = prods[n]
+                        s(f"dx.b{p.i1}[{i}] {'-=' if neg else '+='} {q} * gw{k};")
+                else:
+                    self._y_values(s, p, v, yacc)
+                    s(f"const T wv = {wv_expr};")
+                    if form == 1:
+                        for k in ks:
+                            s(f"const T gw{k} = {gname(k)} * wv;")
+                        prods = self._scaled(s, p, 2, lambda k: f"gw{k}", "qg")
+                        other = lambda j, k: f"y{j}"
+                    elif form == 3:
+                        prods = self._scaled(s, p, 1, lambda j: f"y{j}", "q", weight="wv")
+                        other = lambda j, k: gname(k)
+                    elif form == 4:
+                        prods = self._scaled(s, p, 2, gname, "qg", weight="wv")
+                        other = lambda j, k: f"y{j}"
+                    if form == 2:
+                        sums = {}
+                        for i, j, k, c in p.nnz:
+                            key = (self.lit(abs(c)), i)
+                            term = f"y{j} * {gname(k)}"
+                            if key not in sums:
+                                sums[key] = f"sx{len(sums)}"
+                                s(f"T {sums[key]} = {'-' if c < 0 else ''}{term};")
+                            else:
+                                s(f"{sums[key]} {'-=' if c < 0 else '+='} {term};")
+                        cw = {}
+                        for (m, i), name in sums.items():
+                            if m not in cw:
+                                cw[m] = f"cw{len(cw)}"
+                                s(f"const T {cw[m]} = T({m}) * wv;")
+                            s(f"dx.b{p.i1}[{i}] += {cw[m]} * {name};")
+                    else:
+                        for n, (i, j, k, c) in enumerate(p.nnz):
+                            q, neg = prods[n]
+                            s(f"dx.b{p.i1}[{i}] {'-=' if neg else '+='} {q} * {other(j, k)};")
                 # h_j = sum_ik c x_i g_k is the unweighted dY term of this lane; it also gives
                 # dW = sum_j y_j h_j, so the forward contraction need not be recomputed
                 pair, hstart = {}, set()
@@ -1920,10 +2036,11 @@ def tp_module(low: Lowered, compute_units: int = 256):
                     tp_wf=2 if f32 else 0, tp_wb=3 if (big and not pf_ok) else 2, tp_nt=0,
                     tp_gres=0 if on_demand else 1,
                     tp_sb=1 if on_demand else 0, tp_trs=1, tp_fw=64, tp_pf=1,
-                    tp_dd=1, dd_wa=2, dd_wb=2, tp_mask=0))
+                    tp_dd=1, dd_wa=2, dd_wb=2, tp_mask=0, tp_forms=1))
     em = UvuEmitter(low, acc_budget_words=t["tp_acc"])
     em.nt = t["tp_nt"]
     em.mask_loads = bool(t["tp_mask"])
+    em.forms = bool(t["tp_forms"])
     em.sched_fence = bool(t["tp_sb"])
     em.fence_words = t["tp_fw"]
     em.prefetch_runs = bool(t["tp_pf"])
@@ -1973,7 +2090,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=0, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
                     dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fw=0, conv_pf=0,
-                    conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0))
+                    conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0, tp_forms=1))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -2025,6 +2142,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     break
     em.nt = t["conv_nt"]
     em.mask_loads = bool(t["tp_mask"])
+    em.forms = bool(t["tp_forms"])
     q_fwd = q_bwd = False
     if t["conv_q"] and em.q_supported():
         # bit 0: forward, bit 1: backward. Backward gains nothing at the MACE shape (it is bound by its
