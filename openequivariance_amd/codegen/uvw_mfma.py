@@ -161,7 +161,7 @@ class MfmaEmitter:
         # k-steps d words apart (d odd), fall into 32 different banks.
         self.gstride = self._tile_stride(low.L3)
         from .uvu import tuning
-        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2, uvw_pipe=1, uvw_regs=220, uvw_dma=0,
+        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2, uvw_pipe=1, uvw_regs=220,
                                 uvw_merge=1, uvw_fregs=232, uvw_wregs=232, uvw_xregs=215))
 
     def lit(self, v):
@@ -272,21 +272,6 @@ class MfmaEmitter:
             s.open(f"for (int t = tid; t < {RT * ncols}; t += {nthreads})")
             s(f"const int r = t / {ncols}, c = t % {ncols};")
             s(f"s_g[r][{dst0} + c] = (row0 + r < num_batch) ? L3_grad[(row0 + r) * {low.L3} + {col0} + c] : T(0);")
-            s.close()
-
-    def _dma_g(self, s: Src, tile: str, buf: str):
-        """Request the dZ rows of a tile into s_g[buf] with direct global->LDS loads (each wave its 4 rows,
-        64 lanes x 16 bytes per instruction, landing side by side in LDS). Rows past the end of the batch
-        repeat the last row: what is computed from them is never stored."""
-        low = self.low
-        rpw, nc4 = RT // WAVES, low.L3 // 4
-        for rr in range(rpw):
-            s.open("")
-            s(f"i64 grow = {tile} * {RT} + wave * {rpw} + {rr}; if (grow >= num_batch) grow = num_batch - 1;")
-            for j in range((nc4 + 63) // 64):
-                guard = f"if (lane + {64 * j} < {nc4}) " if (j + 1) * 64 > nc4 else ""
-                s(f"{guard}__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(L3_grad + grow * {low.L3} + 4 * (lane + {64 * j})), "
-                  f"(OEQ_LPTR)(&s_g[{buf}][wave * {rpw} + {rr}][{256 * j}]), 16, 0, 0);")
             s.close()
 
     def _load_x_rows(self, s: Src, dst: str, vp: VPath):
@@ -570,12 +555,8 @@ class MfmaEmitter:
                 self._zero_kernel(s, "L1_grad", low.L1, self.vin[vi0])
                 continue
             paths_all = [vp for _, ps, _ in ker for vp in ps]
-            # the dZ tile: staged through registers, or (uvw_dma) written by direct global->LDS loads into one of
-            # two buffers while the other tile is worked on
-            dma = bool(self.tune["uvw_dma"]) and low.L3 % 4 == 0
-            self.g_at = (lambda row, col: f"sg[{row} * {self.gstride} + {col}]") if dma else (
-                lambda row, col: f"s_g[{row}][{col}]")
-            s(f"__shared__ __attribute__((aligned(16))) T s_g[{'2][' if dma else ''}{RT}][{self.gstride}];")
+            self.g_at = lambda row, col: f"s_g[{row}][{col}]"
+            s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self.gstride}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             s(f"__shared__ T s_dy[{WAVES}][{RT}][{low.L2}];")
             self._prologue(s)
@@ -602,17 +583,10 @@ class MfmaEmitter:
                 s("#pragma unroll")
                 s(f"for (int st = 0; st < {vp.Wn // 4}; ++st) s_wl[{n}][st][tid] = "
                   f"act{vp.vi} ? W[{vp.woff} + u{vp.vi} * {vp.ld} + 4 * st + lq] : T(0);")
-            if dma:
-                s("int buf = 0;")
-                s("if ((i64)blockIdx.x < ntiles) {")
-                s.level += 1
-                self._dma_g(s, "(i64)blockIdx.x", "0")
-                s.close()
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
             s(f"const i64 row0 = tile * {RT};")
             s("__syncthreads();")
-            if not dma:
-                self._stage_g(s)
+            self._stage_g(s)
             self._stage_y(s)
             # X of the lane's 4 (row, channel) pairs: issued before the barrier and the MFMA loop
             s(f"T dy[4][{low.L2}];")
@@ -630,19 +604,7 @@ class MfmaEmitter:
                 s.close()
             s(f"for (int j = 0; j < {low.L2}; ++j) dy[i][j] = T(0);")
             s.close()
-            if dma:
-                # this wave's loads of the tile have landed; after the barrier, everybody's have, and nobody
-                # reads the other buffer any more: the next tile may be requested into it
-                fence = 'asm volatile("" ::: "memory");'
-                s(f"{fence} __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0) */ {fence}")
-                s("__syncthreads();")
-                s.open("if (tile + gridDim.x < ntiles)")
-                self._dma_g(s, "(tile + gridDim.x)", "(buf ^ 1)")
-                s.close()
-                s(f"const T* sg = &s_g[buf][0][0];")
-                s(fence)
-            else:
-                s("__syncthreads();")
+            s("__syncthreads();")
             for vi, ps, first in ker:
                 b1 = self.vin[vi]
                 s.open(f"if (act{vi})")
@@ -665,8 +627,6 @@ class MfmaEmitter:
             s("const T tot = ((s_dy[0][r][c] + s_dy[1][r][c]) + s_dy[2][r][c]) + s_dy[3][r][c];")
             s(f"if (row0 + r < num_batch) L2_grad[(row0 + r) * {low.L2} + c] {'=' if first_dy else '+='} tot;")
             s.close()
-            if dma:
-                s("buf ^= 1;")
             s.close()
             s.close()
             first_dy = False
