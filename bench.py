@@ -44,7 +44,7 @@ def parse():
     ap.add_argument("--with-double", action="store_true",
                     help="with --no-extras: still run the second-order (double backward) side measurement")
     ap.add_argument("--only-tp", default=None, metavar="N",
-                    help="run only the batched tensor-product side measurement for config N (1, 2, 3, 3d, 4, dd) "
+                    help="run only the batched tensor-product side measurement for config N (1, 2, 3, 3d, 4, 4d, dd) "
                          "and print its row; used for per-kernel profiles")
     return ap.parse_args()
 
@@ -142,9 +142,10 @@ def tp_config_table(dev, only=None):
     cases = [("cfg1 single uvu f32", P.config1_single_uvu(), 100000), ("cfg2 nequip uvu f32", P.config2_nequip_uvu(), 200000),
              ("cfg3 mace uvu f32", P.config3_mace_uvu(), 500000), ("cfg3 mace uvu f64", P.config3_mace_uvu(np.float64), 500000),
              ("cfg4 uvw shared f32 (MFMA)", P.config4_uvw_shared(), 262144),
+             ("cfg4 uvw shared f64 (MFMA)", P.config4_uvw_shared(np.float64), 131072),
              ("DiffDock L=1 uvw per-row weights f32", P.diffdock_problems()[0], 100000)]
     if only is not None:
-        cases = [cases[["1", "2", "3", "3d", "4", "dd"].index(only)]]
+        cases = [cases[["1", "2", "3", "3d", "4", "4d", "dd"].index(only)]]
     table = []
     for name, prob, B in cases:
         low = lower(prob)
@@ -169,8 +170,9 @@ def tp_config_table(dev, only=None):
             dense = sum(2 * low.in1[p.i1].mul * low.in2[p.i2].mul * low.out[p.io].mul * low.out[p.io].d for p in low.paths)
             row["fwd_dense_tflops"] = B * dense / tf / 1e9
             row["bwd_dense_tflops"] = 2 * B * dense / tb / 1e9
-            row["fwd_mfma_frac"] = row["fwd_dense_tflops"] / 157.3
-            row["bwd_mfma_frac"] = row["bwd_dense_tflops"] / 157.3
+            peak = 157.3 if es == 4 else 78.6  # dense MFMA TFLOP/s, fp32 / fp64
+            row["fwd_mfma_frac"] = row["fwd_dense_tflops"] / peak
+            row["bwd_mfma_frac"] = row["bwd_dense_tflops"] / peak
         table.append(row)
         del x, y, w, g
         torch.cuda.empty_cache()

@@ -1,10 +1,10 @@
-"""MFMA kernels for shared-weight 'uvw' tensor products (fp32).
+"""MFMA kernels for shared-weight 'uvw' tensor products (fp32 and fp64).
 
 With one weight tensor for the whole batch the channel mix of a path,
 ``Z[b][w,k] += sum_u W[u,w] * T[b][u,k]`` with ``T[b][u,k] = sum_ij c_ijk X[b][u,i] Y[b][j]``,
 is a dense GEMM once rows are batched: ``[(b,k)] x [u] x [w]``. These kernels
 run it on the matrix cores with ``v_mfma_f32_16x16x4_f32`` (true fp32, needed for
-the 1e-5 parity bound) and keep the sparse CG part on the vector ALU. The
+the 1e-5 parity bound) or ``v_mfma_f64_16x16x4_f64`` and keep the sparse CG part on the vector ALU. The
 reference does this mix with a scalar-FMA warp matmul on 32-wide chunks
 (openequivariance/openequivariance/templates/wmm.cuh:1-87,
 loop_unroll_tp.cuh:55-84, 217-272).
@@ -42,9 +42,10 @@ by the same thread of the same block, so the order of these additions is fixed):
 Splitting by irrep keeps each kernel under 256 registers (two waves per SIMD),
 so one wave's LDS/global latencies hide behind the other's MFMAs.
 
-Operand layouts of v_mfma_f32_16x16x4_f32 used below (lane l of 64):
+Operand layouts of the two 16x16x4 instructions used below (lane l of 64):
 A[m][k]: m = l % 16, k = l / 16;  B[k][n]: k = l / 16, n = l % 16;
-D[m][n]: n = l % 16, m = 4 * (l / 16) + i for the i-th of 4 result registers.
+D[m][n]: n = l % 16, and for the i-th of 4 result registers m = 4 * (l / 16) + i in fp32,
+m = l / 16 + 4 * i in fp64.
 """
 
 from __future__ import annotations
@@ -58,8 +59,14 @@ from .lower import Lowered, Path, float_literal
 RT = 16          # rows per tile
 WAVES = 4        # waves per block
 TPAD = RT + 1    # padded row stride of the T tile in LDS (bank spread)
-PIECE = 64       # channels per piece of an irrep block
-MFMA = "__builtin_amdgcn_mfma_f32_16x16x4f32"
+MFMA = "oeq_mfma"  # v_mfma_f32_16x16x4_f32 or v_mfma_f64_16x16x4_f64, see tp_module
+
+
+def piece_of(low: Lowered) -> int:
+    """Channels per piece of an irrep block (``uvw_piece`` overrides: 16, 32, 48 or 64)."""
+    from .uvu import tuning
+    forced = tuning(dict(uvw_piece=0))["uvw_piece"]
+    return forced if forced in (16, 32, 48, 64) else 64
 
 
 @dataclass
@@ -92,16 +99,17 @@ class VPath:
     wb: int
 
 
-def _pieces(blocks) -> List[VBlock]:
+def _pieces(blocks, piece: int) -> List[VBlock]:
     out = []
     for i, b in enumerate(blocks):
-        for c in range((b.mul + PIECE - 1) // PIECE):
-            out.append(VBlock(b.off + c * PIECE * b.d, min(PIECE, b.mul - c * PIECE), b.l, i, c))
+        for c in range((b.mul + piece - 1) // piece):
+            out.append(VBlock(b.off + c * piece * b.d, min(piece, b.mul - c * piece), b.l, i, c))
     return out
 
 
 def _split(low: Lowered):
-    vin, vout = _pieces(low.in1), _pieces(low.out)
+    PIECE = piece_of(low)
+    vin, vout = _pieces(low.in1, PIECE), _pieces(low.out, PIECE)
     vpaths = []
     for p in low.paths:
         wtot = low.out[p.io].mul
@@ -133,7 +141,7 @@ def _groups(vpaths: List[VPath], side: str, n_blocks: int):
 
 
 def supported(low: Lowered) -> bool:
-    if low.mode != "uvw" or not low.shared_weights or low.ctype != "float" or low.ir_mul:
+    if low.mode != "uvw" or not low.shared_weights or low.ctype not in ("float", "double") or low.ir_mul:
         return False
     if low.L3 > 1152 or low.L2 > 32:
         return False
@@ -147,6 +155,7 @@ def supported(low: Lowered) -> bool:
     fwd = max((sum(vp.U // 4 for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
     dxk = max((sum(vp.Wn // 4 for vp in g) for _, g, _ in _groups(vpaths, "vi", len(vin))), default=0)
     dwk = max((sum(4 * (vp.Wn // 16) for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
+    # (register counts in elements: fp64 runs one wave per SIMD with twice the registers)
     return fwd <= 80 and dxk <= 112 and dwk <= 80
 
 
@@ -156,16 +165,26 @@ class MfmaEmitter:
         self.vin, self.vout, self.vpaths = _split(low)
         self.max_d3 = max(low.out[p.io].d for p in low.paths)
         self.max_d1 = max(low.in1[p.i1].d for p in low.paths)
+        self.words = low.elem_size // 4
+        self.vw = 16 // low.elem_size  # elements per 16-byte vector
         # Row stride of the dZ tile in LDS: 4 mod 32 words. Rows then start on 16-byte boundaries (the tile is
         # filled with 16-byte stores), and the 32 lanes of a half-wave that read one column of 16 rows, at two
         # k-steps d words apart (d odd), fall into 32 different banks.
         self.gstride = self._tile_stride(low.L3)
+        # batch row (within the tile) of the i-th of a lane's four results: fp32 4 * (lane / 16) + i, fp64
+        # lane / 16 + 4 * i (the two instructions lay their 16 x 16 result out differently)
+        self.row = (lambda i: f"(4 * lq + {i})") if low.elem_size == 4 else (lambda i: f"(lq + 4 * {i})")
+        self.tlanes = piece_of(low)  # lanes that hold a channel in the CG part (rows of the T tile)
         from .uvu import tuning
-        self.tune = tuning(dict(uvw_wf=2, uvw_wx=2, uvw_ww=2, uvw_blocks=2, uvw_pipe=1, uvw_regs=220,
+        # waves per SIMD: fp64 runs one (512 registers; the register budgets below are in elements, of two
+        # registers there). With 32-channel pieces and two waves fp64 was 2.3x slower: half the waves of a
+        # block sit out the multiplies and there are four times as many kernels.
+        wpe = 2 if self.words == 1 else 1
+        self.tune = tuning(dict(uvw_wf=wpe, uvw_wx=wpe, uvw_ww=wpe, uvw_blocks=2, uvw_pipe=1, uvw_regs=220,
                                 uvw_merge=1, uvw_fregs=232, uvw_wregs=232, uvw_xregs=215))
 
     def lit(self, v):
-        return float_literal(v, "float")
+        return float_literal(v, self.low.ctype)
 
     # ---- CG part of one path for one (row, channel)
     def _emit_path_fns(self, s: Src):
@@ -230,11 +249,10 @@ class MfmaEmitter:
         s(f"s_y[r][c] = (row0 + r < num_batch) ? L2_in[(row0 + r) * {low.L2} + c] : T(0);")
         s.close()
 
-    @staticmethod
-    def _tile_stride(ncols: int) -> int:
-        """Row stride (words) of an LDS tile with ncols columns: 4 mod 32 when rows can start on 16-byte
-        boundaries (see ``gstride``), else 1 mod 32."""
-        want = 4 if ncols % 4 == 0 else 1
+    def _tile_stride(self, ncols: int) -> int:
+        """Row stride (elements) of an LDS tile with ncols columns: 16 bytes mod 128 when rows can start on
+        16-byte boundaries (see ``gstride``), else one element mod 32."""
+        want = self.vw if ncols % self.vw == 0 else 1
         stride = ncols + want
         while stride % 32 != want:
             stride += 1
@@ -248,12 +266,13 @@ class MfmaEmitter:
         ncols = low.L3 if ncols is None else ncols
         dst0 = 0 if local else col0
         nthreads = 64 * WAVES
-        if low.L3 % 4 == 0 and col0 % 4 == 0 and ncols % 4 == 0:
+        VW = self.vw
+        if low.L3 % VW == 0 and col0 % VW == 0 and ncols % VW == 0:
             # each wave moves its 4 rows, 64 lanes x 16 bytes at a time: every address is affine in the lane id
-            rpw, nc4 = RT // WAVES, ncols // 4
+            rpw, nc4 = RT // WAVES, ncols // VW
             J = (nc4 + 63) // 64
             s.open("")
-            s(f"float4 gv[{rpw * J}];")
+            s(f"oeq_vec16 gv[{rpw * J}];")
             for phase in ("load", "store"):
                 for rr in range(rpw):
                     for j in range(J):
@@ -262,11 +281,11 @@ class MfmaEmitter:
                         r = f"(wave * {rpw} + {rr})"
                         if phase == "load":
                             cond = f"row0 + {r} < num_batch" + (f" && {c4} < {nc4}" if part else "")
-                            s(f"gv[{rr * J + j}] = ({cond}) ? *(const float4*)(L3_grad + (row0 + {r}) * {low.L3} + "
-                              f"{col0} + 4 * {c4}) : make_float4(0.f, 0.f, 0.f, 0.f);")
+                            s(f"gv[{rr * J + j}] = ({cond}) ? *(const oeq_vec16*)(L3_grad + (row0 + {r}) * {low.L3} + "
+                              f"{col0} + {VW} * {c4}) : oeq_vec16(T(0));")
                         else:
                             guard = f"if ({c4} < {nc4}) " if part else ""
-                            s(f"{guard}*(float4*)&s_g[{r}][{dst0} + 4 * {c4}] = gv[{rr * J + j}];")
+                            s(f"{guard}*(oeq_vec16*)&s_g[{r}][{dst0} + {VW} * {c4}] = gv[{rr * J + j}];")
             s.close()
         else:
             s.open(f"for (int t = tid; t < {RT * ncols}; t += {nthreads})")
@@ -293,8 +312,12 @@ class MfmaEmitter:
         s(f"const int r = wave * {RT // WAVES} + rr;")
         s(f"T t[{d3}];")
         s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y[r], t);")
+        if self.tlanes < 64:
+            s.open(f"if (lane < {self.tlanes})")
         for k in range(d3):
             s(f"s_T[{buf}][{k}][lane][r] = t[{k}];")
+        if self.tlanes < 64:
+            s.close()
         s.close()
 
     def _dx_paths(self, s: Src, paths: List[VPath], x: str = "x", dx: str = "dx"):
@@ -313,7 +336,7 @@ class MfmaEmitter:
             s(f"T Gk[{d3}];")
             for k in range(d3):
                 s(f"Gk[{k}] = {G}[{k}][i];")
-            s(f"cg_bwd{vp.p.index}({x}[i], s_y[4 * lq + i], Gk, {dx}[i], dy[i]);")
+            s(f"cg_bwd{vp.p.index}({x}[i], s_y[{self.row('i')}], Gk, {dx}[i], dy[i]);")
             s.close()
 
         if pipe == 0:
@@ -322,9 +345,9 @@ class MfmaEmitter:
                 s(f"// path {vp.p.index}, output piece {vp.wb}")
                 s.open("")
                 # G[k] = sum_w dZ[(r,k), w] * W[u, w]   (A = dZ tile, B = W^T slice in registers)
-                s(f"v4f G[{bo.d}];")
+                s(f"v4t G[{bo.d}];")
                 for k in range(bo.d):
-                    s(f"G[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+                    s(f"G[{k}] = v4t{{}};")
                 s("#pragma unroll")
                 s.open(f"for (int st = 0; st < {vp.Wn // 4}; ++st)")
                 for k in range(bo.d):
@@ -338,7 +361,7 @@ class MfmaEmitter:
         s(f"T opa[{CH * maxd}], opb[{CH * maxd}];  // A operands of the current and the next chunk")
         if self.lds_w:
             s(f"T wla[{CH}], wlb[{CH}];  // B operands of a path whose weight slice is kept in LDS")
-        s(f"v4f G[{maxd}];")
+        s(f"v4t G[{maxd}];")
         segs = [(n, c) for n, vp in enumerate(paths) for c in range(vp.Wn // (4 * CH))]
 
         def reads(seg, buf):
@@ -360,7 +383,7 @@ class MfmaEmitter:
             if c == 0:
                 s(f"// path {vp.p.index}, output piece {vp.wb}")
                 for k in range(bo.d):
-                    s(f"G[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+                    s(f"G[{k}] = v4t{{}};")
             if t + 1 < len(segs):
                 reads(segs[t + 1], nxt)
             for q in range(CH):
@@ -397,7 +420,7 @@ class MfmaEmitter:
             s.close()
             cur = half
         for t in range(cur):
-            s(f"if (at + {t} < {n}) (&s_dy[wave][4 * lq][0])[at + {t}] = rv[{t}];")
+            s(f"if (at + {t} < {n}) s_dy[wave][{self.row(f'((at + {t}) / {low.L2})')}][(at + {t}) % {low.L2}] = rv[{t}];")
         s.close()
 
     # ------------------------------------------------------------- forward
@@ -476,7 +499,7 @@ class MfmaEmitter:
                 self._zero_kernel(s, "L3_out", low.L3, self.vout[vo0])
                 continue
             maxd = max(self.vout[vo].d for vo, _, _ in ker)
-            s(f"__shared__ T s_T[2][{maxd}][64][{TPAD}];")
+            s(f"__shared__ T s_T[2][{maxd}][{self.tlanes}][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             self._prologue(s)
             s(f"T xa[{RT // WAVES}][{self.max_d1}], xb[{RT // WAVES}][{self.max_d1}];")
@@ -492,9 +515,9 @@ class MfmaEmitter:
             self._load_x_rows(s, "xa", order_all[0])
             s("__syncthreads();")
             for vo, _, _ in ker:
-                s(f"v4f acc{vo}[{self.vout[vo].d}];")
+                s(f"v4t acc{vo}[{self.vout[vo].d}];")
                 for k in range(self.vout[vo].d):
-                    s(f"acc{vo}[{k}] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+                    s(f"acc{vo}[{k}] = v4t{{}};")
             cur, nxt = "xa", "xb"
             for n, vp in enumerate(order_all):
                 buf = n % 2
@@ -519,7 +542,7 @@ class MfmaEmitter:
                 bo = self.vout[vo]
                 s("#pragma unroll")
                 s.open("for (int i = 0; i < 4; ++i)")
-                s("const i64 row = row0 + 4 * lq + i;")
+                s(f"const i64 row = row0 + {self.row('i')};")
                 s.open(f"if (act{vo} && row < num_batch)")
                 s(f"T* zp = L3_out + row * {low.L3} + {bo.off} + (wave * 16 + l16) * {bo.d};")
                 for k in range(bo.d):
@@ -570,7 +593,9 @@ class MfmaEmitter:
             self.lds_w = []
             if self.tune["uvw_pipe"]:
                 resident = lambda: sum(vp.Wn // 4 for vp in paths_all if vp.index not in self.lds_w)
-                while len(paths_all) - len(self.lds_w) > 1 and len(self.lds_w) < 3 and \
+                # (what LDS has room for beside the dZ tile: a slice takes 16 x 256 elements)
+                room = (150 * 1024 - RT * self.gstride * low.elem_size) // (16 * 64 * WAVES * low.elem_size)
+                while len(paths_all) - len(self.lds_w) > 1 and len(self.lds_w) < min(3, room) and \
                         resident() + fixed(ker) > self.tune["uvw_regs"]:
                     self.lds_w.append(by_cost[len(self.lds_w)].index)
             if self.lds_w:
@@ -594,7 +619,7 @@ class MfmaEmitter:
                 s(f"T x{vi}[4][{self.max_d1}], dx{vi}[4][{self.vin[vi].d}];")
             s("#pragma unroll")
             s.open("for (int i = 0; i < 4; ++i)")
-            s("i64 row = row0 + 4 * lq + i; if (row >= num_batch) row = num_batch - 1;")
+            s(f"i64 row = row0 + {self.row('i')}; if (row >= num_batch) row = num_batch - 1;")
             for vi, _, _ in ker:
                 b1 = self.vin[vi]
                 s.open("")
@@ -611,7 +636,7 @@ class MfmaEmitter:
                 self._dx_paths(s, ps, f"x{vi}", f"dx{vi}")
                 s("#pragma unroll")
                 s.open("for (int i = 0; i < 4; ++i)")
-                s("const i64 row = row0 + 4 * lq + i;")
+                s(f"const i64 row = row0 + {self.row('i')};")
                 s.open("if (row < num_batch)")
                 s(f"T* dp = L1_grad + row * {low.L1} + {b1.off} + u{vi} * {b1.d};")
                 for c in range(b1.d):
@@ -652,7 +677,7 @@ class MfmaEmitter:
             self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_ww"])
             # only these pieces' columns of the dZ tile are needed (and kept)
             s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self._tile_stride(ncols)}];")
-            s(f"__shared__ T s_T[2][{maxd}][64][{TPAD}];")
+            s(f"__shared__ T s_T[2][{maxd}][{self.tlanes}][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             self._prologue(s)
             s("const int u = wave * 16 + l16;")
@@ -661,8 +686,8 @@ class MfmaEmitter:
             # dw<path>[n]: D tile rows = channels u of the wave's slice, columns = w in 16 n .. 16 n + 15
             for vp in order_all:
                 ntile = vp.Wn // 16
-                s(f"v4f dw{vp.index}[{ntile}];")
-                s(f"for (int n = 0; n < {ntile}; ++n) dw{vp.index}[n] = v4f{{0.f, 0.f, 0.f, 0.f}};")
+                s(f"v4t dw{vp.index}[{ntile}];")
+                s(f"for (int n = 0; n < {ntile}; ++n) dw{vp.index}[n] = v4t{{}};")
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
             s(f"const i64 row0 = tile * {RT};")
             s("__syncthreads();")
@@ -699,7 +724,7 @@ class MfmaEmitter:
                 for nn in range(vp.Wn // 16):
                     s("#pragma unroll")
                     s.open("for (int i = 0; i < 4; ++i)")
-                    s(f"prow[{vp.woff} + (wave * 16 + 4 * lq + i) * {vp.ld} + {16 * nn} + l16] = dw{vp.index}[{nn}][i];")
+                    s(f"prow[{vp.woff} + (wave * 16 + {self.row('i')}) * {vp.ld} + {16 * nn} + l16] = dw{vp.index}[{nn}][i];")
                     s.close()
                 s.close()
             s.close()
@@ -712,7 +737,16 @@ def tp_module(low: Lowered, compute_units: int = 256):
     em = MfmaEmitter(low)
     s = Src()
     s(prelude(low.ctype))
-    s("typedef float v4f __attribute__((ext_vector_type(4)));")
+    s("typedef T v4t __attribute__((ext_vector_type(4)));")
+    s(f"typedef T oeq_vec16 __attribute__((ext_vector_type({16 // low.elem_size})));  // 16 bytes")
+    if low.elem_size == 4:
+        s("#define oeq_mfma __builtin_amdgcn_mfma_f32_16x16x4f32")
+    else:
+        s("#define oeq_mfma __builtin_amdgcn_mfma_f64_16x16x4f64")
+        s("template <int CTRL> OEQ_DEV double oeq_dpp(double v) { const long long b = __builtin_bit_cast(long long, v); "
+          "const int lo = __builtin_amdgcn_update_dpp(0, (int)b, CTRL, 0xf, 0xf, true); "
+          "const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, 0xf, 0xf, true); "
+          "return __builtin_bit_cast(double, ((long long)hi << 32) | (unsigned)lo); }")
     # value of the lane that a DPP control word pairs this lane with (row_mirror 0x140, row_half_mirror 0x141,
     # quad_perm otherwise)
     s("template <int CTRL> OEQ_DEV float oeq_dpp(float v) { return __builtin_bit_cast(float, "

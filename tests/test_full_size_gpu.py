@@ -96,15 +96,18 @@ def test_cfg3_full_batch(dtype):
     assert torch.equal(sx, 2.0 * dx) and torch.equal(sy, 2.0 * dy) and torch.equal(sw, 2.0 * dw)
 
 
-def test_cfg4_full_batch_mfma():
-    problem = P.config4_uvw_shared()
-    B = 262144
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+def test_cfg4_full_batch_mfma(dtype):
+    problem = P.config4_uvw_shared(dtype)
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    td = torch.float32 if dtype == np.float32 else torch.float64
+    B = 262144 if dtype == np.float32 else 65536
     gen = torch.Generator(device="cuda").manual_seed(1)
-    x = torch.randn(B, 576, device="cuda", generator=gen, requires_grad=True)
+    x = torch.randn(B, 576, device="cuda", generator=gen, dtype=td, requires_grad=True)
     v = torch.randn(B, 3, device="cuda", generator=gen)
-    y = torch.tensor(spherical_harmonics(2, v.cpu().numpy()).astype(np.float32), device="cuda").requires_grad_(True)
-    w = (torch.randn(45056, device="cuda", generator=gen) / np.sqrt(64 * 11)).requires_grad_(True)
-    g = torch.randn(B, 576, device="cuda", generator=gen)
+    y = torch.tensor(spherical_harmonics(2, v.cpu().numpy()).astype(dtype), device="cuda").requires_grad_(True)
+    w = (torch.randn(45056, device="cuda", generator=gen, dtype=td) / np.sqrt(64 * 11)).requires_grad_(True)
+    g = torch.randn(B, 576, device="cuda", generator=gen, dtype=td)
     tp = oeq.TensorProduct(problem)
     z = tp(x, y, w)
     z.backward(g)
@@ -112,20 +115,20 @@ def test_cfg4_full_batch_mfma():
     ref = R.Problem.from_spec(problem)
     xs, ys, gs = (t[idx].detach().cpu().numpy() for t in (x, y, g))
     wn = w.detach().cpu().numpy()
-    assert err(z[idx], R.tp_forward(ref, xs, ys, wn)) <= 1e-5
+    assert err(z[idx], R.tp_forward(ref, xs, ys, wn)) <= tol
     dx, dy, _ = R.tp_backward(ref, xs, ys, wn, gs)
-    assert err(x.grad[idx], dx) <= 1e-5 and err(y.grad[idx], dy) <= 1e-5
+    assert err(x.grad[idx], dx) <= tol and err(y.grad[idx], dy) <= tol
     # weight gradient: linear in the output gradient; a sum over disjoint row sets adds up
     half = B // 2
     _, _, dw1 = torch.ops.oeq_amd.tp_backward(x[:half].detach(), y[:half].detach(), w.detach(), g[:half], tp.kid)
     _, _, dw2 = torch.ops.oeq_amd.tp_backward(x[half:].detach(), y[half:].detach(), w.detach(), g[half:], tp.kid)
-    assert _rel(dw1 + dw2, w.grad) <= 1e-5
+    assert _rel(dw1 + dw2, w.grad) <= tol
     # and it matches the oracle on a slice small enough to evaluate (first 2048 rows)
     n = 2048
     _, _, dws = torch.ops.oeq_amd.tp_backward(x[:n].detach(), y[:n].detach(), w.detach(), g[:n], tp.kid)
     _, _, dw_ref = R.tp_backward(ref, x[:n].detach().cpu().numpy(), y[:n].detach().cpu().numpy(), wn,
                                  g[:n].cpu().numpy())
-    assert err(dws, dw_ref) <= 1e-5
+    assert err(dws, dw_ref) <= tol
     # deterministic reduction: bitwise equal on a second run
     _, _, dw_again = torch.ops.oeq_amd.tp_backward(x.detach(), y.detach(), w.detach(), g, tp.kid)
     assert torch.equal(dw_again, w.grad)

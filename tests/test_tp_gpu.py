@@ -113,8 +113,12 @@ CASES = [
         "32x0e+16x1o+48x2e", "1x0e+1x1o", "32x0e+16x1e+64x1o",
         [(0, 0, 0, "uvw", True), (0, 1, 2, "uvw", True), (1, 0, 2, "uvw", True, 0.6), (1, 1, 0, "uvw", True)],
         shared_weights=True, internal_weights=False, label="mfma-gaps"), 50),
+    # the same kernels in fp64 (v_mfma_f64_16x16x4_f64, whose result rows are laid out differently)
+    ("mfma-128-f64", lambda: _as_f64(_fc_shared("128x0e+128x1o", "1x0e+1x1o", "128x0e+128x1o")), 45),
+    ("mfma-mixed-f64", lambda: _as_f64(_fc_shared("64x0e+32x1o+16x2e", "1x0e+1x1o", "48x0e+80x1o+16x2e")), 50),
 ]
-MFMA_CASES = {"cfg4-shared", "mfma-32", "mfma-128", "mfma-mixed", "mfma-gaps"}
+MFMA_CASES = {"cfg4-shared", "cfg4-f64", "mfma-32", "mfma-128", "mfma-mixed", "mfma-gaps", "mfma-128-f64",
+              "mfma-mixed-f64"}
 
 
 @pytest.mark.parametrize("name,make,B", CASES, ids=[c[0] for c in CASES])
