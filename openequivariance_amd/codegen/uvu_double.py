@@ -27,7 +27,7 @@ from typing import Dict, List, Optional, Tuple
 
 from .common import Src
 from .lower import Lowered, Path
-from .uvu import UvuEmitter
+from .uvu import UNROLL_V_LIMIT, UvuEmitter
 
 
 # Convolution: above this many paths (after folding of wide rows) the kernels' register needs (two
@@ -95,12 +95,70 @@ class DoubleEmitter(UvuEmitter):
                     f"const int u, D{si}_t& a)"
                 )
                 wacc, cacc = self._w_of("wrow"), self._w_of("crow")
-                for p in self._paths():
-                    if p.io not in seg:
-                        continue
+                seg_paths = [p for p in self._paths() if p.io in seg]
+                preload_w = (self.forms and sum(low.in2[q.i2].mul for q in seg_paths) <= 48
+                             and all(low.in2[q.i2].mul <= UNROLL_V_LIMIT for q in seg_paths))
+                if preload_w:
+                    # the weights are folded into the X operands at the top of every path: all requested here
+                    for q in seg_paths:
+                        for v in range(low.in2[q.i2].mul):
+                            s(f"const T wv{q.index}_{v} = {wacc(q, str(v))};")
+                            s(f"const T cv{q.index}_{v} = {cacc(q, str(v))};")
+                for p in seg_paths:
                     s(f"// path {p.index}")
 
-                    def body(v, p=p):
+                    def body(v, p=p, preload_w=preload_w):
+                        # z''_k = sum c [ y_j (w a_i + c_w x_i) + b_j (w x_i) ]: with the weights folded into two
+                        # per-lane vectors first, a term costs two multiply-adds instead of three plus the
+                        # weighting of two partial results; the coefficient then rides on (|c|, j) products
+                        # or, summing the terms of equal |c| first, on the result - whichever is fewer.
+                        if not self.forms:
+                            return body_plain(v, p)
+                        yacc, bacc = self._y_of("yrow"), self._y_of("brow")
+                        for j in sorted({j for _, j, _, _ in p.nnz}):
+                            s(f"const T y{j} = {yacc(p, v, j)};")
+                            s(f"const T b{j} = {bacc(p, v, j)};")
+                        s(f"const T wv = {f'wv{p.index}_{v}' if preload_w else wacc(p, v)};")
+                        s(f"const T cv = {f'cv{p.index}_{v}' if preload_w else cacc(p, v)};")
+                        for i in sorted({i for i, _, _, _ in p.nnz}):
+                            s(f"const T r{i} = wv * x.b{p.i1}[{i}];")
+                            s(f"const T p{i} = wv * xa.b{p.i1}[{i}] + cv * x.b{p.i1}[{i}];")
+                        cj, ci, ck, nc = self._form_counts(p)
+                        ks = sorted({k for _, _, k, _ in p.nnz})
+                        if ck <= 2 * cj + len(ks):
+                            sums = {}
+                            for i, j, k, c in p.nnz:
+                                key = (self.lit(abs(c)), k)
+                                neg = c < 0
+                                if key not in sums:
+                                    sums[key] = f"s{len(sums)}"
+                                    s(f"T {sums[key]} = {'-' if neg else ''}y{j} * p{i};")
+                                else:
+                                    s(f"{sums[key]} {'-=' if neg else '+='} y{j} * p{i};")
+                                s(f"{sums[key]} {'-=' if neg else '+='} b{j} * r{i};")
+                            for (m, k), name in sums.items():
+                                s(f"a.o{p.io}[{k}] += T({m}) * {name};")
+                        else:
+                            qs = {}
+                            started = set()
+                            for i, j, k, c in p.nnz:
+                                key = (self.lit(abs(c)), j)
+                                if key not in qs:
+                                    qs[key] = len(qs)
+                                    s(f"const T q{qs[key]} = T({key[0]}) * y{j};")
+                                    s(f"const T qb{qs[key]} = T({key[0]}) * b{j};")
+                                n_ = qs[key]
+                                neg = c < 0
+                                if k not in started:
+                                    s(f"T t{k} = {'-' if neg else ''}q{n_} * p{i};")
+                                    started.add(k)
+                                else:
+                                    s(f"t{k} {'-=' if neg else '+='} q{n_} * p{i};")
+                                s(f"t{k} {'-=' if neg else '+='} qb{n_} * r{i};")
+                            for k in sorted(started):
+                                s(f"a.o{p.io}[{k}] += t{k};")
+
+                    def body_plain(v, p):
                         prods = self._two_products(s, p, v)
                         started = set()
                         for n, (i, j, k, c) in enumerate(p.nnz):
@@ -135,6 +193,15 @@ class DoubleEmitter(UvuEmitter):
         wacc, cacc = self._w_of("wrow"), self._w_of("crow")
         ordered = sorted(self._paths(paths), key=lambda q: (q.io, q.index))
         since_fence = 0
+        preload_w = (self.forms and not fwd_acc and sum(low.in2[q.i2].mul for q in ordered) <= 48
+                     and all(low.in2[q.i2].mul <= UNROLL_V_LIMIT for q in ordered))
+        if preload_w:
+            # every path's W and C value is wanted at the top of its code (the weights are folded into the Y
+            # operands first): requested here, all together, or each path would wait for its own pair
+            for q in ordered:
+                for v in range(low.in2[q.i2].mul):
+                    s(f"const T wv{q.index}_{v} = {wacc(q, str(v))};")
+                    s(f"const T cv{q.index}_{v} = {cacc(q, str(v))};")
         for n_path, p in enumerate(ordered):
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
             V = b2.mul
@@ -154,11 +221,25 @@ class DoubleEmitter(UvuEmitter):
             base_slot = self.wslot[p.index]
 
             def body(v, p=p, b1=b1, b2=b2, V=V, gname=gname, base_slot=base_slot):
-                prods = self._two_products(s, p, v)
-                s(f"const T wv = {wacc(p, v)};")
-                s(f"const T cv = {cacc(p, v)};")
                 ks = sorted({k for _, _, k, _ in p.nnz})
                 js = sorted({j for _, j, _, _ in p.nnz})
+                fold = self.forms and not fwd_acc
+                if fold:
+                    # d/dX_i = sum c g_k (w b_j + c_w y_j): the weights are folded into one vector over j first, so
+                    # a term costs one multiply-add (two before, plus the weighting of g_k twice)
+                    yacc, bacc = self._y_of("yrow"), self._y_of("brow")
+                    for j in js:
+                        s(f"const T y{j} = {yacc(p, v, j)};")
+                        s(f"const T b{j} = {bacc(p, v, j)};")
+                    s(f"const T wv = {f'wv{p.index}_{v}' if preload_w else wacc(p, v)};")
+                    s(f"const T cv = {f'cv{p.index}_{v}' if preload_w else cacc(p, v)};")
+                    for j in js:
+                        s(f"const T m{j} = wv * b{j} + cv * y{j};")
+                    prods = self._scaled(s, p, 1, lambda j: f"m{j}", "qm")
+                else:
+                    prods = self._two_products(s, p, v)
+                    s(f"const T wv = {wacc(p, v)};")
+                    s(f"const T cv = {cacc(p, v)};")
                 # One output component k at a time, so that what is derived from g_k (its products with the
                 # weights and with the X / A components) is dead before the next k: in any other order
                 # these temporaries, two sets of them here, cost more registers than the operands.
@@ -168,12 +249,17 @@ class DoubleEmitter(UvuEmitter):
                     s(f"T h{j} = T(0), ha{j} = T(0);")
                 for k in ks:
                     s.open("")
-                    s(f"const T gw = {gname(k)} * wv; const T gc = {gname(k)} * cv;")
                     of_k = [(n, t) for n, t in enumerate(p.nnz) if t[2] == k]
-                    for n, (i, j, _, c) in of_k:
-                        qy, qb, neg = prods[n]
-                        op = "-=" if neg else "+="
-                        s(f"dx.b{p.i1}[{i}] {op} {qb} * gw; dx.b{p.i1}[{i}] {op} {qy} * gc;")
+                    if fold:
+                        for n, (i, j, _, c) in of_k:
+                            qm, neg = prods[n]
+                            s(f"dx.b{p.i1}[{i}] {'-=' if neg else '+='} {qm} * {gname(k)};")
+                    else:
+                        s(f"const T gw = {gname(k)} * wv; const T gc = {gname(k)} * cv;")
+                        for n, (i, j, _, c) in of_k:
+                            qy, qb, neg = prods[n]
+                            op = "-=" if neg else "+="
+                            s(f"dx.b{p.i1}[{i}] {op} {qb} * gw; dx.b{p.i1}[{i}] {op} {qy} * gc;")
                     for i in sorted({t[0] for _, t in of_k}):
                         s(f"{{ const T xg = x.b{p.i1}[{i}] * {gname(k)}; const T ag = xa.b{p.i1}[{i}] * {gname(k)};")
                         for n, (i2, j, _, c) in of_k:
@@ -673,6 +759,7 @@ def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict) -> List[t
     em = DoubleEmitter(low, acc_budget_words=64)
     em.nt = base.nt
     em.mask_loads = base.mask_loads
+    em.forms = base.forms
     em.tr_stores = base.tr_stores
     em.fence_words = 48
     # the accumulator structs of this emitter's (smaller) segments
@@ -717,6 +804,7 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
                     break
     em.nt = base.nt
     em.mask_loads = base.mask_loads
+    em.forms = base.forms
     em.tr_stores = base.tr_stores
     em.fence_words = tune.get("dd_fw", 32)
     em.fence_paths = tune.get("dd_fp", 0)
