@@ -97,3 +97,31 @@ def test_convolution_in_a_graph(deterministic):
 
     # deterministic=False accumulates the sender gradient with float atomics (and what is derived from it here)
     _replay_and_compare(step, [X, Y, W, G], new_values, tol=0.0 if deterministic else 2e-5)
+
+
+@pytest.mark.parametrize("deterministic", [True, False], ids=["sorted", "grouped"])
+def test_uvw_convolution_in_a_graph(deterministic):
+    """The fused 'uvw' convolution (per-edge weights): index build, receiver walk, per-edge backward and the ordered
+    sender-side sum are all recorded; both modes are bitwise reproducible, so every replay equals the eager result."""
+    problem = P.diffdock_problems()[0]
+    coords, rows, cols, _ = periodic_radius_graph(60, 8, 5.0, 3)
+    gr = CoordGraph(coords, rows, cols)
+    n, E = 60, gr.nnz
+    tr, tc, tp = (torch.tensor(a, device="cuda") for a in (gr.rows, gr.cols, gr.transpose_perm))
+    conv = oeq.TensorProductConv(problem, deterministic=deterministic)
+    assert not ops.get_entry(conv.kid).unfused
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    X = torch.randn(n, problem.irreps_in1.dim, device="cuda", generator=gen)
+    Y = torch.randn(E, problem.irreps_in2.dim, device="cuda", generator=gen)
+    W = torch.randn(E, problem.weight_numel, device="cuda", generator=gen)
+    G = torch.randn(n, problem.irreps_out.dim, device="cuda", generator=gen)
+
+    def step():
+        z = ops.conv_forward(X, Y, W, tr, tc, tp, conv.kid)
+        return [z] + list(ops.conv_backward(X, Y, W, G, tr, tc, tp, conv.kid))
+
+    def new_values(seed):
+        gen2 = torch.Generator(device="cuda").manual_seed(300 + seed)
+        return [torch.randn(t.shape, device="cuda", generator=gen2) for t in (X, Y, W, G)]
+
+    _replay_and_compare(step, [X, Y, W, G], new_values)
