@@ -66,6 +66,10 @@ struct TimedLaunch {
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// Entries of the long-segment list that oeq_group_scan leaves behind a cursor array (the kernels in
+// codegen/common.py use the same number).
+constexpr int64_t OEQ_LONG_LIST = 126;
+
 }  // namespace
 
 struct oeq_kernels {
@@ -169,7 +173,7 @@ struct oeq_kernels {
     }
 
     // Item indices grouped by key, in no particular order within a group: ptr[0..n_segments] = group
-    // starts, perm = the grouped indices; cursor (n_segments+1) is scratch.
+    // starts, perm = the grouped indices; cursor (sized by ptr_bytes_of) is scratch.
     int group_unordered(int64_t n_items, int64_t n_segments, const int64_t* keys, int64_t* ptr, int64_t* cursor,
                         int64_t* perm, void* stream) {
         int rc = fill_zero(ptr, (size_t)(n_segments + 1) * sizeof(int64_t), stream);
@@ -187,7 +191,8 @@ struct oeq_kernels {
 
     // Counting sort of the item indices 0..n_items-1 by key: ptr[0..n_segments] = segment starts,
     // perm = item indices grouped by key, ascending within a group (so the result depends on the key
-    // list only); cursor (n_segments+1) and unordered (n_items) are scratch.
+    // list only); cursor (n_segments + 1 entries and the long-segment list, see ptr_bytes_of) and unordered
+    // (n_items) are scratch.
     int group_by_key(int64_t n_items, int64_t n_segments, const int64_t* keys, int64_t* ptr, int64_t* cursor,
                      int64_t* unordered, int64_t* perm, void* stream) {
         int rc = fill_zero(ptr, (size_t)(n_segments + 1) * sizeof(int64_t), stream);
@@ -202,8 +207,12 @@ struct oeq_kernels {
         void* pargs[] = {&n_items, &keys, &cursor, &unordered, &n_segments};
         rc = launch(OEQ_ROLE_GROUP_SCATTER, n_items, pargs, stream);
         if (rc) return rc;
-        void* oargs[] = {&n_segments, &ptr, &unordered, &perm};
-        return launch(OEQ_ROLE_GROUP_ORDER, n_segments, oargs, stream);
+        // the scan left the segments longer than a wave should rank by itself behind the cursor entries
+        const int64_t* long_list = cursor + n_segments + 1;
+        void* oargs[] = {&n_segments, &ptr, &unordered, &perm, &long_list, &n_items};
+        // one wave per segment, and at least one thread per 16 items so that few nodes with many items
+        // still bring a grid wide enough for the long segments
+        return launch(OEQ_ROLE_GROUP_ORDER, std::max(n_segments, n_items / 64), oargs, stream);
     }
 };
 
@@ -379,7 +388,7 @@ int oeq_segment_sum(oeq_kernels* k, int64_t n_segments, int64_t n_items, int64_t
 size_t oeq_grouped_sum_workspace_bytes(const oeq_kernels* k, int64_t n_segments, int64_t n_items) {
     (void)k;
     // [ptr | cursor | perm | scratch perm]
-    return 2 * align_up((size_t)(n_segments + 1) * sizeof(int64_t), 256) +
+    return 2 * align_up((size_t)(n_segments + 1 + 1 + OEQ_LONG_LIST) * sizeof(int64_t), 256) +
            2 * align_up((size_t)n_items * sizeof(int64_t), 256);
 }
 
@@ -394,7 +403,7 @@ int oeq_grouped_sum(oeq_kernels* k, int64_t n_segments, int64_t n_items, int64_t
     size_t need = oeq_grouped_sum_workspace_bytes(k, n_segments, n_items);
     if (!workspace || workspace_bytes < need)
         return fail(OEQ_ERR_INVALID, "oeq_grouped_sum: workspace too small (%zu < %zu bytes)", workspace_bytes, need);
-    const size_t pb = align_up((size_t)(n_segments + 1) * sizeof(int64_t), 256);
+    const size_t pb = align_up((size_t)(n_segments + 1 + 1 + OEQ_LONG_LIST) * sizeof(int64_t), 256);
     const size_t qb = align_up((size_t)n_items * sizeof(int64_t), 256);
     int64_t* ptr = (int64_t*)workspace;
     int64_t* cursor = (int64_t*)((char*)workspace + pb);
@@ -498,7 +507,11 @@ static int check_graph_size(const char* who, int64_t node_count, int64_t nnz) {
 }
 
 // Shared weights, walk kernels: one partial weight-gradient row per wave group of the backward grid.
-static size_t ptr_bytes_of(int64_t node_count) { return align_up((size_t)(node_count + 1) * sizeof(int64_t), 256); }
+// A segment-pointer (or cursor) array: n + 1 entries, and behind them the list of long segments that
+// oeq_group_scan leaves for oeq_group_order (a count and up to OEQ_LONG_LIST entries).
+static size_t ptr_bytes_of(int64_t node_count) {
+    return align_up((size_t)(node_count + 1 + 1 + OEQ_LONG_LIST) * sizeof(int64_t), 256);
+}
 static size_t perm_bytes_of(int64_t nnz) { return align_up((size_t)nnz * sizeof(int64_t), 256); }
 
 static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t node_count) {

@@ -418,6 +418,38 @@ def test_grouped_mode_handles_hubs_and_many_nodes():
         assert err(got, want) <= 1e-5
 
 
+@pytest.mark.parametrize("hubs,degree", [(3, 2100), (130, 2060)], ids=["listed", "more-than-the-list-holds"])
+def test_grouping_orders_long_segments(hubs, degree):
+    """Receivers with more than 2048 edges are ranked by the whole grid instead of one wave (up to 126 of them;
+    beyond that the waves take them again). Either way the grouping is the ascending one: on a list that is
+    already sorted, deterministic=False sums in the order of the sorted list and gives the bits of
+    deterministic=True; on a shuffled list the output keeps the same bits from run to run."""
+    problem = P.config1_single_uvu()
+    rng = np.random.default_rng(hubs)
+    n = hubs + 500
+    rows = np.concatenate([np.repeat(np.arange(hubs, dtype=np.int64), degree), rng.integers(hubs, n, size=4000)])
+    cols = rng.integers(0, n, size=len(rows))
+    order = np.lexsort((cols, rows))
+    rows, cols = rows[order], cols[order]
+    E = len(rows)
+    X, Y, W, G = _buffers(problem, n, E, seed=hubs)
+    z_ref = R.conv_forward(R.Problem.from_spec(problem), X, Y, W, rows, cols)
+    tX, tY, tW, tr, tc = (torch.tensor(a, device="cuda") for a in (X, Y, W, rows, cols))
+    # the sender of the reverse edge need not exist for a forward call: any permutation serves
+    z_sorted = oeq.TensorProductConv(problem, deterministic=True)(tX, tY, tW, tr, tc, torch.arange(E, device="cuda"))
+    conv = oeq.TensorProductConv(problem, deterministic=False)
+    z = conv(tX, tY, tW, tr, tc)
+    assert err(z, z_ref) <= 1e-5
+    assert torch.equal(z, z_sorted)
+    shuffle = torch.tensor(rng.permutation(E), device="cuda")
+    Ys, Ws, rs, cs = (t[shuffle].contiguous() for t in (tY, tW, tr, tc))
+    first = conv(tX, Ys, Ws, rs, cs)
+    assert err(first, z_ref) <= 1e-5
+    for _ in range(3):
+        torch.randn(1 << 22, device="cuda")
+        assert torch.equal(conv(tX, Ys, Ws, rs, cs), first)
+
+
 KNOBS = ["conv_pipe_f=0,conv_pipe_b=1", "conv_pipe_f=1,conv_pipe_b=2", "conv_pipe_f=3,conv_pipe_b=3",
          "conv_xcd=1,conv_gres=0", "conv_nt=0,conv_acc=48", "conv_sort=0,conv_tra=0", "conv_sort=0,conv_pipe_f=3,conv_nt=0",
          "conv_wf=0,conv_wb=0,conv_gf=1,conv_gb=1",

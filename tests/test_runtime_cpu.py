@@ -56,8 +56,9 @@ def test_kernels_create_validates_arguments():
     assert ks.conv_forward_workspace_bytes(10, 10) == 0
     dims["deterministic"] = 1
     ks2 = rt.KernelSet(b"\x7fELFxxxx", dims, [(rt.ROLE_CONV_FORWARD, "forward", 64, 1, 0)])
-    assert ks2.conv_forward_workspace_bytes(31, 10) == 256
-    assert ks2.conv_backward_workspace_bytes(31, 10) == 2 * 256 + 256  # 10*4*4 = 160 -> 256
+    # segment starts: 31 + 1 entries, one count and a list of 126 long segments, 8 bytes each -> 1272 -> 1280
+    assert ks2.conv_forward_workspace_bytes(31, 10) == 1280
+    assert ks2.conv_backward_workspace_bytes(31, 10) == 2 * 1280 + 256  # 10*4*4 = 160 -> 256
 
 
 ALL = [P.config1_single_uvu, P.config2_nequip_uvu, P.config3_mace_uvu, P.config4_uvw_shared,
