@@ -256,13 +256,17 @@ size_t oeq_conv_double_backward_scratch_bytes(const oeq_kernels* k, int64_t node
  * L1_in, L2_in, W and L3_grad (all four fully overwritten). Replaces JITTPImpl::double_backward
  * (extension/tensorproducts.hpp:97-111) as called by jit_tp_double_backward
  * (extension/torch_core.hpp:357-420). Only kernel sets for which oeq_has_double_backward() is non-zero
- * carry these kernels ('uvu' problems with per-row weights); for the others the same result is composed
- * from oeq_tp_forward / oeq_tp_backward calls by the caller. */
+ * carry these kernels ('uvu' problems; with shared weights the batch entry point only); for the others the
+ * same result is composed from oeq_tp_forward / oeq_tp_backward calls by the caller. */
 int oeq_has_double_backward(const oeq_kernels* k);
 int oeq_tp_double_backward(oeq_kernels* k, int64_t num_batch,
                            const void* L1_in, const void* L2_in, const void* W, const void* L3_grad,
                            const void* L1_dgrad, const void* L2_dgrad, const void* W_dgrad,
-                           void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad, void* stream);
+                           void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad,
+                           void* workspace, size_t workspace_bytes, void* stream);
+/* Workspace of oeq_tp_double_backward: partial weight gradients for shared weights (summed in a fixed
+ * order by a second kernel, as in oeq_tp_backward); zero for per-row weights, and then workspace may be NULL. */
+size_t oeq_tp_double_backward_workspace_bytes(const oeq_kernels* k, int64_t num_batch);
 
 /* The same for the fused convolution; replaces JITConvImpl::double_backward
  * (extension/convolution.hpp:138-178) as called by jit_conv_double_backward

@@ -233,9 +233,12 @@ def tp_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor
     a, b, c = L1_dgrad.contiguous(), L2_dgrad.contiguous(), W_dgrad.contiguous()
     dx, dy, dw, gg = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w), torch.empty_like(g)
     with torch.cuda.device(x.device):
-        e.kernels().tp_double_backward(n, x.data_ptr(), y.data_ptr(), w.data_ptr(), g.data_ptr(), a.data_ptr(),
-                                       b.data_ptr(), c.data_ptr(), dx.data_ptr(), dy.data_ptr(), dw.data_ptr(),
-                                       gg.data_ptr(), _stream())
+        ks = e.kernels()
+        nb = ks.tp_double_backward_workspace_bytes(n)
+        ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
+        ks.tp_double_backward(n, x.data_ptr(), y.data_ptr(), w.data_ptr(), g.data_ptr(), a.data_ptr(),
+                              b.data_ptr(), c.data_ptr(), dx.data_ptr(), dy.data_ptr(), dw.data_ptr(),
+                              gg.data_ptr(), ws.data_ptr(), nb, _stream())
     return dx, dy, dw, gg
 
 

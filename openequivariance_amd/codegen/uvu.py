@@ -2062,7 +2062,7 @@ def tp_module(low: Lowered, compute_units: int = 256):
     ]
     from . import uvu_double
     if t["tp_dd"] and uvu_double.supported(low):
-        descs += uvu_double.add_tp_kernels(s, low, em, t)
+        descs += uvu_double.add_tp_kernels(s, low, em, t, G_b, compute_units)
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
                 shared_weights=int(low.shared_weights), deterministic=0,
                 wpartial_per_block=G_b if low.shared_weights else 0)

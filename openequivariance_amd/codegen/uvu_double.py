@@ -18,7 +18,8 @@ passes over the weight-sized tensors for each group.
 
 Work decomposition is that of the first-order kernels (lane = channel, a wave or a group of chunk
 waves per row / per receiver node, register-resident accumulators over a node's edges, per-edge dX
-terms reduced by the sender-ordered second pass). Per-row weights only.
+terms reduced by the sender-ordered second pass). Shared weights: the batch kernels only, with the weight
+gradient summed per wave in registers and across waves by the first-order pass's ordered reduction.
 """
 
 from __future__ import annotations
@@ -39,10 +40,15 @@ CONV_MAX_PATHS = 96
 
 
 def supported(low: Lowered, conv: bool = False) -> bool:
-    if low.mode != "uvu" or low.shared_weights:
+    """Batch kernels: every 'uvu' problem. Convolution: per-edge weights, up to CONV_MAX_PATHS paths."""
+    if low.mode != "uvu" or (conv and low.shared_weights):
         return False
     from .uvu import tuning
     return not conv or len(low.paths) <= tuning(dict(dd_maxp=CONV_MAX_PATHS))["dd_maxp"]
+
+
+def dwv_live(value: str, guard: Optional[str]) -> str:
+    return value if guard in (None, "true") else f"({guard} ? {value} : T(0))"
 
 
 class DoubleEmitter(UvuEmitter):
@@ -61,7 +67,7 @@ class DoubleEmitter(UvuEmitter):
         def w(p: Path, v: str) -> str:
             mul = low.in1[p.i1].mul
             wp = self._ptr(row, (f"{p.woff} + ({v})", low.in2[p.i2].mul), mul)
-            ld = f"__builtin_nontemporal_load({wp})" if self.nt & 1 else f"*{wp}"
+            ld = f"__builtin_nontemporal_load({wp})" if (self.nt & 1) and not low.shared_weights else f"*{wp}"
             return self._operand(mul, ld)
         return w
 
@@ -272,7 +278,10 @@ class DoubleEmitter(UvuEmitter):
                 s(f"dwv += y{js[0]} * ha{js[0]};")
                 for j in js[1:]:
                     s(f"dwv += b{j} * h{j}; dwv += y{j} * ha{j};")
-                if deferred:
+                if low.shared_weights:
+                    # summed over the wave's rows in registers; rows past the end of the batch are duplicates
+                    s(f"dwacc[{base_slot} + {v}] += {dwv_live('dwv', dw_guard)};")
+                elif deferred:
                     s(f"dwkeep[{base_slot} + {v}] = dwv;")
                 else:
                     dwp = self._ptr("dwrow", (f"{p.woff} + ({v})", V))
@@ -343,8 +352,8 @@ class DoubleEmitter(UvuEmitter):
         s(f"const T* arow = L1_dgrad + rowc * {low.L1};")
         s(f"const T* yrow = L2_in + rowc * {low.L2};")
         s(f"const T* brow = L2_dgrad + rowc * {low.L2};")
-        s(f"const T* wrow = W + rowc * {low.WN};")
-        s(f"const T* crow = W_dgrad + rowc * {low.WN};")
+        s(f"const T* wrow = W{'' if low.shared_weights else f' + rowc * {low.WN}'};")
+        s(f"const T* crow = W_dgrad{'' if low.shared_weights else f' + rowc * {low.WN}'};")
         s(f"T* zrow = L3_dgrad + rowc * {low.L3};")
         live = "live"
         if self.R == 1:
@@ -381,13 +390,18 @@ class DoubleEmitter(UvuEmitter):
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_B(i64 num_batch, '
             "const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
             "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
-            "const T* __restrict__ L3_grad, T* __restrict__ L1_grad, T* __restrict__ L2_grad, T* __restrict__ W_grad)"
+            "const T* __restrict__ L3_grad, T* __restrict__ L1_grad, T* __restrict__ L2_grad, T* __restrict__ W_grad, "
+            "T* __restrict__ wpartial)"
         )
         self._lane_prologue(s)
+        shared = low.shared_weights
         if self.NCH > 1:
             s(f"__shared__ T s_dy[{G}][{self.NCH}][{self.l2_pad}];")
         if self.tr_stores & 2 and self.R == 1:
             s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(b.d for b in low.in1)}];")
+        if shared:
+            s(f"T dwacc[{self.n_wslots}];")
+            s(f"for (int t = 0; t < {self.n_wslots}; ++t) dwacc[t] = T(0);")
         s(f"const i64 ngroups = (num_batch + {self.R - 1}) / {self.R};")
         s.open(f"for (i64 base = (i64)blockIdx.x * {G}; base < ngroups; base += (i64)gridDim.x * {G})")
         s("const i64 grp = base + g;")
@@ -398,10 +412,11 @@ class DoubleEmitter(UvuEmitter):
         s(f"const T* arow = L1_dgrad + rowc * {low.L1};")
         s(f"const T* yrow = L2_in + rowc * {low.L2};")
         s(f"const T* brow = L2_dgrad + rowc * {low.L2};")
-        s(f"const T* wrow = W + rowc * {low.WN};")
-        s(f"const T* crow = W_dgrad + rowc * {low.WN};")
+        s(f"const T* wrow = W{'' if shared else f' + rowc * {low.WN}'};")
+        s(f"const T* crow = W_dgrad{'' if shared else f' + rowc * {low.WN}'};")
         s(f"const T* grow = L3_grad + rowc * {low.L3};")
-        s(f"T* dwrow = W_grad + rowc * {low.WN};")
+        if not shared:
+            s(f"T* dwrow = W_grad + rowc * {low.WN};")
         live = "live"
         if self.R == 1:
             s.open("if (live)")
@@ -415,7 +430,7 @@ class DoubleEmitter(UvuEmitter):
             self._zero_x(s, "dx")
             s(f"T dy[{self.l2_pad}];")
             s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
-            deferred = self._dw_deferred(live)
+            deferred = not shared and self._dw_deferred(live)
             if deferred:
                 s(f"T dwkeep[{self.n_wslots}];")
             if resident:
@@ -436,6 +451,22 @@ class DoubleEmitter(UvuEmitter):
         if self.R == 1:
             s.close()
         s.close()
+        if shared:
+            # as in the first-order backward: fold the row groups of the wave, then every wave group writes one
+            # partial row, which a second kernel sums in block order
+            if self.R > 1:
+                s.open(f"for (int t = 0; t < {self.n_wslots}; ++t)")
+                m = self.LPR
+                while m < 64:
+                    s(f"dwacc[t] += __shfl_xor(dwacc[t], {m});")
+                    m *= 2
+                s.close()
+            s(f"T* prow = wpartial + ((i64)blockIdx.x * {G} + g) * {low.WN};")
+            for p, slot in self._dw_slots():
+                b1, V = low.in1[p.i1], low.in2[p.i2].mul
+                s.open(f"if (r == 0 && u < {b1.mul})")
+                s(f"for (int v = 0; v < {V}; ++v) prow[{p.woff} + u * {V} + v] = dwacc[{slot} + v];")
+                s.close()
         s.close()
         return block
 
@@ -752,8 +783,10 @@ class DoubleEmitter(UvuEmitter):
         return block
 
 
-def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict) -> List[tuple]:
-    """Append the batch double-backward kernels to a module; returns their launch descriptors."""
+def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, groups_b: int = 4,
+                   compute_units: int = 256) -> List[tuple]:
+    """Append the batch double-backward kernels to a module; returns their launch descriptors. ``groups_b``:
+    wave groups per block of the first-order backward kernel."""
     from .. import runtime as rt
 
     em = DoubleEmitter(low, acc_budget_words=64)
@@ -767,11 +800,14 @@ def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict) -> List[t
     em.emit_double_cores(s)
     wide = low.n_chunks > 1
     G = 1 if wide else 4
+    # shared weights: kernel B writes one partial weight-gradient row per wave group, as the first-order
+    # backward does, and the runtime sizes both from the same figure (groups per block); bounded grid
+    G_b = 1 if em.NCH > 1 else (groups_b if low.shared_weights else G)
     blk_a = em.emit_tp_double_a(s, G, tune.get("dd_wa", 2))
-    blk_b = em.emit_tp_double_b(s, G, tune.get("dd_wb", 2))
-    G_b = 1 if em.NCH > 1 else G
+    blk_b = em.emit_tp_double_b(s, G_b, tune.get("dd_wb", 2))
     return [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_A", blk_a, G * em.R, 0),
-            (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_b, G_b * em.R, 0)]
+            (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_b, G_b * em.R,
+             compute_units * 8 if low.shared_weights else 0)]
 
 
 def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: int) -> List[tuple]:

@@ -864,22 +864,47 @@ int oeq_conv_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const voi
 // Kernel B alone is a complete set when it also produces kernel A's result (convolution, merged form).
 int oeq_has_double_backward(const oeq_kernels* k) { return k && k->roles[OEQ_ROLE_DOUBLE_BACKWARD_B].present; }
 
+size_t oeq_tp_double_backward_workspace_bytes(const oeq_kernels* k, int64_t num_batch) {
+    if (!k || !k->dims.shared_weights || !k->roles[OEQ_ROLE_DOUBLE_BACKWARD_B].present) return 0;
+    size_t rows = (size_t)k->grid_for(OEQ_ROLE_DOUBLE_BACKWARD_B, num_batch) * (size_t)k->dims.wpartial_per_block;
+    return align_up(rows * (size_t)k->dims.weight_numel * (size_t)k->dims.elem_size, 256);
+}
+
 int oeq_tp_double_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in, const void* L2_in, const void* W,
                            const void* L3_grad, const void* L1_dgrad, const void* L2_dgrad, const void* W_dgrad,
-                           void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad, void* stream) {
+                           void* L1_grad, void* L2_grad, void* W_grad, void* L3_dgrad, void* workspace,
+                           size_t workspace_bytes, void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: NULL kernel set");
     if (!oeq_has_double_backward(k) || !k->roles[OEQ_ROLE_DOUBLE_BACKWARD_A].present)
         return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: this kernel set has no second-order kernels");
     if (num_batch < 0) return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: negative batch");
-    if (num_batch == 0) return OEQ_OK;
+    const bool shared = k->dims.shared_weights != 0;
+    if (num_batch == 0) {
+        // per-row weights: every operand is empty; shared weights: the weight gradient is a sum over no rows
+        if (!shared) return OEQ_OK;
+        if (!W_grad) return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: NULL W_grad");
+        return k->fill_zero(W_grad, (size_t)k->dims.weight_numel * k->dims.elem_size, stream);
+    }
     if (!L1_in || !L2_in || !W || !L3_grad || !L1_dgrad || !L2_dgrad || !W_dgrad || !L1_grad || !L2_grad || !W_grad ||
         !L3_dgrad)
         return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: NULL buffer");
+    size_t need = oeq_tp_double_backward_workspace_bytes(k, num_batch);
+    if (need && (!workspace || workspace_bytes < need))
+        return fail(OEQ_ERR_INVALID, "oeq_tp_double_backward: workspace too small (%zu < %zu bytes)", workspace_bytes,
+                    need);
+    void* wpartial = need ? workspace : nullptr;
     void* a[] = {&num_batch, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_dgrad};
     int rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_A, num_batch, a, stream);
     if (rc) return rc;
-    void* b[] = {&num_batch, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_grad, &L1_grad, &L2_grad, &W_grad};
-    return k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, num_batch, b, stream);
+    void* b[] = {&num_batch, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_grad, &L1_grad, &L2_grad, &W_grad,
+                 &wpartial};
+    rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, num_batch, b, stream);
+    if (rc || !shared) return rc;
+    // shared weights: the partial weight gradients of the wave groups, summed in block order
+    int64_t n_partials = (int64_t)k->grid_for(OEQ_ROLE_DOUBLE_BACKWARD_B, num_batch) * k->dims.wpartial_per_block;
+    int64_t wn = k->dims.weight_numel;
+    void* rargs[] = {&n_partials, &wpartial, &W_grad, &wn};
+    return k->launch(OEQ_ROLE_TP_BACKWARD_WREDUCE, wn, rargs, stream);
 }
 
 int oeq_conv_double_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in,

@@ -151,7 +151,8 @@ EXPORTS = {
     "oeq_conv_double_backward_indexed": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 14 + [_P, _SZ, _P, _SZ, _P]),
     "oeq_conv_double_backward_scratch_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_has_double_backward": (ctypes.c_int, [_P]),
-    "oeq_tp_double_backward": (ctypes.c_int, [_P, _I64] + [_P] * 12),
+    "oeq_tp_double_backward": (ctypes.c_int, [_P, _I64] + [_P] * 12 + [_SZ, _P]),
+    "oeq_tp_double_backward_workspace_bytes": (_SZ, [_P, _I64]),
     "oeq_conv_double_backward": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 15 + [_SZ, _P]),
     "oeq_segment_sum": (ctypes.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _SZ, _P]),
     "oeq_segment_sum_workspace_bytes": (_SZ, [_P, _I64]),
@@ -373,9 +374,12 @@ class KernelSet:
     def has_double_backward(self) -> bool:
         return bool(self._lib.oeq_has_double_backward(self.handle))
 
-    def tp_double_backward(self, n, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg, stream):
-        _check(self._lib.oeq_tp_double_backward(self.handle, n, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg, stream),
-               "oeq_tp_double_backward")
+    def tp_double_backward_workspace_bytes(self, n) -> int:
+        return self._lib.oeq_tp_double_backward_workspace_bytes(self.handle, n)
+
+    def tp_double_backward(self, n, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg, ws, ws_bytes, stream):
+        _check(self._lib.oeq_tp_double_backward(self.handle, n, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg, ws,
+                                                ws_bytes, stream), "oeq_tp_double_backward")
 
     def conv_double_backward(self, nodes, nnz, x, y, w, g, ddx, ddy, ddw, dx, dy, dw, gg, rows, cols, perm, ws,
                              ws_bytes, stream):

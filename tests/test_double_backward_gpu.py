@@ -74,6 +74,23 @@ CASES = [
 ]
 
 
+def _shared(problem):
+    q = problem.clone()
+    q.shared_weights = True
+    return q
+
+
+# shared weights (batch kernels only): one weight vector, its gradient summed over the rows
+SHARED = [
+    ("cfg2-shared", lambda: _shared(P.config2_nequip_uvu()), 257),
+    ("cfg2-shared-f64", lambda: _shared(_f64(P.config2_nequip_uvu())), 129),
+    ("cfg3-shared", lambda: _shared(P.config3_mace_uvu()), 67),
+    ("odd-shared", lambda: _shared(_odd()), 333),
+    ("cfg1-shared", lambda: _shared(P.config1_single_uvu()), 1000),
+    ("folded-gaps-shared", lambda: _shared(_folded()), 61),
+]
+
+
 def _rand(rng, shape, dt):
     return torch.tensor(rng.uniform(-1, 1, size=shape).astype(dt), device="cuda")
 
@@ -84,7 +101,7 @@ def _check(names, fused, composed, tol):
         assert e <= tol, (name, e)
 
 
-@pytest.mark.parametrize("name,make,batch", CASES, ids=[c[0] for c in CASES])
+@pytest.mark.parametrize("name,make,batch", CASES + SHARED, ids=[c[0] for c in CASES + SHARED])
 def test_tp_fused_matches_composition(name, make, batch):
     problem = make()
     tp = oeq.TensorProduct(problem)
@@ -94,7 +111,7 @@ def test_tp_fused_matches_composition(name, make, batch):
     rng = np.random.default_rng(5)
     x, a = (_rand(rng, (batch, e.L1), dt) for _ in range(2))
     y, b = (_rand(rng, (batch, e.L2), dt) for _ in range(2))
-    w, c = (_rand(rng, (batch, e.WN), dt) for _ in range(2))
+    w, c = (_rand(rng, (e.WN,) if problem.shared_weights else (batch, e.WN), dt) for _ in range(2))
     g = _rand(rng, (batch, e.L3), dt)
     fused = ops.tp_double_backward(x, y, w, g, a, b, c, tp.kid)
     composed = ops._second_order(lambda p, q, r: ops.tp_forward(p, q, r, tp.kid),
@@ -176,17 +193,20 @@ def test_conv_fused_isolated_nodes_and_empty():
 
 
 def test_edge_cases_and_refusals():
-    """Empty batch: nothing launched, empty results. Kernel sets without second-order kernels (shared
-    weights) refuse the fused entry point loudly; autograd then composes first-order kernels instead."""
+    """Empty batch: nothing launched, empty results (a shared weight gradient: zeros). Kernel sets without
+    second-order kernels ('uvw') refuse the fused entry point loudly; autograd then composes first-order kernels
+    instead."""
     problem = P.config2_nequip_uvu()
     tp = oeq.TensorProduct(problem)
     e = ops.get_entry(tp.kid)
     empty = [torch.zeros((0, n), device="cuda") for n in (e.L1, e.L2, e.WN, e.L3, e.L1, e.L2, e.WN)]
     out = ops.tp_double_backward(*empty, tp.kid)
     assert [tuple(t.shape) for t in out] == [(0, e.L1), (0, e.L2), (0, e.WN), (0, e.L3)]
-    shared = problem.clone()
-    shared.shared_weights = True
-    tps = oeq.TensorProduct(shared)
+    tsh = oeq.TensorProduct(_shared(problem))
+    empty[2] = empty[6] = torch.rand(e.WN, device="cuda")
+    out = ops.tp_double_backward(*empty, tsh.kid)
+    assert tuple(out[2].shape) == (e.WN,) and float(out[2].abs().max()) == 0.0
+    tps = oeq.TensorProduct(P.config4_uvw_shared())
     es = ops.get_entry(tps.kid)
     assert not es.kernels().has_double_backward()
     rng = np.random.default_rng(1)
@@ -263,7 +283,9 @@ def _oracle_second_order(fn, x, y, w, g, a, b, c):
 
 
 ORACLE_TP = [("cfg1", P.config1_single_uvu, 64), ("cfg2", P.config2_nequip_uvu, 33), ("cfg3", P.config3_mace_uvu, 9),
-             ("cfg3-f64", lambda: _f64(P.config3_mace_uvu()), 5), ("folded-gaps", _folded, 17), ("odd", _odd, 40)]
+             ("cfg3-f64", lambda: _f64(P.config3_mace_uvu()), 5), ("folded-gaps", _folded, 17), ("odd", _odd, 40),
+             ("cfg2-shared", lambda: _shared(P.config2_nequip_uvu()), 33),
+             ("cfg3-shared-f64", lambda: _shared(_f64(P.config3_mace_uvu())), 5), ("odd-shared", lambda: _shared(_odd()), 40)]
 
 
 @pytest.mark.parametrize("name,make,batch", ORACLE_TP, ids=[c[0] for c in ORACLE_TP])
@@ -277,7 +299,7 @@ def test_tp_fused_matches_float64_autograd(name, make, batch):
     rng = np.random.default_rng(15)
     x, a = (_rand(rng, (batch, e.L1), dt) for _ in range(2))
     y, b = (_rand(rng, (batch, e.L2), dt) for _ in range(2))
-    w, c = (_rand(rng, (batch, e.WN), dt) for _ in range(2))
+    w, c = (_rand(rng, (e.WN,) if problem.shared_weights else (batch, e.WN), dt) for _ in range(2))
     g = _rand(rng, (batch, e.L3), dt)
     fused = ops.tp_double_backward(x, y, w, g, a, b, c, tp.kid)
     want = _oracle_second_order(TorchTP(R.Problem.from_spec(problem), torch.float64), x, y, w, g, a, b, c)
