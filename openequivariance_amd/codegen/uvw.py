@@ -12,6 +12,11 @@ Two kernel families are generated:
   the per-``u`` intermediates back from LDS as broadcasts;
 * for shared weights with 64-wide channel blocks, an MFMA kernel (see
   ``uvw_mfma.py``) that batches rows so that the channel mix is a dense GEMM.
+
+The general family also carries the second-order pair ``double_backward_A`` / ``double_backward_B`` (the
+reference's kernels of that name, templates/loop_unroll_batch.cuh:148-317 and
+templates/loop_unroll_conv_det.cuh:296-548): the forward- and backward-shaped kernels written with
+``second=True``, which read the operands of both orders in one pass.
 """
 
 from __future__ import annotations
@@ -32,26 +37,34 @@ class UvwEmitter:
     def __init__(self, low: Lowered):
         assert low.mode == "uvw"
         from .uvu import tuning
-        self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576, uvw_regdw=1, conv_hops=2, conv_fuse_uvw=1))
+        self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576, uvw_regdw=1, conv_hops=2, conv_fuse_uvw=1, uvw_dd=1))
         self.TILE_BYTES = self.tune["uvw_tile"]
         self.low = low
         self.T = low.ctype
         self.l2_pad = _pow2ceil(low.L2)
         self.max_d3 = max(low.out[p.io].d for p in low.paths)
+        self.second = False         # set while the second-order kernel B is being written
+        self.wvec_declared = False
 
     def lit(self, v: float) -> str:
         return float_literal(v, self.T)
 
-    def _products(self, s: Src, p: Path) -> Dict[int, Tuple[str, bool]]:
+    def _products(self, s: Src, p: Path, second: bool = False) -> Dict[int, Tuple[str, bool]]:
+        """|c| * y_j for the distinct (|c|, j) of a path: nnz index -> (name, negative). ``second``: the same
+        products of the second row ``brow`` as well, under the name with a ``b`` appended."""
         b2 = self.low.in2[p.i2]
         for j in sorted({j for _, j, _, _ in p.nnz}):
             s(f"const T y{j} = yrow[{b2.off} + v * {b2.d} + {j}];")
+            if second:
+                s(f"const T b{j} = brow[{b2.off} + v * {b2.d} + {j}];")
         names, out = {}, {}
         for n, (i, j, k, c) in enumerate(p.nnz):
             key = (self.lit(abs(c)), j)
             if key not in names:
                 names[key] = f"q{len(names)}"
                 s(f"const T {names[key]} = T({key[0]}) * y{j};")
+                if second:
+                    s(f"const T {names[key]}b = T({key[0]}) * b{j};")
             out[n] = (names[key], c < 0)
         return out
 
@@ -66,12 +79,16 @@ class UvwEmitter:
         s("const i64 rowc = live ? row : num_batch - 1;")
 
     # ------------------------------------------------------------- forward
-    def _forward_block(self, s: Src, io: int, acc: str = "acc"):
+    def _forward_block(self, s: Src, io: int, acc: str = "acc", second: bool = False):
         """Adds the contribution of one row (xrow, yrow, wrow) to the channels w = wc + lane of output block
         ``io``: the CG contraction with lanes = u goes to the wave's LDS tile, the channel mix reads it
-        back as broadcasts with lanes = w."""
+        back as broadcasts with lanes = w. ``second``: the three forward terms of the second-order pass,
+        F(a, y, w) + F(x, b, w) + F(x, y, c), as two channel mixes: the contraction of (a, y) and (x, b) mixed
+        with w, that of (x, y) with c."""
         low = self.low
         bo = low.out[io]
+        if second:
+            return self._forward_block_second(s, io, acc)
         for p in [q for q in low.paths if q.io == io]:
             b1, b2 = low.in1[p.i1], low.in2[p.i2]
             s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l}) {b1.mul}x{b2.mul}->{bo.mul}")
@@ -115,18 +132,82 @@ class UvwEmitter:
             s.close()
             s.close()
 
-    def emit_forward(self, s: Src):
+    def _forward_block_second(self, s: Src, io: int, acc: str):
+        low = self.low
+        bo = low.out[io]
+        D = self.max_d3
+        for p in [q for q in low.paths if q.io == io]:
+            b1, b2 = low.in1[p.i1], low.in2[p.i2]
+            s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l}) {b1.mul}x{b2.mul}->{bo.mul}")
+            s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
+            s.open(f"for (int uc = 0; uc < {b1.mul}; uc += 64)")
+            s.open("")
+            s("const int u = uc + lane;")
+            s(f"T x[{b1.d}], a[{b1.d}];")
+            s.open(f"if (u < {b1.mul})")
+            for i in range(b1.d):
+                s(f"x[{i}] = xrow[{b1.off} + u * {b1.d} + {i}]; a[{i}] = arow[{b1.off} + u * {b1.d} + {i}];")
+            s.close(" else {")
+            s.level += 1
+            for i in range(b1.d):
+                s(f"x[{i}] = T(0); a[{i}] = T(0);")
+            s.close()
+            prods = self._products(s, p, second=True)
+            started = set()
+            for n, (i, j, k, c) in enumerate(p.nnz):
+                q, neg = prods[n]
+                sg, op = ("-" if neg else ""), ("-=" if neg else "+=")
+                if k not in started:
+                    s(f"T t{k} = {sg}{q} * a[{i}]; T r{k} = {sg}{q} * x[{i}];")
+                    started.add(k)
+                else:
+                    s(f"t{k} {op} {q} * a[{i}]; r{k} {op} {q} * x[{i}];")
+                s(f"t{k} {op} {q}b * x[{i}];")
+            s("oeq_wave_sync();")
+            for k in range(bo.d):
+                s(f"s_t[wave][{k}][lane] = {'t%d' % k if k in started else 'T(0)'};")
+                s(f"s_t[wave][{D + k}][lane] = {'r%d' % k if k in started else 'T(0)'};")
+            s("oeq_wave_sync();")
+            s.close()
+            s(f"const int nu = ({b1.mul} - uc < 64) ? {b1.mul} - uc : 64;")
+            s(f"const i64 woff = {p.woff} + ((i64)uc * {b2.mul} + v) * {bo.mul} + w;")
+            s.open(f"if (w < {bo.mul})")
+            s.open("for (int uu = 0; uu < nu; ++uu)")
+            s(f"const T wv = wrow[woff + (i64)uu * {b2.mul * bo.mul}];")
+            s(f"const T cv = crow[woff + (i64)uu * {b2.mul * bo.mul}];")
+            for k in range(bo.d):
+                s(f"{acc}[{k}] += wv * s_t[wave][{k}][uu]; {acc}[{k}] += cv * s_t[wave][{D + k}][uu];")
+            s.close()
+            s.close()
+            s.close()
+            s.close()
+
+    def emit_forward(self, s: Src, second: bool = False):
+        """``second``: the kernel double_backward_A (three forward terms into L3_dgrad)."""
         low = self.low
         block = 64 * WAVES_PER_BLOCK
-        s.open(
-            f'extern "C" __global__ __launch_bounds__({block}) void forward(i64 num_batch, '
-            "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, T* __restrict__ L3_out)"
-        )
-        s(f"__shared__ T s_t[{WAVES_PER_BLOCK}][{self.max_d3}][64];")
+        if second:
+            s.open(
+                f'extern "C" __global__ __launch_bounds__({block}) void double_backward_A(i64 num_batch, '
+                "const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
+                "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
+                "T* __restrict__ L3_out)"
+            )
+        else:
+            s.open(
+                f'extern "C" __global__ __launch_bounds__({block}) void forward(i64 num_batch, '
+                "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
+                "T* __restrict__ L3_out)"
+            )
+        s(f"__shared__ T s_t[{WAVES_PER_BLOCK}][{self.max_d3 * (2 if second else 1)}][64];")
         self._row_loop_open(s)
         s(f"const T* xrow = L1_in + rowc * {low.L1};")
         s(f"const T* yrow = L2_in + rowc * {low.L2};")
         s(f"const T* wrow = W{'' if low.shared_weights else f' + rowc * {low.WN}'};")
+        if second:
+            s(f"const T* arow = L1_dgrad + rowc * {low.L1};")
+            s(f"const T* brow = L2_dgrad + rowc * {low.L2};")
+            s(f"const T* crow = W_dgrad{'' if low.shared_weights else f' + rowc * {low.WN}'};")
         s(f"T* zrow = L3_out + rowc * {low.L3};")
         for io, bo in enumerate(low.out):
             s(f"// ---- out[{io}]: {bo.mul} x l={bo.l}")
@@ -135,7 +216,7 @@ class UvwEmitter:
             s(f"T acc[{bo.d}];")
             for k in range(bo.d):
                 s(f"acc[{k}] = T(0);")
-            self._forward_block(s, io)
+            self._forward_block(s, io, second=second)
             s.open(f"if (live && w < {bo.mul})")
             for k in range(bo.d):
                 s(f"zrow[{bo.off} + w * {bo.d} + {k}] = acc[{k}];")
@@ -145,13 +226,14 @@ class UvwEmitter:
         s.close()
         return block
 
-    def emit_conv_forward(self, s: Src, kahan: bool = False):
+    def emit_conv_forward(self, s: Src, kahan: bool = False, second: bool = False):
         """Fused convolution, forward: the waves of a block share a receiver node's output segments (64
         channels of one output block each, lanes = w) and each keeps its segments in registers over the
         node's edges, whose senders' rows, Y rows and weight rows it reads in place: no gathered copy of X
         and no per-edge message tensor. The nodes are taken in the walk order of the index, the edges of a
         node in list order (so the sums do not depend on scheduling); with ``kahan`` each edge's message is
-        added with a compensation term. Returns (block size, nodes per block)."""
+        added with a compensation term. ``second``: the kernel double_backward_A of the convolution (the three
+        forward terms of the second-order pass, same walk). Returns (block size, nodes per block)."""
         low = self.low
         assert not low.shared_weights
         segs = [(io, wc) for io, bo in enumerate(low.out) for wc in range(0, bo.mul, 64)
@@ -160,13 +242,22 @@ class UvwEmitter:
         wpn = max(1, min(WAVES_PER_BLOCK, len(segs)))  # waves per node
         G = WAVES_PER_BLOCK // wpn
         block = 64 * wpn * G
-        s.open(
-            f'extern "C" __global__ __launch_bounds__({block}) void forward(i64 node_count, i64 nnz, '
-            "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
-            "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-            "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order)"
-        )
-        s(f"__shared__ T s_t[{wpn * G}][{self.max_d3}][64];")
+        if second:
+            s.open(
+                f'extern "C" __global__ __launch_bounds__({block}) void double_backward_A(i64 node_count, i64 nnz, '
+                "const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
+                "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
+                "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
+                "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order)"
+            )
+        else:
+            s.open(
+                f'extern "C" __global__ __launch_bounds__({block}) void forward(i64 node_count, i64 nnz, '
+                "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
+                "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
+                "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order)"
+            )
+        s(f"__shared__ T s_t[{wpn * G}][{self.max_d3 * (2 if second else 1)}][64];")
         s("const int lane = oeq_lane();")
         s("const int wave = oeq_wave();")
         s(f"const int g = wave / {wpn}, sg = wave % {wpn};")
@@ -199,19 +290,24 @@ class UvwEmitter:
                     s(f"comp[{k}] = T(0);")
             s.open("for (i64 pos = e0; pos < e1; ++pos)")
             s("const i64 e = oeq_idx(OEQ_EDGE(pos), nnz);")
-            s(f"const T* xrow = L1_in + oeq_idx(cols[e], node_count) * {low.L1};")
+            s("const i64 sender = oeq_idx(cols[e], node_count);")
+            s(f"const T* xrow = L1_in + sender * {low.L1};")
             s(f"const T* yrow = L2_in + e * {low.L2};")
             s(f"const T* wrow = W + e * {low.WN};")
+            if second:
+                s(f"const T* arow = L1_dgrad + sender * {low.L1};")
+                s(f"const T* brow = L2_dgrad + e * {low.L2};")
+                s(f"const T* crow = W_dgrad + e * {low.WN};")
             if kahan:
                 s(f"T msg[{bo.d}];")
                 for k in range(bo.d):
                     s(f"msg[{k}] = T(0);")
-                self._forward_block(s, io, "msg")
+                self._forward_block(s, io, "msg", second=second)
                 for k in range(bo.d):
                     s(f"{{ const T y = msg[{k}] - comp[{k}]; const T t = acc[{k}] + y; "
                       f"comp[{k}] = (t - acc[{k}]) - y; acc[{k}] = t; }}")
             else:
-                self._forward_block(s, io)
+                self._forward_block(s, io, second=second)
             s.close()
             s.open(f"if (live && w < {bo.mul})")
             for k in range(bo.d):
@@ -248,14 +344,22 @@ class UvwEmitter:
                                            (min(64, b1.mul - uc) * per_u) % vw == 0 for uc in chunk_starts)
         return elems, (vw if aligned else 1)
 
-    def emit_backward(self, s: Src, conv: bool = False):
+    def emit_backward(self, s: Src, conv: bool = False, second: bool = False, force_waves: int = 0):
         """``conv``: the fused convolution's backward. An edge is a row: X comes from the sender's row,
         the output gradient from the receiver's, the X gradient goes to the edge's row of ``dx_tmp``
         (summed per sender, in the order of the sender-major list, by ``fixup_backward``); per-row
-        weights only. The edges need no order here, so the kernel strides over the edge list as it is."""
+        weights only. The edges need no order here, so the kernel strides over the edge list as it is.
+
+        ``second``: the kernel double_backward_B. With cotangents (a, b, c) of the first-order (dX, dY, dW) and
+        G = W g, H = C g (two channel mixes where the composition of first-order kernels runs three):
+        d/dX_i = sum c (b_j G_k + y_j H_k), d/dY_j = sum c (a_i G_k + x_i H_k),
+        d/dW[u,v,w] = sum_k f_k g[w,k] with f_k = sum c (y_j a_i + b_j x_i). Same work decomposition and weight
+        staging as the first-order kernel, with a second tile for C. ``force_waves``: waves per block (shared
+        weights: the partial weight-gradient rows are counted per block of the first-order kernel)."""
         low = self.low
         shared = low.shared_weights
         assert not (conv and shared)
+        self.second = second
         plans = {p.index: self._tile_plan(p) for p in low.paths}
         tiled = [p for p in low.paths if plans[p.index]]
         waves = WAVES_PER_BLOCK
@@ -264,10 +368,13 @@ class UvwEmitter:
             # their rows hit different banks
             tile_elems = (max(min(64, low.in1[p.i1].mul) * self._row_stride(p) for p in tiled) + 3) // 4 * 4
             vw = 16 // low.elem_size
-            s(f"struct __attribute__((aligned(16))) wvec_t {{ T v[{vw}]; }};")
-            # keep a block's LDS near 40 KB, so that four blocks (and at least four waves) share a CU
-            per_wave = tile_elems * low.elem_size
-            waves = max(1, min(WAVES_PER_BLOCK, 40960 // per_wave))
+            if not getattr(self, "wvec_declared", False):
+                s(f"struct __attribute__((aligned(16))) wvec_t {{ T v[{vw}]; }};")
+                self.wvec_declared = True
+            # keep a block's LDS near 40 KB, so that four blocks (and at least four waves) share a CU; the
+            # second-order kernel holds two tiles per wave and is given twice that
+            per_wave = tile_elems * low.elem_size * (2 if second else 1)
+            waves = max(1, min(WAVES_PER_BLOCK, (81920 if second else 40960) // per_wave))
         # shared weights: each wave sums its rows' weight gradients in an LDS copy of the weight tensor
         # (when that fits) and writes it out once, instead of a read-modify-write of global memory per row
         self.shared_lds = False
@@ -283,20 +390,43 @@ class UvwEmitter:
                 off += low.in1[p.i1].mul * self._row_stride(p)
             self.wsh_elems = off
             if (self.tune["uvw_regdw"] and dw_regs <= 176 and all(1 < low.in1[p.i1].mul <= 64 for p in low.paths)
-                    and off * low.elem_size <= 49152):
+                    and off * low.elem_size * (2 if second else 1) <= 49152
+                    and (not force_waves or force_waves == WAVES_PER_BLOCK)):
                 self.reg_dw = True
                 waves = WAVES_PER_BLOCK
         if shared and not self.reg_dw:
             fit = 65536 // (low.WN * low.elem_size)
-            if fit >= 1:
+            if force_waves:
+                waves = force_waves
+                self.shared_lds = fit >= force_waves
+            elif fit >= 1:
                 self.shared_lds = True
                 waves = min(WAVES_PER_BLOCK, fit)
-        self.backward_waves = waves
+        if not second:
+            self.backward_waves = waves
         block = 64 * waves
+        name = "double_backward_B" if second else "backward"
+        operands = ("const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
+                    "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
+                    "const T* __restrict__ L3_grad, ")
         # register-resident weight gradients: left to one wave per SIMD with up to 512 registers (e3tools
         # transformer block: 0.29 ms against 0.57 ms with spills at 256; uvw_regdw=2 selects the latter)
         attr = " __attribute__((amdgpu_waves_per_eu(2, 2)))" if (self.reg_dw and self.tune["uvw_regdw"] == 2) else ""
-        if conv:
+        if second and conv:
+            s.open(
+                f'extern "C" __global__ __launch_bounds__({block}){attr} void {name}(i64 node_count, i64 nnz, '
+                + operands + "T* __restrict__ L2_grad, T* __restrict__ W_grad, const i64* __restrict__ rows, "
+                "const i64* __restrict__ cols, const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, "
+                "const i64* __restrict__ eperm, T* __restrict__ L3_dgrad, const i64* __restrict__ order)"
+            )
+            s("const i64 num_batch = nnz;")
+        elif second:
+            s.open(
+                f'extern "C" __global__ __launch_bounds__({block}){attr} void {name}(i64 num_batch, '
+                + operands + "T* __restrict__ L1_grad, T* __restrict__ L2_grad, T* __restrict__ W_grad, "
+                "T* __restrict__ wpartial)"
+            )
+        elif conv:
             s.open(
                 f'extern "C" __global__ __launch_bounds__({block}){attr} void backward(i64 node_count, i64 nnz, '
                 "const T* __restrict__ L1_in, T* __restrict__ L1_grad, const T* __restrict__ L2_in, "
@@ -317,14 +447,21 @@ class UvwEmitter:
         if tiled:
             # one path's weights of the row, then (in place) its weight gradients
             s(f"__shared__ __attribute__((aligned(16))) T s_w[{waves}][{tile_elems}];")
+            if second:
+                s(f"__shared__ __attribute__((aligned(16))) T s_c[{waves}][{tile_elems}];")
         if shared:
             s(f"T* prow = wpartial + ((i64)blockIdx.x * {waves} + oeq_wave()) * {low.WN};")
             if self.reg_dw:
                 s(f"__shared__ T s_wsh[{self.wsh_elems}];")
+                if second:
+                    s(f"__shared__ T s_csh[{self.wsh_elems}];")
                 for p in low.paths:
                     per_u, S = low.in2[p.i2].mul * low.out[p.io].mul, self._row_stride(p)
                     s(f"for (int t = threadIdx.x; t < {low.in1[p.i1].mul * per_u}; t += {block}) "
                       f"s_wsh[{self.wsh_base[p.index]} + t / {per_u} * {S - per_u} + t] = W[{p.woff} + t];")
+                    if second:
+                        s(f"for (int t = threadIdx.x; t < {low.in1[p.i1].mul * per_u}; t += {block}) "
+                          f"s_csh[{self.wsh_base[p.index]} + t / {per_u} * {S - per_u} + t] = W_dgrad[{p.woff} + t];")
                     s(f"T dwr{p.index}[{per_u}];")
                     s(f"for (int t = 0; t < {per_u}; ++t) dwr{p.index}[t] = T(0);")
                 s("__syncthreads();")
@@ -339,15 +476,25 @@ class UvwEmitter:
                       for p in low.paths if p.i1 == i1 and plans[p.index]]
             nv_max = max(self._pad_vectors(st[2], st[1] * 64, plans[st[2].index][1]) for st in steps0)
             s(f"wvec_t pf[{nv_max}];  // the next weight tile on its way from global memory to LDS")
+            if second:
+                s(f"wvec_t pfc[{nv_max}];")
         self._row_loop_open(s, waves)
         if conv:
-            s(f"const T* xrow = L1_in + oeq_idx(cols[rowc], node_count) * {low.L1};")
+            s("const i64 sender = oeq_idx(cols[rowc], node_count);")
+            s(f"const T* xrow = L1_in + sender * {low.L1};")
             s(f"const T* grow = L3_grad + oeq_idx(rows[rowc], node_count) * {low.L3};")
             s(f"T* dxrow = dx_tmp + rowc * {low.L1};")
+            if second:
+                s(f"const T* arow = L1_dgrad + sender * {low.L1};")
         else:
             s(f"const T* xrow = L1_in + rowc * {low.L1};")
             s(f"const T* grow = L3_grad + rowc * {low.L3};")
             s(f"T* dxrow = L1_grad + rowc * {low.L1};")
+            if second:
+                s(f"const T* arow = L1_dgrad + rowc * {low.L1};")
+        if second:
+            s(f"const T* brow = L2_dgrad + rowc * {low.L2};")
+            s(f"const T* crow = W_dgrad{'' if shared else f' + rowc * {low.WN}'};")
         s(f"const T* yrow = L2_in + rowc * {low.L2};")
         s(f"const T* wrow = W{'' if shared else f' + rowc * {low.WN}'};")
         if not shared:
@@ -379,6 +526,10 @@ class UvwEmitter:
                 s(f"T x[{b1.d}], dx[{b1.d}];")
                 for i in range(b1.d):
                     s(f"x[{i}] = uok ? xrow[{b1.off} + u * {b1.d} + {i}] : T(0); dx[{i}] = T(0);")
+                if second:
+                    s(f"T a[{b1.d}];")
+                    for i in range(b1.d):
+                        s(f"a[{i}] = uok ? arow[{b1.off} + u * {b1.d} + {i}] : T(0);")
                 for p in paths:
                     b2, bo = low.in2[p.i2], low.out[p.io]
                     s(f"// path {p.index}: l=({b1.l},{b2.l},{bo.l})")
@@ -450,6 +601,25 @@ class UvwEmitter:
         """dx, dy contributions of one (path, v) from G_k, and f_k = sum c x_i y_j (returns the k set)."""
         b2 = self.low.in2[p.i2]
         fstart = set()
+        if getattr(self, "second", False):
+            # second order: G_k = (W g)_k, H_k = (C g)_k; the products of the second row are named q<n>b
+            for n, (i, j, k, c) in enumerate(p.nnz):
+                q, neg = prods[n]
+                op = "-=" if neg else "+="
+                s(f"dx[{i}] {op} {q}b * {gname}{k}; dx[{i}] {op} {q} * H{k};")
+                if k not in fstart:
+                    s(f"T f{k} = {'-' if neg else ''}{q} * a[{i}];")
+                    fstart.add(k)
+                else:
+                    s(f"f{k} {op} {q} * a[{i}];")
+                s(f"f{k} {op} {q}b * x[{i}];")
+            pair = {}
+            for n, (i, j, k, c) in enumerate(p.nnz):
+                if (i, k) not in pair:
+                    pair[(i, k)] = f"xg{len(pair)}"
+                    s(f"const T {pair[(i, k)]} = a[{i}] * {gname}{k} + x[{i}] * H{k};")
+                s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * {pair[(i, k)]};")
+            return sorted(fstart)
         for n, (i, j, k, c) in enumerate(p.nnz):
             q, neg = prods[n]
             s(f"dx[{i}] {'-=' if neg else '+='} {q} * {gname}{k};")
@@ -477,15 +647,21 @@ class UvwEmitter:
         s.open("")
         s(f"const T* gq = grow + {bo.off};  // wave-uniform")
         s(f"const T* wl = s_wsh + {self.wsh_base[p.index]} + (uok ? u : 0) * {S};")
+        second = self.second
+        if second:
+            s(f"const T* cl = s_csh + {self.wsh_base[p.index]} + (uok ? u : 0) * {S};")
         for vv in range(V):
             s.open("")
             s(f"const int v = {vv};")
-            prods = self._products(s, p)
+            prods = self._products(s, p, second)
             for k in range(d3):
-                s(f"T G{k} = T(0);")
+                s(f"T G{k} = T(0);" + (f" T H{k} = T(0);" if second else ""))
             for w in range(Wn):
                 s(f"{{ const T wv = wl[{vv * Wn + w}]; " +
                   " ".join(f"G{k} += wv * gq[{w * d3 + k}];" for k in range(d3)) + " }")
+                if second:
+                    s(f"{{ const T cv = cl[{vv * Wn + w}]; " +
+                      " ".join(f"H{k} += cv * gq[{w * d3 + k}];" for k in range(d3)) + " }")
             ks = self._cg_backward(s, p, prods)
             s.open("if (uok && live)")
             for w in range(Wn):
@@ -506,15 +682,20 @@ class UvwEmitter:
         b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
         Wn, d3 = bo.mul, bo.d
         nchunk = (Wn + 63) // 64
+        second = self.second
         s.open("")
         s(f"T xu[{b1.d}];")
         for i in range(b1.d):
             s(f"xu[{i}] = xrow[{b1.off} + {i}];")
+        if second:
+            s(f"T au[{b1.d}];")
+            for i in range(b1.d):
+                s(f"au[{i}] = arow[{b1.off} + {i}];")
         s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
-        prods = self._products(s, p)
+        prods = self._products(s, p, second)
         s(f"const int wbase = {p.woff} + v * {Wn};")
         for k in range(d3):
-            s(f"T G{k} = T(0);")
+            s(f"T G{k} = T(0);" + (f" T H{k} = T(0);" if second else ""))
         if nchunk == 1:
             s(f"T gv[{d3}];")
         for c in range(nchunk):
@@ -523,31 +704,47 @@ class UvwEmitter:
             s(f"const bool wok = w < {Wn};")
             s(f"const int wc = wok ? w : {Wn - 1};")
             s("const T wv = wok ? wrow[wbase + wc] : T(0);")
+            if second:
+                s("const T cv = wok ? crow[wbase + wc] : T(0);")
             for k in range(d3):
                 ld = f"grow[{bo.off} + wc * {d3} + {k}]"
                 if nchunk == 1:
                     s(f"gv[{k}] = wok ? {ld} : T(0);")
                     s(f"G{k} += wv * gv[{k}];")
+                    if second:
+                        s(f"H{k} += cv * gv[{k}];")
+                elif second:
+                    s(f"{{ const T gl = {ld}; G{k} += wv * gl; H{k} += cv * gl; }}")
                 else:
                     s(f"G{k} += wv * {ld};")
             s.close()
         for k in range(d3):
             for m in (32, 16, 8, 4, 2, 1):
                 s(f"G{k} += __shfl_xor(G{k}, {m});")
+                if second:
+                    s(f"H{k} += __shfl_xor(H{k}, {m});")
         # wave-uniform from here on; only lane 0 (uok) keeps the dX / dY terms
         fstart = set()
         for n, (i, j, k, c) in enumerate(p.nnz):
             q, neg = prods[n]
+            first_op = "xu" if not second else "au"
             if k not in fstart:
-                s(f"T f{k} = {'-' if neg else ''}{q} * xu[{i}];")
+                s(f"T f{k} = {'-' if neg else ''}{q} * {first_op}[{i}];")
                 fstart.add(k)
             else:
-                s(f"f{k} {'-=' if neg else '+='} {q} * xu[{i}];")
+                s(f"f{k} {'-=' if neg else '+='} {q} * {first_op}[{i}];")
+            if second:
+                s(f"f{k} {'-=' if neg else '+='} {q}b * xu[{i}];")
         s.open("if (uok)")
         for n, (i, j, k, c) in enumerate(p.nnz):
             q, neg = prods[n]
-            s(f"dx[{i}] {'-=' if neg else '+='} {q} * G{k};")
-            s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * (xu[{i}] * G{k});")
+            if second:
+                op = "-=" if neg else "+="
+                s(f"dx[{i}] {op} {q}b * G{k}; dx[{i}] {op} {q} * H{k};")
+                s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * (au[{i}] * G{k} + xu[{i}] * H{k});")
+            else:
+                s(f"dx[{i}] {'-=' if neg else '+='} {q} * G{k};")
+                s(f"dy[{b2.off} + v * {b2.d} + {j}] += T({self.lit(c)}) * (xu[{i}] * G{k});")
         s.close()
         ks = sorted(fstart)
         for c in range(nchunk):
@@ -575,17 +772,23 @@ class UvwEmitter:
         low = self.low
         shared = low.shared_weights
         b2, bo = low.in2[p.i2], low.out[p.io]
+        second = self.second
         s.open(f"for (int v = 0; v < {b2.mul}; ++v)")
-        prods = self._products(s, p)
+        prods = self._products(s, p, second)
         s(f"const i64 wbase = {p.woff} + ((i64)u * {b2.mul} + v) * {bo.mul};")
         # G_k = sum_w W[u,v,w] * g[w,k]
         for k in range(bo.d):
-            s(f"T G{k} = T(0);")
+            s(f"T G{k} = T(0);" + (f" T H{k} = T(0);" if second else ""))
         s.open("if (uok)")
         s.open(f"for (int w = 0; w < {bo.mul}; ++w)")
         s("const T wv = wrow[wbase + w];")
+        if second:
+            s("const T cv = crow[wbase + w];")
         for k in range(bo.d):
-            s(f"G{k} += wv * grow[{bo.off} + w * {bo.d} + {k}];")
+            if second:
+                s(f"{{ const T gl = grow[{bo.off} + w * {bo.d} + {k}]; G{k} += wv * gl; H{k} += cv * gl; }}")
+            else:
+                s(f"G{k} += wv * grow[{bo.off} + w * {bo.d} + {k}];")
         s.close()
         s.close()
         ks = self._cg_backward(s, p, prods)
@@ -638,32 +841,35 @@ class UvwEmitter:
         return -(-nel // (64 * vw))
 
     def _pad_issue(self, s: Src, p: Path, uc: int, vw: int):
-        """Request this lane's share of a step's contiguous weight block (coalesced 16-byte reads)."""
+        """Request this lane's share of a step's contiguous weight block (coalesced 16-byte reads); in the
+        second-order kernel the same block of the second weight tensor as well."""
         per_u, nel, tbase, _ = self._pad_geometry(p, uc, vw)
-        for q in range(self._pad_vectors(p, uc, vw)):
-            t = f"(lane + {64 * q}) * {vw}"
-            guard = "" if (64 * q + 64) * vw <= nel else f"if ({t} < {nel}) "
-            if vw > 1:
-                s(f"{guard}pf[{q}] = *(const wvec_t*)(wrow + {tbase} + {t});")
-            else:
-                s(f"{guard}pf[{q}].v[0] = wrow[{tbase} + {t}];")
+        for pf, row in (("pf", "wrow"), ("pfc", "crow"))[:2 if getattr(self, "second", False) else 1]:
+            for q in range(self._pad_vectors(p, uc, vw)):
+                t = f"(lane + {64 * q}) * {vw}"
+                guard = "" if (64 * q + 64) * vw <= nel else f"if ({t} < {nel}) "
+                if vw > 1:
+                    s(f"{guard}{pf}[{q}] = *(const wvec_t*)({row} + {tbase} + {t});")
+                else:
+                    s(f"{guard}{pf}[{q}].v[0] = {row}[{tbase} + {t}];")
 
     def _pad_commit(self, s: Src, p: Path, uc: int, vw: int):
         """Registers -> padded LDS tile (row r of the block starts at r * S)."""
         per_u, nel, _, S = self._pad_geometry(p, uc, vw)
-        for q in range(self._pad_vectors(p, uc, vw)):
-            t = f"(lane + {64 * q}) * {vw}"
-            s.open("" if (64 * q + 64) * vw <= nel else f"if ({t} < {nel})")
-            s(f"const int t = {t};")
-            if per_u % vw == 0:
-                s(f"const int tr = t / {per_u};")
-                s(f"T* dst = tw + tr * {S - per_u} + t;")
-                for i in range(vw):
-                    s(f"dst[{i}] = pf[{q}].v[{i}];")
-            else:  # a vector can straddle two rows
-                for i in range(vw):
-                    s(f"tw[(t + {i}) / {per_u} * {S - per_u} + t + {i}] = pf[{q}].v[{i}];")
-            s.close()
+        for pf, tw in (("pf", "tw"), ("pfc", "tc"))[:2 if getattr(self, "second", False) else 1]:
+            for q in range(self._pad_vectors(p, uc, vw)):
+                t = f"(lane + {64 * q}) * {vw}"
+                s.open("" if (64 * q + 64) * vw <= nel else f"if ({t} < {nel})")
+                s(f"const int t = {t};")
+                if per_u % vw == 0:
+                    s(f"const int tr = t / {per_u};")
+                    s(f"T* dst = {tw} + tr * {S - per_u} + t;")
+                    for i in range(vw):
+                        s(f"dst[{i}] = {pf}[{q}].v[{i}];")
+                else:  # a vector can straddle two rows
+                    for i in range(vw):
+                        s(f"{tw}[(t + {i}) / {per_u} * {S - per_u} + t + {i}] = {pf}[{q}].v[{i}];")
+                s.close()
 
     def _bwd_path_padded(self, s: Src, p: Path, vw: int, uc: int, nxt):
         """One step of the pipelined per-row-weight backward. The step's weights are in ``pf``; they go
@@ -679,7 +885,10 @@ class UvwEmitter:
         per_u, nel, tbase, S = self._pad_geometry(p, uc, vw)
         unroll = max(1, self.tune["uvw_unroll"])
         s.open("")
+        second = self.second
         s("T* tw = s_w[wave];")
+        if second:
+            s("T* tc = s_c[wave];")
         s(f"const T* gq = grow + {bo.off};  // wave-uniform")
         s("oeq_wave_sync();  // the previous step's tile is no longer read")
         self._pad_commit(s, p, uc, vw)
@@ -688,15 +897,21 @@ class UvwEmitter:
         s("oeq_wave_sync();")
         s("const int urow = uok ? lane : 0;  // lanes without a channel read row 0 and store nothing")
         s.open(f"for (int v = 0; v < {V}; ++v)")
-        prods = self._products(s, p)
+        prods = self._products(s, p, second)
         s(f"T* trow = tw + urow * {S} + v * {Wn};")
+        if second:
+            s(f"const T* crw = tc + urow * {S} + v * {Wn};")
         for k in range(bo.d):
-            s(f"T G{k} = T(0);")
+            s(f"T G{k} = T(0);" + (f" T H{k} = T(0);" if second else ""))
         s(f"#pragma unroll {unroll}")
         s.open(f"for (int w = 0; w < {Wn}; ++w)")
         s("const T wv = trow[w];")
+        if second:
+            s("const T cv = crw[w];")
         for k in range(bo.d):
             s(f"G{k} += wv * gq[w * {bo.d} + {k}];")
+            if second:
+                s(f"H{k} += cv * gq[w * {bo.d} + {k}];")
         s.close()
         ks = self._cg_backward(s, p, prods)
         s.open("if (uok)")
@@ -756,7 +971,14 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     blk_b = em.emit_backward(s, conv=True)
     s(fixup_backward_kernel(low.L1, kahan, True))
     cu = compute_units
-    descs = [
+    second = []
+    if em.tune["uvw_dd"] and not kahan:
+        # second-order pair: the same receiver walk / per-edge pass with the operands of both orders
+        blk_da, G_da = em.emit_conv_forward(s, False, second=True)
+        blk_db = em.emit_backward(s, conv=True, second=True)
+        second = [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_A", blk_da, G_da, cu * 32),
+                  (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_db, 1, cu * 16)]
+    descs = second + [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, cu * 16),
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, cu * 16),
         (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f, cu * 32),
@@ -792,7 +1014,15 @@ def tp_module(low: Lowered, compute_units: int = 256, kahan: bool = False):
     blk_f = em.emit_forward(s)
     blk_b = em.emit_backward(s)
     max_blocks_b = compute_units * (3 if em.shared_lds else 2)
-    descs = [
+    second = []
+    if em.tune["uvw_dd"]:
+        blk_da = em.emit_forward(s, second=True)
+        blk_db = em.emit_backward(s, second=True, force_waves=em.backward_waves if low.shared_weights else 0)
+        waves_db = blk_db // 64
+        second = [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_A", blk_da, WAVES_PER_BLOCK, compute_units * 16),
+                  (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_db, waves_db,
+                   max_blocks_b if low.shared_weights else compute_units * 16)]
+    descs = second + [
         (rt.ROLE_TP_FORWARD, "forward", blk_f, WAVES_PER_BLOCK, compute_units * 16),
         (rt.ROLE_TP_BACKWARD, "backward", blk_b, em.backward_waves,
          max_blocks_b if low.shared_weights else compute_units * 16),

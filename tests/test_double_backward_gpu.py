@@ -91,6 +91,36 @@ SHARED = [
 ]
 
 
+def _fc(shared, in2="1x0e+2x1o"):
+    return P.FullyConnectedTPProblem("4x0e+3x1o", in2, "5x0e+2x1o+1x2e", shared_weights=shared,
+                                     internal_weights=False, label="fc-uvw")
+
+
+def _wide_fc(shared):
+    # channel blocks that are no multiples of 16 (no matrix-core path) and wider than a wave
+    return P.FullyConnectedTPProblem("70x0e+20x1o", "1x0e+1x1o", "70x0e+20x1o", shared_weights=shared,
+                                     internal_weights=False, label="wide-fc-uvw")
+
+
+# fully connected ('uvw') problems: per-row weights (weight tiles in LDS, single-channel operands, direct access)
+# and shared weights outside the matrix-core path (gradients in registers, in LDS, or summed in global memory)
+UVW = [
+    ("uvw-fc", lambda: _fc(False), 129),
+    ("uvw-fc-f64", lambda: _f64(_fc(False)), 65),
+    ("uvw-fc-mul2", lambda: _fc(False, "2x0e+3x1o"), 65),
+    ("uvw-diffdock", lambda: P.diffdock_problems()[0], 65),
+    ("uvw-diffdock-f64", lambda: _f64(P.diffdock_problems()[0]), 33),
+    ("uvw-e3tools-conv", lambda: P.e3tools_problems()[0], 65),
+    ("uvw-wide", lambda: _wide_fc(False), 17),
+    ("uvw-fc-shared", lambda: _fc(True), 129),
+    ("uvw-fc-shared-f64", lambda: _f64(_fc(True)), 65),
+    ("uvw-tetris-1-shared", lambda: P.tetris_poly_problems()[0], 129),
+    ("uvw-tetris-2-shared", lambda: P.tetris_poly_problems()[1], 65),
+    ("uvw-wide-shared", lambda: _wide_fc(True), 600),
+]
+UVW_CONV = [c for c in UVW if not c[0].endswith(("shared", "shared-f64"))]
+
+
 def _rand(rng, shape, dt):
     return torch.tensor(rng.uniform(-1, 1, size=shape).astype(dt), device="cuda")
 
@@ -101,7 +131,7 @@ def _check(names, fused, composed, tol):
         assert e <= tol, (name, e)
 
 
-@pytest.mark.parametrize("name,make,batch", CASES + SHARED, ids=[c[0] for c in CASES + SHARED])
+@pytest.mark.parametrize("name,make,batch", CASES + SHARED + UVW, ids=[c[0] for c in CASES + SHARED + UVW])
 def test_tp_fused_matches_composition(name, make, batch):
     problem = make()
     tp = oeq.TensorProduct(problem)
@@ -124,7 +154,7 @@ def _graph(n=60):
     return CoordGraph(coords, rows, cols)
 
 
-CONV_CASES = [c for c in CASES if c[0] not in ("cfg1",)] + [("cfg1", P.config1_single_uvu, 0)]
+CONV_CASES = [c for c in CASES if c[0] not in ("cfg1",)] + [("cfg1", P.config1_single_uvu, 0)] + UVW_CONV
 
 
 @pytest.mark.parametrize("det", [True, False], ids=["sorted", "grouped"])
@@ -285,7 +315,12 @@ def _oracle_second_order(fn, x, y, w, g, a, b, c):
 ORACLE_TP = [("cfg1", P.config1_single_uvu, 64), ("cfg2", P.config2_nequip_uvu, 33), ("cfg3", P.config3_mace_uvu, 9),
              ("cfg3-f64", lambda: _f64(P.config3_mace_uvu()), 5), ("folded-gaps", _folded, 17), ("odd", _odd, 40),
              ("cfg2-shared", lambda: _shared(P.config2_nequip_uvu()), 33),
-             ("cfg3-shared-f64", lambda: _shared(_f64(P.config3_mace_uvu())), 5), ("odd-shared", lambda: _shared(_odd()), 40)]
+             ("cfg3-shared-f64", lambda: _shared(_f64(P.config3_mace_uvu())), 5), ("odd-shared", lambda: _shared(_odd()), 40),
+             ("uvw-fc", lambda: _fc(False), 33), ("uvw-fc-mul2-f64", lambda: _f64(_fc(False, "2x0e+3x1o")), 17),
+             ("uvw-diffdock", lambda: P.diffdock_problems()[0], 9), ("uvw-e3tools-conv", lambda: P.e3tools_problems()[0], 9),
+             ("uvw-fc-shared", lambda: _fc(True), 33), ("uvw-tetris-1-shared", lambda: P.tetris_poly_problems()[0], 17),
+             ("uvw-tetris-2-shared-f64", lambda: _f64(P.tetris_poly_problems()[1]), 9),
+             ("uvw-wide-shared", lambda: _wide_fc(True), 9)]
 
 
 @pytest.mark.parametrize("name,make,batch", ORACLE_TP, ids=[c[0] for c in ORACLE_TP])
@@ -311,7 +346,9 @@ def test_tp_fused_matches_float64_autograd(name, make, batch):
 ORACLE_CONV = [("cfg2", P.config2_nequip_uvu), ("cfg5", P.config5_mace_conv),
                ("cfg5-f64", lambda: _f64(P.config5_mace_conv())), ("folded-gaps", _folded), ("odd", _odd),
                # many paths per output block: kernel A walks smaller output segments (38 and 68 paths)
-               ("sevennet-main", lambda: P.seven_net_problems()[1]), ("nequip-benzene", lambda: P.nequip_problems()[3])]
+               ("sevennet-main", lambda: P.seven_net_problems()[1]), ("nequip-benzene", lambda: P.nequip_problems()[3]),
+               ("uvw-fc", lambda: _fc(False)), ("uvw-fc-mul2-f64", lambda: _f64(_fc(False, "2x0e+3x1o"))),
+               ("uvw-diffdock", lambda: P.diffdock_problems()[0]), ("uvw-e3tools-conv", lambda: P.e3tools_problems()[0])]
 
 
 @pytest.mark.parametrize("det", [True, False], ids=["sorted", "grouped"])
