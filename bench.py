@@ -183,7 +183,8 @@ def tp_config_table(dev, only=None):
 def uvw_conv_table(dev, nodes=12000):
     """Side measurement: the fused 'uvw' convolution with per-edge weights (DiffDock, e3tools) on a graph of
     the headline's density, forward and backward, beside the unfused path (gathered rows, batch kernels,
-    segment sums) that it replaces. Bytes = every operand once (W and dW dominate: 27-30 KB per edge)."""
+    segment sums) that it replaces, and the second-order kernel pair beside the composition of first-order
+    calls. Bytes = every operand once per kernel (W and dW dominate: 27-30 KB per edge)."""
     import numpy as np
     import torch
 
@@ -229,6 +230,20 @@ def uvw_conv_table(dev, nodes=12000):
                 tb = med(lambda: ops.conv_backward(X, Y, W, G, tr, tc, tp, kid))
                 row[key] = {"fwd_ms": tf, "bwd_ms": tb, "fwd_hbm_frac": fb / tf / 1e6 / HBM_PEAK_GBS,
                             "bwd_hbm_frac": bb / tb / 1e6 / HBM_PEAK_GBS}
+                if fuse and ops.get_entry(kid).kernels().has_double_backward():
+                    # second-order pass: the fused kernel pair beside three forward and three backward calls
+                    A_, B_, C_ = torch.randn_like(X), torch.randn_like(Y), torch.randn_like(W)
+                    t2 = med(lambda: ops.conv_double_backward(X, Y, W, G, A_, B_, C_, tr, tc, tp, kid), it=5)
+                    tc2 = med(lambda: ops._second_order(
+                        lambda p, q, r: ops.conv_forward(p, q, r, tr, tc, tp, kid),
+                        lambda p, q, r, s_: ops.conv_backward(p, q, r, s_, tr, tc, tp, kid), X, Y, W, G, A_, B_, C_),
+                        warm=1, it=3)
+                    # per-edge tensors: Y, B, W, C read by both kernels, dY and dW written; node tensors once per
+                    # kernel (the per-edge dX terms and the re-gathered sender rows are not algorithmic)
+                    db = 4 * (E * 5 * (low.WN + low.L2) + nodes * (5 * low.L1 + 2 * low.L3))
+                    row["second_order"] = {"fused_ms": t2, "composed_first_order_ms": tc2,
+                                           "hbm_frac": db / t2 / 1e6 / HBM_PEAK_GBS}
+                    del A_, B_, C_
             table.append(row)
             del X, Y, W, G
             torch.cuda.empty_cache()
