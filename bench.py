@@ -173,6 +173,18 @@ def tp_config_table(dev, only=None):
             peak = 157.3 if es == 4 else 78.6  # dense MFMA TFLOP/s, fp32 / fp64
             row["fwd_mfma_frac"] = row["fwd_dense_tflops"] / peak
             row["bwd_mfma_frac"] = row["bwd_dense_tflops"] / peak
+        if name.startswith(("cfg2", "DiffDock")) and ops.get_entry(tp.kid).kernels().has_double_backward():
+            # second-order pass (the backward of the backward): the fused kernel pair beside the composition of
+            # three forward and three backward calls; bytes = every operand once per kernel
+            a, b, c = torch.randn_like(x), torch.randn_like(y), torch.randn_like(w)
+            t2 = med(lambda: ops.tp_double_backward(x, y, w, g, a, b, c, tp.kid), it=7)
+            tc = med(lambda: ops._second_order(lambda p, q, r: ops.tp_forward(p, q, r, tp.kid),
+                                               lambda p, q, r, s_: ops.tp_backward(p, q, r, s_, tp.kid),
+                                               x, y, w, g, a, b, c), warm=1, it=3)
+            db = B * (5 * low.L1 + 5 * low.L2 + 5 * wrow + 2 * low.L3) * es + 5 * wcall
+            row["second_order"] = {"fused_ms": t2, "composed_first_order_ms": tc,
+                                   "hbm_frac": db / t2 / 1e6 / HBM_PEAK_GBS}
+            del a, b, c
         table.append(row)
         del x, y, w, g
         torch.cuda.empty_cache()

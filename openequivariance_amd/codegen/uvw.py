@@ -37,7 +37,8 @@ class UvwEmitter:
     def __init__(self, low: Lowered):
         assert low.mode == "uvw"
         from .uvu import tuning
-        self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576, uvw_regdw=1, conv_hops=2, conv_fuse_uvw=1, uvw_dd=1))
+        self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576, uvw_regdw=1, conv_hops=2, conv_fuse_uvw=1, uvw_dd=1,
+                                uvw_dda_split=0, uvw_dda_unroll=4))
         self.TILE_BYTES = self.tune["uvw_tile"]
         self.low = low
         self.T = low.ctype
@@ -172,12 +173,27 @@ class UvwEmitter:
             s(f"const int nu = ({b1.mul} - uc < 64) ? {b1.mul} - uc : 64;")
             s(f"const i64 woff = {p.woff} + ((i64)uc * {b2.mul} + v) * {bo.mul} + w;")
             s.open(f"if (w < {bo.mul})")
-            s.open("for (int uu = 0; uu < nu; ++uu)")
-            s(f"const T wv = wrow[woff + (i64)uu * {b2.mul * bo.mul}];")
-            s(f"const T cv = crow[woff + (i64)uu * {b2.mul * bo.mul}];")
-            for k in range(bo.d):
-                s(f"{acc}[{k}] += wv * s_t[wave][{k}][uu]; {acc}[{k}] += cv * s_t[wave][{D + k}][uu];")
-            s.close()
+            mode, unroll = self.tune["uvw_dda_split"], self.tune["uvw_dda_unroll"]
+            if mode:
+                # one weight stream per loop, as in the first-order kernel
+                for row, base in (("wrow", 0), ("crow", D)):
+                    s(f"const T* {row[0]}p = {row} + woff;")
+                    if unroll:
+                        s(f"#pragma unroll {unroll}")
+                    s.open("for (int uu = 0; uu < nu; ++uu)")
+                    s(f"const T wv = {row[0]}p[(i64)uu * {b2.mul * bo.mul}];")
+                    for k in range(bo.d):
+                        s(f"{acc}[{k}] += wv * s_t[wave][{base + k}][uu];")
+                    s.close()
+            else:
+                if unroll:
+                    s(f"#pragma unroll {unroll}")
+                s.open("for (int uu = 0; uu < nu; ++uu)")
+                s(f"const T wv = wrow[woff + (i64)uu * {b2.mul * bo.mul}];")
+                s(f"const T cv = crow[woff + (i64)uu * {b2.mul * bo.mul}];")
+                for k in range(bo.d):
+                    s(f"{acc}[{k}] += wv * s_t[wave][{k}][uu]; {acc}[{k}] += cv * s_t[wave][{D + k}][uu];")
+                s.close()
             s.close()
             s.close()
             s.close()
