@@ -405,6 +405,17 @@ class UvuEmitter:
             conds.append(f"u < {mul}")
         return " && ".join(conds) if conds else None
 
+    @staticmethod
+    def _dump_unless(cond: Optional[str], ptr: str) -> str:
+        """Pointer of a store inside the chain of paths that only some lanes (or rows) may perform: the others
+        are pointed at a scratch array nobody reads, so the store itself is unconditional. A branch around it
+        would split the chain into basic blocks; the compiler then sinks the value's computation into the
+        conditional block and, when registers are short, spills values that live across it from inside that
+        block - with part of the lanes switched off, which leaves those lanes' copies stale. Wrong gradients
+        were measured from exactly this (rows of mixed multiplicity whose weight gradients could not be kept
+        in registers until the end of the row)."""
+        return ptr if not cond else f"(({cond}) ? {ptr} : oeq_dump + ((blockIdx.x & 63u) * 64u + (threadIdx.x & 63u)))"
+
     def _open_if(self, s: Src, cond: Optional[str], values: Sequence[str] = ()):
         """Open the block of a (possibly conditional) store of ``values``. Values that only a
         conditional store uses are first passed through an empty asm statement: the compiler would
@@ -644,6 +655,8 @@ class UvuEmitter:
             # what lanes without a channel read in place of an output-gradient block (see _gptr)
             extent = max((b.d - 1) * self._lane_ptr(b)[1] + 1 for b in partial)
             s(f"__device__ const T oeq_zero_row[{extent}] = {{}};")
+        # where lanes (or rows) that must not store point their store inside a chain of paths (see _dump_unless)
+        s("__device__ T oeq_dump[4096];")
         if self.can_preload and self.q_entries:
             # y: the edge's Y row; yq: the Y values this lane multiplies for the wave's product table
             # (a kernel uses one of the two)
@@ -1359,10 +1372,9 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
                 if dw_mode == "store" and self._dw_deferred(dw_guard):
                     s(f"dwkeep[{base_slot} + {v}] = dwv;")
                 elif dw_mode == "store":
-                    dwp = self._ptr("dwrow", (f"{p.woff} + ({v})", V))
-                    st = (f"__builtin_nontemporal_store(dwv, {dwp});" if self.nt & 2 else f"*{dwp} = dwv;")
-                    cond = self._store_cond(b1.mul, dw_guard)
-                    s(f"if ({cond}) {st}" if cond else st)
+                    dwp = self._dump_unless(self._store_cond(b1.mul, dw_guard),
+                                            self._ptr("dwrow", (f"{p.woff} + ({v})", V)))
+                    s(f"__builtin_nontemporal_store(dwv, {dwp});" if self.nt & 2 else f"*{dwp} = dwv;")
                 else:
                     s(f"dwacc[{base_slot} + {v}] += dwv;")
                 for j in js:

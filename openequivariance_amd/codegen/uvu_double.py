@@ -284,10 +284,9 @@ class DoubleEmitter(UvuEmitter):
                 elif deferred:
                     s(f"dwkeep[{base_slot} + {v}] = dwv;")
                 else:
-                    dwp = self._ptr("dwrow", (f"{p.woff} + ({v})", V))
-                    st = (f"__builtin_nontemporal_store(dwv, {dwp});" if self.nt & 2 else f"*{dwp} = dwv;")
-                    cond = self._store_cond(b1.mul, dw_guard)
-                    s(f"if ({cond}) {st}" if cond else st)
+                    dwp = self._dump_unless(self._store_cond(b1.mul, dw_guard),
+                                            self._ptr("dwrow", (f"{p.woff} + ({v})", V)))
+                    s(f"__builtin_nontemporal_store(dwv, {dwp});" if self.nt & 2 else f"*{dwp} = dwv;")
                 for j in js:
                     s(f"dy[{self._y_index(b2, v, j)}] += cv * h{j}; dy[{self._y_index(b2, v, j)}] += wv * ha{j};")
                 if fwd_acc:

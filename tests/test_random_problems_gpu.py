@@ -133,3 +133,32 @@ def test_random_problem(seed):
             want = _second_order(lambda p, q, s: oracle(p, q, s, torch.tensor(r_), torch.tensor(c_)), X, Y, W, G, A, Bc, C)
             _compare(f"conv second order det={det}", ops.conv_double_backward(X, Y, W, G, A, Bc, C, tr, tc, tpm, conv.kid),
                      want, tol)
+
+
+def test_weight_gradient_stores_of_partial_blocks_inside_the_path_chain():
+    """A row of mixed multiplicity (5, 96, 8 channels) with a second operand too long for the weight gradients
+    to wait in registers until the end of the row: their stores sit inside the chain of paths, and only the lanes
+    with a channel may store. As branches these stores once made the compiler spill, from inside a block that runs
+    with part of the lanes switched off, values that are used after it; dX and dY of fp32 and fp64 rows came out
+    wrong (found by a random draw of the generator above). The idle lanes now store to a scratch array instead."""
+    ins = [(0, 0, 0), (0, 0, 1), (1, 0, 2), (1, 0, 3), (1, 0, 4), (1, 1, 5), (1, 1, 6, 1.4141618459745515), (1, 1, 7),
+           (1, 1, 8), (1, 2, 9), (1, 2, 4), (2, 0, 10), (2, 0, 11, 0.6803777663418822), (2, 0, 12), (2, 1, 13), (2, 1, 14),
+           (2, 1, 15, 0.7911603214136989), (2, 1, 16), (2, 2, 10), (2, 2, 17), (2, 2, 18, 0.3223124028973989)]
+    ins = [(t[0], t[1], t[2], "uvu", True, t[3] if len(t) > 3 else 1.0) for t in ins]
+    out = ("5x1e+5x2e+96x0o+96x2o+96x3o+96x0e+96x1e+96x2e+96x3e+96x1o+8x0e+8x1e+8x3e+8x0o+8x1o+8x2o+8x3o+8x2e+8x3e")
+    for dt in (np.float32, np.float64):
+        problem = oeq.TPProblem("5x2e+96x3o+8x3e+16x0o", "3x3e+1x3o+1x3e", out, ins, shared_weights=False,
+                                internal_weights=False, irrep_dtype=dt, weight_dtype=dt)
+        ref = R.Problem.from_spec(problem)
+        tp = oeq.TensorProduct(problem)
+        e = ops.get_entry(tp.kid)
+        rng = np.random.default_rng(1)
+        B = 19
+        x, y, w, g = (_rand(rng, (B, n), dt) for n in (e.L1, e.L2, e.WN, e.L3))
+        a, b, c = (_rand(rng, (B, n), dt) for n in (e.L1, e.L2, e.WN))
+        tol = 1e-5 if dt == np.float32 else 1e-12
+        xn, yn, wn, gn = (t.cpu().numpy() for t in (x, y, w, g))
+        _compare("backward", ops.tp_backward(x, y, w, g, tp.kid), R.tp_backward(ref, xn, yn, wn, gn), tol)
+        from oracle.torch_ref import TorchTP
+        _compare("second order", ops.tp_double_backward(x, y, w, g, a, b, c, tp.kid),
+                 _second_order(TorchTP(ref, torch.float64), x, y, w, g, a, b, c), tol)
