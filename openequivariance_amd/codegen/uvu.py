@@ -168,8 +168,11 @@ class UvuEmitter:
 
     def _stage_src(self, blk, first_unit: int) -> str:
         """Row offset of the 16-byte unit ``t`` of the wave's slice of a block (units in LDS order)."""
-        if self.ir_mul:  # component i = 16 units of 4 channels each
-            return (f"{blk.off} + ((t - {first_unit}) >> 4) * {blk.mul} + chunk * 64 + ((t - {first_unit}) & 15) * 4")
+        if self.ir_mul:
+            # component i = 16 units of 4 channels each; the components of a piece of a folded block lie the
+            # whole block's multiplicity apart
+            return (f"{blk.off} + ((t - {first_unit}) >> 4) * {blk.cstride or blk.mul} + chunk * 64 + "
+                    f"((t - {first_unit}) & 15) * 4")
         return f"{blk.off} + chunk * {64 * blk.d} + (t - {first_unit}) * 4"
 
     def _stage_x(self, blk, base: int, i: int) -> str:

@@ -45,6 +45,12 @@ PROBLEMS = [
         "100x0e+70x1o+40x2e+96x1e", "1x0e+2x1o", "100x0e+70x1o+100x1o+40x1o+33x2e",
         [(0, 0, 0, "uvu", True), (1, 0, 1, "uvu", True), (0, 1, 2, "uvu", True), (2, 1, 3, "uvu", True, 0.7)],
         shared_weights=False, internal_weights=False, label="folded-gaps")),
+    # every piece exactly 64 channels wide (the shape the convolution's staged operand loads accept), one block
+    # folded into two of them: the staged loads must step a whole block's multiplicity between components
+    ("folded-64s", lambda: oeq.TPProblem(
+        "64x4e+128x3e", "1x1e+1x0e", "64x4e+128x2e+128x3e+128x4e+128x3e",
+        [(0, 1, 0, "uvu", True), (1, 0, 1, "uvu", True), (1, 0, 2, "uvu", True), (1, 0, 3, "uvu", True),
+         (1, 1, 4, "uvu", True)], shared_weights=False, internal_weights=False, label="folded-64s")),
 ]
 
 
@@ -84,7 +90,8 @@ def test_batch_ir_mul(name, make):
     assert err(z.detach(), z_w.cpu().numpy()) <= tol
 
 
-CONV = [c for c in PROBLEMS if c[0] in ("mace-large", "cfg3-f64", "cfg2", "13x5e", "multi-v", "multi-v-shared")]
+CONV = [c for c in PROBLEMS if c[0] in ("mace-large", "cfg3-f64", "cfg2", "13x5e", "multi-v", "multi-v-shared",
+                                        "nequix-first", "sevennet-main", "folded-gaps", "folded-64s")]
 
 
 @pytest.mark.parametrize("name,make", CONV, ids=[c[0] for c in CONV])
