@@ -471,13 +471,14 @@ int oeq_tp_backward(oeq_kernels* k, int64_t num_batch, const void* L1_in, void* 
                     size_t workspace_bytes, void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_tp_backward: NULL kernel set");
     if (num_batch < 0) return fail(OEQ_ERR_INVALID, "oeq_tp_backward: negative batch");
-    if (!W_grad) return fail(OEQ_ERR_INVALID, "oeq_tp_backward: NULL W_grad");
     const bool shared = k->dims.shared_weights != 0;
     if (num_batch == 0) {
-        if (shared) return k->fill_zero(W_grad, (size_t)k->dims.weight_numel * k->dims.elem_size, stream);
-        return OEQ_OK;
+        // per-row weights: every operand is empty; shared weights: the weight gradient is a sum over no rows
+        if (!shared) return OEQ_OK;
+        if (!W_grad) return fail(OEQ_ERR_INVALID, "oeq_tp_backward: NULL W_grad");
+        return k->fill_zero(W_grad, (size_t)k->dims.weight_numel * k->dims.elem_size, stream);
     }
-    if (!L1_in || !L1_grad || !L2_in || !L2_grad || !W || !L3_grad)
+    if (!L1_in || !L1_grad || !L2_in || !L2_grad || !W || !W_grad || !L3_grad)
         return fail(OEQ_ERR_INVALID, "oeq_tp_backward: NULL buffer");
     size_t need = oeq_tp_backward_workspace_bytes(k, num_batch);
     if (need && (!workspace || workspace_bytes < need))

@@ -185,9 +185,21 @@ def test_c_abi_direct_call():
 
 
 def test_empty_batch():
+    """No rows: empty results, nothing launched; through autograd too (the empty gradients have no address).
+    With shared weights the weight gradient is a sum over no rows: zeros."""
     tp = oeq.TensorProduct(P.config1_single_uvu())
-    z = tp(torch.zeros(0, 5, device="cuda"), torch.zeros(0, 7, device="cuda"), torch.zeros(0, 1, device="cuda"))
+    xs = [torch.zeros(0, n, device="cuda", requires_grad=True) for n in (5, 7, 1)]
+    z = tp(*xs)
     assert z.shape == (0, 5)
+    z.backward(torch.zeros(0, 5, device="cuda"))
+    assert [tuple(t.grad.shape) for t in xs] == [(0, 5), (0, 7), (0, 1)]
+    shared = P.config1_single_uvu().clone()
+    shared.shared_weights = True
+    tps = oeq.TensorProduct(shared)
+    xs = [torch.zeros(0, 5, device="cuda", requires_grad=True), torch.zeros(0, 7, device="cuda", requires_grad=True),
+          torch.ones(1, device="cuda", requires_grad=True)]
+    tps(*xs).backward(torch.zeros(0, 5, device="cuda"))
+    assert float(xs[2].grad.abs().max()) == 0.0 and xs[0].grad.shape == (0, 5)
 
 
 def test_full_size_properties_cfg3():
