@@ -59,6 +59,7 @@ from .lower import Lowered, Path, float_literal
 RT = 16          # rows per tile
 WAVES = 4        # waves per block
 TPAD = RT + 1    # padded row stride of the T tile in LDS (bank spread)
+LDS_BUDGET = 160 * 1024 - 2048   # bytes of LDS a kernel may declare (the CU has 160 KB)
 MFMA = "oeq_mfma"  # v_mfma_f32_16x16x4_f32 or v_mfma_f64_16x16x4_f64, see tp_module
 
 
@@ -144,6 +145,10 @@ def supported(low: Lowered) -> bool:
     if low.mode != "uvw" or not low.shared_weights or low.ctype not in ("float", "double") or low.ir_mul:
         return False
     if low.L3 > 1152 or low.L2 > 32:
+        return False
+    # the dX kernels keep a whole 16-row dZ tile in LDS beside the Y rows and the partial dY of the four waves
+    # (fp64: rows of up to about 1 000 elements)
+    if (RT * (low.L3 + 36) + (1 + WAVES) * RT * low.L2) * low.elem_size > LDS_BUDGET:
         return False
     for p in low.paths:
         a, b, o = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
@@ -594,7 +599,8 @@ class MfmaEmitter:
             if self.tune["uvw_pipe"]:
                 resident = lambda: sum(vp.Wn // 4 for vp in paths_all if vp.index not in self.lds_w)
                 # (what LDS has room for beside the dZ tile: a slice takes 16 x 256 elements)
-                room = (150 * 1024 - RT * self.gstride * low.elem_size) // (16 * 64 * WAVES * low.elem_size)
+                room = (LDS_BUDGET - (RT * self.gstride + (1 + WAVES) * RT * low.L2) * low.elem_size) // \
+                    (16 * 64 * WAVES * low.elem_size)
                 while len(paths_all) - len(self.lds_w) > 1 and len(self.lds_w) < min(3, room) and \
                         resident() + fixed(ker) > self.tune["uvw_regs"]:
                     self.lds_w.append(by_cost[len(self.lds_w)].index)
@@ -659,8 +665,19 @@ class MfmaEmitter:
             raise AssertionError("no path")
 
         # ---------------- dW ----------------------------------------------------
-        cost = lambda ker: (sum(4 * (vp.Wn // 16) for g in ker for vp in g[1]) + 2 * (RT // WAVES) * self.max_d1
+        regs = lambda ker: (sum(4 * (vp.Wn // 16) for g in ker for vp in g[1]) + 2 * (RT // WAVES) * self.max_d1
                             + 4 * max(self.vout[g[0]].mul // 16 for g in ker) + 64)
+
+        def dw_lds(ker, nbuf):
+            """Bytes of LDS of a dW kernel: the dZ columns of its pieces, the T tile (one or two copies), Y."""
+            first, last = self.vout[ker[0][0]], self.vout[ker[-1][0]]
+            ncols = last.off + last.mul * last.d - first.off
+            maxd = max(self.vout[g[0]].d for g in ker)
+            return (RT * self._tile_stride(ncols) + nbuf * maxd * self.tlanes * TPAD + RT * low.L2) * low.elem_size
+
+        # a kernel that would not fit the 160 KB of LDS with its pieces merged stays split (the register estimate
+        # is replaced by one beyond any limit)
+        cost = lambda ker: regs(ker) if dw_lds(ker, 1) <= LDS_BUDGET else 1 << 30
         groups = [g for g in _groups(self.vpaths, "vo", len(self.vout)) if g[1]]
         for ker in self._merge(groups, cost, self.tune["uvw_wregs"], self.vout):
             # pieces that share a kernel must be neighbours in the row: one dZ tile covers their columns
@@ -676,8 +693,13 @@ class MfmaEmitter:
             s("// ======== dW of the sub-paths into out pieces " + ", ".join(str(vo) for vo, _, _ in ker))
             self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_ww"])
             # only these pieces' columns of the dZ tile are needed (and kept)
+            # two copies of the T tile let a path's contraction be written while the previous path's is still
+            # being multiplied; where they do not fit (fp64, l = 3 outputs) one copy and a barrier more per path
+            nbuf = 2 if dw_lds(ker, 2) <= LDS_BUDGET else 1
+            if dw_lds(ker, nbuf) > LDS_BUDGET:
+                raise ValueError(f"the dW kernel of output piece {ker[0][0]} needs {dw_lds(ker, nbuf)} bytes of LDS")
             s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self._tile_stride(ncols)}];")
-            s(f"__shared__ T s_T[2][{maxd}][{self.tlanes}][{TPAD}];")
+            s(f"__shared__ T s_T[{nbuf}][{maxd}][{self.tlanes}][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             self._prologue(s)
             s("const int u = wave * 16 + l16;")
@@ -699,8 +721,10 @@ class MfmaEmitter:
             for n, vp in enumerate(order_all):
                 p = vp.p
                 bo = self.vout[vp.vo]
-                buf = n % 2
+                buf = n % nbuf
                 s(f"// path {p.index}: l=({low.in1[p.i1].l},{low.in2[p.i2].l},{bo.l})")
+                if nbuf == 1 and n > 0:
+                    s("__syncthreads();  // the previous path's T tile has been multiplied")
                 self._t_compute(s, vp, cur, str(buf))
                 if n + 1 < len(order_all):
                     self._load_x_rows(s, nxt, order_all[n + 1])

@@ -116,9 +116,17 @@ CASES = [
     # the same kernels in fp64 (v_mfma_f64_16x16x4_f64, whose result rows are laid out differently)
     ("mfma-128-f64", lambda: _as_f64(_fc_shared("128x0e+128x1o", "1x0e+1x1o", "128x0e+128x1o")), 45),
     ("mfma-mixed-f64", lambda: _as_f64(_fc_shared("64x0e+32x1o+16x2e", "1x0e+1x1o", "48x0e+80x1o+16x2e")), 50),
+    # fp64 with l = 3 outputs: two copies of the 64 x 7 x 17 T tile beside the dZ columns exceed the 160 KB of LDS;
+    # the dW kernels then keep one copy, and pieces whose columns would not fit together stay in separate kernels
+    ("mfma-l3-f64", lambda: _as_f64(oeq.TPProblem(
+        "64x1e+64x0e", "1x2o+1x2e+1x0o", "48x1e+80x3o", [(0, 0, 1, "uvw", True, 0.8), (0, 1, 0, "uvw", True)],
+        shared_weights=True, internal_weights=False, label="mfma-l3")), 50),
+    ("mfma-l3-wide-f64", lambda: _as_f64(oeq.TPProblem(
+        "16x1o+128x3o", "1x2o", "96x3e", [(0, 0, 0, "uvw", True), (1, 0, 0, "uvw", True, 0.6)],
+        shared_weights=True, internal_weights=False, label="mfma-l3-wide")), 40),
 ]
 MFMA_CASES = {"cfg4-shared", "cfg4-f64", "mfma-32", "mfma-128", "mfma-mixed", "mfma-gaps", "mfma-128-f64",
-              "mfma-mixed-f64"}
+              "mfma-mixed-f64", "mfma-l3-f64", "mfma-l3-wide-f64"}
 
 
 @pytest.mark.parametrize("name,make,B", CASES, ids=[c[0] for c in CASES])
