@@ -2212,7 +2212,9 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             coalesced = bool(t["conv_tra"]) and em._regular_wave() and not em.ir_mul
             dx_mode = t["conv_dxm"] if t["conv_dxm"] >= 0 else (
                 em.DX_ATOMIC if (mode == rt.CONV_GROUPED and coalesced) else em.DX_TERMS)
-            if dx_mode == em.DX_ARRIVAL and em.R != 1:
+            # arrival counting keeps an edge's terms lane-major, 64 values per (block, component) and chunk: they
+            # fit the edge's row of dx_tmp only when no used block has lanes without a channel
+            if dx_mode == em.DX_ARRIVAL and (em.R != 1 or 64 * em.NCH * em._term_slots()[1] > low.L1):
                 dx_mode = em.DX_TERMS
         blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd_b,
                                       bool(t["conv_tra"]), dx_mode)
