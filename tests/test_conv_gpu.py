@@ -38,6 +38,13 @@ def _odd(shared):
                           (0, 0, 2, "uvu", True)], shared_weights=shared, internal_weights=False, label="odd-uvu")
 
 
+def _ragged():
+    # one row per wave, lanes without a channel in every block
+    return oeq.TPProblem("40x1e+17x2e", "2x1e+1x0e", "40x1e+17x2e+40x0e",
+                         [(0, 0, 0, "uvu", True), (0, 1, 0, "uvu", True), (1, 0, 1, "uvu", True),
+                          (0, 0, 2, "uvu", True)], shared_weights=False, internal_weights=False, label="ragged-uvu")
+
+
 def _fc(shared):
     return P.FullyConnectedTPProblem("4x0e+3x1o", "1x0e+2x1o", "5x0e+2x1o+1x2e", shared_weights=shared,
                                      internal_weights=False, label="fc-uvw")
@@ -467,7 +474,7 @@ def test_kernel_shape_knobs_keep_results(knobs, monkeypatch):
     without the LDS transpose) computes the same convolution."""
     monkeypatch.setenv("OEQ_AMD_TUNE", knobs)
     # (a problem with lanes without a channel as well: the arrival-counting variant must step aside there)
-    for make in (P.config5_mace_conv, P.config2_nequip_uvu, lambda: _odd(False)):
+    for make in (P.config5_mace_conv, P.config2_nequip_uvu, _ragged):
         problem = make()
         coords, rows, cols = _graph(36, 6, seed=4)
         E = len(rows)
