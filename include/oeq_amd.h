@@ -256,9 +256,8 @@ size_t oeq_conv_double_backward_scratch_bytes(const oeq_kernels* k, int64_t node
  * L1_in, L2_in, W and L3_grad (all four fully overwritten). Replaces JITTPImpl::double_backward
  * (extension/tensorproducts.hpp:97-111) as called by jit_tp_double_backward
  * (extension/torch_core.hpp:357-420). Only kernel sets for which oeq_has_double_backward() is non-zero
- * carry these kernels ('uvu' problems, and 'uvw' problems whose channel mix does not run on the matrix cores;
- * with shared weights the batch entry point only); for the others the same result is composed from
- * oeq_tp_forward / oeq_tp_backward calls by the caller. */
+ * carry these kernels (by default every batch kernel set, and the convolutions with per-edge weights); for the
+ * others the same result is composed from oeq_tp_forward / oeq_tp_backward calls by the caller. */
 int oeq_has_double_backward(const oeq_kernels* k);
 int oeq_tp_double_backward(oeq_kernels* k, int64_t num_batch,
                            const void* L1_in, const void* L2_in, const void* W, const void* L3_grad,

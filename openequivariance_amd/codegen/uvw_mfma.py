@@ -186,7 +186,16 @@ class MfmaEmitter:
         # block sit out the multiplies and there are four times as many kernels.
         wpe = 2 if self.words == 1 else 1
         self.tune = tuning(dict(uvw_wf=wpe, uvw_wx=wpe, uvw_ww=wpe, uvw_blocks=2, uvw_pipe=1, uvw_regs=220,
-                                uvw_merge=1, uvw_fregs=232, uvw_wregs=232, uvw_xregs=215))
+                                uvw_merge=1, uvw_fregs=232, uvw_wregs=232, uvw_xregs=215, uvw_mfma_dd=1))
+
+    # Variant of the kernels being written (see second_order_kernels): a name prefix, the kernel signature, the
+    # lines that bind the names the bodies use (L1_in, L2_in, W, ...) to its parameters, whether every result is
+    # added to what the output holds, and whether the contraction T is that of the second-order pass,
+    # T(a, y) + T(x, b), with the second pair of operands bound to L1_alt / L2_alt.
+    prefix = ""
+    alias: List[str] = []
+    accumulate = False
+    t1 = False
 
     def lit(self, v):
         return float_literal(v, self.low.ctype)
@@ -252,6 +261,8 @@ class MfmaEmitter:
         s.open(f"for (int t = tid; t < {RT * low.L2}; t += {64 * WAVES})")
         s(f"const int r = t / {low.L2}, c = t % {low.L2};")
         s(f"s_y[r][c] = (row0 + r < num_batch) ? L2_in[(row0 + r) * {low.L2} + c] : T(0);")
+        if self.t1:
+            s(f"s_y2[r][c] = (row0 + r < num_batch) ? L2_alt[(row0 + r) * {low.L2} + c] : T(0);")
         s.close()
 
     def _tile_stride(self, ncols: int) -> int:
@@ -309,6 +320,10 @@ class MfmaEmitter:
         s(f"const T* xp = L1_in + row * {low.L1} + {a.off} + {lane} * {a.d};")
         for i in range(a.d):
             s(f"{dst}[rr][{i}] = xp[{i}];")
+        if self.t1:
+            s(f"const T* ap = L1_alt + row * {low.L1} + {a.off} + {lane} * {a.d};")
+            for i in range(a.d):
+                s(f"a{dst[1:]}[rr][{i}] = ap[{i}];")
         s.close()
 
     def _t_compute(self, s: Src, vp: VPath, xsrc: str, buf: str):
@@ -316,7 +331,15 @@ class MfmaEmitter:
         s.open(f"for (int rr = 0; rr < {RT // WAVES}; ++rr)")
         s(f"const int r = wave * {RT // WAVES} + rr;")
         s(f"T t[{d3}];")
-        s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y[r], t);")
+        if self.t1:
+            # contraction of the second-order pass: (a, y) and (x, b)
+            s(f"T t2[{d3}];")
+            s(f"cg_fwd{vp.p.index}(a{xsrc[1:]}[rr], s_y[r], t);")
+            s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y2[r], t2);")
+            for k in range(d3):
+                s(f"t[{k}] += t2[{k}];")
+        else:
+            s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y[r], t);")
         if self.tlanes < 64:
             s.open(f"if (lane < {self.tlanes})")
         for k in range(d3):
@@ -456,6 +479,8 @@ class MfmaEmitter:
         if waves_per_eu:
             attr += f" __attribute__((amdgpu_waves_per_eu({waves_per_eu}, {waves_per_eu})))"
         s.open(f'extern "C" __global__ {attr} void {name}{sig}')
+        for line in self.alias:
+            s(line)
 
     def _zero_kernel(self, s: Src, ptr: str, row_len: int, blk: VBlock):
         """A piece that no path touches: zeros."""
@@ -492,22 +517,30 @@ class MfmaEmitter:
         are resident and register allocation is per kernel. Returns the kernel names in launch order."""
         low = self.low
         names = []
+        # (the summed contraction of the second-order pass holds the rows of two operand pairs)
+        xrows = (2 if self.t1 else 1) * 2 * (RT // WAVES) * self.max_d1
         cost = lambda ker: (sum(vp.U // 4 for g in ker for vp in g[1]) + sum(4 * self.vout[g[0]].d for g in ker)
-                            + 2 * (RT // WAVES) * self.max_d1 + 64)
+                            + xrows + 64)
         for ker in self._merge(_groups(self.vpaths, "vo", len(self.vout)), cost, self.tune["uvw_fregs"], self.vout):
             vo0, order0, _ = ker[0]
-            name = "forward" if not names else f"forward_o{vo0}_{order0[0].ub if order0 else 0}"
+            if not order0 and self.accumulate:
+                continue  # nothing to add to a piece no path writes
+            name = (self.prefix + "forward") if not names else f"{self.prefix}forward_o{vo0}_{order0[0].ub if order0 else 0}"
             names.append(name)
             s("// ======== out pieces " + ", ".join(f"{vo}: {self.vout[vo].mul} x l={self.vout[vo].l}" for vo, _, _ in ker))
-            self._kernel_open(s, name, self.FWD_SIG, self.tune["uvw_wf"])
+            self._kernel_open(s, name, self.sig_f, self.tune["uvw_wf"])
             if not order0:
                 self._zero_kernel(s, "L3_out", low.L3, self.vout[vo0])
                 continue
             maxd = max(self.vout[vo].d for vo, _, _ in ker)
             s(f"__shared__ T s_T[2][{maxd}][{self.tlanes}][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
+            if self.t1:
+                s(f"__shared__ T s_y2[{RT}][{low.L2}];")
             self._prologue(s)
             s(f"T xa[{RT // WAVES}][{self.max_d1}], xb[{RT // WAVES}][{self.max_d1}];")
+            if self.t1:
+                s(f"T aa[{RT // WAVES}][{self.max_d1}], ab[{RT // WAVES}][{self.max_d1}];")
             for vo, order, _ in ker:
                 s(f"const bool act{vo} = wave * 16 < {self.vout[vo].mul};  // this wave has output channels in the piece")
             order_all = [vp for _, order, _ in ker for vp in order]
@@ -551,7 +584,7 @@ class MfmaEmitter:
                 s.open(f"if (act{vo} && row < num_batch)")
                 s(f"T* zp = L3_out + row * {low.L3} + {bo.off} + (wave * 16 + l16) * {bo.d};")
                 for k in range(bo.d):
-                    s(f"zp[{k}] {'=' if first else '+='} acc{vo}[{k}][i];")
+                    s(f"zp[{k}] {'=' if first and not self.accumulate else '+='} acc{vo}[{k}][i];")
                 s.close()
                 s.close()
             s.close()
@@ -559,7 +592,10 @@ class MfmaEmitter:
         return names
 
     # ------------------------------------------------------------ backward
-    def emit_backward(self, s: Src) -> List[str]:
+    sig_f = FWD_SIG
+    sig_b = BWD_SIG
+
+    def emit_backward(self, s: Src, parts=("dx", "dw")) -> List[str]:
         """Kernels per piece of an input irrep (dX of the piece and the dY contributions of its sub-paths)
         and per piece of an output irrep (dW of the sub-paths feeding it), launched back to back. A tile is
         always handled by the same block and thread, so what successive kernels add to dY (and to dX, with
@@ -573,12 +609,15 @@ class MfmaEmitter:
         fixed = lambda ker: (sum(8 * self.vin[g[0]].d for g in ker) + 4 * low.L2
                              + 6 * max(self.vout[vp.vo].d for g in ker for vp in g[1]) + 48)
         cost = lambda ker: sum(vp.Wn // 4 for g in ker for vp in g[1]) + fixed(ker)
-        for ker in self._merge(_groups(self.vpaths, "vi", len(self.vin)), cost, self.tune["uvw_xregs"], self.vin):
+        dx_kernels = self._merge(_groups(self.vpaths, "vi", len(self.vin)), cost, self.tune["uvw_xregs"], self.vin)
+        for ker in (dx_kernels if "dx" in parts else []):
             vi0, paths0, _ = ker[0]
-            name = "backward" if not names else f"backward_x{vi0}_{paths0[0].wb if paths0 else 0}"
+            if not paths0 and self.accumulate:
+                continue  # nothing to add to a piece no path reads
+            name = (self.prefix + "backward") if not names else f"{self.prefix}backward_x{vi0}_{paths0[0].wb if paths0 else 0}"
             names.append(name)
             s("// ======== in1 pieces " + ", ".join(f"{vi}: {self.vin[vi].mul} x l={self.vin[vi].l}" for vi, _, _ in ker))
-            self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_wx"])
+            self._kernel_open(s, name, self.sig_b, self.tune["uvw_wx"])
             if not paths0:
                 self._zero_kernel(s, "L1_grad", low.L1, self.vin[vi0])
                 continue
@@ -646,7 +685,7 @@ class MfmaEmitter:
                 s.open("if (row < num_batch)")
                 s(f"T* dp = L1_grad + row * {low.L1} + {b1.off} + u{vi} * {b1.d};")
                 for c in range(b1.d):
-                    s(f"dp[{c}] {'=' if first else '+='} dx{vi}[i][{c}];")
+                    s(f"dp[{c}] {'=' if first and not self.accumulate else '+='} dx{vi}[i][{c}];")
                 s.close()
                 s.close()
                 s.close()
@@ -656,16 +695,20 @@ class MfmaEmitter:
             s.open(f"for (int t = tid; t < {RT * low.L2}; t += {64 * WAVES})")
             s(f"const int r = t / {low.L2}, c = t % {low.L2};")
             s("const T tot = ((s_dy[0][r][c] + s_dy[1][r][c]) + s_dy[2][r][c]) + s_dy[3][r][c];")
-            s(f"if (row0 + r < num_batch) L2_grad[(row0 + r) * {low.L2} + c] {'=' if first_dy else '+='} tot;")
+            s(f"if (row0 + r < num_batch) L2_grad[(row0 + r) * {low.L2} + c] "
+              f"{'=' if first_dy and not self.accumulate else '+='} tot;")
             s.close()
             s.close()
             s.close()
             first_dy = False
-        if first_dy:
+        if first_dy and "dx" in parts:
             raise AssertionError("no path")
+        if "dw" not in parts:
+            return names
 
         # ---------------- dW ----------------------------------------------------
-        regs = lambda ker: (sum(4 * (vp.Wn // 16) for g in ker for vp in g[1]) + 2 * (RT // WAVES) * self.max_d1
+        xrows = (2 if self.t1 else 1) * 2 * (RT // WAVES) * self.max_d1
+        regs = lambda ker: (sum(4 * (vp.Wn // 16) for g in ker for vp in g[1]) + xrows
                             + 4 * max(self.vout[g[0]].mul // 16 for g in ker) + 64)
 
         def dw_lds(ker, nbuf):
@@ -673,7 +716,7 @@ class MfmaEmitter:
             first, last = self.vout[ker[0][0]], self.vout[ker[-1][0]]
             ncols = last.off + last.mul * last.d - first.off
             maxd = max(self.vout[g[0]].d for g in ker)
-            return (RT * self._tile_stride(ncols) + nbuf * maxd * self.tlanes * TPAD + RT * low.L2) * low.elem_size
+            return (RT * self._tile_stride(ncols) + nbuf * maxd * self.tlanes * TPAD + 2 * RT * low.L2) * low.elem_size
 
         # a kernel that would not fit the 160 KB of LDS with its pieces merged stays split (the register estimate
         # is replaced by one beyond any limit)
@@ -688,10 +731,10 @@ class MfmaEmitter:
             col0 = pieces[0].off
             ncols = pieces[-1].off + pieces[-1].mul * pieces[-1].d - col0
             maxd = max(b.d for b in pieces)
-            name = f"backward_w{ker[0][0]}_{order_all[0].ub}"
+            name = f"{self.prefix}backward_w{ker[0][0]}_{order_all[0].ub}"
             names.append(name)
             s("// ======== dW of the sub-paths into out pieces " + ", ".join(str(vo) for vo, _, _ in ker))
-            self._kernel_open(s, name, self.BWD_SIG, self.tune["uvw_ww"])
+            self._kernel_open(s, name, self.sig_b, self.tune["uvw_ww"])
             # only these pieces' columns of the dZ tile are needed (and kept)
             # two copies of the T tile let a path's contraction be written while the previous path's is still
             # being multiplied; where they do not fit (fp64, l = 3 outputs) one copy and a barrier more per path
@@ -701,10 +744,14 @@ class MfmaEmitter:
             s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self._tile_stride(ncols)}];")
             s(f"__shared__ T s_T[{nbuf}][{maxd}][{self.tlanes}][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
+            if self.t1:
+                s(f"__shared__ T s_y2[{RT}][{low.L2}];")
             self._prologue(s)
             s("const int u = wave * 16 + l16;")
             s(f"T* prow = wpartial + (i64)blockIdx.x * {low.WN};")
             s(f"T xa[{RT // WAVES}][{self.max_d1}], xb[{RT // WAVES}][{self.max_d1}];")
+            if self.t1:
+                s(f"T aa[{RT // WAVES}][{self.max_d1}], ab[{RT // WAVES}][{self.max_d1}];")
             # dw<path>[n]: D tile rows = channels u of the wave's slice, columns = w in 16 n .. 16 n + 15
             for vp in order_all:
                 ntile = vp.Wn // 16
@@ -755,6 +802,57 @@ class MfmaEmitter:
         return names
 
 
+    # ------------------------------------------------------- second order
+    SIG_A = ("(i64 num_batch, const T* __restrict__ p_x, const T* __restrict__ p_a, const T* __restrict__ p_y, "
+             "const T* __restrict__ p_b, const T* __restrict__ p_w, const T* __restrict__ p_c, T* __restrict__ p_gg)")
+    SIG_B = ("(i64 num_batch, const T* __restrict__ p_x, const T* __restrict__ p_a, const T* __restrict__ p_y, "
+             "const T* __restrict__ p_b, const T* __restrict__ p_w, const T* __restrict__ p_c, "
+             "const T* __restrict__ p_g, T* __restrict__ p_dx, T* __restrict__ p_dy, T* __restrict__ p_dw, "
+             "T* __restrict__ wpartial)")
+
+    def second_order_kernels(self, s: Src):
+        """The kernels of ``double_backward_A`` / ``double_backward_B`` for the matrix-core path, as variants of the
+        first-order ones (reference: templates/loop_unroll_batch.cuh:148-317). With cotangents (a, b, c) of
+        (dX, dY, dW):
+
+        A  d/d(dZ) = [T(a, y) + T(x, b)] W + T(x, y) C: the forward kernels with the summed contraction, then the
+           plain forward kernels on (x, y, C) adding to the result - two channel mixes where composing first-order
+           calls runs three;
+        B  G = dZ W^T and H = dZ C^T: the dX kernels on (a, b, W), which give dX += c b G and dY += c a G, then on
+           (x, y, C) adding c y H and c x H; dW = [T(a, y) + T(x, b)]^T dZ by the dW kernels with the summed
+           contraction - two dX passes and one dW pass instead of three of each.
+
+        Returns (names of A, names of B) in launch order."""
+        ptr = lambda name, src, const=True: f"{'const ' if const else ''}T* __restrict__ {name} = {src}; (void){name};"
+        names_a, names_b = [], []
+
+        def variant(prefix, sig_f=None, sig_b=None, alias=(), accumulate=False, t1=False):
+            self.prefix, self.alias, self.accumulate, self.t1 = prefix, list(alias), accumulate, t1
+            self.sig_f, self.sig_b = sig_f or self.FWD_SIG, sig_b or self.BWD_SIG
+
+        try:
+            variant("dda1_", sig_f=self.SIG_A, t1=True,
+                    alias=[ptr("L1_in", "p_x"), ptr("L1_alt", "p_a"), ptr("L2_in", "p_y"), ptr("L2_alt", "p_b"),
+                           ptr("W", "p_w"), ptr("L3_out", "p_gg", False)])
+            names_a += self.emit_forward(s)
+            variant("dda2_", sig_f=self.SIG_A, accumulate=True,
+                    alias=[ptr("L1_in", "p_x"), ptr("L2_in", "p_y"), ptr("W", "p_c"), ptr("L3_out", "p_gg", False)])
+            names_a += self.emit_forward(s)
+            outs = [ptr("L1_grad", "p_dx", False), ptr("L2_grad", "p_dy", False), ptr("L3_grad", "p_g")]
+            variant("ddb1_", sig_b=self.SIG_B, alias=[ptr("L1_in", "p_a"), ptr("L2_in", "p_b"), ptr("W", "p_w")] + outs)
+            names_b += self.emit_backward(s, parts=("dx",))
+            variant("ddb2_", sig_b=self.SIG_B, accumulate=True,
+                    alias=[ptr("L1_in", "p_x"), ptr("L2_in", "p_y"), ptr("W", "p_c")] + outs)
+            names_b += self.emit_backward(s, parts=("dx",))
+            variant("ddb3_", sig_b=self.SIG_B, t1=True,
+                    alias=[ptr("L1_in", "p_x"), ptr("L1_alt", "p_a"), ptr("L2_in", "p_y"), ptr("L2_alt", "p_b"),
+                           ptr("L3_grad", "p_g")])
+            names_b += self.emit_backward(s, parts=("dw",))
+        finally:
+            variant("")
+        return names_a, names_b
+
+
 def tp_module(low: Lowered, compute_units: int = 256):
     from .. import runtime as rt
 
@@ -782,6 +880,10 @@ def tp_module(low: Lowered, compute_units: int = 256):
     max_blocks = compute_units * em.tune["uvw_blocks"]
     descs = [(rt.ROLE_TP_FORWARD, n, 64 * WAVES, RT, max_blocks) for n in fwd_names]
     descs += [(rt.ROLE_TP_BACKWARD, n, 64 * WAVES, RT, max_blocks) for n in bwd_names]
+    if em.tune["uvw_mfma_dd"]:
+        names_a, names_b = em.second_order_kernels(s)
+        descs += [(rt.ROLE_DOUBLE_BACKWARD_A, n, 64 * WAVES, RT, max_blocks) for n in names_a]
+        descs += [(rt.ROLE_DOUBLE_BACKWARD_B, n, 64 * WAVES, RT, max_blocks) for n in names_b]
     descs += [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, compute_units * 16),
         (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 64, 0),

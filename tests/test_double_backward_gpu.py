@@ -121,6 +121,25 @@ UVW = [
 UVW_CONV = [c for c in UVW if not c[0].endswith(("shared", "shared-f64"))]
 
 
+def _fc_shared(in1, in2, out):
+    return P.FullyConnectedTPProblem(in1, in2, out, shared_weights=True, internal_weights=False, label=f"fc-shared {in1}")
+
+
+# shared weights with multiplicities that are multiples of 16: the matrix-core kernels (second-order pair = variants
+# of the first-order kernels with the summed contraction, run on both weight tensors)
+MFMA = [
+    ("cfg4", P.config4_uvw_shared, 83),
+    ("cfg4-f64", lambda: P.config4_uvw_shared(np.float64), 37),
+    ("mfma-mixed", lambda: _fc_shared("64x0e+32x1o+16x2e", "1x0e+1x1o", "48x0e+80x1o+16x2e"), 50),
+    ("mfma-mixed-f64", lambda: _f64(_fc_shared("64x0e+32x1o+16x2e", "1x0e+1x1o", "48x0e+80x1o+16x2e")), 33),
+    ("mfma-128", lambda: _fc_shared("128x0e+128x1o", "1x0e+1x1o", "128x0e+128x1o"), 45),
+    ("mfma-gaps", lambda: oeq.TPProblem(
+        "32x0e+16x1o+32x2e", "1x0e+1x1o", "32x0e+16x1o+48x2e+16x1e",
+        [(0, 0, 0, "uvw", True), (1, 1, 0, "uvw", True), (0, 1, 1, "uvw", True), (2, 0, 2, "uvw", True, 0.7)],
+        shared_weights=True, internal_weights=False, label="mfma-gaps"), 50),
+]
+
+
 def _rand(rng, shape, dt):
     return torch.tensor(rng.uniform(-1, 1, size=shape).astype(dt), device="cuda")
 
@@ -131,7 +150,7 @@ def _check(names, fused, composed, tol):
         assert e <= tol, (name, e)
 
 
-@pytest.mark.parametrize("name,make,batch", CASES + SHARED + UVW, ids=[c[0] for c in CASES + SHARED + UVW])
+@pytest.mark.parametrize("name,make,batch", CASES + SHARED + UVW + MFMA, ids=[c[0] for c in CASES + SHARED + UVW + MFMA])
 def test_tp_fused_matches_composition(name, make, batch):
     problem = make()
     tp = oeq.TensorProduct(problem)
@@ -222,10 +241,10 @@ def test_conv_fused_isolated_nodes_and_empty():
             assert float(fused[0].abs().max()) == 0.0 and float(fused[3].abs().max()) == 0.0
 
 
-def test_edge_cases_and_refusals():
+def test_edge_cases_and_refusals(monkeypatch):
     """Empty batch: nothing launched, empty results (a shared weight gradient: zeros). Kernel sets without
-    second-order kernels ('uvw') refuse the fused entry point loudly; autograd then composes first-order kernels
-    instead."""
+    second-order kernels (built with them switched off) refuse the fused entry point loudly; autograd then composes
+    first-order kernels instead."""
     problem = P.config2_nequip_uvu()
     tp = oeq.TensorProduct(problem)
     e = ops.get_entry(tp.kid)
@@ -236,6 +255,8 @@ def test_edge_cases_and_refusals():
     empty[2] = empty[6] = torch.rand(e.WN, device="cuda")
     out = ops.tp_double_backward(*empty, tsh.kid)
     assert tuple(out[2].shape) == (e.WN,) and float(out[2].abs().max()) == 0.0
+    # every batch kernel set carries the pair by default; built without it, the entry point refuses
+    monkeypatch.setenv("OEQ_AMD_TUNE", "uvw_mfma_dd=0")
     tps = oeq.TensorProduct(P.config4_uvw_shared())
     es = ops.get_entry(tps.kid)
     assert not es.kernels().has_double_backward()
@@ -320,7 +341,9 @@ ORACLE_TP = [("cfg1", P.config1_single_uvu, 64), ("cfg2", P.config2_nequip_uvu, 
              ("uvw-diffdock", lambda: P.diffdock_problems()[0], 9), ("uvw-e3tools-conv", lambda: P.e3tools_problems()[0], 9),
              ("uvw-fc-shared", lambda: _fc(True), 33), ("uvw-tetris-1-shared", lambda: P.tetris_poly_problems()[0], 17),
              ("uvw-tetris-2-shared-f64", lambda: _f64(P.tetris_poly_problems()[1]), 9),
-             ("uvw-wide-shared", lambda: _wide_fc(True), 9)]
+             ("uvw-wide-shared", lambda: _wide_fc(True), 9),
+             ("mfma-cfg4", P.config4_uvw_shared, 19), ("mfma-cfg4-f64", lambda: P.config4_uvw_shared(np.float64), 17),
+             ("mfma-mixed", lambda: _fc_shared("64x0e+32x1o+16x2e", "1x0e+1x1o", "48x0e+80x1o+16x2e"), 21)]
 
 
 @pytest.mark.parametrize("name,make,batch", ORACLE_TP, ids=[c[0] for c in ORACLE_TP])

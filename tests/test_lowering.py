@@ -69,7 +69,7 @@ def test_which_sets_carry_fused_second_order_kernels():
     shared.shared_weights = True
     # shared weights: the batch kernels, not the convolution
     assert uvu_double.supported(L.lower(shared)) and not uvu_double.supported(L.lower(shared), conv=True)
-    assert not uvu_double.supported(L.lower(P.config4_uvw_shared()))
+    assert not uvu_double.supported(L.lower(P.config4_uvw_shared()))  # 'uvw' has its own second-order kernels
 
 
 @pytest.mark.parametrize("make,conv", [(lambda: P.nequix_problems()[1], False), (lambda: P.seven_net_problems()[0], True),
