@@ -173,7 +173,7 @@ def tp_config_table(dev, only=None):
             peak = 157.3 if es == 4 else 78.6  # dense MFMA TFLOP/s, fp32 / fp64
             row["fwd_mfma_frac"] = row["fwd_dense_tflops"] / peak
             row["bwd_mfma_frac"] = row["bwd_dense_tflops"] / peak
-        if name.startswith(("cfg2", "DiffDock")) and ops.get_entry(tp.kid).kernels().has_double_backward():
+        if name.startswith(("cfg2", "cfg4 uvw shared f32", "DiffDock")) and ops.get_entry(tp.kid).kernels().has_double_backward():
             # second-order pass (the backward of the backward): the fused kernel pair beside the composition of
             # three forward and three backward calls; bytes = every operand once per kernel
             a, b, c = torch.randn_like(x), torch.randn_like(y), torch.randn_like(w)

@@ -46,6 +46,10 @@ Operand layouts of the two 16x16x4 instructions used below (lane l of 64):
 A[m][k]: m = l % 16, k = l / 16;  B[k][n]: k = l / 16, n = l % 16;
 D[m][n]: n = l % 16, and for the i-th of 4 result registers m = 4 * (l / 16) + i in fp32,
 m = l / 16 + 4 * i in fp64.
+
+The second-order pair (``second_order_kernels``) reuses these kernels under other operand bindings: the
+forward and dW kernels with the contraction ``T(a, y) + T(x, b)`` of both operand pairs, the forward and dX
+kernels once per weight tensor (W, then the cotangent of dW, adding to the first result).
 """
 
 from __future__ import annotations
