@@ -139,7 +139,11 @@ int main(int argc, char** argv) {
         CHECK_HIP(hipMalloc(&tX, bytes(x)));
         CHECK_HIP(hipMalloc(&tY, bytes(y)));
         CHECK_HIP(hipMalloc(&tW, bytes(w)));
-        CHECK_OEQ(oeq_tp_double_backward(k, batch, dX, dY, dW, dG, gX, gY, gW, hX, hY, hW, hG, nullptr, 0, stream));
+        // shared weights: kernel B leaves partial weight gradients in a workspace for the ordered reduction
+        const size_t dd_bytes = oeq_tp_double_backward_workspace_bytes(k, batch);
+        void* dd_ws = nullptr;
+        if (dd_bytes) CHECK_HIP(hipMalloc(&dd_ws, dd_bytes));
+        CHECK_OEQ(oeq_tp_double_backward(k, batch, dX, dY, dW, dG, gX, gY, gW, hX, hY, hW, hG, dd_ws, dd_bytes, stream));
         CHECK_HIP(hipStreamSynchronize(stream));
         std::vector<float> gg(g.size()), ddx(x.size()), gg_ref(g.size(), 0.f), ddx_ref(x.size(), 0.f), t(g.size()),
             tx(x.size());
