@@ -18,8 +18,9 @@ passes over the weight-sized tensors for each group.
 
 Work decomposition is that of the first-order kernels (lane = channel, a wave or a group of chunk
 waves per row / per receiver node, register-resident accumulators over a node's edges, per-edge dX
-terms reduced by the sender-ordered second pass). Shared weights: the batch kernels only, with the weight
-gradient summed per wave in registers and across waves by the first-order pass's ordered reduction.
+terms reduced by the sender-ordered second pass). Shared weights: the weight gradient is summed per wave
+group in registers (over the rows, or the edges of the nodes, the group handles) and across groups by the
+first-order pass's ordered reduction.
 """
 
 from __future__ import annotations
@@ -40,8 +41,8 @@ CONV_MAX_PATHS = 96
 
 
 def supported(low: Lowered, conv: bool = False) -> bool:
-    """Batch kernels: every 'uvu' problem. Convolution: per-edge weights, up to CONV_MAX_PATHS paths."""
-    if low.mode != "uvu" or (conv and low.shared_weights):
+    """Batch kernels: every 'uvu' problem. Convolution: up to CONV_MAX_PATHS paths."""
+    if low.mode != "uvu":
         return False
     from .uvu import tuning
     return not conv or len(low.paths) <= tuning(dict(dd_maxp=CONV_MAX_PATHS))["dd_maxp"]
@@ -483,8 +484,8 @@ class DoubleEmitter(UvuEmitter):
         s(f"const T* arow = L1_dgrad + sender * {low.L1};")
         s(f"const T* yrow = L2_in + eid * {low.L2};")
         s(f"const T* brow = L2_dgrad + eid * {low.L2};")
-        s(f"const T* wrow = W + eid * {low.WN};")
-        s(f"const T* crow = W_dgrad + eid * {low.WN};")
+        s(f"const T* wrow = W{'' if low.shared_weights else f' + eid * {low.WN}'};")
+        s(f"const T* crow = W_dgrad{'' if low.shared_weights else f' + eid * {low.WN}'};")
 
     def emit_conv_double_a(self, s: Src, G: int, waves_per_eu: int = 0, xcd: int = 1, segw: int = 1):
         """Receiver-major walk: the node's accumulators stay in registers over its edges. With ``segw``
@@ -548,14 +549,20 @@ class DoubleEmitter(UvuEmitter):
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
-            "T* __restrict__ L3_dgrad, const i64* __restrict__ order)"
+            "T* __restrict__ L3_dgrad, const i64* __restrict__ order, T* __restrict__ wpartial)"
         )
         self._lane_prologue(s)
+        shared = low.shared_weights
+        assert not (shared and self.merged)
         if self.NCH > 1:
             s(f"__shared__ T s_dy[{G}][{self.NCH}][{self.l2_pad}];")
         if (self.tr_stores & 2 or (self.merged and self.tr_stores & 1)) and self.R == 1:
             dmax = max([low.in1[b].d for b in self.used_in1] + [low.out[io].d for io in self.used_out])
             s(f"__shared__ T s_tr[{self.NCH * G}][{64 * dmax}];")
+        if shared:
+            # summed over all edges of all nodes of the wave group; one partial row per group at the end
+            s(f"T dwacc[{self.n_wslots}];")
+            s(f"for (int t = 0; t < {self.n_wslots}; ++t) dwacc[t] = T(0);")
         resident = self.double_b_resident() or self.merged
         self._node_loop_open(s, G, xcd)
         s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
@@ -573,14 +580,15 @@ class DoubleEmitter(UvuEmitter):
             # of the dY reduction are reached uniformly
             s.open(f"for (i64 e = e0 + r; e < e1; e += {self.R})")
             self._edge_rows(s, "e")
-            s(f"T* dwrow = W_grad + eid * {low.WN};")
+            if not shared:
+                s(f"T* dwrow = W_grad + eid * {low.WN};")
             s("X_t x, xa, dx;")
             self._load_x(s, "xrow", self.used_in1)
             self._load_x(s, "arow", self.used_in1, "xa")
             self._zero_x(s, "dx")
             s(f"T dy[{self.l2_pad}];")
             s(f"for (int t = 0; t < {self.l2_pad}; ++t) dy[t] = T(0);")
-            deferred = self._dw_deferred(None)
+            deferred = not shared and self._dw_deferred(None)
             if deferred:
                 s(f"T dwkeep[{self.n_wslots}];")
             if resident:
@@ -617,6 +625,20 @@ class DoubleEmitter(UvuEmitter):
         if self.merged:
             self._zero_untouched_out(s, f"(L3_dgrad + node * {low.L3})", "r == 0")
         s.close()
+        if shared:
+            if self.R > 1:
+                s.open(f"for (int t = 0; t < {self.n_wslots}; ++t)")
+                m = self.LPR
+                while m < 64:
+                    s(f"dwacc[t] += __shfl_xor(dwacc[t], {m});")
+                    m *= 2
+                s.close()
+            s(f"T* prow = wpartial + ((i64)blockIdx.x * {G} + g) * {low.WN};")
+            for p, slot in self._dw_slots():
+                b1, V = low.in1[p.i1], low.in2[p.i2].mul
+                s.open(f"if (r == 0 && u < {b1.mul})")
+                s(f"for (int v = 0; v < {V}; ++v) prow[{p.woff} + u * {V} + v] = dwacc[{slot} + v];")
+                s.close()
         s.close()
         return block
 
@@ -685,7 +707,7 @@ class DoubleEmitter(UvuEmitter):
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
-            "T* __restrict__ L3_dgrad, const i64* __restrict__ order)"
+            "T* __restrict__ L3_dgrad, const i64* __restrict__ order, T* __restrict__ wpartial)"
         )
         self._lane_prologue(s, SW)
         s(f"__shared__ T s_dy[{SW * self.NCH}][{self.l2_pad}];")
@@ -809,8 +831,11 @@ def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, groups_b:
              compute_units * 8 if low.shared_weights else 0)]
 
 
-def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: int) -> List[tuple]:
-    """Append the convolution double-backward kernels (receiver-major walk) to a module."""
+def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: int, groups_b: int = 0,
+                     compute_units: int = 256) -> List[tuple]:
+    """Append the convolution double-backward kernels (receiver-major walk) to a module. Shared weights: kernel B
+    runs with the first-order backward kernel's wave groups per block (``groups_b``) on a bounded grid, one
+    partial weight-gradient row per group, and is never split between waves or merged with kernel A."""
     from .. import runtime as rt
 
     def kernel_a_need(e: DoubleEmitter) -> int:
@@ -852,8 +877,9 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     # dd_merge=1: one kernel for both results (W, C and the gathered X, A rows are then read once instead of
     # twice). Measured slower on MI355X for every shape tried (MACE shape 37 - 85 ms against 33 ms for the
     # pair): its accumulators on top of kernel B's state spill whatever the split, so it is off by default.
-    em.merged = bool(tune.get("dd_merge", 0))
-    groups = em.plan_double_groups(8 // em.NCH) if tune.get("dd_split", 1) else None
+    shared = low.shared_weights
+    em.merged = bool(tune.get("dd_merge", 0)) and not shared
+    groups = em.plan_double_groups(8 // em.NCH) if tune.get("dd_split", 1) and not shared else None
     if em.merged and not groups and not em.merged_fits_one_wave():
         em.merged = False
         groups = em.plan_double_groups(8 // em.NCH) if tune.get("dd_split", 1) else None
@@ -866,6 +892,10 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     if groups:
         blk_b = em.emit_conv_double_b_split(s, groups, tune.get("dd_wb", 2), xcd)
         G_b = 1
+    elif shared:
+        G_b = 1 if em.NCH > 1 else groups_b
+        blk_b = em.emit_conv_double_b(s, G_b, tune.get("dd_wb", 2), 1)
+        return descs + [(rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_b, G_b, compute_units * 8, 1)]
     else:
         blk_b = em.emit_conv_double_b(s, G, tune.get("dd_wb", 2), xcd)
         G_b = 1 if em.NCH > 1 else G

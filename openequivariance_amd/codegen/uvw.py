@@ -433,7 +433,8 @@ class UvwEmitter:
                 f'extern "C" __global__ __launch_bounds__({block}){attr} void {name}(i64 node_count, i64 nnz, '
                 + operands + "T* __restrict__ L2_grad, T* __restrict__ W_grad, const i64* __restrict__ rows, "
                 "const i64* __restrict__ cols, const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, "
-                "const i64* __restrict__ eperm, T* __restrict__ L3_dgrad, const i64* __restrict__ order)"
+                "const i64* __restrict__ eperm, T* __restrict__ L3_dgrad, const i64* __restrict__ order, "
+                "T* __restrict__ wpartial_unused)"
             )
             s("const i64 num_batch = nnz;")
         elif second:

@@ -515,9 +515,9 @@ static size_t ptr_bytes_of(int64_t node_count) {
 }
 static size_t perm_bytes_of(int64_t nnz) { return align_up((size_t)nnz * sizeof(int64_t), 256); }
 
-static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t node_count) {
-    if (!k->dims.shared_weights || !k->dims.wpartial_per_block) return 0;
-    size_t rows = (size_t)k->grid_for(OEQ_ROLE_CONV_BACKWARD, node_count) * (size_t)k->dims.wpartial_per_block;
+static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t node_count, int role = OEQ_ROLE_CONV_BACKWARD) {
+    if (!k->dims.shared_weights || !k->dims.wpartial_per_block || !k->roles[role].present) return 0;
+    size_t rows = (size_t)k->grid_for(role, node_count) * (size_t)k->dims.wpartial_per_block;
     return align_up(rows * (size_t)k->dims.weight_numel * (size_t)k->dims.elem_size, 256);
 }
 
@@ -564,14 +564,14 @@ struct ScratchLayout {
 };
 
 static ScratchLayout scratch_layout(const oeq_kernels* k, int64_t node_count, int64_t nnz, bool terms, bool arrivals,
-                                    bool wpartial) {
+                                    bool wpartial, int wpartial_role = OEQ_ROLE_CONV_BACKWARD) {
     ScratchLayout w;
     auto take = [&w](size_t bytes) { size_t at = w.total; w.total += bytes; return at; };
     if (arrivals)
         w.arrivals = take(align_up((size_t)node_count * (size_t)std::max(1, k->dims.n_chunks) * sizeof(int32_t), 256));
     if (terms) w.dx_tmp = take(align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256));
     if (wpartial)
-        if (size_t wp = conv_wpartial_bytes(k, node_count)) w.wpartial = take(wp);
+        if (size_t wp = conv_wpartial_bytes(k, node_count, wpartial_role)) w.wpartial = take(wp);
     return w;
 }
 
@@ -679,7 +679,7 @@ size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_coun
 // the second-order kernels always go through the per-edge terms and fixup_backward
 size_t oeq_conv_double_backward_scratch_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
     if (!k || !walk_mode(k)) return 0;
-    return scratch_layout(k, node_count, nnz, true, false, false).total;
+    return scratch_layout(k, node_count, nnz, true, false, true, OEQ_ROLE_DOUBLE_BACKWARD_B).total;
 }
 
 size_t oeq_conv_double_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
@@ -924,6 +924,11 @@ int oeq_conv_double_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t
     if (nnz == 0) {
         int rc = k->fill_zero(L1_grad, (size_t)node_count * k->dims.L1_dim * es, stream);
         if (rc) return rc;
+        if (k->dims.shared_weights) {  // a sum over no edges
+            if (!W_grad) return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: NULL W_grad");
+            rc = k->fill_zero(W_grad, (size_t)k->dims.weight_numel * es, stream);
+            if (rc) return rc;
+        }
         return k->fill_zero(L3_dgrad, (size_t)node_count * k->dims.L3_dim * es, stream);
     }
     if (!L1_in || !L2_in || !W || !L3_grad || !L1_dgrad || !L2_dgrad || !W_dgrad || !L2_grad || !W_grad || !rows ||
@@ -933,11 +938,13 @@ int oeq_conv_double_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t
     int rc = bind_index(k, "oeq_conv_double_backward", index_layout(k, node_count, nnz, true), index, index_bytes,
                         transpose_perm, &ix);
     if (rc) return rc;
-    const ScratchLayout w = scratch_layout(k, node_count, nnz, true, false, false);
+    const ScratchLayout w = scratch_layout(k, node_count, nnz, true, false, true, OEQ_ROLE_DOUBLE_BACKWARD_B);
     if (!scratch || scratch_bytes < w.total)
         return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: workspace too small (%zu < %zu bytes of scratch)",
                     scratch_bytes, w.total);
     void* dx_tmp = at_offset(scratch, w.dx_tmp);
+    // shared weights: kernel B leaves one partial weight-gradient row per wave group, summed in order at the end
+    void* wpartial = at_offset(scratch, w.wpartial);
     void* a[] = {&node_count, &nnz, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_dgrad,
                  &rows,       &cols, &ix.rowptr, &ix.rperm, &ix.order};
     if (k->roles[OEQ_ROLE_DOUBLE_BACKWARD_A].present) {
@@ -945,11 +952,17 @@ int oeq_conv_double_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t
         if (rc) return rc;
     }
     void* b[] = {&node_count, &nnz,     &L1_in,  &L1_dgrad, &L2_in, &L2_dgrad,  &W,         &W_dgrad, &L3_grad,
-                 &L2_grad,    &W_grad,  &rows,   &cols,     &ix.rowptr, &dx_tmp, &ix.rperm, &L3_dgrad, &ix.order};
+                 &L2_grad,    &W_grad,  &rows,   &cols,     &ix.rowptr, &dx_tmp, &ix.rperm, &L3_dgrad, &ix.order,
+                 &wpartial};
     rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count, b, stream);
     if (rc) return rc;
     void* fargs[] = {&node_count, &nnz, &dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};
-    return k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
+    rc = k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
+    if (rc || !wpartial) return rc;
+    int64_t n_partials = (int64_t)k->grid_for(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count) * k->dims.wpartial_per_block;
+    int64_t wn = k->dims.weight_numel;
+    void* rargs[] = {&n_partials, &wpartial, &W_grad, &wn};
+    return k->launch(OEQ_ROLE_TP_BACKWARD_WREDUCE, wn, rargs, stream);
 }
 
 int oeq_conv_double_backward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,

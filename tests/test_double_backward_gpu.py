@@ -207,6 +207,43 @@ def test_conv_fused_matches_composition(name, make, batch, det, monkeypatch):
     _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
 
 
+@pytest.mark.parametrize("name,make,batch", SHARED, ids=[c[0] for c in SHARED])
+def test_conv_shared_weights_fused_matches_composition_and_oracle(name, make, batch):
+    """Shared weights (device-grouped edge lists only): kernel B sums the weight gradient over all edges of a
+    wave group in registers and the groups' partial rows in a fixed order. Against the composition of first-order
+    ops and against float64 autograd through the CPU restatement."""
+    from oracle.torch_ref import TorchConv
+    problem = make()
+    gph = _graph(40)
+    n, E = gph.coords.shape[0], gph.nnz
+    conv = oeq.TensorProductConv(problem, deterministic=False)
+    e = ops.get_entry(conv.kid)
+    assert e.kernels().has_double_backward()
+    dt = np.dtype(problem.irrep_dtype)
+    rng = np.random.default_rng(26)
+    order = rng.permutation(E)
+    rows, cols = gph.rows[order], gph.cols[order]
+    tr, tc, tp = (torch.tensor(v, device="cuda") for v in (rows, cols, np.zeros(0, np.int64)))
+    x, a = (_rand(rng, (n, e.L1), dt) for _ in range(2))
+    y, b = (_rand(rng, (E, e.L2), dt) for _ in range(2))
+    w, c = (_rand(rng, (e.WN,), dt) for _ in range(2))
+    g = _rand(rng, (n, e.L3), dt)
+    fused = ops.conv_double_backward(x, y, w, g, a, b, c, tr, tc, tp, conv.kid)
+    composed = ops._second_order(lambda p, q, r: ops.conv_forward(p, q, r, tr, tc, tp, conv.kid),
+                                 lambda p, q, r, s: ops.conv_backward(p, q, r, s, tr, tc, tp, conv.kid),
+                                 x, y, w, g, a, b, c)
+    _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
+    oracle = TorchConv(R.Problem.from_spec(problem), torch.float64)
+    want = _oracle_second_order(lambda p, q, r: oracle(p, q, r, torch.tensor(rows), torch.tensor(cols)), x, y, w, g, a, b, c)
+    for nm, got, ref in zip(("dx", "dy", "dw", "gg"), fused, want):
+        err = R.normalized_error(got.cpu().numpy(), ref)
+        assert err <= tol_of(problem), (nm, err)
+    # no edges: the weight gradient is a sum over nothing
+    none = torch.zeros(0, dtype=torch.int64, device="cuda")
+    out = ops.conv_double_backward(x, y[:0], w, g, a, b[:0], c, none, none, none, conv.kid)
+    assert float(out[2].abs().max()) == 0.0 and float(out[0].abs().max()) == 0.0
+
+
 def test_conv_single_kernel_variant(monkeypatch):
     """The optional single-kernel form (both results from one walk; OEQ_AMD_TUNE=dd_merge=1)."""
     monkeypatch.setenv("OEQ_AMD_TUNE", "dd_merge=1")

@@ -67,8 +67,8 @@ def test_which_sets_carry_fused_second_order_kernels():
     assert len(seven.paths) <= uvu_double.CONV_MAX_PATHS < 200
     shared = P.config2_nequip_uvu().clone()
     shared.shared_weights = True
-    # shared weights: the batch kernels, not the convolution
-    assert uvu_double.supported(L.lower(shared)) and not uvu_double.supported(L.lower(shared), conv=True)
+    # shared weights: batch and (device-grouped) convolution
+    assert uvu_double.supported(L.lower(shared)) and uvu_double.supported(L.lower(shared), conv=True)
     assert not uvu_double.supported(L.lower(P.config4_uvw_shared()))  # 'uvw' has its own second-order kernels
 
 
