@@ -26,8 +26,9 @@ from .utils import compute_units, oeq_to_torch_dtype, torch_to_oeq_dtype
 
 
 def fused(low) -> bool:
-    """Whether the convolution of this problem runs as fused kernels: every 'uvu' problem, and 'uvw'
-    problems with per-edge weights (``OEQ_AMD_TUNE=conv_fuse_uvw=0`` sends those through the unfused path)."""
+    """Whether the convolution of this problem runs as fused kernels: every 'uvu' problem, and the 'uvw'
+    problems outside the matrix-core path for shared weights (``OEQ_AMD_TUNE=conv_fuse_uvw=0`` sends those
+    through the unfused path, too)."""
     if low.mode == "uvu":
         return True
     from ..codegen import uvw
@@ -44,7 +45,7 @@ def build_conv_module(problem: TPProblem, deterministic: bool, kahan: bool = Fal
     from ..codegen import uvw
     if fused(low):
         return uvw.conv_module(low, deterministic, compute_units(), kahan)
-    # 'uvw' with shared weights: no fused kernel; the batch kernels run on gathered rows and an ordered
+    # 'uvw' with shared weights on the matrix cores: no fused kernel; the batch kernels run on gathered rows and an ordered
     # segment sum scatters the result, like the reference's unfused convolution
     # (core/ConvolutionBase.py:292-301, _torch/TensorProductConv.py:595-640).
     cu = compute_units()

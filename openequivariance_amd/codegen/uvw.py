@@ -251,7 +251,6 @@ class UvwEmitter:
         added with a compensation term. ``second``: the kernel double_backward_A of the convolution (the three
         forward terms of the second-order pass, same walk). Returns (block size, nodes per block)."""
         low = self.low
-        assert not low.shared_weights
         segs = [(io, wc) for io, bo in enumerate(low.out) for wc in range(0, bo.mul, 64)
                 if any(p.io == io for p in low.paths)]
         empty = [io for io in range(len(low.out)) if not any(p.io == io for p in low.paths)]
@@ -309,11 +308,11 @@ class UvwEmitter:
             s("const i64 sender = oeq_idx(cols[e], node_count);")
             s(f"const T* xrow = L1_in + sender * {low.L1};")
             s(f"const T* yrow = L2_in + e * {low.L2};")
-            s(f"const T* wrow = W + e * {low.WN};")
+            s(f"const T* wrow = W{'' if low.shared_weights else f' + e * {low.WN}'};")
             if second:
                 s(f"const T* arow = L1_dgrad + sender * {low.L1};")
                 s(f"const T* brow = L2_dgrad + e * {low.L2};")
-                s(f"const T* crow = W_dgrad + e * {low.WN};")
+                s(f"const T* crow = W_dgrad{'' if low.shared_weights else f' + e * {low.WN}'};")
             if kahan:
                 s(f"T msg[{bo.d}];")
                 for k in range(bo.d):
@@ -363,8 +362,8 @@ class UvwEmitter:
     def emit_backward(self, s: Src, conv: bool = False, second: bool = False, force_waves: int = 0):
         """``conv``: the fused convolution's backward. An edge is a row: X comes from the sender's row,
         the output gradient from the receiver's, the X gradient goes to the edge's row of ``dx_tmp``
-        (summed per sender, in the order of the sender-major list, by ``fixup_backward``); per-row
-        weights only. The edges need no order here, so the kernel strides over the edge list as it is.
+        (summed per sender, in the order of the sender-major list, by ``fixup_backward``). The edges need no
+        order here, so the kernel strides over the edge list as it is.
 
         ``second``: the kernel double_backward_B. With cotangents (a, b, c) of the first-order (dX, dY, dW) and
         G = W g, H = C g (two channel mixes where the composition of first-order kernels runs three):
@@ -374,7 +373,6 @@ class UvwEmitter:
         weights: the partial weight-gradient rows are counted per block of the first-order kernel)."""
         low = self.low
         shared = low.shared_weights
-        assert not (conv and shared)
         self.second = second
         plans = {p.index: self._tile_plan(p) for p in low.paths}
         tiled = [p for p in low.paths if plans[p.index]]
@@ -434,7 +432,7 @@ class UvwEmitter:
                 + operands + "T* __restrict__ L2_grad, T* __restrict__ W_grad, const i64* __restrict__ rows, "
                 "const i64* __restrict__ cols, const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, "
                 "const i64* __restrict__ eperm, T* __restrict__ L3_dgrad, const i64* __restrict__ order, "
-                "T* __restrict__ wpartial_unused)"
+                "T* __restrict__ wpartial)"
             )
             s("const i64 num_batch = nnz;")
         elif second:
@@ -964,8 +962,14 @@ class UvwEmitter:
 
 
 def conv_supported(low: Lowered) -> bool:
-    """Problems the fused 'uvw' convolution kernels cover: per-row (per-edge) weights."""
-    return low.mode == "uvw" and not low.shared_weights
+    """Problems the fused 'uvw' convolution kernels cover: per-edge weights, and shared weights whose channel mix
+    does not run on the matrix cores (those stay with the unfused path: gathered rows through the MFMA kernels)."""
+    if low.mode != "uvw":
+        return False
+    if not low.shared_weights:
+        return True
+    from . import uvw_mfma
+    return not uvw_mfma.supported(low)
 
 
 def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kahan: bool = False):
@@ -979,6 +983,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     from .common import fixup_backward_kernel
 
     assert conv_supported(low)
+    shared = low.shared_weights
     em = UvwEmitter(low)
     s = Src()
     s(prelude(low.ctype))
@@ -988,19 +993,23 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     blk_b = em.emit_backward(s, conv=True)
     s(fixup_backward_kernel(low.L1, kahan, True))
     cu = compute_units
+    # shared weights: every wave of the backward grid writes one partial weight-gradient row (summed in order
+    # by oeq_wreduce), so that grid is bounded
+    max_b = cu * (3 if em.shared_lds else 2) if shared else cu * 16
     second = []
     if em.tune["uvw_dd"] and not kahan:
         # second-order pair: the same receiver walk / per-edge pass with the operands of both orders
         blk_da, G_da = em.emit_conv_forward(s, False, second=True)
-        blk_db = em.emit_backward(s, conv=True, second=True)
+        blk_db = em.emit_backward(s, conv=True, second=True, force_waves=em.backward_waves if shared else 0)
         second = [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_A", blk_da, G_da, cu * 32),
-                  (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_db, 1, cu * 16)]
+                  (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_db, 1, max_b)]
     descs = second + [
         (rt.ROLE_FILL_ZERO, "oeq_fill_zero", 256, 256 * 16, cu * 16),
         (rt.ROLE_SEGMENT_PTR, "oeq_segment_ptr", 256, 256, cu * 16),
         (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f, cu * 32),
         # strides over the edges: the grid need not follow the node count it is derived from
-        (rt.ROLE_CONV_BACKWARD, "backward", blk_b, 1, cu * 16),
+        (rt.ROLE_CONV_BACKWARD, "backward", blk_b, 1, max_b),
+        (rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 64, 0),
         (rt.ROLE_CONV_FIXUP_BACKWARD, "fixup_backward", 256, 1, 0),
         (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, cu * 16),
         (rt.ROLE_GROUP_SCAN, "oeq_group_scan", 1024, 1, 1),
@@ -1010,8 +1019,9 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     ]
     t = em.tune
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
-                shared_weights=0, deterministic=rt.CONV_SORTED if deterministic else rt.CONV_GROUPED,
-                wpartial_per_block=0, dx_mode=rt.DX_TERMS, n_chunks=1, order_hops=max(0, t["conv_hops"]))
+                shared_weights=int(shared), deterministic=rt.CONV_SORTED if deterministic else rt.CONV_GROUPED,
+                wpartial_per_block=em.backward_waves if shared else 0, dx_mode=rt.DX_TERMS, n_chunks=1,
+                order_hops=max(0, t["conv_hops"]))
     return s.text(), dims, descs
 
 

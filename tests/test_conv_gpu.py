@@ -64,13 +64,21 @@ CASES = [
     ("mace-large", lambda: P.mace_problems()[0], 40, 6),
     ("odd", lambda: _odd(False), 40, 6),
     ("odd-shared", lambda: _odd(True), 40, 6),
-    # 'uvw' problems with per-edge weights: fused kernels (receiver walk forward, per-edge backward + ordered
-    # sender-side sum); with shared weights: batch kernels on gathered rows + ordered segment sum
+    # 'uvw' problems: fused kernels (receiver walk forward, per-edge backward + ordered sender-side sum; shared
+    # weights: partial weight-gradient rows per wave, summed in order); shared weights on the matrix cores: batch
+    # kernels on gathered rows + ordered segment sum
     ("uvw", lambda: _fc(False), 40, 6),
     ("uvw-diffdock", lambda: P.diffdock_problems()[0], 40, 6),
     ("uvw-diffdock-f64", lambda: _as_f64(P.diffdock_problems()[1]), 30, 5),
     ("uvw-e3tools-conv", lambda: P.e3tools_problems()[0], 40, 6),
     ("uvw-shared", lambda: _fc(True), 40, 6),
+    ("uvw-shared-lds", lambda: P.FullyConnectedTPProblem(
+        "40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e", shared_weights=True, internal_weights=False,
+        label="uvw-shared-lds"), 40, 6),
+    ("uvw-shared-global-f64", lambda: _as_f64(P.FullyConnectedTPProblem(
+        "100x0e+70x1o", "1x0e+1x1o", "33x0e+20x1o", shared_weights=True, internal_weights=False,
+        label="uvw-shared-global")), 30, 5),
+    ("uvw-shared-tetris", lambda: P.tetris_poly_problems()[0], 40, 6),
     ("uvw-cfg4-mfma", P.config4_uvw_shared, 30, 5),
     # output gradient too large for one wave: forward shares the output segments, backward the output
     # blocks, between several waves of a node (64 channels: one chunk; 128: two)
@@ -151,6 +159,42 @@ def test_uvw_fused_matches_unfused(monkeypatch):
     # the grouped mode orders a node's edges by edge id, which is the order of the sorted list here
     for a, b in zip(out[(1, True)], out[(1, False)]):
         assert torch.equal(a, b)
+
+
+def test_uvw_shared_weights_fused_matches_unfused(monkeypatch):
+    """Shared weights outside the matrix-core path: the fused kernels against the unfused composition, same
+    bits on every run (the partial weight-gradient rows are summed in a fixed order), at a graph large enough
+    for every wave of the bounded backward grid to see edges and at one where most waves see none."""
+    from openequivariance_amd._torch import ops
+    problem = P.FullyConnectedTPProblem("40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e", shared_weights=True,
+                                        internal_weights=False, label="uvw-shared-lds")
+    for n_nodes, deg in ((3000, 12), (20, 3)):
+        coords, rows, cols = _graph(n_nodes, deg, seed=4)
+        E = len(rows)
+        gen = torch.Generator(device="cuda").manual_seed(3)
+        X = torch.randn(n_nodes, problem.irreps_in1.dim, device="cuda", generator=gen)
+        Y = torch.randn(E, problem.irreps_in2.dim, device="cuda", generator=gen)
+        W = torch.randn(problem.weight_numel, device="cuda", generator=gen)
+        G = torch.randn(n_nodes, problem.irreps_out.dim, device="cuda", generator=gen)
+        order = np.random.default_rng(n_nodes).permutation(E)
+        tr, tc = (torch.tensor(a[order], device="cuda") for a in (rows, cols))
+        none = torch.zeros(0, dtype=torch.int64, device="cuda")
+        out = {}
+        for fuse in (1, 0):
+            monkeypatch.setenv("OEQ_AMD_TUNE", f"conv_fuse_uvw={fuse}")
+            conv = oeq.TensorProductConv(problem, deterministic=False)
+            e = ops.get_entry(conv.kid)
+            assert e.unfused == (fuse == 0)
+            runs = []
+            for _ in range(3):
+                z = ops.conv_forward(X, Y, W, tr, tc, none, conv.kid)
+                runs.append((z,) + tuple(ops.conv_backward(X, Y, W, G, tr, tc, none, conv.kid)))
+            for later in runs[1:]:
+                for a, b in zip(runs[0], later):
+                    assert torch.equal(a, b), fuse
+            out[fuse] = runs[0]
+        for a, b in zip(out[1], out[0]):
+            assert (a - b).abs().max() <= 4e-6 * b.abs().max(), n_nodes
 
 
 def test_reference_toy_graph():

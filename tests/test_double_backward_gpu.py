@@ -119,6 +119,12 @@ UVW = [
     ("uvw-wide-shared", lambda: _wide_fc(True), 600),
 ]
 UVW_CONV = [c for c in UVW if not c[0].endswith(("shared", "shared-f64"))]
+# shared weights in the fused convolution: the three ways of summing the weight gradient (registers, LDS copy per
+# wave, partial rows in global memory when the weight tensor exceeds 64 KB)
+UVW_CONV_SHARED = [c for c in UVW if c[0].endswith(("shared", "shared-f64"))] + [
+    ("uvw-big-shared-f64", lambda: _f64(P.FullyConnectedTPProblem(
+        "100x0e+70x1o", "1x0e+1x1o", "33x0e+20x1o", shared_weights=True, internal_weights=False,
+        label="big-fc-uvw")), 0)]
 
 
 def _fc_shared(in1, in2, out):
@@ -207,11 +213,11 @@ def test_conv_fused_matches_composition(name, make, batch, det, monkeypatch):
     _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
 
 
-@pytest.mark.parametrize("name,make,batch", SHARED, ids=[c[0] for c in SHARED])
+@pytest.mark.parametrize("name,make,batch", SHARED + UVW_CONV_SHARED, ids=[c[0] for c in SHARED + UVW_CONV_SHARED])
 def test_conv_shared_weights_fused_matches_composition_and_oracle(name, make, batch):
     """Shared weights (device-grouped edge lists only): kernel B sums the weight gradient over all edges of a
-    wave group in registers and the groups' partial rows in a fixed order. Against the composition of first-order
-    ops and against float64 autograd through the CPU restatement."""
+    wave (group) and the partial rows in a fixed order. Against the composition of first-order ops and against
+    float64 autograd through the CPU restatement."""
     from oracle.torch_ref import TorchConv
     problem = make()
     gph = _graph(40)
