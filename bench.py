@@ -144,8 +144,12 @@ def tp_config_table(dev, only=None):
              ("cfg4 uvw shared f32 (MFMA)", P.config4_uvw_shared(), 262144),
              ("cfg4 uvw shared f64 (MFMA)", P.config4_uvw_shared(np.float64), 131072),
              ("DiffDock L=1 uvw per-row weights f32", P.diffdock_problems()[0], 100000)]
+    # multiplicities that are no multiples of 16 (48 and 10 channels) with shared weights: matrix cores, padded tiles
+    padded = P.diffdock_problems()[0].clone()
+    padded.shared_weights = True
+    cases.append(("DiffDock L=1 uvw shared f32 (MFMA, padded tiles)", padded, 262144))
     if only is not None:
-        cases = [cases[["1", "2", "3", "3d", "4", "4d", "dd"].index(only)]]
+        cases = [cases[["1", "2", "3", "3d", "4", "4d", "dd", "pad"].index(only)]]
     table = []
     for name, prob, B in cases:
         low = lower(prob)

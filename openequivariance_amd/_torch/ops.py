@@ -206,8 +206,7 @@ def _use_fused(kid, ddx, ddy, ddw) -> bool:
         return False
     if sum(t is not None for t in (ddx, ddy, ddw)) < 2:
         return False
-    e = get_entry(kid)
-    return not e.unfused and e.kernels().has_double_backward()
+    return get_entry(kid).kernels().has_double_backward()
 
 
 def _zeros_if_none(t, like):
@@ -428,6 +427,20 @@ def _unfused_backward(e, ks, x, y, w, g, r, c, p, nodes, nnz):
     return _scatter_rows(e, ks, dxe, nodes, c, p if e.deterministic else None), dy, dw
 
 
+def _unfused_double_backward(e, ks, x, y, w, g, a, b, c, r, cc, p, nodes, nnz):
+    """Second-order pass of the unfused convolution: the batch kernel pair on gathered rows, the per-edge
+    sender gradients and second cotangents summed into node rows in the order of the first-order passes."""
+    xe, ae, ge = x.index_select(0, cc), a.index_select(0, cc), g.index_select(0, r)
+    dxe, dy, dw, gge = torch.empty_like(xe), torch.empty_like(y), torch.empty_like(w), torch.empty_like(ge)
+    nb = ks.tp_double_backward_workspace_bytes(nnz)
+    ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
+    ks.tp_double_backward(nnz, xe.data_ptr(), y.data_ptr(), w.data_ptr(), ge.data_ptr(), ae.data_ptr(), b.data_ptr(),
+                          c.data_ptr(), dxe.data_ptr(), dy.data_ptr(), dw.data_ptr(), gge.data_ptr(), ws.data_ptr(), nb,
+                          _stream())
+    return (_scatter_rows(e, ks, dxe, nodes, cc, p if e.deterministic else None), dy, dw,
+            _scatter_rows(e, ks, gge, nodes, r, None))
+
+
 @torch.library.custom_op("oeq_amd::conv_forward", mutates_args=(), device_types="cuda")
 def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows: torch.Tensor,
                  cols: torch.Tensor, transpose_perm: torch.Tensor, kid: int) -> torch.Tensor:
@@ -527,6 +540,9 @@ def conv_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tens
     x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
     a, b, c = L1_dgrad.contiguous(), L2_dgrad.contiguous(), W_dgrad.contiguous()
     r, cc, p = rows.contiguous(), cols.contiguous(), transpose_perm.contiguous()
+    if e.unfused:
+        with torch.cuda.device(x.device):
+            return _unfused_double_backward(e, e.kernels(), x, y, w, g, a, b, c, r, cc, p, nodes, nnz)
     dx, dy, dw, gg = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w), torch.empty_like(g)
     with torch.cuda.device(x.device):
         ks = e.kernels()

@@ -10,7 +10,8 @@ reference does this mix with a scalar-FMA warp matmul on 32-wide chunks
 loop_unroll_tp.cuh:55-84, 217-272).
 
 Work decomposition: irrep blocks are cut into pieces of at most 64 channels
-(multiplicities are multiples of 16), a path into one sub-path per pair of
+(a piece whose channel count is no multiple of 16 is padded to one with zero
+weights: its missing channels are never loaded or stored), a path into one sub-path per pair of
 pieces with its own 64 x 64 (or smaller) corner of the path's weight matrix. A
 block of 4 waves owns a tile of 16 batch rows at a time; wave ``w`` owns output
 channels (forward) or input channels (backward) ``16w .. 16w+15`` of a piece
@@ -65,6 +66,16 @@ WAVES = 4        # waves per block
 TPAD = RT + 1    # padded row stride of the T tile in LDS (bank spread)
 LDS_BUDGET = 160 * 1024 - 2048   # bytes of LDS a kernel may declare (the CU has 160 KB)
 MFMA = "oeq_mfma"  # v_mfma_f32_16x16x4_f32 or v_mfma_f64_16x16x4_f64, see tp_module
+
+
+def c4(n: int) -> int:
+    """k-steps of 4 that cover n channels."""
+    return (n + 3) // 4
+
+
+def c16(n: int) -> int:
+    """16-channel tiles that cover n channels."""
+    return (n + 15) // 16
 
 
 def piece_of(low: Lowered) -> int:
@@ -155,15 +166,24 @@ def supported(low: Lowered) -> bool:
     if (RT * (low.L3 + 36) + (1 + WAVES) * RT * low.L2) * low.elem_size > LDS_BUDGET:
         return False
     for p in low.paths:
-        a, b, o = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
-        if b.mul != 1 or a.mul % 16 or o.mul % 16:
+        if low.in2[p.i2].mul != 1:
             return False
+    vin, vout, vpaths = _split(low)
+    # Multiplicities that are no multiples of 16 run on tiles padded with zero weights. Where nearly all of a
+    # tile would be padding the general kernels are the better choice: ``uvw_mfma_fill`` = least share (percent)
+    # of the multiplies that must be real ones. Measured at 262 144 rows, backward, padded tiles against general
+    # kernels: share 0.80 (48 and 10 channels) 0.54 / 6.8 ms, 0.39 (10 -> 17, 9, 33 channels) 1.4 / 5.3 ms, 0.25
+    # (8 channels) 0.17 / 0.23 ms, 0.06 (tetris polynomial, 1 - 6 channels) 2.5 / 2.0 ms.
+    from .uvu import tuning
+    real = sum(vp.U * vp.Wn for vp in vpaths)
+    padded = sum(16 * c16(vp.U) * 16 * c16(vp.Wn) for vp in vpaths)
+    if 100 * real < tuning(dict(uvw_mfma_fill=30))["uvw_mfma_fill"] * padded:
+        return False
     # register budget of the widest kernel of each pass: 16-channel k-steps of resident weight slices
     # (forward, dX: a few slices may move to LDS there) and 16 x 16 dW tiles
-    vin, vout, vpaths = _split(low)
-    fwd = max((sum(vp.U // 4 for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
-    dxk = max((sum(vp.Wn // 4 for vp in g) for _, g, _ in _groups(vpaths, "vi", len(vin))), default=0)
-    dwk = max((sum(4 * (vp.Wn // 16) for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
+    fwd = max((sum(c4(vp.U) for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
+    dxk = max((sum(4 * c16(vp.Wn) for vp in g) for _, g, _ in _groups(vpaths, "vi", len(vin))), default=0)
+    dwk = max((sum(4 * c16(vp.Wn) for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
     # (register counts in elements: fp64 runs one wave per SIMD with twice the registers)
     return fwd <= 80 and dxk <= 112 and dwk <= 80
 
@@ -347,7 +367,9 @@ class MfmaEmitter:
         if self.tlanes < 64:
             s.open(f"if (lane < {self.tlanes})")
         for k in range(d3):
-            s(f"s_T[{buf}][{k}][lane][r] = t[{k}];")
+            # (rows of channels beyond the piece are multiplied, with zero weights: they hold zeros, not copies)
+            val = f"t[{k}]" if vp.U % 16 == 0 else f"(lane < {vp.U} ? t[{k}] : T(0))"
+            s(f"s_T[{buf}][{k}][lane][r] = {val};")
         if self.tlanes < 64:
             s.close()
         s.close()
@@ -381,9 +403,10 @@ class MfmaEmitter:
                 for k in range(bo.d):
                     s(f"G[{k}] = v4t{{}};")
                 s("#pragma unroll")
-                s.open(f"for (int st = 0; st < {vp.Wn // 4}; ++st)")
+                s.open(f"for (int st = 0; st < {c4(vp.Wn)}; ++st)")
+                wcol = "(4 * st + lq)" if vp.Wn % 4 == 0 else f"min(4 * st + lq, {vp.Wn - 1})"
                 for k in range(bo.d):
-                    s(f"G[{k}] = {MFMA}({self.g_at('l16', f'{bo.off} + (4 * st + lq) * {bo.d} + {k}')}, "
+                    s(f"G[{k}] = {MFMA}({self.g_at('l16', f'{bo.off} + {wcol} * {bo.d} + {k}')}, "
                       f"wreg{vp.index}[st], G[{k}], 0, 0, 0);")
                 s.close()
                 cg_rows(vp, "G")
@@ -394,14 +417,18 @@ class MfmaEmitter:
         if self.lds_w:
             s(f"T wla[{CH}], wlb[{CH}];  // B operands of a path whose weight slice is kept in LDS")
         s(f"v4t G[{maxd}];")
-        segs = [(n, c) for n, vp in enumerate(paths) for c in range(vp.Wn // (4 * CH))]
+        segs = [(n, c) for n, vp in enumerate(paths) for c in range(c16(vp.Wn))]
 
         def reads(seg, buf):
             n, c = seg
             bo = self.vout[paths[n].vo]
             for q in range(CH):
+                w0 = 4 * (c * CH + q)
+                # (columns past the piece meet zero weights; they are read from its last column, which holds
+                # finite values, not from whatever lies behind the row)
+                wcol = f"({w0} + lq)" if w0 + 4 <= paths[n].Wn else f"min({w0} + lq, {paths[n].Wn - 1})"
                 for k in range(bo.d):
-                    s(f"{buf}[{q * bo.d + k}] = {self.g_at('l16', f'{bo.off} + ({4 * (c * CH + q)} + lq) * {bo.d} + {k}')};")
+                    s(f"{buf}[{q * bo.d + k}] = {self.g_at('l16', f'{bo.off} + {wcol} * {bo.d} + {k}')};")
             if paths[n].index in self.lds_w:
                 slot = self.lds_w.index(paths[n].index)
                 for q in range(CH):
@@ -424,7 +451,7 @@ class MfmaEmitter:
                 for k in range(bo.d):
                     s(f"G[{k}] = {MFMA}({cur}[{q * bo.d + k}], {wop}, G[{k}], 0, 0, 0);")
             s("__builtin_amdgcn_sched_barrier(0);")
-            if c == vp.Wn // (4 * CH) - 1:
+            if c == c16(vp.Wn) - 1:
                 cg_rows(vp, "G")
 
     def _reduce_dy(self, s: Src):
@@ -462,14 +489,19 @@ class MfmaEmitter:
         B[k = w = 4 st + lq][n = l16] = W[u][w] (Wn / 4 registers). Waves without channels in the piece load
         nothing (``act`` is in scope)."""
         for vp in vps:
-            n = (vp.Wn if transposed else vp.U) // 4
+            # (k-steps and channels beyond the corner of the weight matrix: zeros)
+            n = 4 * c16(vp.Wn) if transposed else c4(vp.U)
             s(f"T wreg{vp.index}[{n}];")
             s("#pragma unroll")
             if transposed:
-                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = {act} ? "
+                cond = act if vp.Wn % 16 == 0 else f"({act} && 4 * st + lq < {vp.Wn})"
+                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = {cond} ? "
                   f"W[{vp.woff} + {u} * {vp.ld} + 4 * st + lq] : T(0);")
             else:
-                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = {act} ? "
+                more = ("" if vp.U % 4 == 0 else f" && 4 * st + lq < {vp.U}") + \
+                    ("" if vp.Wn % 16 == 0 else f" && wave * 16 + l16 < {vp.Wn}")
+                cond = f"({act}{more})" if more else act
+                s(f"for (int st = 0; st < {n}; ++st) wreg{vp.index}[st] = {cond} ? "
                   f"W[{vp.woff} + (4 * st + lq) * {vp.ld} + wave * 16 + l16] : T(0);")
 
     FWD_SIG = ("(i64 num_batch, const T* __restrict__ L1_in, const T* __restrict__ L2_in, "
@@ -523,7 +555,7 @@ class MfmaEmitter:
         names = []
         # (the summed contraction of the second-order pass holds the rows of two operand pairs)
         xrows = (2 if self.t1 else 1) * 2 * (RT // WAVES) * self.max_d1
-        cost = lambda ker: (sum(vp.U // 4 for g in ker for vp in g[1]) + sum(4 * self.vout[g[0]].d for g in ker)
+        cost = lambda ker: (sum(c4(vp.U) for g in ker for vp in g[1]) + sum(4 * self.vout[g[0]].d for g in ker)
                             + xrows + 64)
         for ker in self._merge(_groups(self.vpaths, "vo", len(self.vout)), cost, self.tune["uvw_fregs"], self.vout):
             vo0, order0, _ = ker[0]
@@ -572,7 +604,7 @@ class MfmaEmitter:
                 s("__syncthreads();")
                 s.open(f"if (act{vp.vo})")
                 s("#pragma unroll")
-                s.open(f"for (int st = 0; st < {vp.U // 4}; ++st)")
+                s.open(f"for (int st = 0; st < {c4(vp.U)}; ++st)")
                 for k in range(bo.d):
                     s(f"acc{vp.vo}[{k}] = {MFMA}(s_T[{buf}][{k}][4 * st + lq][l16], wreg{vp.index}[st], "
                       f"acc{vp.vo}[{k}], 0, 0, 0);")
@@ -585,7 +617,8 @@ class MfmaEmitter:
                 s("#pragma unroll")
                 s.open("for (int i = 0; i < 4; ++i)")
                 s(f"const i64 row = row0 + {self.row('i')};")
-                s.open(f"if (act{vo} && row < num_batch)")
+                wok = "" if bo.mul % 16 == 0 else f" && wave * 16 + l16 < {bo.mul}"
+                s.open(f"if (act{vo} && row < num_batch{wok})")
                 s(f"T* zp = L3_out + row * {low.L3} + {bo.off} + (wave * 16 + l16) * {bo.d};")
                 for k in range(bo.d):
                     s(f"zp[{k}] {'=' if first and not self.accumulate else '+='} acc{vo}[{k}][i];")
@@ -612,7 +645,7 @@ class MfmaEmitter:
         # and the operand chunks
         fixed = lambda ker: (sum(8 * self.vin[g[0]].d for g in ker) + 4 * low.L2
                              + 6 * max(self.vout[vp.vo].d for g in ker for vp in g[1]) + 48)
-        cost = lambda ker: sum(vp.Wn // 4 for g in ker for vp in g[1]) + fixed(ker)
+        cost = lambda ker: sum(4 * c16(vp.Wn) for g in ker for vp in g[1]) + fixed(ker)
         dx_kernels = self._merge(_groups(self.vpaths, "vi", len(self.vin)), cost, self.tune["uvw_xregs"], self.vin)
         for ker in (dx_kernels if "dx" in parts else []):
             vi0, paths0, _ = ker[0]
@@ -626,6 +659,7 @@ class MfmaEmitter:
                 self._zero_kernel(s, "L1_grad", low.L1, self.vin[vi0])
                 continue
             paths_all = [vp for _, ps, _ in ker for vp in ps]
+            uok = lambda vi: f"act{vi}" if self.vin[vi].mul % 16 == 0 else f"uok{vi}"
             self.g_at = lambda row, col: f"s_g[{row}][{col}]"
             s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self.gstride}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
@@ -633,14 +667,19 @@ class MfmaEmitter:
             self._prologue(s)
             for vi, _, _ in ker:
                 s(f"const bool act{vi} = wave * 16 < {self.vin[vi].mul};  // this wave has input channels in the piece")
-                s(f"const int u{vi} = act{vi} ? wave * 16 + l16 : 0;  // channel of this lane in the MFMA result layout")
+                if self.vin[vi].mul % 16 == 0:
+                    s(f"const int u{vi} = act{vi} ? wave * 16 + l16 : 0;  // channel of this lane in the MFMA result layout")
+                else:
+                    # lanes past the piece's channels compute on channel 0 with zero weights and store nothing
+                    s(f"const bool uok{vi} = wave * 16 + l16 < {self.vin[vi].mul};")
+                    s(f"const int u{vi} = uok{vi} ? wave * 16 + l16 : 0;  // channel of this lane in the MFMA result layout")
             # Where the registers exceed the budget of two waves per SIMD, the weight slices of the paths with
             # the fewest multiplies are kept in LDS instead (read like the A operands, one chunk ahead): spilled
             # slices would come back from scratch memory in the middle of the multiply sequence.
             by_cost = sorted(paths_all, key=lambda vp: (self.vout[vp.vo].d, vp.index))
             self.lds_w = []
             if self.tune["uvw_pipe"]:
-                resident = lambda: sum(vp.Wn // 4 for vp in paths_all if vp.index not in self.lds_w)
+                resident = lambda: sum(4 * c16(vp.Wn) for vp in paths_all if vp.index not in self.lds_w)
                 # (what LDS has room for beside the dZ tile: a slice takes 16 x 256 elements)
                 room = (LDS_BUDGET - (RT * self.gstride + (1 + WAVES) * RT * low.L2) * low.elem_size) // \
                     (16 * 64 * WAVES * low.elem_size)
@@ -651,12 +690,14 @@ class MfmaEmitter:
                 s(f"__shared__ T s_wl[{len(self.lds_w)}][16][{64 * WAVES}];")
             for vi, ps, _ in ker:
                 self._load_wreg(s, [vp for vp in ps if vp.index not in self.lds_w], transposed=True,
-                                act=f"act{vi}", u=f"u{vi}")
+                                act=uok(vi), u=f"u{vi}")
             for n, pi in enumerate(self.lds_w):
                 vp = next(q for q in paths_all if q.index == pi)
                 s("#pragma unroll")
-                s(f"for (int st = 0; st < {vp.Wn // 4}; ++st) s_wl[{n}][st][tid] = "
-                  f"act{vp.vi} ? W[{vp.woff} + u{vp.vi} * {vp.ld} + 4 * st + lq] : T(0);")
+                wcond = "" if vp.Wn % 16 == 0 else f" && 4 * st + lq < {vp.Wn}"
+                cond = f"({uok(vp.vi)}{wcond})" if wcond else uok(vp.vi)
+                s(f"for (int st = 0; st < {4 * c16(vp.Wn)}; ++st) s_wl[{n}][st][tid] = "
+                  f"{cond} ? W[{vp.woff} + u{vp.vi} * {vp.ld} + 4 * st + lq] : T(0);")
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
             s(f"const i64 row0 = tile * {RT};")
             s("__syncthreads();")
@@ -686,7 +727,7 @@ class MfmaEmitter:
                 s("#pragma unroll")
                 s.open("for (int i = 0; i < 4; ++i)")
                 s(f"const i64 row = row0 + {self.row('i')};")
-                s.open("if (row < num_batch)")
+                s.open("if (row < num_batch)" if b1.mul % 16 == 0 else f"if (row < num_batch && uok{vi})")
                 s(f"T* dp = L1_grad + row * {low.L1} + {b1.off} + u{vi} * {b1.d};")
                 for c in range(b1.d):
                     s(f"dp[{c}] {'=' if first and not self.accumulate else '+='} dx{vi}[i][{c}];")
@@ -712,8 +753,8 @@ class MfmaEmitter:
 
         # ---------------- dW ----------------------------------------------------
         xrows = (2 if self.t1 else 1) * 2 * (RT // WAVES) * self.max_d1
-        regs = lambda ker: (sum(4 * (vp.Wn // 16) for g in ker for vp in g[1]) + xrows
-                            + 4 * max(self.vout[g[0]].mul // 16 for g in ker) + 64)
+        regs = lambda ker: (sum(4 * c16(vp.Wn) for g in ker for vp in g[1]) + xrows
+                            + 4 * max(c16(self.vout[g[0]].mul) for g in ker) + 64)
 
         def dw_lds(ker, nbuf):
             """Bytes of LDS of a dW kernel: the dZ columns of its pieces, the T tile (one or two copies), Y."""
@@ -758,7 +799,7 @@ class MfmaEmitter:
                 s(f"T aa[{RT // WAVES}][{self.max_d1}], ab[{RT // WAVES}][{self.max_d1}];")
             # dw<path>[n]: D tile rows = channels u of the wave's slice, columns = w in 16 n .. 16 n + 15
             for vp in order_all:
-                ntile = vp.Wn // 16
+                ntile = c16(vp.Wn)
                 s(f"v4t dw{vp.index}[{ntile}];")
                 s(f"for (int n = 0; n < {ntile}; ++n) dw{vp.index}[n] = v4t{{}};")
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
@@ -787,8 +828,10 @@ class MfmaEmitter:
                 s("const int kq = 4 * st + lq;")
                 s("const int kk = kq >> 4, rr = kq & 15;")
                 s(f"const T a = s_T[{buf}][kk][u][rr];")
-                for nn in range(vp.Wn // 16):
-                    s(f"dw{vp.index}[{nn}] = {MFMA}(a, s_g[rr][{bo.off - col0} + ({16 * nn} + l16) * {bo.d} + kk], "
+                for nn in range(c16(vp.Wn)):
+                    # (columns past the piece: its last column again; what they give is not stored)
+                    wcol = f"({16 * nn} + l16)" if 16 * nn + 16 <= vp.Wn else f"min({16 * nn} + l16, {vp.Wn - 1})"
+                    s(f"dw{vp.index}[{nn}] = {MFMA}(a, s_g[rr][{bo.off - col0} + {wcol} * {bo.d} + kk], "
                       f"dw{vp.index}[{nn}], 0, 0, 0);")
                 s.close()
                 s.close()
@@ -796,10 +839,13 @@ class MfmaEmitter:
             s.close()
             for vp in order_all:
                 s.open(f"if (wave * 16 < {vp.U})")
-                for nn in range(vp.Wn // 16):
+                for nn in range(c16(vp.Wn)):
                     s("#pragma unroll")
                     s.open("for (int i = 0; i < 4; ++i)")
-                    s(f"prow[{vp.woff} + (wave * 16 + {self.row('i')}) * {vp.ld} + {16 * nn} + l16] = dw{vp.index}[{nn}][i];")
+                    conds = ([] if vp.U % 16 == 0 else [f"wave * 16 + {self.row('i')} < {vp.U}"]) + \
+                        ([] if 16 * nn + 16 <= vp.Wn else [f"{16 * nn} + l16 < {vp.Wn}"])
+                    guard = f"if ({' && '.join(conds)}) " if conds else ""
+                    s(f"{guard}prow[{vp.woff} + (wave * 16 + {self.row('i')}) * {vp.ld} + {16 * nn} + l16] = dw{vp.index}[{nn}][i];")
                     s.close()
                 s.close()
             s.close()

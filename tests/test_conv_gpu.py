@@ -65,19 +65,22 @@ CASES = [
     ("odd", lambda: _odd(False), 40, 6),
     ("odd-shared", lambda: _odd(True), 40, 6),
     # 'uvw' problems: fused kernels (receiver walk forward, per-edge backward + ordered sender-side sum; shared
-    # weights: partial weight-gradient rows per wave, summed in order); shared weights on the matrix cores: batch
-    # kernels on gathered rows + ordered segment sum
+    # weights: partial weight-gradient rows per wave, summed in order); shared weights on the matrix cores (single-
+    # channel second operand): batch kernels on gathered rows + ordered segment sum
     ("uvw", lambda: _fc(False), 40, 6),
     ("uvw-diffdock", lambda: P.diffdock_problems()[0], 40, 6),
     ("uvw-diffdock-f64", lambda: _as_f64(P.diffdock_problems()[1]), 30, 5),
     ("uvw-e3tools-conv", lambda: P.e3tools_problems()[0], 40, 6),
     ("uvw-shared", lambda: _fc(True), 40, 6),
     ("uvw-shared-lds", lambda: P.FullyConnectedTPProblem(
-        "40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e", shared_weights=True, internal_weights=False,
+        "70x0e+20x1o", "2x0e+1x1o", "70x0e+20x1o", shared_weights=True, internal_weights=False,
         label="uvw-shared-lds"), 40, 6),
     ("uvw-shared-global-f64", lambda: _as_f64(P.FullyConnectedTPProblem(
-        "100x0e+70x1o", "1x0e+1x1o", "33x0e+20x1o", shared_weights=True, internal_weights=False,
+        "100x0e+70x1o", "2x0e+1x1o", "33x0e+20x1o", shared_weights=True, internal_weights=False,
         label="uvw-shared-global")), 30, 5),
+    ("uvw-shared-mfma-padded", lambda: P.FullyConnectedTPProblem(
+        "40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e", shared_weights=True, internal_weights=False,
+        label="uvw-shared-mfma-padded"), 40, 6),
     ("uvw-shared-tetris", lambda: P.tetris_poly_problems()[0], 40, 6),
     ("uvw-cfg4-mfma", P.config4_uvw_shared, 30, 5),
     # output gradient too large for one wave: forward shares the output segments, backward the output
@@ -166,8 +169,8 @@ def test_uvw_shared_weights_fused_matches_unfused(monkeypatch):
     bits on every run (the partial weight-gradient rows are summed in a fixed order), at a graph large enough
     for every wave of the bounded backward grid to see edges and at one where most waves see none."""
     from openequivariance_amd._torch import ops
-    problem = P.FullyConnectedTPProblem("40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e", shared_weights=True,
-                                        internal_weights=False, label="uvw-shared-lds")
+    problem = P.FullyConnectedTPProblem("40x0e+30x1o", "2x0e+1x1o", "25x0e+10x1o+5x2e", shared_weights=True,
+                                        internal_weights=False, label="uvw-shared-regs")
     for n_nodes, deg in ((3000, 12), (20, 3)):
         coords, rows, cols = _graph(n_nodes, deg, seed=4)
         E = len(rows)

@@ -96,9 +96,10 @@ def _fc(shared, in2="1x0e+2x1o"):
                                      internal_weights=False, label="fc-uvw")
 
 
-def _wide_fc(shared):
-    # channel blocks that are no multiples of 16 (no matrix-core path) and wider than a wave
-    return P.FullyConnectedTPProblem("70x0e+20x1o", "1x0e+1x1o", "70x0e+20x1o", shared_weights=shared,
+def _wide_fc(shared, in2="1x0e+1x1o"):
+    # channel blocks that are no multiples of 16 and wider than a wave (shared weights: on the matrix cores with
+    # padded tiles, unless the second operand has several channels)
+    return P.FullyConnectedTPProblem("70x0e+20x1o", in2, "70x0e+20x1o", shared_weights=shared,
                                      internal_weights=False, label="wide-fc-uvw")
 
 
@@ -117,13 +118,14 @@ UVW = [
     ("uvw-tetris-1-shared", lambda: P.tetris_poly_problems()[0], 129),
     ("uvw-tetris-2-shared", lambda: P.tetris_poly_problems()[1], 65),
     ("uvw-wide-shared", lambda: _wide_fc(True), 600),
+    ("uvw-wide-mul2-shared", lambda: _wide_fc(True, "2x0e+1x1o"), 300),
 ]
 UVW_CONV = [c for c in UVW if not c[0].endswith(("shared", "shared-f64"))]
 # shared weights in the fused convolution: the three ways of summing the weight gradient (registers, LDS copy per
 # wave, partial rows in global memory when the weight tensor exceeds 64 KB)
-UVW_CONV_SHARED = [c for c in UVW if c[0].endswith(("shared", "shared-f64"))] + [
+UVW_CONV_SHARED = [c for c in UVW if c[0].endswith(("shared", "shared-f64")) and c[0] != "uvw-wide-shared"] + [
     ("uvw-big-shared-f64", lambda: _f64(P.FullyConnectedTPProblem(
-        "100x0e+70x1o", "1x0e+1x1o", "33x0e+20x1o", shared_weights=True, internal_weights=False,
+        "100x0e+70x1o", "2x0e+1x1o", "33x0e+20x1o", shared_weights=True, internal_weights=False,
         label="big-fc-uvw")), 0)]
 
 
@@ -131,14 +133,18 @@ def _fc_shared(in1, in2, out):
     return P.FullyConnectedTPProblem(in1, in2, out, shared_weights=True, internal_weights=False, label=f"fc-shared {in1}")
 
 
-# shared weights with multiplicities that are multiples of 16: the matrix-core kernels (second-order pair = variants
-# of the first-order kernels with the summed contraction, run on both weight tensors)
+# shared weights and a single-channel second operand: the matrix-core kernels (second-order pair = variants of the
+# first-order kernels with the summed contraction, run on both weight tensors); multiplicities that are no
+# multiples of 16 on padded tiles
 MFMA = [
     ("cfg4", P.config4_uvw_shared, 83),
     ("cfg4-f64", lambda: P.config4_uvw_shared(np.float64), 37),
     ("mfma-mixed", lambda: _fc_shared("64x0e+32x1o+16x2e", "1x0e+1x1o", "48x0e+80x1o+16x2e"), 50),
     ("mfma-mixed-f64", lambda: _f64(_fc_shared("64x0e+32x1o+16x2e", "1x0e+1x1o", "48x0e+80x1o+16x2e")), 33),
     ("mfma-128", lambda: _fc_shared("128x0e+128x1o", "1x0e+1x1o", "128x0e+128x1o"), 45),
+    ("mfma-pad-diffdock", lambda: _shared(P.diffdock_problems()[0]), 50),
+    ("mfma-pad-mid-f64", lambda: _f64(_fc_shared("40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e")), 35),
+    ("mfma-pad-wide", lambda: _fc_shared("100x0e+70x1o", "1x0e+1x1o", "33x0e+20x1o"), 50),
     ("mfma-gaps", lambda: oeq.TPProblem(
         "32x0e+16x1o+32x2e", "1x0e+1x1o", "32x0e+16x1o+48x2e+16x1e",
         [(0, 0, 0, "uvw", True), (1, 1, 0, "uvw", True), (0, 1, 1, "uvw", True), (2, 0, 2, "uvw", True, 0.7)],
@@ -213,7 +219,12 @@ def test_conv_fused_matches_composition(name, make, batch, det, monkeypatch):
     _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
 
 
-@pytest.mark.parametrize("name,make,batch", SHARED + UVW_CONV_SHARED, ids=[c[0] for c in SHARED + UVW_CONV_SHARED])
+# matrix-core problems: the convolution is unfused, its second-order pass the batch kernel pair on gathered rows
+MFMA_CONV = [c for c in MFMA if c[0] in ("cfg4", "mfma-mixed-f64", "mfma-pad-diffdock", "mfma-pad-wide")]
+
+
+@pytest.mark.parametrize("name,make,batch", SHARED + UVW_CONV_SHARED + MFMA_CONV,
+                         ids=[c[0] for c in SHARED + UVW_CONV_SHARED + MFMA_CONV])
 def test_conv_shared_weights_fused_matches_composition_and_oracle(name, make, batch):
     """Shared weights (device-grouped edge lists only): kernel B sums the weight gradient over all edges of a
     wave (group) and the partial rows in a fixed order. Against the composition of first-order ops and against

@@ -4,7 +4,8 @@ no path writes, path weights, 'uvu' and 'uvw', per-row and shared weights, fp32 
 forward / backward, the fused second-order pair where the kernel set has one, and the convolution (caller-sorted
 and device-grouped edge lists; with and without compensated summation) forward / backward / second order. The
 fixed problem zoo of the other test files covers the shapes models use; this sweep looks for generator corner
-cases between them."""
+cases between them. A second generator draws shared-weight fully connected problems for the matrix-core kernels
+with multiplicities that are no multiples of 16."""
 
 import numpy as np
 import pytest
@@ -81,13 +82,45 @@ def _compare(tag, got, want, tol):
         assert e <= tol, (tag, n, e)
 
 
+def random_shared_fully_connected_problem(rng):
+    """Shared weights, single-channel second operand, multiplicities from 3 to 130 of which few are multiples of
+    16: the matrix-core kernels on tiles padded with zero weights (pieces of 64 channels plus a narrow rest, k-steps
+    and output tiles that end inside a group of 4 or 16 channels). None when the draw selected no path."""
+    muls = [3, 5, 10, 12, 17, 20, 24, 33, 40, 48, 50, 64, 70, 100, 130]
+    in1 = [(int(rng.choice(muls)), int(rng.integers(0, 4)), int(rng.choice([1, -1]))) for _ in range(rng.integers(1, 4))]
+    in2 = [(1, int(rng.integers(0, 4)), int(rng.choice([1, -1]))) for _ in range(rng.integers(1, 4))]
+    out = [(int(rng.choice(muls)), int(rng.integers(0, 4)), int(rng.choice([1, -1]))) for _ in range(rng.integers(1, 4))]
+    paths = [(i1, i2, io, "uvw", True, 1.0 if rng.random() < 0.7 else float(rng.uniform(0.3, 2.0)))
+             for i1, (_, l1, p1) in enumerate(in1) for i2, (_, l2, p2) in enumerate(in2)
+             for io, (_, lo, po) in enumerate(out)
+             if abs(l1 - l2) <= lo <= l1 + l2 and po == p1 * p2 and rng.random() < 0.85]
+    if not paths:
+        return None
+    dt = np.float64 if rng.random() < 0.4 else np.float32
+    return oeq.TPProblem(_irreps(in1), _irreps(in2), _irreps(out), paths, shared_weights=True, internal_weights=False,
+                         irrep_dtype=dt, weight_dtype=dt)
+
+
 @pytest.mark.parametrize("seed", range(2000, 2030))
 def test_random_problem(seed):
-    from oracle.torch_ref import TorchConv, TorchTP
     rng = np.random.default_rng(seed)
     problem = random_problem(rng)
     if problem is None:
         pytest.skip("the draw selected no path")
+    _check_every_op(problem, rng)
+
+
+@pytest.mark.parametrize("seed", range(2100, 2116))
+def test_random_shared_weight_problem_on_padded_tiles(seed):
+    rng = np.random.default_rng(seed)
+    problem = random_shared_fully_connected_problem(rng)
+    if problem is None:
+        pytest.skip("the draw selected no path")
+    _check_every_op(problem, rng)
+
+
+def _check_every_op(problem, rng):
+    from oracle.torch_ref import TorchConv, TorchTP
     dt = np.dtype(problem.irrep_dtype)
     tol = 1e-5 if dt == np.float32 else 1e-12
     ref = R.Problem.from_spec(problem)
@@ -128,7 +161,7 @@ def test_random_problem(seed):
                  [R.conv_forward(ref, Xn, Yn, Wn, r_, c_)], tol)
         _compare(f"conv backward det={det}", ops.conv_backward(X, Y, W, G, tr, tc, tpm, conv.kid),
                  R.conv_backward(ref, Xn, Yn, Wn, Gn, r_, c_), tol)
-        if not ec.unfused and ec.kernels().has_double_backward():
+        if ec.kernels().has_double_backward():
             oracle = TorchConv(ref, torch.float64)
             want = _second_order(lambda p, q, s: oracle(p, q, s, torch.tensor(r_), torch.tensor(c_)), X, Y, W, G, A, Bc, C)
             _compare(f"conv second order det={det}", ops.conv_double_backward(X, Y, W, G, A, Bc, C, tr, tc, tpm, conv.kid),

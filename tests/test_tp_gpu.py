@@ -58,6 +58,12 @@ def _fc_shared(in1, in2, out):
                                      label=f"fc-shared {in1}")
 
 
+def _shared(problem):
+    q = problem.clone()
+    q.shared_weights = True
+    return q
+
+
 def _as_f64(problem):
     q = problem.clone()
     q.irrep_dtype, q.weight_dtype = np.float64, np.float64
@@ -124,9 +130,24 @@ CASES = [
     ("mfma-l3-wide-f64", lambda: _as_f64(oeq.TPProblem(
         "16x1o+128x3o", "1x2o", "96x3e", [(0, 0, 0, "uvw", True), (1, 0, 0, "uvw", True, 0.6)],
         shared_weights=True, internal_weights=False, label="mfma-l3-wide")), 40),
+    # multiplicities that are no multiples of 16 (or of 4): tiles padded with zero weights. Channels past a piece are
+    # neither loaded nor stored; 70 and 100 channels leave a narrow second piece; a block no path reads or writes
+    ("mfma-pad-diffdock", lambda: _shared(P.diffdock_problems()[0]), 50),
+    ("mfma-pad-mid", lambda: _fc_shared("40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e"), 67),
+    ("mfma-pad-mid-f64", lambda: _as_f64(_fc_shared("40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e")), 35),
+    ("mfma-pad-wide", lambda: _fc_shared("100x0e+70x1o", "1x0e+1x1o", "33x0e+20x1o"), 50),
+    ("mfma-pad-wide-f64", lambda: _as_f64(_fc_shared("70x0e+20x1o", "1x0e+1x1o", "70x0e+20x1o")), 33),
+    ("mfma-pad-gaps", lambda: oeq.TPProblem(
+        "30x0e+13x1o+45x2e", "1x0e+1x1o", "27x0e+15x1e+61x1o",
+        [(0, 0, 0, "uvw", True), (0, 1, 2, "uvw", True), (1, 0, 2, "uvw", True, 0.6), (1, 1, 0, "uvw", True)],
+        shared_weights=True, internal_weights=False, label="mfma-pad-gaps"), 50),
+    ("mfma-pad-l3", lambda: oeq.TPProblem(
+        "14x1o+90x3o", "1x2o", "75x3e+11x1e", [(0, 0, 0, "uvw", True), (1, 0, 0, "uvw", True, 0.6), (1, 0, 1, "uvw", True)],
+        shared_weights=True, internal_weights=False, label="mfma-pad-l3"), 40),
 ]
 MFMA_CASES = {"cfg4-shared", "cfg4-f64", "mfma-32", "mfma-128", "mfma-mixed", "mfma-gaps", "mfma-128-f64",
-              "mfma-mixed-f64", "mfma-l3-f64", "mfma-l3-wide-f64"}
+              "mfma-mixed-f64", "mfma-l3-f64", "mfma-l3-wide-f64", "mfma-pad-diffdock", "mfma-pad-mid",
+              "mfma-pad-mid-f64", "mfma-pad-wide", "mfma-pad-wide-f64", "mfma-pad-gaps", "mfma-pad-l3"}
 
 
 @pytest.mark.parametrize("name,make,B", CASES, ids=[c[0] for c in CASES])
