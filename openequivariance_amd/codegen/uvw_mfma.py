@@ -9,9 +9,13 @@ reference does this mix with a scalar-FMA warp matmul on 32-wide chunks
 (openequivariance/openequivariance/templates/wmm.cuh:1-87,
 loop_unroll_tp.cuh:55-84, 217-272).
 
+A path whose second operand has V channels is V such mixes, one per channel v with
+the weight matrix ``W[:, v, :]``.
+
 Work decomposition: irrep blocks are cut into pieces of at most 64 channels
 (a piece whose channel count is no multiple of 16 is padded to one with zero
-weights: its missing channels are never loaded or stored), a path into one sub-path per pair of
+weights: its missing channels are never loaded or stored), a path into one sub-path per channel of the second
+operand and pair of
 pieces with its own 64 x 64 (or smaller) corner of the path's weight matrix. A
 block of 4 waves owns a tile of 16 batch rows at a time; wave ``w`` owns output
 channels (forward) or input channels (backward) ``16w .. 16w+15`` of a piece
@@ -113,6 +117,12 @@ class VPath:
     ld: int
     ub: int
     wb: int
+    v: int = 0    # channel of the second operand (its own sub-path: W[u, v, w] is a U x Wn matrix for every v)
+
+    def tag(self, side: str) -> str:
+        """Names the group of sub-paths a kernel takes from the other side of a piece on ``side``."""
+        k = self.ub if side == "vo" else self.wb
+        return f"{k}" if self.v == 0 else f"{k}v{self.v}"
 
 
 def _pieces(blocks, piece: int) -> List[VBlock]:
@@ -128,15 +138,18 @@ def _split(low: Lowered):
     vin, vout = _pieces(low.in1, PIECE), _pieces(low.out, PIECE)
     vpaths = []
     for p in low.paths:
-        wtot = low.out[p.io].mul
-        for vi, a in enumerate(vin):
-            if a.orig != p.i1:
-                continue
-            for vo, o in enumerate(vout):
-                if o.orig != p.io:
+        wtot, V = low.out[p.io].mul, low.in2[p.i2].mul
+        for v in range(V):
+            for vi, a in enumerate(vin):
+                if a.orig != p.i1:
                     continue
-                vpaths.append(VPath(len(vpaths), p, vi, vo, a.mul, o.mul,
-                                    p.woff + a.chunk * PIECE * wtot + o.chunk * PIECE, wtot, a.chunk, o.chunk))
+                for vo, o in enumerate(vout):
+                    if o.orig != p.io:
+                        continue
+                    # W[u, v, w] of the path: rows (u) are V * wtot words apart
+                    vpaths.append(VPath(len(vpaths), p, vi, vo, a.mul, o.mul,
+                                        p.woff + (a.chunk * PIECE * V + v) * wtot + o.chunk * PIECE, V * wtot,
+                                        a.chunk, o.chunk, v))
     return vin, vout, vpaths
 
 
@@ -148,11 +161,11 @@ def _groups(vpaths: List[VPath], side: str, n_blocks: int):
     out = []
     for b in range(n_blocks):
         mine = [vp for vp in vpaths if getattr(vp, side) == b]
-        keys = sorted({getattr(vp, other) for vp in mine})
+        keys = sorted({(getattr(vp, other), vp.v) for vp in mine})
         if not keys:
             out.append((b, [], True))
         for n, key in enumerate(keys):
-            out.append((b, [vp for vp in mine if getattr(vp, other) == key], n == 0))
+            out.append((b, [vp for vp in mine if (getattr(vp, other), vp.v) == key], n == 0))
     return out
 
 
@@ -165,9 +178,6 @@ def supported(low: Lowered) -> bool:
     # (fp64: rows of up to about 1 000 elements)
     if (RT * (low.L3 + 36) + (1 + WAVES) * RT * low.L2) * low.elem_size > LDS_BUDGET:
         return False
-    for p in low.paths:
-        if low.in2[p.i2].mul != 1:
-            return False
     vin, vout, vpaths = _split(low)
     # Multiplicities that are no multiples of 16 run on tiles padded with zero weights. Where nearly all of a
     # tile would be padding the general kernels are the better choice: ``uvw_mfma_fill`` = least share (percent)
@@ -227,6 +237,9 @@ class MfmaEmitter:
     # ---- CG part of one path for one (row, channel)
     def _emit_path_fns(self, s: Src):
         low = self.low
+        # second operands with several channels: the functions take the offset of the channel's values in the row
+        self.multi_v = any(low.in2[p.i2].mul > 1 for p in low.paths)
+        yo, yo_par = (" + yo", ", const int yo") if self.multi_v else ("", "")
         for p in low.paths:
             b1, b2, bo = low.in1[p.i1], low.in2[p.i2], low.out[p.io]
 
@@ -236,12 +249,12 @@ class MfmaEmitter:
                     key = (self.lit(abs(c)), j)
                     if key not in names:
                         names[key] = f"q{len(names)}"
-                        s(f"const T {names[key]} = T({key[0]}) * y[{b2.off + j}];")
+                        s(f"const T {names[key]} = T({key[0]}) * y[{b2.off + j}{yo}];")
                     out[n] = (names[key], c < 0)
                 return out
 
             # t[k] = sum c x_i y_j
-            s.open(f"OEQ_DEV void cg_fwd{p.index}(const T (&x)[{self.max_d1}], const T* y, T (&t)[{bo.d}])")
+            s.open(f"OEQ_DEV void cg_fwd{p.index}(const T (&x)[{self.max_d1}], const T* y, T (&t)[{bo.d}]{yo_par})")
             prods = products()
             started = set()
             for n, (i, j, k, c) in enumerate(p.nnz):
@@ -258,7 +271,7 @@ class MfmaEmitter:
             # given G[k] = sum_w W[u,w] dZ[w,k]:  dx_i += c y_j G_k,  dy_j += c x_i G_k
             s.open(
                 f"OEQ_DEV void cg_bwd{p.index}(const T (&x)[{self.max_d1}], const T* y, const T (&G)[{bo.d}], "
-                f"T (&dx)[{b1.d}], T (&dy)[{low.L2}])"
+                f"T (&dx)[{b1.d}], T (&dy)[{low.L2}]{yo_par})"
             )
             prods = products()
             for n, (i, j, k, c) in enumerate(p.nnz):
@@ -269,7 +282,7 @@ class MfmaEmitter:
                 if (i, k) not in pair:
                     pair[(i, k)] = f"xg{len(pair)}"
                     s(f"const T {pair[(i, k)]} = x[{i}] * G[{k}];")
-                s(f"dy[{b2.off + j}] += T({self.lit(c)}) * {pair[(i, k)]};")
+                s(f"dy[{b2.off + j}{yo}] += T({self.lit(c)}) * {pair[(i, k)]};")
             s.close()
 
     def _prologue(self, s: Src):
@@ -352,18 +365,19 @@ class MfmaEmitter:
 
     def _t_compute(self, s: Src, vp: VPath, xsrc: str, buf: str):
         d3 = self.vout[vp.vo].d
+        yo = f", {vp.v * self.low.in2[vp.p.i2].d}" if self.multi_v else ""
         s.open(f"for (int rr = 0; rr < {RT // WAVES}; ++rr)")
         s(f"const int r = wave * {RT // WAVES} + rr;")
         s(f"T t[{d3}];")
         if self.t1:
             # contraction of the second-order pass: (a, y) and (x, b)
             s(f"T t2[{d3}];")
-            s(f"cg_fwd{vp.p.index}(a{xsrc[1:]}[rr], s_y[r], t);")
-            s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y2[r], t2);")
+            s(f"cg_fwd{vp.p.index}(a{xsrc[1:]}[rr], s_y[r], t{yo});")
+            s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y2[r], t2{yo});")
             for k in range(d3):
                 s(f"t[{k}] += t2[{k}];")
         else:
-            s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y[r], t);")
+            s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y[r], t{yo});")
         if self.tlanes < 64:
             s.open(f"if (lane < {self.tlanes})")
         for k in range(d3):
@@ -390,7 +404,8 @@ class MfmaEmitter:
             s(f"T Gk[{d3}];")
             for k in range(d3):
                 s(f"Gk[{k}] = {G}[{k}][i];")
-            s(f"cg_bwd{vp.p.index}({x}[i], s_y[{self.row('i')}], Gk, {dx}[i], dy[i]);")
+            yo = f", {vp.v * self.low.in2[vp.p.i2].d}" if self.multi_v else ""
+            s(f"cg_bwd{vp.p.index}({x}[i], s_y[{self.row('i')}], Gk, {dx}[i], dy[i]{yo});")
             s.close()
 
         if pipe == 0:
@@ -561,7 +576,7 @@ class MfmaEmitter:
             vo0, order0, _ = ker[0]
             if not order0 and self.accumulate:
                 continue  # nothing to add to a piece no path writes
-            name = (self.prefix + "forward") if not names else f"{self.prefix}forward_o{vo0}_{order0[0].ub if order0 else 0}"
+            name = (self.prefix + "forward") if not names else f"{self.prefix}forward_o{vo0}_{order0[0].tag('vo') if order0 else 0}"
             names.append(name)
             s("// ======== out pieces " + ", ".join(f"{vo}: {self.vout[vo].mul} x l={self.vout[vo].l}" for vo, _, _ in ker))
             self._kernel_open(s, name, self.sig_f, self.tune["uvw_wf"])
@@ -651,7 +666,7 @@ class MfmaEmitter:
             vi0, paths0, _ = ker[0]
             if not paths0 and self.accumulate:
                 continue  # nothing to add to a piece no path reads
-            name = (self.prefix + "backward") if not names else f"{self.prefix}backward_x{vi0}_{paths0[0].wb if paths0 else 0}"
+            name = (self.prefix + "backward") if not names else f"{self.prefix}backward_x{vi0}_{paths0[0].tag('vi') if paths0 else 0}"
             names.append(name)
             s("// ======== in1 pieces " + ", ".join(f"{vi}: {self.vin[vi].mul} x l={self.vin[vi].l}" for vi, _, _ in ker))
             self._kernel_open(s, name, self.sig_b, self.tune["uvw_wx"])
@@ -776,7 +791,7 @@ class MfmaEmitter:
             col0 = pieces[0].off
             ncols = pieces[-1].off + pieces[-1].mul * pieces[-1].d - col0
             maxd = max(b.d for b in pieces)
-            name = f"{self.prefix}backward_w{ker[0][0]}_{order_all[0].ub}"
+            name = f"{self.prefix}backward_w{ker[0][0]}_{order_all[0].tag('vo')}"
             names.append(name)
             s("// ======== dW of the sub-paths into out pieces " + ", ".join(str(vo) for vo, _, _ in ker))
             self._kernel_open(s, name, self.sig_b, self.tune["uvw_ww"])

@@ -96,9 +96,14 @@ def _fc(shared, in2="1x0e+2x1o"):
                                      internal_weights=False, label="fc-uvw")
 
 
+def _fc_general(out):
+    return P.FullyConnectedTPProblem("20x0e+10x1o", "20x0e+5x1o", out, shared_weights=True, internal_weights=False,
+                                     label="general-fc-uvw")
+
+
 def _wide_fc(shared, in2="1x0e+1x1o"):
     # channel blocks that are no multiples of 16 and wider than a wave (shared weights: on the matrix cores with
-    # padded tiles, unless the second operand has several channels)
+    # padded tiles, one sub-path per channel of the second operand)
     return P.FullyConnectedTPProblem("70x0e+20x1o", in2, "70x0e+20x1o", shared_weights=shared,
                                      internal_weights=False, label="wide-fc-uvw")
 
@@ -119,14 +124,15 @@ UVW = [
     ("uvw-tetris-2-shared", lambda: P.tetris_poly_problems()[1], 65),
     ("uvw-wide-shared", lambda: _wide_fc(True), 600),
     ("uvw-wide-mul2-shared", lambda: _wide_fc(True, "2x0e+1x1o"), 300),
+    # off the matrix cores (second operand of more than 32 values): weight gradient in an LDS copy per wave, and in
+    # partial rows in global memory
+    ("uvw-lds-shared", lambda: _fc_general("12x0e+6x1o"), 200),
+    ("uvw-global-shared-f64", lambda: _f64(_fc_general("40x0e+20x1o")), 100),
 ]
 UVW_CONV = [c for c in UVW if not c[0].endswith(("shared", "shared-f64"))]
 # shared weights in the fused convolution: the three ways of summing the weight gradient (registers, LDS copy per
 # wave, partial rows in global memory when the weight tensor exceeds 64 KB)
-UVW_CONV_SHARED = [c for c in UVW if c[0].endswith(("shared", "shared-f64")) and c[0] != "uvw-wide-shared"] + [
-    ("uvw-big-shared-f64", lambda: _f64(P.FullyConnectedTPProblem(
-        "100x0e+70x1o", "2x0e+1x1o", "33x0e+20x1o", shared_weights=True, internal_weights=False,
-        label="big-fc-uvw")), 0)]
+UVW_CONV_SHARED = [c for c in UVW if c[0].endswith(("shared", "shared-f64")) and "wide" not in c[0]]
 
 
 def _fc_shared(in1, in2, out):
@@ -145,6 +151,8 @@ MFMA = [
     ("mfma-pad-diffdock", lambda: _shared(P.diffdock_problems()[0]), 50),
     ("mfma-pad-mid-f64", lambda: _f64(_fc_shared("40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e")), 35),
     ("mfma-pad-wide", lambda: _fc_shared("100x0e+70x1o", "1x0e+1x1o", "33x0e+20x1o"), 50),
+    ("mfma-mul3-f64", lambda: _f64(_fc_shared("64x0e+64x1o", "3x0e+2x1o", "64x0e+64x1o")), 33),
+    ("mfma-mul2-pad", lambda: _fc_shared("40x0e+30x1o", "2x0e+1x1o", "25x0e+10x1o+5x2e"), 50),
     ("mfma-gaps", lambda: oeq.TPProblem(
         "32x0e+16x1o+32x2e", "1x0e+1x1o", "32x0e+16x1o+48x2e+16x1e",
         [(0, 0, 0, "uvw", True), (1, 1, 0, "uvw", True), (0, 1, 1, "uvw", True), (2, 0, 2, "uvw", True, 0.7)],
@@ -220,7 +228,8 @@ def test_conv_fused_matches_composition(name, make, batch, det, monkeypatch):
 
 
 # matrix-core problems: the convolution is unfused, its second-order pass the batch kernel pair on gathered rows
-MFMA_CONV = [c for c in MFMA if c[0] in ("cfg4", "mfma-mixed-f64", "mfma-pad-diffdock", "mfma-pad-wide")]
+MFMA_CONV = [c for c in MFMA if c[0] in ("cfg4", "mfma-mixed-f64", "mfma-pad-diffdock", "mfma-pad-wide")] + \
+    [c for c in UVW if c[0] == "uvw-wide-mul2-shared"]
 
 
 @pytest.mark.parametrize("name,make,batch", SHARED + UVW_CONV_SHARED + MFMA_CONV,

@@ -83,12 +83,14 @@ def _compare(tag, got, want, tol):
 
 
 def random_shared_fully_connected_problem(rng):
-    """Shared weights, single-channel second operand, multiplicities from 3 to 130 of which few are multiples of
-    16: the matrix-core kernels on tiles padded with zero weights (pieces of 64 channels plus a narrow rest, k-steps
-    and output tiles that end inside a group of 4 or 16 channels). None when the draw selected no path."""
+    """Shared weights, multiplicities from 3 to 130 of which few are multiples of 16, one to three channels in the
+    second operand: the matrix-core kernels on tiles padded with zero weights (pieces of 64 channels plus a narrow
+    rest, k-steps and output tiles that end inside a group of 4 or 16 channels, one sub-path per channel of the
+    second operand). None when the draw selected no path."""
     muls = [3, 5, 10, 12, 17, 20, 24, 33, 40, 48, 50, 64, 70, 100, 130]
     in1 = [(int(rng.choice(muls)), int(rng.integers(0, 4)), int(rng.choice([1, -1]))) for _ in range(rng.integers(1, 4))]
-    in2 = [(1, int(rng.integers(0, 4)), int(rng.choice([1, -1]))) for _ in range(rng.integers(1, 4))]
+    in2 = [(int(rng.choice([1, 1, 1, 2, 3])), int(rng.integers(0, 4)), int(rng.choice([1, -1])))
+           for _ in range(rng.integers(1, 4))]
     out = [(int(rng.choice(muls)), int(rng.integers(0, 4)), int(rng.choice([1, -1]))) for _ in range(rng.integers(1, 4))]
     paths = [(i1, i2, io, "uvw", True, 1.0 if rng.random() < 0.7 else float(rng.uniform(0.3, 2.0)))
              for i1, (_, l1, p1) in enumerate(in1) for i2, (_, l2, p2) in enumerate(in2)

@@ -141,13 +141,29 @@ CASES = [
         "30x0e+13x1o+45x2e", "1x0e+1x1o", "27x0e+15x1e+61x1o",
         [(0, 0, 0, "uvw", True), (0, 1, 2, "uvw", True), (1, 0, 2, "uvw", True, 0.6), (1, 1, 0, "uvw", True)],
         shared_weights=True, internal_weights=False, label="mfma-pad-gaps"), 50),
+    # second operands with several channels: one sub-path per channel (rows of its weight matrix V * W words apart)
+    ("mfma-mul2-pad", lambda: _fc_shared("40x0e+30x1o", "2x0e+1x1o", "25x0e+10x1o+5x2e"), 50),
+    ("mfma-mul3-f64", lambda: _as_f64(_fc_shared("64x0e+64x1o", "3x0e+2x1o", "64x0e+64x1o")), 33),
+    ("mfma-mul2-mixed", lambda: oeq.TPProblem(
+        "32x0e+20x1o", "1x0e+3x1o+2x1e", "16x0e+40x1o+24x1e",
+        [(0, 0, 0, "uvw", True), (0, 1, 1, "uvw", True, 0.7), (1, 1, 0, "uvw", True), (1, 2, 1, "uvw", True),
+         (1, 0, 1, "uvw", True), (0, 2, 2, "uvw", True)],
+        shared_weights=True, internal_weights=False, label="mfma-mul2-mixed"), 50),
     ("mfma-pad-l3", lambda: oeq.TPProblem(
         "14x1o+90x3o", "1x2o", "75x3e+11x1e", [(0, 0, 0, "uvw", True), (1, 0, 0, "uvw", True, 0.6), (1, 0, 1, "uvw", True)],
         shared_weights=True, internal_weights=False, label="mfma-pad-l3"), 40),
 ]
 MFMA_CASES = {"cfg4-shared", "cfg4-f64", "mfma-32", "mfma-128", "mfma-mixed", "mfma-gaps", "mfma-128-f64",
               "mfma-mixed-f64", "mfma-l3-f64", "mfma-l3-wide-f64", "mfma-pad-diffdock", "mfma-pad-mid",
-              "mfma-pad-mid-f64", "mfma-pad-wide", "mfma-pad-wide-f64", "mfma-pad-gaps", "mfma-pad-l3"}
+              "mfma-pad-mid-f64", "mfma-pad-wide", "mfma-pad-wide-f64", "mfma-pad-gaps", "mfma-pad-l3", "mfma-mul2-pad",
+              "mfma-mul3-f64", "mfma-mul2-mixed"}
+# shared weights off the matrix cores (second operand of more than 32 values): the general kernels' weight gradient
+# in an LDS copy per wave and in partial rows in global memory
+CASES += [
+    ("uvw-shared-lds", lambda: _fc_shared("20x0e+10x1o", "20x0e+5x1o", "12x0e+6x1o"), 77),
+    ("uvw-shared-lds-wide", lambda: _fc_shared("70x0e+3x1o", "20x0e+5x1o", "3x0e+2x1o"), 77),
+    ("uvw-shared-global-f64", lambda: _as_f64(_fc_shared("20x0e+10x1o", "20x0e+5x1o", "40x0e+20x1o")), 41),
+]
 
 
 @pytest.mark.parametrize("name,make,B", CASES, ids=[c[0] for c in CASES])
