@@ -134,6 +134,55 @@ def test_cfg4_full_batch_mfma(dtype):
     assert torch.equal(dw_again, w.grad)
 
 
+@pytest.mark.parametrize("name", ["diffdock-shared", "mul2-f64"])
+def test_padded_matrix_core_tiles_full_batch(name):
+    """Shared weights with multiplicities that are no multiples of 16 (tiles padded with zero weights; second case:
+    a two-channel second operand, fp64) at 262 144 / 65 536 rows: rows at tile and grid boundaries against the oracle,
+    the weight gradient as a sum over disjoint row sets and against the oracle on a slice, same bits on a second run."""
+    from openequivariance_amd.codegen import uvw_mfma
+    from openequivariance_amd.codegen.lower import lower
+    if name == "diffdock-shared":
+        problem = P.diffdock_problems()[0].clone()
+        problem.shared_weights = True
+        B, dtype = 262144, np.float32
+    else:
+        problem = P.FullyConnectedTPProblem("40x0e+30x1o", "2x0e+1x1o", "25x0e+10x1o+5x2e", shared_weights=True,
+                                            internal_weights=False, irrep_dtype=np.float64, weight_dtype=np.float64)
+        B, dtype = 65536, np.float64
+    low = lower(problem)
+    assert uvw_mfma.supported(low)
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    td = torch.float32 if dtype == np.float32 else torch.float64
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(B, low.L1, device="cuda", generator=gen, dtype=td)
+    y = torch.randn(B, low.L2, device="cuda", generator=gen, dtype=td)
+    w = torch.randn(low.WN, device="cuda", generator=gen, dtype=td) / 8
+    g = torch.randn(B, low.L3, device="cuda", generator=gen, dtype=td)
+    tp = oeq.TensorProduct(problem)
+    ops = torch.ops.oeq_amd
+    z = ops.tp_forward(x, y, w, tp.kid)
+    dx, dy, dw = ops.tp_backward(x, y, w, g, tp.kid)
+    assert all(torch.isfinite(t).all() for t in (z, dx, dy, dw))
+    idx = torch.tensor([0, 1, 15, 16, 17, 8191, 8192, B - 17, B - 16, B - 1], device="cuda")
+    ref = R.Problem.from_spec(problem)
+    xs, ys, gs = (t[idx].cpu().numpy() for t in (x, y, g))
+    wn = w.cpu().numpy()
+    assert err(z[idx], R.tp_forward(ref, xs, ys, wn)) <= tol
+    rx, ry, _ = R.tp_backward(ref, xs, ys, wn, gs)
+    assert err(dx[idx], rx) <= tol and err(dy[idx], ry) <= tol
+    half = B // 2
+    _, _, dw1 = ops.tp_backward(x[:half], y[:half], w, g[:half], tp.kid)
+    _, _, dw2 = ops.tp_backward(x[half:], y[half:], w, g[half:], tp.kid)
+    assert _rel(dw1 + dw2, dw) <= tol
+    n = 2048
+    _, _, dws = ops.tp_backward(x[:n], y[:n], w, g[:n], tp.kid)
+    _, _, dw_ref = R.tp_backward(ref, x[:n].cpu().numpy(), y[:n].cpu().numpy(), wn, g[:n].cpu().numpy())
+    assert err(dws, dw_ref) <= tol
+    again = ops.tp_backward(x, y, w, g, tp.kid)
+    assert torch.equal(again[0], dx) and torch.equal(again[1], dy) and torch.equal(again[2], dw)
+    assert torch.equal(ops.tp_forward(2.0 * x, y, 0.25 * w, tp.kid), 0.5 * z)
+
+
 def test_cfg5_full_graph():
     problem = P.config5_mace_conv()
     N = 50000
