@@ -118,11 +118,12 @@ class VPath:
     ub: int
     wb: int
     v: int = 0    # channel of the second operand (its own sub-path: W[u, v, w] is a U x Wn matrix for every v)
+    part: int = 0  # which part of its group, where the group's weight slices exceed a kernel's registers (_groups)
 
     def tag(self, side: str) -> str:
         """Names the group of sub-paths a kernel takes from the other side of a piece on ``side``."""
         k = self.ub if side == "vo" else self.wb
-        return f"{k}" if self.v == 0 else f"{k}v{self.v}"
+        return f"{k}" + (f"v{self.v}" if self.v else "") + (f"p{self.part}" if self.part else "")
 
 
 def _pieces(blocks, piece: int) -> List[VBlock]:
@@ -153,10 +154,21 @@ def _split(low: Lowered):
     return vin, vout, vpaths
 
 
-def _groups(vpaths: List[VPath], side: str, n_blocks: int):
-    """Kernels of one pass: for every piece on ``side`` ('vo' or 'vi') its sub-paths grouped by the piece
-    index on the other side. Returns [(piece, [sub-paths], first kernel of that piece?)]; a piece without
-    paths gets one entry with an empty list."""
+# Most registers (in elements) that the resident weight slices of one kernel take, per pass: a group of sub-paths
+# beyond that (or beyond what the kernel's other registers leave, see the ``limit`` functions of the emitters) is
+# cut into parts with a kernel each (an irrep fed by more than five 64-channel paths, say).
+SLICE_REGS = {"forward": 80, "dx": 80, "dw": 80}
+
+
+def _slice_regs(vp: VPath, which: str) -> int:
+    return c4(vp.U) if which == "forward" else 4 * c16(vp.Wn)
+
+
+def _groups(vpaths: List[VPath], side: str, n_blocks: int, which: str, limit=None):
+    """Kernels of one pass (``which``: 'forward', 'dx' or 'dw'): for every piece on ``side`` ('vo' or 'vi') its
+    sub-paths grouped by the piece index on the other side and the channel of the second operand, a group cut into
+    parts whose weight slices fit ``limit(piece, sub-paths)`` registers. Returns [(piece, [sub-paths], first
+    kernel of that piece?)]; a piece without paths gets one entry with an empty list."""
     other = "ub" if side == "vo" else "wb"
     out = []
     for b in range(n_blocks):
@@ -165,7 +177,21 @@ def _groups(vpaths: List[VPath], side: str, n_blocks: int):
         if not keys:
             out.append((b, [], True))
         for n, key in enumerate(keys):
-            out.append((b, [vp for vp in mine if (getattr(vp, other), vp.v) == key], n == 0))
+            parts, room = [], 0
+            sel = [q for q in mine if (getattr(q, other), q.v) == key]
+            budget = min(SLICE_REGS[which], limit(b, sel)) if limit else SLICE_REGS[which]
+            total = sum(_slice_regs(vp, which) for vp in sel)
+            if total > budget:  # parts of about equal size
+                budget = max(-(-total // -(-total // budget)), max(_slice_regs(vp, which) for vp in sel))
+            for vp in sel:
+                need = _slice_regs(vp, which)
+                if not parts or need > room:
+                    parts.append([])
+                    room = budget
+                parts[-1].append(vp)
+                room -= need
+                vp.part = len(parts) - 1
+            out += [(b, part, n == 0 and c == 0) for c, part in enumerate(parts)]
     return out
 
 
@@ -189,13 +215,7 @@ def supported(low: Lowered) -> bool:
     padded = sum(16 * c16(vp.U) * 16 * c16(vp.Wn) for vp in vpaths)
     if 100 * real < tuning(dict(uvw_mfma_fill=30))["uvw_mfma_fill"] * padded:
         return False
-    # register budget of the widest kernel of each pass: 16-channel k-steps of resident weight slices
-    # (forward, dX: a few slices may move to LDS there) and 16 x 16 dW tiles
-    fwd = max((sum(c4(vp.U) for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
-    dxk = max((sum(4 * c16(vp.Wn) for vp in g) for _, g, _ in _groups(vpaths, "vi", len(vin))), default=0)
-    dwk = max((sum(4 * c16(vp.Wn) for vp in g) for _, g, _ in _groups(vpaths, "vo", len(vout))), default=0)
-    # (register counts in elements: fp64 runs one wave per SIMD with twice the registers)
-    return fwd <= 80 and dxk <= 112 and dwk <= 80
+    return True
 
 
 class MfmaEmitter:
@@ -572,7 +592,10 @@ class MfmaEmitter:
         xrows = (2 if self.t1 else 1) * 2 * (RT // WAVES) * self.max_d1
         cost = lambda ker: (sum(c4(vp.U) for g in ker for vp in g[1]) + sum(4 * self.vout[g[0]].d for g in ker)
                             + xrows + 64)
-        for ker in self._merge(_groups(self.vpaths, "vo", len(self.vout)), cost, self.tune["uvw_fregs"], self.vout):
+        # (what the accumulators, the X rows and the rest leave for weight slices, at least two 64-channel slices)
+        limit = lambda vo, sub: max(32, self.tune["uvw_fregs"] - (4 * self.vout[vo].d + xrows + 64))
+        for ker in self._merge(_groups(self.vpaths, "vo", len(self.vout), "forward", limit), cost,
+                               self.tune["uvw_fregs"], self.vout):
             vo0, order0, _ = ker[0]
             if not order0 and self.accumulate:
                 continue  # nothing to add to a piece no path writes
@@ -661,7 +684,12 @@ class MfmaEmitter:
         fixed = lambda ker: (sum(8 * self.vin[g[0]].d for g in ker) + 4 * low.L2
                              + 6 * max(self.vout[vp.vo].d for g in ker for vp in g[1]) + 48)
         cost = lambda ker: sum(4 * c16(vp.Wn) for g in ker for vp in g[1]) + fixed(ker)
-        dx_kernels = self._merge(_groups(self.vpaths, "vi", len(self.vin)), cost, self.tune["uvw_xregs"], self.vin)
+        # (a slice of the kernel may live in LDS instead: 16 registers' worth; more of them, which the kernels
+        # below still allow, cost more in operand traffic than a kernel more)
+        limit = lambda vi, sub: max(32, self.tune["uvw_regs"] + 16 - (
+            8 * self.vin[vi].d + 4 * low.L2 + 6 * max(self.vout[vp.vo].d for vp in sub) + 48))
+        dx_kernels = self._merge(_groups(self.vpaths, "vi", len(self.vin), "dx", limit), cost, self.tune["uvw_xregs"],
+                                 self.vin)
         for ker in (dx_kernels if "dx" in parts else []):
             vi0, paths0, _ = ker[0]
             if not paths0 and self.accumulate:
@@ -781,7 +809,8 @@ class MfmaEmitter:
         # a kernel that would not fit the 160 KB of LDS with its pieces merged stays split (the register estimate
         # is replaced by one beyond any limit)
         cost = lambda ker: regs(ker) if dw_lds(ker, 1) <= LDS_BUDGET else 1 << 30
-        groups = [g for g in _groups(self.vpaths, "vo", len(self.vout)) if g[1]]
+        limit = lambda vo, sub: max(32, self.tune["uvw_wregs"] - (xrows + 4 * c16(self.vout[vo].mul) + 64))
+        groups = [g for g in _groups(self.vpaths, "vo", len(self.vout), "dw", limit) if g[1]]
         for ker in self._merge(groups, cost, self.tune["uvw_wregs"], self.vout):
             # pieces that share a kernel must be neighbours in the row: one dZ tile covers their columns
             pieces = [self.vout[vo] for vo, _, _ in ker]

@@ -152,6 +152,9 @@ MFMA = [
     ("mfma-pad-mid-f64", lambda: _f64(_fc_shared("40x0e+30x1o", "1x0e+1x1o", "50x0e+20x1o+10x2e")), 35),
     ("mfma-pad-wide", lambda: _fc_shared("100x0e+70x1o", "1x0e+1x1o", "33x0e+20x1o"), 50),
     ("mfma-mul3-f64", lambda: _f64(_fc_shared("64x0e+64x1o", "3x0e+2x1o", "64x0e+64x1o")), 33),
+    ("mfma-64-l3", lambda: _fc_shared("64x0e+64x1o+64x2e+64x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+64x1o+64x2e+64x3o"), 35),
+    ("mfma-50-l3-f64", lambda: _f64(_fc_shared("50x0e+50x1o+50x2e+50x3o", "1x0e+1x1o+1x2e+1x3o",
+                                               "50x0e+50x1o+50x2e+50x3o")), 33),
     ("mfma-mul2-pad", lambda: _fc_shared("40x0e+30x1o", "2x0e+1x1o", "25x0e+10x1o+5x2e"), 50),
     ("mfma-gaps", lambda: oeq.TPProblem(
         "32x0e+16x1o+32x2e", "1x0e+1x1o", "32x0e+16x1o+48x2e+16x1e",

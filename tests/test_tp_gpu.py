@@ -149,6 +149,13 @@ CASES = [
         [(0, 0, 0, "uvw", True), (0, 1, 1, "uvw", True, 0.7), (1, 1, 0, "uvw", True), (1, 2, 1, "uvw", True),
          (1, 0, 1, "uvw", True), (0, 2, 2, "uvw", True)],
         shared_weights=True, internal_weights=False, label="mfma-mul2-mixed"), 50),
+    # irreps fed by more paths than one kernel holds weight slices for (seven 64-channel paths into l = 3; six per
+    # irrep with both parities): the group of sub-paths is cut into parts, later parts add to the first one's rows
+    ("mfma-64-l3", lambda: _fc_shared("64x0e+64x1o+64x2e+64x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+64x1o+64x2e+64x3o"), 40),
+    ("mfma-50-l3-f64", lambda: _as_f64(_fc_shared("50x0e+50x1o+50x2e+50x3o", "1x0e+1x1o+1x2e+1x3o",
+                                                   "50x0e+50x1o+50x2e+50x3o")), 35),
+    ("mfma-64-l2-both-parities", lambda: _fc_shared("64x0e+64x0o+64x1e+64x1o+64x2e+64x2o", "1x0e+1x1o+1x2e",
+                                                    "64x0e+64x0o+64x1e+64x1o+64x2e+64x2o"), 40),
     ("mfma-pad-l3", lambda: oeq.TPProblem(
         "14x1o+90x3o", "1x2o", "75x3e+11x1e", [(0, 0, 0, "uvw", True), (1, 0, 0, "uvw", True, 0.6), (1, 0, 1, "uvw", True)],
         shared_weights=True, internal_weights=False, label="mfma-pad-l3"), 40),
@@ -156,7 +163,8 @@ CASES = [
 MFMA_CASES = {"cfg4-shared", "cfg4-f64", "mfma-32", "mfma-128", "mfma-mixed", "mfma-gaps", "mfma-128-f64",
               "mfma-mixed-f64", "mfma-l3-f64", "mfma-l3-wide-f64", "mfma-pad-diffdock", "mfma-pad-mid",
               "mfma-pad-mid-f64", "mfma-pad-wide", "mfma-pad-wide-f64", "mfma-pad-gaps", "mfma-pad-l3", "mfma-mul2-pad",
-              "mfma-mul3-f64", "mfma-mul2-mixed"}
+              "mfma-mul3-f64", "mfma-mul2-mixed", "mfma-64-l3", "mfma-50-l3-f64",
+              "mfma-64-l2-both-parities"}
 # shared weights off the matrix cores (second operand of more than 32 values): the general kernels' weight gradient
 # in an LDS copy per wave and in partial rows in global memory
 CASES += [
