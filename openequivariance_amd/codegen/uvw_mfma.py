@@ -198,7 +198,7 @@ def _groups(vpaths: List[VPath], side: str, n_blocks: int, which: str, limit=Non
 def supported(low: Lowered) -> bool:
     if low.mode != "uvw" or not low.shared_weights or low.ctype not in ("float", "double") or low.ir_mul:
         return False
-    if low.L3 > 1152 or low.L2 > 32:
+    if low.L2 > 32:
         return False
     # the dX kernels keep a whole 16-row dZ tile in LDS beside the Y rows and the partial dY of the four waves
     # (fp64: rows of up to about 1 000 elements)
@@ -344,22 +344,26 @@ class MfmaEmitter:
             # each wave moves its 4 rows, 64 lanes x 16 bytes at a time: every address is affine in the lane id
             rpw, nc4 = RT // WAVES, ncols // VW
             J = (nc4 + 63) // 64
-            s.open("")
-            s(f"oeq_vec16 gv[{rpw * J}];")
-            for phase in ("load", "store"):
-                for rr in range(rpw):
-                    for j in range(J):
-                        part = (j + 1) * 64 > nc4
-                        c4 = f"(lane + {64 * j})"
-                        r = f"(wave * {rpw} + {rr})"
-                        if phase == "load":
-                            cond = f"row0 + {r} < num_batch" + (f" && {c4} < {nc4}" if part else "")
-                            s(f"gv[{rr * J + j}] = ({cond}) ? *(const oeq_vec16*)(L3_grad + (row0 + {r}) * {low.L3} + "
-                              f"{col0} + {VW} * {c4}) : oeq_vec16(T(0));")
-                        else:
-                            guard = f"if ({c4} < {nc4}) " if part else ""
-                            s(f"{guard}*(oeq_vec16*)&s_g[{r}][{dst0} + {VW} * {c4}] = gv[{rr * J + j}];")
-            s.close()
+            # (at most five vectors per row in flight: 80 registers; longer rows in several rounds)
+            for j0 in range(0, J, 5):
+                js = range(j0, min(J, j0 + 5))
+                s.open("")
+                s(f"oeq_vec16 gv[{rpw * len(js)}];")
+                for phase in ("load", "store"):
+                    for rr in range(rpw):
+                        for j in js:
+                            part = (j + 1) * 64 > nc4
+                            c4 = f"(lane + {64 * j})"
+                            r = f"(wave * {rpw} + {rr})"
+                            slot = rr * len(js) + j - j0
+                            if phase == "load":
+                                cond = f"row0 + {r} < num_batch" + (f" && {c4} < {nc4}" if part else "")
+                                s(f"gv[{slot}] = ({cond}) ? *(const oeq_vec16*)(L3_grad + (row0 + {r}) * {low.L3} + "
+                                  f"{col0} + {VW} * {c4}) : oeq_vec16(T(0));")
+                            else:
+                                guard = f"if ({c4} < {nc4}) " if part else ""
+                                s(f"{guard}*(oeq_vec16*)&s_g[{r}][{dst0} + {VW} * {c4}] = gv[{slot}];")
+                s.close()
         else:
             s.open(f"for (int t = tid; t < {RT * ncols}; t += {nthreads})")
             s(f"const int r = t / {ncols}, c = t % {ncols};")
