@@ -204,6 +204,15 @@ def supported(low: Lowered) -> bool:
     # (fp64: rows of up to about 1 000 elements)
     if (RT * (low.L3 + 36) + (1 + WAVES) * RT * low.L2) * low.elem_size > LDS_BUDGET:
         return False
+    # ... the forward kernels two copies of the T tile of an output piece (fp64: l <= 4), the dW kernels one copy
+    # beside the piece's dZ columns
+    tl = piece_of(low)
+    for p in low.paths:
+        o = low.out[p.io]
+        cols = min(o.mul, tl) * o.d
+        if max(2 * o.d * tl * TPAD + 2 * RT * low.L2,
+               RT * (cols + 36) + o.d * tl * TPAD + 2 * RT * low.L2) * low.elem_size > LDS_BUDGET:
+            return False
     vin, vout, vpaths = _split(low)
     # Multiplicities that are no multiples of 16 run on tiles padded with zero weights. Where nearly all of a
     # tile would be padding the general kernels are the better choice: ``uvw_mfma_fill`` = least share (percent)
