@@ -105,3 +105,29 @@ def test_blocks_wider_than_1024_channels_fail_with_a_message(mul):
         build_tp_module(problem)
     with pytest.raises(ValueError, match="at most 1024 channels"):
         build_conv_module(problem, True)
+
+
+def test_matrix_core_path_accepts_only_what_its_kernels_can_hold():
+    """Every shared-weight problem the matrix-core path accepts generates (its LDS checks raise otherwise): single
+    paths up to l = 7 in both precisions. fp64 outputs with l >= 5 exceed the LDS and must be refused, not raise."""
+    import numpy as np
+
+    import openequivariance_amd as oeq
+    from openequivariance_amd._torch.tensor_product import build_tp_module
+    from openequivariance_amd.codegen import uvw_mfma
+    from openequivariance_amd.codegen.lower import lower
+    accepted = refused_f64 = 0
+    for l1 in (0, 3, 5, 7):
+        for l2 in (0, 1, 3):
+            for l3 in range(abs(l1 - l2), min(l1 + l2, 7) + 1):
+                for dt in (np.float32, np.float64):
+                    p = oeq.TPProblem(f"64x{l1}e", f"1x{l2}e", f"40x{l3}e", [(0, 0, 0, "uvw", True)], shared_weights=True,
+                                      internal_weights=False, irrep_dtype=dt, weight_dtype=dt)
+                    if uvw_mfma.supported(lower(p)):
+                        src, dims, descs = build_tp_module(p)
+                        assert "oeq_mfma" in src
+                        accepted += 1
+                    else:
+                        assert dt == np.float64 and l3 >= 5, (l1, l2, l3, dt)
+                        refused_f64 += 1
+    assert accepted > 40 and refused_f64 > 5
