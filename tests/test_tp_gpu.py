@@ -152,6 +152,11 @@ CASES = [
     # irreps fed by more paths than one kernel holds weight slices for (seven 64-channel paths into l = 3; six per
     # irrep with both parities): the group of sub-paths is cut into parts, later parts add to the first one's rows
     ("mfma-64-l3", lambda: _fc_shared("64x0e+64x1o+64x2e+64x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+64x1o+64x2e+64x3o"), 40),
+    # l = 7 on either side (15 components per channel)
+    ("mfma-l7", lambda: oeq.TPProblem("64x7e", "1x1e", "40x7e", [(0, 0, 0, "uvw", True)], shared_weights=True,
+                                      internal_weights=False, label="mfma-l7"), 37),
+    ("mfma-l7-in-f64", lambda: _as_f64(oeq.TPProblem("20x7e", "1x4e", "70x3e", [(0, 0, 0, "uvw", True)],
+                                                    shared_weights=True, internal_weights=False, label="mfma-l7-in")), 37),
     # (rows of 2 048 values: the dZ tile of the dX kernels is staged in two rounds)
     ("mfma-128-l3", lambda: _fc_shared("128x0e+128x1o+128x2e+128x3o", "1x0e+1x1o+1x2e+1x3o",
                                        "128x0e+128x1o+128x2e+128x3o"), 21),
@@ -167,7 +172,7 @@ MFMA_CASES = {"cfg4-shared", "cfg4-f64", "mfma-32", "mfma-128", "mfma-mixed", "m
               "mfma-mixed-f64", "mfma-l3-f64", "mfma-l3-wide-f64", "mfma-pad-diffdock", "mfma-pad-mid",
               "mfma-pad-mid-f64", "mfma-pad-wide", "mfma-pad-wide-f64", "mfma-pad-gaps", "mfma-pad-l3", "mfma-mul2-pad",
               "mfma-mul3-f64", "mfma-mul2-mixed", "mfma-64-l3", "mfma-50-l3-f64",
-              "mfma-64-l2-both-parities", "mfma-128-l3"}
+              "mfma-64-l2-both-parities", "mfma-128-l3", "mfma-l7", "mfma-l7-in-f64"}
 # shared weights off the matrix cores (second operand of more than 32 values): the general kernels' weight gradient
 # in an LDS copy per wave and in partial rows in global memory
 CASES += [
