@@ -123,7 +123,7 @@ class VPath:
     def tag(self, side: str) -> str:
         """Names the group of sub-paths a kernel takes from the other side of a piece on ``side``."""
         k = self.ub if side == "vo" else self.wb
-        return f"{k}" + (f"v{self.v}" if self.v else "") + (f"p{self.part}" if self.part else "")
+        return f"{k}" + (f"p{self.part}" if self.part else "")
 
 
 def _pieces(blocks, piece: int) -> List[VBlock]:
@@ -166,19 +166,19 @@ def _slice_regs(vp: VPath, which: str) -> int:
 
 def _groups(vpaths: List[VPath], side: str, n_blocks: int, which: str, limit=None):
     """Kernels of one pass (``which``: 'forward', 'dx' or 'dw'): for every piece on ``side`` ('vo' or 'vi') its
-    sub-paths grouped by the piece index on the other side and the channel of the second operand, a group cut into
+    sub-paths grouped by the piece index on the other side (all channels of the second operand), a group cut into
     parts whose weight slices fit ``limit(piece, sub-paths)`` registers. Returns [(piece, [sub-paths], first
     kernel of that piece?)]; a piece without paths gets one entry with an empty list."""
     other = "ub" if side == "vo" else "wb"
     out = []
     for b in range(n_blocks):
         mine = [vp for vp in vpaths if getattr(vp, side) == b]
-        keys = sorted({(getattr(vp, other), vp.v) for vp in mine})
+        keys = sorted({getattr(vp, other) for vp in mine})
         if not keys:
             out.append((b, [], True))
         for n, key in enumerate(keys):
             parts, room = [], 0
-            sel = [q for q in mine if (getattr(q, other), q.v) == key]
+            sel = sorted((q for q in mine if getattr(q, other) == key), key=lambda q: (q.v, q.index))
             budget = min(SLICE_REGS[which], limit(b, sel)) if limit else SLICE_REGS[which]
             total = sum(_slice_regs(vp, which) for vp in sel)
             if total > budget:  # parts of about equal size
