@@ -10,8 +10,9 @@ Two kernel families are generated:
   input channels ``u`` for the CG contraction and for everything in the backward
   pass; the forward channel mix runs with lanes = output channels ``w`` and reads
   the per-``u`` intermediates back from LDS as broadcasts;
-* for shared weights with 64-wide channel blocks, an MFMA kernel (see
-  ``uvw_mfma.py``) that batches rows so that the channel mix is a dense GEMM.
+* for shared weights, MFMA kernels (see ``uvw_mfma.py``) that batch rows so that the
+  channel mix is a dense GEMM; they take every problem except those whose padded
+  16-channel tiles would be mostly zeros or whose tiles exceed the LDS.
 
 The general family also carries the second-order pair ``double_backward_A`` / ``double_backward_B`` (the
 reference's kernels of that name, templates/loop_unroll_batch.cuh:148-317 and
