@@ -222,7 +222,7 @@ def supported(low: Lowered) -> bool:
     from .uvu import tuning
     real = sum(vp.U * vp.Wn for vp in vpaths)
     padded = sum(16 * c16(vp.U) * 16 * c16(vp.Wn) for vp in vpaths)
-    if 100 * real < tuning(dict(uvw_mfma_fill=30))["uvw_mfma_fill"] * padded:
+    if 100 * real < tuning(dict(uvw_mfma_fill=25))["uvw_mfma_fill"] * padded:
         return False
     return True
 
