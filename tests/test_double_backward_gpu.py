@@ -230,6 +230,44 @@ def test_conv_fused_matches_composition(name, make, batch, det, monkeypatch):
     _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
 
 
+@pytest.mark.parametrize("det", [True, False], ids=["sorted", "grouped"])
+def test_unfused_convolution_second_order_matches_fused(det, monkeypatch):
+    """The unfused convolution (gathered rows, batch kernels, ordered sums; here selected by a knob for a problem
+    that also has fused kernels) runs its second-order pass as the batch kernel pair on the gathered rows of both
+    orders: same results as the fused kernels, in both edge-list modes."""
+    problem = P.diffdock_problems()[0]
+    gph = _graph()
+    n, E = gph.coords.shape[0], gph.nnz
+    rng = np.random.default_rng(8)
+    if det:
+        rows, cols, perm = gph.rows, gph.cols, gph.transpose_perm
+    else:
+        order = rng.permutation(E)
+        rows, cols, perm = gph.rows[order], gph.cols[order], np.zeros(0, np.int64)
+    tr, tc, tp = (torch.tensor(v, device="cuda") for v in (rows, cols, perm))
+    out = {}
+    for fuse in (1, 0):
+        monkeypatch.setenv("OEQ_AMD_TUNE", f"conv_fuse_uvw={fuse}")
+        conv = oeq.TensorProductConv(problem, deterministic=det)
+        e = ops.get_entry(conv.kid)
+        assert e.unfused == (fuse == 0) and e.kernels().has_double_backward()
+        if fuse:
+            x, a = (_rand(rng, (n, e.L1), np.float32) for _ in range(2))
+            y, b = (_rand(rng, (E, e.L2), np.float32) for _ in range(2))
+            w, c = (_rand(rng, (E, e.WN), np.float32) for _ in range(2))
+            g = _rand(rng, (n, e.L3), np.float32)
+        out[fuse] = ops.conv_double_backward(x, y, w, g, a, b, c, tr, tc, tp, conv.kid)
+    _check(("dx", "dy", "dw", "gg"), out[0], out[1], tol_of(problem))
+    # and through autograd, where the op is chosen by the same rule as for the fused kernels
+    monkeypatch.setenv("OEQ_AMD_TUNE", "conv_fuse_uvw=0")
+    conv = oeq.TensorProductConv(problem, deterministic=det)
+    tx, ty, tw, tg = (t.clone().requires_grad_(True) for t in (x, y, w, g))
+    z = conv(tx, ty, tw, tr, tc, tp if det else None)
+    first = torch.autograd.grad(z, (tx, ty, tw), tg, create_graph=True)
+    second = torch.autograd.grad(sum((p * q).sum() for p, q in zip((a, b, c), first)), (tx, ty, tw, tg))
+    _check(("dx", "dy", "dw", "gg"), second, out[1], tol_of(problem))
+
+
 # matrix-core problems: the convolution is unfused, its second-order pass the batch kernel pair on gathered rows
 MFMA_CONV = [c for c in MFMA if c[0] in ("cfg4", "mfma-mixed-f64", "mfma-pad-diffdock", "mfma-pad-wide")] + \
     [c for c in UVW if c[0] == "uvw-wide-mul2-shared"]
