@@ -362,16 +362,16 @@ class MfmaEmitter:
                     for rr in range(rpw):
                         for j in js:
                             part = (j + 1) * 64 > nc4
-                            c4 = f"(lane + {64 * j})"
+                            cv = f"(lane + {64 * j})"
                             r = f"(wave * {rpw} + {rr})"
                             slot = rr * len(js) + j - j0
                             if phase == "load":
-                                cond = f"row0 + {r} < num_batch" + (f" && {c4} < {nc4}" if part else "")
+                                cond = f"row0 + {r} < num_batch" + (f" && {cv} < {nc4}" if part else "")
                                 s(f"gv[{slot}] = ({cond}) ? *(const oeq_vec16*)(L3_grad + (row0 + {r}) * {low.L3} + "
-                                  f"{col0} + {VW} * {c4}) : oeq_vec16(T(0));")
+                                  f"{col0} + {VW} * {cv}) : oeq_vec16(T(0));")
                             else:
-                                guard = f"if ({c4} < {nc4}) " if part else ""
-                                s(f"{guard}*(oeq_vec16*)&s_g[{r}][{dst0} + {VW} * {c4}] = gv[{slot}];")
+                                guard = f"if ({cv} < {nc4}) " if part else ""
+                                s(f"{guard}*(oeq_vec16*)&s_g[{r}][{dst0} + {VW} * {cv}] = gv[{slot}];")
                 s.close()
         else:
             s.open(f"for (int t = tid; t < {RT * ncols}; t += {nthreads})")
