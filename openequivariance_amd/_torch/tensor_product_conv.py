@@ -27,8 +27,9 @@ from .utils import compute_units, oeq_to_torch_dtype, torch_to_oeq_dtype
 
 def fused(low) -> bool:
     """Whether the convolution of this problem runs as fused kernels: every 'uvu' problem, and the 'uvw'
-    problems outside the matrix-core path for shared weights (``OEQ_AMD_TUNE=conv_fuse_uvw=0`` sends those
-    through the unfused path, too)."""
+    problems except shared-weight ones that are faster through the matrix-core batch kernels
+    (``codegen/uvw.py: conv_supported``; ``OEQ_AMD_TUNE=conv_fuse_uvw=0`` sends every 'uvw' problem through the
+    unfused path)."""
     if low.mode == "uvu":
         return True
     from ..codegen import uvw

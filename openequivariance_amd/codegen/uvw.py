@@ -963,14 +963,19 @@ class UvwEmitter:
 
 
 def conv_supported(low: Lowered) -> bool:
-    """Problems the fused 'uvw' convolution kernels cover: per-edge weights, and shared weights whose channel mix
-    does not run on the matrix cores (those stay with the unfused path: gathered rows through the MFMA kernels)."""
+    """Problems the fused 'uvw' convolution kernels cover: per-edge weights, and shared weights unless the unfused
+    path (gathered rows through the MFMA kernels, ordered sums) is the faster one: problems the matrix-core path
+    takes with at least ``conv_mfma_min_weights`` weights. Below that the gathers and sums of the unfused path cost
+    more than the matrix cores save (12 000 nodes / 532 k edges, forward / backward, unfused MFMA against fused
+    general kernels: 256 weights 0.45 / 0.72 against 0.20 / 0.56 ms, 664 weights 0.72 / 1.49 against 0.70 / 0.82 ms,
+    2 190 weights 0.96 / 3.3 against 0.89 / 7.9 ms, 6 928 weights 0.87 / 1.6 against 1.16 / 11.7 ms)."""
     if low.mode != "uvw":
         return False
     if not low.shared_weights:
         return True
     from . import uvw_mfma
-    return not uvw_mfma.supported(low)
+    from .uvu import tuning
+    return not uvw_mfma.supported(low) or low.WN < tuning(dict(conv_mfma_min_weights=2048))["conv_mfma_min_weights"]
 
 
 def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kahan: bool = False):
