@@ -131,3 +131,46 @@ def test_matrix_core_path_accepts_only_what_its_kernels_can_hold():
                         assert dt == np.float64 and l3 >= 5, (l1, l2, l3, dt)
                         refused_f64 += 1
     assert accepted > 40 and refused_f64 > 5
+
+
+def test_matrix_core_kernel_plan_covers_every_sub_path_once():
+    """The kernels of each pass of the matrix-core path partition the sub-paths (piece of the input block x piece of
+    the output block x channel of the second operand): every sub-path in exactly one kernel, exactly one kernel per
+    piece that stores instead of adding, weight corners inside the path's weight block and disjoint, parts within
+    the register budget."""
+    import openequivariance_amd as oeq
+    from openequivariance_amd.codegen import uvw_mfma as M
+    from openequivariance_amd.codegen.lower import lower
+    sh3 = "1x0e+1x1o+1x2e+1x3o"
+    problems = [
+        P.config4_uvw_shared(),
+        P.FullyConnectedTPProblem("64x0e+64x1o+64x2e+64x3o", sh3, "64x0e+64x1o+64x2e+64x3o", shared_weights=True,
+                                  internal_weights=False),
+        P.FullyConnectedTPProblem("70x0e+20x1o", "2x0e+3x1o", "100x0e+33x1o", shared_weights=True, internal_weights=False),
+        P.FullyConnectedTPProblem("130x1o", "1x1o", "5x0e+17x1e+130x2e", shared_weights=True, internal_weights=False),
+    ]
+    for problem in problems:
+        low = lower(problem)
+        assert M.supported(low)
+        vin, vout, vpaths = M._split(low)
+        # the corners of a path tile its weight block
+        for p in low.paths:
+            U, V, W = low.in1[p.i1].mul, low.in2[p.i2].mul, low.out[p.io].mul
+            seen = set()
+            for vp in (q for q in vpaths if q.p is p):
+                assert vp.ld == V * W
+                for u in range(vp.U):
+                    for w in (0, vp.Wn - 1):
+                        at = vp.woff + u * vp.ld + w
+                        assert p.woff <= at < p.woff + U * V * W and at not in seen
+                        seen.add(at)
+            assert sum(q.U * q.Wn for q in vpaths if q.p is p) == U * V * W
+        for side, blocks, which in (("vo", vout, "forward"), ("vi", vin, "dx"), ("vo", vout, "dw")):
+            groups = M._groups(vpaths, side, len(blocks), which)
+            listed = [vp.index for _, sub, _ in groups for vp in sub]
+            assert sorted(listed) == list(range(len(vpaths)))
+            for b in range(len(blocks)):
+                mine = [g for g in groups if g[0] == b]
+                assert sum(1 for g in mine if g[2]) == 1 and mine[0][2]
+            for _, sub, _ in groups:
+                assert sum(M._slice_regs(vp, which) for vp in sub) <= M.SLICE_REGS[which]
