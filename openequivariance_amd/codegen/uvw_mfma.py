@@ -198,7 +198,7 @@ def _groups(vpaths: List[VPath], side: str, n_blocks: int, which: str, limit=Non
 def supported(low: Lowered) -> bool:
     if low.mode != "uvw" or not low.shared_weights or low.ctype not in ("float", "double") or low.ir_mul:
         return False
-    if low.L2 > 32:
+    if low.L2 > 64:  # (per-lane dY accumulators of the dX kernels: 4 rows x L2)
         return False
     # the dX kernels keep a whole 16-row dZ tile in LDS beside the Y rows and the partial dY of the four waves
     # (fp64: rows of up to about 1 000 elements)

@@ -72,16 +72,16 @@ CASES = [
     ("uvw-diffdock-f64", lambda: _as_f64(P.diffdock_problems()[1]), 30, 5),
     ("uvw-e3tools-conv", lambda: P.e3tools_problems()[0], 40, 6),
     ("uvw-shared", lambda: _fc(True), 40, 6),
-    # (second operands of more than 32 values keep a problem off the matrix cores: the general kernels' weight
+    # (second operands of more than 64 values keep a problem off the matrix cores: the general kernels' weight
     # gradient in an LDS copy per wave, with 20 and with 70 channels, and in partial rows in global memory)
     ("uvw-shared-lds", lambda: P.FullyConnectedTPProblem(
-        "20x0e+10x1o", "20x0e+5x1o", "12x0e+6x1o", shared_weights=True, internal_weights=False,
+        "20x0e+10x1o", "40x0e+10x1o", "12x0e+6x1o", shared_weights=True, internal_weights=False,
         label="uvw-shared-lds"), 40, 6),
     ("uvw-shared-lds-wide", lambda: P.FullyConnectedTPProblem(
-        "70x0e+3x1o", "20x0e+5x1o", "3x0e+2x1o", shared_weights=True, internal_weights=False,
+        "70x0e+3x1o", "1x0e+1x1o+1x2e+1x3o+1x4e+1x5o+1x6e+1x7o+1x8e", "3x0e+2x1o", shared_weights=True, internal_weights=False,
         label="uvw-shared-lds-wide"), 40, 6),
     ("uvw-shared-global-f64", lambda: _as_f64(P.FullyConnectedTPProblem(
-        "20x0e+10x1o", "20x0e+5x1o", "40x0e+20x1o", shared_weights=True, internal_weights=False,
+        "20x0e+10x1o", "40x0e+10x1o", "40x0e+20x1o", shared_weights=True, internal_weights=False,
         label="uvw-shared-global")), 30, 5),
     ("uvw-shared-mfma-mul2", lambda: P.FullyConnectedTPProblem(
         "40x0e+30x1o", "2x0e+1x1o", "25x0e+10x1o+5x2e", shared_weights=True, internal_weights=False,
@@ -177,7 +177,7 @@ def test_uvw_shared_weights_fused_matches_unfused(monkeypatch):
     bits on every run (the partial weight-gradient rows are summed in a fixed order), at a graph large enough
     for every wave of the bounded backward grid to see edges and at one where most waves see none."""
     from openequivariance_amd._torch import ops
-    problem = P.FullyConnectedTPProblem("20x0e+10x1o", "20x0e+5x1o", "12x0e+6x1o", shared_weights=True,
+    problem = P.FullyConnectedTPProblem("20x0e+10x1o", "40x0e+10x1o", "12x0e+6x1o", shared_weights=True,
                                         internal_weights=False, label="uvw-shared-lds")
     for n_nodes, deg in ((3000, 12), (20, 3)):
         coords, rows, cols = _graph(n_nodes, deg, seed=4)

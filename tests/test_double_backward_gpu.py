@@ -97,7 +97,7 @@ def _fc(shared, in2="1x0e+2x1o"):
 
 
 def _fc_general(out):
-    return P.FullyConnectedTPProblem("20x0e+10x1o", "20x0e+5x1o", out, shared_weights=True, internal_weights=False,
+    return P.FullyConnectedTPProblem("20x0e+10x1o", "40x0e+10x1o", out, shared_weights=True, internal_weights=False,
                                      label="general-fc-uvw")
 
 
@@ -124,7 +124,7 @@ UVW = [
     ("uvw-tetris-2-shared", lambda: P.tetris_poly_problems()[1], 65),
     ("uvw-wide-shared", lambda: _wide_fc(True), 600),
     ("uvw-wide-mul2-shared", lambda: _wide_fc(True, "2x0e+1x1o"), 300),
-    # off the matrix cores (second operand of more than 32 values): weight gradient in an LDS copy per wave, and in
+    # off the matrix cores (second operand of more than 64 values): weight gradient in an LDS copy per wave, and in
     # partial rows in global memory
     ("uvw-lds-shared", lambda: _fc_general("12x0e+6x1o"), 200),
     ("uvw-global-shared-f64", lambda: _f64(_fc_general("40x0e+20x1o")), 100),

@@ -152,6 +152,12 @@ CASES = [
     # irreps fed by more paths than one kernel holds weight slices for (seven 64-channel paths into l = 3; six per
     # irrep with both parities): the group of sub-paths is cut into parts, later parts add to the first one's rows
     ("mfma-64-l3", lambda: _fc_shared("64x0e+64x1o+64x2e+64x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+64x1o+64x2e+64x3o"), 40),
+    # second operands of 35 to 64 values (many channels; spherical harmonics up to l = 6 and 7)
+    ("mfma-in2-35", lambda: _fc_shared("20x0e+10x1o", "20x0e+5x1o", "12x0e+6x1o"), 45),
+    ("mfma-sh6-f64", lambda: _as_f64(_fc_shared("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e+1x3o+1x4e+1x5o+1x6e",
+                                                "64x0e+64x1o+64x2e")), 35),
+    ("mfma-sh7", lambda: _fc_shared("32x0e+32x1o+32x2e+32x3o", "1x0e+1x1o+1x2e+1x3o+1x4e+1x5o+1x6e+1x7o",
+                                    "32x0e+32x1o+32x2e+32x3o"), 35),
     # l = 7 on either side (15 components per channel)
     ("mfma-l7", lambda: oeq.TPProblem("64x7e", "1x1e", "40x7e", [(0, 0, 0, "uvw", True)], shared_weights=True,
                                       internal_weights=False, label="mfma-l7"), 37),
@@ -172,13 +178,14 @@ MFMA_CASES = {"cfg4-shared", "cfg4-f64", "mfma-32", "mfma-128", "mfma-mixed", "m
               "mfma-mixed-f64", "mfma-l3-f64", "mfma-l3-wide-f64", "mfma-pad-diffdock", "mfma-pad-mid",
               "mfma-pad-mid-f64", "mfma-pad-wide", "mfma-pad-wide-f64", "mfma-pad-gaps", "mfma-pad-l3", "mfma-mul2-pad",
               "mfma-mul3-f64", "mfma-mul2-mixed", "mfma-64-l3", "mfma-50-l3-f64",
-              "mfma-64-l2-both-parities", "mfma-128-l3", "mfma-l7", "mfma-l7-in-f64"}
-# shared weights off the matrix cores (second operand of more than 32 values): the general kernels' weight gradient
+              "mfma-64-l2-both-parities", "mfma-128-l3", "mfma-l7", "mfma-l7-in-f64", "mfma-in2-35",
+              "mfma-sh6-f64", "mfma-sh7"}
+# shared weights off the matrix cores (second operand of more than 64 values): the general kernels' weight gradient
 # in an LDS copy per wave and in partial rows in global memory
 CASES += [
-    ("uvw-shared-lds", lambda: _fc_shared("20x0e+10x1o", "20x0e+5x1o", "12x0e+6x1o"), 77),
-    ("uvw-shared-lds-wide", lambda: _fc_shared("70x0e+3x1o", "20x0e+5x1o", "3x0e+2x1o"), 77),
-    ("uvw-shared-global-f64", lambda: _as_f64(_fc_shared("20x0e+10x1o", "20x0e+5x1o", "40x0e+20x1o")), 41),
+    ("uvw-shared-lds", lambda: _fc_shared("20x0e+10x1o", "40x0e+10x1o", "12x0e+6x1o"), 77),
+    ("uvw-shared-lds-wide", lambda: _fc_shared("70x0e+3x1o", "1x0e+1x1o+1x2e+1x3o+1x4e+1x5o+1x6e+1x7o+1x8e", "3x0e+2x1o"), 77),
+    ("uvw-shared-global-f64", lambda: _as_f64(_fc_shared("20x0e+10x1o", "40x0e+10x1o", "40x0e+20x1o")), 41),
 ]
 
 
