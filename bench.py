@@ -475,6 +475,41 @@ def main():
         }
         del Ys, trs, tcs, tps
 
+        # The same graph plus one hub: node 0 receives from and sends to 20 000 further nodes. Edge segments
+        # longer than dims["hub_limit"] edges are walked in chunks by different wave groups, so the step should
+        # cost what its 2.5 % more edges cost, not the hub's degree times one edge's latency.
+        rng = np.random.default_rng(1)
+        spokes = rng.choice(np.arange(1, N), size=20000, replace=False).astype(np.int64)
+        spokes = spokes[~np.isin(spokes, cols[rows == 0])]  # keep the edge list free of duplicates
+        rows_h = np.concatenate([rows, np.zeros(len(spokes), dtype=np.int64), spokes])
+        cols_h = np.concatenate([cols, spokes, np.zeros(len(spokes), dtype=np.int64)])
+        dirs = rng.normal(size=(len(spokes), 3))
+        vec_h = np.concatenate([vec, dirs, -dirs])
+        gh = CoordGraph(coords, rows_h, cols_h, "periodic-radius-plus-hub")
+        Eh = gh.nnz
+        Yh = torch.tensor(spherical_harmonics(3, vec_h).astype(np.float32)[gh.order], device=dev)
+        Wh = torch.randn(Eh, WN, device=dev, generator=gen)
+        trh, tch, tph = (torch.tensor(a, device=dev) for a in (gh.rows, gh.cols, gh.transpose_perm))
+
+        def step_hub():
+            ops.conv_forward(X, Yh, Wh, trh, tch, tph, kid)
+            ops.conv_backward(X, Yh, Wh, G, trh, tch, tph, kid)
+
+        ms_hub = time_steps(step_hub, max(3, args.steps // 2), 2)
+        ks.timing_enable(True)
+        step_hub()
+        torch.cuda.synchronize()
+        hub_split = {name: ks.timing_collect(role)[0] for name, role in
+                     (("forward", rt.ROLE_CONV_FORWARD), ("fixup_forward", rt.ROLE_CONV_FIXUP_FORWARD),
+                      ("backward", rt.ROLE_CONV_BACKWARD), ("fixup_backward", rt.ROLE_CONV_FIXUP_BACKWARD))}
+        ks.timing_enable(False)
+        modes["deterministic_plus_hub_of_20000_edges"] = {
+            "ms_per_step": ms_hub, "edges": Eh, "edges_per_s": Eh / (ms_hub * 1e-3),
+            "ms_per_step_relative_to_config5": ms_hub / ms_det, "hub_limit": ks.dims.get("hub_limit", 0),
+            "kernel_ms": hub_split,
+        }
+        del Yh, Wh, trh, tch, tph
+
     # Second-order kernels at the same shape (the backward of the backward, as in force training):
     # the fused pair against the composition of three forward and three backward calls.
     if (not args.no_extras or args.with_double) and ks.has_double_backward():

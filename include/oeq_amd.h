@@ -82,7 +82,10 @@ typedef enum {
     OEQ_ROLE_DOUBLE_BACKWARD_A = 13,/* second order: gradient w.r.t. the output gradient (forward-shaped) */
     OEQ_ROLE_DOUBLE_BACKWARD_B = 14,/* second order: gradients w.r.t. X, Y, W (backward-shaped) */
     OEQ_ROLE_ORDER_HOP = 15,        /* convolution walk order: one hop of the node clustering */
-    OEQ_ROLE_COUNT = 16
+    OEQ_ROLE_HUB_COUNT = 16,        /* long edge segments cut into chunks: extra walk positions per node, */
+    OEQ_ROLE_HUB_FILL = 17,         /*   and the list of those positions */
+    OEQ_ROLE_CONV_FIXUP_FORWARD = 18,/* adds the rows written by the extra chunks to their nodes' rows, in chunk order */
+    OEQ_ROLE_COUNT = 19
 } oeq_role;
 
 /* How the convolution kernels of a set find the edges of a node (oeq_problem_dims.deterministic):
@@ -135,6 +138,15 @@ typedef struct {
                                    highest-priority node within this many edges and walked cluster by cluster,
                                    so that nodes sharing senders run side by side and the gathered sender rows
                                    are served by the L2; 0 = nodes are walked by index */
+    int32_t hub_limit;          /* conv, walk modes: > 0 = a node with more edges than this is walked in chunks of
+                                   this many edges by different wave groups (the first chunk at the node's own walk
+                                   position, the others at extra positions listed in the index), so that the time
+                                   of a call does not grow with the largest degree: forward-shaped kernels write
+                                   the extra chunks to scratch rows that fixup_forward adds to the node's row in
+                                   chunk order; 0 = every segment is walked whole. Plays the role of the
+                                   reference's equal edge ranges per warp with fixup_forward
+                                   (templates/loop_unroll_conv_det.cuh:34-66, 96-179,
+                                   core/LoopUnrollConv.py:142-185). */
 } oeq_problem_dims;
 
 int oeq_kernels_create(const void* code, size_t code_size,
@@ -178,6 +190,7 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz,
                      const void* L1_in, const void* L2_in, const void* W,
                      void* L3_out, const int64_t* rows, const int64_t* cols,
                      void* workspace, size_t workspace_bytes, void* stream);
+/* index + scratch (the rows of extra chunks, see oeq_problem_dims.hub_limit; sized for nnz / hub_limit of them) */
 size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
 
 /* oeq_conv_forward for callers that cannot allocate: code under HIP graph capture, tight serving loops,
@@ -190,7 +203,9 @@ size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count
  * oeq_static_scratch_bytes() (32 MiB: e.g. 1.9 M edges over 50 000 nodes with deterministic=False, 4 M
  * nodes in deterministic mode); larger calls are refused with OEQ_ERR_INVALID. Every call on a GPU uses
  * that GPU's one array: calls that overlap in time on one GPU (two streams, two threads) race and must be
- * serialised by the caller. Per-kernel timing (oeq_kernel_timing_enable) is not applied to these calls. */
+ * serialised by the caller. Long edge segments are walked whole here (oeq_problem_dims.hub_limit is not
+ * applied: the rows of extra chunks would need scratch of their own), so the sum over a hub node's edges is
+ * formed in one pass and can differ in the last bits from oeq_conv_forward's. Per-kernel timing (oeq_kernel_timing_enable) is not applied to these calls. */
 int oeq_conv_forward_static(oeq_kernels* k, int64_t node_count, int64_t nnz,
                             const void* L1_in, const void* L2_in, const void* W,
                             void* L3_out, const int64_t* rows, const int64_t* cols,
@@ -220,7 +235,7 @@ size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_coun
  * convolutions over one edge list (forward and backward of every layer of a model) builds it once with
  * oeq_conv_index_build and passes it to the *_indexed variants, which take the same operands, `index` /
  * `index_bytes` / `index_sender_side` as given to the build, and a scratch buffer of
- * oeq_conv_backward_scratch_bytes() / oeq_conv_double_backward_scratch_bytes() (forward needs none).
+ * oeq_conv_forward_scratch_bytes() / oeq_conv_backward_scratch_bytes() / oeq_conv_double_backward_scratch_bytes().
  * The reference keeps the corresponding state (its workspace tensor and, for the deterministic mode, the
  * caller's transpose_perm) in the Python module (_torch/TensorProductConv.py:187-193). The index is read-only
  * after the build, so calls on several streams may share it once the build has completed; it is tied to the
@@ -233,7 +248,9 @@ int oeq_conv_index_build(oeq_kernels* k, int64_t node_count, int64_t nnz,
 int oeq_conv_forward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz,
                              const void* L1_in, const void* L2_in, const void* W, void* L3_out,
                              const int64_t* rows, const int64_t* cols,
-                             const void* index, size_t index_bytes, int index_sender_side, void* stream);
+                             const void* index, size_t index_bytes, int index_sender_side,
+                             void* scratch, size_t scratch_bytes, void* stream);
+size_t oeq_conv_forward_scratch_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz);
 int oeq_conv_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz,
                               const void* L1_in, void* L1_grad, const void* L2_in, void* L2_grad,
                               const void* W, void* W_grad, const void* L3_grad,

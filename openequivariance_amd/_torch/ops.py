@@ -354,6 +354,17 @@ def clear_index_cache():
         _index_cache.clear()
 
 
+def _version_of(t: torch.Tensor) -> Optional[int]:
+    """Version counter of a tensor, None where there is none (tensors made under
+    ``torch.inference_mode()`` do not track one: reading it raises)."""
+    if t.is_inference():
+        return None
+    try:
+        return t._version
+    except RuntimeError:
+        return None
+
+
 def _conv_index(ks, nodes: int, nnz: int, r: torch.Tensor, c: torch.Tensor, p: Optional[torch.Tensor],
                 need_sender_side: bool):
     """(index tensor, sender_side flag) for the edge list; built now unless a valid one is cached."""
@@ -363,10 +374,14 @@ def _conv_index(ks, nodes: int, nnz: int, r: torch.Tensor, c: torch.Tensor, p: O
     # the sender side is cheap to add when the caller brings the sender-major permutation, costly when the
     # library has to group the edges by sender itself: then only the calls that need it build it
     sender_side = need_sender_side or (not grouped and p is not None and p.numel() == nnz)
-    key = (dims["deterministic"], dims.get("order_hops", 0), nodes, nnz, r.data_ptr(), c.data_ptr(),
+    key = (dims["deterministic"], dims.get("order_hops", 0), dims.get("hub_limit", 0), nodes, nnz, r.data_ptr(),
+           c.data_ptr(),
            p.data_ptr() if (p is not None and not grouped) else 0, stream, r.device.index)
-    versions = (r._version, c._version, p._version if (p is not None and not grouped) else 0)
-    caching = INDEX_CACHE_ENTRIES > 0 and not torch.cuda.is_current_stream_capturing()
+    versions = (_version_of(r), _version_of(c), _version_of(p) if (p is not None and not grouped) else 0)
+    # an edge tensor without a version counter could be rewritten unnoticed: such a call builds its index
+    # and keeps nothing
+    caching = (INDEX_CACHE_ENTRIES > 0 and not torch.cuda.is_current_stream_capturing()
+               and None not in versions)
     if caching:
         with _index_cache_lock:
             for i, ent in enumerate(_index_cache):
@@ -463,8 +478,11 @@ def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows
             # by sender as well, both are built now, so that one index serves the whole step
             both = ks.dims["deterministic"] == rt.CONV_GROUPED and ks.dims.get("dx_mode", 0) != rt.DX_ATOMIC
             index, side = _conv_index(ks, nodes, nnz, r, c, perm, both)
+            nb = ks.conv_forward_scratch_bytes(nodes, nnz)
+            ws = torch.empty(max(nb, 1), dtype=torch.uint8, device=x.device)
             ks.conv_forward_indexed(nodes, nnz, x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), r.data_ptr(),
-                                    c.data_ptr(), index.data_ptr(), index.numel(), side, _stream())
+                                    c.data_ptr(), index.data_ptr(), index.numel(), side, ws.data_ptr() if nb else 0, nb,
+                                    _stream())
     return out
 
 

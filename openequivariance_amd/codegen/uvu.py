@@ -1072,21 +1072,54 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             return 1
         return 0
 
+    # Trailing parameters of every kernel that walks receivers: the table of long edge segments cut into
+    # chunks (see _node_loop_open). Forward-shaped kernels also take the rows that the extra chunks write.
+    HUB_PARAMS = (", const i64* __restrict__ hubptr, const i64* __restrict__ hubnode, i64 hub_limit, "
+                  "i64 hub_units")
+    HUB_ROWS_PARAM = ", T* __restrict__ hub_rows"
+
     def _node_loop_open(self, s: Src, G: int, xcd: int):
-        """One wave group per receiver node. Workgroups are handed to the XCDs
-        round-robin; with ``xcd`` > 1 (grid a multiple of it) block ids are remapped
-        so that each XCD walks one contiguous range of nodes and neighbouring
-        receivers share their senders' rows through that XCD's L2."""
+        """One wave group per walk position. A position is a receiver node with its edge segment, or, for
+        a node with more than ``hub_limit`` edges, one chunk of that many edges: the first chunk is the
+        node's own position, the others are listed in ``hubnode`` (``hubptr[v]`` = first extra position of
+        node v, ``hubptr[node_count]`` = their number) and take the first ``hub_units`` positions of the
+        grid, so that a hub's chunks start early and run side by side instead of one wave walking tens of
+        thousands of edges (the role of the reference's fixup_forward scheme,
+        templates/loop_unroll_conv_det.cuh:34-66, 96-179, which cuts the edge list into equal ranges).
+        Leaves ``node``, ``e0``, ``e1`` and ``hubpos`` (the extra position, -1 for a node's own) in scope.
+        Workgroups are handed to the XCDs round-robin; with ``xcd`` > 1 (grid a multiple of it, and so is
+        the number of blocks the extra positions take) block ids are remapped so that each XCD walks one
+        contiguous range of nodes and neighbouring receivers share their senders' rows through that
+        XCD's L2."""
         # ``order`` (may be NULL) lists the nodes in the order in which they are to be walked: nodes that
         # share senders next to each other, so that the blocks resident on one XCD gather from a small set
-        # of sender rows (the library derives it from the graph at every call).
+        # of sender rows (the library derives it from the graph at every index build).
+        s("const i64 walk_end = hub_units + node_count;")
         if xcd > 1:
-            s(f"const i64 vper = (i64)gridDim.x / {xcd};")
-            s(f"const i64 vblk = ((i64)blockIdx.x % {xcd}) * vper + (i64)blockIdx.x / {xcd};")
-            s.open(f"for (i64 vnode = vblk * {G} + g; vnode < node_count; vnode += node_count + 1)")
+            s(f"const i64 hub_blocks = hub_units / {G};")
+            s(f"const i64 vper = ((i64)gridDim.x - hub_blocks) / {xcd};")
+            s(f"const i64 nblk = (i64)blockIdx.x - hub_blocks;")
+            s(f"const i64 vblk = (nblk % {xcd}) * vper + nblk / {xcd};")
+            s(f"const i64 wpos0 = (nblk < 0 ? (i64)blockIdx.x : hub_blocks + vblk) * {G} + g;")
+            s.open("for (i64 wpos = wpos0; wpos < walk_end; wpos += walk_end + 1)")
         else:
-            s.open(f"for (i64 vnode = (i64)blockIdx.x * {G} + g; vnode < node_count; vnode += (i64)gridDim.x * {G})")
-        s("const i64 node = order ? order[vnode] : vnode;")
+            s.open(f"for (i64 wpos = (i64)blockIdx.x * {G} + g; wpos < walk_end; wpos += (i64)gridDim.x * {G})")
+        s("i64 node, e0, e1, hubpos = -1;")
+        s.open("if (wpos < hub_units)")
+        s("if (wpos >= hubptr[node_count]) continue;")
+        s("hubpos = wpos;")
+        s("node = oeq_idx(hubnode[wpos], node_count);")
+        s("e0 = oeq_pos(rowptr[node] + (wpos - hubptr[node] + 1) * hub_limit, nnz);")
+        s("e1 = oeq_pos(rowptr[node + 1], nnz);")
+        s("if (e1 - e0 > hub_limit) e1 = e0 + hub_limit;")
+        s.close()
+        s.open("else")
+        s("const i64 vnode = wpos - hub_units;")
+        s("node = order ? order[vnode] : vnode;")
+        s("e0 = oeq_pos(rowptr[node], nnz);")
+        s("e1 = oeq_pos(rowptr[node + 1], nnz);")
+        s("if (hub_limit > 0 && e1 - e0 > hub_limit) e1 = e0 + hub_limit;")
+        s.close()
 
     def emit_conv_forward(self, s: Src, G: int, deterministic: bool, pipelined: bool, waves_per_eu: int = 0,
                           xcd: int = 1, tr_atomics: bool = True):
@@ -1102,7 +1135,8 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void forward(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
             "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-            "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order)"
+            f"const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order"
+            f"{self.HUB_PARAMS}{self.HUB_ROWS_PARAM})"
         )
         self._lane_prologue(s, segw)
         if self.use_q:
@@ -1156,8 +1190,7 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
 
         if deterministic:
             self._node_loop_open(s, G, xcd)
-            s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
-            s(f"T* zrow = L3_out + node * {low.L3};")
+            s(f"T* zrow = hubpos >= 0 ? hub_rows + hubpos * {low.L3} : L3_out + node * {low.L3};")
             for si in range(len(self.segments)):
                 s.open(f"if (sg == {si % segw})" if segw > 1 else "")
 
@@ -1762,7 +1795,7 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
             "T* __restrict__ wpartial, const i64* __restrict__ colptr, const i64* __restrict__ sperm, "
-            "int* __restrict__ arrivals, const i64* __restrict__ order)"
+            f"int* __restrict__ arrivals, const i64* __restrict__ order{self.HUB_PARAMS})"
         )
         self._lane_prologue(s, SW)
         if self.use_q:
@@ -1773,7 +1806,6 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         s(f"__shared__ T s_dx[{SW}][{self.NCH}][{XW}][64];")
         s("E_t A;")
         self._node_loop_open(s, 1, xcd)
-        s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
         for si in range(SW):
             s.open(f"if (sg == {si})")
 
@@ -1882,7 +1914,7 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             "const T* __restrict__ L3_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
             "T* __restrict__ wpartial, const i64* __restrict__ colptr, const i64* __restrict__ sperm, "
-            "int* __restrict__ arrivals, const i64* __restrict__ order)"
+            f"int* __restrict__ arrivals, const i64* __restrict__ order{self.HUB_PARAMS})"
         )
         self._lane_prologue(s)
         if self.use_q:
@@ -1974,7 +2006,6 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
 
         if deterministic:
             self._node_loop_open(s, G, xcd)
-            s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
 
             def node_body():
                 if resident:
@@ -2105,7 +2136,8 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=0, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
                     dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fw=0, conv_pf=0,
-                    conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0, tp_forms=1))
+                    conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0, tp_forms=1,
+                    conv_hub=256))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -2242,6 +2274,10 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             (rt.ROLE_GROUP_SCATTER, "oeq_group_scatter", 256, 256 * 4, compute_units * 16),
             (rt.ROLE_GROUP_ORDER, "oeq_group_order", 256, 4, compute_units * 32),
             (rt.ROLE_ORDER_HOP, "oeq_order_hop", 256, 256, compute_units * 16),
+            # long edge segments in chunks: table of the extra walk positions, and the sum of their rows
+            (rt.ROLE_HUB_COUNT, "oeq_hub_count", 256, 256, compute_units * 16),
+            (rt.ROLE_HUB_FILL, "oeq_hub_fill", 256, 256, compute_units * 16),
+            (rt.ROLE_CONV_FIXUP_FORWARD, "fixup_forward", 256, 1, compute_units * 32),
         ]
     else:
         # edge ranges: about conv_epw consecutive edges per wave group
@@ -2250,8 +2286,12 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             (rt.ROLE_CONV_FORWARD, "forward", blk_f, G_f * em.R * epw, compute_units * 32),
             (rt.ROLE_CONV_BACKWARD, "backward", blk_b, G_b * em.R * epw, compute_units * 32),
         ]
+    # Segments longer than conv_hub edges are walked in chunks of that many (0: whole). Not with Kahan
+    # summation (its compensation terms belong to one running sum) nor where the second-order kernel B also
+    # forms kernel A's result.
+    hub_limit = max(0, t["conv_hub"]) if (walk and not kahan and not t["dd_merge"]) else 0
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
                 shared_weights=int(low.shared_weights), deterministic=mode,
                 wpartial_per_block=G_b if (walk and low.shared_weights) else 0, dx_mode=dx_mode,
-                n_chunks=em.NCH, order_hops=max(0, t["conv_hops"]) if walk else 0)
+                n_chunks=em.NCH, order_hops=max(0, t["conv_hops"]) if walk else 0, hub_limit=hub_limit)
     return s.text(), dims, descs

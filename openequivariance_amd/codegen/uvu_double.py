@@ -498,14 +498,13 @@ class DoubleEmitter(UvuEmitter):
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void double_backward_A(i64 node_count, '
             f"i64 nnz, {self._CONV_OPERANDS}T* __restrict__ L3_dgrad, const i64* __restrict__ rows, "
             "const i64* __restrict__ cols, const i64* __restrict__ rowptr, const i64* __restrict__ eperm, "
-            "const i64* __restrict__ order)"
+            f"const i64* __restrict__ order{self.HUB_PARAMS}{self.HUB_ROWS_PARAM})"
         )
         self._lane_prologue(s, segw)
         if self.tr_stores & 1 and self.R == 1:
             s(f"__shared__ T s_tr[{self.NCH * G * segw}][{64 * max(low.out[io].d for io in self.used_out)}];")
         self._node_loop_open(s, G, xcd)
-        s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
-        s(f"T* zrow = L3_dgrad + node * {low.L3};")
+        s(f"T* zrow = hubpos >= 0 ? hub_rows + hubpos * {low.L3} : L3_dgrad + node * {low.L3};")
         for si in range(len(self.segments)):
             s.open(f"if (sg == {si % segw})" if segw > 1 else "")
 
@@ -549,7 +548,7 @@ class DoubleEmitter(UvuEmitter):
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
-            "T* __restrict__ L3_dgrad, const i64* __restrict__ order, T* __restrict__ wpartial)"
+            f"T* __restrict__ L3_dgrad, const i64* __restrict__ order, T* __restrict__ wpartial{self.HUB_PARAMS})"
         )
         self._lane_prologue(s)
         shared = low.shared_weights
@@ -565,7 +564,6 @@ class DoubleEmitter(UvuEmitter):
             s(f"for (int t = 0; t < {self.n_wslots}; ++t) dwacc[t] = T(0);")
         resident = self.double_b_resident() or self.merged
         self._node_loop_open(s, G, xcd)
-        s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
 
         def node_body():
             if resident:
@@ -707,7 +705,7 @@ class DoubleEmitter(UvuEmitter):
             f"i64 nnz, {self._CONV_OPERANDS}const T* __restrict__ L3_grad, T* __restrict__ L2_grad, "
             "T* __restrict__ W_grad, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             "const i64* __restrict__ rowptr, T* __restrict__ dx_tmp, const i64* __restrict__ eperm, "
-            "T* __restrict__ L3_dgrad, const i64* __restrict__ order, T* __restrict__ wpartial)"
+            f"T* __restrict__ L3_dgrad, const i64* __restrict__ order, T* __restrict__ wpartial{self.HUB_PARAMS})"
         )
         self._lane_prologue(s, SW)
         s(f"__shared__ T s_dy[{SW * self.NCH}][{self.l2_pad}];")
@@ -715,7 +713,6 @@ class DoubleEmitter(UvuEmitter):
         if self.merged and self.tr_stores & 1:
             s(f"__shared__ T s_tr[{self.NCH * SW}][{64 * max(low.out[io].d for io in self.used_out)}];")
         self._node_loop_open(s, 1, xcd)
-        s("const i64 e0 = oeq_pos(rowptr[node], nnz), e1 = oeq_pos(rowptr[node + 1], nnz);")
         for si in range(SW):
             s.open(f"if (sg == {si})")
 

@@ -126,6 +126,9 @@ struct oeq_kernels {
     // Set by the allocation-free entry point for the duration of its call (on its thread): launches then
     // create no timing events.
     static thread_local bool no_events;
+    // Set by the same entry point: long edge segments are not cut into chunks (their rows would need scratch
+    // that the static buffer does not have).
+    static thread_local bool no_hubs;
 
     bool loaded_on_current_device() {
         int dev = 0;
@@ -172,23 +175,6 @@ struct oeq_kernels {
         return launch(OEQ_ROLE_SEGMENT_PTR, n_items + 1, args, stream);
     }
 
-    // Item indices grouped by key, in no particular order within a group: ptr[0..n_segments] = group
-    // starts, perm = the grouped indices; cursor (sized by ptr_bytes_of) is scratch.
-    int group_unordered(int64_t n_items, int64_t n_segments, const int64_t* keys, int64_t* ptr, int64_t* cursor,
-                        int64_t* perm, void* stream) {
-        int rc = fill_zero(ptr, (size_t)(n_segments + 1) * sizeof(int64_t), stream);
-        if (rc) return rc;
-        void* cargs[] = {&n_items, &keys, &ptr, &n_segments};
-        rc = launch(OEQ_ROLE_GROUP_COUNT, n_items, cargs, stream);
-        if (rc) return rc;
-        int64_t n = n_segments + 1;
-        void* sargs[] = {&n, &ptr, &cursor};
-        rc = launch(OEQ_ROLE_GROUP_SCAN, 1, sargs, stream);
-        if (rc) return rc;
-        void* pargs[] = {&n_items, &keys, &cursor, &perm, &n_segments};
-        return launch(OEQ_ROLE_GROUP_SCATTER, n_items, pargs, stream);
-    }
-
     // Counting sort of the item indices 0..n_items-1 by key: ptr[0..n_segments] = segment starts,
     // perm = item indices grouped by key, ascending within a group (so the result depends on the key
     // list only); cursor (n_segments + 1 entries and the long-segment list, see ptr_bytes_of) and unordered
@@ -217,6 +203,7 @@ struct oeq_kernels {
 };
 
 thread_local bool oeq_kernels::no_events = false;
+thread_local bool oeq_kernels::no_hubs = false;
 
 // ---------------------------------------------------------------------------
 // scratch memory of the allocation-free entry point
@@ -251,7 +238,7 @@ int static_scratch(void** out) {
 extern "C" {
 
 const char* oeq_last_error(void) { return g_error.c_str(); }
-int oeq_abi_version(void) { return 3; }
+int oeq_abi_version(void) { return 4; }
 
 int oeq_get_device_props(int device, oeq_device_props* out) {
     if (!out) return fail(OEQ_ERR_INVALID, "oeq_get_device_props: out is NULL");
@@ -515,10 +502,39 @@ static size_t ptr_bytes_of(int64_t node_count) {
 }
 static size_t perm_bytes_of(int64_t nnz) { return align_up((size_t)nnz * sizeof(int64_t), 256); }
 
-static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t node_count, int role = OEQ_ROLE_CONV_BACKWARD) {
+static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t walk_positions, int role = OEQ_ROLE_CONV_BACKWARD) {
     if (!k->dims.shared_weights || !k->dims.wpartial_per_block || !k->roles[role].present) return 0;
-    size_t rows = (size_t)k->grid_for(role, node_count) * (size_t)k->dims.wpartial_per_block;
+    size_t rows = (size_t)k->grid_for(role, walk_positions) * (size_t)k->dims.wpartial_per_block;
     return align_up(rows * (size_t)k->dims.weight_numel * (size_t)k->dims.elem_size, 256);
+}
+
+// Long edge segments (a hub node) are walked in chunks of `hub_limit` edges: a node's own walk position takes
+// the first chunk, every further chunk is an extra position listed in the index (hubptr / hubnode). 0 = whole
+// segments (kernel sets without the table kernels, and the allocation-free entry point).
+static int64_t hub_limit_of(const oeq_kernels* k) {
+    if (oeq_kernels::no_hubs || k->dims.hub_limit <= 0) return 0;
+    if (!k->roles[OEQ_ROLE_HUB_COUNT].present || !k->roles[OEQ_ROLE_HUB_FILL].present ||
+        !k->roles[OEQ_ROLE_CONV_FIXUP_FORWARD].present)
+        return 0;
+    return k->dims.hub_limit;
+}
+// every extra position follows a full chunk of its node, so there are at most nnz / limit of them
+static int64_t hub_capacity(const oeq_kernels* k, int64_t nnz) {
+    const int64_t limit = hub_limit_of(k);
+    return limit ? nnz / limit : 0;
+}
+// Walk positions that the kernel of `role` reserves for the extra chunks, at the front of its grid: the
+// capacity rounded up to whole blocks and to the grid multiple of the role, so that the blocks behind them
+// still divide evenly among the XCDs.
+static int64_t hub_units(const oeq_kernels* k, int role, int64_t nnz) {
+    const int64_t cap = hub_capacity(k, nnz);
+    if (!cap || !k->roles[role].present) return 0;
+    const int64_t g = std::max(1u, k->roles[role].units_per_block), m = std::max(1u, k->roles[role].grid_multiple);
+    const int64_t blocks = ((cap + g - 1) / g + m - 1) / m * m;
+    return blocks * g;
+}
+static size_t hub_rows_bytes(const oeq_kernels* k, int role, int64_t nnz) {
+    return align_up((size_t)hub_units(k, role, nnz) * (size_t)k->dims.L3_dim * (size_t)k->dims.elem_size, 256);
 }
 
 // The index of an edge list: what the walk kernels derive from (rows, cols) alone. Receiver side: CSR
@@ -527,9 +543,10 @@ static size_t conv_wpartial_bytes(const oeq_kernels* k, int64_t node_count, int 
 // grouped by sender. Byte offsets into the index buffer (SIZE_MAX: piece not present); the pieces after
 // `keep` are temporaries of the build.
 struct IndexLayout {
-    size_t rowptr = SIZE_MAX, colptr = SIZE_MAX, rperm = SIZE_MAX, sperm = SIZE_MAX, order = SIZE_MAX, keep = 0,
-           cursor = SIZE_MAX, scratch = SIZE_MAX, key_a = SIZE_MAX, key_b = SIZE_MAX, optr = SIZE_MAX,
-           ocursor = SIZE_MAX, total = 0;
+    size_t rowptr = SIZE_MAX, colptr = SIZE_MAX, rperm = SIZE_MAX, sperm = SIZE_MAX, order = SIZE_MAX,
+           hubptr = SIZE_MAX, hubnode = SIZE_MAX, shubptr = SIZE_MAX, shubnode = SIZE_MAX, hubcur = SIZE_MAX,
+           keep = 0, cursor = SIZE_MAX, scratch = SIZE_MAX, key_a = SIZE_MAX, key_b = SIZE_MAX, optr = SIZE_MAX,
+           ocursor = SIZE_MAX, oscratch = SIZE_MAX, total = 0;
 };
 
 static IndexLayout index_layout(const oeq_kernels* k, int64_t node_count, int64_t nnz, bool sender_side) {
@@ -543,7 +560,17 @@ static IndexLayout index_layout(const oeq_kernels* k, int64_t node_count, int64_
     if (grouped) w.rperm = take(qb);
     if (grouped && sender_side) w.sperm = take(qb);
     if (ordered) w.order = take(pb);
+    const int64_t hub_cap = hub_capacity(k, nnz);
+    if (hub_cap) {
+        w.hubptr = take(pb);
+        w.hubnode = take(align_up((size_t)hub_cap * sizeof(int64_t), 256));
+        if (sender_side) {  // the same table over the senders' segments, for the ordered sum of the dX terms
+            w.shubptr = take(pb);
+            w.shubnode = take(align_up((size_t)hub_cap * sizeof(int64_t), 256));
+        }
+    }
     w.keep = w.total;
+    if (hub_cap) w.hubcur = take(pb);
     if (grouped) {
         w.cursor = take(pb);
         w.scratch = take(qb);
@@ -553,6 +580,7 @@ static IndexLayout index_layout(const oeq_kernels* k, int64_t node_count, int64_
         w.key_b = take(pb);
         w.optr = take(pb);
         w.ocursor = take(pb);
+        w.oscratch = take(pb);
     }
     return w;
 }
@@ -560,18 +588,30 @@ static IndexLayout index_layout(const oeq_kernels* k, int64_t node_count, int64_
 // What a call needs besides operands and index: `terms` = the per-edge dX terms, `arrivals` = the per-sender
 // arrival counters of OEQ_DX_ARRIVAL, `wpartial` = partial weight-gradient rows (shared weights).
 struct ScratchLayout {
-    size_t arrivals = SIZE_MAX, dx_tmp = SIZE_MAX, wpartial = SIZE_MAX, total = 0;
+    size_t arrivals = SIZE_MAX, dx_tmp = SIZE_MAX, wpartial = SIZE_MAX, hub_rows = SIZE_MAX, shub_rows = SIZE_MAX,
+           total = 0;
 };
 
 static ScratchLayout scratch_layout(const oeq_kernels* k, int64_t node_count, int64_t nnz, bool terms, bool arrivals,
-                                    bool wpartial, int wpartial_role = OEQ_ROLE_CONV_BACKWARD) {
+                                    bool wpartial, int wpartial_role = OEQ_ROLE_CONV_BACKWARD,
+                                    int hub_rows_role = -1) {
     ScratchLayout w;
     auto take = [&w](size_t bytes) { size_t at = w.total; w.total += bytes; return at; };
+    // rows that the extra chunks of long segments write (forward-shaped kernels)
+    if (hub_rows_role >= 0)
+        if (size_t hb = hub_rows_bytes(k, hub_rows_role, nnz)) w.hub_rows = take(hb);
     if (arrivals)
         w.arrivals = take(align_up((size_t)node_count * (size_t)std::max(1, k->dims.n_chunks) * sizeof(int32_t), 256));
-    if (terms) w.dx_tmp = take(align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256));
+    if (terms) {
+        w.dx_tmp = take(align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256));
+        // partial sums of the senders whose terms fixup_backward sums in chunks
+        if (!arrivals)
+            if (int64_t su = hub_units(k, OEQ_ROLE_CONV_FIXUP_BACKWARD, nnz))
+                w.shub_rows = take(align_up((size_t)su * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256));
+    }
     if (wpartial)
-        if (size_t wp = conv_wpartial_bytes(k, node_count, wpartial_role)) w.wpartial = take(wp);
+        if (size_t wp = conv_wpartial_bytes(k, node_count + hub_units(k, wpartial_role, nnz), wpartial_role))
+            w.wpartial = take(wp);
     return w;
 }
 
@@ -579,10 +619,13 @@ struct WalkIndex {
     int64_t *rowptr = nullptr, *colptr = nullptr, *rperm = nullptr;
     const int64_t* sperm = nullptr;
     int64_t* order = nullptr;  // the order in which the walk kernels visit the nodes (NULL: by index)
+    // extra walk positions of the nodes whose edge segments are cut into chunks (NULL / 0: none)
+    int64_t *hubptr = nullptr, *hubnode = nullptr, *shubptr = nullptr, *shubnode = nullptr;
+    int64_t hub_limit = 0;
 };
 
 struct WalkScratch {
-    void *dx_tmp = nullptr, *wpartial = nullptr;
+    void *dx_tmp = nullptr, *wpartial = nullptr, *shub_rows = nullptr;
     int32_t* arrivals = nullptr;
 };
 
@@ -600,6 +643,11 @@ static int bind_index(const oeq_kernels* k, const char* who, const IndexLayout& 
     ix->rperm = (int64_t*)at_offset(index, w.rperm);
     ix->sperm = w.sperm != SIZE_MAX ? (const int64_t*)at_offset(index, w.sperm) : transpose_perm;
     ix->order = (int64_t*)at_offset(index, w.order);
+    ix->hubptr = (int64_t*)at_offset(index, w.hubptr);
+    ix->hubnode = (int64_t*)at_offset(index, w.hubnode);
+    ix->shubptr = (int64_t*)at_offset(index, w.shubptr);
+    ix->shubnode = (int64_t*)at_offset(index, w.shubnode);
+    ix->hub_limit = ix->hubptr ? hub_limit_of(k) : 0;
     return OEQ_OK;
 }
 
@@ -623,10 +671,26 @@ static int build_index(oeq_kernels* k, const char* who, const IndexLayout& w, in
         if (!rc && sender_side)
             rc = k->group_by_key(nnz, node_count, cols, ix.colptr, cursor, scratch, (int64_t*)ix.sperm, stream);
     }
+    // extra positions of long segments: count per node, exclusive scan, list the nodes
+    auto hub_table = [&](int64_t* segptr, int64_t* hubptr, int64_t* hubnode) {
+        int64_t limit = ix.hub_limit, cap = hub_capacity(k, nnz), n1 = node_count + 1;
+        int64_t* hubcur = (int64_t*)at_offset(index, w.hubcur);
+        void* cargs[] = {&node_count, &nnz, &segptr, &limit, &hubptr};
+        int r = k->launch(OEQ_ROLE_HUB_COUNT, n1, cargs, stream);
+        void* sargs[] = {&n1, &hubptr, &hubcur};
+        if (!r) r = k->launch(OEQ_ROLE_GROUP_SCAN, 1, sargs, stream);
+        void* fargs[] = {&node_count, &cap, &hubptr, &hubnode};
+        if (!r) r = k->launch(OEQ_ROLE_HUB_FILL, node_count, fargs, stream);
+        return r;
+    };
+    if (!rc && ix.hubptr) rc = hub_table(ix.rowptr, ix.hubptr, ix.hubnode);
+    if (!rc && ix.shubptr) rc = hub_table(ix.colptr, ix.shubptr, ix.shubnode);
     if (rc || !ix.order) return rc;
     // Walk order: cluster the nodes by the highest-priority node within `order_hops` edges, then list them
-    // cluster by cluster (a counting sort by cluster key; the order inside a cluster is whatever the
-    // scatter's atomics give, which changes which nodes run side by side but no result).
+    // cluster by cluster (a counting sort by cluster key, ascending node index inside a cluster, so that the
+    // order is a function of the edge list: with shared weights the walk kernels sum their weight gradients
+    // per wave group over the nodes the group visits, and which nodes those are must not change between
+    // two builds).
     int64_t* keys[2] = {(int64_t*)at_offset(index, w.key_a), (int64_t*)at_offset(index, w.key_b)};
     const int64_t* key_in = nullptr;
     const int64_t* cperm = ix.rperm;
@@ -637,11 +701,27 @@ static int build_index(oeq_kernels* k, const char* who, const IndexLayout& w, in
         if (rc) return rc;
         key_in = key_out;
     }
-    return k->group_unordered(node_count, node_count, key_in, (int64_t*)at_offset(index, w.optr),
-                              (int64_t*)at_offset(index, w.ocursor), ix.order, stream);
+    return k->group_by_key(node_count, node_count, key_in, (int64_t*)at_offset(index, w.optr),
+                           (int64_t*)at_offset(index, w.ocursor), (int64_t*)at_offset(index, w.oscratch), ix.order,
+                           stream);
 }
 
 static bool walk_mode(const oeq_kernels* k) { return k->dims.deterministic != OEQ_CONV_ATOMIC; }
+
+// L1_grad[s] = sum of the per-edge terms of sender s in sender-major order; senders with more than hub_limit
+// edges in chunks whose partial sums (shub_rows) are added in chunk order afterwards.
+static int sender_sum(oeq_kernels* k, int64_t node_count, int64_t nnz, void* dx_tmp, void* L1_grad,
+                      const WalkIndex& ix, void* shub_rows, void* stream) {
+    int64_t limit = (ix.shubptr && shub_rows) ? ix.hub_limit : 0;
+    int64_t units = limit ? hub_units(k, OEQ_ROLE_CONV_FIXUP_BACKWARD, nnz) : 0;
+    void* fargs[] = {&node_count, &nnz,         &dx_tmp, &L1_grad, (void*)&ix.sperm, (void*)&ix.colptr,
+                     (void*)&ix.shubptr, (void*)&ix.shubnode, &limit, &units, &shub_rows};
+    int rc = k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count + units, fargs, stream);
+    if (rc || !units) return rc;
+    int64_t row_len = k->dims.L1_dim;
+    void* cargs[] = {&node_count, &units, (void*)&ix.shubptr, (void*)&ix.shubnode, &shub_rows, &L1_grad, &row_len};
+    return k->launch(OEQ_ROLE_CONV_FIXUP_FORWARD, units, cargs, stream);
+}
 static bool backward_terms(const oeq_kernels* k) { return k->dims.dx_mode != OEQ_DX_ATOMIC; }
 
 size_t oeq_conv_index_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz, int sender_side) {
@@ -661,8 +741,13 @@ int oeq_conv_index_build(oeq_kernels* k, int64_t node_count, int64_t nnz, const 
                        rows, cols, transpose_perm, index, index_bytes, stream);
 }
 
+size_t oeq_conv_forward_scratch_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
+    if (!k || !walk_mode(k) || node_count < 0 || nnz < 0) return 0;
+    return scratch_layout(k, node_count, nnz, false, false, false, OEQ_ROLE_CONV_BACKWARD, OEQ_ROLE_CONV_FORWARD).total;
+}
+
 size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
-    return oeq_conv_index_bytes(k, node_count, nnz, 0);
+    return oeq_conv_index_bytes(k, node_count, nnz, 0) + oeq_conv_forward_scratch_bytes(k, node_count, nnz);
 }
 
 size_t oeq_conv_backward_scratch_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
@@ -679,7 +764,8 @@ size_t oeq_conv_backward_workspace_bytes(const oeq_kernels* k, int64_t node_coun
 // the second-order kernels always go through the per-edge terms and fixup_backward
 size_t oeq_conv_double_backward_scratch_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
     if (!k || !walk_mode(k)) return 0;
-    return scratch_layout(k, node_count, nnz, true, false, true, OEQ_ROLE_DOUBLE_BACKWARD_B).total;
+    return scratch_layout(k, node_count, nnz, true, false, true, OEQ_ROLE_DOUBLE_BACKWARD_B,
+                          OEQ_ROLE_DOUBLE_BACKWARD_A).total;
 }
 
 size_t oeq_conv_double_backward_workspace_bytes(const oeq_kernels* k, int64_t node_count, int64_t nnz) {
@@ -689,7 +775,8 @@ size_t oeq_conv_double_backward_workspace_bytes(const oeq_kernels* k, int64_t no
 
 int oeq_conv_forward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
                              const void* W, void* L3_out, const int64_t* rows, const int64_t* cols, const void* index,
-                             size_t index_bytes, int index_sender_side, void* stream) {
+                             size_t index_bytes, int index_sender_side, void* scratch, size_t scratch_bytes,
+                             void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL kernel set");
     if (int bad = check_graph_size("oeq_conv_forward", node_count, nnz)) return bad;
     if (node_count == 0) return OEQ_OK;
@@ -699,17 +786,33 @@ int oeq_conv_forward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, co
     if (!L1_in || !L2_in || !W || !rows || !cols) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL buffer");
     WalkIndex ix;
     int rc;
+    int64_t units = 0;
+    void* hub_rows = nullptr;
     if (walk_mode(k)) {
         // the forward reads the receiver side only; the caller's perm stands in where the layout wants one
         rc = bind_index(k, "oeq_conv_forward", index_layout(k, node_count, nnz, index_sender_side != 0), index,
                         index_bytes, rows, &ix);
         if (rc) return rc;
+        if (ix.hub_limit) {
+            units = hub_units(k, OEQ_ROLE_CONV_FORWARD, nnz);
+            const size_t need = hub_rows_bytes(k, OEQ_ROLE_CONV_FORWARD, nnz);
+            if (!scratch || scratch_bytes < need)
+                return fail(OEQ_ERR_INVALID, "oeq_conv_forward: workspace too small (%zu < %zu bytes of scratch)",
+                            scratch_bytes, need);
+            hub_rows = scratch;
+        }
     } else {
         rc = k->fill_zero(L3_out, out_bytes, stream);
         if (rc) return rc;
     }
-    void* args[] = {&node_count, &nnz, &L1_in, &L2_in, &W, &L3_out, &rows, &cols, &ix.rowptr, &ix.rperm, &ix.order};
-    return k->launch(OEQ_ROLE_CONV_FORWARD, walk_mode(k) ? node_count : nnz, args, stream);
+    void* args[] = {&node_count, &nnz,      &L1_in,    &L2_in,      &W,           &L3_out,       &rows,  &cols,
+                    &ix.rowptr,  &ix.rperm, &ix.order, &ix.hubptr, &ix.hubnode, &ix.hub_limit, &units, &hub_rows};
+    rc = k->launch(OEQ_ROLE_CONV_FORWARD, walk_mode(k) ? node_count + units : nnz, args, stream);
+    if (rc || !units) return rc;
+    // the rows of the extra chunks, added to their nodes' rows in chunk order
+    int64_t row_len = k->dims.L3_dim;
+    void* fargs[] = {&node_count, &units, &ix.hubptr, &ix.hubnode, &hub_rows, &L3_out, &row_len};
+    return k->launch(OEQ_ROLE_CONV_FIXUP_FORWARD, units, fargs, stream);
 }
 
 int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void* L1_in, const void* L2_in,
@@ -722,13 +825,17 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void
         if (!L3_out) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL L3_out");
         if (!L1_in || !L2_in || !W || !rows || !cols) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL buffer");
         const IndexLayout w = index_layout(k, node_count, nnz, false);
-        int rc = build_index(k, "oeq_conv_forward", w, node_count, nnz, rows, cols, nullptr, workspace,
-                             workspace_bytes, stream);
+        const size_t need = w.total + oeq_conv_forward_scratch_bytes(k, node_count, nnz);
+        if (!workspace || workspace_bytes < need)
+            return fail(OEQ_ERR_INVALID, "oeq_conv_forward: workspace too small (%zu < %zu bytes)", workspace_bytes,
+                        need);
+        int rc = build_index(k, "oeq_conv_forward", w, node_count, nnz, rows, cols, nullptr, workspace, w.total, stream);
         if (rc) return rc;
         index_bytes = w.total;
     }
     return oeq_conv_forward_indexed(k, node_count, nnz, L1_in, L2_in, W, L3_out, rows, cols, workspace, index_bytes, 0,
-                                    stream);
+                                    workspace ? (char*)workspace + index_bytes : nullptr,
+                                    workspace_bytes > index_bytes ? workspace_bytes - index_bytes : 0, stream);
 }
 
 size_t oeq_static_scratch_bytes(void) { return OEQ_STATIC_SCRATCH_BYTES; }
@@ -737,7 +844,9 @@ int oeq_conv_forward_static(oeq_kernels* k, int64_t node_count, int64_t nnz, con
                             const void* W, void* L3_out, const int64_t* rows, const int64_t* cols, void* stream) {
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_forward_static: NULL kernel set");
     if (node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_forward_static: negative size");
+    oeq_kernels::no_hubs = true;  // whole segments: no rows of extra chunks to hold
     const size_t need = oeq_conv_forward_workspace_bytes(k, node_count, nnz);
+    oeq_kernels::no_hubs = false;
     if (need > OEQ_STATIC_SCRATCH_BYTES)
         return fail(OEQ_ERR_INVALID,
                     "oeq_conv_forward_static: %lld nodes and %lld edges need %zu bytes of index scratch, the static "
@@ -751,9 +860,9 @@ int oeq_conv_forward_static(oeq_kernels* k, int64_t node_count, int64_t nnz, con
     void* ws = nullptr;
     int rc = static_scratch(&ws);
     if (rc) return rc;
-    oeq_kernels::no_events = true;
+    oeq_kernels::no_events = oeq_kernels::no_hubs = true;
     rc = oeq_conv_forward(k, node_count, nnz, L1_in, L2_in, W, L3_out, rows, cols, ws, OEQ_STATIC_SCRATCH_BYTES, stream);
-    oeq_kernels::no_events = false;
+    oeq_kernels::no_events = oeq_kernels::no_hubs = false;
     return rc;
 }
 
@@ -801,6 +910,7 @@ int oeq_conv_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, c
         sc.dx_tmp = at_offset(scratch, w.dx_tmp);
         sc.wpartial = at_offset(scratch, w.wpartial);
         sc.arrivals = (int32_t*)at_offset(scratch, w.arrivals);
+        sc.shub_rows = at_offset(scratch, w.shub_rows);
     }
     if (dx_mode != OEQ_DX_TERMS) {
         // atomics accumulate into the rows; the arrival scheme never visits a node that sends nothing
@@ -812,17 +922,17 @@ int oeq_conv_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, c
                           stream);
         if (rc) return rc;
     }
-    void* args[] = {&node_count, &nnz,     &L1_in, &L1_grad, &L2_in,     &L2_grad,   &W,          &W_grad,   &L3_grad,
-                    &rows,       &cols,    &ix.rowptr, &sc.dx_tmp, &ix.rperm, &sc.wpartial, &ix.colptr, &ix.sperm,
-                    &sc.arrivals, &ix.order};
-    rc = k->launch(OEQ_ROLE_CONV_BACKWARD, walk_mode(k) ? node_count : nnz, args, stream);
+    int64_t units = ix.hub_limit ? hub_units(k, OEQ_ROLE_CONV_BACKWARD, nnz) : 0;
+    void* args[] = {&node_count,  &nnz,      &L1_in,     &L1_grad,    &L2_in,        &L2_grad,     &W,         &W_grad,
+                    &L3_grad,     &rows,     &cols,      &ix.rowptr,  &sc.dx_tmp,    &ix.rperm,    &sc.wpartial,
+                    &ix.colptr,   &ix.sperm, &sc.arrivals, &ix.order, &ix.hubptr,    &ix.hubnode,  &ix.hub_limit,
+                    &units};
+    rc = k->launch(OEQ_ROLE_CONV_BACKWARD, walk_mode(k) ? node_count + units : nnz, args, stream);
     if (rc || !walk_mode(k)) return rc;
-    if (dx_mode == OEQ_DX_TERMS) {
-        void* fargs[] = {&node_count, &nnz, &sc.dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};
-        rc = k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
-    }
+    if (dx_mode == OEQ_DX_TERMS) rc = sender_sum(k, node_count, nnz, sc.dx_tmp, L1_grad, ix, sc.shub_rows, stream);
     if (rc || !wrows) return rc;
-    int64_t n_partials = (int64_t)k->grid_for(OEQ_ROLE_CONV_BACKWARD, node_count) * k->dims.wpartial_per_block;
+    int64_t n_partials =
+        (int64_t)k->grid_for(OEQ_ROLE_CONV_BACKWARD, node_count + units) * k->dims.wpartial_per_block;
     int64_t wn = k->dims.weight_numel;
     void* rargs[] = {&n_partials, &sc.wpartial, &W_grad, &wn};
     return k->launch(OEQ_ROLE_TP_BACKWARD_WREDUCE, wn, rargs, stream);
@@ -938,28 +1048,39 @@ int oeq_conv_double_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t
     int rc = bind_index(k, "oeq_conv_double_backward", index_layout(k, node_count, nnz, true), index, index_bytes,
                         transpose_perm, &ix);
     if (rc) return rc;
-    const ScratchLayout w = scratch_layout(k, node_count, nnz, true, false, true, OEQ_ROLE_DOUBLE_BACKWARD_B);
+    const ScratchLayout w = scratch_layout(k, node_count, nnz, true, false, true, OEQ_ROLE_DOUBLE_BACKWARD_B,
+                                           OEQ_ROLE_DOUBLE_BACKWARD_A);
     if (!scratch || scratch_bytes < w.total)
         return fail(OEQ_ERR_INVALID, "oeq_conv_double_backward: workspace too small (%zu < %zu bytes of scratch)",
                     scratch_bytes, w.total);
     void* dx_tmp = at_offset(scratch, w.dx_tmp);
     // shared weights: kernel B leaves one partial weight-gradient row per wave group, summed in order at the end
     void* wpartial = at_offset(scratch, w.wpartial);
-    void* a[] = {&node_count, &nnz, &L1_in, &L1_dgrad, &L2_in, &L2_dgrad, &W, &W_dgrad, &L3_dgrad,
-                 &rows,       &cols, &ix.rowptr, &ix.rperm, &ix.order};
+    void* hub_rows = at_offset(scratch, w.hub_rows);
+    int64_t units_a = (ix.hub_limit && hub_rows) ? hub_units(k, OEQ_ROLE_DOUBLE_BACKWARD_A, nnz) : 0;
+    int64_t units_b = ix.hub_limit ? hub_units(k, OEQ_ROLE_DOUBLE_BACKWARD_B, nnz) : 0;
+    void* a[] = {&node_count, &nnz,  &L1_in,     &L1_dgrad, &L2_in,    &L2_dgrad,  &W,          &W_dgrad,      &L3_dgrad,
+                 &rows,       &cols, &ix.rowptr, &ix.rperm, &ix.order, &ix.hubptr, &ix.hubnode, &ix.hub_limit, &units_a,
+                 &hub_rows};
     if (k->roles[OEQ_ROLE_DOUBLE_BACKWARD_A].present) {
-        rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_A, node_count, a, stream);
+        rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_A, node_count + units_a, a, stream);
         if (rc) return rc;
+        if (units_a) {
+            int64_t row_len = k->dims.L3_dim;
+            void* fa[] = {&node_count, &units_a, &ix.hubptr, &ix.hubnode, &hub_rows, &L3_dgrad, &row_len};
+            rc = k->launch(OEQ_ROLE_CONV_FIXUP_FORWARD, units_a, fa, stream);
+            if (rc) return rc;
+        }
     }
-    void* b[] = {&node_count, &nnz,     &L1_in,  &L1_dgrad, &L2_in, &L2_dgrad,  &W,         &W_dgrad, &L3_grad,
-                 &L2_grad,    &W_grad,  &rows,   &cols,     &ix.rowptr, &dx_tmp, &ix.rperm, &L3_dgrad, &ix.order,
-                 &wpartial};
-    rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count, b, stream);
+    void* b[] = {&node_count, &nnz,        &L1_in,      &L1_dgrad,     &L2_in,   &L2_dgrad,  &W,         &W_dgrad,
+                 &L3_grad,    &L2_grad,    &W_grad,     &rows,         &cols,    &ix.rowptr, &dx_tmp,    &ix.rperm,
+                 &L3_dgrad,   &ix.order,   &wpartial,   &ix.hubptr,    &ix.hubnode, &ix.hub_limit, &units_b};
+    rc = k->launch(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count + units_b, b, stream);
     if (rc) return rc;
-    void* fargs[] = {&node_count, &nnz, &dx_tmp, &L1_grad, &ix.sperm, &ix.colptr};
-    rc = k->launch(OEQ_ROLE_CONV_FIXUP_BACKWARD, node_count, fargs, stream);
+    rc = sender_sum(k, node_count, nnz, dx_tmp, L1_grad, ix, at_offset(scratch, w.shub_rows), stream);
     if (rc || !wpartial) return rc;
-    int64_t n_partials = (int64_t)k->grid_for(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count) * k->dims.wpartial_per_block;
+    int64_t n_partials =
+        (int64_t)k->grid_for(OEQ_ROLE_DOUBLE_BACKWARD_B, node_count + units_b) * k->dims.wpartial_per_block;
     int64_t wn = k->dims.weight_numel;
     void* rargs[] = {&n_partials, &wpartial, &W_grad, &wn};
     return k->launch(OEQ_ROLE_TP_BACKWARD_WREDUCE, wn, rargs, stream);

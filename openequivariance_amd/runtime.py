@@ -50,10 +50,13 @@ ROLE_GROUP_ORDER = 12
 ROLE_DOUBLE_BACKWARD_A = 13
 ROLE_DOUBLE_BACKWARD_B = 14
 ROLE_ORDER_HOP = 15
+ROLE_HUB_COUNT = 16
+ROLE_HUB_FILL = 17
+ROLE_CONV_FIXUP_FORWARD = 18
 
 CONV_ATOMIC, CONV_SORTED, CONV_GROUPED = 0, 1, 2
 DX_TERMS, DX_ATOMIC, DX_ARRIVAL = 0, 1, 2
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class OeqError(RuntimeError):
@@ -98,6 +101,7 @@ class _ProblemDims(ctypes.Structure):
         ("dx_mode", ctypes.c_int32),
         ("n_chunks", ctypes.c_int32),
         ("order_hops", ctypes.c_int32),
+        ("hub_limit", ctypes.c_int32),
     ]
 
 
@@ -145,7 +149,9 @@ EXPORTS = {
     "oeq_conv_double_backward_workspace_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_index_bytes": (_SZ, [_P, _I64, _I64, ctypes.c_int]),
     "oeq_conv_index_build": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, ctypes.c_int, _P, _SZ, _P]),
-    "oeq_conv_forward_indexed": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _SZ, ctypes.c_int, _P]),
+    "oeq_conv_forward_indexed": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _SZ, ctypes.c_int, _P, _SZ,
+                                                _P]),
+    "oeq_conv_forward_scratch_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_backward_indexed": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 10 + [_P, _SZ, ctypes.c_int, _P, _SZ, _P]),
     "oeq_conv_backward_scratch_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_double_backward_indexed": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 14 + [_P, _SZ, _P, _SZ, _P]),
@@ -349,9 +355,14 @@ class KernelSet:
         _check(self._lib.oeq_conv_index_build(self.handle, nodes, nnz, rows, cols, perm, int(sender_side), index,
                                               index_bytes, stream), "oeq_conv_index_build")
 
-    def conv_forward_indexed(self, nodes, nnz, x, y, w, out, rows, cols, index, index_bytes, sender_side, stream):
+    def conv_forward_scratch_bytes(self, nodes, nnz) -> int:
+        return self._lib.oeq_conv_forward_scratch_bytes(self.handle, nodes, nnz)
+
+    def conv_forward_indexed(self, nodes, nnz, x, y, w, out, rows, cols, index, index_bytes, sender_side, scratch,
+                             scratch_bytes, stream):
         _check(self._lib.oeq_conv_forward_indexed(self.handle, nodes, nnz, x, y, w, out, rows, cols, index, index_bytes,
-                                                  int(sender_side), stream), "oeq_conv_forward_indexed")
+                                                  int(sender_side), scratch, scratch_bytes, stream),
+               "oeq_conv_forward_indexed")
 
     def conv_backward_scratch_bytes(self, nodes, nnz) -> int:
         return self._lib.oeq_conv_backward_scratch_bytes(self.handle, nodes, nnz)

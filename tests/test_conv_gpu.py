@@ -427,8 +427,9 @@ def test_kahan_summation(name, make):
     assert hub_err[True][0] <= 2e-7 and hub_err[True][1] <= 2e-7, hub_err
     print(name, hub_err)
     for plain, comp in zip(hub_err[False], hub_err[True]):
-        # narrow problems pack many rows per wave, which already splits the sum into short partial sums
-        assert comp <= plain and (plain <= 1.5e-7 or comp < 0.5 * plain), hub_err
+        # narrow problems pack many rows per wave, which already splits the sum into short partial sums,
+        # and so does the chunked walk of a long segment in the uncompensated forward
+        assert comp <= max(plain, 1e-7) and (plain <= 1.5e-7 or comp < 0.5 * plain), hub_err
 
 
 @pytest.mark.parametrize("name,make", [("cfg2", P.config2_nequip_uvu), ("cfg5-f32", P.config5_mace_conv),
@@ -519,7 +520,10 @@ KNOBS = ["conv_pipe_f=0,conv_pipe_b=1", "conv_pipe_f=1,conv_pipe_b=2", "conv_pip
          # wave-shared product table forward only, backward only and in both directions; lanes without a
          # channel zeroed after each load
          "conv_dxm=0,conv_hops=0,conv_q=1", "conv_dxm=1,conv_hops=1", "conv_dxm=2,conv_hops=3,conv_q=3",
-         "conv_q=2,conv_qaf=16,conv_qab=200,conv_qpin=0", "tp_mask=1"]
+         "conv_q=2,conv_qaf=16,conv_qab=200,conv_qpin=0", "tp_mask=1",
+         # edge segments cut into chunks of 2 / 3 edges (every node of these graphs has extra walk positions),
+         # and never
+         "conv_hub=2", "conv_hub=3,conv_xcd=1,conv_hops=0", "conv_hub=0"]
 
 
 @pytest.mark.parametrize("knobs", KNOBS)
