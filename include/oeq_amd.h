@@ -245,6 +245,21 @@ size_t oeq_conv_index_bytes(const oeq_kernels* k, int64_t node_count, int64_t nn
 int oeq_conv_index_build(oeq_kernels* k, int64_t node_count, int64_t nnz,
                          const int64_t* rows, const int64_t* cols, const int64_t* transpose_perm,
                          int sender_side, void* index, size_t index_bytes, void* stream);
+/* Where a piece of a built index lies, for inspection (tests, tools): byte offset into the index buffer and
+ * number of int64 entries. No counterpart in the reference. */
+typedef enum {
+    OEQ_INDEX_ROWPTR = 0,    /* CSR pointers over receivers, node_count + 1 */
+    OEQ_INDEX_COLPTR = 1,    /* ... over senders (sender side) */
+    OEQ_INDEX_RPERM = 2,     /* OEQ_CONV_GROUPED: edge ids grouped by receiver, nnz */
+    OEQ_INDEX_SPERM = 3,     /* ... by sender (sender side) */
+    OEQ_INDEX_ORDER = 4,     /* walk order of the nodes, node_count */
+    OEQ_INDEX_HUBPTR = 5,    /* first extra walk position of every node, node_count + 1 (hub_limit > 0) */
+    OEQ_INDEX_HUBNODE = 6,   /* node of every extra walk position, nnz / hub_limit */
+    OEQ_INDEX_SHUBPTR = 7,   /* the same two over the senders' segments (sender side) */
+    OEQ_INDEX_SHUBNODE = 8
+} oeq_index_piece;
+int oeq_conv_index_piece(const oeq_kernels* k, int64_t node_count, int64_t nnz, int sender_side, int piece,
+                         size_t* offset, size_t* entries);
 int oeq_conv_forward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz,
                              const void* L1_in, const void* L2_in, const void* W, void* L3_out,
                              const int64_t* rows, const int64_t* cols,

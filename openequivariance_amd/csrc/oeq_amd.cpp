@@ -729,6 +729,23 @@ size_t oeq_conv_index_bytes(const oeq_kernels* k, int64_t node_count, int64_t nn
     return index_layout(k, node_count, nnz, sender_side != 0).total;
 }
 
+int oeq_conv_index_piece(const oeq_kernels* k, int64_t node_count, int64_t nnz, int sender_side, int piece,
+                         size_t* offset, size_t* entries) {
+    if (!k || !offset || !entries) return fail(OEQ_ERR_INVALID, "oeq_conv_index_piece: NULL argument");
+    if (!walk_mode(k) || node_count < 0 || nnz < 0) return fail(OEQ_ERR_INVALID, "oeq_conv_index_piece: no index");
+    const IndexLayout w = index_layout(k, node_count, nnz, sender_side != 0);
+    const size_t cap = (size_t)hub_capacity(k, nnz);
+    const size_t n1 = (size_t)node_count + 1, n = (size_t)node_count, e = (size_t)nnz;
+    const size_t at[] = {w.rowptr, w.colptr, w.rperm, w.sperm, w.order, w.hubptr, w.hubnode, w.shubptr, w.shubnode};
+    const size_t len[] = {n1, n1, e, e, n, n1, cap, n1, cap};
+    if (piece < 0 || piece >= (int)(sizeof(at) / sizeof(at[0])))
+        return fail(OEQ_ERR_INVALID, "oeq_conv_index_piece: unknown piece %d", piece);
+    if (at[piece] == SIZE_MAX) return fail(OEQ_ERR_INVALID, "oeq_conv_index_piece: piece %d is not part of this index", piece);
+    *offset = at[piece];
+    *entries = len[piece];
+    return OEQ_OK;
+}
+
 int oeq_conv_index_build(oeq_kernels* k, int64_t node_count, int64_t nnz, const int64_t* rows, const int64_t* cols,
                          const int64_t* transpose_perm, int sender_side, void* index, size_t index_bytes,
                          void* stream) {
@@ -821,6 +838,13 @@ int oeq_conv_forward(oeq_kernels* k, int64_t node_count, int64_t nnz, const void
     if (!k) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL kernel set");
     if (int bad = check_graph_size("oeq_conv_forward", node_count, nnz)) return bad;
     size_t index_bytes = 0;
+    if (!oeq_kernels::no_events) {
+        // Where allocating is allowed: resolve the scratch array of oeq_conv_forward_static on this device
+        // (the first look-up of a device symbol may load the library's own code object), so that the static
+        // entry point, whose precondition is one call of this function, finds the address ready.
+        void* unused = nullptr;
+        (void)static_scratch(&unused);
+    }
     if (walk_mode(k) && node_count > 0 && nnz > 0) {
         if (!L3_out) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL L3_out");
         if (!L1_in || !L2_in || !W || !rows || !cols) return fail(OEQ_ERR_INVALID, "oeq_conv_forward: NULL buffer");

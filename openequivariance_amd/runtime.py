@@ -152,6 +152,8 @@ EXPORTS = {
     "oeq_conv_forward_indexed": (ctypes.c_int, [_P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _SZ, ctypes.c_int, _P, _SZ,
                                                 _P]),
     "oeq_conv_forward_scratch_bytes": (_SZ, [_P, _I64, _I64]),
+    "oeq_conv_index_piece": (ctypes.c_int, [_P, _I64, _I64, ctypes.c_int, ctypes.c_int, ctypes.POINTER(_SZ),
+                                            ctypes.POINTER(_SZ)]),
     "oeq_conv_backward_indexed": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 10 + [_P, _SZ, ctypes.c_int, _P, _SZ, _P]),
     "oeq_conv_backward_scratch_bytes": (_SZ, [_P, _I64, _I64]),
     "oeq_conv_double_backward_indexed": (ctypes.c_int, [_P, _I64, _I64] + [_P] * 14 + [_P, _SZ, _P, _SZ, _P]),
@@ -354,6 +356,16 @@ class KernelSet:
     def conv_index_build(self, nodes, nnz, rows, cols, perm, sender_side: bool, index, index_bytes, stream):
         _check(self._lib.oeq_conv_index_build(self.handle, nodes, nnz, rows, cols, perm, int(sender_side), index,
                                               index_bytes, stream), "oeq_conv_index_build")
+
+    INDEX_PIECES = ("rowptr", "colptr", "rperm", "sperm", "order", "hubptr", "hubnode", "shubptr", "shubnode")
+
+    def conv_index_piece(self, nodes, nnz, sender_side: bool, piece: str) -> Tuple[int, int]:
+        """(byte offset, int64 entries) of a piece of a built index (oeq_index_piece)."""
+        off, n = _SZ(), _SZ()
+        _check(self._lib.oeq_conv_index_piece(self.handle, nodes, nnz, int(sender_side),
+                                              self.INDEX_PIECES.index(piece), ctypes.byref(off), ctypes.byref(n)),
+               "oeq_conv_index_piece")
+        return off.value, n.value
 
     def conv_forward_scratch_bytes(self, nodes, nnz) -> int:
         return self._lib.oeq_conv_forward_scratch_bytes(self.handle, nodes, nnz)

@@ -457,6 +457,60 @@ def test_float_atomic_kernels(name, make, monkeypatch):
         assert err(got, want) <= tol
 
 
+def test_float_atomic_kernels_on_a_larger_graph(monkeypatch):
+    """The float-atomics kernels (edge ranges per wave, flush with atomics at every change of receiver) on
+    2 400 nodes and about 19 000 shuffled edges: many ranges per receiver and many receivers per range."""
+    monkeypatch.setenv("OEQ_AMD_TUNE", "conv_sort=0")
+    problem = P.config2_nequip_uvu()
+    n = 2400
+    coords, rows, cols = _graph(n, 8, seed=8)
+    order = np.random.default_rng(4).permutation(len(rows))
+    rows, cols = rows[order], cols[order]
+    E = len(rows)
+    X, Y, W, G = _buffers(problem, n, E, seed=78)
+    ref = R.Problem.from_spec(problem)
+    z_ref = R.conv_forward(ref, X, Y, W, rows, cols)
+    dx_ref, dy_ref, dw_ref = R.conv_backward(ref, X, Y, W, G, rows, cols)
+    conv = oeq.TensorProductConv(problem, deterministic=False)
+    from openequivariance_amd import runtime as rt
+    from openequivariance_amd._torch import ops
+    assert ops.get_entry(conv.kid).kernels().dims["deterministic"] == rt.CONV_ATOMIC
+    tX, tY, tW = (torch.tensor(a, device="cuda", requires_grad=True) for a in (X, Y, W))
+    z = conv(tX, tY, tW, torch.tensor(rows, device="cuda"), torch.tensor(cols, device="cuda"))
+    z.backward(torch.tensor(G, device="cuda"))
+    for got, want in ((z, z_ref), (tX.grad, dx_ref), (tY.grad, dy_ref), (tW.grad, dw_ref)):
+        assert err(got, want) <= 1e-5
+
+
+def test_shared_weight_gradient_bits_do_not_depend_on_the_index_build():
+    """Shared weights: every wave group of the (bounded) backward grid sums the weight gradient over the nodes
+    it visits, so the walk order has to be a function of the edge list: the same bits from three index
+    builds, on a graph with more nodes than the grid has wave groups."""
+    from openequivariance_amd._torch import ops
+    problem = _odd(True)
+    n = 9000
+    coords, rows, cols = _graph(n, 6, seed=10)
+    order = np.random.default_rng(6).permutation(len(rows))
+    rows, cols = rows[order], cols[order]
+    E = len(rows)
+    X, Y, W, G = _buffers(problem, n, E, seed=79)
+    conv = oeq.TensorProductConv(problem, deterministic=False)
+    tX, tY, tW, tG = (torch.tensor(a, device="cuda") for a in (X, Y, W, G))
+    tr, tc = torch.tensor(rows, device="cuda"), torch.tensor(cols, device="cuda")
+    dummy = torch.zeros(1, dtype=torch.int64, device="cuda")
+    ks = ops.get_entry(conv.kid).kernels()
+    assert ks.dims["order_hops"] > 0 and ks.dims["wpartial_per_block"] > 0
+    ops.clear_index_cache()
+    first = ops.conv_backward(tX, tY, tW, tG, tr, tc, dummy, conv.kid)
+    _, _, dw_ref = R.conv_backward(R.Problem.from_spec(problem), X, Y, W, G, rows, cols)
+    assert err(first[2], dw_ref) <= 1e-5
+    for _ in range(3):
+        ops.clear_index_cache()
+        torch.randn(1 << 22, device="cuda")
+        again = ops.conv_backward(tX, tY, tW, tG, tr, tc, dummy, conv.kid)
+        assert torch.equal(again[2], first[2]) and torch.equal(again[1], first[1])
+
+
 def test_grouped_mode_handles_hubs_and_many_nodes():
     """The device-side grouping (histogram, one-block scan, scatter) over more nodes than one scan
     sweep covers, with isolated nodes and one hub that receives from and sends to 5000 nodes."""

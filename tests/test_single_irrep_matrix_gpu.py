@@ -1,8 +1,8 @@
 """Single-instruction problems over the reference's grid of multiplicities and
 irrep triples (tests/batch_test.py:145-264: powers of two, odd multiplicities 5..123,
 wide rows up to 512, mul2 > 1, l up to 7), per-row weights, forward and backward
-against the CPU oracle. Every multiplicity is paired with three of the nine irrep
-triples in rotation, so each triple is visited by at least seven multiplicities."""
+against the CPU oracle: every multiplicity with every one of the nine irrep triples, in
+both precisions, as the reference's grid does."""
 
 import numpy as np
 import pytest
@@ -27,8 +27,9 @@ def _grid(mode):
     for n, m in enumerate(MULS):
         if mode == "uvw" and m[0] > UVW_MAX_MUL:
             continue
-        for q in range(3):
-            out.append((mode, m, IRS[(3 * n + q) % len(IRS)]))
+        for irs in IRS:
+            for dtype in (np.float32, np.float64):
+                out.append((mode, m, irs, dtype))
     return out
 
 
@@ -36,15 +37,13 @@ GRID = _grid("uvu") + _grid("uvw")
 
 
 def _id(case):
-    mode, m, i = case
-    return f"{mode}-{m[0]}x{i[0]}e__x__{m[1]}x{i[1]}e---{m[2]}x{i[2]}e"
+    mode, m, i, dtype = case
+    return f"{mode}-{m[0]}x{i[0]}e__x__{m[1]}x{i[1]}e---{m[2]}x{i[2]}e-{np.dtype(dtype).name}"
 
 
 @pytest.mark.parametrize("case", GRID, ids=[_id(c) for c in GRID])
 def test_single_instruction(case):
-    mode, m, i = case
-    # every fifth case in double precision
-    dtype = np.float64 if (GRID.index(case) % 5 == 4) else np.float32
+    mode, m, i, dtype = case
     problem = oeq.TPProblem(f"{m[0]}x{i[0]}e", f"{m[1]}x{i[1]}e", f"{m[2]}x{i[2]}e", [(0, 0, 0, mode, True)],
                             shared_weights=False, internal_weights=False, irrep_dtype=dtype, weight_dtype=dtype)
     tol = tol_of(problem)

@@ -218,3 +218,29 @@ def test_numpy_interface():
         A = rng.uniform(size=X.shape).astype(np.float32)
         second = conv.double_backward_cpu(X, Y, G, W, np.zeros_like(W), A, np.zeros_like(Y), graph)
         assert err(second[3], R.conv_forward(ref, A, Y, W, graph.rows, graph.cols)) <= 1e-5
+
+
+def test_conv_under_inference_mode():
+    """Edge tensors made under torch.inference_mode() carry no version counter: the ops build the index of
+    such an edge list at every call instead of caching it, and the results are the usual ones."""
+    from openequivariance_amd._torch import ops
+    from openequivariance_amd.core.graph import CoordGraph, periodic_radius_graph
+    problem = P.config2_nequip_uvu()
+    coords, rows, cols, _ = periodic_radius_graph(50, 8.0, 5.0, seed=3)
+    g = CoordGraph(coords, rows, cols)
+    rng = np.random.default_rng(3)
+    X = rng.normal(size=(50, problem.irreps_in1.dim)).astype(np.float32)
+    Y = rng.normal(size=(g.nnz, problem.irreps_in2.dim)).astype(np.float32)
+    W = rng.normal(size=(g.nnz, problem.weight_numel)).astype(np.float32)
+    z_ref = R.conv_forward(R.Problem.from_spec(problem), X, Y, W, g.rows, g.cols)
+    for det in (True, False):
+        conv = oeq.TensorProductConv(problem, deterministic=det)
+        ops.clear_index_cache()
+        with torch.inference_mode():
+            tX, tY, tW = to_gpu(X, Y, W)
+            tr, tc, tp = (torch.tensor(a, device="cuda") for a in (g.rows, g.cols, g.transpose_perm))
+            assert tr.is_inference()
+            z = conv(tX, tY, tW, tr, tc, tp if det else None)
+            z2 = conv(tX, tY, tW, tr, tc, tp if det else None)
+        assert err(z, z_ref) <= 1e-5 and torch.equal(z, z2)
+        assert not ops._index_cache, "nothing is kept for tensors whose changes cannot be seen"

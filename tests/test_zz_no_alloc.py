@@ -49,13 +49,48 @@ def test_static_forward_matches_workspace_forward(deterministic):
                         c.data_ptr(), ws.data_ptr(), nb, stream)
         got = torch.full((n_nodes, L3), float("nan"), device="cuda")
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
+        # free device memory as the driver reports it (hipMemGetInfo): an allocation inside the library would
+        # show here, which torch's own allocator statistics could not see
+        before = torch.cuda.mem_get_info()[0]
         ks.conv_forward_static(n_nodes, E, X.data_ptr(), Y.data_ptr(), W.data_ptr(), got.data_ptr(), r.data_ptr(),
                                c.data_ptr(), stream)
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == before
         assert torch.isfinite(want).all()
         assert torch.equal(got, want), (n_nodes, deterministic)
+
+
+def test_static_forward_under_graph_capture():
+    """The call records nothing but kernel launches, so a HIP graph can hold it: every replay (with eager
+    work and synchronisations in between) reproduces the eager result."""
+    problem = P.config2_nequip_uvu()
+    src, dims, descs = build_conv_module(problem, False)
+    ks = rt.get_kernel_set(src, dims, descs)
+    X, Y, W, r, c = _case(200, 8, 4, False, problem)
+    n_nodes, E = X.shape[0], r.shape[0]
+    want = torch.empty(n_nodes, problem.irreps_out.dim, device="cuda")
+    nb = ks.conv_forward_workspace_bytes(n_nodes, E)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    ks.conv_forward(n_nodes, E, X.data_ptr(), Y.data_ptr(), W.data_ptr(), want.data_ptr(), r.data_ptr(), c.data_ptr(),
+                    ws.data_ptr(), nb, torch.cuda.current_stream().cuda_stream)  # also loads the kernels
+    got = torch.zeros_like(want)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the capture stream
+        ks.conv_forward_static(n_nodes, E, X.data_ptr(), Y.data_ptr(), W.data_ptr(), got.data_ptr(), r.data_ptr(),
+                               c.data_ptr(), side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ks.conv_forward_static(n_nodes, E, X.data_ptr(), Y.data_ptr(), W.data_ptr(), got.data_ptr(), r.data_ptr(),
+                               c.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        got.fill_(float("nan"))
+        torch.randn(1 << 20, device="cuda").sum().item()  # eager work and a synchronisation between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), rep
 
 
 def test_static_forward_refuses_what_it_cannot_do():
