@@ -8,9 +8,14 @@ registrations of fake kernels, autograd and autocast
 (openequivariance/openequivariance/_torch/TensorProduct.py:182-374,
 _torch/TensorProductConv.py:280-568).
 
-The ops take an integer ``kid`` naming a compiled kernel set in a process-wide
-registry instead of a JSON byte tensor. Argument checks raise ``RuntimeError``
-with the reference's wording (torch_core.hpp:109-134).
+Like the reference's ops (``Tensor json_bytes, int hash``, torch_core.hpp:637-643)
+every op takes the description of its kernel set: ``kid``, a 63-bit hash of the
+serialised problem and flags, and ``spec``, a uint8 tensor holding those bytes.
+The hash finds the compiled kernel set in a process-wide registry; a process
+that has never seen it (an exported program loaded elsewhere) rebuilds the set
+from the bytes, so a traced graph means the same thing in every process.
+Callers inside one process may leave ``spec`` out. Argument checks raise
+``RuntimeError`` with the reference's wording (torch_core.hpp:109-134).
 
 Second and higher derivatives need no extra kernels: with
 S(x, y, w, g) = <g, TP(x, y, w)> multilinear, the backward op returns
@@ -20,6 +25,10 @@ forward and three backward calls with one argument replaced by a cotangent.
 
 from __future__ import annotations
 
+import contextlib
+import hashlib
+import json
+import os
 import threading
 from typing import Dict, List, Optional, Tuple
 
@@ -28,8 +37,7 @@ import torch
 from .. import runtime as rt
 
 _registry: Dict[int, "KernelEntry"] = {}
-_registry_lock = threading.Lock()
-_next_id = [1]
+_registry_lock = threading.RLock()
 
 
 class KernelEntry:
@@ -42,6 +50,7 @@ class KernelEntry:
         self.shared = shared
         self.dtype = torch_dtype
         self.deterministic = deterministic
+        self.spec: Optional[torch.Tensor] = None  # the bytes this entry was built from (uint8, host)
         self._ks: Optional[rt.KernelSet] = None
         self._lock = threading.Lock()
 
@@ -54,19 +63,99 @@ class KernelEntry:
         return self._ks
 
 
-def register_entry(entry: KernelEntry) -> int:
+# ---------------------------------------------------------------------------
+# kernel sets by description
+# ---------------------------------------------------------------------------
+
+_tune_lock = threading.RLock()
+
+
+@contextlib.contextmanager
+def _tune_env(tune: str):
+    """The kernel-shape knobs (``OEQ_AMD_TUNE``) that were in force when a description was written are part
+    of it: they are put back while its kernels are generated, whenever and wherever that happens."""
+    with _tune_lock:
+        saved = os.environ.get("OEQ_AMD_TUNE")
+        os.environ["OEQ_AMD_TUNE"] = tune
+        try:
+            yield
+        finally:
+            if saved is None:
+                os.environ.pop("OEQ_AMD_TUNE", None)
+            else:
+                os.environ["OEQ_AMD_TUNE"] = saved
+
+
+def make_spec(kind: str, problem, deterministic: bool = False, kahan: bool = False) -> bytes:
+    """Serialised description of a kernel set: ``kind`` 'tp' or 'conv', the problem, the module's flags and
+    the tuning knobs in force (cf. the reference's kernel JSON, torch_core.hpp:144-178)."""
+    from ..core.spec import problem_to_dict
+    assert kind in ("tp", "conv")
+    desc = {"v": 1, "kind": kind, "problem": problem_to_dict(problem), "deterministic": bool(deterministic),
+            "kahan": bool(kahan), "tune": os.environ.get("OEQ_AMD_TUNE", "")}
+    return json.dumps(desc, sort_keys=True, separators=(",", ":")).encode()
+
+
+def spec_hash(spec: bytes) -> int:
+    return int.from_bytes(hashlib.sha256(spec).digest()[:8], "little") & ((1 << 63) - 1)
+
+
+def _entry_from_spec(spec: bytes) -> KernelEntry:
+    from ..codegen.lower import lower
+    from ..core.spec import problem_from_dict
+    from .tensor_product import build_tp_module
+    from .tensor_product_conv import build_conv_module, fused
+    from .utils import oeq_to_torch_dtype
+    desc = json.loads(spec.decode())
+    if desc.get("v") != 1 or desc.get("kind") not in ("tp", "conv"):
+        raise RuntimeError("unreadable kernel-set description")
+    problem = problem_from_dict(desc["problem"])
+    tune, det, kahan = desc["tune"], desc["deterministic"], desc["kahan"]
+    low = lower(problem)
+    dtype = oeq_to_torch_dtype(problem.irrep_dtype)
+    if desc["kind"] == "tp":
+        def build():
+            with _tune_env(tune):
+                return build_tp_module(problem)
+        entry = KernelEntry(build, low.L1, low.L2, low.L3, low.WN, low.shared_weights, dtype)
+    else:
+        def build():
+            with _tune_env(tune):
+                return build_conv_module(problem, det, kahan)
+        with _tune_env(tune):
+            unfused = not fused(low)
+        entry = KernelEntry(build, low.L1, low.L2, low.L3, low.WN, low.shared_weights, dtype, deterministic=det,
+                            unfused=unfused)
+    entry.spec = torch.frombuffer(bytearray(spec), dtype=torch.uint8)
+    return entry
+
+
+def register_spec(spec: bytes) -> int:
+    """The id of the kernel set a description stands for (its hash); the set is entered into the registry
+    unless it is there already. Kernels are generated and compiled at first use."""
+    kid = spec_hash(spec)
     with _registry_lock:
-        kid = _next_id[0]
-        _next_id[0] += 1
-        _registry[kid] = entry
-        return kid
+        if kid not in _registry:
+            _registry[kid] = _entry_from_spec(spec)
+    return kid
 
 
-def get_entry(kid: int) -> KernelEntry:
+def get_entry(kid: int, spec: Optional[torch.Tensor] = None) -> KernelEntry:
+    entry = _registry.get(kid)
+    if entry is not None:
+        return entry
+    if spec is None:
+        raise RuntimeError(f"unknown kernel id {kid}: no kernel set with this hash in this process, and the "
+                           "call carries no description to build it from")
     try:
-        return _registry[kid]
-    except KeyError:
-        raise RuntimeError(f"unknown kernel id {kid}")
+        data = bytes(spec.detach().cpu().contiguous().numpy().tobytes())
+    except Exception as exc:  # a tensor without data: tracing in a process that never built this kernel set
+        raise RuntimeError(f"kernel id {kid} is unknown in this process and its description cannot be read "
+                           "while tracing; call the module once outside tracing first") from exc
+    if spec_hash(data) != kid:
+        raise RuntimeError(f"kernel id {kid} does not match the description that came with it")
+    register_spec(data)
+    return _registry[kid]
 
 
 _DTYPE_CODE = {torch.float32: 1, torch.float64: 2, torch.int32: 3, torch.int64: 4, torch.uint8: 5}
@@ -101,8 +190,9 @@ def _wshape(e: KernelEntry, n: int) -> List[int]:
 
 
 @torch.library.custom_op("oeq_amd::tp_forward", mutates_args=(), device_types="cuda")
-def tp_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, kid: int) -> torch.Tensor:
-    e = get_entry(kid)
+def tp_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, kid: int,
+               spec: Optional[torch.Tensor] = None) -> torch.Tensor:
+    e = get_entry(kid, spec)
     n = L1_in.shape[0] if L1_in.dim() > 0 else -1
     check_tensor(L1_in, [n, e.L1], e.dtype, "L1_in")
     check_tensor(L2_in, [n, e.L2], e.dtype, "L2_in")
@@ -115,15 +205,15 @@ def tp_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, kid: i
 
 
 @tp_forward.register_fake
-def _(L1_in, L2_in, W, kid):
-    e = get_entry(kid)
+def _(L1_in, L2_in, W, kid, spec=None):
+    e = get_entry(kid, spec)
     return L1_in.new_empty((L1_in.shape[0], e.L3))
 
 
 @torch.library.custom_op("oeq_amd::tp_backward", mutates_args=(), device_types="cuda")
 def tp_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_grad: torch.Tensor,
-                kid: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    e = get_entry(kid)
+                kid: int, spec: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    e = get_entry(kid, spec)
     n = L1_in.shape[0] if L1_in.dim() > 0 else -1
     check_tensor(L1_in, [n, e.L1], e.dtype, "L1_in")
     check_tensor(L2_in, [n, e.L2], e.dtype, "L2_in")
@@ -141,26 +231,26 @@ def tp_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_gr
 
 
 @tp_backward.register_fake
-def _(L1_in, L2_in, W, L3_grad, kid):
+def _(L1_in, L2_in, W, L3_grad, kid, spec=None):
     return torch.empty_like(L1_in), torch.empty_like(L2_in), torch.empty_like(W)
 
 
 def _tp_fwd_setup(ctx, inputs, output):
-    ctx.kid = inputs[3]
+    ctx.kid, ctx.spec = inputs[3], inputs[4]
     ctx.save_for_backward(inputs[0], inputs[1], inputs[2])
 
 
 def _tp_fwd_backward(ctx, grad):
     x, y, w = ctx.saved_tensors
-    dx, dy, dw = tp_backward(x, y, w, grad, ctx.kid)
-    return dx, dy, dw, None
+    dx, dy, dw = tp_backward(x, y, w, grad, ctx.kid, ctx.spec)
+    return dx, dy, dw, None, None
 
 
 tp_forward.register_autograd(_tp_fwd_backward, setup_context=_tp_fwd_setup)
 
 
 def _tp_bwd_setup(ctx, inputs, output):
-    ctx.kid = inputs[4]
+    ctx.kid, ctx.spec = inputs[4], inputs[5]
     ctx.save_for_backward(inputs[0], inputs[1], inputs[2], inputs[3])
 
 
@@ -201,12 +291,12 @@ def _second_order(forward, backward, x, y, w, g, ddx, ddy, ddw):
 FUSED_DOUBLE_BACKWARD = True
 
 
-def _use_fused(kid, ddx, ddy, ddw) -> bool:
+def _use_fused(kid, spec, ddx, ddy, ddw) -> bool:
     if not FUSED_DOUBLE_BACKWARD or torch.is_grad_enabled():
         return False
     if sum(t is not None for t in (ddx, ddy, ddw)) < 2:
         return False
-    return get_entry(kid).kernels().has_double_backward()
+    return get_entry(kid, spec).kernels().has_double_backward()
 
 
 def _zeros_if_none(t, like):
@@ -216,10 +306,11 @@ def _zeros_if_none(t, like):
 @torch.library.custom_op("oeq_amd::tp_double_backward", mutates_args=(), device_types="cuda")
 def tp_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_grad: torch.Tensor,
                        L1_dgrad: torch.Tensor, L2_dgrad: torch.Tensor, W_dgrad: torch.Tensor,
-                       kid: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                       kid: int, spec: Optional[torch.Tensor] = None
+                       ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """(L1_grad, L2_grad, W_grad, L3_dgrad): the op of the reference's jit_tp_double_backward
     (extension/torch_core.hpp:357-420)."""
-    e = get_entry(kid)
+    e = get_entry(kid, spec)
     n = L1_in.shape[0] if L1_in.dim() > 0 else -1
     for t, name in ((L1_in, "L1_in"), (L1_dgrad, "L1_dgrad")):
         check_tensor(t, [n, e.L1], e.dtype, name)
@@ -242,20 +333,20 @@ def tp_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor
 
 
 @tp_double_backward.register_fake
-def _(L1_in, L2_in, W, L3_grad, L1_dgrad, L2_dgrad, W_dgrad, kid):
+def _(L1_in, L2_in, W, L3_grad, L1_dgrad, L2_dgrad, W_dgrad, kid, spec=None):
     return torch.empty_like(L1_in), torch.empty_like(L2_in), torch.empty_like(W), torch.empty_like(L3_grad)
 
 
 def _tp_bwd_backward(ctx, ddx, ddy, ddw):
     x, y, w, g = ctx.saved_tensors
-    kid = ctx.kid
-    if _use_fused(kid, ddx, ddy, ddw):
+    kid, spec = ctx.kid, ctx.spec
+    if _use_fused(kid, spec, ddx, ddy, ddw):
         dx, dy, dw, gg = tp_double_backward(x, y, w, g, _zeros_if_none(ddx, x), _zeros_if_none(ddy, y),
-                                            _zeros_if_none(ddw, w), kid)
-        return dx, dy, dw, gg, None
-    dx, dy, dw, gg = _second_order(lambda a, b, c: tp_forward(a, b, c, kid),
-                                   lambda a, b, c, d: tp_backward(a, b, c, d, kid), x, y, w, g, ddx, ddy, ddw)
-    return dx, dy, dw, gg, None
+                                            _zeros_if_none(ddw, w), kid, spec)
+        return dx, dy, dw, gg, None, None
+    dx, dy, dw, gg = _second_order(lambda a, b, c: tp_forward(a, b, c, kid, spec),
+                                   lambda a, b, c, d: tp_backward(a, b, c, d, kid, spec), x, y, w, g, ddx, ddy, ddw)
+    return dx, dy, dw, gg, None, None
 
 
 tp_backward.register_autograd(_tp_bwd_backward, setup_context=_tp_bwd_setup)
@@ -458,8 +549,9 @@ def _unfused_double_backward(e, ks, x, y, w, g, a, b, c, r, cc, p, nodes, nnz):
 
 @torch.library.custom_op("oeq_amd::conv_forward", mutates_args=(), device_types="cuda")
 def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows: torch.Tensor,
-                 cols: torch.Tensor, transpose_perm: torch.Tensor, kid: int) -> torch.Tensor:
-    e = get_entry(kid)
+                 cols: torch.Tensor, transpose_perm: torch.Tensor, kid: int,
+                 spec: Optional[torch.Tensor] = None) -> torch.Tensor:
+    e = get_entry(kid, spec)
     nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm)
     x, y, w = L1_in.contiguous(), L2_in.contiguous(), W.contiguous()
     r, c = rows.contiguous(), cols.contiguous()
@@ -487,16 +579,16 @@ def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows
 
 
 @conv_forward.register_fake
-def _(L1_in, L2_in, W, rows, cols, transpose_perm, kid):
-    e = get_entry(kid)
+def _(L1_in, L2_in, W, rows, cols, transpose_perm, kid, spec=None):
+    e = get_entry(kid, spec)
     return L1_in.new_empty((L1_in.shape[0], e.L3))
 
 
 @torch.library.custom_op("oeq_amd::conv_backward", mutates_args=(), device_types="cuda")
 def conv_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_grad: torch.Tensor,
                   rows: torch.Tensor, cols: torch.Tensor, transpose_perm: torch.Tensor,
-                  kid: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    e = get_entry(kid)
+                  kid: int, spec: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    e = get_entry(kid, spec)
     nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm, L3_grad)
     x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
     r, c, p = rows.contiguous(), cols.contiguous(), transpose_perm.contiguous()
@@ -522,26 +614,26 @@ def conv_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_
 
 
 @conv_backward.register_fake
-def _(L1_in, L2_in, W, L3_grad, rows, cols, transpose_perm, kid):
+def _(L1_in, L2_in, W, L3_grad, rows, cols, transpose_perm, kid, spec=None):
     return torch.empty_like(L1_in), torch.empty_like(L2_in), torch.empty_like(W)
 
 
 def _conv_fwd_setup(ctx, inputs, output):
-    ctx.kid = inputs[6]
+    ctx.kid, ctx.spec = inputs[6], inputs[7]
     ctx.save_for_backward(*inputs[:6])
 
 
 def _conv_fwd_backward(ctx, grad):
     x, y, w, rows, cols, perm = ctx.saved_tensors
-    dx, dy, dw = conv_backward(x, y, w, grad, rows, cols, perm, ctx.kid)
-    return dx, dy, dw, None, None, None, None
+    dx, dy, dw = conv_backward(x, y, w, grad, rows, cols, perm, ctx.kid, ctx.spec)
+    return dx, dy, dw, None, None, None, None, None
 
 
 conv_forward.register_autograd(_conv_fwd_backward, setup_context=_conv_fwd_setup)
 
 
 def _conv_bwd_setup(ctx, inputs, output):
-    ctx.kid = inputs[7]
+    ctx.kid, ctx.spec = inputs[7], inputs[8]
     ctx.save_for_backward(*inputs[:7])
 
 
@@ -549,10 +641,11 @@ def _conv_bwd_setup(ctx, inputs, output):
 def conv_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_grad: torch.Tensor,
                          L1_dgrad: torch.Tensor, L2_dgrad: torch.Tensor, W_dgrad: torch.Tensor,
                          rows: torch.Tensor, cols: torch.Tensor, transpose_perm: torch.Tensor,
-                         kid: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                         kid: int, spec: Optional[torch.Tensor] = None
+                         ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """(L1_grad, L2_grad, W_grad, L3_dgrad): the op of the reference's jit_conv_double_backward
     (extension/torch_core.hpp:544-625)."""
-    e = get_entry(kid)
+    e = get_entry(kid, spec)
     nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm, L3_grad)
     _conv_checks(e, L1_dgrad, L2_dgrad, W_dgrad, rows, cols, transpose_perm)
     x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
@@ -581,21 +674,21 @@ def conv_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tens
 
 
 @conv_double_backward.register_fake
-def _(L1_in, L2_in, W, L3_grad, L1_dgrad, L2_dgrad, W_dgrad, rows, cols, transpose_perm, kid):
+def _(L1_in, L2_in, W, L3_grad, L1_dgrad, L2_dgrad, W_dgrad, rows, cols, transpose_perm, kid, spec=None):
     return torch.empty_like(L1_in), torch.empty_like(L2_in), torch.empty_like(W), torch.empty_like(L3_grad)
 
 
 def _conv_bwd_backward(ctx, ddx, ddy, ddw):
     x, y, w, g, rows, cols, perm = ctx.saved_tensors
-    kid = ctx.kid
-    if _use_fused(kid, ddx, ddy, ddw):
+    kid, spec = ctx.kid, ctx.spec
+    if _use_fused(kid, spec, ddx, ddy, ddw):
         dx, dy, dw, gg = conv_double_backward(x, y, w, g, _zeros_if_none(ddx, x), _zeros_if_none(ddy, y),
-                                              _zeros_if_none(ddw, w), rows, cols, perm, kid)
-        return dx, dy, dw, gg, None, None, None, None
-    dx, dy, dw, gg = _second_order(lambda a, b, c: conv_forward(a, b, c, rows, cols, perm, kid),
-                                   lambda a, b, c, d: conv_backward(a, b, c, d, rows, cols, perm, kid),
+                                              _zeros_if_none(ddw, w), rows, cols, perm, kid, spec)
+        return dx, dy, dw, gg, None, None, None, None, None
+    dx, dy, dw, gg = _second_order(lambda a, b, c: conv_forward(a, b, c, rows, cols, perm, kid, spec),
+                                   lambda a, b, c, d: conv_backward(a, b, c, d, rows, cols, perm, kid, spec),
                                    x, y, w, g, ddx, ddy, ddw)
-    return dx, dy, dw, gg, None, None, None, None
+    return dx, dy, dw, gg, None, None, None, None, None
 
 
 conv_backward.register_autograd(_conv_bwd_backward, setup_context=_conv_bwd_setup)

@@ -49,11 +49,11 @@ class TensorProduct(TensorProductTiming, torch.nn.Module):
         self.weight_numel = problem.weight_numel
         self.is_uvw = low.mode == "uvw"
         self._low = low
-        entry = ops.KernelEntry(
-            lambda p=problem: build_tp_module(p), low.L1, low.L2, low.L3, low.WN, low.shared_weights,
-            oeq_to_torch_dtype(problem.irrep_dtype),
-        )
-        self.kid = ops.register_entry(entry)
+        # The ops are handed the kernel set's description (a hash and the bytes it is the hash of), so that a
+        # traced or exported graph can rebuild the kernels in a process that never constructed this module.
+        # A plain attribute, not a buffer: it stays in host memory whatever the module is moved to.
+        self.kid = ops.register_spec(ops.make_spec("tp", problem))
+        self.spec = ops.get_entry(self.kid).spec
 
     # -- dtype handling (TensorProduct.py:55-92) ---------------------------------
     def to(self, *args, **kwargs):
@@ -107,4 +107,4 @@ class TensorProduct(TensorProductTiming, torch.nn.Module):
         :param W: ``[batch, weight_numel]``, or ``[weight_numel]`` when ``shared_weights``
         :return: ``[batch, problem.irreps_out.dim]``
         """
-        return ops.tp_forward(x, y, W, self.kid)
+        return ops.tp_forward(x, y, W, self.kid, self.spec)

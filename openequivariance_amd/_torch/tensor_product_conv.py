@@ -97,13 +97,9 @@ class TensorProductConv(ConvolutionTiming, torch.nn.Module):
         self.L1, self.L2, self.L3 = problem.irreps_in1, problem.irreps_in2, problem.irreps_out
         self.L3_dim = low.L3
         self.weight_numel = problem.weight_numel
-        entry = ops.KernelEntry(
-            lambda p=problem, d=deterministic, k=kahan: build_conv_module(p, d, k), low.L1, low.L2, low.L3, low.WN,
-            low.shared_weights, oeq_to_torch_dtype(problem.irrep_dtype), deterministic=deterministic,
-            unfused=not fused(low),
-        )
-        self.kid = ops.register_entry(entry)
-        self._dummy_perm = None
+        # the kernel set's description travels with every op call (see TensorProduct._init_class)
+        self.kid = ops.register_spec(ops.make_spec("conv", problem, deterministic, kahan))
+        self.spec = ops.get_entry(self.kid).spec
 
     def to(self, *args, **kwargs):
         _device, dtype, _nb, _fmt = torch._C._nn._parse_to(*args, **kwargs)
@@ -162,7 +158,7 @@ class TensorProductConv(ConvolutionTiming, torch.nn.Module):
         if sender_perm is None:
             if self.deterministic:
                 raise RuntimeError("Shape mismatch for tensor 'transpose perm'. deterministic=True needs sender_perm")
-            if self._dummy_perm is None or self._dummy_perm.device != rows.device:
-                self._dummy_perm = torch.zeros(1, dtype=torch.int64, device=rows.device)
-            sender_perm = self._dummy_perm
-        return ops.conv_forward(X, Y, W, rows, cols, sender_perm, self.kid)
+            # any int64 tensor fills the op's slot (it is not read in this mode); the receivers are at hand, and
+            # handing them over creates no tensor and sets no attribute while a program is being traced
+            sender_perm = rows
+        return ops.conv_forward(X, Y, W, rows, cols, sender_perm, self.kid, self.spec)

@@ -456,3 +456,48 @@ class TPProblem:
                 f" {ins.path_weight:<6.4f} |"
             )
         return "\n".join(lines) + "\n"
+
+
+def problem_to_dict(problem: TPProblem) -> dict:
+    """The state of a problem as plain JSON-able data, for ``problem_from_dict`` in another process: the
+    constructor's arguments plus what callers may have changed afterwards (dtypes, weight sharing, layout,
+    the normalised instructions). Floats are written as hexadecimal strings, so nothing is rounded.
+    (The reference ships its kernels' description to its ops as JSON bytes the same way,
+    openequivariance/openequivariance/extension/torch_core.hpp:144-178, 637-643.)"""
+    def fl(v):
+        return None if v is None else [float(x).hex() for x in v]
+
+    def raw(ins):
+        ins = tuple(ins)
+        return [int(ins[0]), int(ins[1]), int(ins[2]), str(ins[3]), bool(ins[4])] + \
+            ([float(ins[5]).hex()] if len(ins) > 5 else [])
+
+    return {
+        "irreps_in1": str(problem.irreps_in1), "irreps_in2": str(problem.irreps_in2),
+        "irreps_out": str(problem.irreps_out),
+        "instructions_raw": [raw(i) for i in problem.instructions_raw],
+        "instructions": [[int(i.i_in1), int(i.i_in2), int(i.i_out), str(i.connection_mode), bool(i.has_weight),
+                          float(i.path_weight).hex(), [int(d) for d in i.path_shape]] for i in problem.instructions],
+        "in1_var": fl(problem.in1_var), "in2_var": fl(problem.in2_var), "out_var": fl(problem.out_var),
+        "irrep_normalization": problem.irrep_normalization, "path_normalization": problem.path_normalization,
+        "internal_weights": bool(problem.internal_weights), "shared_weights": bool(problem.shared_weights),
+        "label": problem.label, "layout": problem.layout,
+        "irrep_dtype": np.dtype(problem.irrep_dtype).name, "weight_dtype": np.dtype(problem.weight_dtype).name,
+    }
+
+
+def problem_from_dict(d: dict) -> TPProblem:
+    def fl(v):
+        return None if v is None else [float.fromhex(x) for x in v]
+
+    raw = [tuple(i[:5]) + ((float.fromhex(i[5]),) if len(i) > 5 else ()) for i in d["instructions_raw"]]
+    problem = TPProblem(
+        d["irreps_in1"], d["irreps_in2"], d["irreps_out"], raw, in1_var=fl(d["in1_var"]), in2_var=fl(d["in2_var"]),
+        out_var=fl(d["out_var"]), irrep_normalization=d["irrep_normalization"],
+        path_normalization=d["path_normalization"], internal_weights=d["internal_weights"],
+        shared_weights=d["shared_weights"], label=d["label"],
+        irrep_dtype=np.dtype(d["irrep_dtype"]).type, weight_dtype=np.dtype(d["weight_dtype"]).type, layout=d["layout"])
+    problem.instructions = [Instruction(i[0], i[1], i[2], i[3], i[4], float.fromhex(i[5]), tuple(i[6]))
+                            for i in d["instructions"]]
+    problem.weight_numel = sum(math.prod(ins.path_shape) for ins in problem.instructions if ins.has_weight)
+    return problem
