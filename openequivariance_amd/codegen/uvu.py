@@ -205,33 +205,41 @@ class UvuEmitter:
             s(f"woff{q} = (t >> 4) * {st['U']} + chunk * 64 + (t & 15) * 4;")
             s.close()
 
-    def _emit_stage_issue(self, s: Src, e: str):
+    def _emit_stage_issue(self, s: Src, e: str, x: bool = True, w: bool = True, wbuf: Optional[str] = None):
+        """Request the operands of edge ``e``: ``x`` = the sender's X slice and the edge's Y, ``w`` = the
+        edge's weights, into the second weight buffer of the wave where ``wbuf`` (an expression, 0 or 1)
+        says so."""
         low, st = self.low, self.stage
         s.open("")
         s(f"const i64 eid = OEQ_EDGE({e});")
-        s(f"const T* sx = L1_in + oeq_idx(cols[eid], node_count) * {low.L1};")
-        s(f"const T* sw = W + eid * {low.WN};")
-        for q in range(st["nqx"]):
-            s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sx + xoff{q}), (OEQ_LPTR)(&s_stage[wave][{q * 256}]), 16, 0, 0);")
-        for q in range(st["nqw"]):
-            s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sw + woff{q}), "
-              f"(OEQ_LPTR)(&s_stage[wave][{st['XF'] + q * 256}]), 16, 0, {2 if self.nt & 1 else 0});")
-        if self.use_q:
-            for r in range(self.q_slabs):
-                s(f"yn[{r}] = L2_in[eid * {low.L2} + qt.j[{r}]];")
-        else:
-            for j in range(low.L2):
-                s(f"yn[{j}] = L2_in[eid * {low.L2} + {j}];")
+        if x:
+            s(f"const T* sx = L1_in + oeq_idx(cols[eid], node_count) * {low.L1};")
+            for q in range(st["nqx"]):
+                s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sx + xoff{q}), "
+                  f"(OEQ_LPTR)(&s_stage[wave][{q * 256}]), 16, 0, 0);")
+            if self.use_q:
+                for r in range(self.q_slabs):
+                    s(f"yn[{r}] = L2_in[eid * {low.L2} + qt.j[{r}]];")
+            else:
+                for j in range(low.L2):
+                    s(f"yn[{j}] = L2_in[eid * {low.L2} + {j}];")
+        if w:
+            s(f"const T* sw = W + eid * {low.WN};")
+            base = f"{st['XF']}" if wbuf is None else f"{st['XF']} + ({wbuf}) * {st['nqw'] * 256}"
+            for q in range(st["nqw"]):
+                s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sw + woff{q}), "
+                  f"(OEQ_LPTR)(&s_stage[wave][{base} + {q * 256}]), 16, 0, {2 if self.nt & 1 else 0});")
         s.close()
 
-    def _emit_stage_read(self, s: Src, buf: str):
+    def _emit_stage_read(self, s: Src, buf: str, wbuf: Optional[str] = None):
         low, st = self.low, self.stage
+        wbase = f"{st['XF']}" if wbuf is None else f"{st['XF']} + ({wbuf}) * {st['nqw'] * 256}"
         for b in self.used_in1:
             blk = low.in1[b]
             for i in range(blk.d):
                 s(f"{buf}.x.b{b}[{i}] = s_stage[wave][{self._stage_x(blk, st['xl'][b], i)}];")
         for p in low.paths:
-            s(f"{buf}.w[{self.wslot[p.index]}] = s_stage[wave][{st['XF'] + p.index * 64} + ul];")
+            s(f"{buf}.w[{self.wslot[p.index]}] = s_stage[wave][{wbase} + {p.index * 64} + ul];")
         if self.use_q:
             for r in range(self.q_slabs):
                 s(f"{buf}.yq[{r}] = yn[{r}];")
@@ -1009,6 +1017,44 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             s("e += 2;")
             s.close()
             return
+        if pipelined == 4:
+            # As below (one staging buffer, copied to registers), with the weights two edges ahead in a second
+            # weight buffer: while edge e is computed, X / Y of e+1 and the weights of e+1 and e+2 are in
+            # flight, 16 KB per wave at the MACE shape instead of 10. With 8 waves per CU one edge of prefetch
+            # keeps too few bytes in flight to fill the memory system (the forward with its arithmetic taken
+            # out ran no faster). Vector-memory results return in issue order, so waiting until only the
+            # youngest weight loads are outstanding means everything of edge e has arrived.
+            nqw = self.stage["nqw"]
+            s(f"T yn[{self.q_slabs if self.use_q else self.low.L2}];")
+            s(f"i64 e = {first};")
+            s("int wpar = 0;")
+            s.open(f"if (e < {last})")
+            self._emit_stage_issue(s, "e", x=True, w=True, wbuf="0")
+            s.open(f"if (e + 1 < {last})")
+            self._emit_stage_issue(s, "e + 1", x=False, w=True, wbuf="1")
+            s.close()
+            s.close()
+            s.open(f"while (e < {last})")
+            s.open(f"if (e + 1 < {last})")
+            s(vmcnt(nqw))
+            s.close()
+            s.open("else")
+            s(vmcnt(0))
+            s.close()
+            self._emit_stage_read(s, "A", wbuf="wpar")
+            s(lgkm0)
+            s.open(f"if (e + 1 < {last})")
+            self._emit_stage_issue(s, "e + 1", x=True, w=False)
+            s.open(f"if (e + 2 < {last})")
+            self._emit_stage_issue(s, "e + 2", x=False, w=True, wbuf="wpar")
+            s.close()
+            s.close()
+            if before_edge:
+                before_edge("e")
+            compute("A", "e")
+            s("++e; wpar ^= 1;")
+            s.close()
+            return
         if pipelined == 2:
             # one LDS buffer per wave, copied to registers before the next edge's loads are issued
             s(f"T yn[{self.q_slabs if self.use_q else self.low.L2}];")
@@ -1066,6 +1112,8 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         2: next edge's operands prefetched into the wave's LDS staging buffer."""
         if pipelined == 3 and self.stage3 is not None and not self.use_q:
             return 3
+        if pipelined == 4 and self.stage is not None and self.R == 1:
+            return 4
         if pipelined >= 2 and self.stage is not None:
             return 2
         if pipelined and self.can_preload:
@@ -1130,7 +1178,9 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         segw = self.seg_waves if deterministic else 1
         block = 64 * self.NCH * G * segw
         R = self.R
-        mode = self._edge_mode(pipelined)
+        # weights two edges ahead: only where the loop body issues no stores or atomics (they share the
+        # vector-memory counter with the loads the loop waits for by count)
+        mode = self._edge_mode(pipelined if (deterministic or pipelined != 4) else 2)
         s.open(
             f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void forward(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
@@ -1143,8 +1193,9 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             self._emit_q_prologue(s, block // 64)
         if self.can_preload:
             s("E_t A, B;")
-        if mode == 2:
-            s(f"__shared__ __attribute__((aligned(16))) T s_stage[{self.NCH * G}][{self.stage['floats']}];")
+        if mode in (2, 4):
+            floats = self.stage["floats"] + (self.stage["nqw"] * 256 if mode == 4 else 0)
+            s(f"__shared__ __attribute__((aligned(16))) T s_stage[{self.NCH * G}][{floats}];")
             self._emit_stage_offsets(s)
         if mode == 3:
             for b in "AB":
@@ -1901,7 +1952,7 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         if self.NCH > 1:
             G = 1  # one node (or edge range) per block: the per-edge dY reduction uses block barriers
         block = 64 * self.NCH * G
-        mode = self._edge_mode(pipelined)
+        mode = self._edge_mode(2 if pipelined == 4 else pipelined)  # the body stores: see emit_conv_forward
         if self.can_preload:
             self._emit_load_edge(s, "load_edge_b", self.used_in1, low.paths)
             if self.chunk_split and deterministic:
@@ -1926,8 +1977,9 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             s(f"for (int t = 0; t < {self.n_wslots}; ++t) dwacc[t] = T(0);")
         if self.can_preload:
             s("E_t A, B;")
-        if mode == 2:
-            s(f"__shared__ __attribute__((aligned(16))) T s_stage[{self.NCH * G}][{self.stage['floats']}];")
+        if mode in (2, 4):
+            floats = self.stage["floats"] + (self.stage["nqw"] * 256 if mode == 4 else 0)
+            s(f"__shared__ __attribute__((aligned(16))) T s_stage[{self.NCH * G}][{floats}];")
             self._emit_stage_offsets(s)
         if mode == 3:
             for b in "AB":

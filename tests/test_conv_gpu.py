@@ -568,6 +568,7 @@ def test_grouping_orders_long_segments(hubs, degree):
 
 
 KNOBS = ["conv_pipe_f=0,conv_pipe_b=1", "conv_pipe_f=1,conv_pipe_b=2", "conv_pipe_f=3,conv_pipe_b=3",
+         "conv_pipe_f=4,conv_pipe_b=4", "conv_pipe_f=4,conv_q=1",  # weights two edges ahead (forward)
          "conv_xcd=1,conv_gres=0", "conv_nt=0,conv_acc=48", "conv_sort=0,conv_tra=0", "conv_sort=0,conv_pipe_f=3,conv_nt=0",
          "conv_wf=0,conv_wb=0,conv_gf=1,conv_gb=1",
          # sender gradients: ordered reduction / float atomics / arrival counting; walk order off, 1 and 3 hops;
