@@ -344,6 +344,7 @@ def main():
 
     # per-kernel durations with HIP events on the launch stream, over K more steps
     ks = ops.get_entry(kid).kernels()
+    ks_source = ops.get_entry(kid).build_fn()[0]  # the generated HIP source of this kernel set
     ks.timing_enable(True)
     for _ in range(args.steps):
         step_det()
@@ -375,15 +376,19 @@ def main():
                         "frac": bwd_bytes / (bwd_op_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "index_kernels_ms_per_step": index_ms,
     }
-    # Both bounds of the step (time at 100 % of each peak). The arithmetic is ordinary v_fma_f32: every HIP
-    # file of this build is compiled without packed FP32 instructions, which halves the usable vector rate, so
-    # the step is bounded by its arithmetic before it is bounded by HBM.
+    # Bounds of the step (time at 100 % of a rate). The arithmetic is ordinary v_fma_f32 (every HIP file of this
+    # build is compiled without packed FP32 instructions); the rate the vector units reach with those, and the
+    # rate a stream of reads reaches once writes are mixed in, are measured on this box by ./hbm_stream.
+    ceilings = None if args.no_extras else hbm_ceilings()
     step_flops = (fwd_flops + bwd_flops) * E
     roofline["bounds_ms"] = {
         "hbm_at_8_TBps": (fwd_bytes + bwd_bytes) / HBM_PEAK_GBS / 1e6,
         "fp32_vector_at_published_peak": step_flops / (FP32_VECTOR_PEAK_TFLOPS * 1e9),
-        "fp32_vector_without_packed_instructions": step_flops / (FP32_VECTOR_PEAK_TFLOPS / 2 * 1e9),
     }
+    if ceilings:
+        roofline["bounds_ms"]["fp32_vector_unpacked_as_measured"] = step_flops / (ceilings["valu_fp32_tflops_unpacked"] * 1e9)
+        # this step writes 40 % of its algorithmic bytes: the measured rate of a read stream with writes mixed in
+        roofline["bounds_ms"]["hbm_at_measured_read_write_mix"] = (fwd_bytes + bwd_bytes) / ceilings["read_with_writes_1_2"] / 1e6
 
     modes = {
         "deterministic": {
@@ -558,9 +563,15 @@ def main():
         # this same command (scaled by a copy-kernel calibration); see profiles/conv_cfg5_deterministic.md
         with open(traffic_path) as f:
             tr = json.load(f)
-        if tr.get("edges") == E:
+        # the counters belong to the kernels they were measured on: the file names the hash of that kernel
+        # source, and a different source here means the figures are stale (traffic stays null until the
+        # profile is taken again)
+        if tr.get("edges") == E and tr.get("source_hash") == rt.source_hash(ks_source):
             roofline["traffic"] = tr["backward_bytes_per_launch"]
             roofline["traffic_per_kernel"] = tr.get("per_kernel")
+        else:
+            roofline["traffic_note"] = ("profiles/conv_cfg5_traffic.json was measured on another kernel source "
+                                        f"({tr.get('source_hash')} != {rt.source_hash(ks_source)})")
 
     out = {
         "metric": "fused conv fwd+bwd edges/s at MACE shape (deterministic mode)",
@@ -578,7 +589,12 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "modes": modes,
-        "hbm_stream_ceilings": None if args.no_extras else hbm_ceilings(),
+        "hbm_stream_ceilings": ceilings,
+        # what tells a slow box from a fast one: the device, its nominal clock, and the time of a fixed amount of
+        # vector arithmetic (./hbm_stream: 2 x 524 288 wave64 multiply-adds per SIMD)
+        "device": {"name": torch.cuda.get_device_name(0), "compute_units": rt.device_props(0).compute_units,
+                   "clock_khz_nominal": rt.device_props(0).clock_khz,
+                   "valu_fixed_work_ms": ceilings["valu_fixed_work_ms"] if ceilings else None},
     }
     out.update(extras)
     print(json.dumps(out))

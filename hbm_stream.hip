@@ -3,6 +3,13 @@
 // convolution's per-node edge data). bench.py runs this program (built by __graft_entry__.build()) and
 // puts its JSON line into the bench record; profiles/hbm_ceiling.md summarises it.
 //
+// The same program also reports `read_with_writes_*`: the chunk read again while the blocks write an eighth, half or all
+// of what they read (the convolution forward writes 12 % of its traffic, its backward 57 %): on this part any
+// share of writes brings a read stream down to about the copy rate, so a kernel's mix of reads and writes,
+// not only its byte count, decides which ceiling applies. And `valu_fixed_work_ms`: a fixed amount of
+// independent fp32 multiply-adds (plain v_fma_f32, two waves per SIMD) on every SIMD: the rate at which the vector
+// units issue them under sustained load, which also tells boxes with different sustained clocks apart.
+//
 // `./hbm_stream accumulate` instead runs three kernels that add 8.6 GB worth of values into a buffer small
 // enough to stay in the L2 caches: float atomics from all blocks on one 512 KB buffer, float atomics with each
 // XCD's blocks on their own 512 KB slice, and plain read-modify-write of 1024 private 16 KB slices. Under
@@ -61,6 +68,36 @@ __global__ __launch_bounds__(128) void chunks(const f4* __restrict__ a, f4* __re
         else acc += v;
     }
     if (!WRITE && acc.x + acc.y + acc.z + acc.w == 123.456f) *out = 1.f;
+}
+
+// one chunk per block, read; of every WRITE_EVERY 16-byte pieces read, one is written (0: none)
+template <int WRITE_EVERY>
+__global__ __launch_bounds__(128) void chunks_mixed(const f4* __restrict__ a, f4* __restrict__ b, const int* __restrict__ perm,
+                                                    int chunk_f4, float* out) {
+    const long c = perm[blockIdx.x];
+    const f4* src = a + c * chunk_f4;
+    f4* dst = b + c * chunk_f4;
+    f4 acc = {0, 0, 0, 0};
+    for (int i = threadIdx.x; i < chunk_f4; i += 128) {
+        const f4 v = __builtin_nontemporal_load(src + i);
+        acc += v;
+        // whole 2 KB rows of the block are written or skipped, so that written lines are written in full
+        if (WRITE_EVERY && (i / 128) % WRITE_EVERY == 0) __builtin_nontemporal_store(v, dst + i);
+    }
+    if (acc.x + acc.y + acc.z + acc.w == 123.456f) *out = 1.f;
+}
+
+// 8 independent chains of 65 536 multiply-adds per lane: 524 288 wave instructions per wave
+__global__ __launch_bounds__(256) void valu_fixed_work(float* out, float seed) {
+    float x[8];
+    for (int q = 0; q < 8; ++q) x[q] = seed + threadIdx.x * 1e-3f + q;
+    for (int it = 0; it < 65536; ++it) {
+        #pragma unroll
+        for (int q = 0; q < 8; ++q) x[q] = __builtin_fmaf(x[q], 0.999f, 0.001f);
+    }
+    float t = 0.f;
+    for (int q = 0; q < 8; ++q) t += x[q];
+    if (t == 123.456f) *out = t;
 }
 
 __global__ __launch_bounds__(256) void atomics_shared(float* p, int n_floats, int rounds) {
@@ -161,9 +198,26 @@ int main(int argc, char** argv) {
     const double sc_r = gb / median_ms([&] { chunks<0><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
     const double sc_c = 2 * gb / median_ms([&] { chunks<1><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
     const double memcpy_c = 2 * gb / median_ms([&] { (void)hipMemcpyAsync(b, a, bytes, hipMemcpyDeviceToDevice, 0); }) * 1e3;
+    // bytes read plus bytes written, per second, with writes for 1/8, 1/2 and all of the data read
+    const double mix8 = (1 + 1.0 / 8) * gb / median_ms([&] { chunks_mixed<8><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
+    const double mix2 = (1 + 1.0 / 2) * gb / median_ms([&] { chunks_mixed<2><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
+    const double mix1 = 2 * gb / median_ms([&] { chunks_mixed<1><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
+    const double mix0 = gb / median_ms([&] { chunks_mixed<0><<<n_chunks, 128>>>(a, b, dperm, chunk_f4, out); }) * 1e3;
+    // two waves on every SIMD: 2 x 524 288 instructions of 4 issue cycles each per SIMD
+    hipDeviceProp_t prop;
+    CHECK(hipGetDeviceProperties(&prop, 0));
+    const int cus = prop.multiProcessorCount;
+    const float valu_ms = median_ms([&] { valu_fixed_work<<<cus * 2, 256>>>(out, 1.0f); });
+    // wave64 multiply-adds that one SIMD issues per microsecond, and the same as a chip-wide fp32 rate
+    const double valu_per_simd_us = 2.0 * 524288.0 / (valu_ms * 1e3);
+    const double valu_tflops = (double)cus * 8 * 524288.0 * 64 * 2 / (valu_ms * 1e-3) / 1e12;
     std::printf("{\"unit\": \"GB/s\", \"buffer_gb\": %.2f, \"read_sweep\": %.0f, \"write_sweep\": %.0f, \"copy_sweep\": %.0f, "
                 "\"read_chunks_sequential\": %.0f, \"copy_chunks_sequential\": %.0f, \"read_chunks_scattered\": %.0f, "
-                "\"copy_chunks_scattered\": %.0f, \"hipMemcpy_d2d\": %.0f}\n",
-                gb, best_r, best_w, best_c, seq_r, seq_c, sc_r, sc_c, memcpy_c);
+                "\"copy_chunks_scattered\": %.0f, \"hipMemcpy_d2d\": %.0f, \"read_with_writes_0\": %.0f, "
+                "\"read_with_writes_1_8\": %.0f, \"read_with_writes_1_2\": %.0f, \"read_with_writes_1_1\": %.0f, "
+                "\"valu_fixed_work_ms\": %.4f, \"valu_wave64_fma_per_simd_per_us\": %.1f, \"valu_fp32_tflops_unpacked\": %.1f, "
+                "\"compute_units\": %d, \"clock_khz_nominal\": %d}\n",
+                gb, best_r, best_w, best_c, seq_r, seq_c, sc_r, sc_c, memcpy_c, mix0, mix8, mix2, mix1, valu_ms, valu_per_simd_us, valu_tflops, cus,
+                prop.clockRate);
     return 0;
 }

@@ -200,8 +200,9 @@ size_t oeq_conv_forward_workspace_bytes(const oeq_kernels* k, int64_t node_count
  * caller workspace, and the call itself allocates nothing (no hipMalloc / hipFree, no event or module
  * creation): the kernel set must already be loaded on the current device, i.e. oeq_conv_forward has run on
  * it once. Limits: the scratch needed, oeq_conv_forward_workspace_bytes(), must not exceed
- * oeq_static_scratch_bytes() (32 MiB: e.g. 1.9 M edges over 50 000 nodes with deterministic=False, 4 M
- * nodes in deterministic mode); larger calls are refused with OEQ_ERR_INVALID. Every call on a GPU uses
+ * oeq_static_scratch_bytes() (32 MiB: e.g. 1.85 M edges over 50 000 nodes with deterministic=False, 590 000
+ * nodes in deterministic mode, where the index and the temporaries of its build take 56 bytes per node);
+ * larger calls are refused with OEQ_ERR_INVALID. Every call on a GPU uses
  * that GPU's one array: calls that overlap in time on one GPU (two streams, two threads) race and must be
  * serialised by the caller. Long edge segments are walked whole here (oeq_problem_dims.hub_limit is not
  * applied: the rows of extra chunks would need scratch of their own), so the sum over a hub node's edges is

@@ -153,9 +153,18 @@ def lower(problem: TPProblem) -> Lowered:
     )
     low.ir_mul = problem.layout == "ir_mul"
     _lane_mapping(low)
-    if mode == "uvu" and 1 < low.n_chunks <= 4 and any(in1[p.i1].mul != 64 * low.n_chunks for p in paths):
+    if mode == "uvu" and low.n_chunks > MAX_CHUNKS:
+        # One wave per 64-channel chunk, all in one block of at most 1024 threads: blocks of more than 1024
+        # channels are cut into pieces of that many, each an ordinary block further into the row, and every
+        # path into one path per piece (the reference chunks any multiplicity into warp-sized children,
+        # core/ComputationSchedule.py:185-343).
+        low = _fold_wide_blocks(low, piece=64 * MAX_CHUNKS)
+    elif mode == "uvu" and 1 < low.n_chunks <= 4 and any(in1[p.i1].mul != 64 * low.n_chunks for p in paths):
         low = _fold_wide_blocks(low)
     return low
+
+
+MAX_CHUNKS = 16  # 64-channel chunks of a row that one block of 1024 threads covers
 
 
 def _lane_mapping(low: Lowered) -> None:
@@ -168,15 +177,16 @@ def _lane_mapping(low: Lowered) -> None:
     low.total_nnz = sum(len(p.nnz) for p in paths)
 
 
-def _fold_wide_blocks(low: Lowered) -> Lowered:
+def _fold_wide_blocks(low: Lowered, piece: int = 64) -> Lowered:
     """'uvu' rows wider than a wave whose irreps have different multiplicities (128x0e+64x1o+32x2e,
-    89x0e, ...): cut every block into pieces of at most 64 channels and every path into the paths
+    89x0e, ...): cut every block into pieces of at most ``piece`` = 64 channels and every path into the paths
     between matching pieces. In the [mul, 2l+1] layout a piece is just a block that starts further into
     the row (in the [2l+1, mul] layout: 64 channels further into each component, with the components
     still ``mul`` apart), and its weights start ``64 * mul_v`` further into the path's weights, so the
     result is an ordinary problem with at most 64 channels per block: one wave then owns the whole row and walks the
     pieces one after the other, where waves that each owned one 64-channel slice of every block would
-    mostly have idle lanes or nothing to do."""
+    mostly have idle lanes or nothing to do. With ``piece`` = 1024 the same cut brings blocks of more than
+    1024 channels down to what one block of threads covers; the pieces then still span several waves."""
     def cut(blocks: List[Block], used):
         pieces, index = [], {}
         for b, blk in enumerate(blocks):
@@ -186,13 +196,13 @@ def _fold_wide_blocks(low: Lowered) -> Lowered:
                 index[(b, 0)] = len(pieces)
                 pieces.append(blk)
                 continue
-            for c in range((blk.mul + 63) // 64):
+            for c in range((blk.mul + piece - 1) // piece):
                 index[(b, c)] = len(pieces)
-                n = min(64, blk.mul - c * 64)
+                n = min(piece, blk.mul - c * piece)
                 if low.ir_mul:  # component i of channel u sits at off + i * mul + u
-                    pieces.append(Block(blk.off + c * 64, n, blk.l, cstride=blk.mul))
+                    pieces.append(Block(blk.off + c * piece, n, blk.l, cstride=blk.cstride or blk.mul))
                 else:
-                    pieces.append(Block(blk.off + c * 64 * blk.d, n, blk.l))
+                    pieces.append(Block(blk.off + c * piece * blk.d, n, blk.l))
         return pieces, index
 
     in1, index1 = cut(low.in1, {p.i1 for p in low.paths})
@@ -200,8 +210,8 @@ def _fold_wide_blocks(low: Lowered) -> Lowered:
     paths = []
     for p in low.paths:
         v_mul = low.in2[p.i2].mul
-        for c in range((low.in1[p.i1].mul + 63) // 64):
-            paths.append(Path(len(paths), index1[(p.i1, c)], p.i2, index3[(p.io, c)], p.woff + c * 64 * v_mul,
+        for c in range((low.in1[p.i1].mul + piece - 1) // piece):
+            paths.append(Path(len(paths), index1[(p.i1, c)], p.i2, index3[(p.io, c)], p.woff + c * piece * v_mul,
                               p.coeff, p.nnz, p.l))
     folded = Lowered(mode=low.mode, ctype=low.ctype, elem_size=low.elem_size, shared_weights=low.shared_weights,
                      in1=in1, in2=low.in2, out=out, paths=paths, L1=low.L1, L2=low.L2, L3=low.L3, WN=low.WN,

@@ -58,12 +58,7 @@ class UvuEmitter:
     def __init__(self, low: Lowered, *, acc_budget_words: int = 128, g_resident_words: int = 128,
                  kahan: bool = False):
         assert low.mode == "uvu"
-        if low.n_chunks > 16:
-            # one wave per 64-channel chunk of a row, all in one block: 1024 threads is the block limit
-            widest = max(b.mul for b in list(low.in1) + list(low.out))
-            raise ValueError(f"'uvu' kernels handle at most 1024 channels per irrep block (16 chunks of 64); this "
-                             f"problem has a block of multiplicity {widest}. Split the block into several irreps "
-                             "of at most 1024 channels each (with one instruction per piece).")
+        assert low.n_chunks <= 16, "blocks of more than 1024 channels are cut into pieces by codegen.lower"
         self.low = low
         self.ir_mul = low.ir_mul
         self.kahan = kahan  # conv forward: compensated (Kahan) summation over a receiver's edges
@@ -2251,7 +2246,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         em.q_ahead = (t["conv_qaf"], t["conv_qab"])
         em.build_q_table()
     if walk and len(em.segments) > 1 and t["conv_segw"] and em.stage is None and em.R == 1:
-        em.seg_waves = max(1, min(len(em.segments), t["conv_segw"], 8 // em.NCH))
+        em.seg_waves = max(1, min(len(em.segments), t["conv_segw"], max(1, 8 // em.NCH)))
         t["conv_gf"] = max(1, min(t["conv_gf"], 8 // (em.NCH * em.seg_waves)))
     em.tr_stores = t["conv_trs"]
     # output gradients that do not fit the register budget are loaded per path: fence the paths then
@@ -2275,7 +2270,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     gres = None if t["conv_gres"] < 0 else bool(t["conv_gres"])
     dx_mode = 0
     em.group_budget = t["conv_gbud"]
-    em.bwd_groups = em.plan_backward_groups(8 // em.NCH) if (walk and t["conv_split"] and gres is None) else None
+    em.bwd_groups = em.plan_backward_groups(max(1, 8 // em.NCH)) if (walk and t["conv_split"] and gres is None) else None
     if em.bwd_groups:
         G_b = 1
         wpb = em.NCH * len(em.bwd_groups)

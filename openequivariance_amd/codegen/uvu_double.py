@@ -876,13 +876,13 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     # pair): its accumulators on top of kernel B's state spill whatever the split, so it is off by default.
     shared = low.shared_weights
     em.merged = bool(tune.get("dd_merge", 0)) and not shared
-    groups = em.plan_double_groups(8 // em.NCH) if tune.get("dd_split", 1) and not shared else None
+    groups = em.plan_double_groups(max(1, 8 // em.NCH)) if tune.get("dd_split", 1) and not shared else None
     if em.merged and not groups and not em.merged_fits_one_wave():
         em.merged = False
-        groups = em.plan_double_groups(8 // em.NCH) if tune.get("dd_split", 1) else None
+        groups = em.plan_double_groups(max(1, 8 // em.NCH)) if tune.get("dd_split", 1) else None
     descs = []
     if not em.merged:
-        segw = min(len(em.segments), max(1, tune.get("dd_segw", 4)), 8 // em.NCH) if em.R == 1 else 1
+        segw = min(len(em.segments), max(1, tune.get("dd_segw", 4)), max(1, 8 // em.NCH)) if em.R == 1 else 1
         G_a = max(1, min(G, 8 // (em.NCH * segw)))
         blk_a = em.emit_conv_double_a(s, G_a, tune.get("dd_wa", 2), xcd, segw)
         descs.append((rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_A", blk_a, G_a, 0, xcd))

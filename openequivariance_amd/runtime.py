@@ -109,16 +109,21 @@ def build_library(verbose: bool = False) -> Path:
     """Compile csrc/oeq_amd.cpp into liboeq_amd.so next to this file."""
     # the library carries one device-side object (the scratch array of oeq_conv_forward_static), so it is
     # compiled for the target architecture, with the device flags every kernel here is compiled with
+    # built under a temporary name and moved into place, so that a process loading the library while
+    # another one rebuilds it never maps a half-written file
+    tmp = _LIB_PATH.with_name(f"{_LIB_PATH.name}.tmp{os.getpid()}")
     cmd = [
         "hipcc", "-O2", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={DEFAULT_ARCH}",
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", f"-I{_INCLUDE_DIR}",
-        str(_SRC_PATH), "-o", str(_LIB_PATH), "-lhiprtc",
+        str(_SRC_PATH), "-o", str(tmp), "-lhiprtc",
     ]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
+        tmp.unlink(missing_ok=True)
         raise OeqError(f"building liboeq_amd.so failed:\n{res.stdout}\n{res.stderr}")
+    os.replace(tmp, _LIB_PATH)
     if verbose:
-        print(" ".join(cmd))
+        print(" ".join(cmd).replace(str(tmp), str(_LIB_PATH)))
     return _LIB_PATH
 
 

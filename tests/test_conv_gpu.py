@@ -93,6 +93,10 @@ CASES = [
     ("uvw-cfg4-mfma", P.config4_uvw_shared, 30, 5),
     # output gradient too large for one wave: forward shares the output segments, backward the output
     # blocks, between several waves of a node (64 channels: one chunk; 128: two)
+    # an irrep block of 2048 channels: two pieces of 1024, sixteen chunk waves per node
+    ("uvu-2048", lambda: oeq.TPProblem("2048x1o", "1x1o", "2048x0e+2048x2e",
+                                       [(0, 0, 0, "uvu", True), (0, 0, 1, "uvu", True)], shared_weights=False,
+                                       internal_weights=False, label="uvu-2048"), 24, 4),
     ("nequip-benzene", lambda: P.nequip_problems()[3], 30, 5),
     ("benzene-128", lambda: P.ChannelwiseTPP(
         "128x0o + 128x0e + 128x1o + 128x1e + 128x2o + 128x2e + 128x3o + 128x3e", "0e + 1o + 2e + 3o",

@@ -51,6 +51,10 @@ PROBLEMS = [
         "64x4e+128x3e", "1x1e+1x0e", "64x4e+128x2e+128x3e+128x4e+128x3e",
         [(0, 1, 0, "uvu", True), (1, 0, 1, "uvu", True), (1, 0, 2, "uvu", True), (1, 0, 3, "uvu", True),
          (1, 1, 4, "uvu", True)], shared_weights=False, internal_weights=False, label="folded-64s")),
+    # a block of more than 1024 channels: pieces of 1024 whose components stay the block's multiplicity apart
+    ("uvu-1100", lambda: oeq.TPProblem("1100x1o", "1x1o", "1100x2e+1100x0e",
+                                       [(0, 0, 0, "uvu", True), (0, 0, 1, "uvu", True)], shared_weights=False,
+                                       internal_weights=False, label="uvu-1100")),
 ]
 
 

@@ -92,19 +92,31 @@ def test_generated_sources_compile_for_gfx950(make, conv):
         assert {d[0] for d in descs} >= {rt.ROLE_DOUBLE_BACKWARD_A, rt.ROLE_DOUBLE_BACKWARD_B}
 
 
-@pytest.mark.parametrize("mul", [1088, 2048])
-def test_blocks_wider_than_1024_channels_fail_with_a_message(mul):
-    """One wave per 64-channel chunk and one block per row: 1024 channels is the limit, and exceeding it is
-    reported when the kernels are generated, not as a bad launch descriptor later."""
+@pytest.mark.parametrize("mul", [1088, 2048, 2500])
+@pytest.mark.parametrize("layout", ["mul_ir", "ir_mul"])
+def test_blocks_wider_than_1024_channels_are_cut_into_pieces(mul, layout):
+    """One wave per 64-channel chunk and one block of threads per row: 1024 channels is what a block covers,
+    so wider irrep blocks are lowered as several pieces of at most 1024 channels, each with its own path
+    (the reference chunks any multiplicity, core/ComputationSchedule.py:185-343). The pieces tile the
+    block, the paths tile the weights, and the kernels generate and compile."""
     import openequivariance_amd as oeq
+    from openequivariance_amd import runtime as rt
     from openequivariance_amd._torch.tensor_product import build_tp_module
     from openequivariance_amd._torch.tensor_product_conv import build_conv_module
-    problem = oeq.TPProblem(f"{mul}x1o", "1x1o", f"{mul}x0e", [(0, 0, 0, "uvu", True)], shared_weights=False,
-                            internal_weights=False)
-    with pytest.raises(ValueError, match="at most 1024 channels"):
-        build_tp_module(problem)
-    with pytest.raises(ValueError, match="at most 1024 channels"):
-        build_conv_module(problem, True)
+    from openequivariance_amd.codegen.lower import lower
+    problem = oeq.TPProblem(f"{mul}x1o", "1x1o", f"{mul}x0e+{mul}x2e", [(0, 0, 0, "uvu", True), (0, 0, 1, "uvu", True)],
+                            shared_weights=False, internal_weights=False, layout=layout)
+    low = lower(problem)
+    n_pieces = (mul + 1023) // 1024
+    assert low.n_chunks <= 16 and len(low.paths) == 2 * n_pieces
+    assert [b.mul for b in low.in1] == [min(1024, mul - 1024 * c) for c in range(n_pieces)]
+    assert sorted(p.woff for p in low.paths) == sorted(i * mul + 1024 * c for i in range(2) for c in range(n_pieces))
+    if layout == "mul_ir":
+        assert [b.off for b in low.in1] == [1024 * 3 * c for c in range(n_pieces)]
+    else:
+        assert [(b.off, b.cstride) for b in low.in1] == [(1024 * c, mul) for c in range(n_pieces)]
+    for src, _dims, _descs in (build_tp_module(problem), build_conv_module(problem, True)):
+        assert rt.compile_source(src, use_disk_cache=False)[:4] == b"\x7fELF"
 
 
 def test_matrix_core_path_accepts_only_what_its_kernels_can_hold():

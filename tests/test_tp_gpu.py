@@ -182,6 +182,21 @@ MFMA_CASES = {"cfg4-shared", "cfg4-f64", "mfma-32", "mfma-128", "mfma-mixed", "m
               "mfma-sh6-f64", "mfma-sh7"}
 # shared weights off the matrix cores (second operand of more than 64 values): the general kernels' weight gradient
 # in an LDS copy per wave and in partial rows in global memory
+# irrep blocks of more than 1024 channels, cut into pieces of 1024 by the planner (one block of 1024
+# threads covers 16 chunks of 64): two pieces, a ragged last piece, a second operand with two channels (the
+# component-major layout of such blocks: tests/test_ir_mul_gpu.py)
+CASES += [
+    ("uvu-2048", lambda: oeq.TPProblem("2048x1o", "1x1o", "2048x0e+2048x1e+2048x2e",
+                                       [(0, 0, 0, "uvu", True), (0, 0, 1, "uvu", True), (0, 0, 2, "uvu", True)],
+                                       shared_weights=False, internal_weights=False, label="uvu-2048"), 21),
+    ("uvu-1500-mixed", lambda: oeq.TPProblem("1500x1o+70x0e", "2x1o+1x0e", "1500x2e+70x0e+1500x1o",
+                                             [(0, 0, 0, "uvu", True), (1, 1, 1, "uvu", True), (0, 1, 2, "uvu", True)],
+                                             shared_weights=False, internal_weights=False, label="uvu-1500"), 19),
+    ("uvu-2048-shared-f64", lambda: _as_f64(oeq.TPProblem(
+        "2048x1o", "1x1o", "2048x0e", [(0, 0, 0, "uvu", True)], shared_weights=True, internal_weights=False,
+        label="uvu-2048-shared")), 33),
+]
+
 CASES += [
     ("uvw-shared-lds", lambda: _fc_shared("20x0e+10x1o", "40x0e+10x1o", "12x0e+6x1o"), 77),
     ("uvw-shared-lds-wide", lambda: _fc_shared("70x0e+3x1o", "1x0e+1x1o+1x2e+1x3o+1x4e+1x5o+1x6e+1x7o+1x8e", "3x0e+2x1o"), 77),
