@@ -263,6 +263,33 @@ def uvw_conv_table(dev, nodes=12000):
             table.append(row)
             del X, Y, W, G
             torch.cuda.empty_cache()
+        # Shared weights (one weight tensor for all edges), shuffled edge list: the factored form (contraction
+        # summed per receiver by the fused 'uvu' convolution, then one channel mix per NODE on the matrix
+        # cores) beside the two routes that mix per edge: the matrix-core batch kernels on gathered rows with
+        # ordered segment sums ("per_edge_mfma"), and the fused general kernels ("per_edge_general").
+        shared_dd = P.diffdock_problems()[0].clone()
+        shared_dd.shared_weights = True
+        shared_dd.label = "DiffDock-L=1 shared weights"
+        perm = torch.randperm(E, device=dev)
+        rs, cs = tr[perm].contiguous(), tc[perm].contiguous()
+        none = torch.zeros(0, dtype=torch.int64, device=dev)
+        for prob in (shared_dd, P.config4_uvw_shared()):
+            low = lower(prob)
+            X, Y = torch.randn(nodes, low.L1, device=dev), torch.randn(E, low.L2, device=dev)
+            W, G = torch.randn(low.WN, device=dev), torch.randn(nodes, low.L3, device=dev)
+            A_, B_, C_ = torch.randn_like(X), torch.randn_like(Y), torch.randn_like(W)
+            row = {"config": prob.label, "nodes": nodes, "edges": E, "mode": "deterministic=False, shuffled edges"}
+            for key, knobs in (("factored", "conv_factor=1"), ("per_edge_mfma", "conv_factor=0,conv_mfma_min_weights=0"),
+                               ("per_edge_general", "conv_factor=0,conv_mfma_min_weights=100000000")):
+                os.environ["OEQ_AMD_TUNE"] = ((saved + ",") if saved else "") + knobs
+                kid = oeq.TensorProductConv(prob, deterministic=False).kid
+                row[key] = {"fwd_ms": med(lambda: ops.conv_forward(X, Y, W, rs, cs, none, kid)),
+                            "bwd_ms": med(lambda: ops.conv_backward(X, Y, W, G, rs, cs, none, kid)),
+                            "second_order_ms": med(lambda: ops.conv_double_backward(X, Y, W, G, A_, B_, C_, rs, cs, none,
+                                                                                    kid), warm=1, it=3)}
+            table.append(row)
+            del X, Y, W, G, A_, B_, C_
+            torch.cuda.empty_cache()
     finally:
         if saved is None:
             os.environ.pop("OEQ_AMD_TUNE", None)

@@ -51,6 +51,9 @@ class KernelEntry:
         self.dtype = torch_dtype
         self.deterministic = deterministic
         self.spec: Optional[torch.Tensor] = None  # the bytes this entry was built from (uint8, host)
+        # Shared-weight 'uvw' convolution as contraction + channel mix per node (core/problems.py:
+        # factor_shared_uvw): ids of the two kernel sets that then do the work, else None.
+        self.factored: Optional[Tuple[int, int]] = None
         self._ks: Optional[rt.KernelSet] = None
         self._lock = threading.Lock()
 
@@ -122,10 +125,19 @@ def _entry_from_spec(spec: bytes) -> KernelEntry:
         def build():
             with _tune_env(tune):
                 return build_conv_module(problem, det, kahan)
+        factored = None
         with _tune_env(tune):
-            unfused = not fused(low)
+            from ..codegen.uvu import tuning
+            from ..core.problems import factor_shared_uvw
+            knobs = tuning(dict(conv_fuse_uvw=1, conv_factor=1))
+            parts = factor_shared_uvw(problem) if (knobs["conv_fuse_uvw"] and knobs["conv_factor"]) else None
+            if parts is not None and not det:
+                factored = (register_spec(make_spec("conv", parts[0], False, False)),
+                            register_spec(make_spec("tp", parts[1])))
+            unfused = factored is None and not fused(low)
         entry = KernelEntry(build, low.L1, low.L2, low.L3, low.WN, low.shared_weights, dtype, deterministic=det,
                             unfused=unfused)
+        entry.factored = factored
     entry.spec = torch.frombuffer(bytearray(spec), dtype=torch.uint8)
     return entry
 
@@ -296,7 +308,8 @@ def _use_fused(kid, spec, ddx, ddy, ddw) -> bool:
         return False
     if sum(t is not None for t in (ddx, ddy, ddw)) < 2:
         return False
-    return get_entry(kid, spec).kernels().has_double_backward()
+    entry = get_entry(kid, spec)
+    return bool(entry.factored) or entry.kernels().has_double_backward()
 
 
 def _zeros_if_none(t, like):
@@ -393,6 +406,11 @@ def _check_indices_enabled() -> bool:
     return CHECK_INDICES or os.environ.get("OEQ_AMD_CHECK_INDICES", "0") not in ("", "0")
 
 
+def _walk_dims(e: KernelEntry) -> dict:
+    """Dims of the kernel set that walks the graph for this entry (the contraction part of a factored one)."""
+    return (get_entry(e.factored[0]) if e.factored else e).kernels().dims
+
+
 def _conv_checks(e: KernelEntry, L1_in, L2_in, W, rows, cols, perm, L3_grad=None):
     nodes = L1_in.shape[0] if L1_in.dim() > 0 else -1
     nnz = rows.shape[0] if rows.dim() > 0 else -1
@@ -410,8 +428,8 @@ def _conv_checks(e: KernelEntry, L1_in, L2_in, W, rows, cols, perm, L3_grad=None
     if e.deterministic:
         pass
     elif (torch.are_deterministic_algorithms_enabled() and not e.unfused
-          and (e.kernels().dims["deterministic"] == rt.CONV_ATOMIC
-               or (L3_grad is not None and e.kernels().dims.get("dx_mode", 0) == rt.DX_ATOMIC))):
+          and (_walk_dims(e)["deterministic"] == rt.CONV_ATOMIC
+               or (L3_grad is not None and _walk_dims(e).get("dx_mode", 0) == rt.DX_ATOMIC))):
         # counterpart of at::globalContext().alertNotDeterministic (torch_core.hpp:448) for the calls that
         # use float atomics: the backward of deterministic=False (sender gradients), and both directions
         # of the float-atomics kernels. The grouped forward sums in a fixed order and needs no alert.
@@ -547,6 +565,39 @@ def _unfused_double_backward(e, ks, x, y, w, g, a, b, c, r, cc, p, nodes, nnz):
             _scatter_rows(e, ks, gge, nodes, r, None))
 
 
+_ones_cache: Dict[tuple, torch.Tensor] = {}
+
+
+def _ones(n: int, like: torch.Tensor, cols: Optional[int] = None) -> torch.Tensor:
+    """A tensor of ones ([n] or [n, cols]) in the dtype and on the device of ``like``; the few shapes a model
+    uses are kept (they are read-only operands of the factored convolution)."""
+    key = (n, cols, like.dtype, like.device)
+    t = _ones_cache.get(key)
+    if t is None:
+        if len(_ones_cache) > 64:
+            _ones_cache.clear()
+        t = torch.ones((n,) if cols is None else (n, cols), dtype=like.dtype, device=like.device)
+        _ones_cache[key] = t
+    return t
+
+
+def _factored_forward(e: KernelEntry, x, y, w, r, c, p):
+    """Shared weights, single-channel second operands: contraction summed per receiver by the fused 'uvu'
+    convolution of the first part, then ONE channel mix per node (core/problems.py: factor_shared_uvw)."""
+    kid_a, kid_b = e.factored
+    mid = conv_forward(x, y, _ones(get_entry(kid_a).WN, x), r, c, p, kid_a)
+    return tp_forward(mid, _ones(x.shape[0], x, 1), w, kid_b)
+
+
+def _factored_backward(e: KernelEntry, x, y, w, g, r, c, p):
+    kid_a, kid_b = e.factored
+    ones_a, ones_b = _ones(get_entry(kid_a).WN, x), _ones(x.shape[0], x, 1)
+    mid = conv_forward(x, y, ones_a, r, c, p, kid_a)            # recomputed: one node-sized tensor
+    dmid, _, dw = tp_backward(mid, ones_b, w, g, kid_b)         # mix: gradients of the node sums and of W
+    dx, dy, _ = conv_backward(x, y, ones_a, dmid, r, c, p, kid_a)
+    return dx, dy, dw
+
+
 @torch.library.custom_op("oeq_amd::conv_forward", mutates_args=(), device_types="cuda")
 def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows: torch.Tensor,
                  cols: torch.Tensor, transpose_perm: torch.Tensor, kid: int,
@@ -555,6 +606,8 @@ def conv_forward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, rows
     nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm)
     x, y, w = L1_in.contiguous(), L2_in.contiguous(), W.contiguous()
     r, c = rows.contiguous(), cols.contiguous()
+    if e.factored:
+        return _factored_forward(e, x, y, w, r, c, transpose_perm)
     if e.unfused:
         with torch.cuda.device(x.device):
             return _unfused_forward(e, e.kernels(), x, y, w, r, c, nodes, nnz)
@@ -592,6 +645,8 @@ def conv_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tensor, L3_
     nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm, L3_grad)
     x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
     r, c, p = rows.contiguous(), cols.contiguous(), transpose_perm.contiguous()
+    if e.factored:
+        return _factored_backward(e, x, y, w, g, r, c, p)
     if e.unfused:
         with torch.cuda.device(x.device):
             return _unfused_backward(e, e.kernels(), x, y, w, g, r, c, p, nodes, nnz)
@@ -651,6 +706,13 @@ def conv_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tens
     x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()
     a, b, c = L1_dgrad.contiguous(), L2_dgrad.contiguous(), W_dgrad.contiguous()
     r, cc, p = rows.contiguous(), cols.contiguous(), transpose_perm.contiguous()
+    if e.factored:
+        # the map is linear in each of X, Y, W: its second-order pass is a sum of first-order calls, each of
+        # them the cheap factored form (one channel mix per node)
+        with torch.no_grad():
+            return _second_order(lambda p1, q1, r1: _factored_forward(e, p1, q1, r1, r, cc, p),
+                                 lambda p1, q1, r1, s1: _factored_backward(e, p1, q1, r1, s1, r, cc, p),
+                                 x, y, w, g, a, b, c)
     if e.unfused:
         with torch.cuda.device(x.device):
             return _unfused_double_backward(e, e.kernels(), x, y, w, g, a, b, c, r, cc, p, nodes, nnz)

@@ -221,3 +221,33 @@ def config5_mace_conv(dtype=np.float32) -> TPProblem:
     p = config3_mace_uvu(dtype)
     p.label = "cfg5-mace-conv"
     return p
+
+
+def factor_shared_uvw(problem: TPProblem):
+    """A fully connected ('uvw') problem with ONE weight tensor for all rows and single-channel second
+    operands, written as two problems: ``A`` = the CG contraction without the channel mix, one output block
+    ``U x l3`` per path ('uvu', weights all one), and ``B`` = the channel mix of those blocks ('uvw' against a
+    scalar one, same weight tensor as the original, same order). ``TP(x, y, W) = B(A(x, y, 1), 1, W)`` for one
+    row; over a graph the sum over a receiver's edges commutes with the mix, because the weights do not
+    depend on the edge: ``sum_e B(A(x_e, y_e), W) = B(sum_e A(x_e, y_e), W)``. So the convolution is the
+    fused 'uvu' convolution of ``A`` followed by ``B`` on one row per NODE: the channel mix runs once per node
+    instead of once per edge and nothing of size [edges, L3] exists. (The reference mixes per edge inside its
+    edge loop, templates/loop_unroll_conv_atomic.cuh:52-180 with loop_unroll_tp.cuh:55-84.) None when the
+    problem does not have this shape."""
+    ins = problem.instructions
+    if not problem.shared_weights or not ins or any(i.connection_mode != "uvw" or not i.has_weight for i in ins):
+        return None
+    in1, in2, out = problem.irreps_in1, problem.irreps_in2, problem.irreps_out
+    if any(in2[i.i_in2].mul != 1 for i in ins):
+        return None
+    mid = Irreps([(in1[i.i_in1].mul, out[i.i_out].ir) for i in ins])
+    common = dict(irrep_normalization="none", path_normalization="none", shared_weights=True, internal_weights=False,
+                  irrep_dtype=problem.irrep_dtype, weight_dtype=problem.weight_dtype)
+    # stored coefficient = sqrt(path weight given here). The scalar second operand of B brings the factor
+    # wigner_3j(l, 0, l) = identity / sqrt(2l+1), which A's coefficient makes up for.
+    a = TPProblem(in1, in2, mid, [(i.i_in1, i.i_in2, n, "uvu", True, i.path_weight ** 2 * out[i.i_out].ir.dim)
+                                  for n, i in enumerate(ins)], label=f"{problem.label}-contraction", **common)
+    b = TPProblem(mid, "1x0e", out, [(n, 0, i.i_out, "uvw", True, 1.0) for n, i in enumerate(ins)],
+                  label=f"{problem.label}-mix", **common)
+    assert b.weight_numel == problem.weight_numel
+    return a, b

@@ -212,6 +212,49 @@ def test_uvw_shared_weights_fused_matches_unfused(monkeypatch):
             assert (a - b).abs().max() <= 4e-6 * b.abs().max(), n_nodes
 
 
+SHARED_SINGLE_CHANNEL = ["uvw-cfg4-mfma", "uvw-shared-mfma-padded", "uvw-shared-tetris"]
+
+
+@pytest.mark.parametrize("name", SHARED_SINGLE_CHANNEL)
+def test_shared_weight_uvw_runs_factored(name, monkeypatch):
+    """One weight tensor for all edges and single-channel second operands: the sum over a receiver's edges
+    commutes with the channel mix, so the convolution runs as the fused 'uvu' convolution of the contraction
+    followed by one mix per node (core/problems.py: factor_shared_uvw): no gathered [E, L1] rows, no [E, L3]
+    messages. Same results as the routes that mix per edge (matrix-core batch kernels on gathered rows, fused
+    general kernels), first and second order; problems with several channels in the second operand keep
+    those routes."""
+    from openequivariance_amd._torch import ops
+    make = next(c[1] for c in CASES if c[0] == name)
+    problem = make()
+    coords, rows, cols = _graph(300, 8, seed=12)
+    E = len(rows)
+    order = np.random.default_rng(2).permutation(E)
+    tr, tc = (torch.tensor(a[order], device="cuda") for a in (rows, cols))
+    none = torch.zeros(0, dtype=torch.int64, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    X, A = (torch.randn(300, problem.irreps_in1.dim, device="cuda", generator=gen) for _ in range(2))
+    Y, B = (torch.randn(E, problem.irreps_in2.dim, device="cuda", generator=gen) for _ in range(2))
+    W, C = (torch.randn(problem.weight_numel, device="cuda", generator=gen) for _ in range(2))
+    G = torch.randn(300, problem.irreps_out.dim, device="cuda", generator=gen)
+    out = {}
+    for knobs in ("conv_factor=1", "conv_factor=0,conv_mfma_min_weights=0", "conv_factor=0,conv_mfma_min_weights=100000000"):
+        monkeypatch.setenv("OEQ_AMD_TUNE", knobs)
+        conv = oeq.TensorProductConv(problem, deterministic=False)
+        e = ops.get_entry(conv.kid)
+        assert bool(e.factored) == (knobs == "conv_factor=1") and not (e.factored and e.unfused)
+        out[knobs] = (ops.conv_forward(X, Y, W, tr, tc, none, conv.kid),) + \
+            tuple(ops.conv_backward(X, Y, W, G, tr, tc, none, conv.kid)) + \
+            tuple(ops.conv_double_backward(X, Y, W, G, A, B, C, tr, tc, none, conv.kid))
+    ref = out["conv_factor=1"]
+    for knobs, got in out.items():
+        for a, b in zip(got, ref):
+            assert float((a - b).abs().max() / b.abs().max()) <= 2e-5, knobs
+    # several channels in the second operand: not of this shape
+    monkeypatch.setenv("OEQ_AMD_TUNE", "")
+    multi = next(c[1] for c in CASES if c[0] == "uvw-shared-mfma-mul2")()
+    assert ops.get_entry(oeq.TensorProductConv(multi, deterministic=False).kid).factored is None
+
+
 def test_reference_toy_graph():
     """The 3-node / 4-edge graph of the reference's tutorial
     (tests/example_test.py:46-82): atomic and deterministic calls agree with the
