@@ -98,8 +98,13 @@ CONV = [c for c in PROBLEMS if c[0] in ("mace-large", "cfg3-f64", "cfg2", "13x5e
                                         "nequix-first", "sevennet-main", "folded-gaps", "folded-64s")]
 
 
+@pytest.mark.parametrize("hub", [256, 2], ids=["whole-segments", "chunks-of-2"])
 @pytest.mark.parametrize("name,make", CONV, ids=[c[0] for c in CONV])
-def test_conv_ir_mul(name, make):
+def test_conv_ir_mul(name, make, hub, monkeypatch):
+    # (second run: every edge segment cut into chunks of two edges, so that extra walk positions, the rows they
+    # write and the chunked sender-side sums are exercised in this layout as well)
+    if hub != 256:
+        monkeypatch.setenv("OEQ_AMD_TUNE", f"conv_hub={hub}")
     problem = make()
     tol = tol_of(problem)
     n_nodes = 40
