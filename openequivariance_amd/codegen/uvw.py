@@ -28,6 +28,10 @@ from .common import Src, prelude, utility_kernels
 from .lower import Lowered, Path, float_literal
 
 WAVES_PER_BLOCK = 4
+# the chunk table of long edge segments and the rows of the extra chunks, as the last kernel arguments of the
+# receiver walks
+HUB_PARAMS = (", const i64* __restrict__ hubptr, const i64* __restrict__ hubnode, i64 hub_limit, i64 hub_units, "
+              "T* __restrict__ hub_rows")
 
 
 def _pow2ceil(n: int) -> int:
@@ -39,7 +43,7 @@ class UvwEmitter:
         assert low.mode == "uvw"
         from .uvu import tuning
         self.tune = tuning(dict(uvw_unroll=16, uvw_tile=24576, uvw_regdw=1, conv_hops=2, conv_fuse_uvw=1, uvw_dd=1,
-                                uvw_dda_split=0, uvw_dda_unroll=4))
+                                uvw_dda_split=0, uvw_dda_unroll=4, conv_hub=256))
         self.TILE_BYTES = self.tune["uvw_tile"]
         self.low = low
         self.T = low.ctype
@@ -264,27 +268,46 @@ class UvwEmitter:
                 "const T* __restrict__ L1_in, const T* __restrict__ L1_dgrad, const T* __restrict__ L2_in, "
                 "const T* __restrict__ L2_dgrad, const T* __restrict__ W, const T* __restrict__ W_dgrad, "
                 "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-                "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order)"
+                "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order"
+                f"{HUB_PARAMS})"
             )
         else:
             s.open(
                 f'extern "C" __global__ __launch_bounds__({block}) void forward(i64 node_count, i64 nnz, '
                 "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
                 "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
-                "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order)"
+                "const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order"
+                f"{HUB_PARAMS})"
             )
         s(f"__shared__ T s_t[{wpn * G}][{self.max_d3 * (2 if second else 1)}][64];")
         s("const int lane = oeq_lane();")
         s("const int wave = oeq_wave();")
         s(f"const int g = wave / {wpn}, sg = wave % {wpn};")
-        s.open(f"for (i64 base = (i64)blockIdx.x * {G}; base < node_count; base += (i64)gridDim.x * {G})")
-        s("const i64 vnode = base + g;")
-        s("const bool live = vnode < node_count;")
-        s("const i64 vc = live ? vnode : node_count - 1;")
-        s("const i64 node = order ? oeq_idx(order[vc], node_count) : vc;")
-        s("const i64 e0 = oeq_pos(rowptr[node], nnz);")
-        s("const i64 e1 = live ? oeq_pos(rowptr[node + 1], nnz) : e0;")
-        s(f"T* zrow = L3_out + node * {low.L3};")
+        # Walk positions: the first hub_units of them are the extra chunks of nodes with more than hub_limit
+        # edges (their partial rows go to hub_rows and are added in chunk order afterwards), then one position
+        # per node, which takes the node's first chunk.
+        s("const i64 walk_end = hub_units + node_count;")
+        s.open(f"for (i64 base = (i64)blockIdx.x * {G}; base < walk_end; base += (i64)gridDim.x * {G})")
+        s("const i64 wpos = base + g;")
+        s("const bool extra = wpos < hub_units;")
+        s("const bool live = extra ? wpos < hubptr[node_count] : wpos < walk_end;")
+        s("i64 node = 0, e0 = 0, e1 = 0;")
+        s(f"T* zrow = L3_out;")
+        s.open("if (live && extra)")
+        s("node = oeq_idx(hubnode[wpos], node_count);")
+        s("e0 = oeq_pos(rowptr[node] + (wpos - hubptr[node] + 1) * hub_limit, nnz);")
+        s("e1 = oeq_pos(rowptr[node + 1], nnz);")
+        s("if (e1 - e0 > hub_limit) e1 = e0 + hub_limit;")
+        s(f"zrow = hub_rows + wpos * {low.L3};")
+        s.close()
+        s.open("else if (live)")
+        s("const i64 vnode = wpos - hub_units;")
+        s("node = order ? oeq_idx(order[vnode], node_count) : vnode;")
+        s("e0 = oeq_pos(rowptr[node], nnz);")
+        s("e1 = oeq_pos(rowptr[node + 1], nnz);")
+        s("if (hub_limit > 0 && e1 - e0 > hub_limit) e1 = e0 + hub_limit;")
+        s(f"zrow = L3_out + node * {low.L3};")
+        s.close()
         for io in empty:
             # an output block no path writes: zeros
             bo = low.out[io]
@@ -1022,12 +1045,17 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         (rt.ROLE_GROUP_SCATTER, "oeq_group_scatter", 256, 256 * 4, cu * 16),
         (rt.ROLE_GROUP_ORDER, "oeq_group_order", 256, 4, cu * 32),
         (rt.ROLE_ORDER_HOP, "oeq_order_hop", 256, 256, cu * 16),
+        (rt.ROLE_HUB_COUNT, "oeq_hub_count", 256, 256, cu * 16),
+        (rt.ROLE_HUB_FILL, "oeq_hub_fill", 256, 256, cu * 16),
+        (rt.ROLE_CONV_FIXUP_FORWARD, "fixup_forward", 256, 1, cu * 32),
     ]
     t = em.tune
+    # Compensated sums run over whole segments (a compensation term does not carry across chunks).
+    hub_limit = 0 if kahan else max(0, t["conv_hub"])
     dims = dict(L1_dim=low.L1, L2_dim=low.L2, L3_dim=low.L3, weight_numel=low.WN, elem_size=low.elem_size,
                 shared_weights=int(shared), deterministic=rt.CONV_SORTED if deterministic else rt.CONV_GROUPED,
                 wpartial_per_block=em.backward_waves if shared else 0, dx_mode=rt.DX_TERMS, n_chunks=1,
-                order_hops=max(0, t["conv_hops"]))
+                order_hops=max(0, t["conv_hops"]), hub_limit=hub_limit)
     return s.text(), dims, descs
 
 

@@ -53,6 +53,15 @@ def _odd_shared():
                           (0, 0, 2, "uvu", True)], shared_weights=True, internal_weights=False, label="odd-uvu")
 
 
+def _uvw(shared):
+    # 'uvw' with channels on the second operand as well, so that shared weights do not factor out of the
+    # sum over edges: the fused per-edge walk runs in both cases
+    return oeq.TPProblem("12x0e+7x1o", "2x0e+1x1o", "9x0e+12x1o+5x1e",
+                         [(0, 0, 0, "uvw", True), (1, 1, 0, "uvw", True), (0, 1, 1, "uvw", True),
+                          (1, 0, 1, "uvw", True), (1, 1, 2, "uvw", True)], shared_weights=shared,
+                         internal_weights=False, label="uvw-shared" if shared else "uvw")
+
+
 HUBS = [
     # (name, problem, nodes, hub degree, second hub, background edges)
     ("cfg2-hub12000", P.config2_nequip_uvu, 14000, 12000, 700, 20000),
@@ -61,6 +70,9 @@ HUBS = [
     ("mace-large-hub600", lambda: P.mace_problems()[0], 900, 600, 0, 500),
     ("odd-shared-hub5000", _odd_shared, 6000, 5000, 300, 4000),         # bounded grid, strided walk
     ("benzene-hub700", lambda: P.nequip_problems()[3], 900, 700, 0, 300),  # node shared between waves
+    ("uvw-hub4000", lambda: _uvw(False), 5000, 4000, 300, 3000),        # the channel-mixing walk
+    ("uvw-shared-hub4000", lambda: _uvw(True), 5000, 4000, 300, 3000),
+    ("e3tools-hub700", lambda: P.e3tools_problems()[0], 900, 700, 0, 300),
 ]
 
 
@@ -135,10 +147,11 @@ def test_chunked_walk_is_a_function_of_the_edge_list():
     assert float((dxa - dx).abs().max() / dx.abs().max()) <= 1e-5
 
 
-def test_hub_second_order_matches_composition():
+@pytest.mark.parametrize("make", [P.config2_nequip_uvu, lambda: _uvw(False)], ids=["uvu", "uvw"])
+def test_hub_second_order_matches_composition(make):
     """The fused second-order pair on a hub graph (kernel A writes rows of extra chunks, kernel B walks
     them) against the composition of first-order calls, which is linear algebra on the same operands."""
-    problem = P.config2_nequip_uvu()
+    problem = make()
     n = 2500
     rows, cols = _hub_graph(n, 1500, 2500, seed=6)
     g = CoordGraph(np.zeros((n, 3)), rows, cols)
