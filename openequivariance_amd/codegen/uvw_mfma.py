@@ -249,13 +249,14 @@ class MfmaEmitter:
         # block sit out the multiplies and there are four times as many kernels.
         wpe = 2 if self.words == 1 else 1
         self.tune = tuning(dict(uvw_wf=wpe, uvw_wx=wpe, uvw_ww=wpe, uvw_blocks=2, uvw_pipe=1, uvw_regs=220,
-                                uvw_merge=1, uvw_fregs=232, uvw_wregs=232, uvw_xregs=215, uvw_mfma_dd=1))
+                                uvw_merge=1, uvw_fregs=232, uvw_wregs=232, uvw_xregs=215, uvw_mfma_dd=1, uvw_gdma=1))
 
     # Variant of the kernels being written (see second_order_kernels): a name prefix, the kernel signature, the
     # lines that bind the names the bodies use (L1_in, L2_in, W, ...) to its parameters, whether every result is
     # added to what the output holds, and whether the contraction T is that of the second-order pass,
     # T(a, y) + T(x, b), with the second pair of operands bound to L1_alt / L2_alt.
     prefix = ""
+    sy, sdy = "s_y", "s_dy[wave]"   # where the dX kernels find the tile's Y rows and leave their partial dY
     alias: List[str] = []
     accumulate = False
     t1 = False
@@ -379,6 +380,38 @@ class MfmaEmitter:
             s(f"s_g[r][{dst0} + c] = (row0 + r < num_batch) ? L3_grad[(row0 + r) * {low.L3} + {col0} + c] : T(0);")
             s.close()
 
+    def _dma_g(self, s: Src, tile: str, buf: str):
+        """The dZ tile of ``tile`` -> s_g[buf] by direct global-to-LDS loads (no registers, nothing to wait for
+        here): every wave moves its 4 rows, 64 lanes x 16 bytes per instruction to consecutive LDS addresses.
+        Rows past the batch read the last row (the dX kernels sum nothing over rows, and store nothing for them)."""
+        low = self.low
+        VW, rpw = self.vw, RT // WAVES
+        nc4 = low.L3 // VW
+        s.open("")
+        s(f"const i64 nrow0 = ({tile}) * {RT};")
+        for rr in range(rpw):
+            s.open("")
+            s(f"i64 row = nrow0 + wave * {rpw} + {rr}; if (row >= num_batch) row = num_batch - 1;")
+            s(f"const T* src = L3_grad + row * {low.L3};")
+            for j in range((nc4 + 63) // 64):
+                guard = f"if (lane + {64 * j} < {nc4}) " if (j + 1) * 64 > nc4 else ""
+                s(f"{guard}__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(src + {VW} * (lane + {64 * j})), "
+                  f"(OEQ_LPTR)&s_g[{buf}][wave * {rpw} + {rr}][{VW * 64 * j}], 16, 0, 0);")
+            s.close()
+        s.close()
+
+    def _y_regs(self) -> int:
+        return (RT * self.low.L2 + 64 * WAVES - 1) // (64 * WAVES)
+
+    def _load_flat_rows(self, s: Src, dst: str, src: str, row0: str):
+        """dst[q] = element tid + 256 q of the [16, L2] tile of ``src`` that starts at row ``row0`` (zero past the
+        batch)."""
+        L2 = self.low.L2
+        for q in range(self._y_regs()):
+            t = f"(tid + {64 * WAVES * q})"
+            inside = f"{t} < {RT * L2} && " if (q + 1) * 64 * WAVES > RT * L2 else ""
+            s(f"{dst}[{q}] = ({inside}({row0}) * {L2} + {t} < num_batch * {L2}) ? {src}[({row0}) * {L2} + {t}] : T(0);")
+
     def _load_x_rows(self, s: Src, dst: str, vp: VPath):
         """X of the wave's 4 rows for a sub-path, lanes = channel u of its input piece (T-compute layout);
         lanes beyond the piece read its last channel (their T values are never multiplied)."""
@@ -438,7 +471,7 @@ class MfmaEmitter:
             for k in range(d3):
                 s(f"Gk[{k}] = {G}[{k}][i];")
             yo = f", {vp.v * self.low.in2[vp.p.i2].d}" if self.multi_v else ""
-            s(f"cg_bwd{vp.p.index}({x}[i], s_y[{self.row('i')}], Gk, {dx}[i], dy[i]{yo});")
+            s(f"cg_bwd{vp.p.index}({x}[i], {self.sy}[{self.row('i')}], Gk, {dx}[i], dy[i]{yo});")
             s.close()
 
         if pipe == 0:
@@ -527,7 +560,7 @@ class MfmaEmitter:
             s.close()
             cur = half
         for t in range(cur):
-            s(f"if (at + {t} < {n}) s_dy[wave][{self.row(f'((at + {t}) / {low.L2})')}][(at + {t}) % {low.L2}] = rv[{t}];")
+            s(f"if (at + {t} < {n}) {self.sdy}[{self.row(f'((at + {t}) / {low.L2})')}][(at + {t}) % {low.L2}] = rv[{t}];")
         s.close()
 
     # ------------------------------------------------------------- forward
@@ -716,10 +749,6 @@ class MfmaEmitter:
                 continue
             paths_all = [vp for _, ps, _ in ker for vp in ps]
             uok = lambda vi: f"act{vi}" if self.vin[vi].mul % 16 == 0 else f"uok{vi}"
-            self.g_at = lambda row, col: f"s_g[{row}][{col}]"
-            s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self.gstride}];")
-            s(f"__shared__ T s_y[{RT}][{low.L2}];")
-            s(f"__shared__ T s_dy[{WAVES}][{RT}][{low.L2}];")
             self._prologue(s)
             for vi, _, _ in ker:
                 s(f"const bool act{vi} = wave * 16 < {self.vin[vi].mul};  // this wave has input channels in the piece")
@@ -744,6 +773,25 @@ class MfmaEmitter:
                     self.lds_w.append(by_cost[len(self.lds_w)].index)
             if self.lds_w:
                 s(f"__shared__ T s_wl[{len(self.lds_w)}][16][{64 * WAVES}];")
+            # Two copies of the tile's LDS data (dZ, Y, partial dY), where two blocks per CU still fit (80 KB each):
+            # the next tile's dZ arrives by direct global-to-LDS loads while this one is multiplied, its Y through
+            # registers, and the partial dY of a tile are summed after the next tile's barrier, so a tile costs one
+            # barrier. Else one copy, staged through registers, three barriers per tile.
+            lds_two = 2 * (RT * self.gstride + (1 + WAVES) * RT * low.L2) * low.elem_size + \
+                len(self.lds_w) * 16 * 64 * WAVES * low.elem_size
+            dma = bool(self.tune["uvw_gdma"]) and low.L3 % self.vw == 0 and lds_two <= 80 * 1024 and not self.t1
+            if dma:
+                self.g_at = lambda row, col: f"s_g[gb][{row}][{col}]"
+                self.sy, self.sdy = "s_y[gb]", "s_dy[gb][wave]"
+                s(f"__shared__ __attribute__((aligned(16))) T s_g[2][{RT}][{self.gstride}];")
+                s(f"__shared__ T s_y[2][{RT}][{low.L2}];")
+                s(f"__shared__ T s_dy[2][{WAVES}][{RT}][{low.L2}];")
+            else:
+                self.g_at = lambda row, col: f"s_g[{row}][{col}]"
+                self.sy, self.sdy = "s_y", "s_dy[wave]"
+                s(f"__shared__ __attribute__((aligned(16))) T s_g[{RT}][{self.gstride}];")
+                s(f"__shared__ T s_y[{RT}][{low.L2}];")
+                s(f"__shared__ T s_dy[{WAVES}][{RT}][{low.L2}];")
             for vi, ps, _ in ker:
                 self._load_wreg(s, [vp for vp in ps if vp.index not in self.lds_w], transposed=True,
                                 act=uok(vi), u=f"u{vi}")
@@ -754,11 +802,57 @@ class MfmaEmitter:
                 cond = f"({uok(vp.vi)}{wcond})" if wcond else uok(vp.vi)
                 s(f"for (int st = 0; st < {4 * c16(vp.Wn)}; ++st) s_wl[{n}][st][tid] = "
                   f"{cond} ? W[{vp.woff} + u{vp.vi} * {vp.ld} + 4 * st + lq] : T(0);")
-            s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
-            s(f"const i64 row0 = tile * {RT};")
-            s("__syncthreads();")
-            self._stage_g(s)
-            self._stage_y(s)
+            rmw_dy = not (first_dy and not self.accumulate)
+            ny = self._y_regs()
+            if dma:
+                # first tile: dZ on its way to copy 0, Y through registers
+                def put_y(buf):
+                    for q in range(ny):
+                        guard = f"if (tid + {64 * WAVES * q} < {RT * low.L2}) " if (q + 1) * 64 * WAVES > RT * low.L2 else ""
+                        s(f"{guard}(&s_y[{buf}][0][0])[tid + {64 * WAVES * q}] = ynext[{q}];")
+
+                def finish_dy(buf):
+                    """dY of the tile before (rows from prow0): the four waves' partial sums, in wave order, on top
+                    of what the earlier kernels left there."""
+                    for q in range(ny):
+                        tq = f"(tid + {64 * WAVES * q})"
+                        inside = f"{tq} < {RT * low.L2} && " if (q + 1) * 64 * WAVES > RT * low.L2 else ""
+                        s.open(f"if ({inside}prow0 * {low.L2} + {tq} < num_batch * {low.L2})")
+                        s(f"const int r = {tq} / {low.L2}, c = {tq} % {low.L2};")
+                        s(f"const T tot = ((s_dy[{buf}][0][r][c] + s_dy[{buf}][1][r][c]) + s_dy[{buf}][2][r][c]) + "
+                          f"s_dy[{buf}][3][r][c];")
+                        s(f"L2_grad[prow0 * {low.L2} + {tq}] = {f'dyold[{q}] + tot' if rmw_dy else 'tot'};")
+                        s.close()
+
+                s("int gb = 0;")
+                s("i64 prow0 = -1;  // first row of the tile whose dY is still to be written")
+                s(f"T ynext[{ny}];")
+                if rmw_dy:
+                    s(f"T dyold[{ny}];")
+                s.open("if ((i64)blockIdx.x < ntiles)")
+                self._dma_g(s, "(i64)blockIdx.x", "0")
+                self._load_flat_rows(s, "ynext", "L2_in", f"(i64)blockIdx.x * {RT}")
+                put_y("0")
+                s.close()
+                s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x, gb ^= 1)")
+                s(f"const i64 row0 = tile * {RT};")
+                # This tile's dZ has landed (each wave waits for its own loads, the barrier for everybody's) and its
+                # Y rows are written; the waves' partial dY of the tile before are complete; all reads of the other
+                # copies (two tiles back) are done.
+                s('asm volatile("s_waitcnt vmcnt(0)" ::: "memory");')
+                s("__syncthreads();")
+                s('asm volatile("" ::: "memory");')
+                s("const bool more = tile + gridDim.x < ntiles;")
+                s.open("if (prow0 >= 0)")
+                finish_dy("gb ^ 1")
+                s.close()
+                s("prow0 = row0;")
+            else:
+                s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
+                s(f"const i64 row0 = tile * {RT};")
+                s("__syncthreads();")
+                self._stage_g(s)
+                self._stage_y(s)
             # X of the lane's 4 (row, channel) pairs: issued before the barrier and the MFMA loop
             s(f"T dy[4][{low.L2}];")
             for vi, _, _ in ker:
@@ -775,7 +869,17 @@ class MfmaEmitter:
                 s.close()
             s(f"for (int j = 0; j < {low.L2}; ++j) dy[i][j] = T(0);")
             s.close()
-            s("__syncthreads();")
+            if not dma:
+                s("__syncthreads();")
+            else:
+                # Requested after the X rows: loads return in order, so the wait for X does not include these.
+                if rmw_dy:
+                    # what the earlier kernels left in this tile's dY
+                    self._load_flat_rows(s, "dyold", "L2_grad", "row0")
+                s.open("if (more)")
+                self._load_flat_rows(s, "ynext", "L2_in", f"(tile + gridDim.x) * {RT}")
+                self._dma_g(s, "tile + gridDim.x", "gb ^ 1")
+                s.close()
             for vi, ps, first in ker:
                 b1 = self.vin[vi]
                 s.open(f"if (act{vi})")
@@ -792,12 +896,24 @@ class MfmaEmitter:
                 s.close()
             # dY: sum over the 16 channels of the lane group, then over the 4 waves through LDS
             self._reduce_dy(s)
+            if dma:
+                # Y of the next tile into the other copy (last read two barriers ago)
+                s.open("if (more)")
+                put_y("gb ^ 1")
+                s.close()
+                s.close()  # tiles
+                s("__syncthreads();")
+                s.open("if (prow0 >= 0)")
+                finish_dy("gb ^ 1")  # (gb was flipped on leaving the last tile)
+                s.close()
+                s.close()  # kernel
+                first_dy = False
+                continue
             s("__syncthreads();")
             s.open(f"for (int t = tid; t < {RT * low.L2}; t += {64 * WAVES})")
             s(f"const int r = t / {low.L2}, c = t % {low.L2};")
             s("const T tot = ((s_dy[0][r][c] + s_dy[1][r][c]) + s_dy[2][r][c]) + s_dy[3][r][c];")
-            s(f"if (row0 + r < num_batch) L2_grad[(row0 + r) * {low.L2} + c] "
-              f"{'=' if first_dy and not self.accumulate else '+='} tot;")
+            s(f"if (row0 + r < num_batch) L2_grad[(row0 + r) * {low.L2} + c] {'+=' if rmw_dy else '='} tot;")
             s.close()
             s.close()
             s.close()
