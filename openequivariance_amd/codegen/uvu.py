@@ -2312,8 +2312,8 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         if low.shared_weights:
             descs.append((rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 64, 0))
         from . import uvu_double
-        if t["conv_dd"] and uvu_double.supported(low, conv=True) and not kahan:
-            descs += uvu_double.add_conv_kernels(s, low, em, t, xcd, G_b, compute_units)
+        if t["conv_dd"] and uvu_double.supported(low, conv=True):
+            descs += uvu_double.add_conv_kernels(s, low, em, t, xcd, G_b, compute_units, kahan)
         # counting sort: of the edge indices by node (GROUPED mode) and of the nodes by cluster (walk order)
         descs += [
             (rt.ROLE_GROUP_COUNT, "oeq_group_count", 256, 256 * 4, compute_units * 16),

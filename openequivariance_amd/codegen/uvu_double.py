@@ -512,12 +512,16 @@ class DoubleEmitter(UvuEmitter):
                 if self.cur_chunk is not None and not self._out_of(self.segments[si]):
                     return
                 s(f"D{si}_t a; zero_dseg{si}(a);")
+                if self.kahan:
+                    s(f"D{si}_t c; zero_dseg{si}(c);")
                 s.open(f"for (i64 e = e0 + r; e < e1; e += {self.R})")
                 self._edge_rows(s, "e")
                 s("X_t x, xa;")
                 self._load_x(s, "xrow", self.seg_in1[si])
                 self._load_x(s, "arow", self.seg_in1[si], "xa")
-                s(f"dda_seg{si}{self._sfx()}(x, xa, yrow, brow, wrow, crow, u, a);")
+                s(f"dda_seg{si}{self._sfx()}(x, xa, yrow, brow, wrow, crow, u, {'c' if self.kahan else 'a'});")
+                if self.kahan:
+                    s(f"kahan_dseg{si}(c, a);")
                 s.close()
                 if self.R > 1:
                     for io in self.segments[si]:
@@ -829,7 +833,7 @@ def add_tp_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, groups_b:
 
 
 def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: int, groups_b: int = 0,
-                     compute_units: int = 256) -> List[tuple]:
+                     compute_units: int = 256, kahan: bool = False) -> List[tuple]:
     """Append the convolution double-backward kernels (receiver-major walk) to a module. Shared weights: kernel B
     runs with the first-order backward kernel's wave groups per block (``groups_b``) on a bounded grid, one
     partial weight-gradient row per group, and is never split between waves or merged with kernel A."""
@@ -840,7 +844,7 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
         blocks the segment's paths read, one W and one C value per path."""
         worst = 0
         for si, seg in enumerate(e.segments):
-            acc = sum(low.out[io].d for io in seg)
+            acc = (2 if kahan else 1) * sum(low.out[io].d for io in seg)  # (and their compensation terms)
             xin = sum(low.in1[b].d for b in e.seg_in1[si])
             wc = sum(2 * low.in2[p.i2].mul for p in low.paths if p.io in seg)
             worst = max(worst, e.words * (acc + 2 * xin + wc))
@@ -851,12 +855,14 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     # spill there, up to 149 registers, and take the largest budget that leaves the widest segment under
     # 160 words - with the spills the fused pair was slower than composing first-order kernels.
     if tune.get("dd_acc", 0) > 0:
-        em = DoubleEmitter(low, acc_budget_words=tune["dd_acc"])
+        em = DoubleEmitter(low, acc_budget_words=tune["dd_acc"], kahan=kahan)
     else:
-        em = DoubleEmitter(low, acc_budget_words=112)
+        em = DoubleEmitter(low, acc_budget_words=56 if kahan else 112, kahan=kahan)
         if kernel_a_need(em) > 200:
-            for budget in (80, 64, 48, 32):
-                em = DoubleEmitter(low, acc_budget_words=budget)
+            for budget in (80, 64, 48, 32, 24, 16):
+                if kahan and budget > 48:
+                    continue
+                em = DoubleEmitter(low, acc_budget_words=budget, kahan=kahan)
                 if kernel_a_need(em) <= 160:
                     break
     em.nt = base.nt
@@ -875,7 +881,7 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     # twice). Measured slower on MI355X for every shape tried (MACE shape 37 - 85 ms against 33 ms for the
     # pair): its accumulators on top of kernel B's state spill whatever the split, so it is off by default.
     shared = low.shared_weights
-    em.merged = bool(tune.get("dd_merge", 0)) and not shared
+    em.merged = bool(tune.get("dd_merge", 0)) and not shared and not kahan
     groups = em.plan_double_groups(max(1, 8 // em.NCH)) if tune.get("dd_split", 1) and not shared else None
     if em.merged and not groups and not em.merged_fits_one_wave():
         em.merged = False
@@ -913,3 +919,11 @@ def _emit_segment_structs(s: Src, em: DoubleEmitter, prefix: str):
             for k in range(low.out[io].d):
                 s(f"a.o{io}[{k}] = T(0);")
         s.close()
+        if em.kahan:
+            # c: one edge's terms plus the rounding error carried over; afterwards what did not fit into a
+            s.open(f"OEQ_DEV void kahan_{prefix.lower()}seg{si}({prefix}{si}_t& c, {prefix}{si}_t& a)")
+            for io in seg:
+                for k in range(low.out[io].d):
+                    e = f"o{io}[{k}]"
+                    s(f"{{ const T y = c.{e}; const T t = a.{e} + y; c.{e} = y - (t - a.{e}); a.{e} = t; }}")
+            s.close()

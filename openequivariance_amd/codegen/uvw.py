@@ -1026,9 +1026,10 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     # by oeq_wreduce), so that grid is bounded
     max_b = cu * (3 if em.shared_lds else 2) if shared else cu * 16
     second = []
-    if em.tune["uvw_dd"] and not kahan:
-        # second-order pair: the same receiver walk / per-edge pass with the operands of both orders
-        blk_da, G_da = em.emit_conv_forward(s, False, second=True)
+    if em.tune["uvw_dd"]:
+        # second-order pair: the same receiver walk / per-edge pass with the operands of both orders (with
+        # ``kahan`` kernel A adds each edge's three terms with a compensation term, like the forward kernel)
+        blk_da, G_da = em.emit_conv_forward(s, kahan, second=True)
         blk_db = em.emit_backward(s, conv=True, second=True, force_waves=em.backward_waves if shared else 0)
         second = [(rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_A", blk_da, G_da, cu * 32),
                   (rt.ROLE_DOUBLE_BACKWARD_B, "double_backward_B", blk_db, 1, max_b)]

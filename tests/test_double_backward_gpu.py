@@ -230,6 +230,61 @@ def test_conv_fused_matches_composition(name, make, batch, det, monkeypatch):
     _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
 
 
+KAHAN_CONV = [c for c in CONV_CASES if c[0] in ("cfg2", "cfg3", "odd", "folded", "lips")] + UVW_CONV[:2]
+
+
+@pytest.mark.parametrize("name,make,batch", KAHAN_CONV, ids=[c[0] for c in KAHAN_CONV])
+def test_conv_kahan_has_the_fused_pair(name, make, batch):
+    """kahan=True: kernel A adds each edge's three terms with a compensation term (its sums run over a node's
+    edges like the forward kernel's), kernel B's sender gradients go through the compensated ordered reduction.
+    Against the composition of the kahan first-order kernels and against the plain fused pair."""
+    problem = make()
+    gph = _graph()
+    n, E = gph.coords.shape[0], gph.nnz
+    conv = oeq.TensorProductConv(problem, deterministic=True, kahan=True)
+    plain = oeq.TensorProductConv(problem, deterministic=True)
+    e = ops.get_entry(conv.kid)
+    assert e.kernels().has_double_backward()
+    dt = np.dtype(problem.irrep_dtype)
+    rng = np.random.default_rng(8)
+    tr, tc, tp = (torch.tensor(v, device="cuda") for v in (gph.rows, gph.cols, gph.transpose_perm))
+    x, a = (_rand(rng, (n, e.L1), dt) for _ in range(2))
+    y, b = (_rand(rng, (E, e.L2), dt) for _ in range(2))
+    w, c = (_rand(rng, (E, e.WN), dt) for _ in range(2))
+    g = _rand(rng, (n, e.L3), dt)
+    fused = ops.conv_double_backward(x, y, w, g, a, b, c, tr, tc, tp, conv.kid)
+    composed = ops._second_order(lambda p, q, r: ops.conv_forward(p, q, r, tr, tc, tp, conv.kid),
+                                 lambda p, q, r, s: ops.conv_backward(p, q, r, s, tr, tc, tp, conv.kid),
+                                 x, y, w, g, a, b, c)
+    _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
+    _check(("dx", "dy", "dw", "gg"), fused, ops.conv_double_backward(x, y, w, g, a, b, c, tr, tc, tp, plain.kid),
+           tol_of(problem))
+
+
+def test_conv_kahan_second_order_on_a_hub():
+    """A node with 3000 same-sign terms: the compensated kernel A is closer to the float64 sum than the plain one."""
+    problem = P.config1_single_uvu()
+    n, hub = 3200, 3000
+    rows = np.concatenate([np.zeros(hub, np.int64), np.arange(1, 200)])
+    cols = np.concatenate([np.arange(1, hub + 1), np.arange(2, 201)])
+    gph = CoordGraph(np.zeros((n, 3)), rows, cols)
+    E = gph.nnz
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    mk = lambda *shape: torch.rand(*shape, device="cuda", generator=gen) + 0.5
+    d = ops.get_entry(oeq.TensorProductConv(problem, deterministic=True).kid)
+    x, a, y, b, w, c, g = mk(n, d.L1), mk(n, d.L1), mk(E, d.L2), mk(E, d.L2), mk(E, d.WN), mk(E, d.WN), mk(n, d.L3)
+    tr, tc, tp = (torch.tensor(v, device="cuda") for v in (gph.rows, gph.cols, gph.transpose_perm))
+    got = {}
+    for kahan in (False, True):
+        conv = oeq.TensorProductConv(problem, deterministic=True, kahan=kahan)
+        assert ops.get_entry(conv.kid).kernels().has_double_backward()
+        got[kahan] = ops.conv_double_backward(x, y, w, g, a, b, c, tr, tc, tp, conv.kid)[3][0].double()
+    c64 = oeq.TensorProductConv(_f64(problem), deterministic=True)
+    ref = ops.conv_double_backward(*(t.double() for t in (x, y, w, g, a, b, c)), tr, tc, tp, c64.kid)[3][0]
+    errs = {k: float((v - ref).abs().max() / ref.abs().max()) for k, v in got.items()}
+    assert errs[True] <= max(errs[False], 1e-7) and errs[True] <= 2e-7, errs
+
+
 @pytest.mark.parametrize("det", [True, False], ids=["sorted", "grouped"])
 def test_unfused_convolution_second_order_matches_fused(det, monkeypatch):
     """The unfused convolution (gathered rows, batch kernels, ordered sums; here selected by a knob for a problem
