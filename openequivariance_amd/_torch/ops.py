@@ -54,6 +54,9 @@ class KernelEntry:
         # Shared-weight 'uvw' convolution as contraction + channel mix per node (core/problems.py:
         # factor_shared_uvw): ids of the two kernel sets that then do the work, else None.
         self.factored: Optional[Tuple[int, int]] = None
+        # Float-atomics convolution kernels (conv_sort=0) have no second-order pair of their own: id of the
+        # grouped-walk kernel set of the same problem, whose fused pair takes the edges in any order as well.
+        self.second_order_kid: Optional[int] = None
         self._ks: Optional[rt.KernelSet] = None
         self._lock = threading.Lock()
 
@@ -135,9 +138,14 @@ def _entry_from_spec(spec: bytes) -> KernelEntry:
                 factored = (register_spec(make_spec("conv", parts[0], False, False)),
                             register_spec(make_spec("tp", parts[1])))
             unfused = factored is None and not fused(low)
+            sibling = None
+            if low.mode == "uvu" and not det and not tuning(dict(conv_sort=1))["conv_sort"]:
+                walk = dict(desc, tune=(tune + "," if tune else "") + "conv_sort=1")
+                sibling = register_spec(json.dumps(walk, sort_keys=True, separators=(",", ":")).encode())
         entry = KernelEntry(build, low.L1, low.L2, low.L3, low.WN, low.shared_weights, dtype, deterministic=det,
                             unfused=unfused)
         entry.factored = factored
+        entry.second_order_kid = sibling
     entry.spec = torch.frombuffer(bytearray(spec), dtype=torch.uint8)
     return entry
 
@@ -309,6 +317,8 @@ def _use_fused(kid, spec, ddx, ddy, ddw) -> bool:
     if sum(t is not None for t in (ddx, ddy, ddw)) < 2:
         return False
     entry = get_entry(kid, spec)
+    if entry.second_order_kid is not None:
+        entry = get_entry(entry.second_order_kid)
     return bool(entry.factored) or entry.kernels().has_double_backward()
 
 
@@ -701,6 +711,8 @@ def conv_double_backward(L1_in: torch.Tensor, L2_in: torch.Tensor, W: torch.Tens
     """(L1_grad, L2_grad, W_grad, L3_dgrad): the op of the reference's jit_conv_double_backward
     (extension/torch_core.hpp:544-625)."""
     e = get_entry(kid, spec)
+    if e.second_order_kid is not None:
+        e = get_entry(e.second_order_kid)
     nodes, nnz = _conv_checks(e, L1_in, L2_in, W, rows, cols, transpose_perm, L3_grad)
     _conv_checks(e, L1_dgrad, L2_dgrad, W_dgrad, rows, cols, transpose_perm)
     x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), W.contiguous(), L3_grad.contiguous()

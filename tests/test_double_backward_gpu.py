@@ -8,6 +8,7 @@ import pytest
 import torch
 
 import openequivariance_amd as oeq
+from openequivariance_amd import runtime as rt
 from openequivariance_amd._torch import ops
 from openequivariance_amd.codegen import uvu_double
 from openequivariance_amd.core import problems as P
@@ -283,6 +284,40 @@ def test_conv_kahan_second_order_on_a_hub():
     ref = ops.conv_double_backward(*(t.double() for t in (x, y, w, g, a, b, c)), tr, tc, tp, c64.kid)[3][0]
     errs = {k: float((v - ref).abs().max() / ref.abs().max()) for k, v in got.items()}
     assert errs[True] <= max(errs[False], 1e-7) and errs[True] <= 2e-7, errs
+
+
+def test_float_atomics_convolution_uses_the_grouped_walk_pair(monkeypatch):
+    """conv_sort=0 selects the float-atomics kernels for the first-order ops; their second-order pass runs the fused
+    pair of the grouped-walk kernel set of the same problem (any edge order, fixed summation order) instead of
+    composing six float-atomics launches."""
+    monkeypatch.setenv("OEQ_AMD_TUNE", "conv_sort=0")
+    problem = P.config2_nequip_uvu()
+    conv = oeq.TensorProductConv(problem, deterministic=False)
+    e = ops.get_entry(conv.kid)
+    assert e.kernels().dims["deterministic"] == rt.CONV_ATOMIC and not e.kernels().has_double_backward()
+    assert e.second_order_kid is not None and ops.get_entry(e.second_order_kid).kernels().has_double_backward()
+    gph = _graph(300)
+    n, E = gph.coords.shape[0], gph.nnz
+    rng = np.random.default_rng(9)
+    order = rng.permutation(E)
+    tr, tc = (torch.tensor(v[order], device="cuda") for v in (gph.rows, gph.cols))
+    tp = torch.zeros(0, dtype=torch.int64, device="cuda")
+    x, a = (_rand(rng, (n, e.L1), np.float32) for _ in range(2))
+    y, b = (_rand(rng, (E, e.L2), np.float32) for _ in range(2))
+    w, c = (_rand(rng, (E, e.WN), np.float32) for _ in range(2))
+    g = _rand(rng, (n, e.L3), np.float32)
+    with torch.no_grad():
+        assert ops._use_fused(conv.kid, None, a, b, c)
+        fused = ops.conv_double_backward(x, y, w, g, a, b, c, tr, tc, tp, conv.kid)
+        composed = ops._second_order(lambda p, q, r: ops.conv_forward(p, q, r, tr, tc, tp, conv.kid),
+                                     lambda p, q, r, s: ops.conv_backward(p, q, r, s, tr, tc, tp, conv.kid),
+                                     x, y, w, g, a, b, c)
+    _check(("dx", "dy", "dw", "gg"), fused, composed, tol_of(problem))
+    # and through autograd: the force-training pattern
+    ts = [t.clone().requires_grad_(True) for t in (x, y, w)]
+    first = torch.autograd.grad(conv(*ts, tr, tc), ts, g, create_graph=True)
+    second = torch.autograd.grad(sum((t ** 2).sum() for t in first), ts)
+    assert all(torch.isfinite(t).all() for t in second)
 
 
 @pytest.mark.parametrize("det", [True, False], ids=["sorted", "grouped"])
