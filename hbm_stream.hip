@@ -15,6 +15,10 @@
 // XCD's blocks on their own 512 KB slice, and plain read-modify-write of 1024 private 16 KB slices. Under
 // rocprofv3 --pmc WRITE_SIZE / FETCH_SIZE they show where such updates are carried out: in the L2 (traffic =
 // the buffer, once) or on the memory side (traffic = every update).
+//
+// `./hbm_stream pipes` asks whether FP32 matrix instructions (v_mfma_f32_16x16x4_f32) and FP32 vector instructions
+// overlap on a SIMD: the same counts of each alone, interleaved one to eight inside a wave, and in phases of 64 and
+// 512, with one and with two waves per SIMD on every SIMD. (They do not on MI355X: every arrangement takes the sum.)
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -144,6 +148,75 @@ static int accumulate_modes() {
     return 0;
 }
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+// MODE 0: matrix instructions only; 1: vector only; 2: one matrix instruction then eight vector ones, repeated;
+// 3: 64 matrix instructions, then 512 vector ones. Per iteration every mode that has them issues 64 and 512.
+template <int MODE>
+__global__ __launch_bounds__(256) void pipes_kernel(float* out, float seed, int iters) {
+    v4f g[4];
+    for (int i = 0; i < 4; ++i) g[i] = v4f{0, 0, 0, 0};
+    float x[8];
+    for (int q = 0; q < 8; ++q) x[q] = seed + threadIdx.x * 1e-3f + q;
+    const float a = seed, b = seed * 0.5f;
+    for (int it = 0; it < iters; ++it) {
+        if (MODE == 0 || MODE == 3) {
+#pragma unroll
+            for (int m = 0; m < 64; ++m) g[m & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, g[m & 3], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (MODE == 1 || MODE == 3) {
+#pragma unroll
+            for (int v = 0; v < 64; ++v)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) x[q] = __builtin_fmaf(x[q], 0.999f, 0.001f);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (MODE == 2) {
+#pragma unroll
+            for (int m = 0; m < 64; ++m) {
+                g[m & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, g[m & 3], 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < 8; ++q) x[q] = __builtin_fmaf(x[q], 0.999f, 0.001f);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    float t = 0;
+    for (int q = 0; q < 8; ++q) t += x[q];
+    for (int i = 0; i < 4; ++i) t += g[i][0] + g[i][1] + g[i][2] + g[i][3];
+    if (t == 123.456f) out[0] = t;
+}
+
+template <int MODE>
+static float pipes_ms(int blocks, float* d) {
+    hipEvent_t a, b;
+    (void)hipEventCreate(&a);
+    (void)hipEventCreate(&b);
+    pipes_kernel<MODE><<<blocks, 256>>>(d, 1.0f, 16);
+    (void)hipDeviceSynchronize();
+    (void)hipEventRecord(a);
+    pipes_kernel<MODE><<<blocks, 256>>>(d, 1.0f, 2000);
+    (void)hipEventRecord(b);
+    (void)hipEventSynchronize(b);
+    float ms = 0.f;
+    (void)hipEventElapsedTime(&ms, a, b);
+    return ms;
+}
+
+static int pipes_modes() {
+    float* d = nullptr;
+    CHECK(hipMalloc(&d, 1024));
+    hipDeviceProp_t prop;
+    CHECK(hipGetDeviceProperties(&prop, 0));
+    for (int waves = 1; waves <= 2; ++waves) {
+        const int blocks = prop.multiProcessorCount * waves;  // 4 waves per block: one per SIMD
+        std::printf("waves per SIMD %d, 128 000 matrix and 1 024 000 vector instructions per wave: matrix only %.3f ms, "
+                    "vector only %.3f ms, interleaved in one wave %.3f ms, in phases %.3f ms\n",
+                    waves, pipes_ms<0>(blocks, d), pipes_ms<1>(blocks, d), pipes_ms<2>(blocks, d), pipes_ms<3>(blocks, d));
+    }
+    return 0;
+}
+
 template <typename F>
 static float median_ms(F launch, int iters = 7) {
     hipEvent_t a, b;
@@ -168,6 +241,7 @@ static float median_ms(F launch, int iters = 7) {
 
 int main(int argc, char** argv) {
     if (argc > 1 && std::string(argv[1]) == "accumulate") return accumulate_modes();
+    if (argc > 1 && std::string(argv[1]) == "pipes") return pipes_modes();
     const int n_chunks = 21000, chunk_bytes = 384 * 1024;  // 8.26 GB per buffer
     const int chunk_f4 = chunk_bytes / 16;
     const size_t bytes = (size_t)n_chunks * chunk_bytes, n = bytes / 16;
