@@ -70,6 +70,13 @@ WAVES = 4        # waves per block
 TPAD = RT + 1    # padded row stride of the T tile in LDS (bank spread)
 LDS_BUDGET = 160 * 1024 - 2048   # bytes of LDS a kernel may declare (the CU has 160 KB)
 MFMA = "oeq_mfma"  # v_mfma_f32_16x16x4_f32 or v_mfma_f64_16x16x4_f64, see tp_module
+# fp32 problems, split-operand form: every fp32 operand is written as the sum of three bf16 numbers (8 mantissa bits
+# each: 24 in all, the fp32 mantissa), a product as the six cross products of weight 2^-16 and above, each of them exact
+# in fp32, summed in fp32 by v_mfma_f32_16x16x32_bf16. That instruction does 8 times the multiplies of the fp32 one in
+# half its time (16 against 32 cycles), runs on a pipe of its own (the fp32 matrix instruction shares the vector
+# datapath), and the three dropped products are of the size of an fp32 rounding error.
+BF3_ROW = 72     # elements per row of a bf16 operand plane in LDS: 64 + 8, rows start 36 words apart
+BF3_TERMS = ((2, 0), (0, 2), (1, 1), (1, 0), (0, 1), (0, 0))  # (part of A, part of B), smallest products first
 
 
 def c4(n: int) -> int:
@@ -160,11 +167,13 @@ def _split(low: Lowered):
 SLICE_REGS = {"forward": 80, "dx": 80, "dw": 80}
 
 
-def _slice_regs(vp: VPath, which: str) -> int:
+def _slice_regs(vp: VPath, which: str, bf3: bool = False) -> int:
+    if bf3 and which == "forward":
+        return 12 * ((vp.U + 31) // 32)  # three parts of 8 bf16 (4 registers) per 32 input channels
     return c4(vp.U) if which == "forward" else 4 * c16(vp.Wn)
 
 
-def _groups(vpaths: List[VPath], side: str, n_blocks: int, which: str, limit=None):
+def _groups(vpaths: List[VPath], side: str, n_blocks: int, which: str, limit=None, bf3: bool = False):
     """Kernels of one pass (``which``: 'forward', 'dx' or 'dw'): for every piece on ``side`` ('vo' or 'vi') its
     sub-paths grouped by the piece index on the other side (all channels of the second operand), a group cut into
     parts whose weight slices fit ``limit(piece, sub-paths)`` registers. Returns [(piece, [sub-paths], first
@@ -180,11 +189,11 @@ def _groups(vpaths: List[VPath], side: str, n_blocks: int, which: str, limit=Non
             parts, room = [], 0
             sel = sorted((q for q in mine if getattr(q, other) == key), key=lambda q: (q.v, q.index))
             budget = min(SLICE_REGS[which], limit(b, sel)) if limit else SLICE_REGS[which]
-            total = sum(_slice_regs(vp, which) for vp in sel)
+            total = sum(_slice_regs(vp, which, bf3) for vp in sel)
             if total > budget:  # parts of about equal size
-                budget = max(-(-total // -(-total // budget)), max(_slice_regs(vp, which) for vp in sel))
+                budget = max(-(-total // -(-total // budget)), max(_slice_regs(vp, which, bf3) for vp in sel))
             for vp in sel:
-                need = _slice_regs(vp, which)
+                need = _slice_regs(vp, which, bf3)
                 if not parts or need > room:
                     parts.append([])
                     room = budget
@@ -249,7 +258,14 @@ class MfmaEmitter:
         # block sit out the multiplies and there are four times as many kernels.
         wpe = 2 if self.words == 1 else 1
         self.tune = tuning(dict(uvw_wf=wpe, uvw_wx=wpe, uvw_ww=wpe, uvw_blocks=2, uvw_pipe=1, uvw_regs=220,
-                                uvw_merge=1, uvw_fregs=232, uvw_wregs=232, uvw_xregs=215, uvw_mfma_dd=1, uvw_gdma=1))
+                                uvw_merge=1, uvw_fregs=232, uvw_wregs=232, uvw_xregs=215, uvw_mfma_dd=1, uvw_gdma=1,
+                                uvw_bf3=0))
+        # Forward kernels in the split-operand form (see BF3_TERMS). Off by default: correct to the fp32 bound, but
+        # its weight slices take 24 registers per path where the fp32 form takes 16, so config 4's forward becomes
+        # four kernels instead of two, and what those cost is their passes over X and Z, not their multiplies
+        # (1.09 against 0.90 ms). It pays once one kernel covers all paths of a tile.
+        self.bf3 = (self.words == 1 and bool(self.tune["uvw_bf3"])
+                    and 2 * self.max_d3 * 3 * RT * BF3_ROW * 2 + 2 * RT * low.L2 * 4 <= LDS_BUDGET)
 
     # Variant of the kernels being written (see second_order_kernels): a name prefix, the kernel signature, the
     # lines that bind the names the bodies use (L1_in, L2_in, W, ...) to its parameters, whether every result is
@@ -454,6 +470,72 @@ class MfmaEmitter:
             s.close()
         s.close()
 
+    def _t_compute_bf3(self, s: Src, vp: VPath, xsrc: str, buf: str, by_row: bool):
+        """The contraction T of a sub-path for the wave's 4 rows, lanes = channel u, split into three bf16 parts and
+        written to the operand planes s_Tb[buf][k][part]: ``by_row`` [row][channel] (A operand of the forward
+        multiply: 8 consecutive channels per lane), else [channel][row] (A operand of the dW multiply: 8 consecutive
+        rows). Two rows share every split (the conversions are packed)."""
+        d3 = self.vout[vp.vo].d
+        yo = f", {vp.v * self.low.in2[vp.p.i2].d}" if self.multi_v else ""
+        rpw = RT // WAVES
+        s.open("")
+        s(f"T t[{rpw}][{d3}];")
+        s.open(f"for (int rr = 0; rr < {rpw}; ++rr)")
+        s(f"const int r = wave * {rpw} + rr;")
+        if self.t1:
+            s(f"T t2[{d3}];")
+            s(f"cg_fwd{vp.p.index}(a{xsrc[1:]}[rr], s_y[r], t[rr]{yo});")
+            s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y2[r], t2{yo});")
+            for k in range(d3):
+                s(f"t[rr][{k}] += t2[{k}];")
+        else:
+            s(f"cg_fwd{vp.p.index}({xsrc}[rr], s_y[r], t[rr]{yo});")
+        s.close()
+        for k in range(d3):
+            if by_row:
+                for rp in range(rpw // 2):
+                    va, vb = f"t[{2 * rp}][{k}]", f"t[{2 * rp + 1}][{k}]"
+                    if vp.U < 64:
+                        # (channels beyond the piece are multiplied, with zero weights: they hold zeros)
+                        va, vb = f"(lane < {vp.U} ? {va} : T(0))", f"(lane < {vp.U} ? {vb} : T(0))"
+                    s(f"{{ unsigned q0, q1, q2; oeq_split2({va}, {vb}, q0, q1, q2);")
+                    for c in range(3):
+                        s(f"  s_Tb[{buf}][{k}][{c}][wave * {rpw} + {2 * rp}][lane] = (unsigned short)q{c}; "
+                          f"s_Tb[{buf}][{k}][{c}][wave * {rpw} + {2 * rp + 1}][lane] = (unsigned short)(q{c} >> 16);")
+                    s("}")
+            else:
+                assert rpw == 4
+                s(f"{{ unsigned q0, q1, q2, h0, h1, h2; oeq_split2(t[0][{k}], t[1][{k}], q0, q1, q2); "
+                  f"oeq_split2(t[2][{k}], t[3][{k}], h0, h1, h2);")
+                for c in range(3):
+                    s(f"  *(uint2*)&s_Tb[{buf}][{k}][{c}][lane][wave * {rpw}] = uint2{{q{c}, h{c}}};")
+                s("}")
+        s.close()
+
+    def _load_wb_forward(self, s: Src, vps: List[VPath], act: str):
+        """Weight slices of the forward multiply as bf16 B operands, split in three: for every 32 input channels
+        u' = 32 step + 8 (lane / 16) + i and the lane's output channel w = 16 wave + lane % 16, W[u'][w]."""
+        for vp in vps:
+            steps = (vp.U + 31) // 32
+            s(f"oeq_bf8 wb{vp.index}[{steps}][3];")
+            s.open("")
+            for st in range(steps):
+                s("{ float wv[8];")
+                for i in range(8):
+                    conds = [act]
+                    if 32 * st + 8 * 3 + i >= vp.U:
+                        conds.append(f"{32 * st} + 8 * lq + {i} < {vp.U}")
+                    if vp.Wn % 16:
+                        conds.append(f"wave * 16 + l16 < {vp.Wn}")
+                    s(f"  wv[{i}] = ({' && '.join(conds)}) ? W[{vp.woff} + ({32 * st} + 8 * lq + {i}) * {vp.ld} + wave * 16 + l16] : 0.0f;")
+                s("  unsigned q0[4], q1[4], q2[4];")
+                for j in range(4):
+                    s(f"  oeq_split2(wv[{2 * j}], wv[{2 * j + 1}], q0[{j}], q1[{j}], q2[{j}]);")
+                for c in range(3):
+                    s(f"  wb{vp.index}[{st}][{c}] = __builtin_bit_cast(oeq_bf8, oeq_u4{{q{c}[0], q{c}[1], q{c}[2], q{c}[3]}});")
+                s("}")
+            s.close()
+
     def _dx_paths(self, s: Src, paths: List[VPath], x: str = "x", dx: str = "dx"):
         """G = dZ W^T of every sub-path on the matrix cores, then its CG part on the vector ALU (in scope:
         x, dx, dy, s_g, s_y, wreg<path>). ``uvw_pipe`` = 0: path after path, operand order left to the
@@ -636,11 +718,11 @@ class MfmaEmitter:
         names = []
         # (the summed contraction of the second-order pass holds the rows of two operand pairs)
         xrows = (2 if self.t1 else 1) * 2 * (RT // WAVES) * self.max_d1
-        cost = lambda ker: (sum(c4(vp.U) for g in ker for vp in g[1]) + sum(4 * self.vout[g[0]].d for g in ker)
-                            + xrows + 64)
+        cost = lambda ker: (sum(_slice_regs(vp, "forward", self.bf3) for g in ker for vp in g[1])
+                            + sum(4 * self.vout[g[0]].d for g in ker) + xrows + 64)
         # (what the accumulators, the X rows and the rest leave for weight slices, at least two 64-channel slices)
         limit = lambda vo, sub: max(32, self.tune["uvw_fregs"] - (4 * self.vout[vo].d + xrows + 64))
-        for ker in self._merge(_groups(self.vpaths, "vo", len(self.vout), "forward", limit), cost,
+        for ker in self._merge(_groups(self.vpaths, "vo", len(self.vout), "forward", limit, self.bf3), cost,
                                self.tune["uvw_fregs"], self.vout):
             vo0, order0, _ = ker[0]
             if not order0 and self.accumulate:
@@ -653,7 +735,10 @@ class MfmaEmitter:
                 self._zero_kernel(s, "L3_out", low.L3, self.vout[vo0])
                 continue
             maxd = max(self.vout[vo].d for vo, _, _ in ker)
-            s(f"__shared__ T s_T[2][{maxd}][{self.tlanes}][{TPAD}];")
+            if self.bf3:
+                s(f"__shared__ __attribute__((aligned(16))) unsigned short s_Tb[2][{maxd}][3][{RT}][{BF3_ROW}];")
+            else:
+                s(f"__shared__ T s_T[2][{maxd}][{self.tlanes}][{TPAD}];")
             s(f"__shared__ T s_y[{RT}][{low.L2}];")
             if self.t1:
                 s(f"__shared__ T s_y2[{RT}][{low.L2}];")
@@ -665,7 +750,10 @@ class MfmaEmitter:
                 s(f"const bool act{vo} = wave * 16 < {self.vout[vo].mul};  // this wave has output channels in the piece")
             order_all = [vp for _, order, _ in ker for vp in order]
             for vo, order, _ in ker:
-                self._load_wreg(s, order, transposed=False, act=f"act{vo}")
+                if self.bf3:
+                    self._load_wb_forward(s, order, f"act{vo}")
+                else:
+                    self._load_wreg(s, order, transposed=False, act=f"act{vo}")
             s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x)")
             s(f"const i64 row0 = tile * {RT};")
             s("__syncthreads();  // all reads of the previous tile's LDS data are done")
@@ -682,17 +770,30 @@ class MfmaEmitter:
                 p = vp.p
                 bo = self.vout[vp.vo]
                 s(f"// path {p.index}: l=({low.in1[p.i1].l},{low.in2[p.i2].l},{bo.l}), input piece {vp.ub}")
-                self._t_compute(s, vp, cur, str(buf))
+                if self.bf3:
+                    self._t_compute_bf3(s, vp, cur, str(buf), by_row=True)
+                else:
+                    self._t_compute(s, vp, cur, str(buf))
                 if n + 1 < len(order_all):
                     self._load_x_rows(s, nxt, order_all[n + 1])
                 s("__syncthreads();")
                 s.open(f"if (act{vp.vo})")
-                s("#pragma unroll")
-                s.open(f"for (int st = 0; st < {c4(vp.U)}; ++st)")
-                for k in range(bo.d):
-                    s(f"acc{vp.vo}[{k}] = {MFMA}(s_T[{buf}][{k}][4 * st + lq][l16], wreg{vp.index}[st], "
-                      f"acc{vp.vo}[{k}], 0, 0, 0);")
-                s.close()
+                if self.bf3:
+                    for st in range((vp.U + 31) // 32):
+                        for k in range(bo.d):
+                            s.open("")
+                            for c in range(3):
+                                s(f"const oeq_bf8 a{c} = *(const oeq_bf8*)&s_Tb[{buf}][{k}][{c}][l16][{32 * st} + 8 * lq];")
+                            for ca, cb in BF3_TERMS:
+                                s(f"acc{vp.vo}[{k}] = oeq_mfma_bf(a{ca}, wb{vp.index}[{st}][{cb}], acc{vp.vo}[{k}], 0, 0, 0);")
+                            s.close()
+                else:
+                    s("#pragma unroll")
+                    s.open(f"for (int st = 0; st < {c4(vp.U)}; ++st)")
+                    for k in range(bo.d):
+                        s(f"acc{vp.vo}[{k}] = {MFMA}(s_T[{buf}][{k}][4 * st + lq][l16], wreg{vp.index}[st], "
+                          f"acc{vp.vo}[{k}], 0, 0, 0);")
+                    s.close()
                 s.close()
                 cur, nxt = nxt, cur
             # D layout: rows 4*lq + i, column (channel) l16 of the wave's slice
@@ -1086,6 +1187,21 @@ def tp_module(low: Lowered, compute_units: int = 256):
     s(f"typedef T oeq_vec16 __attribute__((ext_vector_type({16 // low.elem_size})));  // 16 bytes")
     if low.elem_size == 4:
         s("#define oeq_mfma __builtin_amdgcn_mfma_f32_16x16x4f32")
+        s("#define oeq_mfma_bf __builtin_amdgcn_mfma_f32_16x16x32_bf16")
+        s("typedef __bf16 oeq_bf8 __attribute__((ext_vector_type(8)));")
+        s("typedef __bf16 oeq_bf2 __attribute__((ext_vector_type(2)));")
+        s("typedef float oeq_f2 __attribute__((ext_vector_type(2)));")
+        s("typedef unsigned oeq_u4 __attribute__((ext_vector_type(4)));")
+        # a and b as sums of three bf16 numbers each (round to nearest, the remainders are exact in fp32); q<i> holds
+        # the i-th parts, a's in the low half
+        s("OEQ_DEV unsigned oeq_pk_bf16(float a, float b) { const oeq_f2 v = {a, b}; "
+          "return __builtin_bit_cast(unsigned, __builtin_convertvector(v, oeq_bf2)); }")
+        s("OEQ_DEV void oeq_split2(float a, float b, unsigned& q0, unsigned& q1, unsigned& q2) { "
+          "q0 = oeq_pk_bf16(a, b); "
+          "a -= __builtin_bit_cast(float, q0 << 16); b -= __builtin_bit_cast(float, q0 & 0xffff0000u); "
+          "q1 = oeq_pk_bf16(a, b); "
+          "a -= __builtin_bit_cast(float, q1 << 16); b -= __builtin_bit_cast(float, q1 & 0xffff0000u); "
+          "q2 = oeq_pk_bf16(a, b); }")
     else:
         s("#define oeq_mfma __builtin_amdgcn_mfma_f64_16x16x4f64")
         s("template <int CTRL> OEQ_DEV double oeq_dpp(double v) { const long long b = __builtin_bit_cast(long long, v); "

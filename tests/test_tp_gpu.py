@@ -7,6 +7,7 @@ import pytest
 import torch
 
 import openequivariance_amd as oeq
+from openequivariance_amd._torch import ops
 from openequivariance_amd.core import problems as P
 from oracle import e3nn_ref as R
 from gpu_util import err, to_gpu, tol_of, tp_inputs
@@ -228,6 +229,38 @@ def test_forward_backward_match_oracle(name, make, B):
     # a shared weight gradient sums `B` same-sign terms (the inputs are uniform[0,1)); it still has to meet
     # the tolerance of every other result
     assert err(tw.grad, dw_ref) <= tol
+
+
+BF3_CASES = [c for c in CASES if c[0] in ("cfg4-shared", "mfma-mixed", "mfma-pad-diffdock", "mfma-mul2-pad", "mfma-64-l3",
+                                          "mfma-l7")]
+
+
+@pytest.mark.parametrize("name,make,B", BF3_CASES, ids=[c[0] for c in BF3_CASES])
+def test_split_operand_forward(name, make, B, monkeypatch):
+    """uvw_bf3=1: the forward channel mix with every fp32 operand split into three bf16 parts and the six leading
+    cross products on the bf16 matrix instruction (the opt-in form of the matrix-core forward kernels). It meets the
+    same bound as the fp32 instruction; second order as well (its kernel A is made of forward kernels). A problem
+    whose operand planes exceed the LDS (l = 7) keeps the fp32 form."""
+    monkeypatch.setenv("OEQ_AMD_TUNE", "uvw_bf3=1")
+    problem = make()
+    x, y, w, g = tp_inputs(problem, B, seed=4321)
+    ref = R.Problem.from_spec(problem)
+    tp = oeq.TensorProduct(problem)
+    src = ops.get_entry(tp.kid).build_fn()[0]
+    assert ("oeq_mfma_bf(" in src) == (name != "mfma-l7")
+    tx, ty, tw = to_gpu(x, y, w, requires_grad=True)
+    z = tp(tx, ty, tw)
+    assert err(z, R.tp_forward(ref, x, y, w)) <= tol_of(problem)
+    (tg,) = to_gpu(g)
+    first = torch.autograd.grad(z, (tx, ty, tw), tg, create_graph=True)
+    second = torch.autograd.grad(sum((t ** 2).sum() for t in first), (tx, ty, tw))
+    monkeypatch.setenv("OEQ_AMD_TUNE", "")
+    tp0 = oeq.TensorProduct(problem)
+    ux, uy, uw = to_gpu(x, y, w, requires_grad=True)
+    first0 = torch.autograd.grad(tp0(ux, uy, uw), (ux, uy, uw), tg, create_graph=True)
+    second0 = torch.autograd.grad(sum((t ** 2).sum() for t in first0), (ux, uy, uw))
+    for a_, b_ in zip(second, second0):
+        assert float((a_ - b_).abs().max() / b_.abs().max()) <= 1e-5
 
 
 def test_same_precision_reference_is_not_closer_by_accident():
