@@ -263,7 +263,10 @@ class MfmaEmitter:
         # Forward kernels in the split-operand form (see BF3_TERMS). Off by default: correct to the fp32 bound, but
         # its weight slices take 24 registers per path where the fp32 form takes 16, so config 4's forward becomes
         # four kernels instead of two, and what those cost is their passes over X and Z, not their multiplies
-        # (1.09 against 0.90 ms). It pays once one kernel covers all paths of a tile.
+        # (1.09 against 0.90 ms). One kernel over all paths of a tile, with the split weight slices streamed from a
+        # buffer instead of living in registers, was tried as well: 1.10 ms, with the matrix pipe busy 18 % and
+        # the vector unit 20 % of the time - eleven block barriers per 16-row tile with about 600 cycles of matrix
+        # work between them. This form needs tiles whose rows belong to one wave (no barrier per path).
         self.bf3 = (self.words == 1 and bool(self.tune["uvw_bf3"])
                     and 2 * self.max_d3 * 3 * RT * BF3_ROW * 2 + 2 * RT * low.L2 * 4 <= LDS_BUDGET)
 
