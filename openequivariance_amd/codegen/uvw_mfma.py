@@ -266,7 +266,10 @@ class MfmaEmitter:
         # (1.09 against 0.90 ms). One kernel over all paths of a tile, with the split weight slices streamed from a
         # buffer instead of living in registers, was tried as well: 1.10 ms, with the matrix pipe busy 18 % and
         # the vector unit 20 % of the time - eleven block barriers per 16-row tile with about 600 cycles of matrix
-        # work between them. This form needs tiles whose rows belong to one wave (no barrier per path).
+        # work between them. A third form without LDS or barriers (a wave owns 16 rows and all output channels,
+        # lane = (row, 8 input channels): the contraction lands in the A-operand layout in registers; weight
+        # slices streamed from L2) took 1.22 ms: 256 registers leave no room to request the next step's operands
+        # while the current step is multiplied, so every step waits for its loads.
         self.bf3 = (self.words == 1 and bool(self.tune["uvw_bf3"])
                     and 2 * self.max_d3 * 3 * RT * BF3_ROW * 2 + 2 * RT * low.L2 * 4 <= LDS_BUDGET)
 
