@@ -416,6 +416,8 @@ def main():
         roofline["bounds_ms"]["fp32_vector_unpacked_as_measured"] = step_flops / (ceilings["valu_fp32_tflops_unpacked"] * 1e9)
         # this step writes 40 % of its algorithmic bytes: the measured rate of a read stream with writes mixed in
         roofline["bounds_ms"]["hbm_at_measured_read_write_mix"] = (fwd_bytes + bwd_bytes) / ceilings["read_with_writes_1_2"] / 1e6
+        # the step against that measured rate (frac above is against the published 8 TB/s)
+        roofline["step_frac_of_measured_read_write_mix"] = roofline["bounds_ms"]["hbm_at_measured_read_write_mix"] / ms_det
 
     modes = {
         "deterministic": {
