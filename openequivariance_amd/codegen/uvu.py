@@ -916,8 +916,12 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
     @staticmethod
     def _attrs(block: int, waves_per_eu: int) -> str:
         a = f"__launch_bounds__({block})"
-        if waves_per_eu:
+        if waves_per_eu > 0:
+            # exactly that many waves per SIMD: the register budget of that occupancy, and no more waves than that
             a += f" __attribute__((amdgpu_waves_per_eu({waves_per_eu}, {waves_per_eu})))"
+        elif waves_per_eu < 0:
+            # at least that many: the same register budget, but a kernel that needs fewer registers runs more waves
+            a += f" __attribute__((amdgpu_waves_per_eu({-waves_per_eu})))"
         return a
 
     # ---------------------------------------------------------- TP forward
@@ -2261,6 +2265,19 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     em.emit_structs(s)
     em.use_q = q_fwd
     em.emit_forward_cores(s, preloaded=True)
+    # Kernels with few words per lane (output segment, X blocks, weights: first and last layers of a network,
+    # narrow models) need well under 128 registers. The register budget of two waves per SIMD is then no help
+    # and the limit of two waves a loss: they get that budget as a minimum and run as many waves as their
+    # registers allow (config-5 graph, step: SevenNet first layer 3.96 -> 2.58 ms, last layers 3.85 -> 3.49,
+    # NequiX first layer 2.58 -> 2.30, MACE-medium 5.99 -> 5.68, NequIP water 2.18 -> 2.05). Larger kernels keep
+    # exactly two: without the limit the scheduler aims for an occupancy they cannot use (SevenNet main layer
+    # 15.3 -> 21.2 ms).
+    per_lane = (1 if low.elem_size == 4 else 2) * (max(sum(low.out[io].d for io in seg) for seg in em.segments)
+                                                   + sum(low.in1[b].d for b in em.used_in1) + em.n_wslots)
+    if walk and per_lane <= 48:
+        for knob in ("conv_wf", "conv_wb"):
+            if knob not in user_tune:
+                t[knob] = -2
     G_f = t["conv_gf"]
     G_b = 1 if em.NCH > 1 else t["conv_gb"]
     xcd = max(1, t["conv_xcd"])
