@@ -85,7 +85,10 @@ typedef enum {
     OEQ_ROLE_HUB_COUNT = 16,        /* long edge segments cut into chunks: extra walk positions per node, */
     OEQ_ROLE_HUB_FILL = 17,         /*   and the list of those positions */
     OEQ_ROLE_CONV_FIXUP_FORWARD = 18,/* adds the rows written by the extra chunks to their nodes' rows, in chunk order */
-    OEQ_ROLE_COUNT = 19
+    OEQ_ROLE_CONV_BACKWARD_DX = 19, /* OEQ_DX_SENDER_WALK: the sender gradients by a walk over the senders' edge segments
+                                       (forward-shaped: argument list of OEQ_ROLE_CONV_FORWARD with dZ for X, the
+                                       receivers for the senders and the sender-side index) */
+    OEQ_ROLE_COUNT = 20
 } oeq_role;
 
 /* How the convolution kernels of a set find the edges of a node (oeq_problem_dims.deterministic):
@@ -107,8 +110,12 @@ typedef enum {
 typedef enum {
     OEQ_DX_TERMS = 0,    /* terms go to scratch; fixup_backward sums them per sender in sender-major order */
     OEQ_DX_ATOMIC = 1,   /* terms are added into the cleared sender rows with float atomics (not bit-reproducible) */
-    OEQ_DX_ARRIVAL = 2   /* terms go to scratch; the wave that delivers the last term of a sender sums that
+    OEQ_DX_ARRIVAL = 2,  /* terms go to scratch; the wave that delivers the last term of a sender sums that
                             sender's terms in sender-major order (same bits as OEQ_DX_TERMS, no second kernel) */
+    OEQ_DX_SENDER_WALK = 3 /* no terms: OEQ_ROLE_CONV_BACKWARD_DX walks every sender's edges in sender-major order
+                            and forms its gradient row from dZ of the receivers, Y and W (this is the reference's
+                            scheme, loop_unroll_conv_det.cuh:187-293; chosen where rows of X are long and rows of dZ
+                            short) */
 } oeq_dx_mode;
 
 /* Several descriptors may name the same role: those kernels are launched back to back, in

@@ -13,7 +13,7 @@ a register budget.
 from __future__ import annotations
 
 import math
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import List, Tuple
 
 import numpy as np
@@ -226,3 +226,16 @@ def float_literal(v: float, ctype: str) -> str:
     if ctype == "float":
         return float(np.float32(v)).hex() + "f"
     return float(v).hex()
+
+
+def adjoint(low: Lowered) -> Lowered:
+    """The 'uvu' problem whose forward map is the X-gradient of ``low``: the roles of the first operand and the
+    output swapped, every structural non-zero (i, j, k, c) as (k, j, i, c), same weights (a 'uvu' path has one
+    weight per channel, whichever side the channel is read from) and same second operand. With dZ as its
+    first operand, ``forward(dZ, Y, W)`` of this problem is dX of the original."""
+    assert low.mode == "uvu"
+    paths = [Path(p.index, p.io, p.i2, p.i1, p.woff, p.coeff,
+                  sorted(((k, j, i, c) for (i, j, k, c) in p.nnz), key=lambda q: (q[1], q[0], q[2])),
+                  (p.l[2], p.l[1], p.l[0])) for p in low.paths]
+    return replace(low, in1=low.out, out=low.in1, paths=paths, L1=low.L3, L3=low.L1, label=f"{low.label}-adjoint")
+

@@ -1169,7 +1169,7 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         s.close()
 
     def emit_conv_forward(self, s: Src, G: int, deterministic: bool, pipelined: bool, waves_per_eu: int = 0,
-                          xcd: int = 1, tr_atomics: bool = True):
+                          xcd: int = 1, tr_atomics: bool = True, name: str = "forward"):
         low = self.low
         # With several output segments the waves of a node can each own some of them (their accumulators
         # stay in registers) and walk the node's edges side by side, instead of one wave walking the edges
@@ -1181,7 +1181,7 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         # vector-memory counter with the loads the loop waits for by count)
         mode = self._edge_mode(pipelined if (deterministic or pipelined != 4) else 2)
         s.open(
-            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void forward(i64 node_count, i64 nnz, '
+            f'extern "C" __global__ {self._attrs(block, waves_per_eu)} void {name}(i64 node_count, i64 nnz, '
             "const T* __restrict__ L1_in, const T* __restrict__ L2_in, const T* __restrict__ W, "
             "T* __restrict__ L3_out, const i64* __restrict__ rows, const i64* __restrict__ cols, "
             f"const i64* __restrict__ rowptr, const i64* __restrict__ eperm, const i64* __restrict__ order"
@@ -1932,7 +1932,7 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         s.close()
         return block
 
-    DX_TERMS, DX_ATOMIC, DX_ARRIVAL = 0, 1, 2
+    DX_TERMS, DX_ATOMIC, DX_ARRIVAL, DX_SENDER_WALK = 0, 1, 2, 3
 
     def emit_conv_backward(self, s: Src, deterministic: bool, G: int, pipelined: bool, waves_per_eu: int = 0,
                            g_resident: Optional[bool] = None, xcd: int = 1, tr_atomics: bool = True,
@@ -1945,7 +1945,9 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         order of ``sperm`` and writes the row, so the reduction needs no kernel of its own and stays
         bit-identical to ``fixup_backward``. (At the MACE shape the walk kernel is bound by its memory
         traffic, the in-kernel reduction adds the same 13 GB of reads to it, and the sum comes out slower
-        than the separate kernel: 15.0 against 14.6 ms. Hence opt-in, ``conv_dxm=2``.)"""
+        than the separate kernel: 15.0 against 14.6 ms. Hence opt-in, ``conv_dxm=2``.) DX_SENDER_WALK: this kernel
+        leaves dX alone (nothing of it is computed); a second, forward-shaped kernel walks the senders' edge
+        segments and forms dX from dZ, Y and W (``conv_module``)."""
         low = self.low
         shared = low.shared_weights
         if self.NCH > 1:
@@ -2037,10 +2039,12 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
                         s(f'asm volatile("" : "+{"s" if self.R == 1 else "v"}"(grow));')
                     self._bwd_paths(s, xname=xname, yacc=yacc, wacc=wacc, g_on_demand_row="grow",
                                     dw_mode="acc" if shared else "store")
-                self._pin_gradients(s, self.used_in1, deferred)
+                self._pin_gradients(s, [] if dx_mode == self.DX_SENDER_WALK else self.used_in1, deferred)
                 if deferred:
                     self._flush_dwkeep(s, None)
-                if not dx_atomic:
+                if dx_mode == self.DX_SENDER_WALK:
+                    pass  # (dx is dead: the compiler drops its arithmetic)
+                elif not dx_atomic:
                     s(f"T* dxrow = dx_tmp + {e} * {low.L1};")
                     # terms the arrival scheme re-reads soon are stored plainly, so that they stay cached
                     if dx_mode == self.DX_ARRIVAL:
@@ -2188,7 +2192,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=0, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
                     dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fw=0, conv_pf=0,
                     conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0, tp_forms=1,
-                    conv_hub=256))
+                    conv_hub=256, conv_dxs=-1))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
@@ -2312,6 +2316,14 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             # fit the edge's row of dx_tmp only when no used block has lanes without a channel
             if dx_mode == em.DX_ARRIVAL and (em.R != 1 or 64 * em.NCH * em._term_slots()[1] > low.L1):
                 dx_mode = em.DX_TERMS
+            # Rows of X much longer than an edge's weights and an output row together (the last layer of a
+            # network: many irreps in, a few scalars out): the per-edge dX terms, written and read back, would be
+            # most of the backward's traffic (2 L1 words per edge). A second walk over the SENDERS' edge segments
+            # that reads W and Y again and gathers the short dZ rows moves WN + L2 + L3 words per edge instead and
+            # sums in the same list order. It is the forward kernel of the adjoint problem (lower.adjoint).
+            auto = low.L1 >= low.WN + low.L2 + low.L3 and not low.shared_weights and t["conv_dxm"] < 0
+            if (t["conv_dxs"] > 0) or (t["conv_dxs"] < 0 and auto):
+                dx_mode = em.DX_SENDER_WALK
         blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd_b,
                                       bool(t["conv_tra"]), dx_mode)
         G_b = em.backward_groups_per_block
@@ -2328,6 +2340,24 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         ]
         if low.shared_weights:
             descs.append((rt.ROLE_TP_BACKWARD_WREDUCE, "oeq_wreduce", 256, 64, 0))
+        if dx_mode == UvuEmitter.DX_SENDER_WALK:
+            from .lower import adjoint
+            low_x = adjoint(low)
+            ex = UvuEmitter(low_x, acc_budget_words=t["conv_acc"])
+            ex.nt, ex.mask_loads, ex.forms, ex.tr_stores = t["conv_nt"], bool(t["tp_mask"]), bool(t["tp_forms"]), t["conv_trs"]
+            words_x = (1 if low.elem_size == 4 else 2) * (
+                max(sum(low_x.out[io].d for io in seg) for seg in ex.segments)
+                + sum(low_x.in1[b].d for b in ex.used_in1) + ex.n_wslots)
+            # (its structs and contraction functions have the names of the forward kernel's: a namespace of its own)
+            s("namespace oeq_dx {")
+            ex.emit_structs(s)
+            ex.use_q = False
+            ex.emit_forward_cores(s, preloaded=True)
+            G_x = max(1, 4 // low_x.n_chunks)
+            blk_x = ex.emit_conv_forward(s, G_x, True, t["conv_pipe_f"], -2 if words_x <= 48 else 2, xcd,
+                                         bool(t["conv_tra"]), name="backward_dx")
+            s("}  // namespace oeq_dx")
+            descs.append((rt.ROLE_CONV_BACKWARD_DX, "backward_dx", blk_x, G_x, 0, xcd))
         from . import uvu_double
         if t["conv_dd"] and uvu_double.supported(low, conv=True):
             descs += uvu_double.add_conv_kernels(s, low, em, t, xcd, G_b, compute_units, kahan)

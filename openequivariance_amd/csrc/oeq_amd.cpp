@@ -238,7 +238,7 @@ int static_scratch(void** out) {
 extern "C" {
 
 const char* oeq_last_error(void) { return g_error.c_str(); }
-int oeq_abi_version(void) { return 4; }
+int oeq_abi_version(void) { return 5; }
 
 int oeq_get_device_props(int device, oeq_device_props* out) {
     if (!out) return fail(OEQ_ERR_INVALID, "oeq_get_device_props: out is NULL");
@@ -602,7 +602,11 @@ static ScratchLayout scratch_layout(const oeq_kernels* k, int64_t node_count, in
         if (size_t hb = hub_rows_bytes(k, hub_rows_role, nnz)) w.hub_rows = take(hb);
     if (arrivals)
         w.arrivals = take(align_up((size_t)node_count * (size_t)std::max(1, k->dims.n_chunks) * sizeof(int32_t), 256));
-    if (terms) {
+    if (terms && wpartial_role == OEQ_ROLE_CONV_BACKWARD && k->dims.dx_mode == OEQ_DX_SENDER_WALK) {
+        // no terms: the sender-side walk forms the rows itself, and writes those of its extra chunks here
+        if (int64_t su = hub_units(k, OEQ_ROLE_CONV_BACKWARD_DX, nnz))
+            w.shub_rows = take(align_up((size_t)su * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256));
+    } else if (terms) {
         w.dx_tmp = take(align_up((size_t)nnz * (size_t)k->dims.L1_dim * (size_t)k->dims.elem_size, 256));
         // partial sums of the senders whose terms fixup_backward sums in chunks
         if (!arrivals)
@@ -936,7 +940,7 @@ int oeq_conv_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, c
         sc.arrivals = (int32_t*)at_offset(scratch, w.arrivals);
         sc.shub_rows = at_offset(scratch, w.shub_rows);
     }
-    if (dx_mode != OEQ_DX_TERMS) {
+    if (dx_mode == OEQ_DX_ATOMIC || dx_mode == OEQ_DX_ARRIVAL) {
         // atomics accumulate into the rows; the arrival scheme never visits a node that sends nothing
         rc = k->fill_zero(L1_grad, dx_bytes, stream);
         if (rc) return rc;
@@ -954,6 +958,20 @@ int oeq_conv_backward_indexed(oeq_kernels* k, int64_t node_count, int64_t nnz, c
     rc = k->launch(OEQ_ROLE_CONV_BACKWARD, walk_mode(k) ? node_count + units : nnz, args, stream);
     if (rc || !walk_mode(k)) return rc;
     if (dx_mode == OEQ_DX_TERMS) rc = sender_sum(k, node_count, nnz, sc.dx_tmp, L1_grad, ix, sc.shub_rows, stream);
+    if (dx_mode == OEQ_DX_SENDER_WALK) {
+        // The forward kernel of the adjoint problem over the sender side of the index: dZ rows of the receivers
+        // for the rows of X, every sender's segment in sender-major order, long segments in chunks.
+        int64_t limit = (ix.shubptr && sc.shub_rows) ? ix.hub_limit : 0;
+        int64_t xunits = limit ? hub_units(k, OEQ_ROLE_CONV_BACKWARD_DX, nnz) : 0;
+        void* xargs[] = {&node_count, &nnz,       &L3_grad,   &L2_in,     &W,           &L1_grad,      &cols,  &rows,
+                         &ix.colptr,  &ix.sperm,  &ix.order,  &ix.shubptr, &ix.shubnode, &limit,        &xunits, &sc.shub_rows};
+        rc = k->launch(OEQ_ROLE_CONV_BACKWARD_DX, node_count + xunits, xargs, stream);
+        if (!rc && xunits) {
+            int64_t row_len = k->dims.L1_dim;
+            void* cargs[] = {&node_count, &xunits, &ix.shubptr, &ix.shubnode, &sc.shub_rows, &L1_grad, &row_len};
+            rc = k->launch(OEQ_ROLE_CONV_FIXUP_FORWARD, xunits, cargs, stream);
+        }
+    }
     if (rc || !wrows) return rc;
     int64_t n_partials =
         (int64_t)k->grid_for(OEQ_ROLE_CONV_BACKWARD, node_count + units) * k->dims.wpartial_per_block;

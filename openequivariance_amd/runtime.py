@@ -53,10 +53,11 @@ ROLE_ORDER_HOP = 15
 ROLE_HUB_COUNT = 16
 ROLE_HUB_FILL = 17
 ROLE_CONV_FIXUP_FORWARD = 18
+ROLE_CONV_BACKWARD_DX = 19
 
 CONV_ATOMIC, CONV_SORTED, CONV_GROUPED = 0, 1, 2
-DX_TERMS, DX_ATOMIC, DX_ARRIVAL = 0, 1, 2
-ABI_VERSION = 4
+DX_TERMS, DX_ATOMIC, DX_ARRIVAL, DX_SENDER_WALK = 0, 1, 2, 3
+ABI_VERSION = 5
 
 
 class OeqError(RuntimeError):

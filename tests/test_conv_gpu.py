@@ -625,7 +625,10 @@ KNOBS = ["conv_pipe_f=0,conv_pipe_b=1", "conv_pipe_f=1,conv_pipe_b=2", "conv_pip
          "conv_q=2,conv_qaf=16,conv_qab=200,conv_qpin=0", "tp_mask=1",
          # edge segments cut into chunks of 2 / 3 edges (every node of these graphs has extra walk positions),
          # and never
-         "conv_hub=2", "conv_hub=3,conv_xcd=1,conv_hops=0", "conv_hub=0"]
+         "conv_hub=2", "conv_hub=3,conv_xcd=1,conv_hops=0", "conv_hub=0",
+         # sender gradients by a second walk over the senders' edges (forward kernel of the adjoint problem), whole
+         # segments and chunks of 2; and never
+         "conv_dxs=1", "conv_dxs=1,conv_hub=2,conv_hops=1", "conv_dxs=0"]
 
 
 @pytest.mark.parametrize("knobs", KNOBS)

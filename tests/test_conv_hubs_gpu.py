@@ -73,6 +73,9 @@ HUBS = [
     ("uvw-hub4000", lambda: _uvw(False), 5000, 4000, 300, 3000),        # the channel-mixing walk
     ("uvw-shared-hub4000", lambda: _uvw(True), 5000, 4000, 300, 3000),
     ("e3tools-hub700", lambda: P.e3tools_problems()[0], 900, 700, 0, 300),
+    # last layer of a network (long X rows, short output rows): the sender gradients come from the sender-side walk,
+    # whose long segments are cut into chunks like the receiver side's
+    ("last-layer-hub3000", lambda: P.nequix_problems()[2], 4000, 3000, 300, 3000),
 ]
 
 
