@@ -186,3 +186,30 @@ def test_matrix_core_kernel_plan_covers_every_sub_path_once():
                 assert sum(1 for g in mine if g[2]) == 1 and mine[0][2]
             for _, sub, _ in groups:
                 assert sum(M._slice_regs(vp, which) for vp in sub) <= M.SLICE_REGS[which]
+
+
+def test_adjoint_problem_gives_the_first_operand_gradient():
+    """lower.adjoint: g . F(x, y, w) == x . F_adjoint(g, y, w) for every x and g, i.e. the adjoint problem's forward map
+    applied to the output gradient is the gradient with respect to the first operand (evaluated from the lowered
+    non-zeros, one row; folded mixed-multiplicity rows included)."""
+    import numpy as np
+    from openequivariance_amd.codegen.lower import adjoint, lower
+    from openequivariance_amd.core import problems as P
+
+    def forward(lw, x, y, w):
+        z = np.zeros(lw.L3)
+        for p in lw.paths:
+            b1, b2, bo = lw.in1[p.i1], lw.in2[p.i2], lw.out[p.io]
+            for u in range(b1.mul):
+                for (i, j, k, c) in p.nnz:
+                    z[bo.off + u * bo.d + k] += c * x[b1.off + u * b1.d + i] * y[b2.off + j] * w[p.woff + u]
+        return z
+
+    rng = np.random.default_rng(0)
+    for problem in (P.nequix_problems()[2], P.config2_nequip_uvu(), P.seven_net_problems()[0]):
+        low = lower(problem)
+        adj = adjoint(low)
+        assert (adj.L1, adj.L3, adj.WN, adj.L2) == (low.L3, low.L1, low.WN, low.L2)
+        x, y, w, g = (rng.normal(size=n) for n in (low.L1, low.L2, low.WN, low.L3))
+        lhs, rhs = g @ forward(low, x, y, w), x @ forward(adj, g, y, w)
+        assert abs(lhs - rhs) <= 1e-12 * max(1.0, abs(lhs))
