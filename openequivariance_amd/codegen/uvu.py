@@ -916,7 +916,10 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
     @staticmethod
     def _attrs(block: int, waves_per_eu: int) -> str:
         a = f"__launch_bounds__({block})"
-        if waves_per_eu > 0:
+        if waves_per_eu >= 10:
+            # two digits: the register budget of the first, at most as many waves as the second
+            a += f" __attribute__((amdgpu_waves_per_eu({waves_per_eu // 10}, {waves_per_eu % 10})))"
+        elif waves_per_eu > 0:
             # exactly that many waves per SIMD: the register budget of that occupancy, and no more waves than that
             a += f" __attribute__((amdgpu_waves_per_eu({waves_per_eu}, {waves_per_eu})))"
         elif waves_per_eu < 0:
@@ -2187,7 +2190,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
 
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
     t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
-                    conv_wf=2, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
+                    conv_wf=23, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=0, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
                     dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fw=0, conv_pf=0,
@@ -2274,8 +2277,10 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     # and the limit of two waves a loss: they get that budget as a minimum and run as many waves as their
     # registers allow (config-5 graph, step: SevenNet first layer 3.96 -> 2.58 ms, last layers 3.85 -> 3.49,
     # NequiX first layer 2.58 -> 2.30, MACE-medium 5.99 -> 5.68, NequIP water 2.18 -> 2.05). Larger kernels keep
-    # exactly two: without the limit the scheduler aims for an occupancy they cannot use (SevenNet main layer
-    # 15.3 -> 21.2 ms).
+    # the budget of two: without a limit the scheduler aims for an occupancy they cannot use (SevenNet main layer
+    # 15.3 -> 21.2 ms); the forward kernel may run a third wave where its registers allow (conv_wf=23: NequiX /
+    # SevenNet main layers' forward -10 % / -16 %, nothing else moves), the backward kernel not (SevenNet main
+    # layer +30 %).
     per_lane = (1 if low.elem_size == 4 else 2) * (max(sum(low.out[io].d for io in seg) for seg in em.segments)
                                                    + sum(low.in1[b].d for b in em.used_in1) + em.n_wslots)
     if walk and per_lane <= 48:
