@@ -156,6 +156,12 @@ typedef struct {
                                    core/LoopUnrollConv.py:142-185). */
 } oeq_problem_dims;
 
+/* `code` is a code object as oeq_jit_compile returns it, or a pack of several (the kernels of a large set
+ * compiled side by side, in different processes; every kernel in exactly one of them): the 8 bytes "OEQPACK1",
+ * a uint64 count, that many uint64 byte sizes, then the code objects in that order, each starting at the next
+ * multiple of 64 bytes from the start of the pack (little endian). Kernel names are looked up in all of them.
+ * No counterpart in the reference, whose kernel sets are one NVRTC / hiprtc program each
+ * (extension/backend/backend_hip.hpp:217-288). */
 int oeq_kernels_create(const void* code, size_t code_size,
                        const oeq_problem_dims* dims,
                        const oeq_kernel_desc* descs, int n_descs,

@@ -55,8 +55,17 @@ struct RoleInfo {
 };
 
 struct DeviceSlot {
-    hipModule_t module = nullptr;
+    std::vector<hipModule_t> modules;  // one per code object of the set, empty until first use on the device
     std::vector<hipFunction_t> fn[OEQ_ROLE_COUNT];
+};
+
+// A kernel set's code is one code object or a pack of several (the kernels of a large set compiled side by
+// side, every kernel in exactly one of them): the 8 bytes "OEQPACK1", a uint64 count, that many uint64 byte
+// sizes, then the code objects in that order, each starting on the next multiple of 64 bytes from the start
+// of the pack.
+constexpr char kPackMagic[8] = {'O', 'E', 'Q', 'P', 'A', 'C', 'K', '1'};
+struct CodePart {
+    size_t offset, size;
 };
 
 struct TimedLaunch {
@@ -74,6 +83,7 @@ constexpr int64_t OEQ_LONG_LIST = 126;
 
 struct oeq_kernels {
     std::vector<char> code;
+    std::vector<CodePart> parts;  // the code objects within `code`
     oeq_problem_dims dims{};
     RoleInfo roles[OEQ_ROLE_COUNT];
     std::mutex mu;
@@ -91,23 +101,37 @@ struct oeq_kernels {
         if (dev < 0 || dev >= kMaxDevices) return fail(OEQ_ERR_INVALID, "device index %d out of range", dev);
         std::lock_guard<std::mutex> lock(mu);
         DeviceSlot& s = slots[dev];
-        if (!s.module) {
-            HIP_TRY(hipModuleLoadData(&s.module, code.data()));
+        if (s.modules.empty()) {
+            auto unload = [&s]() {
+                for (hipModule_t m : s.modules) (void)hipModuleUnload(m);
+                s.modules.clear();
+            };
+            for (const CodePart& part : parts) {
+                hipModule_t m = nullptr;
+                hipError_t e = hipModuleLoadData(&m, code.data() + part.offset);
+                if (e != hipSuccess) {
+                    unload();
+                    return fail(OEQ_ERR_HIP, "hipModuleLoadData failed: %s", hipGetErrorString(e));
+                }
+                s.modules.push_back(m);
+            }
             for (int r = 0; r < OEQ_ROLE_COUNT; ++r) {
                 if (!roles[r].present) continue;
                 s.fn[r].clear();
                 for (const std::string& name : roles[r].names) {
                     hipFunction_t f = nullptr;
-                    hipError_t e = hipModuleGetFunction(&f, s.module, name.c_str());
+                    hipError_t e = hipErrorNotFound;
+                    for (size_t m = 0; m < s.modules.size() && e != hipSuccess; ++m)
+                        e = hipModuleGetFunction(&f, s.modules[m], name.c_str());
                     if (e != hipSuccess) {
-                        (void)hipModuleUnload(s.module);
-                        s.module = nullptr;
+                        unload();
                         return fail(OEQ_ERR_HIP, "kernel '%s' not found in code object: %s", name.c_str(),
                                     hipGetErrorString(e));
                     }
                     s.fn[r].push_back(f);
                 }
             }
+            (void)hipGetLastError();  // lookups that missed in the first code objects of a pack are no error
         }
         *out = &s.fn[role];
         return OEQ_OK;
@@ -134,7 +158,7 @@ struct oeq_kernels {
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return false;
         std::lock_guard<std::mutex> lock(mu);
-        return slots[dev].module != nullptr;
+        return !slots[dev].modules.empty();
     }
 
     int launch(int role, int64_t units, void** args, void* stream) {
@@ -238,7 +262,7 @@ int static_scratch(void** out) {
 extern "C" {
 
 const char* oeq_last_error(void) { return g_error.c_str(); }
-int oeq_abi_version(void) { return 5; }
+int oeq_abi_version(void) { return 6; }
 
 int oeq_get_device_props(int device, oeq_device_props* out) {
     if (!out) return fail(OEQ_ERR_INVALID, "oeq_get_device_props: out is NULL");
@@ -318,6 +342,26 @@ int oeq_kernels_create(const void* code, size_t code_size, const oeq_problem_dim
     oeq_kernels* k = new (std::nothrow) oeq_kernels();
     if (!k) return fail(OEQ_ERR_NOMEM, "oeq_kernels_create: out of memory");
     k->code.assign((const char*)code, (const char*)code + code_size);
+    if (code_size >= 16 && !memcmp(code, kPackMagic, 8)) {
+        uint64_t count = 0;
+        memcpy(&count, (const char*)code + 8, 8);
+        bool ok = count >= 1 && count <= (code_size - 16) / 8;
+        size_t at = ok ? 16 + 8 * (size_t)count : 0;
+        for (uint64_t i = 0; ok && i < count; ++i) {
+            uint64_t size = 0;
+            memcpy(&size, (const char*)code + 16 + 8 * i, 8);
+            at = align_up(at, 64);
+            ok = size > 0 && at <= code_size && size <= code_size - at;
+            if (ok) k->parts.push_back({at, (size_t)size});
+            at += (size_t)size;
+        }
+        if (!ok) {
+            delete k;
+            return fail(OEQ_ERR_INVALID, "oeq_kernels_create: malformed code pack");
+        }
+    } else {
+        k->parts.push_back({0, code_size});
+    }
     k->dims = *dims;
     for (int i = 0; i < n_descs; ++i) {
         const oeq_kernel_desc& d = descs[i];
@@ -345,7 +389,7 @@ void oeq_kernels_destroy(oeq_kernels* k) {
         (void)hipEventDestroy(t.stop);
     }
     for (auto& s : k->slots)
-        if (s.module) (void)hipModuleUnload(s.module);
+        for (hipModule_t m : s.modules) (void)hipModuleUnload(m);
     delete k;
 }
 

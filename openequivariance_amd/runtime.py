@@ -57,7 +57,7 @@ ROLE_CONV_BACKWARD_DX = 19
 
 CONV_ATOMIC, CONV_SORTED, CONV_GROUPED = 0, 1, 2
 DX_TERMS, DX_ATOMIC, DX_ARRIVAL, DX_SENDER_WALK = 0, 1, 2, 3
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class OeqError(RuntimeError):
@@ -249,14 +249,7 @@ def source_hash(source: str, arch: str = DEFAULT_ARCH, options: Optional[Sequenc
     return h.hexdigest()[:24]
 
 
-def compile_source(source: str, arch: str = DEFAULT_ARCH, options: Optional[Sequence[str]] = None,
-                   use_disk_cache: bool = True) -> bytes:
-    """HIP source -> code object bytes (hiprtc; needs no GPU)."""
-    opts = list(options if options is not None else HIPRTC_OPTIONS)
-    key = source_hash(source, arch, opts)
-    path = cache_dir() / f"{key}.hsaco"
-    if use_disk_cache and path.exists():
-        return path.read_bytes()
+def _compile_one(source: str, arch: str, opts: Sequence[str]) -> bytes:
     lib = load_library()
     c_opts = (ctypes.c_char_p * len(opts))(*[o.encode() for o in opts])
     code = _P()
@@ -264,9 +257,129 @@ def compile_source(source: str, arch: str = DEFAULT_ARCH, options: Optional[Sequ
     rc = lib.oeq_jit_compile(source.encode(), arch.encode(), c_opts, len(opts), ctypes.byref(code), ctypes.byref(size))
     _check(rc, "oeq_jit_compile")
     try:
-        blob = ctypes.string_at(code.value, size.value)
+        return ctypes.string_at(code.value, size.value)
     finally:
         lib.oeq_free(code)
+
+
+# Large kernel sets are compiled side by side. hiprtc compiles one program at a time per process (eight threads
+# take as long as one: 94 s against 98 s for the 327 kernels of a 128-channel, l <= 3 shared-weight 'uvw' problem),
+# so the kernels are dealt out to that many child processes, each of which compiles the set's shared declarations
+# and device functions with its share of the kernels (the same problem on 8 cores: 16 s). The code objects travel
+# as one pack, which oeq_kernels_create takes apart (layout: see pack_code).
+PACK_MAGIC = b"OEQPACK1"
+PARALLEL_MIN_BYTES = 256 * 1024  # kernel text below which a set is compiled in this process (a few seconds)
+_WORKER_PATH = _PKG_DIR / "_compile_worker.py"
+
+
+def compile_jobs() -> int:
+    """Child processes a large kernel set is compiled in (``OEQ_AMD_COMPILE_JOBS``; 1 = never split)."""
+    env = os.environ.get("OEQ_AMD_COMPILE_JOBS")
+    if env:
+        return max(1, int(env))
+    return max(1, min(16, os.cpu_count() or 1))
+
+
+def split_kernels(source: str) -> Tuple[str, List[str]]:
+    """(everything but the kernels, [kernel definitions]) of a generated module. A kernel definition runs from a
+    line that starts with ``extern "C" __global__`` to the next line that is a lone closing brace (the emitters
+    indent everything inside a definition); one inside a ``namespace x {`` ... ``}  // namespace x`` pair of such
+    lines is returned wrapped in that namespace, whose other members stay where they are."""
+    common, kernels, cur, space = [], [], None, None
+    for ln in source.split("\n"):
+        if cur is not None:
+            cur.append(ln)
+            if ln == "}":
+                text = "\n".join(cur)
+                kernels.append(f"namespace {space} {{\n{text}\n}}" if space else text)
+                cur = None
+            continue
+        if ln.startswith('extern "C" __global__'):
+            cur = [ln]
+            continue
+        if ln.startswith("namespace ") and ln.rstrip().endswith("{"):
+            space = ln[len("namespace "):].rstrip()[:-1].strip()
+        elif space and ln.startswith("}") and f"namespace {space}" in ln:
+            space = None
+        common.append(ln)
+    if cur is not None:  # not laid out like a generated module: nothing to split
+        return source, []
+    return "\n".join(common), kernels
+
+
+def pack_code(blobs: Sequence[bytes]) -> bytes:
+    """Several code objects as one: ``PACK_MAGIC``, a uint64 count, that many uint64 sizes, then the objects in
+    order, each from the next multiple of 64 bytes (little endian; what oeq_kernels_create accepts in place of
+    a single code object)."""
+    import struct
+    out = bytearray(PACK_MAGIC + struct.pack(f"<Q{len(blobs)}Q", len(blobs), *[len(b) for b in blobs]))
+    for b in blobs:
+        out += b"\0" * (-len(out) % 64)
+        out += b
+    return bytes(out)
+
+
+def unpack_code(blob: bytes) -> List[bytes]:
+    """The code objects of what compile_source returned (one, unless it is a pack)."""
+    import struct
+    if not blob.startswith(PACK_MAGIC):
+        return [blob]
+    (count,) = struct.unpack_from("<Q", blob, 8)
+    sizes = struct.unpack_from(f"<{count}Q", blob, 16)
+    out, at = [], 16 + 8 * count
+    for n in sizes:
+        at += -at % 64
+        out.append(blob[at:at + n])
+        at += n
+    return out
+
+
+def _compile_parallel(source: str, arch: str, opts: Sequence[str], jobs: int) -> Optional[bytes]:
+    """The pack of a large module's code objects, or None when the module is small, has a single kernel, or a
+    child process could not be run or failed (the caller then compiles in this process, which also reports a
+    compile error in full)."""
+    import sys
+    import tempfile
+    common, kernels = split_kernels(source)
+    if len(kernels) < 2 or sum(map(len, kernels)) < PARALLEL_MIN_BYTES:
+        return None
+    # longest first into the emptiest bin: compile time goes with the amount of kernel text
+    bins: List[List[int]] = [[] for _ in range(min(jobs, len(kernels)))]
+    load = [0] * len(bins)
+    for i in sorted(range(len(kernels)), key=lambda i: -len(kernels[i])):
+        b = load.index(min(load))
+        bins[b].append(i)
+        load[b] += len(kernels[i])
+    load_library()  # built before the children look for it
+    try:
+        with tempfile.TemporaryDirectory(prefix="oeq_compile_") as tmp:
+            procs = []
+            for n, mine in enumerate(b for b in bins if b):
+                src, out = Path(tmp) / f"part{n}.hip", Path(tmp) / f"part{n}.hsaco"
+                src.write_text(common + "\n" + "\n".join(kernels[i] for i in sorted(mine)) + "\n")
+                procs.append((out, subprocess.Popen(
+                    [sys.executable, str(_WORKER_PATH), str(lib_path()), arch, str(src), str(out), *opts],
+                    stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)))
+            ok = [proc.wait() == 0 for _out, proc in procs]  # (every child is waited for)
+            if not all(ok):
+                return None
+            return pack_code([out.read_bytes() for out, _proc in procs])
+    except OSError:
+        return None
+
+
+def compile_source(source: str, arch: str = DEFAULT_ARCH, options: Optional[Sequence[str]] = None,
+                   use_disk_cache: bool = True) -> bytes:
+    """HIP source -> code object bytes, or a pack of them (hiprtc; needs no GPU)."""
+    opts = list(options if options is not None else HIPRTC_OPTIONS)
+    key = source_hash(source, arch, opts)
+    path = cache_dir() / f"{key}.hsaco"
+    if use_disk_cache and path.exists():
+        return path.read_bytes()
+    jobs = compile_jobs()
+    blob = _compile_parallel(source, arch, opts, jobs) if jobs > 1 else None
+    if blob is None:
+        blob = _compile_one(source, arch, opts)
     if use_disk_cache:
         tmp = path.with_suffix(f".tmp{os.getpid()}")
         tmp.write_bytes(blob)

@@ -758,3 +758,33 @@ def test_edge_list_index_is_reused_and_invalidated():
         finally:
             ks.conv_index_build = real
             ops.clear_index_cache()
+
+
+def test_kernel_set_compiled_side_by_side_runs(monkeypatch, tmp_path):
+    """A kernel set whose kernels were compiled in shares by child processes reaches the library as a pack of
+    code objects: it loads, every kernel is found (one of them sits inside a namespace), and it computes the
+    bits of the set compiled whole."""
+    from openequivariance_amd import runtime as rt
+    problem = P.nequix_problems()[2]
+    coords, rows, cols = _graph(60, 8, seed=11)
+    g = CoordGraph(coords, rows, cols)
+    X, Y, W, G = _buffers(problem, 60, g.nnz, seed=5)
+
+    def run():
+        conv = oeq.TensorProductConv(problem, deterministic=True)
+        tX, tY, tW = (torch.tensor(a, device="cuda", requires_grad=True) for a in (X, Y[g.order], W[g.order]))
+        z = conv(tX, tY, tW, torch.tensor(g.rows, device="cuda"), torch.tensor(g.cols, device="cuda"),
+                 torch.tensor(g.transpose_perm, device="cuda"))
+        z.backward(torch.tensor(G, device="cuda"))
+        return [t.detach().cpu().numpy() for t in (z, tX.grad, tY.grad, tW.grad)]
+
+    whole = run()
+    monkeypatch.setattr(rt, "PARALLEL_MIN_BYTES", 0)
+    monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "4")
+    monkeypatch.setenv("OEQ_AMD_CACHE_DIR", str(tmp_path))
+    monkeypatch.setenv("OEQ_AMD_TUNE", "conv_hub=255")  # (a kernel set of its own: nothing to find in any cache)
+    shares = run()
+    packs = [f for f in tmp_path.iterdir() if f.read_bytes().startswith(rt.PACK_MAGIC)]
+    assert len(packs) == 1 and len(rt.unpack_code(packs[0].read_bytes())) == 4
+    for a, b in zip(whole, shares):
+        assert np.array_equal(a, b)

@@ -70,7 +70,7 @@ def test_generated_tp_sources_compile_for_gfx950(make):
     from openequivariance_amd._torch.tensor_product import build_tp_module
     src, dims, descs = build_tp_module(make())
     blob = rt.compile_source(src)
-    assert blob[:4] == b"\x7fELF"
+    assert all(part[:4] == b"\x7fELF" for part in rt.unpack_code(blob))
     names = {d[1] for d in descs}
     assert {"forward", "backward"} <= names
     for n in names:
@@ -99,6 +99,73 @@ def test_float_atomics_conv_kernels_compile(monkeypatch):
     src, dims, descs = build_conv_module(P.config5_mace_conv(), False)
     assert dims["deterministic"] == rt.CONV_ATOMIC and "fixup_backward" not in {d[1] for d in descs}
     assert "oeq_atomic_add" in src and len(rt.compile_source(src)) > 0
+
+
+def _elf_functions(blob: bytes):
+    """Names of the function symbols an ELF64 code object defines."""
+    import struct
+    shoff, = struct.unpack_from("<Q", blob, 0x28)
+    shentsize, shnum = struct.unpack_from("<HH", blob, 0x3A)
+    sections = [struct.unpack_from("<IIQQQQIIQQ", blob, shoff + i * shentsize) for i in range(shnum)]
+    out = set()
+    for _name, kind, _flags, _addr, off, size, link, _info, _align, entsize in sections:
+        if kind != 2:  # SHT_SYMTAB
+            continue
+        str_off = sections[link][4]
+        for at in range(off, off + size, entsize):
+            st_name, st_info, _other, st_shndx = struct.unpack_from("<IBBH", blob, at)
+            if st_info & 0xF == 2 and st_shndx != 0:  # STT_FUNC, defined
+                end = blob.index(b"\0", str_off + st_name)
+                out.add(blob[str_off + st_name:end].decode())
+    return out
+
+
+def test_large_kernel_sets_compile_side_by_side(monkeypatch, tmp_path):
+    """A module above the size limit is split at its kernel definitions, the shares are compiled by child
+    processes and come back as one pack that the library accepts; a kernel inside a namespace keeps it."""
+    from openequivariance_amd._torch.tensor_product_conv import build_conv_module
+    # (last layer: its sender gradients come from a kernel emitted inside a namespace of its own)
+    src, dims, descs = build_conv_module(P.nequix_problems()[2], True)
+    assert "namespace oeq_dx {" in src
+    common, kernels = rt.split_kernels(src)
+    assert "__global__" not in common and len(kernels) == src.count('extern "C" __global__')
+    inside = [k for k in kernels if k.startswith("namespace oeq_dx {")]
+    assert len(inside) == 1 and "void backward_dx(" in inside[0]
+    names = {d[1] for d in descs}
+    assert all(sum(f" {n}(" in k.split("\n")[1 if k.startswith("namespace") else 0] for k in kernels) == 1
+               for n in names)
+    monkeypatch.setattr(rt, "PARALLEL_MIN_BYTES", 0)
+    monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "3")
+    monkeypatch.setenv("OEQ_AMD_CACHE_DIR", str(tmp_path))
+    blob = rt.compile_source(src)
+    parts = rt.unpack_code(blob)
+    assert blob.startswith(rt.PACK_MAGIC) and len(parts) == 3 and all(p[:4] == b"\x7fELF" for p in parts)
+    assert rt.pack_code(parts) == blob and (tmp_path / f"{rt.source_hash(src)}.hsaco").read_bytes() == blob
+    defined = [_elf_functions(p) for p in parts]
+    for n in names:  # every kernel in exactly one code object
+        assert sum(n in d for d in defined) == 1, n
+    rt.KernelSet(blob, dims, descs)
+    # one job, or a failing child: compiled in this process
+    monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "1")
+    assert rt.compile_source(src, use_disk_cache=False)[:4] == b"\x7fELF"
+    monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "3")
+    monkeypatch.setattr(rt, "_WORKER_PATH", tmp_path / "missing.py")
+    assert rt.compile_source(src, use_disk_cache=False)[:4] == b"\x7fELF"
+
+
+def test_malformed_code_packs_are_rejected():
+    import struct
+    dims = dict(L1_dim=4, L2_dim=4, L3_dim=4, weight_numel=4, elem_size=4)
+    desc = [(rt.ROLE_TP_FORWARD, "forward", 64, 1, 0)]
+    elf = b"\x7fELF" + b"x" * 60
+    rt.KernelSet(rt.pack_code([elf, elf]), dims, desc)
+    for bad in (rt.PACK_MAGIC + struct.pack("<Q", 0),                          # no code object
+                rt.PACK_MAGIC + struct.pack("<QQ", 2, 64) + b"\0" * 200,        # count beyond the sizes present
+                rt.PACK_MAGIC + struct.pack("<QQ", 1, 1 << 40) + b"\0" * 200,   # size beyond the pack
+                rt.PACK_MAGIC + struct.pack("<QQ", 1, 0) + b"\0" * 200,         # empty code object
+                rt.pack_code([elf, elf])[:-1]):                                 # truncated
+        with pytest.raises(rt.OeqError, match="malformed code pack"):
+            rt.KernelSet(bad, dims, desc)
 
 
 def test_lowering_lane_mapping():
