@@ -76,7 +76,7 @@ class UvuEmitter:
         self.seg_waves = 1  # conv forward: waves per node that share its output segments between them
         self.bwd_groups: Optional[List[List[int]]] = None  # conv backward: output blocks owned by each wave
         self.group_budget = 0  # gradient words per wave when a node is shared between waves (0: default)
-        self.fit_words = 280  # estimate of backward_words up to which one wave keeps a node's whole gradient
+        self.fit_words = 300  # estimate of backward_words up to which one wave keeps a node's whole gradient
         # plain stores of [64 x d] channel blocks go through the s_tr tile as well: bit 0 = forward outputs,
         # bit 1 = backward dX (kernels that use it declare the tile)
         self.tr_stores = 0
@@ -1802,9 +1802,11 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         with them the paths) between several waves of the node so that each keeps its share resident.
         Returns the blocks per wave, or None when that is not possible or not needed."""
         low = self.low
-        # Up to an estimate of 280 words the one-wave kernel compiles to at most 255 registers without scratch
-        # memory (21 mixed-multiplicity problems compiled, estimates 207..275), and it beats the shared node there
-        # (config-5 graph, backward: NequiX main layer 7.52 -> 5.89 ms, five more such problems -14 %).
+        # Up to an estimate of about 285 words the one-wave kernel compiles to at most 256 registers with no or a
+        # few words of scratch memory (35 problems compiled: mixed multiplicities 207..285 none, uniform ones 28 B at
+        # 277), and it beats the shared node there (config-5 graph, backward: NequiX main layer 7.52 -> 5.89 ms; 64 /
+        # 128 channels with harmonics up to l = 4 -15 % .. -30 %; an estimate of 285 -19 %). At 318 (80 B of scratch)
+        # the two are level, from 330 on the one-wave kernel loses by far (SevenNet main layer 25.6 against 10.1 ms).
         fits = self.g_resident and self.backward_words(True) <= self.fit_words
         if fits or low.shared_weights or not self.can_preload or self.R != 1:
             return None
@@ -2197,7 +2199,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_wf=23, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=0, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
-                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fit=280, conv_fw=0, conv_pf=0,
+                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fit=300, conv_fw=0, conv_pf=0,
                     conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0, tp_forms=1,
                     conv_hub=256, conv_dxs=-1))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
