@@ -2179,7 +2179,8 @@ def tp_module(low: Lowered, compute_units: int = 256):
     return s.text(), dims, descs
 
 
-def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kahan: bool = False):
+def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kahan: bool = False,
+                override: Optional[Dict[str, int]] = None):
     """Source + launch descriptors for the fused convolution (forward, backward).
 
     ``deterministic``: the caller passes receiver-sorted edges and the sender-major permutation; the
@@ -2191,7 +2192,10 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
 
     ``kahan`` (deterministic mode only): compensated summation where rows are summed over edges, i.e.
     the receiver's output in `forward` and the sender's gradient in `fixup_backward`, as in the
-    reference (templates/loop_unroll_conv_det.cuh:70-94, 135-160, 227-271)."""
+    reference (templates/loop_unroll_conv_det.cuh:70-94, 135-160, 227-271).
+
+    ``override``: knob values that take precedence over ``OEQ_AMD_TUNE`` (the function's own second attempt,
+    see the end)."""
     from .. import runtime as rt
 
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
@@ -2203,6 +2207,11 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0, tp_forms=1,
                     conv_hub=256, conv_dxs=-1))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
+    # knobs somebody set: the rules below leave those alone
+    user_tune = os.environ.get("OEQ_AMD_TUNE", "")
+    if override:
+        t.update(override)
+        user_tune = ",".join([user_tune, *override])
     if kahan:  # the compensation terms double the accumulator registers: walk the outputs in more passes
         t["conv_acc"] = min(t["conv_acc"], 48)
     if deterministic:
@@ -2215,7 +2224,6 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     # operand set) fits the 512 registers a lane has at one wave per SIMD, that beats walking the edges once
     # per output segment / sharing the node between waves (MACE shape, fp64: forward 18.4 -> 12.5 ms,
     # backward 42.1 -> 26.4 ms). The same plan loses for every fp32 problem tried.
-    user_tune = os.environ.get("OEQ_AMD_TUNE", "")
     wide64 = low.elem_size == 8 and em.R == 1 and not kahan and walk and not low.shared_weights
     if wide64 and "conv_acc" not in user_tune and "conv_wf" not in user_tune:
         x_all = sum(low.in1[b].d for b in em.used_in1)
@@ -2265,6 +2273,13 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     if walk and len(em.segments) > 1 and t["conv_segw"] and em.stage is None and em.R == 1:
         em.seg_waves = max(1, min(len(em.segments), t["conv_segw"], max(1, 8 // em.NCH)))
         t["conv_gf"] = max(1, min(t["conv_gf"], 8 // (em.NCH * em.seg_waves)))
+    if walk and len(em.segments) > 1 and "conv_gf" not in user_tune:
+        # Several output segments (a wave walks the node's edges once per segment it owns): one node per block.
+        # Blocks of several nodes hold all their wave slots until the slowest wave is through; over 118 problems
+        # on the config-5 graph one node per block is never slower (+0.3 % at worst) and up to 30 % faster
+        # (forward: SevenNet main layer 4.36 -> 3.09 ms, NequiX main layer 2.51 -> 2.21, NequIP benzene
+        # 8.33 -> 7.98).
+        t["conv_gf"] = 1
     em.tr_stores = t["conv_trs"]
     # output gradients that do not fit the register budget are loaded per path: fence the paths then
     em.sched_fence = (not em.g_resident) if t["conv_sb"] < 0 else bool(t["conv_sb"])
@@ -2293,6 +2308,11 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         for knob in ("conv_wf", "conv_wb"):
             if knob not in user_tune:
                 t[knob] = -2
+    elif walk and not low.shared_weights and low.elem_size == 4 and "conv_gb" not in user_tune:
+        # One node per block for the backward kernel as well where a row fits one wave and the kernel is not a
+        # small one (blocks of four nodes keep their wave slots until the slowest is through; same 118 problems,
+        # fp32: -8 % .. +0.3 %, mean -1.7 %; NequiX main layer 6.13 -> 5.77 ms; small kernels: up to +1.4 %)
+        t["conv_gb"] = 1
     G_f = t["conv_gf"]
     G_b = 1 if em.NCH > 1 else t["conv_gb"]
     xcd = max(1, t["conv_xcd"])
@@ -2400,4 +2420,14 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                 shared_weights=int(low.shared_weights), deterministic=mode,
                 wpartial_per_block=G_b if (walk and low.shared_weights) else 0, dx_mode=dx_mode,
                 n_chunks=em.NCH, order_hops=max(0, t["conv_hops"]) if walk else 0, hub_limit=hub_limit)
-    return s.text(), dims, descs
+    src = s.text()
+    if em.seg_waves > 1 and "conv_segw" not in user_tune:
+        # Waves that share a node's output segments: with two operand sets in flight and three or more segments
+        # the compiler has been seen to need more registers for the kernel that selects a wave's segments by
+        # branches than for the one that walks them one after the other (64x{0e,1e,2e,3e} with l <= 3 harmonics:
+        # 256 registers and 280 B of scratch memory per lane against 227 and none; forward 14.5 against 4.0 ms).
+        # The code object says so (compiled here, cached like any other): then one wave owns the node.
+        _lds, scratch = rt.kernel_resources(rt.compile_source(src)).get("forward", (0, 0))
+        if scratch > 64:
+            return conv_module(low, deterministic, compute_units, kahan, dict(override or {}, conv_segw=0))
+    return src, dims, descs

@@ -334,6 +334,33 @@ def unpack_code(blob: bytes) -> List[bytes]:
     return out
 
 
+def kernel_resources(blob: bytes) -> Dict[str, Tuple[int, int]]:
+    """{kernel name: (bytes of LDS, bytes of scratch memory per lane)} of the kernels in what compile_source
+    returned, from the kernel descriptors (the 64-byte objects ``<name>.kd`` of an amdhsa code object, whose
+    first two 32-bit words are group_segment_fixed_size and private_segment_fixed_size). A kernel that the
+    compiler could not fit into its register budget has a non-zero scratch size."""
+    import struct
+    out: Dict[str, Tuple[int, int]] = {}
+    for elf in unpack_code(blob):
+        shoff, = struct.unpack_from("<Q", elf, 0x28)
+        shentsize, shnum = struct.unpack_from("<HH", elf, 0x3A)
+        sections = [struct.unpack_from("<IIQQQQIIQQ", elf, shoff + i * shentsize) for i in range(shnum)]
+        for _name, kind, _flags, _addr, off, size, link, _info, _align, entsize in sections:
+            if kind != 2:  # SHT_SYMTAB
+                continue
+            str_off = sections[link][4]
+            for at in range(off, off + size, entsize):
+                st_name, _st_info, _other, st_shndx, st_value, st_size = struct.unpack_from("<IBBHQQ", elf, at)
+                end = elf.index(b"\0", str_off + st_name)
+                name = elf[str_off + st_name:end].decode()
+                if not name.endswith(".kd") or st_size != 64 or not 0 < st_shndx < shnum:
+                    continue
+                sec = sections[st_shndx]
+                lds, scratch = struct.unpack_from("<II", elf, sec[4] + st_value - sec[3])
+                out[name[:-3]] = (lds, scratch)
+    return out
+
+
 def _compile_parallel(source: str, arch: str, opts: Sequence[str], jobs: int) -> Optional[bytes]:
     """The pack of a large module's code objects, or None when the module is small, has a single kernel, or a
     child process could not be run or failed (the caller then compiles in this process, which also reports a

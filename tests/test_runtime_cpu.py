@@ -153,6 +153,31 @@ def test_large_kernel_sets_compile_side_by_side(monkeypatch, tmp_path):
     assert rt.compile_source(src, use_disk_cache=False)[:4] == b"\x7fELF"
 
 
+def test_forward_kernel_that_spills_gives_way_to_one_wave_per_node():
+    """Waves that share a node's output segments: where the compiler cannot fit that kernel into its registers (the
+    code object's kernel descriptor shows scratch memory), the module is generated again with one wave per node."""
+    from openequivariance_amd._torch.tensor_product_conv import build_conv_module
+    harmonics = "1x0e+1x1e+1x2e+1x3e"
+    problem = P.CTPP("64x0e+64x1e+64x2e+64x3e", harmonics, "0e+1e+2e+3e", "four-irreps-even")
+    os.environ.pop("OEQ_AMD_TUNE", None)
+    src, _dims, descs = build_conv_module(problem, True)
+    forward = next(d for d in descs if d[1] == "forward")
+    assert forward[2] == 64 and forward[3] == 1                     # one wave, one node per block
+    assert rt.kernel_resources(rt.compile_source(src))["forward"][1] == 0
+    # the shared form, forced: three waves per node, and it spills
+    os.environ["OEQ_AMD_TUNE"] = "conv_segw=4"
+    try:
+        src, _dims, descs = build_conv_module(problem, True)
+    finally:
+        os.environ.pop("OEQ_AMD_TUNE", None)
+    forward = next(d for d in descs if d[1] == "forward")
+    assert forward[2] == 192 and rt.kernel_resources(rt.compile_source(src))["forward"][1] > 64
+    # a problem whose shared form fits keeps it (mixed multiplicities, three segments)
+    src, _dims, descs = build_conv_module(P.seven_net_problems()[1], True)
+    forward = next(d for d in descs if d[1] == "forward")
+    assert forward[2] == 192 and forward[3] == 1 and rt.kernel_resources(rt.compile_source(src))["forward"][1] == 0
+
+
 def test_malformed_code_packs_are_rejected():
     import struct
     dims = dict(L1_dim=4, L2_dim=4, L3_dim=4, weight_numel=4, elem_size=4)
