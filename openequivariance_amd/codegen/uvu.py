@@ -76,6 +76,7 @@ class UvuEmitter:
         self.seg_waves = 1  # conv forward: waves per node that share its output segments between them
         self.bwd_groups: Optional[List[List[int]]] = None  # conv backward: output blocks owned by each wave
         self.group_budget = 0  # gradient words per wave when a node is shared between waves (0: default)
+        self.group_count = 0  # that many waves share a node in the backward kernel, whatever their registers (0: by budget)
         self.fit_words = 300  # estimate of backward_words up to which one wave keeps a node's whole gradient
         # plain stores of [64 x d] channel blocks go through the s_tr tile as well: bit 0 = forward outputs,
         # bit 1 = backward dX (kernels that use it declare the tile)
@@ -1800,21 +1801,24 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
     def plan_backward_groups(self, max_waves: int) -> Optional[List[List[int]]]:
         """When a node's output gradient does not fit one wave's registers, share the output blocks (and
         with them the paths) between several waves of the node so that each keeps its share resident.
-        Returns the blocks per wave, or None when that is not possible or not needed."""
+        Returns the blocks per wave, or None when that is not possible or not needed.
+
+        The estimate of ``backward_words`` decides, for the whole gradient and for a wave's share of it alike.
+        Up to about 285 words the one-wave kernel compiles to at most 256 registers with no or a few words of
+        scratch memory (35 problems compiled: mixed multiplicities 207..285 none, uniform ones 28 B at 277) and
+        beats the shared node (config-5 graph, backward: NequiX main layer 7.52 -> 5.89 ms; 64 / 128 channels with
+        harmonics up to l = 4 -15 % .. -30 %; an estimate of 285 -19 %); at 318 (80 B of scratch) the two are
+        level, from 330 on it loses by far (SevenNet main layer 25.6 against 10.1 ms). Of the group counts 1, 2, 3,
+        4, 6 and 8, forced on 24 problems with estimates from 266 to 643, the best was always the smallest of 1, 2
+        and 4 whose share stays under that same limit (shares of 273 and 281 words: two waves, -54 % and -16 %
+        against the four and five that a fixed share of 64 gradient words gave; 311 and more: four waves); three,
+        six and eight waves never won, and five or seven cost up to 2x."""
         low = self.low
-        # Up to an estimate of about 285 words the one-wave kernel compiles to at most 256 registers with no or a
-        # few words of scratch memory (35 problems compiled: mixed multiplicities 207..285 none, uniform ones 28 B at
-        # 277), and it beats the shared node there (config-5 graph, backward: NequiX main layer 7.52 -> 5.89 ms; 64 /
-        # 128 channels with harmonics up to l = 4 -15 % .. -30 %; an estimate of 285 -19 %). At 318 (80 B of scratch)
-        # the two are level, from 330 on the one-wave kernel loses by far (SevenNet main layer 25.6 against 10.1 ms).
-        fits = self.g_resident and self.backward_words(True) <= self.fit_words
-        if fits or low.shared_weights or not self.can_preload or self.R != 1:
+        if low.shared_weights or not self.can_preload or self.R != 1:
             return None
-        # room for the edge operands, dX, dY (and deferred dW) beside the wave's share of the gradient
-        budget = max(1, (self.group_budget or (96 if not self.ragged() else 64)) // self.words)
         sizes = [low.out[io].d for io in self.used_out]
-        n = max(2 if self.g_resident else 1, -(-sum(sizes) // budget))
-        while n <= max_waves:
+
+        def balanced(n: int) -> List[List[int]]:
             target = -(-sum(sizes) // n)
             groups, cur, tot = [], [], 0
             for io, d in zip(self.used_out, sizes):
@@ -1824,6 +1828,29 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
                 cur.append(io)
                 tot += d
             groups.append(cur)
+            return groups
+
+        def share_words(n: int) -> int:
+            """backward_words with a wave's share, 1 / n, of the gradient and of the weights."""
+            x = sum(low.in1[b].d for b in self.used_in1)
+            w = self.n_wslots * (2 if self.ragged() else 1)
+            return self.words * (-(-sum(sizes) // n) + 2 * x + self.l2_pad + -(-w // n) + low.L2) + 40
+
+        if self.group_count:  # forced
+            return balanced(max(1, min(self.group_count, max_waves, len(sizes))))
+        if self.backward_words(True) <= self.fit_words:
+            # one wave: the ordinary kernel where it keeps the gradient in registers by its own rule, else the
+            # shared-node kernel with a single owner (which always does)
+            return None if self.g_resident else [list(self.used_out)]
+        if not self.group_budget:
+            for n in (2, 4, 8):
+                if n <= max_waves and n <= len(sizes) and share_words(n) <= self.fit_words:
+                    return balanced(n)
+        # a fixed share of gradient words per wave (group_budget; or nothing above fitted)
+        budget = max(1, (self.group_budget or (96 if not self.ragged() else 64)) // self.words)
+        n = max(2 if self.g_resident else 1, -(-sum(sizes) // budget))
+        while n <= max_waves:
+            groups = balanced(n)
             if all(sum(low.out[io].d for io in grp) <= budget for grp in groups):
                 return groups
             n += 1
@@ -2203,7 +2230,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_wf=23, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=0, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
-                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_fit=300, conv_fw=0, conv_pf=0,
+                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_ngrp=0, conv_fit=300, conv_fw=0, conv_pf=0,
                     conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0, tp_forms=1,
                     conv_hub=256, conv_dxs=-1))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"
@@ -2323,6 +2350,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     dx_mode = 0
     em.group_budget = t["conv_gbud"]
     em.fit_words = t["conv_fit"]
+    em.group_count = t["conv_ngrp"]
     em.bwd_groups = em.plan_backward_groups(max(1, 8 // em.NCH)) if (walk and t["conv_split"] and gres is None) else None
     if em.bwd_groups:
         G_b = 1

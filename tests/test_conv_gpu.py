@@ -101,6 +101,15 @@ CASES = [
     ("benzene-128", lambda: P.ChannelwiseTPP(
         "128x0o + 128x0e + 128x1o + 128x1e + 128x2o + 128x2e + 128x3o + 128x3e", "0e + 1o + 2e + 3o",
         "128x0o + 128x0e + 128x1o + 128x1e + 128x2o + 128x2e + 128x3o + 128x3e", "benzene-128"), 24, 4),
+    # the backward kernel that shares a node between waves, with a single owner (135 gradient words: more than the
+    # ordinary kernel keeps in registers, few enough for one wave), with two (SevenNet main layer) and with four
+    # (benzene above); and the forward kernel regenerated with one wave per node because its shared form spills
+    ("one-owner", lambda: P.ChannelwiseTPP("64x0e+64x1o+64x2e+64x3o", "0e+1o+2e+3o", "0e+1o+2e+3o+4e", "one-owner"), 30, 5),
+    ("one-owner-128", lambda: P.ChannelwiseTPP("128x0e+128x1o+128x2e+128x3o", "0e+1o+2e+3o", "0e+1o+2e+3o+4e",
+                                               "one-owner-128"), 24, 4),
+    ("sevennet-main", lambda: P.seven_net_problems()[1], 30, 5),
+    ("four-irreps-even", lambda: P.ChannelwiseTPP("64x0e+64x1e+64x2e+64x3e", "1x0e+1x1e+1x2e+1x3e", "0e+1e+2e+3e",
+                                                  "four-irreps-even"), 30, 5),
 ]
 
 
@@ -628,7 +637,9 @@ KNOBS = ["conv_pipe_f=0,conv_pipe_b=1", "conv_pipe_f=1,conv_pipe_b=2", "conv_pip
          "conv_hub=2", "conv_hub=3,conv_xcd=1,conv_hops=0", "conv_hub=0",
          # sender gradients by a second walk over the senders' edges (forward kernel of the adjoint problem), whole
          # segments and chunks of 2; and never
-         "conv_dxs=1", "conv_dxs=1,conv_hub=2,conv_hops=1", "conv_dxs=0"]
+         "conv_dxs=1", "conv_dxs=1,conv_hub=2,conv_hops=1", "conv_dxs=0",
+         # a node's output gradient shared between that many waves in the backward kernel (1: a single owner)
+         "conv_ngrp=1", "conv_ngrp=2,conv_hub=2", "conv_ngrp=3", "conv_ngrp=4,conv_hub=3"]
 
 
 @pytest.mark.parametrize("knobs", KNOBS)
