@@ -2230,7 +2230,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                     conv_wf=23, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=0, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
-                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, conv_gbud=0, conv_ngrp=0, conv_fit=300, conv_fw=0, conv_pf=0,
+                    dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, dd_ngrp=0, conv_gbud=0, conv_ngrp=0, conv_fit=300, conv_fw=0, conv_pf=0,
                     conv_dxm=-1, conv_q=0, conv_hops=2, conv_qpin=1, conv_qaf=48, conv_qab=24, tp_mask=0, tp_forms=1,
                     conv_hub=256, conv_dxs=-1))
     assert deterministic or not kahan, "kahan=True requires deterministic=True"

@@ -670,13 +670,14 @@ class DoubleEmitter(UvuEmitter):
         def need(grp):
             return fixed + self.words * sum(low.out[io].d * (2 if self.merged else 1) + per_path[io] for io in grp)
 
-        if need(self.used_out) <= self.need_limit:
+        forced = getattr(self, "group_count", 0)
+        if need(self.used_out) <= self.need_limit and not forced:
             return None
         # the waves exchange their dX terms through LDS: [waves][chunks][X components][64 lanes]
         lds_per_wave = self.NCH * x * 64 * low.elem_size
-        max_waves = min(max_waves, 60000 // lds_per_wave)
-        n = 2
-        while n <= max_waves:
+        max_waves = min(max_waves, 60000 // lds_per_wave, len(sizes))
+
+        def balanced(n: int) -> List[List[int]]:
             target = -(-sum(sizes) // n)
             groups, cur, tot = [], [], 0
             for io, d in zip(self.used_out, sizes):
@@ -686,6 +687,23 @@ class DoubleEmitter(UvuEmitter):
                 cur.append(io)
                 tot += d
             groups.append(cur)
+            return groups
+
+        if forced:
+            return None if forced == 1 or max_waves < 2 else balanced(min(forced, max_waves))
+        # Two waves while half of what varies with the share (gradient slice, W and C values) fits beside what
+        # every wave holds, else four: with the count forced to 1 .. 4 on 15 problems (config-5 graph) two waves
+        # were best up to an estimate of 231 words for such a share (SevenNet main layer: -16 % against the three
+        # that a fixed limit per wave gave) and four from 343 on (NequIP benzene -14 % against seven); three never
+        # won.
+        if self.need_limit == 200 and max_waves >= 2:
+            share2 = fixed + -(-(need(self.used_out) - fixed) // 2)
+            if share2 <= 250 or max_waves < 4:
+                return balanced(2)
+            return balanced(4)
+        n = 2
+        while n <= max_waves:
+            groups = balanced(n)
             if all(need(grp) <= self.need_limit for grp in groups) or n == max_waves:
                 return groups
             n += 1
@@ -877,6 +895,7 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     em.emit_double_cores(s)
     G = max(1, tune.get("dd_g", 2) // em.NCH) if em.R == 1 else 4
     em.need_limit = tune.get("dd_need", 200)
+    em.group_count = tune.get("dd_ngrp", 0)
     # dd_merge=1: one kernel for both results (W, C and the gathered X, A rows are then read once instead of
     # twice). Measured slower on MI355X for every shape tried (MACE shape 37 - 85 ms against 33 ms for the
     # pair): its accumulators on top of kernel B's state spill whatever the split, so it is off by default.
