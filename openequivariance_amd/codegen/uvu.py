@@ -2300,12 +2300,12 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     if walk and len(em.segments) > 1 and t["conv_segw"] and em.stage is None and em.R == 1:
         em.seg_waves = max(1, min(len(em.segments), t["conv_segw"], max(1, 8 // em.NCH)))
         t["conv_gf"] = max(1, min(t["conv_gf"], 8 // (em.NCH * em.seg_waves)))
-    if walk and len(em.segments) > 1 and "conv_gf" not in user_tune:
+    if walk and (len(em.segments) > 1 or low.elem_size == 8) and "conv_gf" not in user_tune:
         # Several output segments (a wave walks the node's edges once per segment it owns): one node per block.
         # Blocks of several nodes hold all their wave slots until the slowest wave is through; over 118 problems
         # on the config-5 graph one node per block is never slower (+0.3 % at worst) and up to 30 % faster
         # (forward: SevenNet main layer 4.36 -> 3.09 ms, NequiX main layer 2.51 -> 2.21, NequIP benzene
-        # 8.33 -> 7.98).
+        # 8.33 -> 7.98). fp64 kernels likewise, whatever their segments (18 problems: 0 .. -12 %).
         t["conv_gf"] = 1
     em.tr_stores = t["conv_trs"]
     # output gradients that do not fit the register budget are loaded per path: fence the paths then
@@ -2335,10 +2335,11 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         for knob in ("conv_wf", "conv_wb"):
             if knob not in user_tune:
                 t[knob] = -2
-    elif walk and not low.shared_weights and low.elem_size == 4 and "conv_gb" not in user_tune:
+    elif walk and not low.shared_weights and "conv_gb" not in user_tune:
         # One node per block for the backward kernel as well where a row fits one wave and the kernel is not a
         # small one (blocks of four nodes keep their wave slots until the slowest is through; same 118 problems,
-        # fp32: -8 % .. +0.3 %, mean -1.7 %; NequiX main layer 6.13 -> 5.77 ms; small kernels: up to +1.4 %)
+        # fp32: -8 % .. +0.3 %, mean -1.7 %; NequiX main layer 6.13 -> 5.77 ms; small kernels: up to +1.4 %; 18
+        # problems in fp64: -8 % .. +1 %)
         t["conv_gb"] = 1
     G_f = t["conv_gf"]
     G_b = 1 if em.NCH > 1 else t["conv_gb"]
