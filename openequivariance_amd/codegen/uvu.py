@@ -2377,12 +2377,15 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             # fit the edge's row of dx_tmp only when no used block has lanes without a channel
             if dx_mode == em.DX_ARRIVAL and (em.R != 1 or 64 * em.NCH * em._term_slots()[1] > low.L1):
                 dx_mode = em.DX_TERMS
-            # Rows of X much longer than an edge's weights and an output row together (the last layer of a
-            # network: many irreps in, a few scalars out): the per-edge dX terms, written and read back, would be
-            # most of the backward's traffic (2 L1 words per edge). A second walk over the SENDERS' edge segments
-            # that reads W and Y again and gathers the short dZ rows moves WN + L2 + L3 words per edge instead and
-            # sums in the same list order. It is the forward kernel of the adjoint problem (lower.adjoint).
-            auto = low.L1 >= low.WN + low.L2 + low.L3 and not low.shared_weights and t["conv_dxm"] < 0
+            # Rows of X that are long against an edge's weights and an output row (the last layer of a network:
+            # many irreps in, a few scalars out; few paths per input irrep): the per-edge dX terms, written and read
+            # back, are then most of the backward's traffic (2 L1 words per edge). A second walk over the SENDERS'
+            # edge segments that reads W and Y again and gathers the dZ rows moves WN + L2 + L3 words per edge
+            # instead (the gathered rows mostly from the L2) and sums in the same list order. It is the forward
+            # kernel of the adjoint problem (lower.adjoint). Measured over 128 problems on the config-5 graph,
+            # backward op: ratio (WN + L2 + L3) / L1 of 1.1 .. 3.5: -16 % .. -57 %; 4.0 (NequIP aspirin, water):
+            # -5 %; 4.6: -2 % .. -6 %; 5.1: +-3 %; 5.3 and more: slower, +27 % at config 5 (7.6).
+            auto = 9 * low.L1 >= 2 * (low.WN + low.L2 + low.L3) and not low.shared_weights and t["conv_dxm"] < 0
             if (t["conv_dxs"] > 0) or (t["conv_dxs"] < 0 and auto):
                 dx_mode = em.DX_SENDER_WALK
         blk_b = em.emit_conv_backward(s, walk, G_b, t["conv_pipe_b"], t["conv_wb"], gres, xcd_b,
