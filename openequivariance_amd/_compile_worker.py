@@ -2,15 +2,20 @@
 
 Run as a script (``python _compile_worker.py <library> <arch> <source file> <output file> [hiprtc options...]``);
 it loads the C library directly and imports nothing of the package, so that it starts in a fraction of a second.
-hiprtc needs no GPU and this process makes no other HIP call.
+hiprtc needs no GPU and this process makes no other HIP call. ``OEQ_AMD_WORKER_PRELOAD`` lists the HIP runtime and
+hiprtc files of the parent process (those of the torch wheel when torch is loaded there): they are loaded first, so
+that the C library binds to them and this process compiles with the parent's compiler.
 """
 
 import ctypes
+import os
 import sys
 
 
 def main(argv) -> int:
     lib_file, arch, src_file, out_file, *opts = argv
+    for path in filter(None, os.environ.get("OEQ_AMD_WORKER_PRELOAD", "").split(os.pathsep)):
+        ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
     lib = ctypes.CDLL(lib_file)
     lib.oeq_jit_compile.restype = ctypes.c_int
     lib.oeq_jit_compile.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_char_p), ctypes.c_int,

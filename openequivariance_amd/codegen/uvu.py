@@ -253,11 +253,14 @@ class UvuEmitter:
             return None
         st = dict(self.stage)
         npaths = len(self.low.paths)
-        st["XF"] = st["nux"] * 4
+        # Both parts are whole 64-lane instructions (the lanes beyond the data repeat its last unit into padding):
+        # a direct load under a lane condition sits in divergent control flow, where one compiler version has been
+        # seen to merge two of them into one instruction with the LDS base of the first active lane.
+        st["XF"] = st["nqx"] * 256
         st["YOFF"] = st["XF"] + 64 * npaths
         st["nuwy"] = 16 * npaths + self.low.L2 // 4
         st["nqw"] = (st["nuwy"] + 63) // 64
-        st["floats"] = st["XF"] + st["nuwy"] * 4
+        st["floats"] = st["XF"] + st["nqw"] * 256
         return st
 
     def _emit_stage3_offsets(self, s: Src):
@@ -295,14 +298,10 @@ class UvuEmitter:
         s(f"const T* sw = W + eid * {low.WN};")
         s(f"const T* sy = L2_in + eid * {low.L2};")
         for q in range(st["nqx"]):
-            n = min(64, st["nux"] - q * 64)
-            guard = f"if (lane < {n}) " if n < 64 else ""
-            s(f"{guard}__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sx + xoff{q}), "
+            s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(sx + xoff{q}), "
               f"(OEQ_LPTR)(&s_stage{buf}[wave][{q * 256}]), 16, 0, 0);")
         for q in range(st["nqw"]):
-            n = min(64, st["nuwy"] - q * 64)
-            guard = f"if (lane < {n}) " if n < 64 else ""
-            s(f"{guard}__builtin_amdgcn_global_load_lds((const OEQ_GPTR)((wsel{q} ? sw : sy) + woff{q}), "
+            s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)((wsel{q} ? sw : sy) + woff{q}), "
               f"(OEQ_LPTR)(&s_stage{buf}[wave][{st['XF'] + q * 256}]), 16, 0, 0);")
         s.close()
 

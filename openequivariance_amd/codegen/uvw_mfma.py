@@ -405,7 +405,12 @@ class MfmaEmitter:
     def _dma_g(self, s: Src, tile: str, buf: str):
         """The dZ tile of ``tile`` -> s_g[buf] by direct global-to-LDS loads (no registers, nothing to wait for
         here): every wave moves its 4 rows, 64 lanes x 16 bytes per instruction to consecutive LDS addresses.
-        Rows past the batch read the last row (the dX kernels sum nothing over rows, and store nothing for them)."""
+        Rows past the batch read the last row (the dX kernels sum nothing over rows, and store nothing for them).
+        Only whole instructions go that way. The rest of a row (fewer than 64 vectors) is loaded into ``gtail``
+        here and stored by ``_put_g_tail``: a direct load under a lane condition sits in divergent control flow, and
+        there one compiler version (the hiprtc of ROCm 7.2) has been seen to merge it with the next row's direct load
+        into one instruction whose LDS base is taken from the first active lane - a float64 problem with 65 vectors
+        per row then got wrong sender gradients."""
         low = self.low
         VW, rpw = self.vw, RT // WAVES
         nc4 = low.L3 // VW
@@ -415,12 +420,25 @@ class MfmaEmitter:
             s.open("")
             s(f"i64 row = nrow0 + wave * {rpw} + {rr}; if (row >= num_batch) row = num_batch - 1;")
             s(f"const T* src = L3_grad + row * {low.L3};")
-            for j in range((nc4 + 63) // 64):
-                guard = f"if (lane + {64 * j} < {nc4}) " if (j + 1) * 64 > nc4 else ""
-                s(f"{guard}__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(src + {VW} * (lane + {64 * j})), "
+            for j in range(nc4 // 64):
+                s(f"__builtin_amdgcn_global_load_lds((const OEQ_GPTR)(src + {VW} * (lane + {64 * j})), "
                   f"(OEQ_LPTR)&s_g[{buf}][wave * {rpw} + {rr}][{VW * 64 * j}], 16, 0, 0);")
+            if nc4 % 64:
+                jt = nc4 // 64
+                s(f"gtail[{rr}] = (lane + {64 * jt} < {nc4}) ? *(const oeq_vec16*)(src + {VW} * (lane + {64 * jt})) : "
+                  f"oeq_vec16(T(0));")
             s.close()
         s.close()
+
+    def _put_g_tail(self, s: Src, buf: str):
+        """The part of the tile's rows that ``_dma_g`` left in registers -> s_g[buf]."""
+        VW, rpw = self.vw, RT // WAVES
+        nc4 = self.low.L3 // VW
+        if nc4 % 64:
+            jt = nc4 // 64
+            for rr in range(rpw):
+                s(f"if (lane + {64 * jt} < {nc4}) *(oeq_vec16*)&s_g[{buf}][wave * {rpw} + {rr}][{VW} * (lane + {64 * jt})] = "
+                  f"gtail[{rr}];")
 
     def _y_regs(self) -> int:
         return (RT * self.low.L2 + 64 * WAVES - 1) // (64 * WAVES)
@@ -886,7 +904,13 @@ class MfmaEmitter:
             # barrier. Else one copy, staged through registers, three barriers per tile.
             lds_two = 2 * (RT * self.gstride + (1 + WAVES) * RT * low.L2) * low.elem_size + \
                 len(self.lds_w) * 16 * 64 * WAVES * low.elem_size
-            dma = bool(self.tune["uvw_gdma"]) and low.L3 % self.vw == 0 and lds_two <= 80 * 1024 and not self.t1
+            # (rows of whole 64-vector instructions, or rows shorter than one, which then travel through registers
+            # like Y and still gain from the single barrier: DiffDock 0.54 -> 0.49 ms, e3tools 0.60 -> 0.54. Rows
+            # with whole instructions and a rest keep the one-copy form: with the rest in registers config 4's kernels
+            # spill and lose what the direct loads gain, 1.95 against 1.85 ms.)
+            nvec = low.L3 // self.vw
+            dma = (bool(self.tune["uvw_gdma"]) and low.L3 % self.vw == 0 and lds_two <= 80 * 1024 and not self.t1
+                   and (nvec % 64 == 0 or nvec < 64))
             if dma:
                 self.g_at = lambda row, col: f"s_g[gb][{row}][{col}]"
                 self.sy, self.sdy = "s_y[gb]", "s_dy[gb][wave]"
@@ -934,12 +958,15 @@ class MfmaEmitter:
                 s("int gb = 0;")
                 s("i64 prow0 = -1;  // first row of the tile whose dY is still to be written")
                 s(f"T ynext[{ny}];")
+                if (low.L3 // self.vw) % 64:
+                    s(f"oeq_vec16 gtail[{RT // WAVES}];")
                 if rmw_dy:
                     s(f"T dyold[{ny}];")
                 s.open("if ((i64)blockIdx.x < ntiles)")
                 self._dma_g(s, "(i64)blockIdx.x", "0")
                 self._load_flat_rows(s, "ynext", "L2_in", f"(i64)blockIdx.x * {RT}")
                 put_y("0")
+                self._put_g_tail(s, "0")
                 s.close()
                 s.open("for (i64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x, gb ^= 1)")
                 s(f"const i64 row0 = tile * {RT};")
@@ -1007,6 +1034,7 @@ class MfmaEmitter:
                 # Y of the next tile into the other copy (last read two barriers ago)
                 s.open("if (more)")
                 put_y("gb ^ 1")
+                self._put_g_tail(s, "gb ^ 1")
                 s.close()
                 s.close()  # tiles
                 s("__syncthreads();")

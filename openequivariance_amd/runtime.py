@@ -378,6 +378,20 @@ def _compile_parallel(source: str, arch: str, opts: Sequence[str], jobs: int) ->
         bins[b].append(i)
         load[b] += len(kernels[i])
     load_library()  # built before the children look for it
+    # The children must compile with the compiler this process would use: under torch that is the HIP runtime and
+    # hiprtc the torch wheel carries (loaded before this library, which then binds to them), elsewhere the system's.
+    # The two differ in version and in the code they generate, so the children load the same files first.
+    wanted, found = ("libamdhip64", "libhiprtc"), {}
+    try:
+        with open("/proc/self/maps") as maps:
+            for line in maps:
+                path = line.split()[-1]
+                for name in wanted:
+                    if os.path.basename(path).startswith(name + ".so"):
+                        found.setdefault(name, path)
+    except OSError:
+        pass
+    env = dict(os.environ, OEQ_AMD_WORKER_PRELOAD=os.pathsep.join(found[n] for n in wanted if n in found))
     try:
         with tempfile.TemporaryDirectory(prefix="oeq_compile_") as tmp:
             procs = []
@@ -386,7 +400,7 @@ def _compile_parallel(source: str, arch: str, opts: Sequence[str], jobs: int) ->
                 src.write_text(common + "\n" + "\n".join(kernels[i] for i in sorted(mine)) + "\n")
                 procs.append((out, subprocess.Popen(
                     [sys.executable, str(_WORKER_PATH), str(lib_path()), arch, str(src), str(out), *opts],
-                    stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)))
+                    stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, env=env)))
             ok = [proc.wait() == 0 for _out, proc in procs]  # (every child is waited for)
             if not all(ok):
                 return None
