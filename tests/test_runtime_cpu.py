@@ -102,21 +102,23 @@ def test_float_atomics_conv_kernels_compile(monkeypatch):
 
 
 def _elf_functions(blob: bytes):
-    """Names of the function symbols an ELF64 code object defines."""
+    """{name: machine code} of the function symbols an ELF64 code object defines."""
     import struct
     shoff, = struct.unpack_from("<Q", blob, 0x28)
     shentsize, shnum = struct.unpack_from("<HH", blob, 0x3A)
     sections = [struct.unpack_from("<IIQQQQIIQQ", blob, shoff + i * shentsize) for i in range(shnum)]
-    out = set()
+    out = {}
     for _name, kind, _flags, _addr, off, size, link, _info, _align, entsize in sections:
         if kind != 2:  # SHT_SYMTAB
             continue
         str_off = sections[link][4]
         for at in range(off, off + size, entsize):
-            st_name, st_info, _other, st_shndx = struct.unpack_from("<IBBH", blob, at)
-            if st_info & 0xF == 2 and st_shndx != 0:  # STT_FUNC, defined
+            st_name, st_info, _other, st_shndx, st_value, st_size = struct.unpack_from("<IBBHQQ", blob, at)
+            if st_info & 0xF == 2 and 0 < st_shndx < shnum:  # STT_FUNC, defined
                 end = blob.index(b"\0", str_off + st_name)
-                out.add(blob[str_off + st_name:end].decode())
+                sec = sections[st_shndx]
+                start = sec[4] + st_value - sec[3]
+                out[blob[str_off + st_name:end].decode()] = blob[start:start + st_size]
     return out
 
 
@@ -147,7 +149,16 @@ def test_large_kernel_sets_compile_side_by_side(monkeypatch, tmp_path):
     rt.KernelSet(blob, dims, descs)
     # one job, or a failing child: compiled in this process
     monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "1")
-    assert rt.compile_source(src, use_disk_cache=False)[:4] == b"\x7fELF"
+    whole = rt.compile_source(src, use_disk_cache=False)
+    assert whole[:4] == b"\x7fELF"
+    # The children compile with the compiler of this process (under torch: the hiprtc of the torch wheel, not the
+    # system's, which generates other code): kernels that make no reference to other symbols are the same bytes.
+    code = _elf_functions(whole)
+    for part in defined:
+        for name in ("oeq_hub_fill", "oeq_segment_sum"):
+            if name in part:
+                assert part[name] == code[name], name
+        assert all(len(part[name]) == len(code[name]) for name in part if name in names)
     monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "3")
     monkeypatch.setattr(rt, "_WORKER_PATH", tmp_path / "missing.py")
     assert rt.compile_source(src, use_disk_cache=False)[:4] == b"\x7fELF"
