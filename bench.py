@@ -595,12 +595,12 @@ def main():
         # the counters belong to the kernels they were measured on: the file names the hash of that kernel
         # source, and a different source here means the figures are stale (traffic stays null until the
         # profile is taken again)
-        if tr.get("edges") == E and tr.get("source_hash") == rt.source_hash(ks_source):
+        if tr.get("edges") == E and tr.get("source_hash") == rt.cache_key(ks_source):
             roofline["traffic"] = tr["backward_bytes_per_launch"]
             roofline["traffic_per_kernel"] = tr.get("per_kernel")
         else:
             roofline["traffic_note"] = ("profiles/conv_cfg5_traffic.json was measured on another kernel source "
-                                        f"({tr.get('source_hash')} != {rt.source_hash(ks_source)})")
+                                        f"or by another compiler ({tr.get('source_hash')} != {rt.cache_key(ks_source)})")
 
     out = {
         "metric": "fused conv fwd+bwd edges/s at MACE shape (deterministic mode)",

@@ -139,29 +139,51 @@ def test_large_kernel_sets_compile_side_by_side(monkeypatch, tmp_path):
     monkeypatch.setattr(rt, "PARALLEL_MIN_BYTES", 0)
     monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "3")
     monkeypatch.setenv("OEQ_AMD_CACHE_DIR", str(tmp_path))
+    # with the compiler of this process (under torch: the hiprtc of the torch wheel)
+    monkeypatch.setenv("OEQ_AMD_COMPILER", "process")
+    monkeypatch.setattr(rt, "_compiler_choice", None)
+    assert rt.compiler()[0] == "process"
     blob = rt.compile_source(src)
     parts = rt.unpack_code(blob)
     assert blob.startswith(rt.PACK_MAGIC) and len(parts) == 3 and all(p[:4] == b"\x7fELF" for p in parts)
-    assert rt.pack_code(parts) == blob and (tmp_path / f"{rt.source_hash(src)}.hsaco").read_bytes() == blob
+    assert rt.pack_code(parts) == blob and rt.cache_path(src).read_bytes() == blob
+    assert rt.cache_path(src).name == f"{rt.source_hash(src)}-{rt.compiler()[1]}.hsaco"
     defined = [_elf_functions(p) for p in parts]
     for n in names:  # every kernel in exactly one code object
         assert sum(n in d for d in defined) == 1, n
     rt.KernelSet(blob, dims, descs)
-    # one job, or a failing child: compiled in this process
+    # one job: compiled in this process
     monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "1")
     whole = rt.compile_source(src, use_disk_cache=False)
     assert whole[:4] == b"\x7fELF"
-    # The children compile with the compiler of this process (under torch: the hiprtc of the torch wheel, not the
-    # system's, which generates other code): kernels that make no reference to other symbols are the same bytes.
+    # The children loaded this process's HIP libraries first and so compiled with the same hiprtc (the system's
+    # generates other code): kernels that make no reference to other symbols are the same bytes.
     code = _elf_functions(whole)
     for part in defined:
         for name in ("oeq_hub_fill", "oeq_segment_sum"):
             if name in part:
                 assert part[name] == code[name], name
         assert all(len(part[name]) == len(code[name]) for name in part if name in names)
+    # a child that cannot be run: compiled in this process
     monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "3")
+    worker = rt._WORKER_PATH
     monkeypatch.setattr(rt, "_WORKER_PATH", tmp_path / "missing.py")
-    assert rt.compile_source(src, use_disk_cache=False)[:4] == b"\x7fELF"
+    assert rt.compile_source(src, use_disk_cache=False) == whole
+    monkeypatch.setattr(rt, "_WORKER_PATH", worker)
+    # with the system's hiprtc: every compile runs in a child process, the code object is named for that release;
+    # when no child can be run the process goes back to its own compiler
+    monkeypatch.setenv("OEQ_AMD_COMPILER", "system")
+    monkeypatch.setattr(rt, "_compiler_choice", None)
+    if rt.compiler()[0] == "system":
+        other = rt.compile_source(src)
+        assert rt.cache_path(src).read_bytes() == other and rt.compiler()[1] in rt.cache_path(src).name
+        monkeypatch.setenv("OEQ_AMD_COMPILE_JOBS", "1")
+        one = rt.compile_source(src, use_disk_cache=False)
+        assert one[:4] == b"\x7fELF" and {k: len(v) for k, v in _elf_functions(one).items()} == \
+            {k: len(v) for p in rt.unpack_code(other) for k, v in _elf_functions(p).items()}
+        monkeypatch.setattr(rt, "_WORKER_PATH", tmp_path / "missing.py")
+        assert rt.compile_source(src, use_disk_cache=False) == whole and rt.compiler()[0] == "process"
+    monkeypatch.setattr(rt, "_compiler_choice", None)
 
 
 def test_forward_kernel_that_spills_gives_way_to_one_wave_per_node():
