@@ -442,12 +442,13 @@ _compiler_choice: Optional[Tuple[str, str]] = None
 
 
 def compiler() -> Tuple[str, str]:
-    """("process" | "system", version) of the hiprtc that kernels are compiled with. Inside a torch process the C
-    library binds to the hiprtc of the torch wheel; a child process without torch gets the system's. Where the
-    system's is the newer one it is used (every compile then runs in a child process): on the convolution of the
-    MACE shape the kernels of hiprtc 7.2 are 4 % faster than those of 7.0 (forward 4.62 -> 4.25 ms), 0 - 5 % on the
-    other shapes tried. ``OEQ_AMD_COMPILER=process`` / ``system`` decides otherwise. The version is part of a code
-    object's name in the cache."""
+    """("process" | "system", release) of the hiprtc that kernels are compiled with. Inside a torch process the C
+    library binds to the hiprtc of the torch wheel; a child process without torch gets the system's, which a
+    torch-free caller of the C ABI also gets. ``OEQ_AMD_COMPILER=system`` has every kernel set compiled by child
+    processes with that one (so that both kinds of caller run the same code objects); the default is the compiler of
+    this process. The two releases at hand (ROCm 7.0 in the torch wheel, 7.2 in /opt/rocm) generate different code
+    for nearly every kernel and the same speed: config 5's step 18.49 / 18.50 ms, forward 4.61 / 4.61 ms, in one run
+    on one GPU. The release is part of a code object's name in the cache."""
     global _compiler_choice
     if _compiler_choice is None:
         import sys
@@ -455,7 +456,7 @@ def compiler() -> Tuple[str, str]:
         here = _rocm_version(_loaded_rocm_libraries().get("libamdhip64", "libamdhip64.so")) or (0, 0, 0)
         want = os.environ.get("OEQ_AMD_COMPILER", "")
         system = None
-        if want != "process":
+        if want == "system":
             # What a child process would compile with is asked of one, once: the answer is kept beside the code
             # objects, under the identity of the C library and of the system's ROCm directory, so that later
             # processes (one under a profiler, say) start no child for it.
@@ -481,7 +482,7 @@ def compiler() -> Tuple[str, str]:
                         os.replace(tmp, note)
                 except (OSError, ValueError, IndexError, subprocess.SubprocessError):
                     system = None
-        if system is not None and (want == "system" or system > here):
+        if system is not None:
             _compiler_choice = ("system", "%d.%d.%d" % system)
         else:
             _compiler_choice = ("process", "%d.%d.%d" % here)
