@@ -143,6 +143,79 @@ class TensorProductConv(ConvolutionTiming, torch.nn.Module):
     def name():
         return "LoopUnrollConv"
 
+    # Kernel shapes that `autotune` tries beside the default (knobs of codegen/uvu.py: conv_module). The defaults
+    # are rules fitted to sweeps over some 130 problems; on a tenth of those one of these was 10 - 30 % faster in the
+    # forward kernel (another split of the outputs into register-resident segments, one operand set in flight
+    # instead of two, a third wave per SIMD), and the number of waves that share a node in the backward kernel and
+    # the route of the sender gradients have break-even points that a given graph may move.
+    AUTOTUNE_FORWARD = ("conv_acc=96", "conv_acc=64", "conv_pipe_f=0", "conv_wf=3")
+    AUTOTUNE_BACKWARD = ("conv_gb=4", "conv_ngrp=1", "conv_ngrp=2", "conv_ngrp=4", "conv_dxs=1", "conv_dxs=0")
+
+    def autotune(self, X: torch.Tensor, Y: torch.Tensor, W: torch.Tensor, rows: torch.Tensor, cols: torch.Tensor,
+                 sender_perm: Optional[torch.Tensor] = None, *, repeats: int = 5, margin: float = 0.03,
+                 verbose: bool = False) -> str:
+        """Times alternative kernel shapes for this problem on the given inputs (forward, then backward with a
+        random output gradient) and adopts the fastest where it beats the current one by more than ``margin``.
+        Every alternative computes the same convolution (they are the variants the knob tests cover); each costs a
+        kernel compile the first time. Returns the knob string in force afterwards: exporting it as
+        ``OEQ_AMD_TUNE`` makes the choice permanent for modules built later. 'uvw' problems have no alternatives
+        and are left as they are. No counterpart in the reference."""
+        import json
+        import numpy as np
+        if self._low.mode != "uvu":
+            return json.loads(bytes(self.spec.tolist()).decode())["tune"]
+        if sender_perm is None:
+            if self.deterministic:
+                raise RuntimeError("deterministic=True needs sender_perm")
+            sender_perm = rows
+        problem, det, kahan = self.config, self.deterministic, bool(self.input_args["kahan"])
+        base = json.loads(bytes(self.spec.tolist()).decode())["tune"]
+        G = torch.randn(X.shape[0], self.L3_dim, device=X.device, dtype=X.dtype)
+
+        def build(tune: str):
+            with ops._tune_env(tune):
+                kid = ops.register_spec(ops.make_spec("conv", problem, det, kahan))
+            ops.get_entry(kid).kernels()
+            return kid
+
+        def clock(fn) -> float:
+            fn()
+            times = []
+            for _ in range(repeats):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                fn()
+                b.record()
+                torch.cuda.synchronize()
+                times.append(a.elapsed_time(b))
+            return float(np.median(times))
+
+        def best_of(current: str, candidates, run) -> str:
+            best, best_ms = current, clock(lambda: run(build(current)))
+            for cand in candidates:
+                tune = ",".join(t for t in (current, cand) if t)
+                try:
+                    ms = clock(lambda: run(build(tune)))
+                except (AssertionError, RuntimeError) as err:  # a shape this problem does not have
+                    if verbose:
+                        print(f"[autotune] {cand}: skipped ({type(err).__name__})")
+                    continue
+                if verbose:
+                    print(f"[autotune] {cand}: {ms:.3f} ms")
+                if ms < best_ms * (1.0 - margin):
+                    best, best_ms = tune, ms
+            return best
+
+        with torch.no_grad():
+            tune = best_of(base, self.AUTOTUNE_FORWARD,
+                           lambda kid: ops.conv_forward(X, Y, W, rows, cols, sender_perm, kid))
+            tune = best_of(tune, self.AUTOTUNE_BACKWARD,
+                           lambda kid: ops.conv_backward(X, Y, W, G, rows, cols, sender_perm, kid))
+        if tune != base:
+            self.kid = build(tune)
+            self.spec = ops.get_entry(self.kid).spec
+        return tune
+
     def forward(self, X: torch.Tensor, Y: torch.Tensor, W: torch.Tensor, rows: torch.Tensor, cols: torch.Tensor,
                 sender_perm: Optional[torch.Tensor] = None) -> torch.Tensor:
         r"""

@@ -799,3 +799,33 @@ def test_kernel_set_compiled_side_by_side_runs(monkeypatch, tmp_path):
     assert len(packs) == 1 and len(rt.unpack_code(packs[0].read_bytes())) == 4
     for a, b in zip(whole, shares):
         assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("det", [True, False])
+def test_autotune_keeps_results(det):
+    """`TensorProductConv.autotune` times the alternative kernel shapes on the given inputs and may adopt one: the
+    module computes the same convolution afterwards, and the knob string it returns rebuilds the adopted shape."""
+    import json
+    problem = P.ChannelwiseTPP("96x0e+96x1o", "0e+1o+2e+3o", "0e+1o+2e+3o+4e", "autotuned")
+    coords, rows, cols = _graph(300, 12, seed=3)
+    g = CoordGraph(coords, rows, cols)
+    X, Y, W, G = _buffers(problem, 300, g.nnz, seed=8)
+    ref = R.Problem.from_spec(problem)
+    z_ref = R.conv_forward(ref, X, Y, W, rows, cols)
+    dx_ref, dy_ref, dw_ref = R.conv_backward(ref, X, Y, W, G, rows, cols)
+    conv = oeq.TensorProductConv(problem, deterministic=det)
+    args = [torch.tensor(a, device="cuda") for a in (X, Y[g.order], W[g.order], g.rows, g.cols)]
+    perm = torch.tensor(g.transpose_perm, device="cuda") if det else None
+    allowed = set(conv.AUTOTUNE_FORWARD) | set(conv.AUTOTUNE_BACKWARD)
+    tune = conv.autotune(*args, perm, repeats=2)
+    assert set(filter(None, tune.split(","))) <= allowed
+    assert json.loads(bytes(conv.spec.tolist()).decode())["tune"] == tune
+    tX, tY, tW = (a.clone().requires_grad_(True) for a in args[:3])
+    z = conv(tX, tY, tW, args[3], args[4], perm)
+    z.backward(torch.tensor(G, device="cuda"))
+    assert err(z, z_ref) <= 1e-5 and err(tX.grad, dx_ref) <= 1e-5
+    assert err(tY.grad.cpu().numpy(), dy_ref[g.order]) <= 1e-5 and err(tW.grad.cpu().numpy(), dw_ref[g.order]) <= 1e-5
+    # a 'uvw' problem has no alternatives
+    fc = oeq.TensorProductConv(_fc(False), deterministic=False)
+    before = fc.kid
+    assert fc.autotune(*[torch.zeros(1, device="cuda")] * 3, args[3][:1], args[4][:1]) == "" and fc.kid == before
