@@ -25,6 +25,8 @@ first-order pass's ordered reduction.
 
 from __future__ import annotations
 
+import os
+
 from typing import Dict, List, Optional, Tuple
 
 from .common import Src
@@ -909,6 +911,10 @@ def add_conv_kernels(s: Src, low: Lowered, base: UvuEmitter, tune: dict, xcd: in
     if not em.merged:
         segw = min(len(em.segments), max(1, tune.get("dd_segw", 4)), max(1, 8 // em.NCH)) if em.R == 1 else 1
         G_a = max(1, min(G, 8 // (em.NCH * segw)))
+        if len(em.segments) > 1 and "dd_g" not in os.environ.get("OEQ_AMD_TUNE", ""):
+            # several output segments: one node per block, as in the first-order forward kernel (second-order op:
+            # SevenNet main layer -4 %, three more mixed-multiplicity shapes -2 % .. -3 %, nothing slower)
+            G_a = 1
         blk_a = em.emit_conv_double_a(s, G_a, tune.get("dd_wa", 2), xcd, segw)
         descs.append((rt.ROLE_DOUBLE_BACKWARD_A, "double_backward_A", blk_a, G_a, 0, xcd))
     if groups:
