@@ -100,6 +100,70 @@ class TensorProduct(TensorProductTiming, torch.nn.Module):
     def name():
         return "LoopUnrollTP"
 
+    # Kernel shapes that `autotune` tries beside the default (knobs of codegen/uvu.py: tp_module): how many waves a
+    # SIMD may hold, rows per block, and whether the backward kernel keeps a row's output gradient in registers. Over
+    # the reference's zoo the defaults are within a few percent of the best of these, except for kernels with few
+    # words per lane, where another occupancy was up to 18 % faster for some problems and 8 % slower for others.
+    AUTOTUNE_FORWARD = ("tp_wf=-2", "tp_wf=23", "tp_gf=2")
+    AUTOTUNE_BACKWARD = ("tp_wb=-2", "tp_wb=23", "tp_gb=2", "tp_gres=1", "tp_gres=0")
+
+    def autotune(self, x: torch.Tensor, y: torch.Tensor, W: torch.Tensor, *, repeats: int = 5, margin: float = 0.03,
+                 verbose: bool = False) -> str:
+        """Times alternative kernel shapes for this problem on the given inputs (forward, then backward with a
+        random output gradient) and adopts the fastest where it beats the current one by more than ``margin``.
+        Every alternative computes the same product; each costs a kernel compile the first time. Returns the knob
+        string in force afterwards (exporting it as ``OEQ_AMD_TUNE`` makes the choice permanent for modules built
+        later). 'uvw' problems have no alternatives and are left as they are. No counterpart in the reference."""
+        import json
+        import numpy as np
+        base = json.loads(bytes(self.spec.tolist()).decode())["tune"]
+        if self.is_uvw:
+            return base
+        problem = self.config
+        g = torch.randn(x.shape[0], self.L3_dim, device=x.device, dtype=x.dtype)
+
+        def build(tune: str):
+            with ops._tune_env(tune):
+                kid = ops.register_spec(ops.make_spec("tp", problem))
+            ops.get_entry(kid).kernels()
+            return kid
+
+        def clock(fn) -> float:
+            fn()
+            times = []
+            for _ in range(repeats):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                fn()
+                b.record()
+                torch.cuda.synchronize()
+                times.append(a.elapsed_time(b))
+            return float(np.median(times))
+
+        def best_of(current: str, candidates, run) -> str:
+            best, best_ms = current, clock(lambda: run(build(current)))
+            for cand in candidates:
+                tune = ",".join(t for t in (current, cand) if t)
+                try:
+                    ms = clock(lambda: run(build(tune)))
+                except (AssertionError, RuntimeError) as err:  # a shape this problem does not have
+                    if verbose:
+                        print(f"[autotune] {cand}: skipped ({type(err).__name__})")
+                    continue
+                if verbose:
+                    print(f"[autotune] {cand}: {ms:.3f} ms")
+                if ms < best_ms * (1.0 - margin):
+                    best, best_ms = tune, ms
+            return best
+
+        with torch.no_grad():
+            tune = best_of(base, self.AUTOTUNE_FORWARD, lambda kid: ops.tp_forward(x, y, W, kid))
+            tune = best_of(tune, self.AUTOTUNE_BACKWARD, lambda kid: ops.tp_backward(x, y, W, g, kid))
+        if tune != base:
+            self.kid = build(tune)
+            self.spec = ops.get_entry(self.kid).spec
+        return tune
+
     def forward(self, x: torch.Tensor, y: torch.Tensor, W: torch.Tensor) -> torch.Tensor:
         r"""
         :param x: ``[batch, problem.irreps_in1.dim]``

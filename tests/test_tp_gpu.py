@@ -423,3 +423,48 @@ def test_kernel_shape_knobs_keep_results(knobs, monkeypatch):
         assert err(z, z_ref) <= 1e-5
         for got, want in zip((tx.grad, ty.grad, tw.grad), grads_ref):
             assert err(got, want) <= 1e-5, knobs
+
+
+def test_autotune_keeps_results():
+    """`TensorProduct.autotune` times the alternative kernel shapes (also the occupancy forms that the knob test
+    above does not name) and may adopt one: the module computes the same product afterwards, and the knob string it
+    returns is the one in its kernel-set description."""
+    import json
+    for make in (lambda: P.seven_net_problems()[0], P.config2_nequip_uvu):
+        problem = make()
+        x, y, w, g = tp_inputs(problem, 500, seed=9)
+        ref = R.Problem.from_spec(problem)
+        z_ref = R.tp_forward(ref, x, y, w)
+        grads_ref = R.tp_backward(ref, x, y, w, g)
+        tp = oeq.TensorProduct(problem)
+        tune = tp.autotune(*to_gpu(x, y, w), repeats=2)
+        assert set(filter(None, tune.split(","))) <= set(tp.AUTOTUNE_FORWARD) | set(tp.AUTOTUNE_BACKWARD)
+        assert json.loads(bytes(tp.spec.tolist()).decode())["tune"] == tune
+        tx, ty, tw = to_gpu(x, y, w, requires_grad=True)
+        z = tp(tx, ty, tw)
+        z.backward(torch.tensor(g, device="cuda"))
+        assert err(z, z_ref) <= 1e-5
+        for got, want in zip((tx.grad, ty.grad, tw.grad), grads_ref):
+            assert err(got, want) <= 1e-5
+    shared = oeq.TensorProduct(P.config4_uvw_shared())
+    before = shared.kid
+    assert shared.autotune(*[torch.zeros(1, device="cuda")] * 3) == "" and shared.kid == before
+
+
+@pytest.mark.parametrize("knobs", ["tp_wf=-2,tp_wb=-2", "tp_wf=23,tp_wb=23,tp_gres=1"])
+def test_occupancy_forms_keep_results(knobs, monkeypatch):
+    """The occupancy forms that `autotune` may adopt (a minimum only; a minimum and a maximum) on a small, a large and
+    a shared-weight problem."""
+    monkeypatch.setenv("OEQ_AMD_TUNE", knobs)
+    for make in (P.config3_mace_uvu, lambda: P.seven_net_problems()[2], lambda: _odd_uvu(True)):
+        problem = make()
+        x, y, w, g = tp_inputs(problem, 45, seed=6)
+        ref = R.Problem.from_spec(problem)
+        z_ref = R.tp_forward(ref, x, y, w)
+        grads_ref = R.tp_backward(ref, x, y, w, g)
+        tx, ty, tw = to_gpu(x, y, w, requires_grad=True)
+        z = oeq.TensorProduct(problem)(tx, ty, tw)
+        z.backward(torch.tensor(g, device="cuda"))
+        assert err(z, z_ref) <= 1e-5
+        for got, want in zip((tx.grad, ty.grad, tw.grad), grads_ref):
+            assert err(got, want) <= 1e-5, knobs
