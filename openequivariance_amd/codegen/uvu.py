@@ -828,18 +828,37 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         return (self.R == 1 and all(low.in1[b].mul == U for b in self.used_in1)
                 and all(low.out[io].mul == U for io in self.used_out))
 
-    def _atomic_block_transposed(self, s: Src, rowexpr: str, off: int, d: int, val: Callable[[int], str]):
+    def _atomics_coalesce(self) -> bool:
+        """The sender-gradient atomics of the backward kernel can go through the LDS transpose: rows that fill the
+        wave's chunks, or rows of one chunk whatever the multiplicities of their blocks."""
+        return self._regular_wave() or (self.R == 1 and self.NCH == 1)
+
+    def _atomic_block_transposed(self, s: Src, rowexpr: str, off: int, d: int, val: Callable[[int], str],
+                                 mul: Optional[int] = None):
         """Atomic accumulation of one [64 x d] channel block. The lane-per-channel registers go
         through a wave-private LDS tile so that every atomic instruction of the wave covers 64
-        consecutive elements (two cache lines) instead of 64 elements ``d`` apart."""
+        consecutive elements (two cache lines) instead of 64 elements ``d`` apart. ``mul`` < 64 (rows of one
+        chunk only): a block of that many channels, whose mul * d values are consecutive as well."""
         # lanes exchange data through the tile: the wave-scope fences keep the compiler from
         # reordering one lane's reads against its own (different-address) writes
         s("oeq_wave_sync();")
+        if mul is None or mul == 64 * self.NCH:
+            for k in range(d):
+                s(f"s_tr[wave][ul * {d} + {k}] = {val(k)};")
+            s("oeq_wave_sync();")
+            for t in range(d):
+                s(f"oeq_atomic_add({rowexpr} + {off} + chunk * {64 * d} + {t * 64} + ul, s_tr[wave][{t * 64} + ul]);")
+            return
+        assert self.NCH == 1 and mul < 64
+        s.open(f"if (ul < {mul})")
         for k in range(d):
             s(f"s_tr[wave][ul * {d} + {k}] = {val(k)};")
+        s.close()
         s("oeq_wave_sync();")
-        for t in range(d):
-            s(f"oeq_atomic_add({rowexpr} + {off} + chunk * {64 * d} + {t * 64} + ul, s_tr[wave][{t * 64} + ul]);")
+        n = mul * d
+        for t in range((n + 63) // 64):
+            guard = f"if ({t * 64} + ul < {n}) " if (t + 1) * 64 > n else ""
+            s(f"{guard}oeq_atomic_add({rowexpr} + {off} + {t * 64} + ul, s_tr[wave][{t * 64} + ul]);")
 
     def _store_block_transposed(self, s: Src, rowexpr: str, off: int, d: int, val: Callable[[int], str],
                                 nt: bool = False):
@@ -1580,7 +1599,7 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         if atomic and self.tr_atomics:
             for b in self._in1_of(self.used_in1):
                 blk = low.in1[b]
-                self._atomic_block_transposed(s, rowexpr, blk.off, blk.d, lambda i, b=b: f"dx.b{b}[{i}]")
+                self._atomic_block_transposed(s, rowexpr, blk.off, blk.d, lambda i, b=b: f"dx.b{b}[{i}]", blk.mul)
             return
         for b in self._in1_of(self.used_in1):
             blk = low.in1[b]
@@ -2022,7 +2041,7 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
                 s(f"__shared__ __attribute__((aligned(16))) T s_stage{b}[{self.NCH * G}][{self.stage3['floats']}];")
             self._emit_stage3_offsets(s)
         dx_atomic = (not deterministic) or dx_mode == self.DX_ATOMIC
-        self.tr_atomics = dx_atomic and tr_atomics and self._regular_wave() and not self.ir_mul
+        self.tr_atomics = dx_atomic and tr_atomics and self._atomics_coalesce() and not self.ir_mul
         if self.tr_atomics or (self.tr_stores & 2 and self.R == 1):
             s(f"__shared__ T s_tr[{self.NCH * G}][{64 * max(low.in1[b].d for b in self.used_in1)}];")
         resident = deterministic and (self.g_resident if g_resident is None else g_resident)
@@ -2369,7 +2388,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             # (only where a row fills the wave and the atomics go through the LDS transpose, 64 consecutive
             # floats per instruction: per-lane atomics of packed or ragged rows are several times slower than
             # the ordered reduction)
-            coalesced = bool(t["conv_tra"]) and em._regular_wave() and not em.ir_mul
+            coalesced = bool(t["conv_tra"]) and em._atomics_coalesce() and not em.ir_mul
             dx_mode = t["conv_dxm"] if t["conv_dxm"] >= 0 else (
                 em.DX_ATOMIC if (mode == rt.CONV_GROUPED and coalesced) else em.DX_TERMS)
             # arrival counting keeps an edge's terms lane-major, 64 values per (block, component) and chunk: they
