@@ -209,7 +209,9 @@ class TensorProductConv(ConvolutionTiming, torch.nn.Module):
         with torch.no_grad():
             tune = best_of(base, self.AUTOTUNE_FORWARD,
                            lambda kid: ops.conv_forward(X, Y, W, rows, cols, sender_perm, kid))
-            tune = best_of(tune, self.AUTOTUNE_BACKWARD,
+            # (how the sender gradients travel is a choice only where the bits need not repeat from run to run)
+            travel = () if det else ("conv_dxm=0", "conv_dxm=1")
+            tune = best_of(tune, self.AUTOTUNE_BACKWARD + travel,
                            lambda kid: ops.conv_backward(X, Y, W, G, rows, cols, sender_perm, kid))
         if tune != base:
             self.kid = build(tune)

@@ -1874,11 +1874,13 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             n += 1
         return None
 
-    def emit_conv_backward_split(self, s: Src, waves_per_eu: int = 0, xcd: int = 1) -> int:
+    def emit_conv_backward_split(self, s: Src, waves_per_eu: int = 0, xcd: int = 1, dx_atomic: bool = False) -> int:
         """Deterministic-walk backward for problems whose output gradient exceeds one wave's registers:
         the waves of a block all walk the edges of one node; wave ``sg`` keeps the gradient of its output
         blocks resident and handles the paths into them (their dW is final); the partial dX and dY of an
-        edge are summed over the waves through LDS, in a fixed order."""
+        edge are summed over the waves through LDS, in a fixed order. ``dx_atomic``: the summed sender gradient of
+        an edge is added to the sender's row with float atomics (64 consecutive values per instruction, read
+        across the LDS copy) instead of being written to ``dx_tmp`` for the ordered reduction."""
         low = self.low
         groups = self.bwd_groups
         SW = len(groups)
@@ -1951,12 +1953,29 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
                 s.close()
                 s("__syncthreads();")
                 # the used input blocks are shared out between the waves for the final sum and store
-                s(f"T* dxrow = dx_tmp + eid * {low.L1};")
+                if dx_atomic:
+                    s(f"T* dxrow = L1_grad + oeq_idx(cols[eid], node_count) * {low.L1};")
+                else:
+                    s(f"T* dxrow = dx_tmp + eid * {low.L1};")
                 for n, b in enumerate(self.used_in1):
                     if n % SW != si or not self._has(low.in1[b].mul):
                         continue
                     blk = low.in1[b]
                     contributors = [c for c in range(SW) if b in gin1[c]]
+                    if dx_atomic:
+                        # the chunk's channels of the block, channel-major in memory: value f of them is component
+                        # f % d of channel f / d
+                        if not contributors:
+                            continue
+                        ch = min(64, blk.mul - 64 * self.cur_chunk) if self.cur_chunk is not None else min(64, blk.mul)
+                        first = f"chunk * {64 * blk.d}" if self.NCH > 1 else "0"
+                        for tt in range((ch * blk.d + 63) // 64):
+                            s.open(f"if ({tt * 64} + ul < {ch * blk.d})" if (tt + 1) * 64 > ch * blk.d else "")
+                            s(f"const int f = {tt * 64} + ul, fu = f / {blk.d}, fi = f % {blk.d};")
+                            terms = " + ".join(f"s_dx[{c}][chunk][{xoff[b]} + fi][fu]" for c in contributors)
+                            s(f"oeq_atomic_add(dxrow + {blk.off} + {first} + f, {terms});")
+                            s.close()
+                        continue
                     self._open_if(s, self._store_cond(blk.mul))
                     base, st = self._lane_ptr(blk)
                     s(f"T* dp = {self._ptr('dxrow', base)};")
@@ -1969,7 +1988,8 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
                             s(f"dp[{i * st}] = {val};")
                     s.close()
                 if si == 0:
-                    self._zero_untouched_in1(s, "dxrow", "true")
+                    if not dx_atomic:  # (the library clears the sender rows before a launch that adds to them)
+                        self._zero_untouched_in1(s, "dxrow", "true")
                     s.open(f"if (chunk == 0)")
                     s.open(f"for (int j = lane; j < {low.L2}; j += 64)")
                     s("T tot = s_dy[0][j];")
@@ -2378,7 +2398,13 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             # blocks of 3 waves leave a quarter of the wave slots empty at 2 waves per SIMD (8 per CU); at 3
             # per SIMD they fill them (SevenNet main layer: 14.6 -> 10.1 ms)
             t["conv_wb"] = 3
-        blk_b = em.emit_conv_backward_split(s, t["conv_wb"], xcd)
+        # deterministic=False, on request (conv_dxm=1): the edge's summed sender gradient leaves as float atomics
+        # from the LDS copy it is summed in. Against the per-edge terms and their ordered reduction, backward op on
+        # the config-5 graph: SevenNet main layer 9.47 -> 8.96 ms and a 512-word row -6 %, but rows of 864 words
+        # and more +21 % .. +41 % (NequIP benzene 21.9 -> 26.5 ms): the one-wave kernel's rule does not carry over.
+        split_atomic = (mode == rt.CONV_GROUPED and not kahan and not em.ir_mul and t["conv_dxm"] == em.DX_ATOMIC)
+        dx_mode = em.DX_ATOMIC if split_atomic else em.DX_TERMS
+        blk_b = em.emit_conv_backward_split(s, t["conv_wb"], xcd, split_atomic)
     else:
         # what becomes of the walk's per-edge dX terms (UvuEmitter.emit_conv_backward)
         if walk and not kahan:

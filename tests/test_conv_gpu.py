@@ -639,7 +639,9 @@ KNOBS = ["conv_pipe_f=0,conv_pipe_b=1", "conv_pipe_f=1,conv_pipe_b=2", "conv_pip
          # segments and chunks of 2; and never
          "conv_dxs=1", "conv_dxs=1,conv_hub=2,conv_hops=1", "conv_dxs=0",
          # a node's output gradient shared between that many waves in the backward kernel (1: a single owner)
-         "conv_ngrp=1", "conv_ngrp=2,conv_hub=2", "conv_ngrp=3", "conv_ngrp=4,conv_hub=3"]
+         "conv_ngrp=1", "conv_ngrp=2,conv_hub=2", "conv_ngrp=3", "conv_ngrp=4,conv_hub=3",
+         # ... whose summed sender gradient leaves as float atomics (deterministic=False; the sorted mode ignores it)
+         "conv_ngrp=2,conv_dxm=1"]
 
 
 @pytest.mark.parametrize("knobs", KNOBS)
@@ -816,7 +818,7 @@ def test_autotune_keeps_results(det):
     conv = oeq.TensorProductConv(problem, deterministic=det)
     args = [torch.tensor(a, device="cuda") for a in (X, Y[g.order], W[g.order], g.rows, g.cols)]
     perm = torch.tensor(g.transpose_perm, device="cuda") if det else None
-    allowed = set(conv.AUTOTUNE_FORWARD) | set(conv.AUTOTUNE_BACKWARD)
+    allowed = set(conv.AUTOTUNE_FORWARD) | set(conv.AUTOTUNE_BACKWARD) | {"conv_dxm=0", "conv_dxm=1"}
     tune = conv.autotune(*args, perm, repeats=2)
     assert set(filter(None, tune.split(","))) <= allowed
     assert json.loads(bytes(conv.spec.tolist()).decode())["tune"] == tune
