@@ -830,8 +830,9 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
 
     def _atomics_coalesce(self) -> bool:
         """The sender-gradient atomics of the backward kernel can go through the LDS transpose: rows that fill the
-        wave's chunks, or rows of one chunk whatever the multiplicities of their blocks."""
-        return self._regular_wave() or (self.R == 1 and self.NCH == 1)
+        wave's chunks, or rows of one chunk (or less: several rows to a wave) whatever the multiplicities of their
+        blocks."""
+        return self._regular_wave() or self.NCH == 1
 
     def _atomic_block_transposed(self, s: Src, rowexpr: str, off: int, d: int, val: Callable[[int], str],
                                  mul: Optional[int] = None):
@@ -842,23 +843,26 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
         # lanes exchange data through the tile: the wave-scope fences keep the compiler from
         # reordering one lane's reads against its own (different-address) writes
         s("oeq_wave_sync();")
-        if mul is None or mul == 64 * self.NCH:
+        if self.R == 1 and (mul is None or mul == 64 * self.NCH):
             for k in range(d):
                 s(f"s_tr[wave][ul * {d} + {k}] = {val(k)};")
             s("oeq_wave_sync();")
             for t in range(d):
                 s(f"oeq_atomic_add({rowexpr} + {off} + chunk * {64 * d} + {t * 64} + ul, s_tr[wave][{t * 64} + ul]);")
             return
-        assert self.NCH == 1 and mul < 64
+        # (rows narrower than the wave: each group of lanes has its own row and its own part of the tile)
+        assert self.NCH == 1 and mul <= self.LPR
+        lpr = self.LPR
+        mine = f"r * {lpr * d} + " if self.R > 1 else ""
         s.open(f"if (ul < {mul})")
         for k in range(d):
-            s(f"s_tr[wave][ul * {d} + {k}] = {val(k)};")
+            s(f"s_tr[wave][{mine}ul * {d} + {k}] = {val(k)};")
         s.close()
         s("oeq_wave_sync();")
         n = mul * d
-        for t in range((n + 63) // 64):
-            guard = f"if ({t * 64} + ul < {n}) " if (t + 1) * 64 > n else ""
-            s(f"{guard}oeq_atomic_add({rowexpr} + {off} + {t * 64} + ul, s_tr[wave][{t * 64} + ul]);")
+        for t in range((n + lpr - 1) // lpr):
+            guard = f"if ({t * lpr} + ul < {n}) " if (t + 1) * lpr > n else ""
+            s(f"{guard}oeq_atomic_add({rowexpr} + {off} + {t * lpr} + ul, s_tr[wave][{mine}{t * lpr} + ul]);")
 
     def _store_block_transposed(self, s: Src, rowexpr: str, off: int, d: int, val: Callable[[int], str],
                                 nt: bool = False):
