@@ -2248,6 +2248,35 @@ def tp_module(low: Lowered, compute_units: int = 256):
     return s.text(), dims, descs
 
 
+def _forward_plan(low: Lowered, first_budget: int) -> Tuple[UvuEmitter, bool]:
+    """(emitter, two operand sets in flight?) for a walk kernel without LDS staging: the accumulators of an output
+    segment, the edge's operands (X blocks, the weights of the segment's paths, Y) once or twice, within the registers
+    of two waves per SIMD. The segment budget shrinks until that fits; the prefetch goes when 48-word segments do
+    not fit with it."""
+    words = 1 if low.elem_size == 4 else 2
+
+    def plan(budget, sets):
+        e = UvuEmitter(low, acc_budget_words=budget)
+        need = max(sets * words * (sum(low.in1[b].d for b in e.seg_in1[si]) + low.L2 +
+                                   sum(low.in2[p.i2].mul for p in low.paths if p.io in seg))
+                   + words * sum(low.out[io].d for io in seg) for si, seg in enumerate(e.segments))
+        return e, need + (40 if e.ragged() else 0)
+
+    e = UvuEmitter(low, acc_budget_words=first_budget)
+    if e.stage is not None or not e.can_preload:
+        return e, True
+    budgets = (first_budget, 96, 64, 48)
+    for budget in budgets:
+        e, need = plan(budget, 2)
+        if need <= 170:
+            return e, True
+    for budget in budgets:
+        e, need = plan(budget, 1)
+        if need <= 190:
+            break
+    return e, False
+
+
 def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kahan: bool = False,
                 override: Optional[Dict[str, int]] = None):
     """Source + launch descriptors for the fused convolution (forward, backward).
@@ -2455,7 +2484,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         if dx_mode == UvuEmitter.DX_SENDER_WALK:
             from .lower import adjoint
             low_x = adjoint(low)
-            ex = UvuEmitter(low_x, acc_budget_words=t["conv_acc"])
+            ex, pipe_x = _forward_plan(low_x, t["conv_acc"])
             ex.nt, ex.mask_loads, ex.forms, ex.tr_stores = t["conv_nt"], bool(t["tp_mask"]), bool(t["tp_forms"]), t["conv_trs"]
             words_x = (1 if low.elem_size == 4 else 2) * (
                 max(sum(low_x.out[io].d for io in seg) for seg in ex.segments)
@@ -2466,8 +2495,8 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             ex.use_q = False
             ex.emit_forward_cores(s, preloaded=True)
             G_x = max(1, 4 // low_x.n_chunks)
-            blk_x = ex.emit_conv_forward(s, G_x, True, t["conv_pipe_f"], -2 if words_x <= 48 else 2, xcd,
-                                         bool(t["conv_tra"]), name="backward_dx")
+            blk_x = ex.emit_conv_forward(s, G_x, True, t["conv_pipe_f"] if pipe_x else 0, -2 if words_x <= 48 else 2,
+                                         xcd, bool(t["conv_tra"]), name="backward_dx")
             s("}  // namespace oeq_dx")
             descs.append((rt.ROLE_CONV_BACKWARD_DX, "backward_dx", blk_x, G_x, 0, xcd))
         from . import uvu_double
@@ -2501,6 +2530,12 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
                 wpartial_per_block=G_b if (walk and low.shared_weights) else 0, dx_mode=dx_mode,
                 n_chunks=em.NCH, order_hops=max(0, t["conv_hops"]) if walk else 0, hub_limit=hub_limit)
     src = s.text()
+    if dx_mode == UvuEmitter.DX_SENDER_WALK and t["conv_dxs"] < 0:
+        # the sender walk was chosen by its rule, not asked for: not with a kernel that does not fit its registers
+        # (forced on shapes beyond the rule, adjoint kernels with 200 - 320 B of scratch ran 3x slower than the terms)
+        _lds, scratch = rt.kernel_resources(rt.compile_source(src)).get("backward_dx", (0, 0))
+        if scratch > 64:
+            return conv_module(low, deterministic, compute_units, kahan, dict(override or {}, conv_dxs=0))
     if em.seg_waves > 1 and "conv_segw" not in user_tune:
         # Waves that share a node's output segments: with two operand sets in flight and three or more segments
         # the compiler has been seen to need more registers for the kernel that selects a wave's segments by
