@@ -30,6 +30,7 @@ loop_unroll_conv_det.cuh:96-293) with a different decomposition:
 from __future__ import annotations
 
 import os
+import re
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 from .common import Src, fixup_backward_kernel, prelude, utility_kernels
@@ -2545,4 +2546,26 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         _lds, scratch = rt.kernel_resources(rt.compile_source(src)).get("forward", (0, 0))
         if scratch > 64:
             return conv_module(low, deterministic, compute_units, kahan, dict(override or {}, conv_segw=0))
+    if walk and t["conv_wf"] == 23 and "conv_wf" not in user_tune and low.elem_size == 4:
+        # A forward kernel that the compiler gave more than a third of a SIMD's registers runs two waves there.
+        # Held to a third it runs three, which pays where the compiler manages that without scratch memory (fp32,
+        # config-5 graph, forward: 96 channels of l <= 3 with l <= 3 harmonics 176 -> 168 registers, -18 %; 64
+        # channels of l <= 3, l <= 2 harmonics 197 -> 160, -10 %; all five such shapes of 128 tried gained 9 - 19 %)
+        # and costs where it does not (12 B of scratch: +21 % and +28 %; 100 B and more: +40 % .. +144 %).
+        # The code objects say which it is (compiled here, cached like any other; of the second form only the
+        # forward kernel).
+        if rt.kernel_registers(rt.compile_source(src)).get("forward", 0) > 168:
+            third = conv_module(low, deterministic, compute_units, kahan, dict(override or {}, conv_wf=3))
+            if _forward_scratch(third[0]) == 0:
+                return third
     return src, dims, descs
+
+
+def _forward_scratch(source: str) -> int:
+    """Bytes of scratch memory per lane of a convolution module's forward kernel, compiled without the module's
+    other kernels."""
+    from .. import runtime as rt
+    common, kernels = rt.split_kernels(source)
+    own = [k for k in kernels if re.search(r"\bvoid\s+forward\s*\(", k)]
+    blob = rt.compile_source(common + "\n" + own[0] if len(own) == 1 else source)
+    return rt.kernel_resources(blob).get("forward", (0, 0))[1]

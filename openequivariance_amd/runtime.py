@@ -334,13 +334,11 @@ def unpack_code(blob: bytes) -> List[bytes]:
     return out
 
 
-def kernel_resources(blob: bytes) -> Dict[str, Tuple[int, int]]:
-    """{kernel name: (bytes of LDS, bytes of scratch memory per lane)} of the kernels in what compile_source
-    returned, from the kernel descriptors (the 64-byte objects ``<name>.kd`` of an amdhsa code object, whose
-    first two 32-bit words are group_segment_fixed_size and private_segment_fixed_size). A kernel that the
-    compiler could not fit into its register budget has a non-zero scratch size."""
+def _kernel_descriptors(blob: bytes) -> Dict[str, bytes]:
+    """{kernel name: its 64-byte kernel descriptor} (the objects ``<name>.kd`` of an amdhsa code object) of the
+    kernels in what compile_source returned."""
     import struct
-    out: Dict[str, Tuple[int, int]] = {}
+    out: Dict[str, bytes] = {}
     for elf in unpack_code(blob):
         shoff, = struct.unpack_from("<Q", elf, 0x28)
         shentsize, shnum = struct.unpack_from("<HH", elf, 0x3A)
@@ -356,9 +354,28 @@ def kernel_resources(blob: bytes) -> Dict[str, Tuple[int, int]]:
                 if not name.endswith(".kd") or st_size != 64 or not 0 < st_shndx < shnum:
                     continue
                 sec = sections[st_shndx]
-                lds, scratch = struct.unpack_from("<II", elf, sec[4] + st_value - sec[3])
-                out[name[:-3]] = (lds, scratch)
+                start = sec[4] + st_value - sec[3]
+                out[name[:-3]] = elf[start:start + 64]
     return out
+
+
+def kernel_resources(blob: bytes) -> Dict[str, Tuple[int, int]]:
+    """{kernel name: (bytes of LDS, bytes of scratch memory per lane)} of the kernels in what compile_source
+    returned, from the kernel descriptors (whose first two 32-bit words are group_segment_fixed_size and
+    private_segment_fixed_size). A kernel that the compiler could not fit into its register budget has a
+    non-zero scratch size."""
+    import struct
+    return {name: struct.unpack_from("<II", kd, 0) for name, kd in _kernel_descriptors(blob).items()}
+
+
+def kernel_registers(blob: bytes) -> Dict[str, int]:
+    """{kernel name: vector registers a lane of it is allocated} (architectural and accumulation registers
+    together, in the granules of eight that gfx90a and later allocate: bits 5:0 of compute_pgm_rsrc1, the
+    32-bit word at byte 48 of the kernel descriptor, hold the granule count minus one). A SIMD's 512 registers
+    per lane divided by this number is how many waves of the kernel it holds."""
+    import struct
+    return {name: ((struct.unpack_from("<I", kd, 48)[0] & 0x3F) + 1) * 8
+            for name, kd in _kernel_descriptors(blob).items()}
 
 
 def _loaded_rocm_libraries() -> Dict[str, str]:

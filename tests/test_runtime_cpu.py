@@ -211,6 +211,38 @@ def test_forward_kernel_that_spills_gives_way_to_one_wave_per_node():
     assert forward[2] == 192 and forward[3] == 1 and rt.kernel_resources(rt.compile_source(src))["forward"][1] == 0
 
 
+def test_forward_kernel_takes_a_third_wave_where_that_costs_no_scratch_memory():
+    """A forward kernel that the compiler gave more than a third of a SIMD's registers is generated again held
+    to a third, and that form is kept where its code object shows no scratch memory."""
+    from openequivariance_amd._torch.tensor_product_conv import build_conv_module
+
+    def forward_bounds(src):
+        head = src[:src.index("void forward(")]
+        return re.findall(r"amdgpu_waves_per_eu\(([^)]*)\)", head)[-1].replace(" ", "")
+
+    os.environ.pop("OEQ_AMD_TUNE", None)
+    harmonics = "1x0e+1x1o+1x2e+1x3o"
+    fits = P.CTPP("96x0e+96x1o+96x2e+96x3o", harmonics, "0e+1o+2e+3o", "96-channels")
+    src, _dims, _descs = build_conv_module(fits, True)
+    assert forward_bounds(src) == "3,3"
+    blob = rt.compile_source(src)
+    assert rt.kernel_registers(blob)["forward"] <= 168 and rt.kernel_resources(blob)["forward"][1] == 0
+    os.environ["OEQ_AMD_TUNE"] = "conv_wf=23"
+    try:
+        src, _dims, _descs = build_conv_module(fits, True)
+    finally:
+        os.environ.pop("OEQ_AMD_TUNE", None)
+    assert forward_bounds(src) == "2,3" and rt.kernel_registers(rt.compile_source(src))["forward"] > 168
+    # held to a third this kernel would spill: it keeps its two waves
+    spills = P.CTPP("128x0e+96x1e+64x2e", harmonics.replace("o", "e"), "0e+1e+2e", "mixed-channels")
+    src, _dims, _descs = build_conv_module(spills, True)
+    assert forward_bounds(src) == "2,3" and rt.kernel_registers(rt.compile_source(src))["forward"] > 168
+    # double precision is left alone
+    src, _dims, _descs = build_conv_module(P.CTPP("96x0e+96x1o+96x2e+96x3o", harmonics, "0e+1o+2e+3o", "96-channels-f64",
+                                                  irrep_dtype=np.float64, weight_dtype=np.float64), True)
+    assert forward_bounds(src) == "2,3"
+
+
 def test_malformed_code_packs_are_rejected():
     import struct
     dims = dict(L1_dim=4, L2_dim=4, L3_dim=4, weight_numel=4, elem_size=4)
