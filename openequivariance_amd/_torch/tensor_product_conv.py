@@ -20,6 +20,7 @@ import torch
 
 from ..codegen.lower import lower
 from ..core.spec import TPProblem
+from .. import runtime as rt
 from . import ops
 from .benchmarking import ConvolutionTiming
 from .utils import compute_units, oeq_to_torch_dtype, torch_to_oeq_dtype
@@ -42,7 +43,6 @@ def build_conv_module(problem: TPProblem, deterministic: bool, kahan: bool = Fal
     if low.mode == "uvu":
         from ..codegen import uvu
         return uvu.conv_module(low, deterministic, compute_units(), kahan)
-    from .. import runtime as rt
     from ..codegen import uvw
     if fused(low):
         return uvw.conv_module(low, deterministic, compute_units(), kahan)
@@ -213,6 +213,10 @@ class TensorProductConv(ConvolutionTiming, torch.nn.Module):
             travel = () if det else ("conv_dxm=0", "conv_dxm=1")
             tune = best_of(tune, self.AUTOTUNE_BACKWARD + travel,
                            lambda kid: ops.conv_backward(X, Y, W, G, rows, cols, sender_perm, kid))
+            if ops.get_entry(build(tune)).kernels().dims.get("dx_mode", 0) == rt.DX_SENDER_WALK:
+                # the sender-walk kernel with a third wave per SIMD where its registers allow
+                tune = best_of(tune, ("conv_wx=23",),
+                               lambda kid: ops.conv_backward(X, Y, W, G, rows, cols, sender_perm, kid))
         if tune != base:
             self.kid = build(tune)
             self.spec = ops.get_entry(self.kid).spec

@@ -2299,7 +2299,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
 
     assert not (deterministic and low.shared_weights), "deterministic convolution needs per-edge weights"
     t = tuning(dict(conv_acc=128, conv_gf=max(1, 4 // low.n_chunks), conv_gb=4, conv_pipe_f=2, conv_pipe_b=0,
-                    conv_wf=23, conv_wb=2, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
+                    conv_wf=23, conv_wb=2, conv_wx=0, conv_gres=-1, conv_xcd=8, conv_tra=1, conv_nt=15, conv_epw=8,
                     conv_sort=1, conv_trs=3 if low.elem_size == 8 else 0, conv_sb=-1,
                     conv_segw=4, conv_split=1, conv_dd=1, dd_acc=0, dd_g=2, dd_wa=2, dd_wb=2, dd_fp=0, dd_fw=32,
                     dd_gres=-1, dd_split=1, dd_segw=4, dd_merge=0, dd_need=200, dd_ngrp=0, conv_gbud=0, conv_ngrp=0, conv_fit=300, conv_fw=0, conv_pf=0,
@@ -2496,7 +2496,8 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             ex.use_q = False
             ex.emit_forward_cores(s, preloaded=True)
             G_x = max(1, 4 // low_x.n_chunks)
-            blk_x = ex.emit_conv_forward(s, G_x, True, t["conv_pipe_f"] if pipe_x else 0, -2 if words_x <= 48 else 2,
+            waves_x = t["conv_wx"] if t["conv_wx"] else (-2 if words_x <= 48 else 2)
+            blk_x = ex.emit_conv_forward(s, G_x, True, t["conv_pipe_f"] if pipe_x else 0, waves_x,
                                          xcd, bool(t["conv_tra"]), name="backward_dx")
             s("}  // namespace oeq_dx")
             descs.append((rt.ROLE_CONV_BACKWARD_DX, "backward_dx", blk_x, G_x, 0, xcd))

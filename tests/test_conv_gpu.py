@@ -641,6 +641,8 @@ KNOBS = ["conv_pipe_f=0,conv_pipe_b=1", "conv_pipe_f=1,conv_pipe_b=2", "conv_pip
          # sender gradients by a second walk over the senders' edges (forward kernel of the adjoint problem), whole
          # segments and chunks of 2; and never
          "conv_dxs=1", "conv_dxs=1,conv_hub=2,conv_hops=1", "conv_dxs=0",
+         # ... that kernel with a third wave per SIMD where its registers allow, and held to it
+         "conv_dxs=1,conv_wx=23", "conv_dxs=1,conv_wx=3",
          # a node's output gradient shared between that many waves in the backward kernel (1: a single owner)
          "conv_ngrp=1", "conv_ngrp=2,conv_hub=2", "conv_ngrp=3", "conv_ngrp=4,conv_hub=3",
          # ... whose summed sender gradient leaves as float atomics (deterministic=False; the sorted mode ignores it)
