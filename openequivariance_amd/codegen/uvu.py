@@ -1877,7 +1877,13 @@ f"const T* __restrict__ W, const i64* __restrict__ cols, const i64 node_count, c
             if all(sum(low.out[io].d for io in grp) <= budget for grp in groups):
                 return groups
             n += 1
-        return None
+        # No count brings a wave's share under the limit (double precision with many output blocks: NequIP benzene
+        # and eight synthetic shapes of 276 problems in both precisions). The unshared kernel, which reads a node's
+        # gradient per edge, is the slowest choice there: as many waves as allowed (config-5 graph, fp64, backward:
+        # benzene 103.5 -> 61.8 ms; six other shapes -11 % .. -28 %, one +2 %; four waves instead of eight:
+        # -35 % .. +20 %).
+        n = min(8, max_waves, len(sizes))
+        return balanced(n) if n >= 2 else None
 
     def emit_conv_backward_split(self, s: Src, waves_per_eu: int = 0, xcd: int = 1, dx_atomic: bool = False) -> int:
         """Deterministic-walk backward for problems whose output gradient exceeds one wave's registers:

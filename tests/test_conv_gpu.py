@@ -110,6 +110,8 @@ CASES = [
     ("sevennet-main", lambda: P.seven_net_problems()[1], 30, 5),
     ("four-irreps-even", lambda: P.ChannelwiseTPP("64x0e+64x1e+64x2e+64x3e", "1x0e+1x1e+1x2e+1x3e", "0e+1e+2e+3e",
                                                   "four-irreps-even"), 30, 5),
+    # eight waves share a node in the backward kernel: no smaller count brings a wave's share under the register limit
+    ("benzene-f64", lambda: _as_f64(P.nequip_problems()[3]), 24, 4),
     # the forward kernel held to a third of a SIMD's registers (it fits them without scratch memory)
     ("96-channels", lambda: P.ChannelwiseTPP("96x0e+96x1o+96x2e+96x3o", "1x0e+1x1o+1x2e+1x3o", "0e+1o+2e+3o",
                                              "96-channels"), 30, 5),

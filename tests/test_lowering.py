@@ -213,3 +213,26 @@ def test_adjoint_problem_gives_the_first_operand_gradient():
         x, y, w, g = (rng.normal(size=n) for n in (low.L1, low.L2, low.WN, low.L3))
         lhs, rhs = g @ forward(low, x, y, w), x @ forward(adj, g, y, w)
         assert abs(lhs - rhs) <= 1e-12 * max(1.0, abs(lhs))
+
+
+def test_backward_wave_count_per_node():
+    """Waves that share a node's output gradient in the convolution's backward kernel: one where the register
+    estimate fits, else the smallest of two and four whose share fits, and all eight where none does."""
+    from openequivariance_amd.codegen import uvu
+
+    def count(problem):
+        em = uvu.UvuEmitter(L.lower(problem))
+        groups = em.plan_backward_groups(max(1, 8 // em.NCH))
+        if groups is not None:  # every output block once, in order
+            assert [io for grp in groups for io in grp] == list(em.used_out)
+        return 0 if groups is None else len(groups)
+
+    def f64(problem):
+        out = problem.clone()
+        out.irrep_dtype = out.weight_dtype = np.float64
+        return out
+
+    assert count(P.config5_mace_conv()) == 0                      # fits one wave's registers by the ordinary rule
+    assert count(P.seven_net_problems()[1]) == 2
+    assert count(P.nequip_problems()[3]) == 4                     # benzene
+    assert count(f64(P.nequip_problems()[3])) == 8                # ... whose shares in double precision never fit
