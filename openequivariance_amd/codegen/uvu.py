@@ -2330,6 +2330,13 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
     # per output segment / sharing the node between waves (MACE shape, fp64: forward 18.4 -> 12.5 ms,
     # backward 42.1 -> 26.4 ms). The same plan loses for every fp32 problem tried.
     wide64 = low.elem_size == 8 and em.R == 1 and not kahan and walk and not low.shared_weights
+    wide64_forward = False
+    if low.elem_size == 8 and "conv_wf" not in user_tune:
+        # fp64 forward kernels get the plain budget of two waves per SIMD: allowed a third, the compiler stays
+        # under 256 registers without reaching 168 and the kernel runs at half speed (config-5 graph, forward:
+        # 128x{0e,1o,2e} with l <= 3 harmonics, 216 registers, 10.5 against 5.4 ms; 128x{0e..3o} 12.9 / 7.5 and
+        # 36.2 / 19.4); the zoo's eleven fp64 kernels of this kind are within -4.3 % .. +1.4 % either way.
+        t["conv_wf"] = 2
     if wide64 and "conv_acc" not in user_tune and "conv_wf" not in user_tune:
         x_all = sum(low.in1[b].d for b in em.used_in1)
         need_f = 2 * (sum(low.out[io].d for io in em.used_out) + x_all + em.n_wslots + low.L2) + 40
@@ -2337,6 +2344,7 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
             t["conv_acc"], t["conv_wf"] = 1 << 20, 1
             t["conv_trs"] &= ~1
             em = UvuEmitter(low, acc_budget_words=t["conv_acc"], kahan=kahan)
+            wide64_forward = True
     if wide64 and not any(k in user_tune for k in ("conv_wb", "conv_gres", "conv_split")):
         if 240 < em.backward_words(True) <= 480:
             t["conv_wb"], t["conv_gres"], t["conv_split"] = 1, 1, 0
@@ -2553,6 +2561,14 @@ def conv_module(low: Lowered, deterministic: bool, compute_units: int = 256, kah
         _lds, scratch = rt.kernel_resources(rt.compile_source(src)).get("forward", (0, 0))
         if scratch > 64:
             return conv_module(low, deterministic, compute_units, kahan, dict(override or {}, conv_segw=0))
+    if wide64_forward:
+        # fp64 with a node's whole output row in one wave's 512 registers: the estimate that admits this plan is
+        # optimistic for rows of 96 channels (two waves' lanes, the second half empty). With scratch memory the
+        # kernel loses to the output segments it was meant to beat (config-5 graph, forward, 96x{0e..3o}: 484 B,
+        # 25.9 against 8.3 ms; 228 B, 15.4 / 8.7; 96x{0e,1o,2e}: 196 B, 11.3 / 6.8).
+        _lds, scratch = rt.kernel_resources(rt.compile_source(src)).get("forward", (0, 0))
+        if scratch > 64:
+            return conv_module(low, deterministic, compute_units, kahan, dict(override or {}, conv_wf=2))
     if walk and t["conv_wf"] == 23 and "conv_wf" not in user_tune and low.elem_size == 4:
         # A forward kernel that the compiler gave more than a third of a SIMD's registers runs two waves there.
         # Held to a third it runs three, which pays where the compiler manages that without scratch memory (fp32,

@@ -237,10 +237,10 @@ def test_forward_kernel_takes_a_third_wave_where_that_costs_no_scratch_memory():
     spills = P.CTPP("128x0e+96x1e+64x2e", harmonics.replace("o", "e"), "0e+1e+2e", "mixed-channels")
     src, _dims, _descs = build_conv_module(spills, True)
     assert forward_bounds(src) == "2,3" and rt.kernel_registers(rt.compile_source(src))["forward"] > 168
-    # double precision is left alone
+    # double precision keeps the plain budget of two waves
     src, _dims, _descs = build_conv_module(P.CTPP("96x0e+96x1o+96x2e+96x3o", harmonics, "0e+1o+2e+3o", "96-channels-f64",
                                                   irrep_dtype=np.float64, weight_dtype=np.float64), True)
-    assert forward_bounds(src) == "2,3"
+    assert forward_bounds(src) == "2,2"
 
 
 def test_malformed_code_packs_are_rejected():
